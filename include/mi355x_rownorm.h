@@ -1,0 +1,160 @@
+/*
+ * mi355x_rownorm.h -- C ABI of the MI355X (gfx950) row-wise reduce-then-normalize kernels.
+ *
+ * This is the whole surface the host operator layer binds.  It replaces the
+ * kernel-entry functions of intel/torch-xpu-ops that take at::Tensor
+ * (src/ATen/native/xpu/sycl/LayerNormKernels.h:19-59 and
+ * src/ATen/native/xpu/sycl/SoftMaxKernels.h:19-43) with plain pointers and
+ * sizes, so that any host (the C++ ATen layer in csrc/host, ctypes, a test
+ * binary) can call the kernels without linking libtorch.
+ *
+ * Conventions
+ *  - Every pointer is a DEVICE pointer into memory the caller owns.  No
+ *    alignment beyond the element size is required of any pointer.
+ *  - Tensors are dense row-major [M, N] (rows x normalized size); mean/rstd
+ *    are float32 [M] whatever the input dtype, as at::toAccumulateType gives
+ *    in src/ATen/native/xpu/LayerNorm.cpp:72-75.
+ *  - Nothing here allocates, frees, synchronizes or throws.  Work is enqueued
+ *    on `stream` (a hipStream_t passed as void*; NULL = the default stream)
+ *    and the call returns at once; it is safe to call from several threads.
+ *  - Return value: 0 on success, a negative ROWNORM_ERR_* for a rejected
+ *    argument (nothing was launched), or a positive hipError_t value when a
+ *    launch failed.  mi355x_rownorm_error_string() renders either.
+ *  - M == 0 or N == 0 is a successful no-op, like the `if (M > 0)` guards in
+ *    LayerNorm.cpp:77,236,301 and `numel() > 0` in SoftMaxKernels.cpp:2150.
+ */
+#ifndef MI355X_ROWNORM_H_
+#define MI355X_ROWNORM_H_
+
+#include <stddef.h>
+#include <stdint.h>
+
+#ifdef __cplusplus
+extern "C" {
+#endif
+
+typedef enum {
+  ROWNORM_F32 = 0,
+  ROWNORM_F16 = 1,
+  ROWNORM_BF16 = 2
+} rownorm_dtype;
+
+enum {
+  ROWNORM_OK = 0,
+  ROWNORM_ERR_DTYPE = -1,     /* unknown dtype code or unsupported dtype pair */
+  ROWNORM_ERR_SHAPE = -2,     /* negative size, or N beyond 2^30 elements */
+  ROWNORM_ERR_NULL = -3,      /* a required pointer is NULL */
+  ROWNORM_ERR_WORKSPACE = -4, /* workspace missing or smaller than *_workspace_bytes() */
+  ROWNORM_ERR_OVERRIDE = -5   /* a forced variant cannot run this shape */
+};
+
+/* Operation ids for mi355x_rownorm_plan / mi355x_rownorm_set_override. */
+typedef enum {
+  ROWNORM_OP_LAYER_NORM_FWD = 0,
+  ROWNORM_OP_LAYER_NORM_BWD = 1,
+  ROWNORM_OP_RMS_NORM_FWD = 2,
+  ROWNORM_OP_RMS_NORM_BWD = 3,
+  ROWNORM_OP_SOFTMAX_FWD = 4,
+  ROWNORM_OP_SOFTMAX_BWD = 5,
+  ROWNORM_OP_COUNT = 6
+} rownorm_op;
+
+/* How one call is laid out on the GPU.  Replaces the reference's NormConfig
+ * heuristics (src/ATen/native/xpu/sycl/Norm.h:225-370) and get_wgroup_size
+ * (SoftMaxKernels.cpp:139-182); exposed so tests and logs can see the choice. */
+typedef struct {
+  int32_t resident;        /* 1: the row lives in registers (one HBM pass); 0: multi-pass streaming kernel */
+  int32_t lanes_per_row;   /* G: lanes that share one row (8..1024) */
+  int32_t packs_per_lane;  /* V: 16-byte packs each lane holds per row */
+  int32_t block_threads;   /* threads per workgroup */
+  int32_t rows_per_block;  /* rows a workgroup handles per iteration */
+  int32_t reserved;
+  int64_t grid_blocks;     /* workgroups launched (persistent, grid-stride over rows) */
+  int64_t partial_rows;    /* rows of the fp32 [partial_rows, N] column-sum workspace (backward only) */
+} rownorm_plan;
+
+const char* mi355x_rownorm_error_string(int code);
+
+/* ABI revision; bumped when a signature changes. */
+int mi355x_rownorm_abi_version(void);
+
+/* native_layer_norm forward.  Replaces layer_norm_kernel(X, gamma, beta, M, N, eps, Y*, mean*, rstd*)
+ * (LayerNormKernels.h:19-28).  gamma/beta may be NULL (treated as 1 / 0,
+ * LayerNormKernels.cpp:281-285); mean/rstd may be NULL (not written).
+ * w_dtype is the dtype of gamma and beta: equal to x_dtype, or ROWNORM_F32
+ * with a 16-bit x (mixed precision, a CPU-ATen feature the reference lacks). */
+int mi355x_layer_norm_fwd(const void* x, const void* gamma, const void* beta, void* y,
+                          float* mean, float* rstd, int64_t M, int64_t N, float eps,
+                          rownorm_dtype x_dtype, rownorm_dtype w_dtype, void* stream);
+
+/* Bytes of scratch mi355x_layer_norm_bwd needs for this call (0 when neither
+ * dgamma nor dbeta is wanted).  Replaces the at::empty/at::zeros scratch the
+ * reference allocates inside its entry point (LayerNormKernels.cpp:1255-1264). */
+size_t mi355x_layer_norm_bwd_workspace_bytes(int64_t M, int64_t N, rownorm_dtype x_dtype,
+                                             rownorm_dtype w_dtype, int want_dgamma,
+                                             int want_dbeta);
+
+/* native_layer_norm_backward.  Replaces layer_norm_backward_kernel(dY, X, mean, rstd, gamma, M, N,
+ * dX*, dgamma*, dbeta*) (LayerNormKernels.h:30-40).  Any of dx/dgamma/dbeta
+ * may be NULL and is then skipped (LayerNormKernels.cpp:1140,1270-1406).
+ * dx has x_dtype; dgamma/dbeta have w_dtype and are written in full (no
+ * accumulation into previous contents).  Column sums are accumulated in fp32
+ * and reduced in a fixed order: results are run-to-run deterministic. */
+int mi355x_layer_norm_bwd(const void* dy, const void* x, const float* mean, const float* rstd,
+                          const void* gamma, void* dx, void* dgamma, void* dbeta,
+                          void* workspace, size_t workspace_bytes, int64_t M, int64_t N,
+                          rownorm_dtype x_dtype, rownorm_dtype w_dtype, void* stream);
+
+/* _fused_rms_norm forward.  Replaces rms_norm_kernel(X, gamma, M, N, eps, Y*, rstd*)
+ * (LayerNormKernels.h:42-49). */
+int mi355x_rms_norm_fwd(const void* x, const void* gamma, void* y, float* rstd, int64_t M,
+                        int64_t N, float eps, rownorm_dtype x_dtype, rownorm_dtype w_dtype,
+                        void* stream);
+
+size_t mi355x_rms_norm_bwd_workspace_bytes(int64_t M, int64_t N, rownorm_dtype x_dtype,
+                                           rownorm_dtype w_dtype, int want_dgamma);
+
+/* _fused_rms_norm_backward.  Replaces rms_norm_backward_kernel(dY, X, rstd, gamma, M, N, dX*, dgamma*)
+ * (LayerNormKernels.h:51-59). */
+int mi355x_rms_norm_bwd(const void* dy, const void* x, const float* rstd, const void* gamma,
+                        void* dx, void* dgamma, void* workspace, size_t workspace_bytes,
+                        int64_t M, int64_t N, rownorm_dtype x_dtype, rownorm_dtype w_dtype,
+                        void* stream);
+
+/* _softmax / _log_softmax over the innermost dimension of a dense [rows, N]
+ * tensor.  Replaces _softmax_kernel / _log_softmax_kernel (SoftMaxKernels.h:19-29)
+ * for the inner_size == 1 case (SoftMaxKernels.cpp:1663-1720).  out_dtype is
+ * in_dtype, or ROWNORM_F32 with a ROWNORM_F16 input (half_to_float,
+ * SoftMaxKernels.cpp:2131-2135). */
+int mi355x_softmax_fwd(const void* x, void* y, int64_t rows, int64_t N, rownorm_dtype in_dtype,
+                       rownorm_dtype out_dtype, int is_log, void* stream);
+
+/* _softmax_backward_data / _log_softmax_backward_data.  Replaces
+ * _softmax_backward_kernel / _log_softmax_backward_kernel (SoftMaxKernels.h:31-43).
+ * grad and y (the forward OUTPUT) share grad_dtype; gi has gi_dtype, which is
+ * grad_dtype, or ROWNORM_F16 with ROWNORM_F32 grads (half_to_float,
+ * src/ATen/native/xpu/SoftMax.cpp:49-55). */
+int mi355x_softmax_bwd(const void* grad, const void* y, void* gi, int64_t rows, int64_t N,
+                       rownorm_dtype grad_dtype, rownorm_dtype gi_dtype, int is_log,
+                       void* stream);
+
+/* Reports the launch layout a call with these sizes would use on the current
+ * device (no launch; needs no GPU when the device query fails: 256 compute
+ * units are assumed).  x_dtype is the row dtype, w_dtype the weight dtype
+ * (ignored by the softmax ops). */
+int mi355x_rownorm_plan(rownorm_op op, int64_t M, int64_t N, rownorm_dtype x_dtype,
+                        rownorm_dtype w_dtype, rownorm_plan* out);
+
+/* Test and tuning hook: force lanes_per_row / packs_per_lane / threads per
+ * workgroup / workgroups per compute unit for one op (0 keeps the automatic
+ * choice for that field; lanes_per_row == -1 forces the multi-pass kernel).  Process-global and not
+ * synchronized with concurrent calls; production callers never use it.  A
+ * call whose shape the forced variant cannot hold fails with
+ * ROWNORM_ERR_OVERRIDE instead of silently choosing another. */
+int mi355x_rownorm_set_override(rownorm_op op, int lanes_per_row, int packs_per_lane,
+                                int block_threads, int blocks_per_cu);
+
+#ifdef __cplusplus
+}
+#endif
+#endif /* MI355X_ROWNORM_H_ */

@@ -1,0 +1,90 @@
+"""Shared input generators, tolerances and comparison helpers for the test suite."""
+import numpy as np
+import torch
+
+# Tolerances stated for this operator family: float32 results within rtol = atol = 1e-5 of the
+# CPU result; float16 / bfloat16 results within atol 1e-2, rtol 1.6e-2 of a reference that
+# accumulates in float32 or better (saved mean / rstd included).
+TOL = {torch.float32: (1e-5, 1e-5), torch.float16: (1.6e-2, 1e-2), torch.bfloat16: (1.6e-2, 1e-2)}
+
+
+def tol_for(dtype):
+    return TOL[dtype]
+
+
+def to_np32(t):
+    if t is None:
+        return None
+    return t.detach().to("cpu", torch.float32).contiguous().numpy()
+
+
+def excess(actual, expected, rtol, atol, slack=None):
+    """max over elements of |a - e| / (atol + rtol * |e| [+ slack]); <= 1 passes.
+    NaN/inf positions must agree exactly."""
+    a = torch.as_tensor(actual).detach().to("cpu", torch.float64).reshape(-1)
+    e = torch.as_tensor(expected).detach().to("cpu", torch.float64).reshape(-1)
+    assert a.shape == e.shape, (a.shape, e.shape)
+    if a.numel() == 0:
+        return 0.0
+    fin = torch.isfinite(e)
+    same_special = torch.equal(torch.isnan(a), torch.isnan(e)) and torch.equal(
+        a[~fin & ~torch.isnan(e)], e[~fin & ~torch.isnan(e)])
+    if not same_special:
+        return float("inf")
+    if not bool(fin.any()):
+        return 0.0
+    d = (a[fin] - e[fin]).abs()
+    bound = atol + rtol * e[fin].abs()
+    if slack is not None:
+        bound = bound + torch.as_tensor(slack).detach().to("cpu", torch.float64).reshape(-1)[fin]
+    return float((d / bound).max())
+
+
+def assert_close(actual, expected, dtype, what, slack=None, scale=1.0):
+    rtol, atol = tol_for(dtype)
+    ex = excess(actual, expected, rtol * scale, atol * scale, slack)
+    assert ex <= 1.0, "%s: error is %.3g x the tolerance (rtol %g, atol %g)" % (
+        what, ex, rtol * scale, atol * scale)
+    return ex
+
+
+def abs_err(a, b):
+    a = torch.as_tensor(a).detach().to("cpu", torch.float64)
+    b = torch.as_tensor(b).detach().to("cpu", torch.float64)
+    d = (a - b).abs()
+    d = torch.where(torch.isfinite(d), d, torch.zeros_like(d))
+    return d
+
+
+def gen(seed):
+    g = torch.Generator()
+    g.manual_seed(seed)
+    return g
+
+
+def offset_view(t, offset=2):
+    """A copy of `t` living `offset` elements into a fresh 256-byte aligned buffer, so its data
+    pointer is only offset*itemsize aligned."""
+    buf = torch.empty(t.numel() + offset + 64, dtype=t.dtype, device=t.device)
+    v = buf[offset:offset + t.numel()].view(t.shape)
+    v.copy_(t)
+    assert v.data_ptr() % 16 == (offset * t.element_size()) % 16
+    return v
+
+
+def stress_rows(M, N, seed, dtype=torch.float32):
+    """N(0,1) rows with 0.1% of entries replaced by +-1e4 and row 0 constant (1.5)."""
+    g = gen(seed)
+    x = torch.randn(M, N, generator=g)
+    mask = torch.rand(M, N, generator=g) < 0.001
+    sign = torch.where(torch.rand(M, N, generator=g) < 0.5, -1.0, 1.0)
+    x = torch.where(mask, 1e4 * sign, x)
+    x[0] = 1.5
+    return x.to(dtype)
+
+
+def causal_scores(B, H, T, seed, dtype=torch.bfloat16):
+    g = gen(seed)
+    s = 3.0 * torch.randn(B, H, T, T, generator=g)
+    s.masked_fill_(torch.triu(torch.ones(T, T), 1).bool(), float("-inf"))
+    return s.to(dtype)

@@ -1,0 +1,231 @@
+"""ctypes bindings of the extern "C" launcher ABI declared in include/mi355x_rownorm.h.
+
+The functions here take torch tensors purely as device memory (``data_ptr()``) plus the current
+HIP stream; shapes are [M, N] views of contiguous tensors.  They allocate outputs and the
+backward workspace with torch, call the ABI, and raise ``RuntimeError`` on a non-zero status.
+"""
+import ctypes
+import os
+
+_HERE = os.path.dirname(os.path.abspath(__file__))
+_KERNEL_LIB = os.path.join(_HERE, "lib", "libmi355x_rownorm.so")
+
+F32, F16, BF16 = 0, 1, 2
+OP_LAYER_NORM_FWD, OP_LAYER_NORM_BWD, OP_RMS_NORM_FWD, OP_RMS_NORM_BWD = 0, 1, 2, 3
+OP_SOFTMAX_FWD, OP_SOFTMAX_BWD = 4, 5
+
+EXPORTED_SYMBOLS = (
+    "mi355x_rownorm_error_string", "mi355x_rownorm_abi_version", "mi355x_layer_norm_fwd",
+    "mi355x_layer_norm_bwd_workspace_bytes", "mi355x_layer_norm_bwd", "mi355x_rms_norm_fwd",
+    "mi355x_rms_norm_bwd_workspace_bytes", "mi355x_rms_norm_bwd", "mi355x_softmax_fwd",
+    "mi355x_softmax_bwd", "mi355x_rownorm_plan", "mi355x_rownorm_set_override",
+)
+
+
+class Plan(ctypes.Structure):
+    _fields_ = [("resident", ctypes.c_int32), ("lanes_per_row", ctypes.c_int32),
+                ("packs_per_lane", ctypes.c_int32), ("block_threads", ctypes.c_int32),
+                ("rows_per_block", ctypes.c_int32), ("reserved", ctypes.c_int32),
+                ("grid_blocks", ctypes.c_int64), ("partial_rows", ctypes.c_int64)]
+
+    def as_dict(self):
+        return {k: getattr(self, k) for k, _ in self._fields_ if k != "reserved"}
+
+
+_lib = None
+_vp, _i64, _int, _f = ctypes.c_void_p, ctypes.c_int64, ctypes.c_int, ctypes.c_float
+
+
+def lib():
+    """The kernel library; raises if it has not been built (there is no fallback)."""
+    global _lib
+    if _lib is None:
+        if not os.path.exists(_KERNEL_LIB):
+            raise RuntimeError("%s is missing: run build.py next to this file" % _KERNEL_LIB)
+        L = ctypes.CDLL(_KERNEL_LIB)
+        L.mi355x_rownorm_error_string.restype = ctypes.c_char_p
+        L.mi355x_rownorm_error_string.argtypes = [_int]
+        L.mi355x_rownorm_abi_version.restype = _int
+        L.mi355x_layer_norm_fwd.argtypes = [_vp, _vp, _vp, _vp, _vp, _vp, _i64, _i64, _f, _int,
+                                            _int, _vp]
+        L.mi355x_rms_norm_fwd.argtypes = [_vp, _vp, _vp, _vp, _i64, _i64, _f, _int, _int, _vp]
+        L.mi355x_layer_norm_bwd_workspace_bytes.restype = ctypes.c_size_t
+        L.mi355x_layer_norm_bwd_workspace_bytes.argtypes = [_i64, _i64, _int, _int, _int, _int]
+        L.mi355x_rms_norm_bwd_workspace_bytes.restype = ctypes.c_size_t
+        L.mi355x_rms_norm_bwd_workspace_bytes.argtypes = [_i64, _i64, _int, _int, _int]
+        L.mi355x_layer_norm_bwd.argtypes = [_vp, _vp, _vp, _vp, _vp, _vp, _vp, _vp, _vp,
+                                            ctypes.c_size_t, _i64, _i64, _int, _int, _vp]
+        L.mi355x_rms_norm_bwd.argtypes = [_vp, _vp, _vp, _vp, _vp, _vp, _vp, ctypes.c_size_t,
+                                          _i64, _i64, _int, _int, _vp]
+        L.mi355x_softmax_fwd.argtypes = [_vp, _vp, _i64, _i64, _int, _int, _int, _vp]
+        L.mi355x_softmax_bwd.argtypes = [_vp, _vp, _vp, _i64, _i64, _int, _int, _int, _vp]
+        L.mi355x_rownorm_plan.argtypes = [_int, _i64, _i64, _int, _int, ctypes.POINTER(Plan)]
+        L.mi355x_rownorm_set_override.argtypes = [_int, _int, _int, _int, _int]
+        for name in ("mi355x_layer_norm_fwd", "mi355x_rms_norm_fwd", "mi355x_layer_norm_bwd",
+                     "mi355x_rms_norm_bwd", "mi355x_softmax_fwd", "mi355x_softmax_bwd",
+                     "mi355x_rownorm_plan", "mi355x_rownorm_set_override"):
+            getattr(L, name).restype = _int
+        _lib = L
+    return _lib
+
+
+def error_string(code):
+    return lib().mi355x_rownorm_error_string(code).decode()
+
+
+def _check(code, what):
+    if code != 0:
+        raise RuntimeError("%s failed: %s (code %d)" % (what, error_string(code), code))
+
+
+def dtype_code(dt):
+    import torch
+    try:
+        return {torch.float32: F32, torch.float16: F16, torch.bfloat16: BF16}[dt]
+    except KeyError:
+        raise RuntimeError("dtype %s is not implemented by the MI355X kernels" % dt)
+
+
+def plan(op, M, N, x_dtype=F32, w_dtype=F32):
+    p = Plan()
+    _check(lib().mi355x_rownorm_plan(op, M, N, x_dtype, w_dtype, ctypes.byref(p)), "plan")
+    return p.as_dict()
+
+
+def set_override(op, lanes_per_row=0, packs_per_lane=0, block_threads=0, blocks_per_cu=0):
+    _check(lib().mi355x_rownorm_set_override(op, lanes_per_row, packs_per_lane, block_threads,
+                                             blocks_per_cu), "set_override")
+
+
+def clear_overrides():
+    for op in range(6):
+        set_override(op)
+
+
+def _ptr(t):
+    return None if t is None else ctypes.c_void_p(t.data_ptr())
+
+
+def _stream():
+    import torch
+    return ctypes.c_void_p(torch.cuda.current_stream().cuda_stream)
+
+
+def _gpu(*tensors):
+    for t in tensors:
+        if t is not None and not t.is_cuda:
+            raise RuntimeError("expected a HIP GPU tensor, got device %s (no CPU path)" % t.device)
+
+
+def _rows(x, n_norm_dims):
+    axis = x.dim() - n_norm_dims
+    M = 1
+    for s in x.shape[:axis]:
+        M *= s
+    N = 1
+    for s in x.shape[axis:]:
+        N *= s
+    return M, N
+
+
+def _wd(x, *ws):
+    for w in ws:
+        if w is not None:
+            return dtype_code(w.dtype)
+    return dtype_code(x.dtype)
+
+
+def layer_norm_fwd(x, gamma, beta, eps, n_norm_dims=1, y=None, mean=None, rstd=None):
+    """-> (y, mean[M], rstd[M]); x is viewed as [M, N] (must be dense)."""
+    import torch
+    _gpu(x, gamma, beta)
+    M, N = _rows(x, n_norm_dims)
+    y = torch.empty_like(x) if y is None else y
+    mean = torch.empty(M, dtype=torch.float32, device=x.device) if mean is None else mean
+    rstd = torch.empty(M, dtype=torch.float32, device=x.device) if rstd is None else rstd
+    _check(lib().mi355x_layer_norm_fwd(_ptr(x), _ptr(gamma), _ptr(beta), _ptr(y), _ptr(mean),
+                                       _ptr(rstd), M, N, eps, dtype_code(x.dtype),
+                                       _wd(x, gamma, beta), _stream()), "layer_norm_fwd")
+    return y, mean, rstd
+
+
+def rms_norm_fwd(x, gamma, eps, n_norm_dims=1, y=None, rstd=None):
+    import torch
+    _gpu(x, gamma)
+    M, N = _rows(x, n_norm_dims)
+    y = torch.empty_like(x) if y is None else y
+    rstd = torch.empty(M, dtype=torch.float32, device=x.device) if rstd is None else rstd
+    _check(lib().mi355x_rms_norm_fwd(_ptr(x), _ptr(gamma), _ptr(y), _ptr(rstd), M, N, eps,
+                                     dtype_code(x.dtype), _wd(x, gamma), _stream()),
+           "rms_norm_fwd")
+    return y, rstd
+
+
+def layer_norm_bwd(dy, x, mean, rstd, gamma, n_norm_dims=1, want=(True, True, True),
+                   w_dtype=None, dx=None, dgamma=None, dbeta=None, workspace=None):
+    import torch
+    _gpu(dy, x, mean, rstd, gamma)
+    M, N = _rows(x, n_norm_dims)
+    wdt = w_dtype if w_dtype is not None else (gamma.dtype if gamma is not None else x.dtype)
+    if want[0] and dx is None:
+        dx = torch.empty_like(x)
+    if want[1] and dgamma is None:
+        dgamma = torch.empty(N, dtype=wdt, device=x.device)
+    if want[2] and dbeta is None:
+        dbeta = torch.empty(N, dtype=wdt, device=x.device)
+    xd, wd = dtype_code(x.dtype), dtype_code(wdt)
+    nbytes = lib().mi355x_layer_norm_bwd_workspace_bytes(M, N, xd, wd, int(dgamma is not None),
+                                                         int(dbeta is not None))
+    if workspace is None and nbytes:
+        workspace = torch.empty(nbytes, dtype=torch.uint8, device=x.device)
+    _check(lib().mi355x_layer_norm_bwd(_ptr(dy), _ptr(x), _ptr(mean), _ptr(rstd), _ptr(gamma),
+                                       _ptr(dx), _ptr(dgamma), _ptr(dbeta), _ptr(workspace),
+                                       0 if workspace is None else workspace.numel(), M, N, xd, wd,
+                                       _stream()), "layer_norm_bwd")
+    return dx, dgamma, dbeta
+
+
+def rms_norm_bwd(dy, x, rstd, gamma, n_norm_dims=1, want=(True, True), w_dtype=None, dx=None,
+                 dgamma=None, workspace=None):
+    import torch
+    _gpu(dy, x, rstd, gamma)
+    M, N = _rows(x, n_norm_dims)
+    wdt = w_dtype if w_dtype is not None else (gamma.dtype if gamma is not None else x.dtype)
+    if want[0] and dx is None:
+        dx = torch.empty_like(x)
+    if want[1] and dgamma is None:
+        dgamma = torch.empty(N, dtype=wdt, device=x.device)
+    xd, wd = dtype_code(x.dtype), dtype_code(wdt)
+    nbytes = lib().mi355x_rms_norm_bwd_workspace_bytes(M, N, xd, wd, int(dgamma is not None))
+    if workspace is None and nbytes:
+        workspace = torch.empty(nbytes, dtype=torch.uint8, device=x.device)
+    _check(lib().mi355x_rms_norm_bwd(_ptr(dy), _ptr(x), _ptr(rstd), _ptr(gamma), _ptr(dx),
+                                     _ptr(dgamma), _ptr(workspace),
+                                     0 if workspace is None else workspace.numel(), M, N, xd, wd,
+                                     _stream()), "rms_norm_bwd")
+    return dx, dgamma
+
+
+def softmax_fwd(x, is_log=False, out_dtype=None, y=None):
+    import torch
+    _gpu(x)
+    N = x.shape[-1] if x.dim() else 1
+    rows = x.numel() // N if N else 0
+    od = x.dtype if out_dtype is None else out_dtype
+    y = torch.empty(x.shape, dtype=od, device=x.device) if y is None else y
+    _check(lib().mi355x_softmax_fwd(_ptr(x), _ptr(y), rows, N, dtype_code(x.dtype),
+                                    dtype_code(y.dtype), int(is_log), _stream()), "softmax_fwd")
+    return y
+
+
+def softmax_bwd(grad, y, is_log=False, gi_dtype=None, gi=None):
+    import torch
+    _gpu(grad, y)
+    N = y.shape[-1] if y.dim() else 1
+    rows = y.numel() // N if N else 0
+    od = grad.dtype if gi_dtype is None else gi_dtype
+    gi = torch.empty(y.shape, dtype=od, device=y.device) if gi is None else gi
+    _check(lib().mi355x_softmax_bwd(_ptr(grad), _ptr(y), _ptr(gi), rows, N,
+                                    dtype_code(grad.dtype), dtype_code(gi.dtype), int(is_log),
+                                    _stream()), "softmax_bwd")
+    return gi

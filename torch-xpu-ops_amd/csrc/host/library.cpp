@@ -1,0 +1,58 @@
+// Operator registration: torch.ops.mi355x.<name> with the schemas of the ATen
+// ops the reference implements (its registration goes through PyTorch's
+// native_functions.yaml XPU dispatch keys and REGISTER_XPU_DISPATCH,
+// src/ATen/native/xpu/LayerNorm.cpp:198-201).  The ops are registered for
+// every backend key and reject non-GPU tensors themselves, so a wrong device
+// is a clear error instead of a missing-kernel message.  Nothing here touches
+// the aten:: namespace; routing aten ops to these kernels is an explicit
+// opt-in done from Python.
+#include <torch/library.h>
+
+#include "norm_ops.h"
+#include "softmax_ops.h"
+
+TORCH_LIBRARY(mi355x, m) {
+  m.def(
+      "native_layer_norm(Tensor input, int[] normalized_shape, Tensor? weight, Tensor? bias, "
+      "float eps) -> (Tensor, Tensor, Tensor)",
+      &mi355x::native_layer_norm);
+  m.def(
+      "native_layer_norm_backward(Tensor grad_out, Tensor input, int[] normalized_shape, "
+      "Tensor mean, Tensor rstd, Tensor? weight, Tensor? bias, bool[3] output_mask) -> "
+      "(Tensor, Tensor, Tensor)",
+      &mi355x::native_layer_norm_backward);
+  m.def(
+      "_fused_rms_norm(Tensor input, int[] normalized_shape, Tensor? weight, float? eps) -> "
+      "(Tensor, Tensor)",
+      &mi355x::_fused_rms_norm);
+  m.def(
+      "_fused_rms_norm_backward(Tensor grad_out, Tensor input, int[] normalized_shape, "
+      "Tensor rstd, Tensor? weight, bool[2] output_mask) -> (Tensor, Tensor)",
+      &mi355x::_fused_rms_norm_backward);
+  m.def("_softmax(Tensor self, int dim, bool half_to_float) -> Tensor", &mi355x::_softmax);
+  m.def("_log_softmax(Tensor self, int dim, bool half_to_float) -> Tensor",
+        &mi355x::_log_softmax);
+  m.def("_softmax.out(Tensor self, int dim, bool half_to_float, *, Tensor(a!) out) -> Tensor(a!)",
+        &mi355x::_softmax_out);
+  m.def(
+      "_log_softmax.out(Tensor self, int dim, bool half_to_float, *, Tensor(a!) out) -> "
+      "Tensor(a!)",
+      &mi355x::_log_softmax_out);
+  m.def(
+      "_softmax_backward_data(Tensor grad_output, Tensor output, int dim, ScalarType "
+      "input_dtype) -> Tensor",
+      &mi355x::_softmax_backward_data);
+  m.def(
+      "_log_softmax_backward_data(Tensor grad_output, Tensor output, int dim, ScalarType "
+      "input_dtype) -> Tensor",
+      &mi355x::_log_softmax_backward_data);
+  m.def(
+      "_softmax_backward_data.out(Tensor grad_output, Tensor output, int dim, ScalarType "
+      "input_dtype, *, Tensor(a!) grad_input) -> Tensor(a!)",
+      &mi355x::_softmax_backward_data_out);
+  m.def(
+      "_log_softmax_backward_data.out(Tensor grad_output, Tensor output, int dim, ScalarType "
+      "input_dtype, *, Tensor(a!) out) -> Tensor(a!)",
+      &mi355x::_log_softmax_backward_data_out);
+  m.def("install_layer_norm_dispatch_stubs() -> ()", &mi355x::install_layer_norm_dispatch_stubs);
+}

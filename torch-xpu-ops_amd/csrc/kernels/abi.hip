@@ -1,0 +1,306 @@
+// extern "C" surface of libmi355x_rownorm.so (declared in include/mi355x_rownorm.h).
+// Validates arguments, picks the launch layout and forwards to the typed
+// launch templates; allocates nothing and never synchronizes.
+#include "../../../include/mi355x_rownorm.h"
+
+#include <atomic>
+#include "launch.hpp"
+
+namespace rownorm {
+// defined in the per-dtype translation units
+extern template int launch_norm_fwd<float, float, false>(const Plan&, const NormFwdArgs&, hipStream_t);
+extern template int launch_norm_fwd<float, float, true>(const Plan&, const NormFwdArgs&, hipStream_t);
+extern template int launch_norm_fwd<f16, f16, false>(const Plan&, const NormFwdArgs&, hipStream_t);
+extern template int launch_norm_fwd<f16, f16, true>(const Plan&, const NormFwdArgs&, hipStream_t);
+extern template int launch_norm_fwd<f16, float, false>(const Plan&, const NormFwdArgs&, hipStream_t);
+extern template int launch_norm_fwd<f16, float, true>(const Plan&, const NormFwdArgs&, hipStream_t);
+extern template int launch_norm_fwd<bf16, bf16, false>(const Plan&, const NormFwdArgs&, hipStream_t);
+extern template int launch_norm_fwd<bf16, bf16, true>(const Plan&, const NormFwdArgs&, hipStream_t);
+extern template int launch_norm_fwd<bf16, float, false>(const Plan&, const NormFwdArgs&, hipStream_t);
+extern template int launch_norm_fwd<bf16, float, true>(const Plan&, const NormFwdArgs&, hipStream_t);
+extern template int launch_norm_bwd<float, float, false>(const Plan&, const NormBwdArgs&, hipStream_t);
+extern template int launch_norm_bwd<float, float, true>(const Plan&, const NormBwdArgs&, hipStream_t);
+extern template int launch_norm_bwd<f16, f16, false>(const Plan&, const NormBwdArgs&, hipStream_t);
+extern template int launch_norm_bwd<f16, f16, true>(const Plan&, const NormBwdArgs&, hipStream_t);
+extern template int launch_norm_bwd<f16, float, false>(const Plan&, const NormBwdArgs&, hipStream_t);
+extern template int launch_norm_bwd<f16, float, true>(const Plan&, const NormBwdArgs&, hipStream_t);
+extern template int launch_norm_bwd<bf16, bf16, false>(const Plan&, const NormBwdArgs&, hipStream_t);
+extern template int launch_norm_bwd<bf16, bf16, true>(const Plan&, const NormBwdArgs&, hipStream_t);
+extern template int launch_norm_bwd<bf16, float, false>(const Plan&, const NormBwdArgs&, hipStream_t);
+extern template int launch_norm_bwd<bf16, float, true>(const Plan&, const NormBwdArgs&, hipStream_t);
+extern template int launch_softmax_fwd<float, float>(const Plan&, const SoftmaxFwdArgs&, hipStream_t);
+extern template int launch_softmax_fwd<f16, f16>(const Plan&, const SoftmaxFwdArgs&, hipStream_t);
+extern template int launch_softmax_fwd<bf16, bf16>(const Plan&, const SoftmaxFwdArgs&, hipStream_t);
+extern template int launch_softmax_fwd<f16, float>(const Plan&, const SoftmaxFwdArgs&, hipStream_t);
+extern template int launch_softmax_bwd<float, float>(const Plan&, const SoftmaxBwdArgs&, hipStream_t);
+extern template int launch_softmax_bwd<f16, f16>(const Plan&, const SoftmaxBwdArgs&, hipStream_t);
+extern template int launch_softmax_bwd<bf16, bf16>(const Plan&, const SoftmaxBwdArgs&, hipStream_t);
+extern template int launch_softmax_bwd<float, f16>(const Plan&, const SoftmaxBwdArgs&, hipStream_t);
+}  // namespace rownorm
+
+using namespace rownorm;
+
+namespace {
+
+constexpr int64_t kMaxN = int64_t(1) << 30;
+constexpr int kMaxDevices = 64;
+
+// Compute units per device, looked up once per device (0 = not yet known).
+std::atomic<int> g_num_cus[kMaxDevices];
+
+int current_num_cus() {
+  int dev = 0;
+  if (hipGetDevice(&dev) != hipSuccess) {
+    (void)hipGetLastError();
+    return 256;
+  }
+  if (dev < 0 || dev >= kMaxDevices) return 256;
+  int n = g_num_cus[dev].load(std::memory_order_relaxed);
+  if (n > 0) return n;
+  int v = 0;
+  if (hipDeviceGetAttribute(&v, hipDeviceAttributeMultiprocessorCount, dev) != hipSuccess ||
+      v <= 0) {
+    (void)hipGetLastError();
+    v = 256;
+  }
+  g_num_cus[dev].store(v, std::memory_order_relaxed);
+  return v;
+}
+
+// Forced variants for tests and tuning (process-global, see the header).
+Override g_override[ROWNORM_OP_COUNT];
+
+int esize_of(int dt) {
+  switch (dt) {
+    case ROWNORM_F32: return 4;
+    case ROWNORM_F16: return 2;
+    case ROWNORM_BF16: return 2;
+  }
+  return 0;
+}
+
+bool norm_dtypes_ok(int x, int w) {
+  if (esize_of(x) == 0 || esize_of(w) == 0) return false;
+  return w == x || (w == ROWNORM_F32);
+}
+
+OpClass class_of(int op) {
+  switch (op) {
+    case ROWNORM_OP_LAYER_NORM_FWD:
+    case ROWNORM_OP_RMS_NORM_FWD: return OC_NORM_FWD;
+    case ROWNORM_OP_LAYER_NORM_BWD:
+    case ROWNORM_OP_RMS_NORM_BWD: return OC_NORM_BWD;
+    case ROWNORM_OP_SOFTMAX_FWD: return OC_SOFTMAX_FWD;
+    default: return OC_SOFTMAX_BWD;
+  }
+}
+
+int shape_check(int64_t M, int64_t N) {
+  if (M < 0 || N < 0 || N > kMaxN) return ROWNORM_ERR_SHAPE;
+  return 0;
+}
+
+template <bool RMS>
+int norm_fwd(const void* x, const void* gamma, const void* beta, void* y, float* mean,
+             float* rstd, int64_t M, int64_t N, float eps, int xd, int wd, void* stream) {
+  if (!norm_dtypes_ok(xd, wd)) return ROWNORM_ERR_DTYPE;
+  if (int e = shape_check(M, N)) return e;
+  if (M == 0 || N == 0) return 0;
+  if (!x || !y) return ROWNORM_ERR_NULL;
+  Plan plan;
+  const int op = RMS ? ROWNORM_OP_RMS_NORM_FWD : ROWNORM_OP_LAYER_NORM_FWD;
+  if (int e = make_plan(OC_NORM_FWD, M, N, esize_of(xd), current_num_cus(), g_override[op],
+                        false, &plan))
+    return e;
+  NormFwdArgs a{x, gamma, RMS ? nullptr : beta, y, RMS ? nullptr : mean, rstd, M, (int)N, eps};
+  hipStream_t s = (hipStream_t)stream;
+  if (xd == ROWNORM_F32) return launch_norm_fwd<float, float, RMS>(plan, a, s);
+  if (xd == ROWNORM_F16)
+    return wd == ROWNORM_F32 ? launch_norm_fwd<f16, float, RMS>(plan, a, s)
+                             : launch_norm_fwd<f16, f16, RMS>(plan, a, s);
+  return wd == ROWNORM_F32 ? launch_norm_fwd<bf16, float, RMS>(plan, a, s)
+                           : launch_norm_fwd<bf16, bf16, RMS>(plan, a, s);
+}
+
+size_t norm_bwd_workspace(int op, int64_t M, int64_t N, int xd, int wd, int nparts) {
+  if (!norm_dtypes_ok(xd, wd) || shape_check(M, N) || M == 0 || N == 0 || nparts == 0) return 0;
+  Plan plan;
+  if (make_plan(OC_NORM_BWD, M, N, esize_of(xd), current_num_cus(), g_override[op], true, &plan))
+    return 0;
+  return (size_t)plan.partial_rows * (size_t)N * sizeof(float) * (size_t)nparts;
+}
+
+template <bool RMS>
+int norm_bwd(const void* dy, const void* x, const float* mean, const float* rstd,
+             const void* gamma, void* dx, void* dgamma, void* dbeta, void* workspace,
+             size_t workspace_bytes, int64_t M, int64_t N, int xd, int wd, void* stream) {
+  if (!norm_dtypes_ok(xd, wd)) return ROWNORM_ERR_DTYPE;
+  if (int e = shape_check(M, N)) return e;
+  if (M == 0 || N == 0) return 0;
+  if (RMS) dbeta = nullptr;
+  const bool want_cols = dgamma != nullptr || dbeta != nullptr;
+  if (!dx && !want_cols) return 0;
+  if (!dy || !x || !rstd || (!RMS && !mean)) return ROWNORM_ERR_NULL;
+  Plan plan;
+  const int op = RMS ? ROWNORM_OP_RMS_NORM_BWD : ROWNORM_OP_LAYER_NORM_BWD;
+  if (int e = make_plan(OC_NORM_BWD, M, N, esize_of(xd), current_num_cus(), g_override[op],
+                        want_cols, &plan))
+    return e;
+  float* part_dg = nullptr;
+  float* part_db = nullptr;
+  if (want_cols) {
+    const size_t one = (size_t)plan.partial_rows * (size_t)N * sizeof(float);
+    const size_t need = one * (RMS ? 1 : 2);
+    if (!workspace || workspace_bytes < need) return ROWNORM_ERR_WORKSPACE;
+    part_dg = (float*)workspace;
+    part_db = RMS ? nullptr : (float*)((char*)workspace + one);
+  }
+  NormBwdArgs a{dy, x, mean, rstd, gamma, dx, dgamma, dbeta, part_dg, part_db, M, (int)N};
+  hipStream_t s = (hipStream_t)stream;
+  if (xd == ROWNORM_F32) return launch_norm_bwd<float, float, RMS>(plan, a, s);
+  if (xd == ROWNORM_F16)
+    return wd == ROWNORM_F32 ? launch_norm_bwd<f16, float, RMS>(plan, a, s)
+                             : launch_norm_bwd<f16, f16, RMS>(plan, a, s);
+  return wd == ROWNORM_F32 ? launch_norm_bwd<bf16, float, RMS>(plan, a, s)
+                           : launch_norm_bwd<bf16, bf16, RMS>(plan, a, s);
+}
+
+}  // namespace
+
+extern "C" {
+
+const char* mi355x_rownorm_error_string(int code) {
+  switch (code) {
+    case ROWNORM_OK: return "success";
+    case ROWNORM_ERR_DTYPE: return "mi355x_rownorm: unsupported dtype or dtype pair";
+    case ROWNORM_ERR_SHAPE: return "mi355x_rownorm: invalid shape (negative size or N > 2^30)";
+    case ROWNORM_ERR_NULL: return "mi355x_rownorm: a required pointer is NULL";
+    case ROWNORM_ERR_WORKSPACE: return "mi355x_rownorm: workspace missing or too small";
+    case ROWNORM_ERR_OVERRIDE: return "mi355x_rownorm: forced variant cannot run this shape";
+  }
+  if (code > 0) return hipGetErrorString((hipError_t)code);
+  return "mi355x_rownorm: unknown error code";
+}
+
+int mi355x_rownorm_abi_version(void) { return 1; }
+
+int mi355x_layer_norm_fwd(const void* x, const void* gamma, const void* beta, void* y,
+                          float* mean, float* rstd, int64_t M, int64_t N, float eps,
+                          rownorm_dtype x_dtype, rownorm_dtype w_dtype, void* stream) {
+  return norm_fwd<false>(x, gamma, beta, y, mean, rstd, M, N, eps, (int)x_dtype, (int)w_dtype,
+                         stream);
+}
+
+int mi355x_rms_norm_fwd(const void* x, const void* gamma, void* y, float* rstd, int64_t M,
+                        int64_t N, float eps, rownorm_dtype x_dtype, rownorm_dtype w_dtype,
+                        void* stream) {
+  return norm_fwd<true>(x, gamma, nullptr, y, nullptr, rstd, M, N, eps, (int)x_dtype,
+                        (int)w_dtype, stream);
+}
+
+size_t mi355x_layer_norm_bwd_workspace_bytes(int64_t M, int64_t N, rownorm_dtype x_dtype,
+                                             rownorm_dtype w_dtype, int want_dgamma,
+                                             int want_dbeta) {
+  return norm_bwd_workspace(ROWNORM_OP_LAYER_NORM_BWD, M, N, (int)x_dtype, (int)w_dtype,
+                            (want_dgamma || want_dbeta) ? 2 : 0);
+}
+
+size_t mi355x_rms_norm_bwd_workspace_bytes(int64_t M, int64_t N, rownorm_dtype x_dtype,
+                                           rownorm_dtype w_dtype, int want_dgamma) {
+  return norm_bwd_workspace(ROWNORM_OP_RMS_NORM_BWD, M, N, (int)x_dtype, (int)w_dtype,
+                            want_dgamma ? 1 : 0);
+}
+
+int mi355x_layer_norm_bwd(const void* dy, const void* x, const float* mean, const float* rstd,
+                          const void* gamma, void* dx, void* dgamma, void* dbeta,
+                          void* workspace, size_t workspace_bytes, int64_t M, int64_t N,
+                          rownorm_dtype x_dtype, rownorm_dtype w_dtype, void* stream) {
+  return norm_bwd<false>(dy, x, mean, rstd, gamma, dx, dgamma, dbeta, workspace, workspace_bytes,
+                         M, N, (int)x_dtype, (int)w_dtype, stream);
+}
+
+int mi355x_rms_norm_bwd(const void* dy, const void* x, const float* rstd, const void* gamma,
+                        void* dx, void* dgamma, void* workspace, size_t workspace_bytes,
+                        int64_t M, int64_t N, rownorm_dtype x_dtype, rownorm_dtype w_dtype,
+                        void* stream) {
+  return norm_bwd<true>(dy, x, nullptr, rstd, gamma, dx, dgamma, nullptr, workspace,
+                        workspace_bytes, M, N, (int)x_dtype, (int)w_dtype, stream);
+}
+
+int mi355x_softmax_fwd(const void* x, void* y, int64_t rows, int64_t N, rownorm_dtype in_dtype,
+                       rownorm_dtype out_dtype, int is_log, void* stream) {
+  const int id = (int)in_dtype, od = (int)out_dtype;
+  if (esize_of(id) == 0 || esize_of(od) == 0) return ROWNORM_ERR_DTYPE;
+  if (!(od == id || (id == ROWNORM_F16 && od == ROWNORM_F32))) return ROWNORM_ERR_DTYPE;
+  if (int e = shape_check(rows, N)) return e;
+  if (rows == 0 || N == 0) return 0;
+  if (!x || !y) return ROWNORM_ERR_NULL;
+  Plan plan;
+  if (int e = make_plan(OC_SOFTMAX_FWD, rows, N, esize_of(id), current_num_cus(),
+                        g_override[ROWNORM_OP_SOFTMAX_FWD], false, &plan))
+    return e;
+  SoftmaxFwdArgs a{x, y, rows, (int)N, is_log ? 1 : 0};
+  hipStream_t s = (hipStream_t)stream;
+  if (id == ROWNORM_F32) return launch_softmax_fwd<float, float>(plan, a, s);
+  if (id == ROWNORM_BF16) return launch_softmax_fwd<bf16, bf16>(plan, a, s);
+  return od == ROWNORM_F32 ? launch_softmax_fwd<f16, float>(plan, a, s)
+                           : launch_softmax_fwd<f16, f16>(plan, a, s);
+}
+
+int mi355x_softmax_bwd(const void* grad, const void* y, void* gi, int64_t rows, int64_t N,
+                       rownorm_dtype grad_dtype, rownorm_dtype gi_dtype, int is_log,
+                       void* stream) {
+  const int gd = (int)grad_dtype, od = (int)gi_dtype;
+  if (esize_of(gd) == 0 || esize_of(od) == 0) return ROWNORM_ERR_DTYPE;
+  if (!(od == gd || (gd == ROWNORM_F32 && od == ROWNORM_F16))) return ROWNORM_ERR_DTYPE;
+  if (int e = shape_check(rows, N)) return e;
+  if (rows == 0 || N == 0) return 0;
+  if (!grad || !y || !gi) return ROWNORM_ERR_NULL;
+  Plan plan;
+  if (int e = make_plan(OC_SOFTMAX_BWD, rows, N, esize_of(gd), current_num_cus(),
+                        g_override[ROWNORM_OP_SOFTMAX_BWD], false, &plan))
+    return e;
+  SoftmaxBwdArgs a{grad, y, gi, rows, (int)N, is_log ? 1 : 0};
+  hipStream_t s = (hipStream_t)stream;
+  if (gd == ROWNORM_BF16) return launch_softmax_bwd<bf16, bf16>(plan, a, s);
+  if (gd == ROWNORM_F16) return launch_softmax_bwd<f16, f16>(plan, a, s);
+  return od == ROWNORM_F16 ? launch_softmax_bwd<float, f16>(plan, a, s)
+                           : launch_softmax_bwd<float, float>(plan, a, s);
+}
+
+int mi355x_rownorm_plan(rownorm_op op, int64_t M, int64_t N, rownorm_dtype x_dtype,
+                        rownorm_dtype w_dtype, rownorm_plan* out) {
+  (void)w_dtype;
+  if ((int)op < 0 || (int)op >= ROWNORM_OP_COUNT) return ROWNORM_ERR_SHAPE;
+  if (!out) return ROWNORM_ERR_NULL;
+  if (esize_of((int)x_dtype) == 0) return ROWNORM_ERR_DTYPE;
+  if (int e = shape_check(M, N)) return e;
+  Plan plan;
+  const OpClass oc = class_of((int)op);
+  if (int e = make_plan(oc, M, N, esize_of((int)x_dtype), current_num_cus(), g_override[(int)op],
+                        oc == OC_NORM_BWD, &plan))
+    return e;
+  out->resident = plan.resident ? 1 : 0;
+  out->lanes_per_row = plan.G;
+  out->packs_per_lane = plan.V;
+  out->block_threads = plan.block;
+  out->rows_per_block = plan.rpb;
+  out->reserved = 0;
+  out->grid_blocks = plan.grid;
+  out->partial_rows = plan.partial_rows;
+  return 0;
+}
+
+int mi355x_rownorm_set_override(rownorm_op op, int lanes_per_row, int packs_per_lane,
+                                int block_threads, int blocks_per_cu) {
+  if ((int)op < 0 || (int)op >= ROWNORM_OP_COUNT) return ROWNORM_ERR_SHAPE;
+  Override o;
+  o.G = lanes_per_row;
+  o.V = packs_per_lane;
+  o.block = block_threads;
+  o.bpc = blocks_per_cu;
+  g_override[(int)op] = o;
+  return 0;
+}
+
+}  // extern "C"

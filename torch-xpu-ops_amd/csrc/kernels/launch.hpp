@@ -1,0 +1,91 @@
+// Typed launch entry points shared by the per-dtype translation units and the
+// C ABI file.  Each launch_* template is defined in *_launch.hpp and explicitly
+// instantiated in one of the *.hip files, so the kernels compile in parallel.
+#pragma once
+#include <hip/hip_runtime.h>
+#include <stdint.h>
+#include "device/pack.hpp"
+#include "plan.hpp"
+
+namespace rownorm {
+
+struct NormFwdArgs {
+  const void* x;
+  const void* gamma;
+  const void* beta;
+  void* y;
+  float* mean;
+  float* rstd;
+  int64_t M;
+  int N;
+  float eps;
+};
+
+struct NormBwdArgs {
+  const void* dy;
+  const void* x;
+  const float* mean;
+  const float* rstd;
+  const void* gamma;
+  void* dx;
+  void* dgamma;
+  void* dbeta;
+  float* part_dg;  // [plan.partial_rows, N] fp32, or null when no column sums are wanted
+  float* part_db;
+  int64_t M;
+  int N;
+};
+
+struct SoftmaxFwdArgs {
+  const void* x;
+  void* y;
+  int64_t M;
+  int N;
+  int is_log;
+};
+
+struct SoftmaxBwdArgs {
+  const void* grad;
+  const void* y;
+  void* gi;
+  int64_t M;
+  int N;
+  int is_log;
+};
+
+// All return 0 or a hipError_t value.
+template <class T, class WT, bool RMS>
+int launch_norm_fwd(const Plan& plan, const NormFwdArgs& a, hipStream_t stream);
+template <class T, class WT, bool RMS>
+int launch_norm_bwd(const Plan& plan, const NormBwdArgs& a, hipStream_t stream);
+template <class TI, class TO>
+int launch_softmax_fwd(const Plan& plan, const SoftmaxFwdArgs& a, hipStream_t stream);
+template <class TG, class TO>
+int launch_softmax_bwd(const Plan& plan, const SoftmaxBwdArgs& a, hipStream_t stream);
+
+// Compile-time walk over every (G, V, BLOCK) a kernel family may be built for;
+// L<G, V, BLOCK>::run(ctx) returns true when it matched the plan and launched.
+template <int... Is>
+struct ilist {};
+using GList = ilist<8, 16, 32, 64, 128, 256, 512, 1024>;
+using VList = ilist<1, 2, 4, 8, 16>;
+using BList = ilist<256, 512, 1024>;
+
+template <template <int, int, int> class L, class Ctx, int G, int V, int... Bs>
+inline bool try_blocks(const Ctx& c, ilist<Bs...>) {
+  return (L<G, V, Bs>::run(c) || ...);
+}
+template <template <int, int, int> class L, class Ctx, int G, int... Vs>
+inline bool try_packs(const Ctx& c, ilist<Vs...>) {
+  return (try_blocks<L, Ctx, G, Vs>(c, BList{}) || ...);
+}
+template <template <int, int, int> class L, class Ctx, int... Gs>
+inline bool try_lanes(const Ctx& c, ilist<Gs...>) {
+  return (try_packs<L, Ctx, Gs>(c, VList{}) || ...);
+}
+template <template <int, int, int> class L, class Ctx>
+inline bool launch_variant(const Ctx& c) {
+  return try_lanes<L, Ctx>(c, GList{});
+}
+
+}  // namespace rownorm

@@ -1,0 +1,6 @@
+// LayerNorm / RMSNorm fwd kernels, rows bf16, weights bf16.
+#include "norm_launch.hpp"
+namespace rownorm {
+template int launch_norm_fwd<bf16, bf16, false>(const Plan&, const NormFwdArgs&, hipStream_t);
+template int launch_norm_fwd<bf16, bf16, true>(const Plan&, const NormFwdArgs&, hipStream_t);
+}  // namespace rownorm

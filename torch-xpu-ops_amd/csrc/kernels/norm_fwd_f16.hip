@@ -1,0 +1,6 @@
+// LayerNorm / RMSNorm fwd kernels, rows f16, weights f16.
+#include "norm_launch.hpp"
+namespace rownorm {
+template int launch_norm_fwd<f16, f16, false>(const Plan&, const NormFwdArgs&, hipStream_t);
+template int launch_norm_fwd<f16, f16, true>(const Plan&, const NormFwdArgs&, hipStream_t);
+}  // namespace rownorm

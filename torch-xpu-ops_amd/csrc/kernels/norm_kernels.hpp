@@ -1,0 +1,522 @@
+// LayerNorm / RMSNorm forward and backward kernels for gfx950 (wave64).
+//
+// Layout of one call: the input is a dense [M, N] matrix.  G lanes share one
+// row; lane l of the group owns the 16-byte packs number l, l+G, l+2G, ...
+// (V of them), so each wave-wide access covers one contiguous kilobyte.  A
+// workgroup of BLOCK threads handles BLOCK/G rows per iteration and strides
+// over the rows persistently, which lets the per-column quantities (gamma,
+// beta, and in the backward pass the dgamma/dbeta partial sums) stay in
+// registers from the first row to the last.
+//
+// What these kernels stand in for in the reference (the arithmetic, not the
+// code shape):
+//   forward   VectorizedLayerNormKernelFunctor + compute_stats,
+//             src/ATen/native/xpu/sycl/LayerNormKernels.cpp:394-586, and the
+//             scalar pair RowwiseMomentsFunctor / LayerNormForwardKernelFunctor
+//             (:203-320) used for unaligned pointers or N % 4 != 0;
+//   backward  FusedNormKernelFunctor (src/ATen/native/xpu/sycl/Norm.h:485-526)
+//             with LayerNormBackward::reduce_combine/update
+//             (LayerNormKernels.cpp:86-186) for dX, and
+//             GammaBetaBackwardSimpleKernelFunctor (:885-1024) /
+//             GammaBetaReduceFunctor (:709-874) + at::sum (:1312-1314) for
+//             dgamma/dbeta.
+// Differences by design: X and dY are read once (the reference reads them
+// twice for dX and a third time for dgamma/dbeta); the column partial sums
+// are fp32 whatever the weight dtype; every access is 128 bits wide for any
+// pointer alignment; the weight dtype is independent of the row dtype.
+#pragma once
+#include "device/pack.hpp"
+#include "device/reduce.hpp"
+
+namespace rownorm {
+
+template <int G>
+struct block_for {
+  static constexpr int value = G <= 256 ? 256 : G;
+};
+
+// ---------------------------------------------------------------------------
+// Forward, row resident in registers: one read of X, one write of Y.
+//
+// LayerNorm statistics: mean0 = sum(x)/N, then the centred sums
+// s1 = sum(x - mean0), s2 = sum((x - mean0)^2) over the registers give
+// mean = mean0 + s1/N and var = (s2 - s1*s1/N)/N.  On a constant row the
+// correction cancels the rounding of mean0 exactly, so mean is the constant
+// and y is beta bit for bit, which is what the CPU kernel's Welford pass gives
+// (Welford recurrence being followed: src/ATen/native/xpu/sycl/
+// SharedReduceOps.h:56-88).
+template <class T, class WT, int G, int V, int BLOCK, bool RMS>
+__global__ void __launch_bounds__(BLOCK)
+norm_fwd_resident_kernel(const T* __restrict__ x, const WT* __restrict__ gamma,
+                         const WT* __restrict__ beta, T* __restrict__ y,
+                         float* __restrict__ mean, float* __restrict__ rstd, int64_t M, int N,
+                         float eps) {
+  constexpr int E = elems_per_pack<T>::value;
+  constexpr int RPB = BLOCK / G;
+  __shared__ float red[reduce_lds_floats<G, BLOCK, 2>::value];
+  int phase = 0;
+  const int slot = threadIdx.x / G;
+  const int lane = threadIdx.x % G;
+  const float fN = (float)N;
+
+  float gam[V][E];
+  float bet[RMS ? 1 : V][RMS ? 1 : E];
+#pragma unroll
+  for (int c = 0; c < V; ++c) {
+    const int e0 = (c * G + lane) * E;
+    Pack<WT, E> pg = gamma ? load_row_pack<WT, E, false>(gamma, e0, N, true, 1.0f)
+                           : Pack<WT, E>::splat(1.0f);
+#pragma unroll
+    for (int i = 0; i < E; ++i) gam[c][i] = pg.get(i);
+    if constexpr (!RMS) {
+      Pack<WT, E> pb = beta ? load_row_pack<WT, E, false>(beta, e0, N, true, 0.0f)
+                            : Pack<WT, E>::zero();
+#pragma unroll
+      for (int i = 0; i < E; ++i) bet[c][i] = pb.get(i);
+    }
+  }
+
+  const int64_t nrb = (M + RPB - 1) / RPB;
+  for (int64_t rb = blockIdx.x; rb < nrb; rb += gridDim.x) {
+    const int64_t row = rb * RPB + slot;
+    const bool ok = row < M;
+    const T* xr = x + row * (int64_t)N;
+    T* yr = y + row * (int64_t)N;
+
+    float xf[V][E];
+#pragma unroll
+    for (int c = 0; c < V; ++c) {
+      const int e0 = (c * G + lane) * E;
+      const Pack<T, E> p = load_row_pack<T, E, true>(xr, e0, N, ok, 0.0f);
+#pragma unroll
+      for (int i = 0; i < E; ++i) xf[c][i] = p.get(i);
+    }
+
+    float mu = 0.0f, rs;
+    if constexpr (RMS) {
+      float acc[1] = {0.0f};
+#pragma unroll
+      for (int c = 0; c < V; ++c)
+#pragma unroll
+        for (int i = 0; i < E; ++i) acc[0] = fmaf(xf[c][i], xf[c][i], acc[0]);
+      group_allreduce<G, BLOCK, 1, SumOp>(acc, red, phase);
+      rs = 1.0f / sqrtf(acc[0] / fN + eps);
+    } else {
+      float acc0[1] = {0.0f};
+#pragma unroll
+      for (int c = 0; c < V; ++c)
+#pragma unroll
+        for (int i = 0; i < E; ++i) acc0[0] += xf[c][i];
+      group_allreduce<G, BLOCK, 1, SumOp>(acc0, red, phase);
+      const float mean0 = acc0[0] / fN;
+      float acc[2] = {0.0f, 0.0f};
+#pragma unroll
+      for (int c = 0; c < V; ++c) {
+        const int e0 = (c * G + lane) * E;
+        const int nvalid = ok ? N - e0 : 0;  // elements of this pack inside the row
+#pragma unroll
+        for (int i = 0; i < E; ++i) {
+          const float d = (i < nvalid) ? xf[c][i] - mean0 : 0.0f;
+          acc[0] += d;
+          acc[1] = fmaf(d, d, acc[1]);
+        }
+      }
+      group_allreduce<G, BLOCK, 2, SumOp>(acc, red, phase);
+      const float m1 = acc[0] / fN;
+      mu = mean0 + m1;
+      const float var = fmaxf((acc[1] - acc[0] * m1) / fN, 0.0f);
+      rs = 1.0f / sqrtf(var + eps);
+    }
+
+#pragma unroll
+    for (int c = 0; c < V; ++c) {
+      const int e0 = (c * G + lane) * E;
+      Pack<T, E> o;
+#pragma unroll
+      for (int i = 0; i < E; ++i) {
+        float v;
+        if constexpr (RMS)
+          v = (xf[c][i] * rs) * gam[c][i];
+        else
+          v = ((xf[c][i] - mu) * rs) * gam[c][i] + bet[c][i];
+        o.set(i, v);
+      }
+      store_row_pack<T, E, true>(yr, e0, N, ok, o);
+    }
+    if (ok && lane == 0) {
+      if constexpr (!RMS)
+        if (mean) mean[row] = mu;
+      if (rstd) rstd[row] = rs;
+    }
+  }
+}
+
+// ---------------------------------------------------------------------------
+// Forward for rows too wide to hold in registers: one workgroup per row, the
+// row is streamed from memory three times (sum, centred sums, normalize); the
+// second and third pass hit L2 / Infinity Cache for any realistic row.
+template <class T, class WT, int BLOCK, bool RMS>
+__global__ void __launch_bounds__(BLOCK)
+norm_fwd_stream_kernel(const T* __restrict__ x, const WT* __restrict__ gamma,
+                       const WT* __restrict__ beta, T* __restrict__ y,
+                       float* __restrict__ mean, float* __restrict__ rstd, int64_t M, int N,
+                       float eps) {
+  constexpr int E = elems_per_pack<T>::value;
+  __shared__ float red[reduce_lds_floats<BLOCK, BLOCK, 2>::value];
+  int phase = 0;
+  const float fN = (float)N;
+  const int npacks = (N + E - 1) / E;
+  for (int64_t row = blockIdx.x; row < M; row += gridDim.x) {
+    const T* xr = x + row * (int64_t)N;
+    T* yr = y + row * (int64_t)N;
+    float mu = 0.0f, rs;
+    if constexpr (RMS) {
+      float acc[1] = {0.0f};
+      for (int pk = threadIdx.x; pk < npacks; pk += BLOCK) {
+        const Pack<T, E> p = load_row_pack<T, E, false>(xr, pk * E, N, true, 0.0f);
+#pragma unroll
+        for (int i = 0; i < E; ++i) acc[0] = fmaf(p.get(i), p.get(i), acc[0]);
+      }
+      group_allreduce<BLOCK, BLOCK, 1, SumOp>(acc, red, phase);
+      rs = 1.0f / sqrtf(acc[0] / fN + eps);
+    } else {
+      float acc0[1] = {0.0f};
+      for (int pk = threadIdx.x; pk < npacks; pk += BLOCK) {
+        const Pack<T, E> p = load_row_pack<T, E, false>(xr, pk * E, N, true, 0.0f);
+#pragma unroll
+        for (int i = 0; i < E; ++i) acc0[0] += p.get(i);
+      }
+      group_allreduce<BLOCK, BLOCK, 1, SumOp>(acc0, red, phase);
+      const float mean0 = acc0[0] / fN;
+      float acc[2] = {0.0f, 0.0f};
+      for (int pk = threadIdx.x; pk < npacks; pk += BLOCK) {
+        const Pack<T, E> p = load_row_pack<T, E, false>(xr, pk * E, N, true, 0.0f);
+        const int nvalid = N - pk * E;
+#pragma unroll
+        for (int i = 0; i < E; ++i) {
+          const float d = (i < nvalid) ? p.get(i) - mean0 : 0.0f;
+          acc[0] += d;
+          acc[1] = fmaf(d, d, acc[1]);
+        }
+      }
+      group_allreduce<BLOCK, BLOCK, 2, SumOp>(acc, red, phase);
+      const float m1 = acc[0] / fN;
+      mu = mean0 + m1;
+      const float var = fmaxf((acc[1] - acc[0] * m1) / fN, 0.0f);
+      rs = 1.0f / sqrtf(var + eps);
+    }
+    for (int pk = threadIdx.x; pk < npacks; pk += BLOCK) {
+      const int e0 = pk * E;
+      const Pack<T, E> p = load_row_pack<T, E, true>(xr, e0, N, true, 0.0f);
+      const Pack<WT, E> pg = gamma ? load_row_pack<WT, E, false>(gamma, e0, N, true, 1.0f)
+                                   : Pack<WT, E>::splat(1.0f);
+      Pack<WT, E> pb = Pack<WT, E>::zero();
+      if constexpr (!RMS)
+        if (beta) pb = load_row_pack<WT, E, false>(beta, e0, N, true, 0.0f);
+      Pack<T, E> o;
+#pragma unroll
+      for (int i = 0; i < E; ++i) {
+        float v;
+        if constexpr (RMS)
+          v = (p.get(i) * rs) * pg.get(i);
+        else
+          v = ((p.get(i) - mu) * rs) * pg.get(i) + pb.get(i);
+        o.set(i, v);
+      }
+      store_row_pack<T, E, true>(yr, e0, N, true, o);
+    }
+    if (threadIdx.x == 0) {
+      if constexpr (!RMS)
+        if (mean) mean[row] = mu;
+      if (rstd) rstd[row] = rs;
+    }
+  }
+}
+
+// ---------------------------------------------------------------------------
+// Backward, rows resident in registers: X and dY are read once, dX written
+// once, and each lane keeps the dgamma/dbeta sums of its own columns in fp32
+// registers over all the rows its workgroup visits.  At the end the BLOCK/G
+// row slots of the workgroup are folded together through LDS in a fixed order
+// and one fp32 row per workgroup goes to the [gridDim.x, N] partial buffers;
+// colsum_finalize_kernel adds those up.
+//
+//   s1 = sum dy*gamma            s2 = sum dy*gamma*xhat       xhat = (x-mean)*rstd
+//   dx = (rstd/N) * (N*gamma*dy - xhat*s2 - s1)               (RMS: mean = 0, no s1)
+//   dgamma[j] = sum_rows dy*xhat   dbeta[j] = sum_rows dy
+template <class T, class WT, int G, int V, int BLOCK, bool RMS>
+__global__ void __launch_bounds__(BLOCK)
+norm_bwd_resident_kernel(const T* __restrict__ dy, const T* __restrict__ x,
+                         const float* __restrict__ mean, const float* __restrict__ rstd,
+                         const WT* __restrict__ gamma, T* __restrict__ dx,
+                         float* __restrict__ part_dg, float* __restrict__ part_db, int64_t M,
+                         int N) {
+  constexpr int E = elems_per_pack<T>::value;
+  constexpr int RPB = BLOCK / G;
+  constexpr int FOLD_FLOATS = (RPB > 1) ? G * V * E : 1;
+  __shared__ float red[reduce_lds_floats<G, BLOCK, 2>::value];
+  __shared__ float fold[FOLD_FLOATS];
+  int phase = 0;
+  const int slot = threadIdx.x / G;
+  const int lane = threadIdx.x % G;
+  const float fN = (float)N;
+  const bool want_cols = part_dg != nullptr;  // uniform
+
+  float gam[V][E];
+  float dg[V][E];
+  float db[RMS ? 1 : V][RMS ? 1 : E];
+#pragma unroll
+  for (int c = 0; c < V; ++c) {
+    const int e0 = (c * G + lane) * E;
+    Pack<WT, E> pg = gamma ? load_row_pack<WT, E, false>(gamma, e0, N, true, 1.0f)
+                           : Pack<WT, E>::splat(1.0f);
+#pragma unroll
+    for (int i = 0; i < E; ++i) {
+      gam[c][i] = pg.get(i);
+      dg[c][i] = 0.0f;
+      if constexpr (!RMS) db[c][i] = 0.0f;
+    }
+  }
+
+  const int64_t nrb = (M + RPB - 1) / RPB;
+  for (int64_t rb = blockIdx.x; rb < nrb; rb += gridDim.x) {
+    const int64_t row = rb * RPB + slot;
+    const bool ok = row < M;
+    const T* xr = x + row * (int64_t)N;
+    const T* gr = dy + row * (int64_t)N;
+    float mu = 0.0f;
+    if constexpr (!RMS) mu = ok ? mean[row] : 0.0f;
+    const float rs = ok ? rstd[row] : 0.0f;
+
+    float xh[V][E];  // xhat
+    float gy[V][E];  // dy
+#pragma unroll
+    for (int c = 0; c < V; ++c) {
+      const int e0 = (c * G + lane) * E;
+      const Pack<T, E> px = load_row_pack<T, E, true>(xr, e0, N, ok, 0.0f);
+      const Pack<T, E> pd = load_row_pack<T, E, true>(gr, e0, N, ok, 0.0f);
+#pragma unroll
+      for (int i = 0; i < E; ++i) {
+        xh[c][i] = RMS ? px.get(i) * rs : (px.get(i) - mu) * rs;
+        gy[c][i] = pd.get(i);
+      }
+    }
+    float acc[2] = {0.0f, 0.0f};
+#pragma unroll
+    for (int c = 0; c < V; ++c)
+#pragma unroll
+      for (int i = 0; i < E; ++i) {
+        const float g = gy[c][i] * gam[c][i];
+        if constexpr (!RMS) acc[0] += g;
+        acc[1] = fmaf(g, xh[c][i], acc[1]);
+        dg[c][i] = fmaf(gy[c][i], xh[c][i], dg[c][i]);
+        if constexpr (!RMS) db[c][i] += gy[c][i];
+      }
+    group_allreduce<G, BLOCK, 2, SumOp>(acc, red, phase);
+    if (dx != nullptr) {
+      T* dr = dx + row * (int64_t)N;
+      const float term1 = rs / fN;
+#pragma unroll
+      for (int c = 0; c < V; ++c) {
+        const int e0 = (c * G + lane) * E;
+        Pack<T, E> o;
+#pragma unroll
+        for (int i = 0; i < E; ++i) {
+          float f = fN * (gy[c][i] * gam[c][i]);
+          f -= xh[c][i] * acc[1];
+          if constexpr (!RMS) f -= acc[0];
+          o.set(i, f * term1);
+        }
+        store_row_pack<T, E, true>(dr, e0, N, ok, o);
+      }
+    }
+  }
+
+  if (!want_cols) return;
+  // Fold the row slots that own the same columns, then emit one partial row.
+  float* out_g = part_dg + (int64_t)blockIdx.x * N;
+  float* out_b = RMS ? nullptr : part_db + (int64_t)blockIdx.x * N;
+  if constexpr (RPB == 1) {
+#pragma unroll
+    for (int c = 0; c < V; ++c) {
+      const int e0 = (c * G + lane) * E;
+      Pack<float, E> pg, pb;
+#pragma unroll
+      for (int i = 0; i < E; ++i) {
+        pg.set(i, dg[c][i]);
+        if constexpr (!RMS) pb.set(i, db[c][i]);
+      }
+      store_row_pack<float, E, false>(out_g, e0, N, true, pg);
+      if constexpr (!RMS) store_row_pack<float, E, false>(out_b, e0, N, true, pb);
+    }
+  } else {
+    constexpr int NPASS = RMS ? 1 : 2;
+#pragma unroll
+    for (int pass = 0; pass < NPASS; ++pass) {
+      // Row slots inside one wavefront (G < 64) are folded with shuffles first.
+      if constexpr (G < 64) {
+#pragma unroll
+        for (int c = 0; c < V; ++c)
+#pragma unroll
+          for (int i = 0; i < E; ++i) {
+            float v = pass == 0 ? dg[c][i] : db[RMS ? 0 : c][RMS ? 0 : i];
+#pragma unroll
+            for (int off = G; off < 64; off <<= 1) v += __shfl_xor(v, off, 64);
+            if (pass == 0)
+              dg[c][i] = v;
+            else
+              db[RMS ? 0 : c][RMS ? 0 : i] = v;
+          }
+      }
+      constexpr int UNIT = G < 64 ? 64 : G;         // threads per fold unit
+      constexpr int NUNIT = BLOCK / UNIT;           // units folded through LDS, in order
+      const int unit = threadIdx.x / UNIT;
+      const bool owner = (threadIdx.x % UNIT) < G;  // one lane group per unit holds the sums
+#pragma unroll 1
+      for (int u = 0; u < NUNIT; ++u) {
+        if (unit == u && owner) {
+#pragma unroll
+          for (int c = 0; c < V; ++c) {
+            const int e0 = (c * G + lane) * E;
+#pragma unroll
+            for (int i = 0; i < E; ++i) {
+              const float v = pass == 0 ? dg[c][i] : db[RMS ? 0 : c][RMS ? 0 : i];
+              fold[e0 + i] = (u == 0) ? v : fold[e0 + i] + v;
+            }
+          }
+        }
+        __syncthreads();
+      }
+      float* out = pass == 0 ? out_g : out_b;
+      for (int j = threadIdx.x; j < N; j += BLOCK) out[j] = fold[j];
+      __syncthreads();
+    }
+  }
+}
+
+// ---------------------------------------------------------------------------
+// Backward dX for rows too wide for registers: one workgroup per row, two
+// streaming passes over X and dY (sums, then dX).
+template <class T, class WT, int BLOCK, bool RMS>
+__global__ void __launch_bounds__(BLOCK)
+norm_bwd_stream_dx_kernel(const T* __restrict__ dy, const T* __restrict__ x,
+                          const float* __restrict__ mean, const float* __restrict__ rstd,
+                          const WT* __restrict__ gamma, T* __restrict__ dx, int64_t M, int N) {
+  constexpr int E = elems_per_pack<T>::value;
+  __shared__ float red[reduce_lds_floats<BLOCK, BLOCK, 2>::value];
+  int phase = 0;
+  const float fN = (float)N;
+  const int npacks = (N + E - 1) / E;
+  for (int64_t row = blockIdx.x; row < M; row += gridDim.x) {
+    const T* xr = x + row * (int64_t)N;
+    const T* gr = dy + row * (int64_t)N;
+    T* dr = dx + row * (int64_t)N;
+    const float mu = RMS ? 0.0f : mean[row];
+    const float rs = rstd[row];
+    float acc[2] = {0.0f, 0.0f};
+    for (int pk = threadIdx.x; pk < npacks; pk += BLOCK) {
+      const int e0 = pk * E;
+      const Pack<T, E> px = load_row_pack<T, E, false>(xr, e0, N, true, 0.0f);
+      const Pack<T, E> pd = load_row_pack<T, E, false>(gr, e0, N, true, 0.0f);
+      const Pack<WT, E> pg = gamma ? load_row_pack<WT, E, false>(gamma, e0, N, true, 1.0f)
+                                   : Pack<WT, E>::splat(1.0f);
+#pragma unroll
+      for (int i = 0; i < E; ++i) {
+        const float g = pd.get(i) * pg.get(i);
+        acc[0] += g;
+        acc[1] = fmaf(g, (px.get(i) - mu) * rs, acc[1]);
+      }
+    }
+    group_allreduce<BLOCK, BLOCK, 2, SumOp>(acc, red, phase);
+    const float term1 = rs / fN;
+    for (int pk = threadIdx.x; pk < npacks; pk += BLOCK) {
+      const int e0 = pk * E;
+      const Pack<T, E> px = load_row_pack<T, E, true>(xr, e0, N, true, 0.0f);
+      const Pack<T, E> pd = load_row_pack<T, E, true>(gr, e0, N, true, 0.0f);
+      const Pack<WT, E> pg = gamma ? load_row_pack<WT, E, false>(gamma, e0, N, true, 1.0f)
+                                   : Pack<WT, E>::splat(1.0f);
+      Pack<T, E> o;
+#pragma unroll
+      for (int i = 0; i < E; ++i) {
+        float f = fN * (pd.get(i) * pg.get(i));
+        f -= ((px.get(i) - mu) * rs) * acc[1];
+        if constexpr (!RMS) f -= acc[0];
+        o.set(i, f * term1);
+      }
+      store_row_pack<T, E, true>(dr, e0, N, true, o);
+    }
+  }
+}
+
+// Column sums for rows too wide for registers: workgroup (bx, by) owns the
+// BLOCK*E columns starting at bx*BLOCK*E and the rows by, by+gridDim.y, ...;
+// it writes row `by` of the [gridDim.y, N] partial buffers.
+template <class T, int BLOCK, bool RMS>
+__global__ void __launch_bounds__(BLOCK)
+norm_bwd_stream_colsum_kernel(const T* __restrict__ dy, const T* __restrict__ x,
+                              const float* __restrict__ mean, const float* __restrict__ rstd,
+                              float* __restrict__ part_dg, float* __restrict__ part_db,
+                              int64_t M, int N) {
+  constexpr int E = elems_per_pack<T>::value;
+  const int e0 = (blockIdx.x * BLOCK + threadIdx.x) * E;
+  float dg[E], db[E];
+#pragma unroll
+  for (int i = 0; i < E; ++i) dg[i] = db[i] = 0.0f;
+  for (int64_t row = blockIdx.y; row < M; row += gridDim.y) {
+    const float mu = RMS ? 0.0f : mean[row];
+    const float rs = rstd[row];
+    const Pack<T, E> px = load_row_pack<T, E, false>(x + row * (int64_t)N, e0, N, true, 0.0f);
+    const Pack<T, E> pd = load_row_pack<T, E, false>(dy + row * (int64_t)N, e0, N, true, 0.0f);
+#pragma unroll
+    for (int i = 0; i < E; ++i) {
+      dg[i] = fmaf(pd.get(i), (px.get(i) - mu) * rs, dg[i]);
+      db[i] += pd.get(i);
+    }
+  }
+#pragma unroll
+  for (int i = 0; i < E; ++i)
+    if (e0 + i < N) {
+      part_dg[(int64_t)blockIdx.y * N + e0 + i] = dg[i];
+      if constexpr (!RMS) part_db[(int64_t)blockIdx.y * N + e0 + i] = db[i];
+    }
+}
+
+// ---------------------------------------------------------------------------
+// Second stage of the dgamma/dbeta reduction: out[j] = sum_p part[p][j], rows
+// added in a fixed order.  A workgroup of 256 threads covers 64 columns with
+// 4 row lanes per column... see COLS/ROWS below: COLS threads across (4-byte
+// coalesced), ROWS threads down, LDS tree over the ROWS partial sums.
+// blockIdx.y selects dgamma (0) or dbeta (1).
+template <class WT>
+__global__ void __launch_bounds__(256)
+colsum_finalize_kernel(const float* __restrict__ part0, const float* __restrict__ part1,
+                       WT* __restrict__ out0, WT* __restrict__ out1, int P, int N) {
+  constexpr int COLS = 32, ROWS = 8;
+  __shared__ float tile[ROWS][COLS + 1];
+  const float* part = blockIdx.y == 0 ? part0 : part1;
+  WT* out = blockIdx.y == 0 ? out0 : out1;
+  if (part == nullptr || out == nullptr) return;  // uniform per workgroup
+  const int cx = threadIdx.x % COLS, ry = threadIdx.x / COLS;
+  const int col = blockIdx.x * COLS + cx;
+  float a0 = 0.0f, a1 = 0.0f, a2 = 0.0f, a3 = 0.0f;
+  if (col < N) {
+    int p = ry;
+    for (; p + 3 * ROWS < P; p += 4 * ROWS) {
+      a0 += part[(int64_t)p * N + col];
+      a1 += part[(int64_t)(p + ROWS) * N + col];
+      a2 += part[(int64_t)(p + 2 * ROWS) * N + col];
+      a3 += part[(int64_t)(p + 3 * ROWS) * N + col];
+    }
+    for (; p < P; p += ROWS) a0 += part[(int64_t)p * N + col];
+  }
+  tile[ry][cx] = (a0 + a1) + (a2 + a3);
+  __syncthreads();
+  if (ry == 0 && col < N) {
+    float s = tile[0][cx];
+#pragma unroll
+    for (int r = 1; r < ROWS; ++r) s += tile[r][cx];
+    out[col] = (WT)s;
+  }
+}
+
+}  // namespace rownorm

@@ -1,0 +1,111 @@
+// Host dispatch of the LayerNorm / RMSNorm kernels: plan -> template instance.
+#pragma once
+#include "launch.hpp"
+#include "norm_kernels.hpp"
+
+namespace rownorm {
+
+template <class T, class WT, bool RMS>
+struct NormFwdCtx {
+  const Plan& plan;
+  const NormFwdArgs& a;
+  hipStream_t stream;
+};
+
+template <class T, class WT, bool RMS>
+struct NormFwdLauncher {
+  template <int G, int V, int BLOCK>
+  struct At {
+    static bool run(const NormFwdCtx<T, WT, RMS>& c) {
+      if constexpr (variant_built(OC_NORM_FWD, sizeof(T), G, V) &&
+                    block_built(OC_NORM_FWD, G, BLOCK)) {
+        if (c.plan.G == G && c.plan.V == V && c.plan.block == BLOCK) {
+          hipLaunchKernelGGL((norm_fwd_resident_kernel<T, WT, G, V, BLOCK, RMS>),
+                             dim3((unsigned)c.plan.grid), dim3(BLOCK), 0, c.stream,
+                             (const T*)c.a.x, (const WT*)c.a.gamma, (const WT*)c.a.beta,
+                             (T*)c.a.y, c.a.mean, c.a.rstd, c.a.M, c.a.N, c.a.eps);
+          return true;
+        }
+      }
+      return false;
+    }
+  };
+};
+
+template <class T, class WT, bool RMS>
+int launch_norm_fwd(const Plan& plan, const NormFwdArgs& a, hipStream_t stream) {
+  if (plan.resident) {
+    NormFwdCtx<T, WT, RMS> ctx{plan, a, stream};
+    if (!launch_variant<NormFwdLauncher<T, WT, RMS>::template At>(ctx))
+      return (int)hipErrorInvalidConfiguration;
+  } else {
+    hipLaunchKernelGGL((norm_fwd_stream_kernel<T, WT, kStreamBlock, RMS>),
+                       dim3((unsigned)plan.grid), dim3(kStreamBlock), 0, stream, (const T*)a.x,
+                       (const WT*)a.gamma, (const WT*)a.beta, (T*)a.y, a.mean, a.rstd, a.M, a.N,
+                       a.eps);
+  }
+  return (int)hipGetLastError();
+}
+
+template <class T, class WT, bool RMS>
+struct NormBwdCtx {
+  const Plan& plan;
+  const NormBwdArgs& a;
+  hipStream_t stream;
+};
+
+template <class T, class WT, bool RMS>
+struct NormBwdLauncher {
+  template <int G, int V, int BLOCK>
+  struct At {
+    static bool run(const NormBwdCtx<T, WT, RMS>& c) {
+      if constexpr (variant_built(OC_NORM_BWD, sizeof(T), G, V) &&
+                    block_built(OC_NORM_BWD, G, BLOCK)) {
+        if (c.plan.G == G && c.plan.V == V && c.plan.block == BLOCK) {
+          hipLaunchKernelGGL((norm_bwd_resident_kernel<T, WT, G, V, BLOCK, RMS>),
+                             dim3((unsigned)c.plan.grid), dim3(BLOCK), 0, c.stream,
+                             (const T*)c.a.dy, (const T*)c.a.x, c.a.mean, c.a.rstd,
+                             (const WT*)c.a.gamma, (T*)c.a.dx, c.a.part_dg, c.a.part_db, c.a.M,
+                             c.a.N);
+          return true;
+        }
+      }
+      return false;
+    }
+  };
+};
+
+template <class T, class WT, bool RMS>
+int launch_norm_bwd(const Plan& plan, const NormBwdArgs& a, hipStream_t stream) {
+  const bool want_cols = a.part_dg != nullptr;
+  if (plan.resident) {
+    NormBwdCtx<T, WT, RMS> ctx{plan, a, stream};
+    if (!launch_variant<NormBwdLauncher<T, WT, RMS>::template At>(ctx))
+      return (int)hipErrorInvalidConfiguration;
+  } else {
+    constexpr int E = elems_per_pack<T>::value;
+    if (a.dx != nullptr) {
+      hipLaunchKernelGGL((norm_bwd_stream_dx_kernel<T, WT, kStreamBlock, RMS>),
+                         dim3((unsigned)plan.grid), dim3(kStreamBlock), 0, stream,
+                         (const T*)a.dy, (const T*)a.x, a.mean, a.rstd, (const WT*)a.gamma,
+                         (T*)a.dx, a.M, a.N);
+    }
+    if (want_cols) {
+      constexpr int CB = 256;
+      const unsigned gx = (unsigned)((a.N + CB * E - 1) / (CB * E));
+      hipLaunchKernelGGL((norm_bwd_stream_colsum_kernel<T, CB, RMS>),
+                         dim3(gx, (unsigned)plan.partial_rows), dim3(CB), 0, stream,
+                         (const T*)a.dy, (const T*)a.x, a.mean, a.rstd, a.part_dg, a.part_db,
+                         a.M, a.N);
+    }
+  }
+  int err = (int)hipGetLastError();
+  if (err != 0 || !want_cols) return err;
+  const unsigned gx = (unsigned)((a.N + 31) / 32);
+  hipLaunchKernelGGL((colsum_finalize_kernel<WT>), dim3(gx, RMS ? 1 : 2), dim3(256), 0, stream,
+                     (const float*)a.part_dg, (const float*)a.part_db, (WT*)a.dgamma,
+                     (WT*)a.dbeta, (int)plan.partial_rows, a.N);
+  return (int)hipGetLastError();
+}
+
+}  // namespace rownorm

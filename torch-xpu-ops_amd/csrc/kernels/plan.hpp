@@ -1,0 +1,171 @@
+// Host-side choice of the launch layout for one call (no HIP types in here).
+//
+// Stands in for the reference's work-split heuristics: NormConfig
+// (src/ATen/native/xpu/sycl/Norm.h:225-370), layer_norm_wg_size_select
+// (LayerNormKernels.cpp:588-616) and get_wgroup_size (SoftMaxKernels.cpp:
+// 139-182).  Those are written around Intel EU counts and SIMD32 sub-groups;
+// here the split is a small table over the row size for 256 compute units of
+// 64-wide wavefronts.
+//
+// The rule.  A row of N elements is ceil(N / E) 16-byte packs (E = 4 for fp32,
+// 8 for 16-bit types).  G lanes share a row and each holds V packs:
+//   G = smallest power of two in [8, 1024] with G * V_pref >= packs,
+//   V = smallest power of two with G * V >= packs.
+// If V exceeds the per-op register budget V_max the multi-pass streaming
+// kernel is used instead.  Workgroups are 256 threads (BLOCK/G rows each) or G
+// threads when G > 256; the grid is persistent: min(row blocks, CUs * k).
+#pragma once
+#include <stdint.h>
+
+namespace rownorm {
+
+enum OpClass { OC_NORM_FWD = 0, OC_NORM_BWD = 1, OC_SOFTMAX_FWD = 2, OC_SOFTMAX_BWD = 3 };
+
+struct Override {
+  int G = 0, V = 0, block = 0, bpc = 0;  // 0 = automatic; G = -1 = force the streaming kernel
+};
+
+struct Plan {
+  bool resident = true;
+  int G = 0, V = 0, block = 0, rpb = 0;
+  int64_t grid = 0;
+  int64_t partial_rows = 0;
+};
+
+constexpr int kMinG = 8;
+constexpr int kMaxG = 1024;
+constexpr int kMaxV = 16;
+constexpr int kStreamBlock = 1024;
+
+// Preferred packs per lane: what the G ladder aims for.
+constexpr int v_pref(OpClass oc, int esize) {
+  switch (oc) {
+    case OC_NORM_FWD: return esize == 4 ? 8 : 8;
+    case OC_NORM_BWD: return esize == 4 ? 4 : 2;
+    case OC_SOFTMAX_FWD: return esize == 4 ? 8 : 4;
+    case OC_SOFTMAX_BWD: return esize == 4 ? 4 : 4;
+  }
+  return 1;
+}
+
+// Largest packs per lane the register file holds for a G-lane row group.
+// G = 1024 means 16 wavefronts per workgroup, i.e. at most 128 VGPRs a lane.
+constexpr int v_max(OpClass oc, int esize, int G) {
+  int v = 1;
+  switch (oc) {
+    case OC_NORM_FWD: v = esize == 4 ? 16 : 8; break;
+    case OC_NORM_BWD: v = esize == 4 ? 8 : 4; break;
+    case OC_SOFTMAX_FWD: v = esize == 4 ? 16 : 8; break;
+    case OC_SOFTMAX_BWD: v = esize == 4 ? 16 : 8; break;
+  }
+  if (G >= 1024 && v > 1) v /= 2;
+  return v;
+}
+
+constexpr int block_threads(OpClass, int G) { return G <= 256 ? 256 : G; }
+
+// Workgroup sizes a G-lane variant is compiled for.
+constexpr bool block_built(OpClass oc, int G, int block) {
+  if (block < G || block < 256 || block > 1024 || (block & (block - 1))) return false;
+#ifdef ROWNORM_TUNE_WIDE
+  return true;
+#else
+  return block == block_threads(oc, G);
+#endif
+}
+
+// Workgroups per compute unit of the persistent grid.
+constexpr int default_bpc(OpClass oc, int block) {
+  const bool bwd_cols = oc == OC_NORM_BWD;  // each workgroup emits a partial row: keep few
+  if (block <= 256) return bwd_cols ? 2 : 8;
+  if (block <= 512) return bwd_cols ? 1 : 4;
+  return bwd_cols ? 1 : 2;
+}
+
+// Which (G, V) kernels exist in the library.  Kept in one place so the
+// dispatcher, the planner and the forced-variant check agree.
+constexpr bool variant_built(OpClass oc, int esize, int G, int V) {
+  if (G < kMinG || G > kMaxG || (G & (G - 1)) || V < 1 || V > kMaxV || (V & (V - 1)))
+    return false;
+  if (V > v_max(oc, esize, G)) return false;
+#ifdef ROWNORM_TUNE_WIDE
+  return true;
+#else
+  if (G == kMinG) return V <= v_pref(oc, esize);
+  return V >= v_pref(oc, esize);
+#endif
+}
+
+inline int pow2_ceil(int64_t v) {
+  int p = 1;
+  while (p < v) p <<= 1;
+  return p;
+}
+
+// Returns 0, or -5 (ROWNORM_ERR_OVERRIDE) when a forced variant cannot hold the row.
+inline int make_plan(OpClass oc, int64_t M, int64_t N, int esize, int num_cus, const Override& ov,
+                     bool want_cols, Plan* out) {
+  Plan p;
+  const int E = 16 / esize;
+  const int64_t packs = (N + E - 1) / E;
+  if (num_cus <= 0) num_cus = 256;
+  bool stream = ov.G < 0;
+  if (!stream) {
+    int G, V;
+    if (ov.G > 0) {
+      G = ov.G;
+    } else {
+      G = pow2_ceil((packs + v_pref(oc, esize) - 1) / v_pref(oc, esize));
+      if (G < kMinG) G = kMinG;
+      if (G > kMaxG) G = kMaxG;
+    }
+    if (ov.V > 0) {
+      V = ov.V;
+    } else {
+      V = pow2_ceil((packs + G - 1) / G);
+    }
+    const bool holds = (int64_t)G * V >= packs;
+    const int block = ov.block > 0 ? ov.block : block_threads(oc, G);
+    const bool built = variant_built(oc, esize, G, V) && block_built(oc, G, block);
+    if (ov.G > 0 || ov.V > 0 || ov.block > 0) {
+      if (!holds || !built) return -5;
+    }
+    if (holds && built) {
+      p.resident = true;
+      p.G = G;
+      p.V = V;
+      p.block = block;
+      p.rpb = p.block / G;
+    } else {
+      stream = true;
+    }
+  }
+  if (stream) {
+    p.resident = false;
+    p.G = kStreamBlock;
+    p.V = 0;
+    p.block = kStreamBlock;
+    p.rpb = 1;
+  }
+  const int64_t nrb = (M + p.rpb - 1) / p.rpb;
+  const int bpc = ov.bpc > 0 ? ov.bpc : default_bpc(oc, p.block);
+  int64_t grid = (int64_t)num_cus * bpc;
+  if (grid > nrb) grid = nrb;
+  if (grid < 1) grid = 1;
+  p.grid = grid;
+  p.partial_rows = 0;
+  if (oc == OC_NORM_BWD && want_cols) {
+    // resident: one partial row per workgroup; streaming: a separate column-sum
+    // kernel whose grid.y is the partial-row count.
+    if (p.resident) {
+      p.partial_rows = grid;
+    } else {
+      int64_t pr = M < 64 ? M : 64;
+      p.partial_rows = pr < 1 ? 1 : pr;
+    }
+  }
+  *out = p;
+  return 0;
+}
+
+}  // namespace rownorm
