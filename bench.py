@@ -1,0 +1,312 @@
+#!/usr/bin/env python3
+"""Headline benchmark: HBM GB/s and % of peak of the row-wise norm family on one MI355X.
+
+One "step" is one pass of the hot path over one batch of synthetic input: `_fused_rms_norm`
+forward + backward on bf16 [16384 tokens, 4096] (Llama-3-8B hidden), bf16 weight, eps 1e-6,
+called through the extern "C" ABI of libmi355x_rownorm.so.  `value` is algorithmic bytes per step
+(every input read once, every output written once: forward 2*M*N*2 + N*2 + M*4, backward
+3*M*N*2 + M*4 + 2*N*2) divided by the measured time per step.  Inputs are resident in HBM before
+the timed region; successive steps rotate over buffer sets larger than the 256 MB Infinity
+Cache so that every step streams from HBM.
+
+    python bench.py [--gpus 1] [--steps K] [--warmup W] [--no-ops] [--no-cpu]
+
+prints ONE JSON line (see the keys below).  `roofline` covers the dominant operation of the step,
+one mi355x_rms_norm_bwd call (norm_bwd_resident_kernel + colsum_finalize_kernel), timed with HIP
+events on the launch stream inside the timed region.  `cpu_baseline` is the scalar C oracle
+(oracle/, a port of the same arithmetic) timed on one host core; `cpu_aten` is PyTorch's CPU ATen
+path (the parity target) on all host cores.  `ops` lists every op of the family at its
+Llama-class configuration (informational, measured after the timed region).
+"""
+import argparse
+import ctypes
+import importlib.util
+import json
+import os
+import sys
+import time
+
+ROOT = os.path.dirname(os.path.abspath(__file__))
+HBM_PEAK_GBS = 8000.0  # MI355X published HBM3E bandwidth
+
+
+def load_package():
+    pdir = os.path.join(ROOT, "torch-xpu-ops_amd")
+    if "torch_xpu_ops_amd" in sys.modules:
+        return sys.modules["torch_xpu_ops_amd"]
+    spec = importlib.util.spec_from_file_location(
+        "torch_xpu_ops_amd", os.path.join(pdir, "__init__.py"), submodule_search_locations=[pdir])
+    mod = importlib.util.module_from_spec(spec)
+    sys.modules["torch_xpu_ops_amd"] = mod
+    spec.loader.exec_module(mod)
+    return mod
+
+
+def main():
+    ap = argparse.ArgumentParser()
+    ap.add_argument("--gpus", type=int, default=1)
+    ap.add_argument("--steps", type=int, default=200)
+    ap.add_argument("--warmup", type=int, default=20)
+    ap.add_argument("--no-ops", action="store_true", help="skip the per-op table")
+    ap.add_argument("--no-cpu", action="store_true", help="skip the CPU baselines")
+    args = ap.parse_args()
+    if args.gpus != 1 or int(os.environ.get("WORLD_SIZE", "1")) != 1:
+        print("bench.py: this operator family runs whole on one GPU (rows are independent; "
+              "nothing communicates), so only --gpus 1 is measured", file=sys.stderr)
+        sys.exit(2)
+
+    import torch
+    if not torch.cuda.is_available():
+        print("bench.py: no GPU visible; the kernels have no CPU path", file=sys.stderr)
+        sys.exit(3)
+    pkg = load_package()
+    cabi = pkg.cabi
+    L = cabi.lib()  # raises if the HIP library is missing
+    dev = torch.device("cuda:0")
+    torch.cuda.set_device(dev)
+    stream = ctypes.c_void_p(torch.cuda.current_stream().cuda_stream)
+    P = lambda t: ctypes.c_void_p(t.data_ptr()) if t is not None else None  # noqa: E731
+    BF, F32 = cabi.BF16, cabi.F32
+
+    # ---- workload: BASELINE config 2 ------------------------------------------------------
+    M, N, eps = 16384, 4096, 1e-6
+    fwd_bytes = 2 * M * N * 2 + N * 2 + M * 4
+    bwd_bytes = 3 * M * N * 2 + M * 4 + 2 * N * 2
+    g = torch.Generator(device="cpu").manual_seed(1234 + 2)
+    w = (1 + 0.02 * torch.randn(N, generator=g)).to(torch.bfloat16).to(dev)
+    nsets = 4
+    sets = []
+    for _ in range(nsets):
+        x = torch.randn(M, N, generator=g).to(torch.bfloat16).to(dev)
+        dy = torch.randn(M, N, generator=g).to(torch.bfloat16).to(dev)
+        sets.append(dict(x=x, dy=dy, y=torch.empty_like(x), rstd=torch.empty(M, device=dev),
+                         dx=torch.empty_like(x), dw=torch.empty_like(w)))
+    ws_bytes = L.mi355x_rms_norm_bwd_workspace_bytes(M, N, BF, BF, 1)
+    ws = torch.empty(max(ws_bytes, 1), dtype=torch.uint8, device=dev)
+
+    def fwd(s):
+        return L.mi355x_rms_norm_fwd(P(s["x"]), P(w), P(s["y"]), P(s["rstd"]), M, N, eps, BF, BF,
+                                     stream)
+
+    def bwd(s):
+        return L.mi355x_rms_norm_bwd(P(s["dy"]), P(s["x"]), P(s["rstd"]), P(w), P(s["dx"]),
+                                     P(s["dw"]), P(ws), ws_bytes, M, N, BF, BF, stream)
+
+    for i in range(args.warmup):
+        s = sets[i % nsets]
+        rc = fwd(s) or bwd(s)
+        if rc != 0:
+            raise RuntimeError("kernel launch failed: " + cabi.error_string(rc))
+    ev = [(torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True))
+          for _ in range(args.steps)]
+    torch.cuda.synchronize()
+    t0 = time.perf_counter()
+    for i in range(args.steps):
+        s = sets[i % nsets]
+        fwd(s)
+        ev[i][0].record()
+        bwd(s)
+        ev[i][1].record()
+    torch.cuda.synchronize()
+    t1 = time.perf_counter()
+    ms_per_step = (t1 - t0) * 1e3 / args.steps
+    value = (fwd_bytes + bwd_bytes) / (ms_per_step * 1e-3) / 1e9
+    bwd_us = sum(a.elapsed_time(b) for a, b in ev) * 1e3 / args.steps
+    achieved = bwd_bytes / (bwd_us * 1e-6) / 1e9
+
+    out = {
+        "metric": "HBM GB/s & % peak: LayerNorm/RMSNorm/softmax fwd+bwd bf16, Llama shapes",
+        "value": round(value, 1),
+        "unit": "GB/s",
+        "pct_of_hbm_peak": round(100.0 * value / HBM_PEAK_GBS, 2),
+        "n_gpus": 1,
+        "steps": args.steps,
+        "warmup": args.warmup,
+        "ms_per_step": round(ms_per_step, 5),
+        "higher_is_better": True,
+        "scaling": "weak",
+        "vs_baseline": None,
+        "dtype": "bf16",
+        "data": "synthetic",
+        "config": {"workload": "_fused_rms_norm forward+backward, bf16 [16384, 4096], bf16 weight "
+                               "[4096], eps 1e-6 (BASELINE config 2)",
+                   "algorithmic_bytes_per_step": fwd_bytes + bwd_bytes,
+                   "buffer_sets_rotated": nsets},
+        "roofline": {
+            "bound": "hbm",
+            "kernel": "mi355x_rms_norm_bwd = norm_bwd_resident_kernel + colsum_finalize_kernel",
+            "achieved": round(achieved, 1),
+            "peak": HBM_PEAK_GBS,
+            "unit": "GB/s",
+            "frac": round(achieved / HBM_PEAK_GBS, 4),
+            "avg_us_per_launch": round(bwd_us, 2),
+            "algorithmic_bytes_per_launch": bwd_bytes,
+            "traffic": None,
+        },
+    }
+    traffic_file = os.path.join(ROOT, "profiles", "rms_norm_bwd_bf16_16384x4096_traffic.json")
+    if os.path.exists(traffic_file):
+        try:
+            with open(traffic_file) as f:
+                out["roofline"]["traffic"] = json.load(f).get("hbm_bytes_per_launch")
+        except Exception:
+            pass
+
+    if not args.no_ops:
+        out["ops"] = per_op_table(torch, cabi, L, dev, stream, P)
+    del sets
+    if not args.no_cpu:
+        out["cpu_baseline"], out["cpu_aten"] = cpu_baselines(torch, M, N, eps, fwd_bytes + bwd_bytes)
+    print(json.dumps(out))
+
+
+def _time_rotating(torch, fns, iters=30, warm=5):
+    n = len(fns)
+    for i in range(warm):
+        fns[i % n]()
+    torch.cuda.synchronize()
+    a, b = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+    a.record()
+    for i in range(iters):
+        fns[i % n]()
+    b.record()
+    torch.cuda.synchronize()
+    return a.elapsed_time(b) * 1e3 / iters
+
+
+def per_op_table(torch, cabi, L, dev, stream, P):
+    """Every op of the family at its BASELINE configuration: avg microseconds per call (HIP events
+    over 30 back-to-back calls rotating over buffer sets), algorithmic GB/s, fraction of 8 TB/s."""
+    BF, F32 = cabi.BF16, cabi.F32
+    rows = []
+
+    def add(name, nbytes, fns):
+        us = _time_rotating(torch, fns)
+        gbs = nbytes / us / 1e3
+        rows.append({"op": name, "us": round(us, 2), "GB/s": round(gbs, 1),
+                     "frac": round(gbs / HBM_PEAK_GBS, 4)})
+
+    # C1: native_layer_norm forward fp32 [4096, 1024] (32 MiB: cache resident, informational)
+    M, N = 4096, 1024
+    g = 1 + 0.1 * torch.randn(N, device=dev)
+    b = 0.1 * torch.randn(N, device=dev)
+    sets = [(torch.randn(M, N, device=dev), torch.empty(M, N, device=dev),
+             torch.empty(M, device=dev), torch.empty(M, device=dev)) for _ in range(16)]
+    add("C1 native_layer_norm fwd fp32 [4096,1024]", 2 * M * N * 4 + 2 * N * 4 + 2 * M * 4,
+        [(lambda s=s: L.mi355x_layer_norm_fwd(P(s[0]), P(g), P(b), P(s[1]), P(s[2]), P(s[3]), M, N,
+                                              1e-5, F32, F32, stream)) for s in sets])
+    del sets
+
+    # C2: _fused_rms_norm bf16 [16384, 4096]
+    M, N = 16384, 4096
+    w = (1 + 0.02 * torch.randn(N, device=dev)).bfloat16()
+    sets = []
+    for _ in range(4):
+        x = torch.randn(M, N, device=dev).bfloat16()
+        sets.append((x, torch.randn(M, N, device=dev).bfloat16(), torch.empty_like(x),
+                     torch.empty(M, device=dev), torch.empty_like(x), torch.empty_like(w)))
+    nws = L.mi355x_rms_norm_bwd_workspace_bytes(M, N, BF, BF, 1)
+    ws = torch.empty(max(nws, 1), dtype=torch.uint8, device=dev)
+    add("C2 _fused_rms_norm fwd bf16 [16384,4096]", 2 * M * N * 2 + N * 2 + M * 4,
+        [(lambda s=s: L.mi355x_rms_norm_fwd(P(s[0]), P(w), P(s[2]), P(s[3]), M, N, 1e-6, BF, BF,
+                                            stream)) for s in sets])
+    add("C2 _fused_rms_norm bwd bf16 [16384,4096]", 3 * M * N * 2 + M * 4 + 2 * N * 2,
+        [(lambda s=s: L.mi355x_rms_norm_bwd(P(s[1]), P(s[0]), P(s[3]), P(w), P(s[4]), P(s[5]),
+                                            P(ws), nws, M, N, BF, BF, stream)) for s in sets])
+    del sets
+
+    # C4: native_layer_norm bf16 rows, fp32 gamma/beta [16384, 8192]
+    M, N = 16384, 8192
+    g = 1 + 0.1 * torch.randn(N, device=dev)
+    b = 0.1 * torch.randn(N, device=dev)
+    sets = []
+    for _ in range(3):
+        x = torch.randn(M, N, device=dev).bfloat16()
+        s = (x, torch.randn(M, N, device=dev).bfloat16(), torch.empty_like(x),
+             torch.empty(M, device=dev), torch.empty(M, device=dev), torch.empty_like(x),
+             torch.empty_like(g), torch.empty_like(g))
+        L.mi355x_layer_norm_fwd(P(s[0]), P(g), P(b), P(s[2]), P(s[3]), P(s[4]), M, N, 1e-5, BF, F32,
+                                stream)
+        sets.append(s)
+    nws = L.mi355x_layer_norm_bwd_workspace_bytes(M, N, BF, F32, 1, 1)
+    ws = torch.empty(max(nws, 1), dtype=torch.uint8, device=dev)
+    add("C4 native_layer_norm fwd bf16/fp32w [16384,8192]", 2 * M * N * 2 + 2 * N * 4 + 2 * M * 4,
+        [(lambda s=s: L.mi355x_layer_norm_fwd(P(s[0]), P(g), P(b), P(s[2]), P(s[3]), P(s[4]), M, N,
+                                              1e-5, BF, F32, stream)) for s in sets])
+    add("C4 native_layer_norm bwd bf16/fp32w [16384,8192]", 3 * M * N * 2 + 2 * M * 4 + 3 * N * 4,
+        [(lambda s=s: L.mi355x_layer_norm_bwd(P(s[1]), P(s[0]), P(s[3]), P(s[4]), P(g), P(s[5]),
+                                              P(s[6]), P(s[7]), P(ws), nws, M, N, BF, F32, stream))
+         for s in sets])
+    del sets
+
+    # C3: softmax / log_softmax bf16 [4, 32, 2048, 2048] with a causal -inf mask
+    R, N = 4 * 32 * 2048, 2048
+    sets = []
+    for _ in range(2):
+        s = 3 * torch.randn(32, 2048, 2048, device=dev)
+        s.masked_fill_(torch.triu(torch.ones(2048, 2048, device=dev), 1).bool(), float("-inf"))
+        s = s.bfloat16().repeat(4, 1, 1).view(R, N)
+        sets.append((s, torch.randn(R, N, device=dev).bfloat16(), torch.empty_like(s),
+                     torch.empty_like(s)))
+    for is_log, nm in ((0, "_softmax"), (1, "_log_softmax")):
+        add("C3 %s fwd bf16 [4,32,2048,2048]" % nm, 2 * R * N * 2,
+            [(lambda s=s: L.mi355x_softmax_fwd(P(s[0]), P(s[2]), R, N, BF, BF, is_log, stream))
+             for s in sets])
+        add("C3 %s bwd bf16 [4,32,2048,2048]" % nm, 3 * R * N * 2,
+            [(lambda s=s: L.mi355x_softmax_bwd(P(s[1]), P(s[2]), P(s[3]), R, N, BF, BF, is_log,
+                                               stream)) for s in sets])
+    del sets
+    torch.cuda.empty_cache()
+    return rows
+
+
+def cpu_baselines(torch, M, N, eps, step_bytes):
+    """(oracle port on one core, CPU ATen on all cores) for the same fwd+bwd workload.  Bounded:
+    the oracle runs the full [M, N] batch once (about 1-3 s of scalar double arithmetic); ATen
+    runs it for at least 3 iterations or 5 s."""
+    import numpy as np
+    sys.path.insert(0, ROOT)
+    import oracle
+    g = torch.Generator().manual_seed(99)
+    x = torch.randn(M, N, generator=g).to(torch.bfloat16)
+    dy = torch.randn(M, N, generator=g).to(torch.bfloat16)
+    w = (1 + 0.02 * torch.randn(N, generator=g)).to(torch.bfloat16)
+    xn, dyn, wn = x.float().numpy(), dy.float().numpy(), w.float().numpy()
+    oracle.lib()
+    t0 = time.perf_counter()
+    _, rstd = oracle.rms_norm_fwd(xn, (N,), wn, eps)
+    oracle.rms_norm_bwd(dyn, xn, (N,), rstd, wn)
+    t_or = time.perf_counter() - t0
+    port = {"value": round(step_bytes / t_or / 1e9, 3), "unit": "GB/s", "cores": 1, "kind": "port",
+            "sample": "oracle/rownorm_oracle.c (scalar C, double accumulators): one full "
+                      "[%d, %d] forward+backward, %.2f s" % (M, N, t_or)}
+    del xn, dyn
+
+    xr = x.clone().requires_grad_()
+    wr = w.clone().requires_grad_()
+
+    def step():
+        xr.grad = None
+        wr.grad = None
+        y = torch.nn.functional.rms_norm(xr, (N,), wr, eps)
+        y.backward(dy)
+
+    for _ in range(2):
+        step()
+    n, t0 = 0, time.perf_counter()
+    while n < 3 or time.perf_counter() - t0 < 5.0:
+        step()
+        n += 1
+        if time.perf_counter() - t0 > 25.0:
+            break
+    t_at = (time.perf_counter() - t0) / n
+    aten = {"value": round(step_bytes / t_at / 1e9, 3), "unit": "GB/s",
+            "cores": torch.get_num_threads(), "host_cpus": os.cpu_count(),
+            "sample": "PyTorch %s CPU ATen: F.rms_norm forward + autograd backward (ATen has no "
+                      "CPU _fused_rms_norm_backward), full [%d, %d] bf16 batch, %d iterations, "
+                      "%.3f s each" % (torch.__version__, M, N, n, t_at)}
+    return port, aten
+
+
+if __name__ == "__main__":
+    main()

@@ -1,0 +1,110 @@
+"""Writes tests/golden/aten_cpu_golden.npz: input/output vectors of PyTorch's CPU ATen
+implementation of the operator family (the arithmetic parity target named for this path).
+
+Nothing from the reference repository is imported or run: the vectors come from the installed
+torch wheel (torch 2.10.0 when this file was last run; the version is stored in the archive).
+They pin what no closed form pins: where low-precision outputs are rounded, bit-exact beta on
+constant rows, -inf / NaN propagation, and the +-1e4 outlier behaviour.
+
+    python tests/golden/make_golden.py            # rewrites the .npz next to this file
+
+Layout of the archive: "<case>/<tensor>" arrays.  16-bit tensors are stored as uint16 bit
+patterns ("...:bf16" / "...:f16" suffix in the key) so numpy needs no bfloat16 support.
+"""
+import os
+
+import numpy as np
+import torch
+
+HERE = os.path.dirname(os.path.abspath(__file__))
+SHAPES = [(7, 64), (5, 127), (3, 4097)]
+DTYPES = {"f32": torch.float32, "f16": torch.float16, "bf16": torch.bfloat16}
+
+
+def put(store, key, t):
+    t = t.detach().contiguous()
+    if t.dtype == torch.float32:
+        store[key] = t.numpy()
+    elif t.dtype == torch.float16:
+        store[key + ":f16"] = t.view(torch.int16).numpy().view(np.uint16)
+    elif t.dtype == torch.bfloat16:
+        store[key + ":bf16"] = t.view(torch.int16).numpy().view(np.uint16)
+    else:
+        raise TypeError(t.dtype)
+
+
+def stress_rows(M, N, g):
+    x = torch.randn(M, N, generator=g)
+    mask = torch.rand(M, N, generator=g) < 0.002
+    sign = torch.where(torch.rand(M, N, generator=g) < 0.5, -1.0, 1.0)
+    x = torch.where(mask, 1e4 * sign, x)
+    x[0] = 1.5  # one all-constant row
+    return x
+
+
+def main():
+    torch.manual_seed(0)
+    torch.set_num_threads(1)
+    store = {"meta/torch_version": np.frombuffer(torch.__version__.encode(), dtype=np.uint8)}
+    for dname, dt in DTYPES.items():
+        for (M, N) in SHAPES:
+            g = torch.Generator().manual_seed(1000 + N)
+            case = "%s_%dx%d" % (dname, M, N)
+            x = stress_rows(M, N, g).to(dt)
+            dy = torch.randn(M, N, generator=g).to(dt)
+            gamma = (1 + 0.1 * torch.randn(N, generator=g)).to(dt)
+            beta = (0.1 * torch.randn(N, generator=g)).to(dt)
+            for k, v in (("x", x), ("dy", dy), ("gamma", gamma), ("beta", beta)):
+                put(store, case + "/" + k, v)
+            # LayerNorm, eps 1e-5.  CPU ATen returns mean/rstd in the input dtype for unmixed
+            # 16-bit inputs; they are stored as returned.
+            y, mean, rstd = torch.ops.aten.native_layer_norm(x, [N], gamma, beta, 1e-5)
+            put(store, case + "/ln_y", y)
+            put(store, case + "/ln_mean", mean.reshape(-1))
+            put(store, case + "/ln_rstd", rstd.reshape(-1))
+            dx, dg, db = torch.ops.aten.native_layer_norm_backward(
+                dy, x, [N], mean, rstd, gamma, beta, [True, True, True])
+            put(store, case + "/ln_dx", dx)
+            put(store, case + "/ln_dgamma", dg)
+            put(store, case + "/ln_dbeta", db)
+            # mixed precision: 16-bit rows with float32 gamma/beta (fp32 statistics)
+            if dt != torch.float32:
+                g32, b32 = gamma.float(), beta.float()
+                y, mean, rstd = torch.ops.aten.native_layer_norm(x, [N], g32, b32, 1e-5)
+                put(store, case + "/lnmix_y", y)
+                put(store, case + "/lnmix_mean", mean.reshape(-1))
+                put(store, case + "/lnmix_rstd", rstd.reshape(-1))
+                dx, dg, db = torch.ops.aten.native_layer_norm_backward(
+                    dy, x, [N], mean, rstd, g32, b32, [True, True, True])
+                put(store, case + "/lnmix_dx", dx)
+                put(store, case + "/lnmix_dgamma", dg)
+                put(store, case + "/lnmix_dbeta", db)
+            # RMSNorm, eps 1e-6 (forward op; backward through autograd: ATen has no CPU
+            # _fused_rms_norm_backward kernel)
+            xr, gr = x.clone().requires_grad_(), gamma.clone().requires_grad_()
+            y, rstd = torch.ops.aten._fused_rms_norm(xr, [N], gr, 1e-6)
+            put(store, case + "/rms_y", y)
+            put(store, case + "/rms_rstd", rstd.reshape(-1).float())
+            y.backward(dy)
+            put(store, case + "/rms_dx", xr.grad)
+            put(store, case + "/rms_dgamma", gr.grad)
+            # softmax / log_softmax on scores with a masked tail and one fully masked row
+            s = (3.0 * torch.randn(M, N, generator=g))
+            s[1, N // 2:] = float("-inf")
+            s[2, :] = float("-inf")
+            s = s.to(dt)
+            put(store, case + "/sm_x", s)
+            for is_log, nm in ((False, "sm"), (True, "lsm")):
+                fwd = torch.ops.aten._log_softmax if is_log else torch.ops.aten._softmax
+                bwd = (torch.ops.aten._log_softmax_backward_data if is_log
+                       else torch.ops.aten._softmax_backward_data)
+                out = fwd(s, -1, False)
+                put(store, case + "/%s_y" % nm, out)
+                put(store, case + "/%s_gi" % nm, bwd(dy, out, -1, dt))
+    path = os.path.join(HERE, "aten_cpu_golden.npz")
+    np.savez_compressed(path, **store)
+    print("wrote", path, os.path.getsize(path), "bytes,", len(store), "arrays")
+
+
+if __name__ == "__main__":
+    main()

@@ -88,3 +88,50 @@ def causal_scores(B, H, T, seed, dtype=torch.bfloat16):
     s = 3.0 * torch.randn(B, H, T, T, generator=g)
     s.masked_fill_(torch.triu(torch.ones(T, T), 1).bool(), float("-inf"))
     return s.to(dtype)
+
+
+def load_golden():
+    """tests/golden/aten_cpu_golden.npz as {case: {name: torch tensor}} with the stored dtypes."""
+    import os
+    path = os.path.join(os.path.dirname(os.path.abspath(__file__)), "golden", "aten_cpu_golden.npz")
+    z = np.load(path, allow_pickle=False)
+    cases = {}
+    for key in z.files:
+        case, name = key.split("/", 1)
+        if case == "meta":
+            continue
+        arr = z[key]
+        if name.endswith(":bf16"):
+            t = torch.from_numpy(arr.view(np.int16).copy()).view(torch.bfloat16)
+            name = name[:-5]
+        elif name.endswith(":f16"):
+            t = torch.from_numpy(arr.view(np.int16).copy()).view(torch.float16)
+            name = name[:-4]
+        else:
+            t = torch.from_numpy(arr.copy())
+        cases.setdefault(case, {})[name] = t
+    return cases
+
+
+GOLDEN_DTYPES = {"f32": torch.float32, "f16": torch.float16, "bf16": torch.bfloat16}
+
+
+EPS32 = 2.0 ** -24
+
+
+def colsum_slack(terms):
+    """Allowance for a float32 column sum over many rows: 16 * 2^-24 * ||terms||_2 per column.
+    A sum of M float32 products carries a rounding error that grows like eps * sqrt(M) * rms(term)
+    whatever the order of summation, while rtol * |result| shrinks to nothing on the columns whose
+    terms cancel; the CPU kernel's float32 sums show the same behaviour."""
+    t = torch.as_tensor(terms).to(torch.float64)
+    return 16.0 * EPS32 * t.pow(2).sum(0).sqrt()
+
+
+def rowsum_slack(terms, weight):
+    """Allowance for an output of the form weight * (float32 sum of `terms` over a row): the sum's
+    rounding, 16 * 2^-24 * ||terms||_2 per row, times |weight| per element."""
+    t = torch.as_tensor(terms).to(torch.float64)
+    w = torch.as_tensor(weight).to(torch.float64).abs()
+    w = torch.where(torch.isfinite(w), w, torch.zeros_like(w))
+    return w * (16.0 * EPS32 * t.pow(2).sum(-1, keepdim=True).sqrt())

@@ -1,0 +1,124 @@
+"""CPU-only checks of the C ABI library: it loads without a GPU, exports every symbol declared in
+include/mi355x_rownorm.h, validates arguments before touching the device, and plans launches the
+way the header documents.  No kernel is launched here."""
+import ctypes
+import os
+import re
+
+import pytest
+
+ROOT = os.path.dirname(os.path.dirname(os.path.abspath(__file__)))
+HEADER = os.path.join(ROOT, "include", "mi355x_rownorm.h")
+
+
+def declared_functions():
+    text = open(HEADER).read()
+    text = re.sub(r"/\*.*?\*/", "", text, flags=re.S)
+    return sorted(set(re.findall(r"\b(mi355x_\w+)\s*\(", text)))
+
+
+def test_header_and_python_binding_agree(cabi):
+    assert declared_functions() == sorted(cabi.EXPORTED_SYMBOLS)
+
+
+def test_library_exports_every_declared_symbol(cabi):
+    lib = cabi.lib()
+    for name in declared_functions():
+        assert getattr(lib, name) is not None, name
+    assert lib.mi355x_rownorm_abi_version() == 1
+
+
+def test_error_strings(cabi):
+    assert cabi.error_string(0) == "success"
+    for code in (-1, -2, -3, -4, -5):
+        assert "mi355x_rownorm" in cabi.error_string(code)
+    assert cabi.error_string(-99).startswith("mi355x_rownorm: unknown")
+
+
+def test_argument_validation_happens_before_any_launch(cabi):
+    L = cabi.lib()
+    null = None
+    # unknown dtype code, unsupported dtype pair
+    assert L.mi355x_layer_norm_fwd(null, null, null, null, null, null, 4, 8, 1e-5, 7, 0, null) == -1
+    assert L.mi355x_rms_norm_fwd(null, null, null, null, 4, 8, 1e-5, cabi.F32, cabi.BF16, null) == -1
+    assert L.mi355x_softmax_fwd(null, null, 4, 8, cabi.BF16, cabi.F32, 0, null) == -1  # only f16->f32
+    assert L.mi355x_softmax_bwd(null, null, null, 4, 8, cabi.F32, cabi.BF16, 0, null) == -1
+    # negative sizes / oversize rows
+    assert L.mi355x_layer_norm_fwd(null, null, null, null, null, null, -1, 8, 1e-5, 0, 0, null) == -2
+    assert L.mi355x_softmax_fwd(null, null, 4, (1 << 30) + 1, 0, 0, 0, null) == -2
+    # empty problems are a successful no-op even with null pointers (M == 0 or N == 0)
+    assert L.mi355x_layer_norm_fwd(null, null, null, null, null, null, 0, 8, 1e-5, 0, 0, null) == 0
+    assert L.mi355x_rms_norm_bwd(null, null, null, null, null, null, null, 0, 5, 0, 0, 0, null) == 0
+    assert L.mi355x_softmax_bwd(null, null, null, 0, 8, 0, 0, 1, null) == 0
+    # required pointers
+    assert L.mi355x_layer_norm_fwd(null, null, null, null, null, null, 4, 8, 1e-5, 0, 0, null) == -3
+    assert L.mi355x_softmax_fwd(null, null, 4, 8, 0, 0, 0, null) == -3
+    # backward with column sums wanted but no workspace
+    one = ctypes.c_void_p(256)  # never dereferenced: the call is rejected before launching
+    assert L.mi355x_layer_norm_bwd(one, one, one, one, one, one, one, one, null, 0, 4, 8, 0, 0,
+                                   null) == -4
+    assert L.mi355x_rms_norm_bwd(one, one, one, one, one, one, null, 0, 4, 8, 0, 0, null) == -4
+    # nothing requested: no-op
+    assert L.mi355x_rms_norm_bwd(one, one, one, one, null, null, null, 0, 4, 8, 0, 0, null) == 0
+
+
+def test_workspace_size_follows_the_plan(cabi):
+    L = cabi.lib()
+    p = cabi.plan(cabi.OP_RMS_NORM_BWD, 16384, 4096, cabi.BF16, cabi.BF16)
+    assert p["partial_rows"] == p["grid_blocks"] > 0
+    assert L.mi355x_rms_norm_bwd_workspace_bytes(16384, 4096, cabi.BF16, cabi.BF16, 1) == \
+        p["partial_rows"] * 4096 * 4
+    assert L.mi355x_rms_norm_bwd_workspace_bytes(16384, 4096, cabi.BF16, cabi.BF16, 0) == 0
+    p = cabi.plan(cabi.OP_LAYER_NORM_BWD, 16384, 8192, cabi.BF16, cabi.F32)
+    assert L.mi355x_layer_norm_bwd_workspace_bytes(16384, 8192, cabi.BF16, cabi.F32, 1, 1) == \
+        2 * p["partial_rows"] * 8192 * 4
+    assert L.mi355x_layer_norm_bwd_workspace_bytes(16384, 8192, cabi.BF16, cabi.F32, 0, 0) == 0
+    assert L.mi355x_layer_norm_bwd_workspace_bytes(0, 8192, cabi.BF16, cabi.F32, 1, 1) == 0
+
+
+@pytest.mark.parametrize("op", range(6))
+@pytest.mark.parametrize("dt", [0, 1, 2])
+def test_plan_invariants(cabi, op, dt):
+    esize = 4 if dt == 0 else 2
+    E = 16 // esize
+    for N in (1, 7, 8, 64, 127, 1000, 1024, 2048, 4096, 4097, 5120, 8192, 16384, 40000, 1 << 20):
+        for M in (1, 3, 1000, 1 << 20):
+            p = cabi.plan(op, M, N, dt, dt)
+            assert p["grid_blocks"] >= 1
+            if p["resident"]:
+                G, V = p["lanes_per_row"], p["packs_per_lane"]
+                assert 8 <= G <= 1024 and G & (G - 1) == 0 and V >= 1
+                assert G * V * E >= N, "row must fit the lanes' registers"
+                assert p["block_threads"] % G == 0 and p["block_threads"] <= 1024
+                assert p["rows_per_block"] == p["block_threads"] // G
+                assert p["grid_blocks"] <= (M + p["rows_per_block"] - 1) // p["rows_per_block"]
+            else:
+                assert p["rows_per_block"] == 1 and p["grid_blocks"] <= M
+            if op in (cabi.OP_LAYER_NORM_BWD, cabi.OP_RMS_NORM_BWD):
+                assert p["partial_rows"] >= 1
+            else:
+                assert p["partial_rows"] == 0
+
+
+def test_plan_picks_resident_kernels_for_the_llama_shapes(cabi):
+    for op, M, N, dt in ((cabi.OP_LAYER_NORM_FWD, 4096, 1024, cabi.F32),
+                         (cabi.OP_RMS_NORM_FWD, 16384, 4096, cabi.BF16),
+                         (cabi.OP_RMS_NORM_BWD, 16384, 4096, cabi.BF16),
+                         (cabi.OP_SOFTMAX_FWD, 262144, 2048, cabi.BF16),
+                         (cabi.OP_SOFTMAX_BWD, 262144, 2048, cabi.BF16),
+                         (cabi.OP_LAYER_NORM_FWD, 16384, 8192, cabi.BF16),
+                         (cabi.OP_LAYER_NORM_BWD, 16384, 8192, cabi.BF16),
+                         (cabi.OP_LAYER_NORM_BWD, 8192, 16384, cabi.F32)):
+        assert cabi.plan(op, M, N, dt, dt)["resident"] == 1, (op, M, N, dt)
+    # rows far beyond the register file stream through the multi-pass kernels
+    assert cabi.plan(cabi.OP_SOFTMAX_FWD, 4, 1 << 20, cabi.F32, cabi.F32)["resident"] == 0
+
+
+def test_forced_variants(cabi):
+    cabi.set_override(cabi.OP_SOFTMAX_FWD, -1)
+    assert cabi.plan(cabi.OP_SOFTMAX_FWD, 64, 2048, cabi.BF16, cabi.BF16)["resident"] == 0
+    cabi.set_override(cabi.OP_SOFTMAX_FWD, 64, 1)  # 64 lanes x 1 pack cannot hold 2048 bf16
+    with pytest.raises(RuntimeError, match="forced variant"):
+        cabi.plan(cabi.OP_SOFTMAX_FWD, 64, 2048, cabi.BF16, cabi.BF16)
+    cabi.clear_overrides()
+    assert cabi.plan(cabi.OP_SOFTMAX_FWD, 64, 2048, cabi.BF16, cabi.BF16)["resident"] == 1

@@ -1,0 +1,221 @@
+"""The ATen-signature host layer (torch.ops.mi355x.*) on the GPU against PyTorch's CPU ATen ops:
+shapes and dtypes of the saved tensors, output masks, empty inputs, non-contiguous inputs,
+softmax over any dimension, out= forms, half_to_float, and the opt-in aten override with
+autograd end to end.  Mirrors test/regressions/test_softmax.py:18-46,
+test/regressions/test_rms_norm.py:52-160 and test/repro/test_layer_norm_group_norm_align.py:25-78
+of the reference ("compute on CPU, compute on the device, compare")."""
+import pytest
+import torch
+import torch.nn.functional as F
+
+from helpers import assert_close, gen
+
+pytestmark = pytest.mark.gpu
+
+
+@pytest.mark.parametrize("dtype", [torch.float32, torch.float16, torch.bfloat16], ids=str)
+def test_native_layer_norm_contract(ops, gpu, dtype):
+    x = torch.randn(2, 3, 4, 5, generator=gen(1)).to(dtype)
+    w = torch.randn(4, 5, generator=gen(2)).to(dtype)
+    b = torch.randn(4, 5, generator=gen(3)).to(dtype)
+    y, mean, rstd = ops.native_layer_norm(x.to(gpu), [4, 5], w.to(gpu), b.to(gpu), 1e-5)
+    # statistics are float32 whatever the input dtype (LayerNorm.cpp:72-75 in the reference),
+    # shaped input.shape[:axis] + [1] * k (:82-94)
+    assert y.shape == x.shape and y.dtype == dtype and y.is_contiguous()
+    assert mean.shape == (2, 3, 1, 1) and rstd.shape == (2, 3, 1, 1)
+    assert mean.dtype == torch.float32 and rstd.dtype == torch.float32
+    cy, cm, cr = torch.ops.aten.native_layer_norm(x.float(), [4, 5], w.float(), b.float(), 1e-5)
+    assert_close(y, cy, dtype, "y")
+    assert_close(mean, cm, dtype, "mean")
+    assert_close(rstd, cr, dtype, "rstd")
+    dy = torch.randn(2, 3, 4, 5, generator=gen(4)).to(dtype)
+    dx, dg, db = ops.native_layer_norm_backward(dy.to(gpu), x.to(gpu), [4, 5], mean, rstd, w.to(gpu),
+                                                b.to(gpu), [True, True, True])
+    cdx, cdg, cdb = torch.ops.aten.native_layer_norm_backward(
+        dy.float(), x.float(), [4, 5], cm, cr, w.float(), b.float(), [True, True, True])
+    assert dx.shape == x.shape and dg.shape == (4, 5) and db.shape == (4, 5)
+    assert dx.dtype == dtype and dg.dtype == dtype and db.dtype == dtype
+    assert_close(dx, cdx, dtype, "dx")
+    assert_close(dg, cdg, dtype, "dgamma")
+    assert_close(db, cdb, dtype, "dbeta")
+    # output masks: undefined tensors come back as None
+    a, bb, c = ops.native_layer_norm_backward(dy.to(gpu), x.to(gpu), [4, 5], mean, rstd, w.to(gpu),
+                                              b.to(gpu), [True, False, False])
+    assert bb is None and c is None and torch.equal(a, dx)
+    a, bb, c = ops.native_layer_norm_backward(dy.to(gpu), x.to(gpu), [4, 5], mean, rstd, w.to(gpu),
+                                              b.to(gpu), [False, True, True])
+    assert a is None and torch.equal(bb, dg) and torch.equal(c, db)
+
+
+def test_layer_norm_mixed_precision_and_noncontiguous(ops, gpu):
+    # bf16 rows with float32 gamma/beta: a CPU-ATen feature the reference's kernels lack
+    x = torch.randn(33, 48, 96, generator=gen(5)).bfloat16()
+    xt = x.transpose(0, 1)  # non-contiguous input
+    w = torch.randn(96, generator=gen(6))
+    b = torch.randn(96, generator=gen(7))
+    y, mean, rstd = ops.native_layer_norm(xt.to(gpu), [96], w.to(gpu), b.to(gpu), 1e-5)
+    cy, cm, cr = torch.ops.aten.native_layer_norm(xt.float(), [96], w, b, 1e-5)
+    assert y.dtype == torch.bfloat16 and mean.shape == (48, 33, 1)
+    assert_close(y, cy, torch.bfloat16, "y")
+    dy = torch.randn(48, 33, 96, generator=gen(8)).bfloat16()
+    dx, dg, db = ops.native_layer_norm_backward(dy.to(gpu), xt.to(gpu), [96], mean, rstd, w.to(gpu),
+                                                b.to(gpu), [True, True, True])
+    cdx, cdg, cdb = torch.ops.aten.native_layer_norm_backward(dy.float(), xt.float(), [96], cm, cr, w,
+                                                              b, [True, True, True])
+    assert dx.dtype == torch.bfloat16 and dg.dtype == torch.float32 and db.dtype == torch.float32
+    assert_close(dx, cdx, torch.bfloat16, "dx")
+    assert_close(dg, cdg, torch.bfloat16, "dgamma")
+    assert_close(db, cdb, torch.bfloat16, "dbeta")
+
+
+def test_empty_batches(ops, gpu):
+    # LayerNorm.cpp:77,150-181 in the reference: M == 0 launches nothing; dgamma/dbeta are zeros
+    x = torch.empty(0, 16, device=gpu)
+    w = torch.ones(16, device=gpu)
+    y, mean, rstd = ops.native_layer_norm(x, [16], w, w, 1e-5)
+    assert y.shape == (0, 16) and mean.shape == (0, 1) and rstd.shape == (0, 1)
+    dx, dg, db = ops.native_layer_norm_backward(x, x, [16], mean, rstd, w, w, [True, True, True])
+    assert dx.shape == (0, 16) and bool((dg == 0).all()) and bool((db == 0).all())
+    y, rstd = ops._fused_rms_norm(x, [16], w, None)
+    assert y.shape == (0, 16) and rstd.shape == (0, 1)
+    dx, dg = ops._fused_rms_norm_backward(x, x, [16], rstd, w, [True, True])
+    assert dx.shape == (0, 16) and bool((dg == 0).all())
+    assert ops._softmax(x, -1, False).shape == (0, 16)
+    assert ops._softmax(torch.empty(4, 0, device=gpu), -1, False).shape == (4, 0)
+
+
+@pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16], ids=str)
+def test_fused_rms_norm_contract(ops, gpu, dtype):
+    x = torch.randn(2, 3, 4, 5, generator=gen(9)).to(dtype)
+    w = torch.randn(4, 5, generator=gen(10)).to(dtype)
+    for eps in (1e-6, None):
+        y, rstd = ops._fused_rms_norm(x.to(gpu), [4, 5], w.to(gpu), eps)
+        cy, crstd = torch.ops.aten._fused_rms_norm(x.float(), [4, 5], w.float(), eps)
+        assert y.dtype == dtype and rstd.dtype == torch.float32 and rstd.shape == (2, 3, 1, 1)
+        assert_close(y, cy, dtype, "y")
+        assert_close(rstd, crstd, dtype, "rstd")
+    # eps=None means FLT_EPSILON for every supported dtype (LayerNorm.cpp:218-224): closed form
+    x32 = x.float()
+    closed = x32 * torch.rsqrt(x32.pow(2).mean((-2, -1), keepdim=True) + torch.finfo(torch.float32).eps) * w.float()
+    assert_close(y, closed, dtype, "y vs closed form")
+    dy = torch.randn(2, 3, 4, 5, generator=gen(11)).to(dtype)
+    dx, dg = ops._fused_rms_norm_backward(dy.to(gpu), x.to(gpu), [4, 5], rstd, w.to(gpu), [True, True])
+    xr, wr = x.float().requires_grad_(), w.float().requires_grad_()
+    F.rms_norm(xr, (4, 5), wr, torch.finfo(torch.float32).eps).backward(dy.float())
+    assert_close(dx, xr.grad, dtype, "dx", scale=2.0)
+    assert_close(dg, wr.grad, dtype, "dgamma", scale=2.0)
+    a, b = ops._fused_rms_norm_backward(dy.to(gpu), x.to(gpu), [4, 5], rstd, w.to(gpu), [True, False])
+    assert b is None and torch.equal(a, dx)
+
+
+SOFTMAX_SHAPES = [(), (7,), (31, 23), (32, 1536), (33, 2049), (4, 5, 600), (2, 3, 4, 5)]
+
+
+@pytest.mark.parametrize("shape", SOFTMAX_SHAPES, ids=str)
+@pytest.mark.parametrize("dtype", [torch.float32, torch.float16, torch.bfloat16], ids=str)
+def test_softmax_every_dim(ops, gpu, shape, dtype):
+    # test/regressions/test_softmax.py:18-46 and test/xpu/test_nn_xpu.py:14056-14106: every dim,
+    # forward and backward, against the CPU
+    x = (2 * torch.randn(shape, generator=gen(12))).to(dtype)
+    g = torch.randn(shape, generator=gen(13)).to(dtype)
+    for dim in range(-1, max(len(shape), 1) - 1):
+        for is_log in (False, True):
+            fwd = ops._log_softmax if is_log else ops._softmax
+            bwd = ops._log_softmax_backward_data if is_log else ops._softmax_backward_data
+            cfwd = torch.ops.aten._log_softmax if is_log else torch.ops.aten._softmax
+            cbwd = (torch.ops.aten._log_softmax_backward_data if is_log
+                    else torch.ops.aten._softmax_backward_data)
+            y = fwd(x.to(gpu), dim, False)
+            assert y.shape == x.shape and y.dtype == dtype
+            cy = cfwd(x.float(), dim, False)
+            assert_close(y, cy, dtype, "y dim=%d" % dim)
+            gi = bwd(g.to(gpu), y, dim, dtype)
+            cgi = cbwd(g.float(), y.cpu().float(), dim, torch.float32)
+            assert gi.shape == x.shape and gi.dtype == dtype
+            assert_close(gi, cgi, dtype, "grad_input dim=%d" % dim, scale=2.0)
+
+
+def test_softmax_sliced_rows_and_out_variants(ops, gpu):
+    # rows of a (1,1)-sliced tensor start at arbitrary alignments (test_nn_xpu.py:14071-14078)
+    base = torch.randn(34, 2050, generator=gen(14))
+    xs = base.to(gpu)[1:, 1:]
+    y = ops._softmax(xs, 1, False)
+    assert_close(y, torch.ops.aten._softmax(base[1:, 1:], 1, False), torch.float32, "sliced y")
+    y0 = ops._softmax(xs, 0, False)
+    assert_close(y0, torch.ops.aten._softmax(base[1:, 1:], 0, False), torch.float32, "sliced y dim 0")
+    out = torch.empty(33, 2049, device=gpu)
+    r = ops._softmax.out(xs, 1, False, out=out)
+    assert r.data_ptr() == out.data_ptr() and torch.equal(out, y)
+    g = torch.randn(33, 2049, generator=gen(15)).to(gpu)
+    gi = ops._softmax_backward_data(g, y, 1, torch.float32)
+    gout = torch.empty(33, 2049, device=gpu)
+    ops._softmax_backward_data.out(g, y, 1, torch.float32, grad_input=gout)
+    assert torch.equal(gi, gout)
+    lout = torch.empty(33, 2049, device=gpu)
+    ops._log_softmax.out(xs, 1, False, out=lout)
+    assert torch.equal(lout, ops._log_softmax(xs, 1, False))
+
+
+def test_softmax_half_to_float(ops, gpu):
+    # test/xpu/test_nn_xpu.py:15036-15047: softmax(half, dtype=float) == softmax(float(half))
+    x = torch.randn(32, 100, generator=gen(16)).half().to(gpu)
+    y = ops._softmax(x, -1, True)
+    assert y.dtype == torch.float32
+    assert_close(y, ops._softmax(x.float(), -1, False), torch.float32, "half_to_float y")
+    g = torch.randn(32, 100, generator=gen(17)).to(gpu)
+    gi = ops._softmax_backward_data(g, y, -1, torch.float16)
+    assert gi.dtype == torch.float16
+    assert_close(gi, ops._softmax_backward_data(g, y, -1, torch.float32), torch.float16, "grad_input")
+    with pytest.raises(RuntimeError, match="Half type only"):
+        ops._softmax(x.bfloat16(), -1, True)
+
+
+def test_unsupported_dtype_is_an_error_not_a_fallback(ops, gpu):
+    x = torch.randn(4, 8, dtype=torch.float64, device=gpu)
+    with pytest.raises(RuntimeError, match="not implemented by the MI355X kernels"):
+        ops.native_layer_norm(x, [8], None, None, 1e-5)
+    with pytest.raises(RuntimeError, match="not implemented by the MI355X kernels"):
+        ops._softmax(x, -1, False)
+
+
+def test_aten_override_runs_autograd_end_to_end(pkg, gpu):
+    """Explicit opt-in routing of the aten ops to these kernels: F.layer_norm / F.rms_norm /
+    F.softmax / F.log_softmax with autograd on the GPU against the same on the CPU."""
+    import warnings
+    with warnings.catch_warnings():
+        warnings.simplefilter("ignore")
+        pkg.override_aten_ops()
+    for dtype in (torch.float32, torch.bfloat16):
+        x = torch.randn(6, 40, 256, generator=gen(20)).to(dtype)
+        w = torch.randn(256, generator=gen(21)).to(dtype)
+        b = torch.randn(256, generator=gen(22)).to(dtype)
+        dy = torch.randn(6, 40, 256, generator=gen(23)).to(dtype)
+        # one op at a time (a chain of bfloat16 ops rounds between the ops, which a float32
+        # reference chain does not), plus the whole chain in float32
+        stages = {
+            "layer_norm": lambda xs, ws, bs: F.layer_norm(xs, (256,), ws, bs, 1e-5),
+            "rms_norm": lambda xs, ws, bs: F.rms_norm(xs, (256,), ws, 1e-6),
+            "softmax": lambda xs, ws, bs: F.softmax(xs * ws + bs, -1),
+            "log_softmax": lambda xs, ws, bs: F.log_softmax(xs * ws + bs, -1),
+        }
+        if dtype == torch.float32:
+            stages["chain"] = lambda xs, ws, bs: (
+                F.softmax(F.rms_norm(F.layer_norm(xs, (256,), ws, bs, 1e-5), (256,), ws, 1e-6), -1)
+                + F.log_softmax(F.layer_norm(xs, (256,), ws, bs, 1e-5), -1))
+
+        for name, fn in stages.items():
+            def run(dev, upcast):
+                cast = (lambda t: t.float()) if upcast else (lambda t: t)
+                xs, ws, bs = (cast(t).to(dev).requires_grad_() for t in (x, w, b))
+                out = fn(xs, ws, bs)
+                out.backward(cast(dy).to(dev))
+                return out, xs.grad, ws.grad, bs.grad
+
+            got = run(gpu, False)
+            ref = run("cpu", True)
+            for a, r, nm in zip(got, ref, ("out", "dx", "dw", "db")):
+                if r is None:  # rms_norm has no bias
+                    assert a is None
+                    continue
+                assert a.dtype == dtype
+                assert_close(a, r, dtype, "%s %s" % (name, nm), scale=4.0)

@@ -187,8 +187,8 @@ Tensor& _log_softmax_out(const Tensor& self, int64_t dim, bool half_to_float, Te
 
 Tensor _softmax_backward_data(const Tensor& grad_output, const Tensor& output, int64_t dim,
                               at::ScalarType input_dtype) {
-  check_gpu(grad_output, "mi355x::_softmax_backward_data", "grad_output");
   const bool h2f = backward_half_to_float(grad_output, input_dtype);
+  check_gpu(grad_output, "mi355x::_softmax_backward_data", "grad_output");
   Tensor gi = at::empty_like(grad_output, grad_output.options().dtype(input_dtype),
                              at::MemoryFormat::Contiguous);
   _softmax_backward_kernel(grad_output, output, dim, h2f, gi);
@@ -196,8 +196,8 @@ Tensor _softmax_backward_data(const Tensor& grad_output, const Tensor& output, i
 }
 Tensor _log_softmax_backward_data(const Tensor& grad_output, const Tensor& output, int64_t dim,
                                   at::ScalarType input_dtype) {
-  check_gpu(grad_output, "mi355x::_log_softmax_backward_data", "grad_output");
   const bool h2f = backward_half_to_float(grad_output, input_dtype);
+  check_gpu(grad_output, "mi355x::_log_softmax_backward_data", "grad_output");
   Tensor gi = at::empty_like(grad_output, grad_output.options().dtype(input_dtype),
                              at::MemoryFormat::Contiguous);
   _log_softmax_backward_kernel(grad_output, output, dim, h2f, gi);

@@ -80,6 +80,21 @@ struct Pack {
   __device__ __forceinline__ void set(int i, float f) { v[i] = (T)f; }
 };
 
+// Optimization barrier on a register-resident pack of 16-bit elements.  A row
+// that must survive a cross-lane reduction is kept in storage format (two
+// elements per VGPR) and widened to fp32 again in each pass over it; without
+// the barrier the compiler would keep the widened copy alive across the
+// reduction instead, doubling the registers the row occupies.
+template <class T, int E>
+__device__ __forceinline__ void keep_packed(Pack<T, E>& p) {
+  if constexpr (sizeof(T) == 2 && E == 8) {
+    typedef uint32_t raw_t __attribute__((ext_vector_type(4)));
+    raw_t r = __builtin_bit_cast(raw_t, p.v);
+    asm volatile("" : "+v"(r));
+    p.v = __builtin_bit_cast(typename Pack<T, E>::vec_t, r);
+  }
+}
+
 // Loads the pack that starts at element `e0` of a row of `n` elements.  A pack
 // that lies wholly inside the row is one 128-bit load; the (at most one) pack
 // that straddles the end of the row is read element by element and padded with
@@ -112,6 +127,43 @@ __device__ __forceinline__ void store_row_pack(T* row, int e0, int n, bool row_o
 #pragma unroll
     for (int i = 0; i < E; ++i)
       if (e0 + i < n) row[e0 + i] = p.v[i];
+  }
+}
+
+// Row accessors used by the register-resident kernels.
+//
+// FAST (the row length is a whole number of packs): the load is unconditional
+// -- a lane whose pack lies beyond the row reads the row's first pack instead
+// and the value is replaced by `fill` with a select -- so the V loads of a lane
+// are straight-line code that the hardware issues back to back.  `row` must
+// point at a readable row even when `ok` is false (callers clamp the index).
+// Otherwise: the general loader above (handles a pack that straddles the row
+// end element by element, at the price of a branch per pack).
+template <class T, int E, bool STREAM, bool FAST>
+__device__ __forceinline__ Pack<T, E> row_load(const T* row, int e0, int n, bool ok, float fill) {
+  if constexpr (FAST) {
+    const bool inb = e0 < n;
+    const T* p = row + (inb ? e0 : 0);
+    Pack<T, E> r = STREAM ? Pack<T, E>::load_stream(p) : Pack<T, E>::load(p);
+    const Pack<T, E> f = Pack<T, E>::splat(fill);
+    if (!(inb && ok)) r = f;
+    return r;
+  } else {
+    return load_row_pack<T, E, STREAM>(row, e0, n, ok, fill);
+  }
+}
+
+template <class T, int E, bool STREAM, bool FAST>
+__device__ __forceinline__ void row_store(T* row, int e0, int n, bool ok, const Pack<T, E>& p) {
+  if constexpr (FAST) {
+    if (ok && e0 < n) {
+      if (STREAM)
+        p.store_stream(row + e0);
+      else
+        p.store(row + e0);
+    }
+  } else {
+    store_row_pack<T, E, STREAM>(row, e0, n, ok, p);
   }
 }
 

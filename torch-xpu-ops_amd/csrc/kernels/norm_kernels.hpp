@@ -25,15 +25,12 @@
 // are fp32 whatever the weight dtype; every access is 128 bits wide for any
 // pointer alignment; the weight dtype is independent of the row dtype.
 #pragma once
+#include <type_traits>
+
 #include "device/pack.hpp"
 #include "device/reduce.hpp"
 
 namespace rownorm {
-
-template <int G>
-struct block_for {
-  static constexpr int value = G <= 256 ? 256 : G;
-};
 
 // ---------------------------------------------------------------------------
 // Forward, row resident in registers: one read of X, one write of Y.
@@ -45,7 +42,9 @@ struct block_for {
 // and y is beta bit for bit, which is what the CPU kernel's Welford pass gives
 // (Welford recurrence being followed: src/ATen/native/xpu/sycl/
 // SharedReduceOps.h:56-88).
-template <class T, class WT, int G, int V, int BLOCK, bool RMS>
+//
+// FAST: N is a whole number of packs (see row_load in device/pack.hpp).
+template <class T, class WT, int G, int V, int BLOCK, bool RMS, bool FAST>
 __global__ void __launch_bounds__(BLOCK)
 norm_fwd_resident_kernel(const T* __restrict__ x, const WT* __restrict__ gamma,
                          const WT* __restrict__ beta, T* __restrict__ y,
@@ -59,46 +58,44 @@ norm_fwd_resident_kernel(const T* __restrict__ x, const WT* __restrict__ gamma,
   const int lane = threadIdx.x % G;
   const float fN = (float)N;
 
-  float gam[V][E];
-  float bet[RMS ? 1 : V][RMS ? 1 : E];
+  // gamma/beta of this lane's columns stay in registers for all rows: widened to
+  // fp32 once when they are few, otherwise in storage format and widened per row.
+  constexpr bool kWideWeights = V * E <= 16;
+  const bool exact = N == G * V * E;  // every pack of every lane lies inside the row
+  Pack<WT, E> gp[V];
+  Pack<WT, E> bp[RMS ? 1 : V];
 #pragma unroll
   for (int c = 0; c < V; ++c) {
     const int e0 = (c * G + lane) * E;
-    Pack<WT, E> pg = gamma ? load_row_pack<WT, E, false>(gamma, e0, N, true, 1.0f)
-                           : Pack<WT, E>::splat(1.0f);
-#pragma unroll
-    for (int i = 0; i < E; ++i) gam[c][i] = pg.get(i);
-    if constexpr (!RMS) {
-      Pack<WT, E> pb = beta ? load_row_pack<WT, E, false>(beta, e0, N, true, 0.0f)
-                            : Pack<WT, E>::zero();
-#pragma unroll
-      for (int i = 0; i < E; ++i) bet[c][i] = pb.get(i);
-    }
+    gp[c] = gamma ? load_row_pack<WT, E, false>(gamma, e0, N, true, 1.0f)
+                  : Pack<WT, E>::splat(1.0f);
+    if constexpr (!RMS)
+      bp[c] = beta ? load_row_pack<WT, E, false>(beta, e0, N, true, 0.0f) : Pack<WT, E>::zero();
   }
 
   const int64_t nrb = (M + RPB - 1) / RPB;
   for (int64_t rb = blockIdx.x; rb < nrb; rb += gridDim.x) {
     const int64_t row = rb * RPB + slot;
-    const bool ok = row < M;
-    const T* xr = x + row * (int64_t)N;
+    const bool ok = RPB == 1 ? true : row < M;
+    const T* xr = x + (ok ? row : 0) * (int64_t)N;
     T* yr = y + row * (int64_t)N;
 
-    float xf[V][E];
+    Pack<T, E> xp[V];
 #pragma unroll
-    for (int c = 0; c < V; ++c) {
-      const int e0 = (c * G + lane) * E;
-      const Pack<T, E> p = load_row_pack<T, E, true>(xr, e0, N, ok, 0.0f);
-#pragma unroll
-      for (int i = 0; i < E; ++i) xf[c][i] = p.get(i);
-    }
+    for (int c = 0; c < V; ++c)
+      xp[c] = row_load<T, E, true, FAST>(xr, (c * G + lane) * E, N, ok, 0.0f);
 
     float mu = 0.0f, rs;
+    float mean0 = 0.0f, m1 = 0.0f;
     if constexpr (RMS) {
       float acc[1] = {0.0f};
 #pragma unroll
       for (int c = 0; c < V; ++c)
 #pragma unroll
-        for (int i = 0; i < E; ++i) acc[0] = fmaf(xf[c][i], xf[c][i], acc[0]);
+        for (int i = 0; i < E; ++i) {
+          const float v = xp[c].get(i);
+          acc[0] = fmaf(v, v, acc[0]);
+        }
       group_allreduce<G, BLOCK, 1, SumOp>(acc, red, phase);
       rs = 1.0f / sqrtf(acc[0] / fN + eps);
     } else {
@@ -106,42 +103,61 @@ norm_fwd_resident_kernel(const T* __restrict__ x, const WT* __restrict__ gamma,
 #pragma unroll
       for (int c = 0; c < V; ++c)
 #pragma unroll
-        for (int i = 0; i < E; ++i) acc0[0] += xf[c][i];
+        for (int i = 0; i < E; ++i) acc0[0] += xp[c].get(i);
       group_allreduce<G, BLOCK, 1, SumOp>(acc0, red, phase);
-      const float mean0 = acc0[0] / fN;
+      mean0 = acc0[0] / fN;
       float acc[2] = {0.0f, 0.0f};
+      // MASKED: some packs reach past the row end; their elements must not count.
+      auto centred_sums = [&](auto masked) {
+        constexpr bool MASKED = decltype(masked)::value;
 #pragma unroll
-      for (int c = 0; c < V; ++c) {
-        const int e0 = (c * G + lane) * E;
-        const int nvalid = ok ? N - e0 : 0;  // elements of this pack inside the row
+        for (int c = 0; c < V; ++c) {
+          keep_packed(xp[c]);
+          const int nvalid = ok ? N - (c * G + lane) * E : 0;  // elements inside the row
 #pragma unroll
-        for (int i = 0; i < E; ++i) {
-          const float d = (i < nvalid) ? xf[c][i] - mean0 : 0.0f;
-          acc[0] += d;
-          acc[1] = fmaf(d, d, acc[1]);
+          for (int i = 0; i < E; ++i) {
+            float d = xp[c].get(i) - mean0;
+            if constexpr (MASKED) d = (i < nvalid) ? d : 0.0f;
+            acc[0] += d;
+            acc[1] = fmaf(d, d, acc[1]);
+          }
         }
-      }
+      };
+      if (exact)
+        centred_sums(std::false_type{});
+      else
+        centred_sums(std::true_type{});
       group_allreduce<G, BLOCK, 2, SumOp>(acc, red, phase);
-      const float m1 = acc[0] / fN;
+      m1 = acc[0] / fN;
       mu = mean0 + m1;
       const float var = fmaxf((acc[1] - acc[0] * m1) / fN, 0.0f);
       rs = 1.0f / sqrtf(var + eps);
     }
 
+    // y = gamma * (rstd * (x - mean)) + beta with x - mean taken as (x - mean0) - m1:
+    // both differences are exact where it matters (constant rows give beta bit for
+    // bit) and the rounding of mean0 + m1 to one float never enters y.  (Keeping
+    // x - mean0 in fp32 registers from the previous pass would save two VALU ops an
+    // element; it measured slower: fewer wavefronts stay resident.)
 #pragma unroll
     for (int c = 0; c < V; ++c) {
-      const int e0 = (c * G + lane) * E;
+      keep_packed(xp[c]);
+      if constexpr (!kWideWeights) {
+        keep_packed(gp[c]);
+        if constexpr (!RMS) keep_packed(bp[c]);
+      }
       Pack<T, E> o;
 #pragma unroll
       for (int i = 0; i < E; ++i) {
         float v;
-        if constexpr (RMS)
-          v = (xf[c][i] * rs) * gam[c][i];
-        else
-          v = ((xf[c][i] - mu) * rs) * gam[c][i] + bet[c][i];
+        if constexpr (RMS) {
+          v = (xp[c].get(i) * rs) * gp[c].get(i);
+        } else {
+          v = (((xp[c].get(i) - mean0) - m1) * rs) * gp[c].get(i) + bp[c].get(i);
+        }
         o.set(i, v);
       }
-      store_row_pack<T, E, true>(yr, e0, N, ok, o);
+      row_store<T, E, true, FAST>(yr, (c * G + lane) * E, N, ok, o);
     }
     if (ok && lane == 0) {
       if constexpr (!RMS)
@@ -244,7 +260,7 @@ norm_fwd_stream_kernel(const T* __restrict__ x, const WT* __restrict__ gamma,
 //   s1 = sum dy*gamma            s2 = sum dy*gamma*xhat       xhat = (x-mean)*rstd
 //   dx = (rstd/N) * (N*gamma*dy - xhat*s2 - s1)               (RMS: mean = 0, no s1)
 //   dgamma[j] = sum_rows dy*xhat   dbeta[j] = sum_rows dy
-template <class T, class WT, int G, int V, int BLOCK, bool RMS>
+template <class T, class WT, int G, int V, int BLOCK, bool RMS, bool FAST>
 __global__ void __launch_bounds__(BLOCK)
 norm_bwd_resident_kernel(const T* __restrict__ dy, const T* __restrict__ x,
                          const float* __restrict__ mean, const float* __restrict__ rstd,
@@ -261,18 +277,18 @@ norm_bwd_resident_kernel(const T* __restrict__ dy, const T* __restrict__ x,
   const int lane = threadIdx.x % G;
   const float fN = (float)N;
   const bool want_cols = part_dg != nullptr;  // uniform
+  constexpr bool kWideWeights = V * E <= 16;  // few weights: widen to fp32 once, not per row
 
-  float gam[V][E];
+  Pack<WT, E> gp[V];
   float dg[V][E];
   float db[RMS ? 1 : V][RMS ? 1 : E];
 #pragma unroll
   for (int c = 0; c < V; ++c) {
     const int e0 = (c * G + lane) * E;
-    Pack<WT, E> pg = gamma ? load_row_pack<WT, E, false>(gamma, e0, N, true, 1.0f)
-                           : Pack<WT, E>::splat(1.0f);
+    gp[c] = gamma ? load_row_pack<WT, E, false>(gamma, e0, N, true, 1.0f)
+                  : Pack<WT, E>::splat(1.0f);
 #pragma unroll
     for (int i = 0; i < E; ++i) {
-      gam[c][i] = pg.get(i);
       dg[c][i] = 0.0f;
       if constexpr (!RMS) db[c][i] = 0.0f;
     }
@@ -281,53 +297,77 @@ norm_bwd_resident_kernel(const T* __restrict__ dy, const T* __restrict__ x,
   const int64_t nrb = (M + RPB - 1) / RPB;
   for (int64_t rb = blockIdx.x; rb < nrb; rb += gridDim.x) {
     const int64_t row = rb * RPB + slot;
-    const bool ok = row < M;
-    const T* xr = x + row * (int64_t)N;
-    const T* gr = dy + row * (int64_t)N;
+    const bool ok = RPB == 1 ? true : row < M;
+    const int64_t rowc = ok ? row : 0;
+    const T* xr = x + rowc * (int64_t)N;
+    const T* gr = dy + rowc * (int64_t)N;
     float mu = 0.0f;
-    if constexpr (!RMS) mu = ok ? mean[row] : 0.0f;
-    const float rs = ok ? rstd[row] : 0.0f;
+    if constexpr (!RMS) mu = mean[rowc];
+    const float rs = rstd[rowc];
 
-    float xh[V][E];  // xhat
-    float gy[V][E];  // dy
+    // A row slot past the end of the tensor gets all-zero x and dy, so it adds
+    // nothing to the column sums; its dx is not stored.
+    Pack<T, E> xp[V], dp[V];
 #pragma unroll
     for (int c = 0; c < V; ++c) {
       const int e0 = (c * G + lane) * E;
-      const Pack<T, E> px = load_row_pack<T, E, true>(xr, e0, N, ok, 0.0f);
-      const Pack<T, E> pd = load_row_pack<T, E, true>(gr, e0, N, ok, 0.0f);
-#pragma unroll
-      for (int i = 0; i < E; ++i) {
-        xh[c][i] = RMS ? px.get(i) * rs : (px.get(i) - mu) * rs;
-        gy[c][i] = pd.get(i);
-      }
+      xp[c] = row_load<T, E, true, FAST>(xr, e0, N, ok, 0.0f);
+      dp[c] = row_load<T, E, true, FAST>(gr, e0, N, ok, 0.0f);
     }
+    // 16-bit rows: xhat = x*rs - mu*rs in one FMA (rounding far below a 16-bit
+    // ulp); fp32 rows keep the cancellation-free (x - mu) * rs.
+    const float nmr = -mu * rs;
     float acc[2] = {0.0f, 0.0f};
 #pragma unroll
-    for (int c = 0; c < V; ++c)
+    for (int c = 0; c < V; ++c) {
+      if constexpr (!kWideWeights) keep_packed(gp[c]);
 #pragma unroll
       for (int i = 0; i < E; ++i) {
-        const float g = gy[c][i] * gam[c][i];
+        const float xh = RMS ? xp[c].get(i) * rs
+                             : (sizeof(T) == 2 ? fmaf(xp[c].get(i), rs, nmr)
+                                               : (xp[c].get(i) - mu) * rs);
+        const float gy = dp[c].get(i);
+        const float g = gy * gp[c].get(i);
         if constexpr (!RMS) acc[0] += g;
-        acc[1] = fmaf(g, xh[c][i], acc[1]);
-        dg[c][i] = fmaf(gy[c][i], xh[c][i], dg[c][i]);
-        if constexpr (!RMS) db[c][i] += gy[c][i];
+        acc[1] = fmaf(g, xh, acc[1]);
+        dg[c][i] = fmaf(gy, xh, dg[c][i]);
+        if constexpr (!RMS) db[c][i] += gy;
       }
+    }
     group_allreduce<G, BLOCK, 2, SumOp>(acc, red, phase);
     if (dx != nullptr) {
       T* dr = dx + row * (int64_t)N;
+      // dx = (rs/N) * (N*g - xhat*s2 - s1), g = dy*gamma.  fp32 rows evaluate it
+      // in this order (N*g - s1 cancels exactly where it should).  16-bit rows
+      // use the regrouped rs*g - x*(rs*a) + (mu*rs*a - b), a = s2*rs/N,
+      // b = s1*rs/N: two FMAs, rounding far below a 16-bit ulp.
       const float term1 = rs / fN;
+      const float a = acc[1] * term1;
+      const float b = RMS ? 0.0f : acc[0] * term1;
+      const float ra = rs * a;
+      const float cc = mu * ra - b;
 #pragma unroll
       for (int c = 0; c < V; ++c) {
-        const int e0 = (c * G + lane) * E;
+        keep_packed(xp[c]);
+        keep_packed(dp[c]);
+        if constexpr (!kWideWeights) keep_packed(gp[c]);
         Pack<T, E> o;
 #pragma unroll
         for (int i = 0; i < E; ++i) {
-          float f = fN * (gy[c][i] * gam[c][i]);
-          f -= xh[c][i] * acc[1];
-          if constexpr (!RMS) f -= acc[0];
-          o.set(i, f * term1);
+          const float g = dp[c].get(i) * gp[c].get(i);
+          float f;
+          if constexpr (sizeof(T) == 2) {
+            f = fmaf(xp[c].get(i), -ra, fmaf(g, rs, cc));
+          } else {
+            const float xh = RMS ? xp[c].get(i) * rs : (xp[c].get(i) - mu) * rs;
+            f = fN * g;
+            f -= xh * acc[1];
+            if constexpr (!RMS) f -= acc[0];
+            f *= term1;
+          }
+          o.set(i, f);
         }
-        store_row_pack<T, E, true>(dr, e0, N, ok, o);
+        row_store<T, E, true, FAST>(dr, (c * G + lane) * E, N, ok, o);
       }
     }
   }
@@ -483,39 +523,57 @@ norm_bwd_stream_colsum_kernel(const T* __restrict__ dy, const T* __restrict__ x,
 
 // ---------------------------------------------------------------------------
 // Second stage of the dgamma/dbeta reduction: out[j] = sum_p part[p][j], rows
-// added in a fixed order.  A workgroup of 256 threads covers 64 columns with
-// 4 row lanes per column... see COLS/ROWS below: COLS threads across (4-byte
-// coalesced), ROWS threads down, LDS tree over the ROWS partial sums.
-// blockIdx.y selects dgamma (0) or dbeta (1).
+// added in a fixed order (deterministic).  A workgroup of 1024 threads covers
+// 64 columns: 16 threads across, each owning 4 adjacent columns (one 16-byte
+// load per partial row), 64 threads down striding over the P partial rows; the
+// 64 row sums of a column are then added through LDS.  blockIdx.y selects
+// dgamma (0) or dbeta (1).  Stands in for the at::sum(0) over the block
+// buffers in the reference (LayerNormKernels.cpp:1312-1314).
+constexpr int kFinalizeCols = 64;
+
 template <class WT>
-__global__ void __launch_bounds__(256)
+__global__ void __launch_bounds__(1024)
 colsum_finalize_kernel(const float* __restrict__ part0, const float* __restrict__ part1,
                        WT* __restrict__ out0, WT* __restrict__ out1, int P, int N) {
-  constexpr int COLS = 32, ROWS = 8;
-  __shared__ float tile[ROWS][COLS + 1];
+  constexpr int CQ = kFinalizeCols / 4, RL = 1024 / CQ;
+  __shared__ float tile[RL][kFinalizeCols + 1];
   const float* part = blockIdx.y == 0 ? part0 : part1;
   WT* out = blockIdx.y == 0 ? out0 : out1;
   if (part == nullptr || out == nullptr) return;  // uniform per workgroup
-  const int cx = threadIdx.x % COLS, ry = threadIdx.x / COLS;
-  const int col = blockIdx.x * COLS + cx;
-  float a0 = 0.0f, a1 = 0.0f, a2 = 0.0f, a3 = 0.0f;
-  if (col < N) {
-    int p = ry;
-    for (; p + 3 * ROWS < P; p += 4 * ROWS) {
-      a0 += part[(int64_t)p * N + col];
-      a1 += part[(int64_t)(p + ROWS) * N + col];
-      a2 += part[(int64_t)(p + 2 * ROWS) * N + col];
-      a3 += part[(int64_t)(p + 3 * ROWS) * N + col];
-    }
-    for (; p < P; p += ROWS) a0 += part[(int64_t)p * N + col];
-  }
-  tile[ry][cx] = (a0 + a1) + (a2 + a3);
-  __syncthreads();
-  if (ry == 0 && col < N) {
-    float s = tile[0][cx];
+  const int cq = threadIdx.x % CQ, rl = threadIdx.x / CQ;
+  const int col0 = blockIdx.x * kFinalizeCols + cq * 4;
+  float a[4] = {0.0f, 0.0f, 0.0f, 0.0f};
+  float b[4] = {0.0f, 0.0f, 0.0f, 0.0f};
+  int p = rl;
+  for (; p + RL < P; p += 2 * RL) {
+    const Pack<float, 4> v0 = load_row_pack<float, 4, false>(part + (int64_t)p * N, col0, N, true, 0.0f);
+    const Pack<float, 4> v1 =
+        load_row_pack<float, 4, false>(part + (int64_t)(p + RL) * N, col0, N, true, 0.0f);
 #pragma unroll
-    for (int r = 1; r < ROWS; ++r) s += tile[r][cx];
-    out[col] = (WT)s;
+    for (int i = 0; i < 4; ++i) {
+      a[i] += v0.get(i);
+      b[i] += v1.get(i);
+    }
+  }
+  if (p < P) {
+    const Pack<float, 4> v0 = load_row_pack<float, 4, false>(part + (int64_t)p * N, col0, N, true, 0.0f);
+#pragma unroll
+    for (int i = 0; i < 4; ++i) a[i] += v0.get(i);
+  }
+#pragma unroll
+  for (int i = 0; i < 4; ++i) tile[rl][cq * 4 + i] = a[i] + b[i];
+  __syncthreads();
+  if (threadIdx.x < kFinalizeCols) {
+    const int col = blockIdx.x * kFinalizeCols + threadIdx.x;
+    float s0 = 0.0f, s1 = 0.0f, s2 = 0.0f, s3 = 0.0f;
+#pragma unroll
+    for (int r = 0; r < RL; r += 4) {
+      s0 += tile[r][threadIdx.x];
+      s1 += tile[r + 1][threadIdx.x];
+      s2 += tile[r + 2][threadIdx.x];
+      s3 += tile[r + 3][threadIdx.x];
+    }
+    if (col < N) out[col] = (WT)((s0 + s1) + (s2 + s3));
   }
 }
 

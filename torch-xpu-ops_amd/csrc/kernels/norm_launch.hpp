@@ -12,15 +12,15 @@ struct NormFwdCtx {
   hipStream_t stream;
 };
 
-template <class T, class WT, bool RMS>
+template <class T, class WT, bool RMS, bool FAST>
 struct NormFwdLauncher {
   template <int G, int V, int BLOCK>
   struct At {
     static bool run(const NormFwdCtx<T, WT, RMS>& c) {
-      if constexpr (variant_built(OC_NORM_FWD, sizeof(T), G, V) &&
+      if constexpr (variant_built(OC_NORM_FWD, sizeof(T), G, V, FAST) &&
                     block_built(OC_NORM_FWD, G, BLOCK)) {
         if (c.plan.G == G && c.plan.V == V && c.plan.block == BLOCK) {
-          hipLaunchKernelGGL((norm_fwd_resident_kernel<T, WT, G, V, BLOCK, RMS>),
+          hipLaunchKernelGGL((norm_fwd_resident_kernel<T, WT, G, V, BLOCK, RMS, FAST>),
                              dim3((unsigned)c.plan.grid), dim3(BLOCK), 0, c.stream,
                              (const T*)c.a.x, (const WT*)c.a.gamma, (const WT*)c.a.beta,
                              (T*)c.a.y, c.a.mean, c.a.rstd, c.a.M, c.a.N, c.a.eps);
@@ -36,8 +36,10 @@ template <class T, class WT, bool RMS>
 int launch_norm_fwd(const Plan& plan, const NormFwdArgs& a, hipStream_t stream) {
   if (plan.resident) {
     NormFwdCtx<T, WT, RMS> ctx{plan, a, stream};
-    if (!launch_variant<NormFwdLauncher<T, WT, RMS>::template At>(ctx))
-      return (int)hipErrorInvalidConfiguration;
+    const bool launched =
+        plan.fast ? launch_variant<NormFwdLauncher<T, WT, RMS, true>::template At>(ctx)
+                  : launch_variant<NormFwdLauncher<T, WT, RMS, false>::template At>(ctx);
+    if (!launched) return (int)hipErrorInvalidConfiguration;
   } else {
     hipLaunchKernelGGL((norm_fwd_stream_kernel<T, WT, kStreamBlock, RMS>),
                        dim3((unsigned)plan.grid), dim3(kStreamBlock), 0, stream, (const T*)a.x,
@@ -54,15 +56,15 @@ struct NormBwdCtx {
   hipStream_t stream;
 };
 
-template <class T, class WT, bool RMS>
+template <class T, class WT, bool RMS, bool FAST>
 struct NormBwdLauncher {
   template <int G, int V, int BLOCK>
   struct At {
     static bool run(const NormBwdCtx<T, WT, RMS>& c) {
-      if constexpr (variant_built(OC_NORM_BWD, sizeof(T), G, V) &&
+      if constexpr (variant_built(OC_NORM_BWD, sizeof(T), G, V, FAST) &&
                     block_built(OC_NORM_BWD, G, BLOCK)) {
         if (c.plan.G == G && c.plan.V == V && c.plan.block == BLOCK) {
-          hipLaunchKernelGGL((norm_bwd_resident_kernel<T, WT, G, V, BLOCK, RMS>),
+          hipLaunchKernelGGL((norm_bwd_resident_kernel<T, WT, G, V, BLOCK, RMS, FAST>),
                              dim3((unsigned)c.plan.grid), dim3(BLOCK), 0, c.stream,
                              (const T*)c.a.dy, (const T*)c.a.x, c.a.mean, c.a.rstd,
                              (const WT*)c.a.gamma, (T*)c.a.dx, c.a.part_dg, c.a.part_db, c.a.M,
@@ -80,8 +82,10 @@ int launch_norm_bwd(const Plan& plan, const NormBwdArgs& a, hipStream_t stream) 
   const bool want_cols = a.part_dg != nullptr;
   if (plan.resident) {
     NormBwdCtx<T, WT, RMS> ctx{plan, a, stream};
-    if (!launch_variant<NormBwdLauncher<T, WT, RMS>::template At>(ctx))
-      return (int)hipErrorInvalidConfiguration;
+    const bool launched =
+        plan.fast ? launch_variant<NormBwdLauncher<T, WT, RMS, true>::template At>(ctx)
+                  : launch_variant<NormBwdLauncher<T, WT, RMS, false>::template At>(ctx);
+    if (!launched) return (int)hipErrorInvalidConfiguration;
   } else {
     constexpr int E = elems_per_pack<T>::value;
     if (a.dx != nullptr) {
@@ -101,8 +105,8 @@ int launch_norm_bwd(const Plan& plan, const NormBwdArgs& a, hipStream_t stream) 
   }
   int err = (int)hipGetLastError();
   if (err != 0 || !want_cols) return err;
-  const unsigned gx = (unsigned)((a.N + 31) / 32);
-  hipLaunchKernelGGL((colsum_finalize_kernel<WT>), dim3(gx, RMS ? 1 : 2), dim3(256), 0, stream,
+  const unsigned gx = (unsigned)((a.N + kFinalizeCols - 1) / kFinalizeCols);
+  hipLaunchKernelGGL((colsum_finalize_kernel<WT>), dim3(gx, RMS ? 1 : 2), dim3(1024), 0, stream,
                      (const float*)a.part_dg, (const float*)a.part_db, (WT*)a.dgamma,
                      (WT*)a.dbeta, (int)plan.partial_rows, a.N);
   return (int)hipGetLastError();

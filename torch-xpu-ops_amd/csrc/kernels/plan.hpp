@@ -12,8 +12,10 @@
 //   G = smallest power of two in [8, 1024] with G * V_pref >= packs,
 //   V = smallest power of two with G * V >= packs.
 // If V exceeds the per-op register budget V_max the multi-pass streaming
-// kernel is used instead.  Workgroups are 256 threads (BLOCK/G rows each) or G
-// threads when G > 256; the grid is persistent: min(row blocks, CUs * k).
+// kernel is used instead.  Rows whose length is a whole number of packs take
+// the branch-free "fast" kernels; ragged rows (N % E != 0) take the general
+// ones, which exist for V = V_pref only.  Workgroup size and grid size per op
+// class are set by block_threads() and default_bpc() below.
 #pragma once
 #include <stdint.h>
 
@@ -27,6 +29,7 @@ struct Override {
 
 struct Plan {
   bool resident = true;
+  bool fast = true;  // N % E == 0: branch-free row access
   int G = 0, V = 0, block = 0, rpb = 0;
   int64_t grid = 0;
   int64_t partial_rows = 0;
@@ -38,15 +41,10 @@ constexpr int kMaxV = 16;
 constexpr int kStreamBlock = 1024;
 
 // Preferred packs per lane: what the G ladder aims for.
-constexpr int v_pref(OpClass oc, int esize) {
-  switch (oc) {
-    case OC_NORM_FWD: return esize == 4 ? 8 : 8;
-    case OC_NORM_BWD: return esize == 4 ? 4 : 2;
-    case OC_SOFTMAX_FWD: return esize == 4 ? 8 : 4;
-    case OC_SOFTMAX_BWD: return esize == 4 ? 4 : 4;
-  }
-  return 1;
-}
+// Measured on MI355X: 16 elements a lane (two 16-bit packs, four fp32 packs)
+// keeps the register count low enough for 8 wavefronts per SIMD, which beats
+// fewer, fatter lanes on every op of the family.
+constexpr int v_pref(OpClass, int esize) { return esize == 4 ? 4 : 2; }
 
 // Largest packs per lane the register file holds for a G-lane row group.
 // G = 1024 means 16 wavefronts per workgroup, i.e. at most 128 VGPRs a lane.
@@ -62,7 +60,15 @@ constexpr int v_max(OpClass oc, int esize, int G) {
   return v;
 }
 
-constexpr int block_threads(OpClass, int G) { return G <= 256 ? 256 : G; }
+// Threads per workgroup for a G-lane row group (measured choices):
+//   norm forward    256 (BLOCK/G rows per workgroup), G itself above that;
+//   norm backward   512 at least: two or more row slots share one partial row
+//                   of the dgamma/dbeta reduction;
+//   softmax         512 at least.
+constexpr int block_threads(OpClass oc, int G) {
+  const int floor_threads = oc == OC_NORM_FWD ? 256 : 512;
+  return G <= floor_threads ? floor_threads : G;
+}
 
 // Workgroup sizes a G-lane variant is compiled for.
 constexpr bool block_built(OpClass oc, int G, int block) {
@@ -74,20 +80,28 @@ constexpr bool block_built(OpClass oc, int G, int block) {
 #endif
 }
 
-// Workgroups per compute unit of the persistent grid.
+// Workgroups per compute unit of the grid-stride launch.  The norm kernels keep
+// gamma/beta (and the backward column sums) in registers across the rows of a
+// workgroup.  Forward: four times as many workgroups as fit on the machine at
+// once, so that they drift out of phase (a grid that is exactly resident runs
+// its load and store phases in lockstep and loses 5-10% bandwidth) while each
+// still amortizes its weight loads over several rows.  Backward: every
+// workgroup emits one partial row of the dgamma/dbeta reduction, so the grid
+// is just what is resident at 1024 threads per CU.  Softmax has no per-column
+// state: one workgroup per row block.
 constexpr int default_bpc(OpClass oc, int block) {
-  const bool bwd_cols = oc == OC_NORM_BWD;  // each workgroup emits a partial row: keep few
-  if (block <= 256) return bwd_cols ? 2 : 8;
-  if (block <= 512) return bwd_cols ? 1 : 4;
-  return bwd_cols ? 1 : 2;
+  if (oc == OC_NORM_FWD) return 4 * (2048 / block);
+  if (oc == OC_NORM_BWD) return 1024 / block;
+  return 1 << 20;
 }
 
 // Which (G, V) kernels exist in the library.  Kept in one place so the
 // dispatcher, the planner and the forced-variant check agree.
-constexpr bool variant_built(OpClass oc, int esize, int G, int V) {
+constexpr bool variant_built(OpClass oc, int esize, int G, int V, bool fast) {
   if (G < kMinG || G > kMaxG || (G & (G - 1)) || V < 1 || V > kMaxV || (V & (V - 1)))
     return false;
   if (V > v_max(oc, esize, G)) return false;
+  if (!fast) return V == v_pref(oc, esize);
 #ifdef ROWNORM_TUNE_WIDE
   return true;
 #else
@@ -108,6 +122,7 @@ inline int make_plan(OpClass oc, int64_t M, int64_t N, int esize, int num_cus, c
   Plan p;
   const int E = 16 / esize;
   const int64_t packs = (N + E - 1) / E;
+  p.fast = (N % E) == 0;
   if (num_cus <= 0) num_cus = 256;
   bool stream = ov.G < 0;
   if (!stream) {
@@ -123,10 +138,11 @@ inline int make_plan(OpClass oc, int64_t M, int64_t N, int esize, int num_cus, c
       V = ov.V;
     } else {
       V = pow2_ceil((packs + G - 1) / G);
+      if (!p.fast && V < v_pref(oc, esize)) V = v_pref(oc, esize);
     }
     const bool holds = (int64_t)G * V >= packs;
     const int block = ov.block > 0 ? ov.block : block_threads(oc, G);
-    const bool built = variant_built(oc, esize, G, V) && block_built(oc, G, block);
+    const bool built = variant_built(oc, esize, G, V, p.fast) && block_built(oc, G, block);
     if (ov.G > 0 || ov.V > 0 || ov.block > 0) {
       if (!holds || !built) return -5;
     }

@@ -31,7 +31,7 @@ __device__ __forceinline__ float row_exp(float v) {
     return __expf(v);
 }
 
-template <class TI, class TO, int G, int V, int BLOCK>
+template <class TI, class TO, int G, int V, int BLOCK, bool FAST>
 __global__ void __launch_bounds__(BLOCK)
 softmax_fwd_resident_kernel(const TI* __restrict__ x, TO* __restrict__ y, int64_t M, int N,
                             int is_log) {
@@ -45,17 +45,18 @@ softmax_fwd_resident_kernel(const TI* __restrict__ x, TO* __restrict__ y, int64_
   const int64_t nrb = (M + RPB - 1) / RPB;
   for (int64_t rb = blockIdx.x; rb < nrb; rb += gridDim.x) {
     const int64_t row = rb * RPB + slot;
-    const bool ok = row < M;
-    const TI* xr = x + row * (int64_t)N;
+    const bool ok = RPB == 1 ? true : row < M;
+    const TI* xr = x + (ok ? row : 0) * (int64_t)N;
     TO* yr = y + row * (int64_t)N;
+    Pack<TI, E> xp[V];
+#pragma unroll
+    for (int c = 0; c < V; ++c)
+      xp[c] = row_load<TI, E, true, FAST>(xr, (c * G + lane) * E, N, ok, -INFINITY);
     float xf[V][E];
 #pragma unroll
-    for (int c = 0; c < V; ++c) {
-      const int e0 = (c * G + lane) * E;
-      const Pack<TI, E> p = load_row_pack<TI, E, true>(xr, e0, N, ok, -INFINITY);
+    for (int c = 0; c < V; ++c)
 #pragma unroll
-      for (int i = 0; i < E; ++i) xf[c][i] = p.get(i);
-    }
+      for (int i = 0; i < E; ++i) xf[c][i] = xp[c].get(i);
     float mx[1] = {-INFINITY};
 #pragma unroll
     for (int c = 0; c < V; ++c)
@@ -90,7 +91,7 @@ softmax_fwd_resident_kernel(const TI* __restrict__ x, TO* __restrict__ y, int64_
       Pack<TO, E> o;
 #pragma unroll
       for (int i = 0; i < E; ++i) o.set(i, is_log ? xf[c][i] - k : xf[c][i] * k);
-      store_row_pack<TO, E, true>(yr, e0, N, ok, o);
+      row_store<TO, E, true, FAST>(yr, e0, N, ok, o);
     }
   }
 }
@@ -140,7 +141,7 @@ softmax_fwd_stream_kernel(const TI* __restrict__ x, TO* __restrict__ y, int64_t 
 
 // Backward.  TG: dtype of grad and of y (the saved forward output); TO: dtype
 // of the input gradient.
-template <class TG, class TO, int G, int V, int BLOCK>
+template <class TG, class TO, int G, int V, int BLOCK, bool FAST>
 __global__ void __launch_bounds__(BLOCK)
 softmax_bwd_resident_kernel(const TG* __restrict__ grad, const TG* __restrict__ y,
                             TO* __restrict__ gi, int64_t M, int N, int is_log) {
@@ -154,22 +155,26 @@ softmax_bwd_resident_kernel(const TG* __restrict__ grad, const TG* __restrict__ 
   const int64_t nrb = (M + RPB - 1) / RPB;
   for (int64_t rb = blockIdx.x; rb < nrb; rb += gridDim.x) {
     const int64_t row = rb * RPB + slot;
-    const bool ok = row < M;
-    const TG* gr = grad + row * (int64_t)N;
-    const TG* yr = y + row * (int64_t)N;
+    const bool ok = RPB == 1 ? true : row < M;
+    const int64_t rowc = ok ? row : 0;
+    const TG* gr = grad + rowc * (int64_t)N;
+    const TG* yr = y + rowc * (int64_t)N;
     TO* outr = gi + row * (int64_t)N;
-    float gf[V][E], yf[V][E];
+    Pack<TG, E> pg[V], py[V];
 #pragma unroll
     for (int c = 0; c < V; ++c) {
       const int e0 = (c * G + lane) * E;
-      const Pack<TG, E> pg = load_row_pack<TG, E, true>(gr, e0, N, ok, 0.0f);
-      const Pack<TG, E> py = load_row_pack<TG, E, true>(yr, e0, N, ok, 0.0f);
+      pg[c] = row_load<TG, E, true, FAST>(gr, e0, N, ok, 0.0f);
+      py[c] = row_load<TG, E, true, FAST>(yr, e0, N, ok, 0.0f);
+    }
+    float gf[V][E], yf[V][E];
+#pragma unroll
+    for (int c = 0; c < V; ++c)
 #pragma unroll
       for (int i = 0; i < E; ++i) {
-        gf[c][i] = pg.get(i);
-        yf[c][i] = py.get(i);
+        gf[c][i] = pg[c].get(i);
+        yf[c][i] = py[c].get(i);
       }
-    }
     float sum[1] = {0.0f};
     if (is_log) {
 #pragma unroll
@@ -194,7 +199,7 @@ softmax_bwd_resident_kernel(const TG* __restrict__ grad, const TG* __restrict__ 
                                : yf[c][i] * (gf[c][i] - s);
         o.set(i, v);
       }
-      store_row_pack<TO, E, true>(outr, e0, N, ok, o);
+      row_store<TO, E, true, FAST>(outr, e0, N, ok, o);
     }
   }
 }
