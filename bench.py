@@ -12,8 +12,8 @@ Cache so that every step streams from HBM.
     python bench.py [--gpus 1] [--steps K] [--warmup W] [--no-ops] [--no-cpu]
 
 prints ONE JSON line (see the keys below).  `roofline` covers the dominant operation of the step,
-one mi355x_rms_norm_bwd call (norm_bwd_resident_kernel + colsum_finalize_kernel), timed with HIP
-events on the launch stream inside the timed region.  `cpu_baseline` is the scalar C oracle
+one mi355x_rms_norm_bwd call (norm_bwd_resident_kernel + colsum_finalize_kernel), timed with a
+HIP event pair per call on the launch stream over a second run of the same K steps.  `cpu_baseline` is the scalar C oracle
 (oracle/, a port of the same arithmetic) timed on one host core; `cpu_aten` is PyTorch's CPU ATen
 path (the parity target) on all host cores.  `ops` lists every op of the family at its
 Llama-class configuration (informational, measured after the timed region).
@@ -49,6 +49,9 @@ def main():
     ap.add_argument("--warmup", type=int, default=20)
     ap.add_argument("--no-ops", action="store_true", help="skip the per-op table")
     ap.add_argument("--no-cpu", action="store_true", help="skip the CPU baselines")
+    ap.add_argument("--calibrate-copy", action="store_true",
+                    help="also run a plain 256 MiB device copy 10 times (torch copy_), the "
+                         "known-size kernel that FETCH_SIZE / WRITE_SIZE readings are scaled by")
     args = ap.parse_args()
     if args.gpus != 1 or int(os.environ.get("WORLD_SIZE", "1")) != 1:
         print("bench.py: this operator family runs whole on one GPU (rows are independent; "
@@ -92,15 +95,36 @@ def main():
         return L.mi355x_rms_norm_bwd(P(s["dy"]), P(s["x"]), P(s["rstd"]), P(w), P(s["dx"]),
                                      P(s["dw"]), P(ws), ws_bytes, M, N, BF, BF, stream)
 
+    if args.calibrate_copy:
+        src = torch.empty(256 << 20, dtype=torch.uint8, device=dev).random_(0, 255)
+        dst = torch.empty_like(src)
+        for _ in range(10):
+            dst.copy_(src)
+        torch.cuda.synchronize()
+        del src, dst
+
     for i in range(args.warmup):
         s = sets[i % nsets]
         rc = fwd(s) or bwd(s)
         if rc != 0:
             raise RuntimeError("kernel launch failed: " + cabi.error_string(rc))
-    ev = [(torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True))
-          for _ in range(args.steps)]
+    # timed region: exactly K steps, bracketed by a device synchronize on both sides
     torch.cuda.synchronize()
     t0 = time.perf_counter()
+    for i in range(args.steps):
+        s = sets[i % nsets]
+        fwd(s)
+        bwd(s)
+    torch.cuda.synchronize()
+    t1 = time.perf_counter()
+    ms_per_step = (t1 - t0) * 1e3 / args.steps
+    value = (fwd_bytes + bwd_bytes) / (ms_per_step * 1e-3) / 1e9
+
+    # roofline of the dominant operation: the same steps again with a HIP event pair around
+    # every backward call on the launch stream (kept out of the timed region: an event record
+    # between two launches costs the GPU a few microseconds of idle time)
+    ev = [(torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True))
+          for _ in range(args.steps)]
     for i in range(args.steps):
         s = sets[i % nsets]
         fwd(s)
@@ -108,9 +132,6 @@ def main():
         bwd(s)
         ev[i][1].record()
     torch.cuda.synchronize()
-    t1 = time.perf_counter()
-    ms_per_step = (t1 - t0) * 1e3 / args.steps
-    value = (fwd_bytes + bwd_bytes) / (ms_per_step * 1e-3) / 1e9
     bwd_us = sum(a.elapsed_time(b) for a, b in ev) * 1e3 / args.steps
     achieved = bwd_bytes / (bwd_us * 1e-6) / 1e9
 

@@ -67,7 +67,7 @@ typedef struct {
   int32_t lanes_per_row;   /* G: lanes that share one row (8..1024) */
   int32_t packs_per_lane;  /* V: 16-byte packs each lane holds per row */
   int32_t block_threads;   /* threads per workgroup */
-  int32_t rows_per_block;  /* rows a workgroup handles per iteration */
+  int32_t rows_per_block;  /* rows a workgroup handles per iteration: block_threads / lanes_per_row */
   int32_t reserved;
   int64_t grid_blocks;     /* workgroups launched (persistent, grid-stride over rows) */
   int64_t partial_rows;    /* rows of the fp32 [partial_rows, N] column-sum workspace (backward only) */

@@ -44,15 +44,21 @@ namespace rownorm {
 // SharedReduceOps.h:56-88).
 //
 // FAST: N is a whole number of packs (see row_load in device/pack.hpp).
-template <class T, class WT, int G, int V, int BLOCK, bool RMS, bool FAST>
+// R: rows each lane group works on per iteration; their loads are issued
+// together and their sums share one reduction (one barrier for R rows).  The
+// library is built with R = 1: on MI355X R = 2 measured only 1-3% faster at
+// G >= 256 (and slower in the backward, whose two-row body needs over 150
+// VGPRs), not worth twice the kernels.
+template <class T, class WT, int G, int V, int BLOCK, int R, bool RMS, bool FAST>
 __global__ void __launch_bounds__(BLOCK)
 norm_fwd_resident_kernel(const T* __restrict__ x, const WT* __restrict__ gamma,
                          const WT* __restrict__ beta, T* __restrict__ y,
                          float* __restrict__ mean, float* __restrict__ rstd, int64_t M, int N,
                          float eps) {
   constexpr int E = elems_per_pack<T>::value;
-  constexpr int RPB = BLOCK / G;
-  __shared__ float red[reduce_lds_floats<G, BLOCK, 2>::value];
+  constexpr int RPB = BLOCK / G;  // row slots of the workgroup
+  constexpr int RPI = RPB * R;    // rows per workgroup iteration
+  __shared__ float red[reduce_lds_floats<G, BLOCK, 2 * R>::value];
   int phase = 0;
   const int slot = threadIdx.x / G;
   const int lane = threadIdx.x % G;
@@ -73,53 +79,70 @@ norm_fwd_resident_kernel(const T* __restrict__ x, const WT* __restrict__ gamma,
       bp[c] = beta ? load_row_pack<WT, E, false>(beta, e0, N, true, 0.0f) : Pack<WT, E>::zero();
   }
 
-  const int64_t nrb = (M + RPB - 1) / RPB;
+  const int64_t nrb = (M + RPI - 1) / RPI;
   for (int64_t rb = blockIdx.x; rb < nrb; rb += gridDim.x) {
-    const int64_t row = rb * RPB + slot;
-    const bool ok = RPB == 1 ? true : row < M;
-    const T* xr = x + (ok ? row : 0) * (int64_t)N;
-    T* yr = y + row * (int64_t)N;
-
-    Pack<T, E> xp[V];
+    const int64_t row0 = (rb * RPB + slot) * R;
+    bool ok[R];
+    Pack<T, E> xp[R][V];
 #pragma unroll
-    for (int c = 0; c < V; ++c)
-      xp[c] = row_load<T, E, true, FAST>(xr, (c * G + lane) * E, N, ok, 0.0f);
+    for (int r = 0; r < R; ++r) {
+      ok[r] = (RPI == 1) ? true : row0 + r < M;
+      const T* xr = x + (ok[r] ? row0 + r : 0) * (int64_t)N;
+#pragma unroll
+      for (int c = 0; c < V; ++c)
+        xp[r][c] = row_load<T, E, true, FAST>(xr, (c * G + lane) * E, N, ok[r], 0.0f);
+    }
 
-    float mu = 0.0f, rs;
-    float mean0 = 0.0f, m1 = 0.0f;
+    float mean0[R], m1[R], rs[R];
     if constexpr (RMS) {
-      float acc[1] = {0.0f};
+      float acc[R];
 #pragma unroll
-      for (int c = 0; c < V; ++c)
+      for (int r = 0; r < R; ++r) {
+        acc[r] = 0.0f;
 #pragma unroll
-        for (int i = 0; i < E; ++i) {
-          const float v = xp[c].get(i);
-          acc[0] = fmaf(v, v, acc[0]);
-        }
-      group_allreduce<G, BLOCK, 1, SumOp>(acc, red, phase);
-      rs = 1.0f / sqrtf(acc[0] / fN + eps);
+        for (int c = 0; c < V; ++c)
+#pragma unroll
+          for (int i = 0; i < E; ++i) {
+            const float v = xp[r][c].get(i);
+            acc[r] = fmaf(v, v, acc[r]);
+          }
+      }
+      group_allreduce<G, BLOCK, R, SumOp>(acc, red, phase);
+#pragma unroll
+      for (int r = 0; r < R; ++r) {
+        rs[r] = 1.0f / sqrtf(acc[r] / fN + eps);
+        mean0[r] = m1[r] = 0.0f;
+      }
     } else {
-      float acc0[1] = {0.0f};
+      float acc0[R];
 #pragma unroll
-      for (int c = 0; c < V; ++c)
+      for (int r = 0; r < R; ++r) {
+        acc0[r] = 0.0f;
 #pragma unroll
-        for (int i = 0; i < E; ++i) acc0[0] += xp[c].get(i);
-      group_allreduce<G, BLOCK, 1, SumOp>(acc0, red, phase);
-      mean0 = acc0[0] / fN;
-      float acc[2] = {0.0f, 0.0f};
+        for (int c = 0; c < V; ++c)
+#pragma unroll
+          for (int i = 0; i < E; ++i) acc0[r] += xp[r][c].get(i);
+      }
+      group_allreduce<G, BLOCK, R, SumOp>(acc0, red, phase);
+      float acc[2 * R];
       // MASKED: some packs reach past the row end; their elements must not count.
       auto centred_sums = [&](auto masked) {
         constexpr bool MASKED = decltype(masked)::value;
 #pragma unroll
-        for (int c = 0; c < V; ++c) {
-          keep_packed(xp[c]);
-          const int nvalid = ok ? N - (c * G + lane) * E : 0;  // elements inside the row
+        for (int r = 0; r < R; ++r) {
+          mean0[r] = acc0[r] / fN;
+          acc[2 * r] = acc[2 * r + 1] = 0.0f;
 #pragma unroll
-          for (int i = 0; i < E; ++i) {
-            float d = xp[c].get(i) - mean0;
-            if constexpr (MASKED) d = (i < nvalid) ? d : 0.0f;
-            acc[0] += d;
-            acc[1] = fmaf(d, d, acc[1]);
+          for (int c = 0; c < V; ++c) {
+            keep_packed(xp[r][c]);
+            const int nvalid = ok[r] ? N - (c * G + lane) * E : 0;  // elements inside the row
+#pragma unroll
+            for (int i = 0; i < E; ++i) {
+              float d = xp[r][c].get(i) - mean0[r];
+              if constexpr (MASKED) d = (i < nvalid) ? d : 0.0f;
+              acc[2 * r] += d;
+              acc[2 * r + 1] = fmaf(d, d, acc[2 * r + 1]);
+            }
           }
         }
       };
@@ -127,11 +150,13 @@ norm_fwd_resident_kernel(const T* __restrict__ x, const WT* __restrict__ gamma,
         centred_sums(std::false_type{});
       else
         centred_sums(std::true_type{});
-      group_allreduce<G, BLOCK, 2, SumOp>(acc, red, phase);
-      m1 = acc[0] / fN;
-      mu = mean0 + m1;
-      const float var = fmaxf((acc[1] - acc[0] * m1) / fN, 0.0f);
-      rs = 1.0f / sqrtf(var + eps);
+      group_allreduce<G, BLOCK, 2 * R, SumOp>(acc, red, phase);
+#pragma unroll
+      for (int r = 0; r < R; ++r) {
+        m1[r] = acc[2 * r] / fN;
+        const float var = fmaxf((acc[2 * r + 1] - acc[2 * r] * m1[r]) / fN, 0.0f);
+        rs[r] = 1.0f / sqrtf(var + eps);
+      }
     }
 
     // y = gamma * (rstd * (x - mean)) + beta with x - mean taken as (x - mean0) - m1:
@@ -140,29 +165,32 @@ norm_fwd_resident_kernel(const T* __restrict__ x, const WT* __restrict__ gamma,
     // x - mean0 in fp32 registers from the previous pass would save two VALU ops an
     // element; it measured slower: fewer wavefronts stay resident.)
 #pragma unroll
-    for (int c = 0; c < V; ++c) {
-      keep_packed(xp[c]);
-      if constexpr (!kWideWeights) {
-        keep_packed(gp[c]);
-        if constexpr (!RMS) keep_packed(bp[c]);
-      }
-      Pack<T, E> o;
+    for (int r = 0; r < R; ++r) {
+      T* yr = y + (row0 + r) * (int64_t)N;
 #pragma unroll
-      for (int i = 0; i < E; ++i) {
-        float v;
-        if constexpr (RMS) {
-          v = (xp[c].get(i) * rs) * gp[c].get(i);
-        } else {
-          v = (((xp[c].get(i) - mean0) - m1) * rs) * gp[c].get(i) + bp[c].get(i);
+      for (int c = 0; c < V; ++c) {
+        keep_packed(xp[r][c]);
+        if constexpr (!kWideWeights) {
+          keep_packed(gp[c]);
+          if constexpr (!RMS) keep_packed(bp[c]);
         }
-        o.set(i, v);
+        Pack<T, E> o;
+#pragma unroll
+        for (int i = 0; i < E; ++i) {
+          float v;
+          if constexpr (RMS)
+            v = (xp[r][c].get(i) * rs[r]) * gp[c].get(i);
+          else
+            v = (((xp[r][c].get(i) - mean0[r]) - m1[r]) * rs[r]) * gp[c].get(i) + bp[c].get(i);
+          o.set(i, v);
+        }
+        row_store<T, E, true, FAST>(yr, (c * G + lane) * E, N, ok[r], o);
       }
-      row_store<T, E, true, FAST>(yr, (c * G + lane) * E, N, ok, o);
-    }
-    if (ok && lane == 0) {
-      if constexpr (!RMS)
-        if (mean) mean[row] = mu;
-      if (rstd) rstd[row] = rs;
+      if (ok[r] && lane == 0) {
+        if constexpr (!RMS)
+          if (mean) mean[row0 + r] = mean0[r] + m1[r];
+        if (rstd) rstd[row0 + r] = rs[r];
+      }
     }
   }
 }
@@ -260,7 +288,7 @@ norm_fwd_stream_kernel(const T* __restrict__ x, const WT* __restrict__ gamma,
 //   s1 = sum dy*gamma            s2 = sum dy*gamma*xhat       xhat = (x-mean)*rstd
 //   dx = (rstd/N) * (N*gamma*dy - xhat*s2 - s1)               (RMS: mean = 0, no s1)
 //   dgamma[j] = sum_rows dy*xhat   dbeta[j] = sum_rows dy
-template <class T, class WT, int G, int V, int BLOCK, bool RMS, bool FAST>
+template <class T, class WT, int G, int V, int BLOCK, int R, bool RMS, bool FAST>
 __global__ void __launch_bounds__(BLOCK)
 norm_bwd_resident_kernel(const T* __restrict__ dy, const T* __restrict__ x,
                          const float* __restrict__ mean, const float* __restrict__ rstd,
@@ -268,9 +296,10 @@ norm_bwd_resident_kernel(const T* __restrict__ dy, const T* __restrict__ x,
                          float* __restrict__ part_dg, float* __restrict__ part_db, int64_t M,
                          int N) {
   constexpr int E = elems_per_pack<T>::value;
-  constexpr int RPB = BLOCK / G;
+  constexpr int RPB = BLOCK / G;  // row slots of the workgroup
+  constexpr int RPI = RPB * R;    // rows per workgroup iteration (R per slot, see the forward)
   constexpr int FOLD_FLOATS = (RPB > 1) ? G * V * E : 1;
-  __shared__ float red[reduce_lds_floats<G, BLOCK, 2>::value];
+  __shared__ float red[reduce_lds_floats<G, BLOCK, 2 * R>::value];
   __shared__ float fold[FOLD_FLOATS];
   int phase = 0;
   const int slot = threadIdx.x / G;
@@ -294,80 +323,90 @@ norm_bwd_resident_kernel(const T* __restrict__ dy, const T* __restrict__ x,
     }
   }
 
-  const int64_t nrb = (M + RPB - 1) / RPB;
+  const int64_t nrb = (M + RPI - 1) / RPI;
   for (int64_t rb = blockIdx.x; rb < nrb; rb += gridDim.x) {
-    const int64_t row = rb * RPB + slot;
-    const bool ok = RPB == 1 ? true : row < M;
-    const int64_t rowc = ok ? row : 0;
-    const T* xr = x + rowc * (int64_t)N;
-    const T* gr = dy + rowc * (int64_t)N;
-    float mu = 0.0f;
-    if constexpr (!RMS) mu = mean[rowc];
-    const float rs = rstd[rowc];
-
+    const int64_t row0 = (rb * RPB + slot) * R;
+    bool ok[R];
+    float mu[R], rs[R];
     // A row slot past the end of the tensor gets all-zero x and dy, so it adds
     // nothing to the column sums; its dx is not stored.
-    Pack<T, E> xp[V], dp[V];
+    Pack<T, E> xp[R][V], dp[R][V];
 #pragma unroll
-    for (int c = 0; c < V; ++c) {
-      const int e0 = (c * G + lane) * E;
-      xp[c] = row_load<T, E, true, FAST>(xr, e0, N, ok, 0.0f);
-      dp[c] = row_load<T, E, true, FAST>(gr, e0, N, ok, 0.0f);
-    }
-    // 16-bit rows: xhat = x*rs - mu*rs in one FMA (rounding far below a 16-bit
-    // ulp); fp32 rows keep the cancellation-free (x - mu) * rs.
-    const float nmr = -mu * rs;
-    float acc[2] = {0.0f, 0.0f};
-#pragma unroll
-    for (int c = 0; c < V; ++c) {
-      if constexpr (!kWideWeights) keep_packed(gp[c]);
-#pragma unroll
-      for (int i = 0; i < E; ++i) {
-        const float xh = RMS ? xp[c].get(i) * rs
-                             : (sizeof(T) == 2 ? fmaf(xp[c].get(i), rs, nmr)
-                                               : (xp[c].get(i) - mu) * rs);
-        const float gy = dp[c].get(i);
-        const float g = gy * gp[c].get(i);
-        if constexpr (!RMS) acc[0] += g;
-        acc[1] = fmaf(g, xh, acc[1]);
-        dg[c][i] = fmaf(gy, xh, dg[c][i]);
-        if constexpr (!RMS) db[c][i] += gy;
-      }
-    }
-    group_allreduce<G, BLOCK, 2, SumOp>(acc, red, phase);
-    if (dx != nullptr) {
-      T* dr = dx + row * (int64_t)N;
-      // dx = (rs/N) * (N*g - xhat*s2 - s1), g = dy*gamma.  fp32 rows evaluate it
-      // in this order (N*g - s1 cancels exactly where it should).  16-bit rows
-      // use the regrouped rs*g - x*(rs*a) + (mu*rs*a - b), a = s2*rs/N,
-      // b = s1*rs/N: two FMAs, rounding far below a 16-bit ulp.
-      const float term1 = rs / fN;
-      const float a = acc[1] * term1;
-      const float b = RMS ? 0.0f : acc[0] * term1;
-      const float ra = rs * a;
-      const float cc = mu * ra - b;
+    for (int r = 0; r < R; ++r) {
+      ok[r] = (RPI == 1) ? true : row0 + r < M;
+      const int64_t rowc = ok[r] ? row0 + r : 0;
+      mu[r] = RMS ? 0.0f : mean[rowc];
+      rs[r] = rstd[rowc];
 #pragma unroll
       for (int c = 0; c < V; ++c) {
-        keep_packed(xp[c]);
-        keep_packed(dp[c]);
+        const int e0 = (c * G + lane) * E;
+        xp[r][c] = row_load<T, E, true, FAST>(x + rowc * (int64_t)N, e0, N, ok[r], 0.0f);
+        dp[r][c] = row_load<T, E, true, FAST>(dy + rowc * (int64_t)N, e0, N, ok[r], 0.0f);
+      }
+    }
+    float acc[2 * R];
+#pragma unroll
+    for (int r = 0; r < R; ++r) {
+      // 16-bit rows: xhat = x*rs - mu*rs in one FMA (rounding far below a 16-bit
+      // ulp); fp32 rows keep the cancellation-free (x - mu) * rs.
+      const float nmr = -mu[r] * rs[r];
+      acc[2 * r] = acc[2 * r + 1] = 0.0f;
+#pragma unroll
+      for (int c = 0; c < V; ++c) {
         if constexpr (!kWideWeights) keep_packed(gp[c]);
-        Pack<T, E> o;
 #pragma unroll
         for (int i = 0; i < E; ++i) {
-          const float g = dp[c].get(i) * gp[c].get(i);
-          float f;
-          if constexpr (sizeof(T) == 2) {
-            f = fmaf(xp[c].get(i), -ra, fmaf(g, rs, cc));
-          } else {
-            const float xh = RMS ? xp[c].get(i) * rs : (xp[c].get(i) - mu) * rs;
-            f = fN * g;
-            f -= xh * acc[1];
-            if constexpr (!RMS) f -= acc[0];
-            f *= term1;
-          }
-          o.set(i, f);
+          const float xv = xp[r][c].get(i);
+          const float xh = RMS ? xv * rs[r]
+                               : (sizeof(T) == 2 ? fmaf(xv, rs[r], nmr) : (xv - mu[r]) * rs[r]);
+          const float gy = dp[r][c].get(i);
+          const float g = gy * gp[c].get(i);
+          if constexpr (!RMS) acc[2 * r] += g;
+          acc[2 * r + 1] = fmaf(g, xh, acc[2 * r + 1]);
+          dg[c][i] = fmaf(gy, xh, dg[c][i]);
+          if constexpr (!RMS) db[c][i] += gy;
         }
-        row_store<T, E, true, FAST>(dr, (c * G + lane) * E, N, ok, o);
+      }
+    }
+    group_allreduce<G, BLOCK, 2 * R, SumOp>(acc, red, phase);
+    if (dx != nullptr) {
+#pragma unroll
+      for (int r = 0; r < R; ++r) {
+        T* dr = dx + (row0 + r) * (int64_t)N;
+        // dx = (rs/N) * (N*g - xhat*s2 - s1), g = dy*gamma.  fp32 rows evaluate it
+        // in this order (N*g - s1 cancels exactly where it should).  16-bit rows
+        // use the regrouped rs*g - x*(rs*a) + (mu*rs*a - b), a = s2*rs/N,
+        // b = s1*rs/N: two FMAs, rounding far below a 16-bit ulp.
+        const float s1 = acc[2 * r], s2 = acc[2 * r + 1];
+        const float term1 = rs[r] / fN;
+        const float a = s2 * term1;
+        const float b = RMS ? 0.0f : s1 * term1;
+        const float ra = rs[r] * a;
+        const float cc = mu[r] * ra - b;
+#pragma unroll
+        for (int c = 0; c < V; ++c) {
+          keep_packed(xp[r][c]);
+          keep_packed(dp[r][c]);
+          if constexpr (!kWideWeights) keep_packed(gp[c]);
+          Pack<T, E> o;
+#pragma unroll
+          for (int i = 0; i < E; ++i) {
+            const float g = dp[r][c].get(i) * gp[c].get(i);
+            float f;
+            if constexpr (sizeof(T) == 2) {
+              f = fmaf(xp[r][c].get(i), -ra, fmaf(g, rs[r], cc));
+            } else {
+              const float xv = xp[r][c].get(i);
+              const float xh = RMS ? xv * rs[r] : (xv - mu[r]) * rs[r];
+              f = fN * g;
+              f -= xh * s2;
+              if constexpr (!RMS) f -= s1;
+              f *= term1;
+            }
+            o.set(i, f);
+          }
+          row_store<T, E, true, FAST>(dr, (c * G + lane) * E, N, ok[r], o);
+        }
       }
     }
   }

@@ -20,7 +20,7 @@ struct NormFwdLauncher {
       if constexpr (variant_built(OC_NORM_FWD, sizeof(T), G, V, FAST) &&
                     block_built(OC_NORM_FWD, G, BLOCK)) {
         if (c.plan.G == G && c.plan.V == V && c.plan.block == BLOCK) {
-          hipLaunchKernelGGL((norm_fwd_resident_kernel<T, WT, G, V, BLOCK, RMS, FAST>),
+          hipLaunchKernelGGL((norm_fwd_resident_kernel<T, WT, G, V, BLOCK, 1, RMS, FAST>),
                              dim3((unsigned)c.plan.grid), dim3(BLOCK), 0, c.stream,
                              (const T*)c.a.x, (const WT*)c.a.gamma, (const WT*)c.a.beta,
                              (T*)c.a.y, c.a.mean, c.a.rstd, c.a.M, c.a.N, c.a.eps);
@@ -64,7 +64,7 @@ struct NormBwdLauncher {
       if constexpr (variant_built(OC_NORM_BWD, sizeof(T), G, V, FAST) &&
                     block_built(OC_NORM_BWD, G, BLOCK)) {
         if (c.plan.G == G && c.plan.V == V && c.plan.block == BLOCK) {
-          hipLaunchKernelGGL((norm_bwd_resident_kernel<T, WT, G, V, BLOCK, RMS, FAST>),
+          hipLaunchKernelGGL((norm_bwd_resident_kernel<T, WT, G, V, BLOCK, 1, RMS, FAST>),
                              dim3((unsigned)c.plan.grid), dim3(BLOCK), 0, c.stream,
                              (const T*)c.a.dy, (const T*)c.a.x, c.a.mean, c.a.rstd,
                              (const WT*)c.a.gamma, (T*)c.a.dx, c.a.part_dg, c.a.part_db, c.a.M,

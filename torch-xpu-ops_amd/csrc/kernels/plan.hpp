@@ -152,6 +152,7 @@ inline int make_plan(OpClass oc, int64_t M, int64_t N, int esize, int num_cus, c
       p.V = V;
       p.block = block;
       p.rpb = p.block / G;
+
     } else {
       stream = true;
     }
