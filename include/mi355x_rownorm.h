@@ -138,6 +138,39 @@ int mi355x_softmax_bwd(const void* grad, const void* y, void* gi, int64_t rows, 
                        rownorm_dtype grad_dtype, rownorm_dtype gi_dtype, int is_log,
                        void* stream);
 
+/* _safe_softmax: softmax whose rows without any finite element (all -inf) come
+ * out as zeros instead of NaN.  Replaces _safe_softmax_kernel
+ * (SoftMaxKernels.h:45-46, SoftMaxKernels.cpp:2278-2299; the is_safe_softmax
+ * branches at SoftMaxKernels.cpp:328-346).  Dtypes as for mi355x_softmax_fwd. */
+int mi355x_safe_softmax_fwd(const void* x, void* y, int64_t rows, int64_t N,
+                            rownorm_dtype in_dtype, rownorm_dtype out_dtype, void* stream);
+
+/* _masked_softmax over the innermost dimension: elements whose mask byte is
+ * non-zero are left out (treated as -inf); a row with every element masked is
+ * NaN.  Replaces masked_softmax_kernel (SoftMaxKernels.h:48-52,
+ * SoftMaxKernels.cpp:1901-2020 and 2301-2359).  `mask` is a dense
+ * [mask_rows, N] buffer of one-byte booleans in device memory; data row r uses
+ * mask row (r / mask_row_div) * mask_row_stride + r % mask_row_mod:
+ *   mask of the input's shape            mask_rows = rows, div 1,   stride 1, mod 1
+ *   [B, T] under a [B, H, T, T] input    mask_rows = B,    div H*T, stride 1, mod 1
+ *   [T, T] under a [B, H, T, T] input    mask_rows = T,    div 1,   stride 0, mod T
+ *   [B, 1, T, T] under [B, H, T, T]      mask_rows = B*T,  div H*T, stride T, mod T
+ * A mapping that could leave the mask buffer, or rows >= 2^31, is rejected
+ * with ROWNORM_ERR_SHAPE.  Input and output share `dtype`. */
+int mi355x_masked_softmax_fwd(const void* x, const void* mask, void* y, int64_t rows, int64_t N,
+                              int64_t mask_rows, int64_t mask_row_div, int64_t mask_row_stride,
+                              int64_t mask_row_mod, rownorm_dtype dtype, void* stream);
+
+/* _masked_softmax_backward: softmax backward with the saved output taken as 0
+ * where the mask byte is non-zero, so those positions get a zero gradient.
+ * Replaces masked_softmax_backward_kernel (SoftMaxKernels.h:54-58,
+ * SoftMaxKernels.cpp:2022-2118 and 2361-2401).  Mask arguments as above;
+ * grad, y and gi share `dtype`. */
+int mi355x_masked_softmax_bwd(const void* grad, const void* y, const void* mask, void* gi,
+                              int64_t rows, int64_t N, int64_t mask_rows, int64_t mask_row_div,
+                              int64_t mask_row_stride, int64_t mask_row_mod, rownorm_dtype dtype,
+                              void* stream);
+
 /* Reports the launch layout a call with these sizes would use on the current
  * device (no launch; needs no GPU when the device query fails: 256 compute
  * units are assumed).  x_dtype is the row dtype, w_dtype the weight dtype

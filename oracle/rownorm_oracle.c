@@ -23,8 +23,9 @@
  * forms (mean/var, scipy.special.softmax/log_softmax), (3) central finite
  * differences of the forward functions for each backward function, and
  * (4) invariants (sum softmax = 1, sum softmax-backward = 0, dbeta of a
- * sum() loss = row count, constant row -> beta).  No function is "parity
- * unpinned".
+ * sum() loss = row count, constant row -> beta), (5) for the masked and
+ * safe softmax variants, the plain functions applied to the unmasked
+ * elements alone.  No function is "parity unpinned".
  *
  * All arrays are dense row-major float32; low-precision inputs are passed
  * already widened to float32 (exactly representable), outputs are returned
@@ -258,5 +259,67 @@ void oracle_softmax_bwd(const float* g, const float* y, float* gi,
       for (int64_t j = 0; j < N; ++j)
         o[j] = (float)((double)yr[j] * ((double)gr[j] - s));
     }
+  }
+}
+
+/* _safe_softmax: softmax whose rows with no finite element come out as zeros.
+ * is_safe_softmax branches, SoftMaxKernels.cpp:328-346 (max == -inf -> 0). */
+void oracle_safe_softmax_fwd(const float* x, float* y, int64_t rows, int64_t N) {
+  oracle_softmax_fwd(x, y, rows, N, 0);
+  for (int64_t r = 0; r < rows; ++r) {
+    int all_ninf = 1;
+    for (int64_t j = 0; j < N; ++j)
+      if (!(x[r * N + j] == -INFINITY)) all_ninf = 0;
+    if (all_ninf)
+      for (int64_t j = 0; j < N; ++j) y[r * N + j] = 0.0f;
+  }
+}
+
+/* _masked_softmax over the last dimension; mask is [rows, N] bytes, non-zero
+ * = leave the element out.  SoftMaxKernels.cpp:257-272 replaces masked
+ * elements by -inf before the max; :331-332 turns a zero sum (every element
+ * masked) into NaN. */
+void oracle_masked_softmax_fwd(const float* x, const uint8_t* mask, float* y,
+                               int64_t rows, int64_t N) {
+  for (int64_t r = 0; r < rows; ++r) {
+    const float* xr = x + r * N;
+    const uint8_t* mr = mask + r * N;
+    float* yr = y + r * N;
+    double m = -INFINITY;
+    int has_nan = 0, any = 0;
+    for (int64_t j = 0; j < N; ++j) {
+      if (mr[j]) continue;
+      any = 1;
+      if (xr[j] != xr[j]) has_nan = 1;
+      if ((double)xr[j] > m) m = (double)xr[j];
+    }
+    if (has_nan) m = NAN;
+    double s = 0;
+    for (int64_t j = 0; j < N; ++j)
+      if (!mr[j]) s += exp((double)xr[j] - m);
+    for (int64_t j = 0; j < N; ++j) {
+      if (!any || s == 0)
+        yr[j] = NAN;
+      else
+        yr[j] = mr[j] ? 0.0f : (float)(exp((double)xr[j] - m) / s);
+    }
+  }
+}
+
+/* _masked_softmax_backward: softmax backward with the saved output read as 0
+ * at masked positions (SoftMaxKernels.cpp:991-1001), hence gi = 0 there. */
+void oracle_masked_softmax_bwd(const float* g, const float* y,
+                               const uint8_t* mask, float* gi, int64_t rows,
+                               int64_t N) {
+  for (int64_t r = 0; r < rows; ++r) {
+    const float* gr = g + r * N;
+    const float* yr = y + r * N;
+    const uint8_t* mr = mask + r * N;
+    float* o = gi + r * N;
+    double s = 0;
+    for (int64_t j = 0; j < N; ++j)
+      if (!mr[j]) s += (double)yr[j] * (double)gr[j];
+    for (int64_t j = 0; j < N; ++j)
+      o[j] = mr[j] ? 0.0f : (float)((double)yr[j] * ((double)gr[j] - s));
   }
 }

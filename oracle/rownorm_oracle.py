@@ -46,6 +46,13 @@ def lib():
         L.oracle_rms_norm_bwd.argtypes = [_f32p, _f32p, _f32p, _f32p, _f32p, _f32p, _f64p, _i64, _i64]
         L.oracle_softmax_fwd.argtypes = [_f32p, _f32p, _i64, _i64, ctypes.c_int]
         L.oracle_softmax_bwd.argtypes = [_f32p, _f32p, _f32p, _i64, _i64, ctypes.c_int]
+        _u8p = ctypes.POINTER(ctypes.c_uint8)
+        L.oracle_safe_softmax_fwd.argtypes = [_f32p, _f32p, _i64, _i64]
+        L.oracle_masked_softmax_fwd.argtypes = [_f32p, _u8p, _f32p, _i64, _i64]
+        L.oracle_masked_softmax_bwd.argtypes = [_f32p, _f32p, _u8p, _f32p, _i64, _i64]
+        for f in ("oracle_safe_softmax_fwd", "oracle_masked_softmax_fwd",
+                  "oracle_masked_softmax_bwd"):
+            getattr(L, f).restype = None
         for f in ("oracle_welford_moments", "oracle_layer_norm_fwd", "oracle_rms_norm_fwd",
                   "oracle_layer_norm_bwd", "oracle_rms_norm_bwd", "oracle_softmax_fwd",
                   "oracle_softmax_bwd"):
@@ -161,4 +168,41 @@ def softmax_bwd(grad, y, is_log=False):
     if y.size:
         N = y.shape[-1] if y.ndim else 1
         lib().oracle_softmax_bwd(_p(grad), _p(y), _p(gi), y.size // N, N, int(is_log))
+    return gi
+
+
+def safe_softmax_fwd(x):
+    """_safe_softmax over the last dimension (rows of -inf give zeros)."""
+    x = _c(x)
+    y = np.empty_like(x)
+    if x.size:
+        N = x.shape[-1] if x.ndim else 1
+        lib().oracle_safe_softmax_fwd(_p(x), _p(y), x.size // N, N)
+    return y
+
+
+def _mask_bytes(mask, shape):
+    m = np.ascontiguousarray(np.broadcast_to(np.asarray(mask).astype(bool), shape), dtype=np.uint8)
+    return m, m.ctypes.data_as(ctypes.POINTER(ctypes.c_uint8))
+
+
+def masked_softmax_fwd(x, mask):
+    """_masked_softmax over the last dimension; mask (True = leave out) broadcasts to x."""
+    x = _c(x)
+    y = np.empty_like(x)
+    if x.size:
+        N = x.shape[-1] if x.ndim else 1
+        m, mp = _mask_bytes(mask, x.shape)
+        lib().oracle_masked_softmax_fwd(_p(x), mp, _p(y), x.size // N, N)
+    return y
+
+
+def masked_softmax_bwd(grad, y, mask):
+    """_masked_softmax_backward over the last dimension."""
+    grad, y = _c(grad), _c(y)
+    gi = np.empty_like(y)
+    if y.size:
+        N = y.shape[-1] if y.ndim else 1
+        m, mp = _mask_bytes(mask, y.shape)
+        lib().oracle_masked_softmax_bwd(_p(grad), _p(y), mp, _p(gi), y.size // N, N)
     return gi

@@ -29,6 +29,8 @@ def put(store, key, t):
         store[key + ":f16"] = t.view(torch.int16).numpy().view(np.uint16)
     elif t.dtype == torch.bfloat16:
         store[key + ":bf16"] = t.view(torch.int16).numpy().view(np.uint16)
+    elif t.dtype == torch.bool:
+        store[key] = t.numpy().astype(np.uint8)
     else:
         raise TypeError(t.dtype)
 
@@ -101,6 +103,22 @@ def main():
                 out = fwd(s, -1, False)
                 put(store, case + "/%s_y" % nm, out)
                 put(store, case + "/%s_gi" % nm, bwd(dy, out, -1, dt))
+            # _safe_softmax on the same scores (row 2 is all -inf -> zeros), and
+            # _masked_softmax / _masked_softmax_backward with ~30% of the elements masked,
+            # row 3 untouched and row 4 fully masked
+            put(store, case + "/ssm_y", torch.ops.aten._safe_softmax(s, -1))
+            mask = torch.rand(M, N, generator=g) < 0.3
+            if M > 3:
+                mask[3] = False
+            if M > 4:
+                mask[4] = True
+            put(store, case + "/msk", mask)
+            finite = (3.0 * torch.randn(M, N, generator=g)).to(dt)
+            put(store, case + "/msm_x", finite)
+            out = torch.ops.aten._masked_softmax(finite, mask, -1, 2)
+            put(store, case + "/msm_y", out)
+            put(store, case + "/msm_gi",
+                torch.ops.aten._masked_softmax_backward(dy, out, mask, -1))
     path = os.path.join(HERE, "aten_cpu_golden.npz")
     np.savez_compressed(path, **store)
     print("wrote", path, os.path.getsize(path), "bytes,", len(store), "arrays")

@@ -62,6 +62,50 @@ def test_argument_validation_happens_before_any_launch(cabi):
     assert L.mi355x_rms_norm_bwd(one, one, one, one, null, null, null, 0, 4, 8, 0, 0, null) == 0
 
 
+def test_mask_row_mapping_is_bounds_checked_before_any_launch(cabi):
+    L = cabi.lib()
+    one, null = ctypes.c_void_p(256), None  # never dereferenced: every call here is rejected
+    fwd = lambda rows, N, mrows, div, stride, mod, mask=one: L.mi355x_masked_softmax_fwd(
+        one, mask, one, rows, N, mrows, div, stride, mod, cabi.F32, null)
+    bwd = lambda rows, N, mrows, div, stride, mod, mask=one: L.mi355x_masked_softmax_bwd(
+        one, one, mask, one, rows, N, mrows, div, stride, mod, cabi.F32, null)
+    for call in (fwd, bwd):
+        assert call(8, 16, 8, 1, 1, 1, mask=null) == -3          # mask missing
+        assert call(0, 16, 0, 1, 1, 1, mask=null) == 0           # empty problem: no-op
+        assert call(8, 16, 7, 1, 1, 1) == -2                     # full mask one row short
+        assert call(8, 16, 8, 0, 1, 1) == -2                     # div must be positive
+        assert call(8, 16, 8, 1, -1, 1) == -2                    # negative stride
+        assert call(8, 16, 8, 1, 1, 0) == -2                     # mod must be positive
+        assert call(2 * 3 * 4, 4, 1, 12, 1, 1) == -2             # [B, T] mask with B = 2 given 1 row
+        assert call(2 * 3 * 4, 4, 3, 1, 0, 4) == -2              # [T, T] mask with T = 4 given 3 rows
+        assert call(2 * 3 * 4, 4, 7, 12, 4, 4) == -2             # [B, 1, T, T] needs B*T = 8 rows
+        assert call(1 << 31, 4, 1 << 31, 1, 1, 1) == -2          # masked calls stop at 2^31 rows
+    # dtype pairs: the masked entry points take one dtype for everything
+    assert L.mi355x_masked_softmax_fwd(one, one, one, 8, 16, 8, 1, 1, 1, 9, null) == -1
+    assert L.mi355x_safe_softmax_fwd(null, null, 4, 8, cabi.BF16, cabi.F32, null) == -1
+    assert L.mi355x_safe_softmax_fwd(null, null, 4, 8, cabi.F16, cabi.F32, null) == -3
+    assert L.mi355x_safe_softmax_fwd(null, null, 0, 8, cabi.F16, cabi.F32, null) == 0
+
+
+def test_mask_row_map_helper(cabi):
+    assert cabi.mask_row_map((2, 3, 4, 4), (2, 3, 4, 4)) == (24, 1, 1, 1)
+    assert cabi.mask_row_map((2, 3, 4, 4), (2, 4)) == (2, 12, 1, 1)
+    assert cabi.mask_row_map((2, 3, 4, 4), (4, 4)) == (4, 1, 0, 4)
+    assert cabi.mask_row_map((2, 3, 4, 4), (2, 1, 4, 4)) == (8, 12, 4, 4)
+    with pytest.raises(RuntimeError, match="does not fit"):
+        cabi.mask_row_map((2, 3, 4, 4), (3, 4))
+    # brute force: the mapping names the same mask row as numpy broadcasting does
+    import numpy as np
+    B, H, T = 2, 3, 4
+    for mshape, view in (((B, T), (B, 1, 1, T)), ((T, T), (1, 1, T, T)), ((B, 1, T, T),) * 2,
+                         ((B, H, T, T),) * 2):
+        mrows, div, stride, mod = cabi.mask_row_map((B, H, T, T), mshape)
+        ids = np.arange(mrows)[:, None].repeat(T, 1).reshape(mshape)       # mask row id per element
+        full = np.broadcast_to(ids.reshape(view), (B, H, T, T)).reshape(-1, T)[:, 0]
+        mapped = [(r // div) * stride + r % mod for r in range(B * H * T)]
+        assert mapped == list(full), mshape
+
+
 def test_workspace_size_follows_the_plan(cabi):
     L = cabi.lib()
     p = cabi.plan(cabi.OP_RMS_NORM_BWD, 16384, 4096, cabi.BF16, cabi.BF16)

@@ -21,6 +21,9 @@ def test_ops_are_registered_with_the_reference_schemas(ops):
         "_log_softmax": "(Tensor self, int dim, bool half_to_float) -> Tensor",
         "_softmax_backward_data": "(Tensor grad_output, Tensor output, int dim, ScalarType input_dtype) -> Tensor",
         "_log_softmax_backward_data": "(Tensor grad_output, Tensor output, int dim, ScalarType input_dtype) -> Tensor",
+        "_safe_softmax": "(Tensor self, int dim, ScalarType? dtype=None) -> Tensor",
+        "_masked_softmax": "(Tensor self, Tensor mask, int? dim=None, int? mask_type=None) -> Tensor",
+        "_masked_softmax_backward": "(Tensor grad_output, Tensor output, Tensor mask, int? dim=None) -> Tensor",
     }
     for name, sig in expect.items():
         schema = str(getattr(ops, name).default._schema)
@@ -58,6 +61,9 @@ def test_cpu_tensors_are_rejected_loudly(ops):
         lambda: ops._log_softmax(x, -1, False),
         lambda: ops._softmax_backward_data(x, x, -1, torch.float32),
         lambda: ops._log_softmax_backward_data(x, x, -1, torch.float32),
+        lambda: ops._safe_softmax(x, -1),
+        lambda: ops._masked_softmax(x, x > 0, -1, 2),
+        lambda: ops._masked_softmax_backward(x, x, x > 0, -1),
     ]
     for fn in calls:
         with pytest.raises(RuntimeError, match="no CPU path"):
@@ -80,3 +86,23 @@ def test_ctypes_layer_rejects_cpu_tensors(cabi):
         cabi.rms_norm_fwd(x, None, 1e-6)
     with pytest.raises(RuntimeError, match="not implemented"):
         cabi.dtype_code(torch.float64)
+
+
+def test_masked_softmax_argument_errors(ops):
+    # the checks and messages of masked_softmax_kernel / masked_softmax_backward_kernel
+    # (SoftMaxKernels.cpp:2308-2338 and 2382-2390 in the reference); CPU ATen words the shape
+    # errors differently and accepts a missing mask type, the reference does not
+    x = torch.randn(2, 3, 4, 4)
+    ok = torch.zeros(2, 3, 4, 4, dtype=torch.bool)
+    assert _aten_message(lambda: ops._masked_softmax(x, ok.float(), -1, 2)) == \
+        _aten_message(lambda: torch.ops.aten._masked_softmax(x, ok.float(), -1, 2))
+    with pytest.raises(RuntimeError, match="Mask Type should be defined"):
+        ops._masked_softmax(x, ok, -1, None)
+    with pytest.raises(RuntimeError, match="Mask Type should be 0 .src_mask., 1 .src_key_padding"):
+        ops._masked_softmax(x, ok, -1, 3)
+    with pytest.raises(RuntimeError, match="Mask shape should match input. mask: .2, 2, 4, 4."):
+        ops._masked_softmax(x, ok[:, :2], -1, 2)
+    with pytest.raises(RuntimeError, match="Mask shape should match input"):
+        ops._masked_softmax(x, ok[0, 0], -1, 1)  # [T, T] is not a key-padding mask
+    with pytest.raises(RuntimeError, match="Mask shape should match input"):
+        ops._masked_softmax(x, ok[:, 0, 0], -1, 0)  # [B, T] is not a src mask

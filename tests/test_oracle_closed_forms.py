@@ -234,3 +234,48 @@ def test_softmax_bwd_closed_form_and_finite_differences(oracle):
     ly = oracle.softmax_fwd(x, True)
     ly[0, 3] = -np.inf
     assert oracle.softmax_bwd(g, ly, True)[0, 3] == g[0, 3]
+
+
+# ---------------------------------------------- masked and safe softmax ----
+def test_masked_softmax_is_softmax_of_the_unmasked_elements(oracle):
+    rng = np.random.default_rng(7)
+    M, N = 6, 37
+    x, g = _rand(M, N) * 3, _rand(M, N)
+    mask = rng.random((M, N)) < 0.4
+    mask[0] = False
+    mask[1, 1:] = True  # a single survivor
+    mask[1, 0] = False
+    y = oracle.masked_softmax_fwd(x, mask)
+    gi = oracle.masked_softmax_bwd(g, y, mask)
+    for r in range(M):
+        keep = ~mask[r]
+        ref = scipy.special.softmax(x[r, keep].astype(np.float64))
+        np.testing.assert_allclose(y[r, keep], ref, rtol=2e-7, atol=1e-12)
+        assert np.all(y[r, mask[r]] == 0) and np.all(gi[r, mask[r]] == 0)
+        # backward of the compacted row with the plain formula
+        yd, gd = y[r, keep].astype(np.float64), g[r, keep].astype(np.float64)
+        np.testing.assert_allclose(gi[r, keep], yd * (gd - (yd * gd).sum()), rtol=1e-6, atol=1e-7)
+    assert y[1, 0] == 1.0
+    # broadcasting: a [N] mask applies to every row
+    yb = oracle.masked_softmax_fwd(x, mask[2])
+    assert np.array_equal(yb[5], oracle.masked_softmax_fwd(x[5:6], mask[2:3])[0])
+    # every element masked -> NaN row, zero gradient
+    full = np.ones((M, N), bool)
+    assert np.all(np.isnan(oracle.masked_softmax_fwd(x, full)))
+    assert np.all(oracle.masked_softmax_bwd(g, y, full) == 0)
+    # masking with the mask equals feeding -inf to the plain softmax
+    xm = np.where(mask, -np.inf, x).astype(np.float32)
+    np.testing.assert_array_equal(y, oracle.softmax_fwd(xm))
+
+
+def test_safe_softmax_differs_from_softmax_only_on_all_neg_inf_rows(oracle):
+    x = _rand(5, 33) * 3
+    x[1, 10:] = -np.inf
+    x[3, :] = -np.inf
+    s, ss = oracle.softmax_fwd(x), oracle.safe_softmax_fwd(x)
+    keep = [0, 1, 2, 4]
+    np.testing.assert_array_equal(ss[keep], s[keep])
+    assert np.all(np.isnan(s[3])) and np.all(ss[3] == 0)
+    # a NaN input still poisons its row
+    x[0, 5] = np.nan
+    assert np.all(np.isnan(oracle.safe_softmax_fwd(x)[0]))

@@ -74,3 +74,21 @@ def test_softmax_matches_golden(oracle, case):
         # terms is only good to a few 1e-5
         assert_close(gi, c[nm + "_gi"], dt, case + " " + nm + " grad_input",
                      scale=8.0 if (is_log and dt == torch.float32) else 1.0)
+
+
+@pytest.mark.parametrize("case", NAMES)
+def test_safe_and_masked_softmax_match_golden(oracle, case):
+    c = CASES[case]
+    dt = GOLDEN_DTYPES[case.split("_")[0]]
+    y = oracle.safe_softmax_fwd(to_np32(c["sm_x"]))
+    assert_close(y, c["ssm_y"], dt, case + " safe y")
+    assert np.all(y[2] == 0)  # the all -inf row
+    mask = c["msk"].numpy().astype(bool)
+    y = oracle.masked_softmax_fwd(to_np32(c["msm_x"]), mask)
+    assert_close(y, c["msm_y"], dt, case + " masked y")
+    if mask.shape[0] > 4:
+        assert np.all(np.isnan(y[4]))  # every element masked
+    assert np.all(y[mask & ~np.isnan(y)] == 0)
+    gi = oracle.masked_softmax_bwd(to_np32(c["dy"]), to_np32(c["msm_y"]), mask)
+    assert_close(gi, c["msm_gi"], dt, case + " masked grad_input")
+    assert np.all(gi[mask] == 0)

@@ -18,7 +18,8 @@ EXPORTED_SYMBOLS = (
     "mi355x_rownorm_error_string", "mi355x_rownorm_abi_version", "mi355x_layer_norm_fwd",
     "mi355x_layer_norm_bwd_workspace_bytes", "mi355x_layer_norm_bwd", "mi355x_rms_norm_fwd",
     "mi355x_rms_norm_bwd_workspace_bytes", "mi355x_rms_norm_bwd", "mi355x_softmax_fwd",
-    "mi355x_softmax_bwd", "mi355x_rownorm_plan", "mi355x_rownorm_set_override",
+    "mi355x_softmax_bwd", "mi355x_safe_softmax_fwd", "mi355x_masked_softmax_fwd",
+    "mi355x_masked_softmax_bwd", "mi355x_rownorm_plan", "mi355x_rownorm_set_override",
 )
 
 
@@ -59,11 +60,17 @@ def lib():
                                           _i64, _i64, _int, _int, _vp]
         L.mi355x_softmax_fwd.argtypes = [_vp, _vp, _i64, _i64, _int, _int, _int, _vp]
         L.mi355x_softmax_bwd.argtypes = [_vp, _vp, _vp, _i64, _i64, _int, _int, _int, _vp]
+        L.mi355x_safe_softmax_fwd.argtypes = [_vp, _vp, _i64, _i64, _int, _int, _vp]
+        L.mi355x_masked_softmax_fwd.argtypes = [_vp, _vp, _vp, _i64, _i64, _i64, _i64, _i64, _i64,
+                                                _int, _vp]
+        L.mi355x_masked_softmax_bwd.argtypes = [_vp, _vp, _vp, _vp, _i64, _i64, _i64, _i64, _i64,
+                                                _i64, _int, _vp]
         L.mi355x_rownorm_plan.argtypes = [_int, _i64, _i64, _int, _int, ctypes.POINTER(Plan)]
         L.mi355x_rownorm_set_override.argtypes = [_int, _int, _int, _int, _int]
         for name in ("mi355x_layer_norm_fwd", "mi355x_rms_norm_fwd", "mi355x_layer_norm_bwd",
                      "mi355x_rms_norm_bwd", "mi355x_softmax_fwd", "mi355x_softmax_bwd",
-                     "mi355x_rownorm_plan", "mi355x_rownorm_set_override"):
+                     "mi355x_safe_softmax_fwd", "mi355x_masked_softmax_fwd",
+                     "mi355x_masked_softmax_bwd", "mi355x_rownorm_plan", "mi355x_rownorm_set_override"):
             getattr(L, name).restype = _int
         _lib = L
     return _lib
@@ -228,4 +235,70 @@ def softmax_bwd(grad, y, is_log=False, gi_dtype=None, gi=None):
     _check(lib().mi355x_softmax_bwd(_ptr(grad), _ptr(y), _ptr(gi), rows, N,
                                     dtype_code(grad.dtype), dtype_code(gi.dtype), int(is_log),
                                     _stream()), "softmax_bwd")
+    return gi
+
+
+def safe_softmax_fwd(x, out_dtype=None, y=None):
+    """softmax over the last dim; rows that are all -inf give zeros."""
+    import torch
+    _gpu(x)
+    N = x.shape[-1] if x.dim() else 1
+    rows = x.numel() // N if N else 0
+    od = x.dtype if out_dtype is None else out_dtype
+    y = torch.empty(x.shape, dtype=od, device=x.device) if y is None else y
+    _check(lib().mi355x_safe_softmax_fwd(_ptr(x), _ptr(y), rows, N, dtype_code(x.dtype),
+                                         dtype_code(y.dtype), _stream()), "safe_softmax_fwd")
+    return y
+
+
+def mask_row_map(shape, mask_shape):
+    """(mask_rows, div, stride, mod) for a bool mask of ``mask_shape`` under last-dim softmax of a
+    dense tensor of ``shape``: the mask's own shape, [B, T] or [T, T] or [B, 1, T, T] under
+    [B, H, T, T]."""
+    shape, mask_shape = tuple(shape), tuple(mask_shape)
+    N = shape[-1]
+    rows = 1
+    for s in shape[:-1]:
+        rows *= s
+    if mask_shape == shape:
+        return rows, 1, 1, 1
+    if len(shape) == 4:
+        B, H, T, _ = shape
+        if mask_shape == (B, N) and T == N:
+            return B, H * T, 1, 1
+        if mask_shape == (T, N) and T == N:
+            return T, 1, 0, T
+        if mask_shape == (B, 1, T, N):
+            return B * T, H * T, T, T
+    raise RuntimeError("mask shape %s does not fit input %s" % (mask_shape, shape))
+
+
+def masked_softmax_fwd(x, mask, y=None, row_map=None):
+    """mask: torch.bool, True = leave the element out."""
+    import torch
+    _gpu(x, mask)
+    if mask.dtype != torch.bool:
+        raise RuntimeError("Mask should be a boolean tensor")
+    N = x.shape[-1] if x.dim() else 1
+    rows = x.numel() // N if N else 0
+    mrows, div, stride, mod = row_map or mask_row_map(x.shape, mask.shape)
+    y = torch.empty_like(x) if y is None else y
+    _check(lib().mi355x_masked_softmax_fwd(_ptr(x), _ptr(mask), _ptr(y), rows, N, mrows, div,
+                                           stride, mod, dtype_code(x.dtype), _stream()),
+           "masked_softmax_fwd")
+    return y
+
+
+def masked_softmax_bwd(grad, y, mask, gi=None, row_map=None):
+    import torch
+    _gpu(grad, y, mask)
+    if mask.dtype != torch.bool:
+        raise RuntimeError("Mask should be a boolean tensor")
+    N = y.shape[-1] if y.dim() else 1
+    rows = y.numel() // N if N else 0
+    mrows, div, stride, mod = row_map or mask_row_map(y.shape, mask.shape)
+    gi = torch.empty_like(grad) if gi is None else gi
+    _check(lib().mi355x_masked_softmax_bwd(_ptr(grad), _ptr(y), _ptr(mask), _ptr(gi), rows, N,
+                                           mrows, div, stride, mod, dtype_code(grad.dtype),
+                                           _stream()), "masked_softmax_bwd")
     return gi

@@ -54,5 +54,14 @@ TORCH_LIBRARY(mi355x, m) {
       "_log_softmax_backward_data.out(Tensor grad_output, Tensor output, int dim, ScalarType "
       "input_dtype, *, Tensor(a!) out) -> Tensor(a!)",
       &mi355x::_log_softmax_backward_data_out);
+  m.def("_safe_softmax(Tensor self, int dim, ScalarType? dtype=None) -> Tensor",
+        &mi355x::_safe_softmax);
+  m.def(
+      "_masked_softmax(Tensor self, Tensor mask, int? dim=None, int? mask_type=None) -> Tensor",
+      &mi355x::_masked_softmax);
+  m.def(
+      "_masked_softmax_backward(Tensor grad_output, Tensor output, Tensor mask, int? dim=None) "
+      "-> Tensor",
+      &mi355x::_masked_softmax_backward);
   m.def("install_layer_norm_dispatch_stubs() -> ()", &mi355x::install_layer_norm_dispatch_stubs);
 }

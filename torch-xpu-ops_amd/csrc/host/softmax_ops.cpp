@@ -17,15 +17,21 @@ namespace {
 
 using at::Tensor;
 
+enum class Mode { kSoftmax, kLogSoftmax, kSafeSoftmax };
+
 // Forward on dense [rows, N] data where `dim` is already innermost.
-void forward_lastdim(const Tensor& in, const Tensor& out, bool is_log, const char* op) {
+void forward_lastdim(const Tensor& in, const Tensor& out, Mode mode, const char* op) {
   const int64_t N = in.dim() == 0 ? 1 : in.size(-1);
   const int64_t rows = N == 0 ? 0 : in.numel() / N;
-  check_status(mi355x_softmax_fwd(in.const_data_ptr(), out.mutable_data_ptr(), rows, N,
-                                  to_rownorm_dtype(in.scalar_type(), op),
-                                  to_rownorm_dtype(out.scalar_type(), op), is_log ? 1 : 0,
-                                  current_stream(in)),
-               op);
+  const rownorm_dtype id = to_rownorm_dtype(in.scalar_type(), op);
+  const rownorm_dtype od = to_rownorm_dtype(out.scalar_type(), op);
+  const int rc =
+      mode == Mode::kSafeSoftmax
+          ? mi355x_safe_softmax_fwd(in.const_data_ptr(), out.mutable_data_ptr(), rows, N, id, od,
+                                    current_stream(in))
+          : mi355x_softmax_fwd(in.const_data_ptr(), out.mutable_data_ptr(), rows, N, id, od,
+                               mode == Mode::kLogSoftmax ? 1 : 0, current_stream(in));
+  check_status(rc, op);
 }
 
 void backward_lastdim(const Tensor& grad, const Tensor& y, const Tensor& gi, bool is_log,
@@ -44,7 +50,7 @@ void backward_lastdim(const Tensor& grad, const Tensor& y, const Tensor& gi, boo
 // input (:2131-2135); 0-dim tensors are viewed as [1] (:2143-2144); an empty
 // tensor is a no-op (:2150).
 void softmax_forward_entry(const Tensor& input_, int64_t dim_, bool half_to_float,
-                           const Tensor& output, bool is_log, const char* op) {
+                           const Tensor& output, Mode mode, const char* op) {
   check_gpu(input_, op, "input");
   check_same_device(input_, output, op, "output");
   if (half_to_float) {
@@ -65,16 +71,16 @@ void softmax_forward_entry(const Tensor& input_, int64_t dim_, bool half_to_floa
   if (dim == input.dim() - 1) {
     const Tensor in_c = input.contiguous();
     if (out.is_contiguous()) {
-      forward_lastdim(in_c, out, is_log, op);
+      forward_lastdim(in_c, out, mode, op);
     } else {
       Tensor tmp = at::empty_like(out, out.options(), at::MemoryFormat::Contiguous);
-      forward_lastdim(in_c, tmp, is_log, op);
+      forward_lastdim(in_c, tmp, mode, op);
       out.copy_(tmp);
     }
   } else {
     const Tensor in_t = input.movedim(dim, -1).contiguous();
     Tensor out_t = at::empty(in_t.sizes(), out.options());
-    forward_lastdim(in_t, out_t, is_log, op);
+    forward_lastdim(in_t, out_t, mode, op);
     out.copy_(out_t.movedim(-1, dim));
   }
 }
@@ -142,14 +148,167 @@ bool backward_half_to_float(const Tensor& grad, at::ScalarType input_dtype) {
   return h2f;
 }
 
+// How a boolean mask lines up with the rows of a dense tensor whose softmax
+// dimension is innermost: data row r reads mask row (r / div) * stride + r % mod.
+struct MaskLayout {
+  Tensor mask;  // dense [mask_rows, N] bool
+  int64_t mask_rows, div, stride, mod;
+};
+
+// The shapes masked_softmax_kernel accepts (SoftMaxKernels.cpp:2315-2338): the
+// input's own shape, a [B, T] key-padding mask (mask_type 1) or a [T, T] mask
+// (mask_type 0) under a [B, H, T, T] input.  The two small masks are read in
+// place; any other broadcastable mask is expanded once.
+MaskLayout mask_layout_lastdim(const Tensor& input, const Tensor& mask, bool is_BxT,
+                               bool is_TxT) {
+  const int64_t N = input.size(-1);
+  const int64_t rows = N == 0 ? 0 : input.numel() / N;
+  if (is_BxT) {
+    return {mask.contiguous(), mask.size(0), input.size(1) * input.size(2), 1, 1};
+  }
+  if (is_TxT) {
+    return {mask.contiguous(), mask.size(0), 1, 0, mask.size(0)};
+  }
+  return {mask.expand(input.sizes()).contiguous(), rows, 1, 1, 1};
+}
+
 }  // namespace
 
+// _safe_softmax_kernel, SoftMaxKernels.cpp:2278-2299.
+Tensor _safe_softmax_kernel(const Tensor& self, int64_t dim, bool half_to_float) {
+  check_gpu(self, "mi355x::_safe_softmax", "self");
+  Tensor out = alloc_forward_output(self, half_to_float);
+  softmax_forward_entry(self, dim, half_to_float, out, Mode::kSafeSoftmax,
+                        "mi355x::_safe_softmax");
+  return out;
+}
+
+// _safe_softmax_xpu, SoftMax.cpp:102-110: Half -> Float is fused into the
+// kernel, any other dtype request converts the input first.
+Tensor _safe_softmax(const Tensor& self, int64_t dim, std::optional<at::ScalarType> dtype) {
+  check_gpu(self, "mi355x::_safe_softmax", "self");
+  if (self.scalar_type() == at::kHalf && dtype == at::kFloat)
+    return _safe_softmax_kernel(self, dim, true);
+  const Tensor converted = dtype.has_value() ? self.toType(dtype.value()) : self;
+  return _safe_softmax_kernel(converted, dim, false);
+}
+
+// masked_softmax_kernel, SoftMaxKernels.cpp:2301-2359.
+Tensor masked_softmax_kernel(const Tensor& input_, const Tensor& mask_,
+                             std::optional<int64_t> dim_, std::optional<int64_t> mask_type_) {
+  const char* op = "mi355x::_masked_softmax";
+  TORCH_CHECK(mask_.scalar_type() == at::kBool, "Mask should be a boolean tensor");
+  TORCH_CHECK(mask_type_.has_value(), "Mask Type should be defined");
+  const int64_t mask_type = mask_type_.value();
+  TORCH_CHECK(mask_type == 0 || mask_type == 1 || mask_type == 2,
+              "Mask Type should be 0 (src_mask), 1 (src_key_padding_mask), or 2 (default_mask)");
+  const bool is_BxT = mask_type == 1 && input_.dim() == 4 && mask_.dim() == 2 &&
+                      input_.size(0) == mask_.size(0) && input_.size(2) == mask_.size(1) &&
+                      input_.size(3) == mask_.size(1);
+  const bool is_TxT = mask_type == 0 && input_.dim() == 4 && mask_.dim() == 2 &&
+                      input_.size(3) == mask_.size(1) && input_.size(2) == mask_.size(0) &&
+                      mask_.size(0) == mask_.size(1);
+  TORCH_CHECK(mask_.sizes() == input_.sizes() || is_BxT || is_TxT,
+              "Mask shape should match input. mask: ", mask_.sizes(), " input: ", input_.sizes());
+  check_gpu(input_, op, "input");
+  check_same_device(input_, mask_, op, "mask");
+  const rownorm_dtype dt = to_rownorm_dtype(input_.scalar_type(), op);
+  Tensor output = at::empty_like(input_, input_.options(), at::MemoryFormat::Contiguous);
+  Tensor input = input_.dim() == 0 ? input_.view(1) : input_;
+  Tensor mask = mask_.dim() == 0 ? mask_.view(1) : mask_;
+  Tensor out = output.dim() == 0 ? output.view(1) : output;
+  const int64_t dim =
+      dim_.has_value() ? at::maybe_wrap_dim(dim_.value(), input.dim()) : input.dim() - 1;
+  if (input.numel() == 0) return output;
+  c10::DeviceGuard guard(input.device());
+  auto run = [&](const Tensor& in, const MaskLayout& ml, const Tensor& o) {
+    const int64_t N = in.size(-1);
+    check_status(mi355x_masked_softmax_fwd(in.const_data_ptr(), ml.mask.const_data_ptr(),
+                                           o.mutable_data_ptr(), in.numel() / N, N, ml.mask_rows,
+                                           ml.div, ml.stride, ml.mod, dt, current_stream(in)),
+                 op);
+  };
+  if (dim == input.dim() - 1) {
+    const Tensor in_c = input.contiguous();
+    run(in_c, mask_layout_lastdim(in_c, mask, is_BxT, is_TxT), out);
+  } else {
+    // the mask follows the input through the transposition
+    Tensor full = is_BxT ? mask.view({mask.size(0), 1, 1, mask.size(1)}) : mask;
+    full = full.expand(input.sizes());
+    const Tensor in_t = input.movedim(dim, -1).contiguous();
+    const Tensor mask_t = full.movedim(dim, -1).contiguous();
+    Tensor out_t = at::empty(in_t.sizes(), out.options());
+    run(in_t, MaskLayout{mask_t, in_t.numel() / in_t.size(-1), 1, 1, 1}, out_t);
+    out.copy_(out_t.movedim(-1, dim));
+  }
+  return output;
+}
+
+// masked_softmax_backward_kernel, SoftMaxKernels.cpp:2361-2401.
+Tensor masked_softmax_backward_kernel(const Tensor& grad_, const Tensor& output_,
+                                      const Tensor& mask_, std::optional<int64_t> dim_) {
+  const char* op = "mi355x::_masked_softmax_backward";
+  check_gpu(grad_, op, "grad_output");
+  check_same_device(grad_, output_, op, "output");
+  check_same_device(grad_, mask_, op, "mask");
+  Tensor grad_input = at::empty_like(grad_, grad_.options(), at::MemoryFormat::Contiguous);
+  if (grad_.numel() == 0) return grad_input;
+  Tensor grad = grad_.contiguous();
+  Tensor output = output_.contiguous();
+  Tensor mask = mask_.contiguous();
+  const int64_t dim =
+      dim_.has_value() ? at::maybe_wrap_dim(dim_.value(), output.dim()) : output.dim() - 1;
+  grad = grad.dim() == 0 ? grad.view(1) : grad;
+  mask = mask.dim() == 0 ? mask.view(1) : mask;
+  output = output.dim() == 0 ? output.view(1) : output;
+  Tensor gi = grad_input.dim() == 0 ? grad_input.view(1) : grad_input;
+  TORCH_CHECK(dim >= 0 && dim < grad.dim(),
+              "dim must be non-negative and less than input dimensions");
+  TORCH_CHECK(grad.sizes() == mask.sizes(), "Mask shape should match grad shape");
+  TORCH_CHECK(grad.sizes() == output.sizes(), op, ": grad_output and output must share a shape");
+  TORCH_CHECK(mask.scalar_type() == at::kBool, "Mask should be a boolean tensor");
+  TORCH_CHECK(grad.scalar_type() == output.scalar_type(), op, ": grad_output dtype ",
+              grad.scalar_type(), " differs from output dtype ", output.scalar_type());
+  const rownorm_dtype dt = to_rownorm_dtype(grad.scalar_type(), op);
+  c10::DeviceGuard guard(grad.device());
+  auto run = [&](const Tensor& g, const Tensor& y, const Tensor& m, const Tensor& o) {
+    const int64_t N = g.size(-1);
+    const int64_t rows = g.numel() / N;
+    check_status(mi355x_masked_softmax_bwd(g.const_data_ptr(), y.const_data_ptr(),
+                                           m.const_data_ptr(), o.mutable_data_ptr(), rows, N, rows,
+                                           1, 1, 1, dt, current_stream(g)),
+                 op);
+  };
+  if (dim == grad.dim() - 1) {
+    run(grad, output, mask, gi);
+  } else {
+    const Tensor g_t = grad.movedim(dim, -1).contiguous();
+    const Tensor y_t = output.movedim(dim, -1).contiguous();
+    const Tensor m_t = mask.movedim(dim, -1).contiguous();
+    Tensor gi_t = at::empty(g_t.sizes(), gi.options());
+    run(g_t, y_t, m_t, gi_t);
+    gi.copy_(gi_t.movedim(-1, dim));
+  }
+  return grad_input;
+}
+
+// masked_softmax_xpu / masked_softmax_backward_xpu, SoftMax.cpp:112-126.
+Tensor _masked_softmax(const Tensor& self, const Tensor& mask, std::optional<int64_t> dim,
+                       std::optional<int64_t> mask_type) {
+  return masked_softmax_kernel(self, mask, dim, mask_type);
+}
+Tensor _masked_softmax_backward(const Tensor& grad_output, const Tensor& output,
+                                const Tensor& mask, std::optional<int64_t> dim) {
+  return masked_softmax_backward_kernel(grad_output, output, mask, dim);
+}
+
 void _softmax_kernel(const Tensor& input, int64_t dim, bool half_to_float, const Tensor& output) {
-  softmax_forward_entry(input, dim, half_to_float, output, false, "mi355x::_softmax");
+  softmax_forward_entry(input, dim, half_to_float, output, Mode::kSoftmax, "mi355x::_softmax");
 }
 void _log_softmax_kernel(const Tensor& input, int64_t dim, bool half_to_float,
                          const Tensor& output) {
-  softmax_forward_entry(input, dim, half_to_float, output, true, "mi355x::_log_softmax");
+  softmax_forward_entry(input, dim, half_to_float, output, Mode::kLogSoftmax,
+                        "mi355x::_log_softmax");
 }
 void _softmax_backward_kernel(const Tensor& grad, const Tensor& output, int64_t dim,
                               bool half_to_float, const Tensor& grad_input) {

@@ -165,6 +165,69 @@ int norm_bwd(const void* dy, const void* x, const float* mean, const float* rstd
                            : launch_norm_bwd<bf16, bf16, RMS>(plan, a, s);
 }
 
+// How the rows of a mask buffer map onto data rows: data row r reads mask row
+// (r / div) * stride + r % mod of a [rows, N] byte buffer.
+struct MaskRows {
+  int64_t rows = 0, div = 1, stride = 0, mod = 1;
+};
+
+// Rejects a mapping that could index outside the mask buffer.
+int mask_check(const MaskRows& m, int64_t data_rows) {
+  if (data_rows >= (int64_t(1) << 31)) return ROWNORM_ERR_SHAPE;
+  if (m.rows <= 0 || m.div <= 0 || m.mod <= 0 || m.stride < 0) return ROWNORM_ERR_SHAPE;
+  if (m.div >= (int64_t(1) << 32) || m.mod >= (int64_t(1) << 32)) return ROWNORM_ERR_SHAPE;
+  const int64_t last = data_rows - 1;
+  const int64_t hi_outer = last / m.div;
+  if (m.stride != 0 && hi_outer > (m.rows - 1) / m.stride) return ROWNORM_ERR_SHAPE;
+  const int64_t hi_inner = last < m.mod - 1 ? last : m.mod - 1;
+  if (hi_outer * m.stride + hi_inner > m.rows - 1) return ROWNORM_ERR_SHAPE;
+  return 0;
+}
+
+int softmax_fwd(const void* x, const void* mask, void* y, int64_t rows, int64_t N,
+                const MaskRows& mr, int id, int od, int flags, void* stream) {
+  if (esize_of(id) == 0 || esize_of(od) == 0) return ROWNORM_ERR_DTYPE;
+  if (!(od == id || (id == ROWNORM_F16 && od == ROWNORM_F32))) return ROWNORM_ERR_DTYPE;
+  if (int e = shape_check(rows, N)) return e;
+  if (rows == 0 || N == 0) return 0;
+  if (!x || !y) return ROWNORM_ERR_NULL;
+  if (mask)
+    if (int e = mask_check(mr, rows)) return e;
+  Plan plan;
+  if (int e = make_plan(OC_SOFTMAX_FWD, rows, N, esize_of(id), current_num_cus(),
+                        g_override[ROWNORM_OP_SOFTMAX_FWD], false, &plan))
+    return e;
+  SoftmaxFwdArgs a{x,    y, (const uint8_t*)mask, (uint32_t)mr.div, (uint32_t)mr.mod, mr.stride,
+                   rows, (int)N, flags};
+  hipStream_t s = (hipStream_t)stream;
+  if (id == ROWNORM_F32) return launch_softmax_fwd<float, float>(plan, a, s);
+  if (id == ROWNORM_BF16) return launch_softmax_fwd<bf16, bf16>(plan, a, s);
+  return od == ROWNORM_F32 ? launch_softmax_fwd<f16, float>(plan, a, s)
+                           : launch_softmax_fwd<f16, f16>(plan, a, s);
+}
+
+int softmax_bwd(const void* grad, const void* y, const void* mask, void* gi, int64_t rows,
+                int64_t N, const MaskRows& mr, int gd, int od, int flags, void* stream) {
+  if (esize_of(gd) == 0 || esize_of(od) == 0) return ROWNORM_ERR_DTYPE;
+  if (!(od == gd || (gd == ROWNORM_F32 && od == ROWNORM_F16))) return ROWNORM_ERR_DTYPE;
+  if (int e = shape_check(rows, N)) return e;
+  if (rows == 0 || N == 0) return 0;
+  if (!grad || !y || !gi) return ROWNORM_ERR_NULL;
+  if (mask)
+    if (int e = mask_check(mr, rows)) return e;
+  Plan plan;
+  if (int e = make_plan(OC_SOFTMAX_BWD, rows, N, esize_of(gd), current_num_cus(),
+                        g_override[ROWNORM_OP_SOFTMAX_BWD], false, &plan))
+    return e;
+  SoftmaxBwdArgs a{grad, y, gi, (const uint8_t*)mask, (uint32_t)mr.div, (uint32_t)mr.mod,
+                   mr.stride, rows, (int)N, flags};
+  hipStream_t s = (hipStream_t)stream;
+  if (gd == ROWNORM_BF16) return launch_softmax_bwd<bf16, bf16>(plan, a, s);
+  if (gd == ROWNORM_F16) return launch_softmax_bwd<f16, f16>(plan, a, s);
+  return od == ROWNORM_F16 ? launch_softmax_bwd<float, f16>(plan, a, s)
+                           : launch_softmax_bwd<float, float>(plan, a, s);
+}
+
 }  // namespace
 
 extern "C" {
@@ -229,43 +292,40 @@ int mi355x_rms_norm_bwd(const void* dy, const void* x, const float* rstd, const 
 
 int mi355x_softmax_fwd(const void* x, void* y, int64_t rows, int64_t N, rownorm_dtype in_dtype,
                        rownorm_dtype out_dtype, int is_log, void* stream) {
-  const int id = (int)in_dtype, od = (int)out_dtype;
-  if (esize_of(id) == 0 || esize_of(od) == 0) return ROWNORM_ERR_DTYPE;
-  if (!(od == id || (id == ROWNORM_F16 && od == ROWNORM_F32))) return ROWNORM_ERR_DTYPE;
-  if (int e = shape_check(rows, N)) return e;
-  if (rows == 0 || N == 0) return 0;
-  if (!x || !y) return ROWNORM_ERR_NULL;
-  Plan plan;
-  if (int e = make_plan(OC_SOFTMAX_FWD, rows, N, esize_of(id), current_num_cus(),
-                        g_override[ROWNORM_OP_SOFTMAX_FWD], false, &plan))
-    return e;
-  SoftmaxFwdArgs a{x, y, rows, (int)N, is_log ? 1 : 0};
-  hipStream_t s = (hipStream_t)stream;
-  if (id == ROWNORM_F32) return launch_softmax_fwd<float, float>(plan, a, s);
-  if (id == ROWNORM_BF16) return launch_softmax_fwd<bf16, bf16>(plan, a, s);
-  return od == ROWNORM_F32 ? launch_softmax_fwd<f16, float>(plan, a, s)
-                           : launch_softmax_fwd<f16, f16>(plan, a, s);
+  return softmax_fwd(x, nullptr, y, rows, N, MaskRows{}, (int)in_dtype, (int)out_dtype,
+                     is_log ? kSoftmaxLog : 0, stream);
+}
+
+int mi355x_safe_softmax_fwd(const void* x, void* y, int64_t rows, int64_t N,
+                            rownorm_dtype in_dtype, rownorm_dtype out_dtype, void* stream) {
+  return softmax_fwd(x, nullptr, y, rows, N, MaskRows{}, (int)in_dtype, (int)out_dtype,
+                     kSoftmaxSafe, stream);
+}
+
+int mi355x_masked_softmax_fwd(const void* x, const void* mask, void* y, int64_t rows, int64_t N,
+                              int64_t mask_rows, int64_t mask_row_div, int64_t mask_row_stride,
+                              int64_t mask_row_mod, rownorm_dtype dtype, void* stream) {
+  if (rows > 0 && N > 0 && !mask) return ROWNORM_ERR_NULL;
+  return softmax_fwd(x, mask, y, rows, N,
+                     MaskRows{mask_rows, mask_row_div, mask_row_stride, mask_row_mod}, (int)dtype,
+                     (int)dtype, 0, stream);
 }
 
 int mi355x_softmax_bwd(const void* grad, const void* y, void* gi, int64_t rows, int64_t N,
                        rownorm_dtype grad_dtype, rownorm_dtype gi_dtype, int is_log,
                        void* stream) {
-  const int gd = (int)grad_dtype, od = (int)gi_dtype;
-  if (esize_of(gd) == 0 || esize_of(od) == 0) return ROWNORM_ERR_DTYPE;
-  if (!(od == gd || (gd == ROWNORM_F32 && od == ROWNORM_F16))) return ROWNORM_ERR_DTYPE;
-  if (int e = shape_check(rows, N)) return e;
-  if (rows == 0 || N == 0) return 0;
-  if (!grad || !y || !gi) return ROWNORM_ERR_NULL;
-  Plan plan;
-  if (int e = make_plan(OC_SOFTMAX_BWD, rows, N, esize_of(gd), current_num_cus(),
-                        g_override[ROWNORM_OP_SOFTMAX_BWD], false, &plan))
-    return e;
-  SoftmaxBwdArgs a{grad, y, gi, rows, (int)N, is_log ? 1 : 0};
-  hipStream_t s = (hipStream_t)stream;
-  if (gd == ROWNORM_BF16) return launch_softmax_bwd<bf16, bf16>(plan, a, s);
-  if (gd == ROWNORM_F16) return launch_softmax_bwd<f16, f16>(plan, a, s);
-  return od == ROWNORM_F16 ? launch_softmax_bwd<float, f16>(plan, a, s)
-                           : launch_softmax_bwd<float, float>(plan, a, s);
+  return softmax_bwd(grad, y, nullptr, gi, rows, N, MaskRows{}, (int)grad_dtype, (int)gi_dtype,
+                     is_log ? kSoftmaxLog : 0, stream);
+}
+
+int mi355x_masked_softmax_bwd(const void* grad, const void* y, const void* mask, void* gi,
+                              int64_t rows, int64_t N, int64_t mask_rows, int64_t mask_row_div,
+                              int64_t mask_row_stride, int64_t mask_row_mod, rownorm_dtype dtype,
+                              void* stream) {
+  if (rows > 0 && N > 0 && !mask) return ROWNORM_ERR_NULL;
+  return softmax_bwd(grad, y, mask, gi, rows, N,
+                     MaskRows{mask_rows, mask_row_div, mask_row_stride, mask_row_mod}, (int)dtype,
+                     (int)dtype, 0, stream);
 }
 
 int mi355x_rownorm_plan(rownorm_op op, int64_t M, int64_t N, rownorm_dtype x_dtype,

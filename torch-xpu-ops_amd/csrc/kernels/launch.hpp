@@ -36,21 +36,30 @@ struct NormBwdArgs {
   int N;
 };
 
+constexpr int kSoftmaxLog = 1;   // log_softmax instead of softmax
+constexpr int kSoftmaxSafe = 2;  // rows with no finite element give 0 instead of NaN
+
 struct SoftmaxFwdArgs {
   const void* x;
   void* y;
+  const uint8_t* mask;  // null = unmasked; else data row r uses mask row (r / div) * stride + r % mod
+  uint32_t mask_div, mask_mod;
+  int64_t mask_stride;
   int64_t M;
   int N;
-  int is_log;
+  int flags;  // kSoftmaxLog | kSoftmaxSafe
 };
 
 struct SoftmaxBwdArgs {
   const void* grad;
   const void* y;
   void* gi;
+  const uint8_t* mask;
+  uint32_t mask_div, mask_mod;
+  int64_t mask_stride;
   int64_t M;
   int N;
-  int is_log;
+  int flags;
 };
 
 // All return 0 or a hipError_t value.

@@ -1,4 +1,5 @@
-// Last-dimension softmax / log_softmax forward and backward for gfx950.
+// Last-dimension softmax / log_softmax forward and backward for gfx950, with
+// the masked and "safe" variants.
 //
 // Same row layout as the norm kernels: G lanes share a row, each lane holds V
 // 16-byte packs in registers, a workgroup handles BLOCK/G rows per iteration.
@@ -14,9 +15,20 @@
 // The arithmetic follows :300-357 (max, sum of exp(x - max), then
 // exp(x-max)/sum or x - max - log(sum)) and :1031-1047 (y*(g - sum y*g) or
 // g - exp(y)*sum g).
+//
+// Masked (is_masked in the reference, :257-272 and :991-1001): a boolean mask
+// marks elements to leave out; forward treats them as -inf, backward treats the
+// saved output there as 0.  The mask row that belongs to data row r is
+// (r / div) * stride + r % mod, which covers a mask of the input's own shape
+// (div 1, stride 1, mod 1), a [B, T] key-padding mask under [B, H, T, T] scores
+// (div H*T, stride 1, mod 1), a [T, T] mask (stride 0, mod T) and a
+// [B, 1, T, T] mask (div H*T, stride T, mod T).
+// Safe (is_safe_softmax, :328-346): a row with no finite maximum comes out as
+// zeros instead of NaN.
 #pragma once
 #include "device/pack.hpp"
 #include "device/reduce.hpp"
+#include "launch.hpp"
 
 namespace rownorm {
 
@@ -31,10 +43,44 @@ __device__ __forceinline__ float row_exp(float v) {
     return __expf(v);
 }
 
-template <class TI, class TO, int G, int V, int BLOCK, bool FAST>
+struct MaskRef {
+  const uint8_t* data;  // one byte per element, non-zero = masked out
+  uint32_t div, mod;    // mask row of data row r: (r / div) * stride + r % mod
+  int64_t stride;
+};
+
+// Start of the mask row for data row `r` (masked calls are limited to 2^31 rows).
+__device__ __forceinline__ const uint8_t* mask_row_ptr(const MaskRef& m, int64_t r, int n) {
+  const uint32_t r32 = (uint32_t)r;
+  const int64_t mr = (int64_t)(r32 / m.div) * m.stride + (int64_t)(r32 % m.mod);
+  return m.data + mr * (int64_t)n;
+}
+
+// E mask bytes for the pack starting at element e0 of a mask row (fill: not masked).
+template <int E, bool FAST>
+__device__ __forceinline__ Pack<uint8_t, E> load_mask_pack(const uint8_t* mrow, int e0, int n,
+                                                           bool ok) {
+  Pack<uint8_t, E> m;
+  if constexpr (FAST) {
+    const bool inb = e0 < n;
+    m = Pack<uint8_t, E>::load(mrow + (inb ? e0 : 0));
+    (void)ok;
+  } else {
+#pragma unroll
+    for (int i = 0; i < E; ++i) m.v[i] = 0;
+    if (ok) {
+#pragma unroll
+      for (int i = 0; i < E; ++i)
+        if (e0 + i < n) m.v[i] = mrow[e0 + i];
+    }
+  }
+  return m;
+}
+
+template <class TI, class TO, int G, int V, int BLOCK, bool FAST, bool MASKED>
 __global__ void __launch_bounds__(BLOCK)
-softmax_fwd_resident_kernel(const TI* __restrict__ x, TO* __restrict__ y, int64_t M, int N,
-                            int is_log) {
+softmax_fwd_resident_kernel(const TI* __restrict__ x, TO* __restrict__ y, MaskRef mask, int64_t M,
+                            int N, int flags) {
   constexpr int E = elems_per_pack<TI>::value;
   constexpr int RPB = BLOCK / G;
   constexpr bool PRECISE = sizeof(TO) == 4;
@@ -42,11 +88,14 @@ softmax_fwd_resident_kernel(const TI* __restrict__ x, TO* __restrict__ y, int64_
   int phase = 0;
   const int slot = threadIdx.x / G;
   const int lane = threadIdx.x % G;
+  const bool is_log = (flags & kSoftmaxLog) != 0;
+  const bool is_safe = (flags & kSoftmaxSafe) != 0;
   const int64_t nrb = (M + RPB - 1) / RPB;
   for (int64_t rb = blockIdx.x; rb < nrb; rb += gridDim.x) {
     const int64_t row = rb * RPB + slot;
     const bool ok = RPB == 1 ? true : row < M;
-    const TI* xr = x + (ok ? row : 0) * (int64_t)N;
+    const int64_t rowc = ok ? row : 0;
+    const TI* xr = x + rowc * (int64_t)N;
     TO* yr = y + row * (int64_t)N;
     Pack<TI, E> xp[V];
 #pragma unroll
@@ -57,6 +106,15 @@ softmax_fwd_resident_kernel(const TI* __restrict__ x, TO* __restrict__ y, int64_
     for (int c = 0; c < V; ++c)
 #pragma unroll
       for (int i = 0; i < E; ++i) xf[c][i] = xp[c].get(i);
+    if constexpr (MASKED) {
+      const uint8_t* mrow = mask_row_ptr(mask, rowc, N);
+#pragma unroll
+      for (int c = 0; c < V; ++c) {
+        const Pack<uint8_t, E> mk = load_mask_pack<E, FAST>(mrow, (c * G + lane) * E, N, ok);
+#pragma unroll
+        for (int i = 0; i < E; ++i) xf[c][i] = mk.v[i] ? -INFINITY : xf[c][i];
+      }
+    }
     float mx[1] = {-INFINITY};
 #pragma unroll
     for (int c = 0; c < V; ++c)
@@ -85,54 +143,76 @@ softmax_fwd_resident_kernel(const TI* __restrict__ x, TO* __restrict__ y, int64_
     }
     group_allreduce<G, BLOCK, 1, SumOp>(sum, red, phase);
     const float k = is_log ? logf(sum[0]) : 1.0f / sum[0];
+    const bool zero_row = is_safe && m == -INFINITY;  // no finite element in the row
 #pragma unroll
     for (int c = 0; c < V; ++c) {
       const int e0 = (c * G + lane) * E;
       Pack<TO, E> o;
 #pragma unroll
-      for (int i = 0; i < E; ++i) o.set(i, is_log ? xf[c][i] - k : xf[c][i] * k);
+      for (int i = 0; i < E; ++i) {
+        const float v = is_log ? xf[c][i] - k : xf[c][i] * k;
+        o.set(i, zero_row ? 0.0f : v);
+      }
       row_store<TO, E, true, FAST>(yr, e0, N, ok, o);
     }
   }
 }
 
 // Rows too wide for registers: one workgroup per row, three streaming passes.
-template <class TI, class TO, int BLOCK>
+template <class TI, class TO, int BLOCK, bool MASKED>
 __global__ void __launch_bounds__(BLOCK)
-softmax_fwd_stream_kernel(const TI* __restrict__ x, TO* __restrict__ y, int64_t M, int N,
-                          int is_log) {
+softmax_fwd_stream_kernel(const TI* __restrict__ x, TO* __restrict__ y, MaskRef mask, int64_t M,
+                          int N, int flags) {
   constexpr int E = elems_per_pack<TI>::value;
   constexpr bool PRECISE = sizeof(TO) == 4;
   __shared__ float red[reduce_lds_floats<BLOCK, BLOCK, 1>::value];
   int phase = 0;
+  const bool is_log = (flags & kSoftmaxLog) != 0;
+  const bool is_safe = (flags & kSoftmaxSafe) != 0;
   const int npacks = (N + E - 1) / E;
   for (int64_t row = blockIdx.x; row < M; row += gridDim.x) {
     const TI* xr = x + row * (int64_t)N;
     TO* yr = y + row * (int64_t)N;
+    const uint8_t* mrow =
+        MASKED ? mask_row_ptr(mask, row, N) : nullptr;
+    // element i of pack pk, with the mask applied
+    auto masked_value = [&](const Pack<TI, E>& p, const Pack<uint8_t, E>& mk, int i) {
+      const float v = p.get(i);
+      if constexpr (MASKED) return mk.v[i] ? -INFINITY : v;
+      return v;
+    };
     float mx[1] = {-INFINITY};
     for (int pk = threadIdx.x; pk < npacks; pk += BLOCK) {
       const Pack<TI, E> p = load_row_pack<TI, E, false>(xr, pk * E, N, true, -INFINITY);
+      Pack<uint8_t, E> mk;
+      if constexpr (MASKED) mk = load_mask_pack<E, false>(mrow, pk * E, N, true);
 #pragma unroll
-      for (int i = 0; i < E; ++i) mx[0] = fmaxf(mx[0], p.get(i));
+      for (int i = 0; i < E; ++i) mx[0] = fmaxf(mx[0], masked_value(p, mk, i));
     }
     group_allreduce<BLOCK, BLOCK, 1, MaxOp>(mx, red, phase);
     const float m = mx[0];
     float sum[1] = {0.0f};
     for (int pk = threadIdx.x; pk < npacks; pk += BLOCK) {
       const Pack<TI, E> p = load_row_pack<TI, E, false>(xr, pk * E, N, true, -INFINITY);
+      Pack<uint8_t, E> mk;
+      if constexpr (MASKED) mk = load_mask_pack<E, false>(mrow, pk * E, N, true);
 #pragma unroll
-      for (int i = 0; i < E; ++i) sum[0] += row_exp<PRECISE>(p.get(i) - m);
+      for (int i = 0; i < E; ++i) sum[0] += row_exp<PRECISE>(masked_value(p, mk, i) - m);
     }
     group_allreduce<BLOCK, BLOCK, 1, SumOp>(sum, red, phase);
     const float k = is_log ? logf(sum[0]) : 1.0f / sum[0];
+    const bool zero_row = is_safe && m == -INFINITY;
     for (int pk = threadIdx.x; pk < npacks; pk += BLOCK) {
       const int e0 = pk * E;
       const Pack<TI, E> p = load_row_pack<TI, E, true>(xr, e0, N, true, -INFINITY);
+      Pack<uint8_t, E> mk;
+      if constexpr (MASKED) mk = load_mask_pack<E, false>(mrow, e0, N, true);
       Pack<TO, E> o;
 #pragma unroll
       for (int i = 0; i < E; ++i) {
-        const float d = p.get(i) - m;
-        o.set(i, is_log ? d - k : row_exp<PRECISE>(d) * k);
+        const float d = masked_value(p, mk, i) - m;
+        const float v = is_log ? d - k : row_exp<PRECISE>(d) * k;
+        o.set(i, zero_row ? 0.0f : v);
       }
       store_row_pack<TO, E, true>(yr, e0, N, true, o);
     }
@@ -141,10 +221,10 @@ softmax_fwd_stream_kernel(const TI* __restrict__ x, TO* __restrict__ y, int64_t 
 
 // Backward.  TG: dtype of grad and of y (the saved forward output); TO: dtype
 // of the input gradient.
-template <class TG, class TO, int G, int V, int BLOCK, bool FAST>
+template <class TG, class TO, int G, int V, int BLOCK, bool FAST, bool MASKED>
 __global__ void __launch_bounds__(BLOCK)
 softmax_bwd_resident_kernel(const TG* __restrict__ grad, const TG* __restrict__ y,
-                            TO* __restrict__ gi, int64_t M, int N, int is_log) {
+                            TO* __restrict__ gi, MaskRef mask, int64_t M, int N, int flags) {
   constexpr int E = elems_per_pack<TG>::value;
   constexpr int RPB = BLOCK / G;
   constexpr bool PRECISE = sizeof(TO) == 4 && sizeof(TG) == 4;
@@ -152,6 +232,7 @@ softmax_bwd_resident_kernel(const TG* __restrict__ grad, const TG* __restrict__ 
   int phase = 0;
   const int slot = threadIdx.x / G;
   const int lane = threadIdx.x % G;
+  const bool is_log = (flags & kSoftmaxLog) != 0;
   const int64_t nrb = (M + RPB - 1) / RPB;
   for (int64_t rb = blockIdx.x; rb < nrb; rb += gridDim.x) {
     const int64_t row = rb * RPB + slot;
@@ -175,6 +256,15 @@ softmax_bwd_resident_kernel(const TG* __restrict__ grad, const TG* __restrict__ 
         gf[c][i] = pg[c].get(i);
         yf[c][i] = py[c].get(i);
       }
+    if constexpr (MASKED) {
+      const uint8_t* mrow = mask_row_ptr(mask, rowc, N);
+#pragma unroll
+      for (int c = 0; c < V; ++c) {
+        const Pack<uint8_t, E> mk = load_mask_pack<E, FAST>(mrow, (c * G + lane) * E, N, ok);
+#pragma unroll
+        for (int i = 0; i < E; ++i) yf[c][i] = mk.v[i] ? 0.0f : yf[c][i];
+      }
+    }
     float sum[1] = {0.0f};
     if (is_log) {
 #pragma unroll
@@ -204,19 +294,27 @@ softmax_bwd_resident_kernel(const TG* __restrict__ grad, const TG* __restrict__ 
   }
 }
 
-template <class TG, class TO, int BLOCK>
+template <class TG, class TO, int BLOCK, bool MASKED>
 __global__ void __launch_bounds__(BLOCK)
 softmax_bwd_stream_kernel(const TG* __restrict__ grad, const TG* __restrict__ y,
-                          TO* __restrict__ gi, int64_t M, int N, int is_log) {
+                          TO* __restrict__ gi, MaskRef mask, int64_t M, int N, int flags) {
   constexpr int E = elems_per_pack<TG>::value;
   constexpr bool PRECISE = sizeof(TO) == 4 && sizeof(TG) == 4;
   __shared__ float red[reduce_lds_floats<BLOCK, BLOCK, 1>::value];
   int phase = 0;
+  const bool is_log = (flags & kSoftmaxLog) != 0;
   const int npacks = (N + E - 1) / E;
   for (int64_t row = blockIdx.x; row < M; row += gridDim.x) {
     const TG* gr = grad + row * (int64_t)N;
     const TG* yr = y + row * (int64_t)N;
     TO* outr = gi + row * (int64_t)N;
+    const uint8_t* mrow =
+        MASKED ? mask_row_ptr(mask, row, N) : nullptr;
+    auto saved_output = [&](const Pack<TG, E>& p, const Pack<uint8_t, E>& mk, int i) {
+      const float v = p.get(i);
+      if constexpr (MASKED) return mk.v[i] ? 0.0f : v;
+      return v;
+    };
     float sum[1] = {0.0f};
     for (int pk = threadIdx.x; pk < npacks; pk += BLOCK) {
       const Pack<TG, E> pg = load_row_pack<TG, E, false>(gr, pk * E, N, true, 0.0f);
@@ -225,8 +323,10 @@ softmax_bwd_stream_kernel(const TG* __restrict__ grad, const TG* __restrict__ y,
         for (int i = 0; i < E; ++i) sum[0] += pg.get(i);
       } else {
         const Pack<TG, E> py = load_row_pack<TG, E, false>(yr, pk * E, N, true, 0.0f);
+        Pack<uint8_t, E> mk;
+        if constexpr (MASKED) mk = load_mask_pack<E, false>(mrow, pk * E, N, true);
 #pragma unroll
-        for (int i = 0; i < E; ++i) sum[0] = fmaf(py.get(i), pg.get(i), sum[0]);
+        for (int i = 0; i < E; ++i) sum[0] = fmaf(saved_output(py, mk, i), pg.get(i), sum[0]);
       }
     }
     group_allreduce<BLOCK, BLOCK, 1, SumOp>(sum, red, phase);
@@ -235,11 +335,13 @@ softmax_bwd_stream_kernel(const TG* __restrict__ grad, const TG* __restrict__ y,
       const int e0 = pk * E;
       const Pack<TG, E> pg = load_row_pack<TG, E, true>(gr, e0, N, true, 0.0f);
       const Pack<TG, E> py = load_row_pack<TG, E, true>(yr, e0, N, true, 0.0f);
+      Pack<uint8_t, E> mk;
+      if constexpr (MASKED) mk = load_mask_pack<E, false>(mrow, e0, N, true);
       Pack<TO, E> o;
 #pragma unroll
       for (int i = 0; i < E; ++i) {
-        const float v = is_log ? pg.get(i) - row_exp<PRECISE>(py.get(i)) * s
-                               : py.get(i) * (pg.get(i) - s);
+        const float yv = saved_output(py, mk, i);
+        const float v = is_log ? pg.get(i) - row_exp<PRECISE>(yv) * s : yv * (pg.get(i) - s);
         o.set(i, v);
       }
       store_row_pack<TO, E, true>(outr, e0, N, true, o);
