@@ -276,7 +276,23 @@ def per_op_table(torch, cabi, L, dev, stream, P):
         add("C3 %s bwd bf16 [4,32,2048,2048]" % nm, 3 * R * N * 2,
             [(lambda s=s: L.mi355x_softmax_bwd(P(s[1]), P(s[2]), P(s[3]), R, N, BF, BF, is_log,
                                                stream)) for s in sets])
-    del sets
+    # the same scores through _safe_softmax, and through _masked_softmax with the causal mask
+    # as a [T, T] bool tensor read in place and as a full-shape bool tensor
+    add("C3 _safe_softmax fwd bf16 [4,32,2048,2048]", 2 * R * N * 2,
+        [(lambda s=s: L.mi355x_safe_softmax_fwd(P(s[0]), P(s[2]), R, N, BF, BF, stream))
+         for s in sets])
+    causal = torch.triu(torch.ones(2048, 2048, device=dev), 1).bool()
+    full = causal.expand(4 * 32, 2048, 2048).contiguous().view(R, N)
+    add("C3 _masked_softmax fwd bf16, [T,T] mask", 2 * R * N * 2 + N * N,
+        [(lambda s=s: L.mi355x_masked_softmax_fwd(P(s[1]), P(causal), P(s[2]), R, N, N, 1, 0, N, BF,
+                                                  stream)) for s in sets])
+    add("C3 _masked_softmax fwd bf16, full mask", 2 * R * N * 2 + R * N,
+        [(lambda s=s: L.mi355x_masked_softmax_fwd(P(s[1]), P(full), P(s[2]), R, N, R, 1, 1, 1, BF,
+                                                  stream)) for s in sets])
+    add("C3 _masked_softmax_backward bf16, full mask", 3 * R * N * 2 + R * N,
+        [(lambda s=s: L.mi355x_masked_softmax_bwd(P(s[1]), P(s[2]), P(full), P(s[3]), R, N, R, 1, 1,
+                                                  1, BF, stream)) for s in sets])
+    del sets, full
     torch.cuda.empty_cache()
     return rows
 

@@ -220,3 +220,69 @@ def test_aten_override_runs_autograd_end_to_end(pkg, gpu):
                 assert a is not None, "%s: %s is missing on the GPU" % (name, nm)
                 assert a.dtype == dtype
                 assert_close(a, r, dtype, "%s %s" % (name, nm), scale=4.0)
+
+
+def test_aten_override_masked_and_safe_softmax_autograd(pkg, gpu):
+    """torch._masked_softmax / torch._safe_softmax on GPU tensors after the opt-in, forward and
+    through autograd, against the CPU: the sizes, dims and mask types of
+    test/xpu/test_nn_xpu.py:13744-13965 (test_masked_softmax_mask_types, _lowp, _grad) and
+    test/regressions/test_safe_softmax.py:18-52 in the reference."""
+    import warnings
+    with warnings.catch_warnings():
+        warnings.simplefilter("ignore")
+        pkg.override_aten_ops()
+    g = gen(50)
+    for (B, H, L) in ((1, 1, 32), (3, 4, 310), (2, 2, 1200)):
+        src = torch.randint(0, 2, (L, L), generator=g).bool()
+        pad = torch.randint(0, 2, (B, L), generator=g).bool()
+        generic = torch.randint(0, 2, (B, H, L, L), generator=g).bool()
+        expanded = {0: src.reshape(1, 1, L, L).expand(B, H, L, L),
+                    1: pad.reshape(B, 1, 1, L).expand(B, H, L, L), 2: generic}
+        for dtype in (torch.float32, torch.bfloat16):
+            x = torch.randn(B, H, L, L, generator=g).to(dtype)
+            dy = torch.randn(B, H, L, L, generator=g).to(dtype)
+            for dim in (0, 3):
+                for mask, mtype in ((src, 0), (pad, 1), (generic, 2)):
+                    print("case override masked", (B, H, L), dtype, dim, mtype, flush=True)
+                    dead = expanded[mtype].all(dim, keepdim=True).expand(B, H, L, L)
+                    # forward with the mask in its own layout
+                    out = torch._masked_softmax(x.to(gpu), mask.to(gpu), dim, mtype)
+                    ref = torch._masked_softmax(x.float(), mask, dim, mtype)
+                    assert out.dtype == dtype
+                    # fully masked slices are unspecified in the reference's tests (NaN or 0)
+                    assert_close(out.cpu().masked_fill(dead, 0), ref.masked_fill(dead, 0), dtype,
+                                 "masked out")
+                    if mtype == 0:
+                        continue
+                    # autograd hands the forward's mask to _masked_softmax_backward, which wants
+                    # it in the gradient's shape: expanded masks, as test_masked_softmax_lowp uses
+                    full = expanded[mtype]
+                    xs = x.detach().clone().to(gpu).requires_grad_()
+                    out = torch._masked_softmax(xs, full.to(gpu), dim, mtype)
+                    out.backward(dy.to(gpu))
+                    xr = x.float().detach().clone().requires_grad_()
+                    torch._masked_softmax(xr, full, dim, mtype).backward(dy.float())
+                    assert xs.grad.dtype == dtype
+                    assert_close(out.detach().cpu().masked_fill(dead, 0), ref.masked_fill(dead, 0),
+                                 dtype, "masked out (expanded mask)")
+                    assert_close(xs.grad.cpu().masked_fill(dead, 0), xr.grad.masked_fill(dead, 0), dtype,
+                                 "masked dx", scale=2.0)
+                    assert bool((xs.grad.cpu()[full & ~dead] == 0).all())
+    for dtype in (torch.float32, torch.float16, torch.bfloat16):
+        x = torch.randn(32, 48, 64, generator=g).to(dtype)
+        dy = torch.randn(32, 48, 64, generator=g).to(dtype)
+        for dim, sl in ((-1, (0, 0, slice(None))), (1, (0, slice(None), 0)), (0, (slice(None), 0, 0))):
+            for poison in (False, True):
+                xc = x.clone()
+                if poison:
+                    xc[sl] = float("-inf")
+                xs = xc.detach().clone().to(gpu).requires_grad_()
+                out = torch.ops.aten._safe_softmax(xs, dim)
+                out.backward(dy.to(gpu))
+                xr = xc.float().detach().clone().requires_grad_()
+                ref = torch.ops.aten._safe_softmax(xr, dim)
+                ref.backward(dy.float())
+                assert_close(out, ref, dtype, "safe out dim=%d" % dim)
+                assert_close(xs.grad, xr.grad, dtype, "safe dx dim=%d" % dim, scale=2.0)
+                if poison:
+                    assert bool((out.detach()[sl] == 0).all())
