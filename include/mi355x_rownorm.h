@@ -56,8 +56,17 @@ typedef enum {
   ROWNORM_OP_RMS_NORM_BWD = 3,
   ROWNORM_OP_SOFTMAX_FWD = 4,
   ROWNORM_OP_SOFTMAX_BWD = 5,
-  ROWNORM_OP_COUNT = 6
+  ROWNORM_OP_SOFTMAX_STRIDED_FWD = 6, /* mi355x_softmax_strided_fwd (override / strided_plan only) */
+  ROWNORM_OP_SOFTMAX_STRIDED_BWD = 7,
+  ROWNORM_OP_COUNT = 8
 } rownorm_op;
+
+/* `mode` of the strided softmax entry points. */
+enum {
+  ROWNORM_SOFTMAX = 0,
+  ROWNORM_LOG_SOFTMAX = 1,
+  ROWNORM_SAFE_SOFTMAX = 2 /* forward only: slices with no finite element give 0 */
+};
 
 /* How one call is laid out on the GPU.  Replaces the reference's NormConfig
  * heuristics (src/ATen/native/xpu/sycl/Norm.h:225-370) and get_wgroup_size
@@ -171,10 +180,37 @@ int mi355x_masked_softmax_bwd(const void* grad, const void* y, const void* mask,
                               int64_t mask_row_stride, int64_t mask_row_mod, rownorm_dtype dtype,
                               void* stream);
 
+/* _softmax / _log_softmax / _safe_softmax over a dimension that is not
+ * innermost: the dense tensor is viewed as [outer, dim_size, inner] and each of
+ * the outer * inner columns of dim_size elements (inner apart in memory) is
+ * normalized.  Replaces the spatial branch of host_softmax
+ * (SoftMaxKernels.cpp:1721-1736, SpatialSoftmaxForwardKernelFunctor :725-950),
+ * which the reference takes whenever inner_size != 1.  inner == 1 forwards to
+ * the innermost-dimension kernels.  Dtypes as for mi355x_softmax_fwd; dim_size
+ * and inner are limited to 2^30. */
+int mi355x_softmax_strided_fwd(const void* x, void* y, int64_t outer, int64_t dim_size,
+                               int64_t inner, rownorm_dtype in_dtype, rownorm_dtype out_dtype,
+                               int mode, void* stream);
+
+/* Backward of the above (SpatialSoftmaxBackwardKernelFunctor,
+ * SoftMaxKernels.cpp:1387-1564, dispatched at :1877-1894).  mode is
+ * ROWNORM_SOFTMAX or ROWNORM_LOG_SOFTMAX; dtypes as for mi355x_softmax_bwd. */
+int mi355x_softmax_strided_bwd(const void* grad, const void* y, void* gi, int64_t outer,
+                               int64_t dim_size, int64_t inner, rownorm_dtype grad_dtype,
+                               rownorm_dtype gi_dtype, int mode, void* stream);
+
+/* Launch layout of a strided softmax call (no launch).  In the result,
+ * lanes_per_row is the number of lanes along `inner` (one 16-byte pack each),
+ * rows_per_block the number of threads along dim_size that share one such
+ * lane position, packs_per_lane the dim_size rows each of those holds;
+ * resident == 0 means the multi-pass kernel. */
+int mi355x_softmax_strided_plan(int backward, int64_t outer, int64_t dim_size, int64_t inner,
+                                rownorm_dtype dtype, rownorm_plan* out);
+
 /* Reports the launch layout a call with these sizes would use on the current
  * device (no launch; needs no GPU when the device query fails: 256 compute
  * units are assumed).  x_dtype is the row dtype, w_dtype the weight dtype
- * (ignored by the softmax ops). */
+ * (ignored by the softmax ops).  The strided softmax ops have their own query above. */
 int mi355x_rownorm_plan(rownorm_op op, int64_t M, int64_t N, rownorm_dtype x_dtype,
                         rownorm_dtype w_dtype, rownorm_plan* out);
 

@@ -166,3 +166,50 @@ def test_forced_variants(cabi):
         cabi.plan(cabi.OP_SOFTMAX_FWD, 64, 2048, cabi.BF16, cabi.BF16)
     cabi.clear_overrides()
     assert cabi.plan(cabi.OP_SOFTMAX_FWD, 64, 2048, cabi.BF16, cabi.BF16)["resident"] == 1
+
+
+def test_strided_softmax_validation_and_plans(cabi):
+    L = cabi.lib()
+    one, null = ctypes.c_void_p(256), None
+    f = L.mi355x_softmax_strided_fwd
+    b = L.mi355x_softmax_strided_bwd
+    assert f(one, one, 2, 3, 4, cabi.BF16, cabi.F32, 0, null) == -1       # only f16 -> f32
+    assert f(one, one, 2, -1, 4, 0, 0, 0, null) == -2
+    assert f(one, one, 2, 3, (1 << 30) + 1, 0, 0, 0, null) == -2
+    assert f(one, one, 2, 3, 4, 0, 0, 3, null) == -2                       # unknown mode
+    assert b(one, one, one, 2, 3, 4, 0, 0, cabi.SAFE_SOFTMAX, null) == -2  # no safe backward
+    assert f(null, null, 2, 3, 4, 0, 0, 0, null) == -3
+    assert b(one, null, one, 2, 3, 4, 0, 0, 0, null) == -3
+    for dims in ((0, 3, 4), (2, 0, 4), (2, 3, 0)):
+        assert f(null, null, *dims, 0, 0, 0, null) == 0
+        assert b(null, null, null, *dims, 0, 0, 0, null) == 0
+    for dt, E in ((cabi.F32, 4), (cabi.BF16, 8)):
+        for outer in (1, 7, 4096):
+            for D in (1, 2, 5, 32, 100, 256, 257, 2048, 100000):
+                for inner in (2, 3, 8, 9, 100, 512, 513, 65536):
+                    for bwd in (0, 1):
+                        p = cabi.strided_plan(bwd, outer, D, inner, dt)
+                        TX, TY, V = p["lanes_per_row"], p["rows_per_block"], p["packs_per_lane"]
+                        assert 1 <= TX <= 64 and TX & (TX - 1) == 0 and TY & (TY - 1) == 0
+                        assert TX * TY <= p["block_threads"] == 256
+                        packs = -(-inner // E)
+                        assert TX <= max(1, 1 << (packs - 1).bit_length())
+                        tiles = outer * -(-packs // TX)
+                        groups = 256 // (TX * TY)
+                        assert 1 <= p["grid_blocks"] <= -(-tiles // groups)
+                        if p["resident"]:
+                            assert V in (1, 2, 4, 8) and TY * V >= D, "every row of D must be held"
+                            if TX * TY > 64:  # more than a wavefront only when rows would get too short
+                                assert TX <= 8
+                        else:
+                            assert D > 8 * 256 // min(4, 1 << (packs - 1).bit_length())
+    # D = 256 fits the registers once the lanes along inner shrink to 8
+    p = cabi.strided_plan(0, 4, 256, 4096, cabi.BF16)
+    assert p["resident"] == 1 and p["lanes_per_row"] == 8 and p["packs_per_lane"] == 8
+    # forced layouts that cannot hold D are refused
+    cabi.set_override(cabi.OP_SOFTMAX_STRIDED_FWD, 64, 1)
+    with pytest.raises(RuntimeError, match="forced variant"):
+        cabi.strided_plan(0, 4, 5, 4096, cabi.BF16)
+    cabi.set_override(cabi.OP_SOFTMAX_STRIDED_FWD, -1)
+    assert cabi.strided_plan(0, 4, 5, 4096, cabi.BF16)["resident"] == 0
+    cabi.clear_overrides()

@@ -13,13 +13,16 @@ _KERNEL_LIB = os.path.join(_HERE, "lib", "libmi355x_rownorm.so")
 F32, F16, BF16 = 0, 1, 2
 OP_LAYER_NORM_FWD, OP_LAYER_NORM_BWD, OP_RMS_NORM_FWD, OP_RMS_NORM_BWD = 0, 1, 2, 3
 OP_SOFTMAX_FWD, OP_SOFTMAX_BWD = 4, 5
+OP_SOFTMAX_STRIDED_FWD, OP_SOFTMAX_STRIDED_BWD = 6, 7
+SOFTMAX, LOG_SOFTMAX, SAFE_SOFTMAX = 0, 1, 2
 
 EXPORTED_SYMBOLS = (
     "mi355x_rownorm_error_string", "mi355x_rownorm_abi_version", "mi355x_layer_norm_fwd",
     "mi355x_layer_norm_bwd_workspace_bytes", "mi355x_layer_norm_bwd", "mi355x_rms_norm_fwd",
     "mi355x_rms_norm_bwd_workspace_bytes", "mi355x_rms_norm_bwd", "mi355x_softmax_fwd",
     "mi355x_softmax_bwd", "mi355x_safe_softmax_fwd", "mi355x_masked_softmax_fwd",
-    "mi355x_masked_softmax_bwd", "mi355x_rownorm_plan", "mi355x_rownorm_set_override",
+    "mi355x_masked_softmax_bwd", "mi355x_softmax_strided_fwd", "mi355x_softmax_strided_bwd",
+    "mi355x_softmax_strided_plan", "mi355x_rownorm_plan", "mi355x_rownorm_set_override",
 )
 
 
@@ -65,12 +68,19 @@ def lib():
                                                 _int, _vp]
         L.mi355x_masked_softmax_bwd.argtypes = [_vp, _vp, _vp, _vp, _i64, _i64, _i64, _i64, _i64,
                                                 _i64, _int, _vp]
+        L.mi355x_softmax_strided_fwd.argtypes = [_vp, _vp, _i64, _i64, _i64, _int, _int, _int, _vp]
+        L.mi355x_softmax_strided_bwd.argtypes = [_vp, _vp, _vp, _i64, _i64, _i64, _int, _int, _int,
+                                                 _vp]
+        L.mi355x_softmax_strided_plan.argtypes = [_int, _i64, _i64, _i64, _int,
+                                                  ctypes.POINTER(Plan)]
         L.mi355x_rownorm_plan.argtypes = [_int, _i64, _i64, _int, _int, ctypes.POINTER(Plan)]
         L.mi355x_rownorm_set_override.argtypes = [_int, _int, _int, _int, _int]
         for name in ("mi355x_layer_norm_fwd", "mi355x_rms_norm_fwd", "mi355x_layer_norm_bwd",
                      "mi355x_rms_norm_bwd", "mi355x_softmax_fwd", "mi355x_softmax_bwd",
                      "mi355x_safe_softmax_fwd", "mi355x_masked_softmax_fwd",
-                     "mi355x_masked_softmax_bwd", "mi355x_rownorm_plan", "mi355x_rownorm_set_override"):
+                     "mi355x_masked_softmax_bwd", "mi355x_softmax_strided_fwd",
+                     "mi355x_softmax_strided_bwd", "mi355x_softmax_strided_plan",
+                     "mi355x_rownorm_plan", "mi355x_rownorm_set_override"):
             getattr(L, name).restype = _int
         _lib = L
     return _lib
@@ -104,8 +114,15 @@ def set_override(op, lanes_per_row=0, packs_per_lane=0, block_threads=0, blocks_
                                              blocks_per_cu), "set_override")
 
 
+def strided_plan(backward, outer, dim_size, inner, dtype=F32):
+    p = Plan()
+    _check(lib().mi355x_softmax_strided_plan(int(backward), outer, dim_size, inner, dtype,
+                                             ctypes.byref(p)), "strided_plan")
+    return p.as_dict()
+
+
 def clear_overrides():
-    for op in range(6):
+    for op in range(8):
         set_override(op)
 
 
@@ -301,4 +318,39 @@ def masked_softmax_bwd(grad, y, mask, gi=None, row_map=None):
     _check(lib().mi355x_masked_softmax_bwd(_ptr(grad), _ptr(y), _ptr(mask), _ptr(gi), rows, N,
                                            mrows, div, stride, mod, dtype_code(grad.dtype),
                                            _stream()), "masked_softmax_bwd")
+    return gi
+
+
+def _outer_dim_inner(shape, dim):
+    dim = dim % len(shape)
+    outer = inner = 1
+    for s in shape[:dim]:
+        outer *= s
+    for s in shape[dim + 1:]:
+        inner *= s
+    return outer, shape[dim], inner
+
+
+def softmax_strided_fwd(x, dim, mode=SOFTMAX, out_dtype=None, y=None):
+    """softmax (mode SOFTMAX / LOG_SOFTMAX / SAFE_SOFTMAX) over any dim of a dense tensor."""
+    import torch
+    _gpu(x)
+    outer, D, inner = _outer_dim_inner(x.shape, dim)
+    od = x.dtype if out_dtype is None else out_dtype
+    y = torch.empty(x.shape, dtype=od, device=x.device) if y is None else y
+    _check(lib().mi355x_softmax_strided_fwd(_ptr(x), _ptr(y), outer, D, inner, dtype_code(x.dtype),
+                                            dtype_code(y.dtype), mode, _stream()),
+           "softmax_strided_fwd")
+    return y
+
+
+def softmax_strided_bwd(grad, y, dim, mode=SOFTMAX, gi_dtype=None, gi=None):
+    import torch
+    _gpu(grad, y)
+    outer, D, inner = _outer_dim_inner(y.shape, dim)
+    od = grad.dtype if gi_dtype is None else gi_dtype
+    gi = torch.empty(y.shape, dtype=od, device=y.device) if gi is None else gi
+    _check(lib().mi355x_softmax_strided_bwd(_ptr(grad), _ptr(y), _ptr(gi), outer, D, inner,
+                                            dtype_code(grad.dtype), dtype_code(gi.dtype), mode,
+                                            _stream()), "softmax_strided_bwd")
     return gi

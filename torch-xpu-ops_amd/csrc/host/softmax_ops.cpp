@@ -2,9 +2,10 @@
 // src/ATen/native/xpu/SoftMax.cpp:22-100 and the host_softmax /
 // host_softmax_backward entry code in SoftMaxKernels.cpp:2125-2276.
 //
-// The kernels reduce over the innermost dimension of a dense tensor.  A
-// reduction over another dimension is served by moving that dimension last
-// (one transposing copy in, one out) rather than by a separate strided kernel.
+// The kernels work on dense tensors: the innermost-dimension kernels for
+// dim == -1, the [outer, dim, inner] kernels for any other dimension (no
+// transposing copies).  Only a masked softmax over a non-innermost dimension
+// moves that dimension last first.
 #include "softmax_ops.h"
 
 #include <ATen/WrapDimUtils.h>
@@ -19,30 +20,33 @@ using at::Tensor;
 
 enum class Mode { kSoftmax, kLogSoftmax, kSafeSoftmax };
 
-// Forward on dense [rows, N] data where `dim` is already innermost.
-void forward_lastdim(const Tensor& in, const Tensor& out, Mode mode, const char* op) {
-  const int64_t N = in.dim() == 0 ? 1 : in.size(-1);
-  const int64_t rows = N == 0 ? 0 : in.numel() / N;
-  const rownorm_dtype id = to_rownorm_dtype(in.scalar_type(), op);
-  const rownorm_dtype od = to_rownorm_dtype(out.scalar_type(), op);
-  const int rc =
-      mode == Mode::kSafeSoftmax
-          ? mi355x_safe_softmax_fwd(in.const_data_ptr(), out.mutable_data_ptr(), rows, N, id, od,
-                                    current_stream(in))
-          : mi355x_softmax_fwd(in.const_data_ptr(), out.mutable_data_ptr(), rows, N, id, od,
-                               mode == Mode::kLogSoftmax ? 1 : 0, current_stream(in));
-  check_status(rc, op);
+// Forward over dimension `dim` of the dense tensor `in` into the dense `out`.
+void forward_dense(const Tensor& in, const Tensor& out, int64_t dim, Mode mode, const char* op) {
+  int64_t outer = 1, inner = 1;
+  for (int64_t i = 0; i < dim; ++i) outer *= in.size(i);
+  for (int64_t i = dim + 1; i < in.dim(); ++i) inner *= in.size(i);
+  const int abi_mode = mode == Mode::kSafeSoftmax  ? ROWNORM_SAFE_SOFTMAX
+                       : mode == Mode::kLogSoftmax ? ROWNORM_LOG_SOFTMAX
+                                                   : ROWNORM_SOFTMAX;
+  check_status(mi355x_softmax_strided_fwd(in.const_data_ptr(), out.mutable_data_ptr(), outer,
+                                          in.size(dim), inner,
+                                          to_rownorm_dtype(in.scalar_type(), op),
+                                          to_rownorm_dtype(out.scalar_type(), op), abi_mode,
+                                          current_stream(in)),
+               op);
 }
 
-void backward_lastdim(const Tensor& grad, const Tensor& y, const Tensor& gi, bool is_log,
-                      const char* op) {
-  const int64_t N = y.dim() == 0 ? 1 : y.size(-1);
-  const int64_t rows = N == 0 ? 0 : y.numel() / N;
-  check_status(mi355x_softmax_bwd(grad.const_data_ptr(), y.const_data_ptr(),
-                                  gi.mutable_data_ptr(), rows, N,
-                                  to_rownorm_dtype(grad.scalar_type(), op),
-                                  to_rownorm_dtype(gi.scalar_type(), op), is_log ? 1 : 0,
-                                  current_stream(y)),
+void backward_dense(const Tensor& grad, const Tensor& y, const Tensor& gi, int64_t dim,
+                    bool is_log, const char* op) {
+  int64_t outer = 1, inner = 1;
+  for (int64_t i = 0; i < dim; ++i) outer *= y.size(i);
+  for (int64_t i = dim + 1; i < y.dim(); ++i) inner *= y.size(i);
+  check_status(mi355x_softmax_strided_bwd(grad.const_data_ptr(), y.const_data_ptr(),
+                                          gi.mutable_data_ptr(), outer, y.size(dim), inner,
+                                          to_rownorm_dtype(grad.scalar_type(), op),
+                                          to_rownorm_dtype(gi.scalar_type(), op),
+                                          is_log ? ROWNORM_LOG_SOFTMAX : ROWNORM_SOFTMAX,
+                                          current_stream(y)),
                op);
 }
 
@@ -68,20 +72,13 @@ void softmax_forward_entry(const Tensor& input_, int64_t dim_, bool half_to_floa
   const int64_t dim = at::maybe_wrap_dim(dim_, input.dim());
   if (input.numel() == 0) return;
   c10::DeviceGuard guard(input.device());
-  if (dim == input.dim() - 1) {
-    const Tensor in_c = input.contiguous();
-    if (out.is_contiguous()) {
-      forward_lastdim(in_c, out, mode, op);
-    } else {
-      Tensor tmp = at::empty_like(out, out.options(), at::MemoryFormat::Contiguous);
-      forward_lastdim(in_c, tmp, mode, op);
-      out.copy_(tmp);
-    }
+  const Tensor in_c = input.contiguous();
+  if (out.is_contiguous()) {
+    forward_dense(in_c, out, dim, mode, op);
   } else {
-    const Tensor in_t = input.movedim(dim, -1).contiguous();
-    Tensor out_t = at::empty(in_t.sizes(), out.options());
-    forward_lastdim(in_t, out_t, mode, op);
-    out.copy_(out_t.movedim(-1, dim));
+    Tensor tmp = at::empty_like(out, out.options(), at::MemoryFormat::Contiguous);
+    forward_dense(in_c, tmp, dim, mode, op);
+    out.copy_(tmp);
   }
 }
 
@@ -112,22 +109,14 @@ void softmax_backward_entry(const Tensor& grad_, const Tensor& output_, int64_t 
   const int64_t dim = at::maybe_wrap_dim(dim_, grad.dim());
   if (grad.numel() == 0) return;
   c10::DeviceGuard guard(grad.device());
-  if (dim == grad.dim() - 1) {
-    const Tensor g_c = grad.contiguous();
-    const Tensor y_c = y.contiguous();
-    if (gi.is_contiguous()) {
-      backward_lastdim(g_c, y_c, gi, is_log, op);
-    } else {
-      Tensor tmp = at::empty_like(gi, gi.options(), at::MemoryFormat::Contiguous);
-      backward_lastdim(g_c, y_c, tmp, is_log, op);
-      gi.copy_(tmp);
-    }
+  const Tensor g_c = grad.contiguous();
+  const Tensor y_c = y.contiguous();
+  if (gi.is_contiguous()) {
+    backward_dense(g_c, y_c, gi, dim, is_log, op);
   } else {
-    const Tensor g_t = grad.movedim(dim, -1).contiguous();
-    const Tensor y_t = y.movedim(dim, -1).contiguous();
-    Tensor gi_t = at::empty(g_t.sizes(), gi.options());
-    backward_lastdim(g_t, y_t, gi_t, is_log, op);
-    gi.copy_(gi_t.movedim(-1, dim));
+    Tensor tmp = at::empty_like(gi, gi.options(), at::MemoryFormat::Contiguous);
+    backward_dense(g_c, y_c, tmp, dim, is_log, op);
+    gi.copy_(tmp);
   }
 }
 

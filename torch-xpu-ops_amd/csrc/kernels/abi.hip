@@ -36,6 +36,14 @@ extern template int launch_softmax_bwd<float, float>(const Plan&, const SoftmaxB
 extern template int launch_softmax_bwd<f16, f16>(const Plan&, const SoftmaxBwdArgs&, hipStream_t);
 extern template int launch_softmax_bwd<bf16, bf16>(const Plan&, const SoftmaxBwdArgs&, hipStream_t);
 extern template int launch_softmax_bwd<float, f16>(const Plan&, const SoftmaxBwdArgs&, hipStream_t);
+extern template int launch_softmax_strided_fwd<float, float>(const StridedPlan&, const SoftmaxStridedFwdArgs&, hipStream_t);
+extern template int launch_softmax_strided_fwd<f16, f16>(const StridedPlan&, const SoftmaxStridedFwdArgs&, hipStream_t);
+extern template int launch_softmax_strided_fwd<bf16, bf16>(const StridedPlan&, const SoftmaxStridedFwdArgs&, hipStream_t);
+extern template int launch_softmax_strided_fwd<f16, float>(const StridedPlan&, const SoftmaxStridedFwdArgs&, hipStream_t);
+extern template int launch_softmax_strided_bwd<float, float>(const StridedPlan&, const SoftmaxStridedBwdArgs&, hipStream_t);
+extern template int launch_softmax_strided_bwd<f16, f16>(const StridedPlan&, const SoftmaxStridedBwdArgs&, hipStream_t);
+extern template int launch_softmax_strided_bwd<bf16, bf16>(const StridedPlan&, const SoftmaxStridedBwdArgs&, hipStream_t);
+extern template int launch_softmax_strided_bwd<float, f16>(const StridedPlan&, const SoftmaxStridedBwdArgs&, hipStream_t);
 }  // namespace rownorm
 
 using namespace rownorm;
@@ -228,6 +236,23 @@ int softmax_bwd(const void* grad, const void* y, const void* mask, void* gi, int
                            : launch_softmax_bwd<float, float>(plan, a, s);
 }
 
+int softmax_mode_flags(int mode, bool forward, int* flags) {
+  switch (mode) {
+    case ROWNORM_SOFTMAX: *flags = 0; return 0;
+    case ROWNORM_LOG_SOFTMAX: *flags = kSoftmaxLog; return 0;
+    case ROWNORM_SAFE_SOFTMAX:
+      if (!forward) break;  // its backward is the plain softmax backward
+      *flags = kSoftmaxSafe;
+      return 0;
+  }
+  return ROWNORM_ERR_SHAPE;
+}
+
+int strided_shape_check(int64_t outer, int64_t D, int64_t inner) {
+  if (outer < 0 || D < 0 || inner < 0 || D > kMaxN || inner > kMaxN) return ROWNORM_ERR_SHAPE;
+  return 0;
+}
+
 }  // namespace
 
 extern "C" {
@@ -328,10 +353,81 @@ int mi355x_masked_softmax_bwd(const void* grad, const void* y, const void* mask,
                      (int)dtype, 0, stream);
 }
 
+int mi355x_softmax_strided_fwd(const void* x, void* y, int64_t outer, int64_t dim_size,
+                               int64_t inner, rownorm_dtype in_dtype, rownorm_dtype out_dtype,
+                               int mode, void* stream) {
+  const int id = (int)in_dtype, od = (int)out_dtype;
+  int flags = 0;
+  if (esize_of(id) == 0 || esize_of(od) == 0) return ROWNORM_ERR_DTYPE;
+  if (!(od == id || (id == ROWNORM_F16 && od == ROWNORM_F32))) return ROWNORM_ERR_DTYPE;
+  if (int e = strided_shape_check(outer, dim_size, inner)) return e;
+  if (int e = softmax_mode_flags(mode, true, &flags)) return e;
+  if (outer == 0 || dim_size == 0 || inner == 0) return 0;
+  if (inner == 1)  // the reduced dimension is innermost after all
+    return softmax_fwd(x, nullptr, y, outer, dim_size, MaskRows{}, id, od, flags, stream);
+  if (!x || !y) return ROWNORM_ERR_NULL;
+  StridedPlan plan;
+  if (int e = make_strided_plan(false, outer, dim_size, inner, esize_of(id), current_num_cus(),
+                                g_override[ROWNORM_OP_SOFTMAX_STRIDED_FWD], &plan))
+    return e;
+  SoftmaxStridedFwdArgs a{x, y, outer, (int)dim_size, (int)inner, flags};
+  hipStream_t s = (hipStream_t)stream;
+  if (id == ROWNORM_F32) return launch_softmax_strided_fwd<float, float>(plan, a, s);
+  if (id == ROWNORM_BF16) return launch_softmax_strided_fwd<bf16, bf16>(plan, a, s);
+  return od == ROWNORM_F32 ? launch_softmax_strided_fwd<f16, float>(plan, a, s)
+                           : launch_softmax_strided_fwd<f16, f16>(plan, a, s);
+}
+
+int mi355x_softmax_strided_bwd(const void* grad, const void* y, void* gi, int64_t outer,
+                               int64_t dim_size, int64_t inner, rownorm_dtype grad_dtype,
+                               rownorm_dtype gi_dtype, int mode, void* stream) {
+  const int gd = (int)grad_dtype, od = (int)gi_dtype;
+  int flags = 0;
+  if (esize_of(gd) == 0 || esize_of(od) == 0) return ROWNORM_ERR_DTYPE;
+  if (!(od == gd || (gd == ROWNORM_F32 && od == ROWNORM_F16))) return ROWNORM_ERR_DTYPE;
+  if (int e = strided_shape_check(outer, dim_size, inner)) return e;
+  if (int e = softmax_mode_flags(mode, false, &flags)) return e;
+  if (outer == 0 || dim_size == 0 || inner == 0) return 0;
+  if (inner == 1)
+    return softmax_bwd(grad, y, nullptr, gi, outer, dim_size, MaskRows{}, gd, od, flags, stream);
+  if (!grad || !y || !gi) return ROWNORM_ERR_NULL;
+  StridedPlan plan;
+  if (int e = make_strided_plan(true, outer, dim_size, inner, esize_of(gd), current_num_cus(),
+                                g_override[ROWNORM_OP_SOFTMAX_STRIDED_BWD], &plan))
+    return e;
+  SoftmaxStridedBwdArgs a{grad, y, gi, outer, (int)dim_size, (int)inner, flags};
+  hipStream_t s = (hipStream_t)stream;
+  if (gd == ROWNORM_BF16) return launch_softmax_strided_bwd<bf16, bf16>(plan, a, s);
+  if (gd == ROWNORM_F16) return launch_softmax_strided_bwd<f16, f16>(plan, a, s);
+  return od == ROWNORM_F16 ? launch_softmax_strided_bwd<float, f16>(plan, a, s)
+                           : launch_softmax_strided_bwd<float, float>(plan, a, s);
+}
+
+int mi355x_softmax_strided_plan(int backward, int64_t outer, int64_t dim_size, int64_t inner,
+                                rownorm_dtype dtype, rownorm_plan* out) {
+  if (!out) return ROWNORM_ERR_NULL;
+  if (esize_of((int)dtype) == 0) return ROWNORM_ERR_DTYPE;
+  if (int e = strided_shape_check(outer, dim_size, inner)) return e;
+  StridedPlan plan;
+  const int op = backward ? ROWNORM_OP_SOFTMAX_STRIDED_BWD : ROWNORM_OP_SOFTMAX_STRIDED_FWD;
+  if (int e = make_strided_plan(backward != 0, outer, dim_size, inner, esize_of((int)dtype),
+                                current_num_cus(), g_override[op], &plan))
+    return e;
+  out->resident = plan.resident ? 1 : 0;
+  out->lanes_per_row = 1 << plan.tx_log2;
+  out->packs_per_lane = plan.V;
+  out->block_threads = plan.block;
+  out->rows_per_block = 1 << plan.ty_log2;
+  out->reserved = 0;
+  out->grid_blocks = plan.grid;
+  out->partial_rows = 0;
+  return 0;
+}
+
 int mi355x_rownorm_plan(rownorm_op op, int64_t M, int64_t N, rownorm_dtype x_dtype,
                         rownorm_dtype w_dtype, rownorm_plan* out) {
   (void)w_dtype;
-  if ((int)op < 0 || (int)op >= ROWNORM_OP_COUNT) return ROWNORM_ERR_SHAPE;
+  if ((int)op < 0 || (int)op > ROWNORM_OP_SOFTMAX_BWD) return ROWNORM_ERR_SHAPE;
   if (!out) return ROWNORM_ERR_NULL;
   if (esize_of((int)x_dtype) == 0) return ROWNORM_ERR_DTYPE;
   if (int e = shape_check(M, N)) return e;

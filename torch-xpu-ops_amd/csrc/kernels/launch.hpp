@@ -62,6 +62,23 @@ struct SoftmaxBwdArgs {
   int flags;
 };
 
+struct SoftmaxStridedFwdArgs {
+  const void* x;
+  void* y;
+  int64_t outer;
+  int D, inner;
+  int flags;
+};
+
+struct SoftmaxStridedBwdArgs {
+  const void* grad;
+  const void* y;
+  void* gi;
+  int64_t outer;
+  int D, inner;
+  int flags;
+};
+
 // All return 0 or a hipError_t value.
 template <class T, class WT, bool RMS>
 int launch_norm_fwd(const Plan& plan, const NormFwdArgs& a, hipStream_t stream);
@@ -71,6 +88,13 @@ template <class TI, class TO>
 int launch_softmax_fwd(const Plan& plan, const SoftmaxFwdArgs& a, hipStream_t stream);
 template <class TG, class TO>
 int launch_softmax_bwd(const Plan& plan, const SoftmaxBwdArgs& a, hipStream_t stream);
+
+template <class TI, class TO>
+int launch_softmax_strided_fwd(const StridedPlan& plan, const SoftmaxStridedFwdArgs& a,
+                               hipStream_t stream);
+template <class TG, class TO>
+int launch_softmax_strided_bwd(const StridedPlan& plan, const SoftmaxStridedBwdArgs& a,
+                               hipStream_t stream);
 
 // Compile-time walk over every (G, V, BLOCK) a kernel family may be built for;
 // L<G, V, BLOCK>::run(ctx) returns true when it matched the plan and launched.

@@ -185,4 +185,95 @@ inline int make_plan(OpClass oc, int64_t M, int64_t N, int esize, int num_cus, c
   return 0;
 }
 
+// ---- softmax over a non-innermost dimension: [outer, D, inner] ----------------
+//
+// A group of TX * TY threads owns one tile: TX lanes along `inner` (one 16-byte
+// pack each) by TY threads along D, each holding V packs, so the registers
+// cover D <= TY * V rows.  The rule: V = 8 packs a lane (fewer when D is
+// smaller; 4 for the 16-bit backward of D <= 32), TY = the power of two that then covers D, and TX = as many lanes
+// as a row of `inner` has packs, capped so that a group is one wavefront where
+// that leaves at least 8 lanes (128-byte segments) per row, and 256 threads
+// otherwise.  A group of one wavefront reduces with shuffles alone.  D beyond
+// 64 rows x 8 packs x 4 lanes takes the multi-pass kernel.
+struct StridedPlan {
+  bool resident = true;
+  bool fast = true;  // inner % E == 0
+  int tx_log2 = 0, ty_log2 = 0, V = 0, block = 0;
+  int64_t grid = 0;
+};
+
+constexpr int kStridedBlock = 256;
+constexpr int kStridedMaxV = 8;
+
+inline int log2_of_pow2(int v) {
+  int l = 0;
+  while ((1 << l) < v) ++l;
+  return l;
+}
+
+// Override: G = lanes along inner (power of two 1..64; -1 forces the multi-pass
+// kernel), V = packs per lane.  Returns 0 or -5.
+inline int make_strided_plan(bool backward, int64_t outer, int64_t D, int64_t inner, int esize,
+                             int num_cus, const Override& ov, StridedPlan* out) {
+  StridedPlan p;
+  const int E = 16 / esize;
+  const int64_t packs = (inner + E - 1) / E;
+  p.fast = (inner % E) == 0;
+  p.block = kStridedBlock;
+  if (num_cus <= 0) num_cus = 256;
+  const int px = packs >= 64 ? 64 : pow2_ceil(packs);  // lanes a row of `inner` can use
+  int V = ov.V > 0 ? ov.V : (D >= kStridedMaxV ? kStridedMaxV : pow2_ceil(D));
+  // measured: the 16-bit backward (two packed rows per lane) runs faster with 4
+  // packs a lane while a wavefront still covers D
+  if (ov.V == 0 && backward && esize == 2 && D > 4 && D <= 32) V = 4;
+  if (V < 1 || V > kStridedMaxV || (V & (V - 1))) return -5;
+  const int64_t ty_need = pow2_ceil((D + V - 1) / V);
+  int TX = 0, TY = 0;
+  // rows are never cut below 4 lanes (64 bytes) to make room for a larger D
+  const int ty_max = kStridedBlock / (px < 4 ? px : 4);
+  bool stream = ov.G < 0 || (ov.G == 0 && ty_need > ty_max) || ty_need > kStridedBlock;
+  if (!stream) {
+    TY = (int)ty_need;
+    if (ov.G > 0) {
+      if (ov.G > 64 || (ov.G & (ov.G - 1))) return -5;
+      TX = ov.G;
+    } else {
+      int cap = 64 / TY;                 // one wavefront per group ...
+      if (cap < 8) cap = 8;              // ... unless rows would shrink below 128 bytes
+      if (cap * TY > kStridedBlock) cap = kStridedBlock / TY;
+      TX = px < cap ? px : cap;
+    }
+    if ((int64_t)TX * TY > kStridedBlock || TX < 1) {
+      if (ov.G > 0 || ov.V > 0) return -5;
+      stream = true;
+    }
+  } else if (ov.G > 0 || ov.V > 0) {
+    return -5;
+  }
+  if (stream) {
+    // one group per workgroup; few lanes along inner, fewer still while the
+    // problem has less than two workgroups per compute unit
+    TX = px < 8 ? px : 8;
+    while (TX > 2 && outer * ((packs + TX - 1) / TX) < 2 * (int64_t)num_cus) TX >>= 1;
+    TY = kStridedBlock / TX;
+    V = 0;
+  }
+  p.resident = !stream;
+  p.tx_log2 = log2_of_pow2(TX);
+  p.ty_log2 = log2_of_pow2(TY);
+  p.V = V;
+  const int64_t xtiles = (packs + TX - 1) / TX;
+  const int64_t ntiles = outer * xtiles;
+  const int groups = kStridedBlock / (TX * TY);
+  const int64_t nblocks = (ntiles + groups - 1) / groups;
+  const int bpc = ov.bpc > 0 ? ov.bpc : (1 << 20);
+  int64_t grid = (int64_t)num_cus * bpc;
+  if (grid > nblocks) grid = nblocks;
+  if (grid > 0x7fffffff) grid = 0x7fffffff;
+  if (grid < 1) grid = 1;
+  p.grid = grid;
+  *out = p;
+  return 0;
+}
+
 }  // namespace rownorm

@@ -1,0 +1,342 @@
+// softmax / log_softmax over a dimension that is NOT innermost, on a dense
+// tensor viewed as [outer, D, inner] (inner > 1 contiguous elements).
+//
+// Every one of the `inner` columns of an [D, inner] slab is its own softmax
+// problem whose D elements lie `inner` apart in memory.  A group of TX * TY
+// threads takes a tile of TX consecutive 16-byte packs of the inner dimension
+// and all D rows: thread (ty, tx) holds the packs of rows ty, ty + TY, ... of
+// pack column tx in registers (V packs), so each lane keeps E independent
+// running maxima and sums, one per element of its pack.  The TX lanes of a row
+// read one contiguous TX * 16 byte segment.  The reduction over D runs across
+// the TY threads that share tx: butterfly shuffles inside a wavefront and, only
+// when a group is wider than a wavefront, one LDS exchange among its
+// wavefronts.  A workgroup holds BLOCK / (TX * TY) such groups, each on its own
+// tile.  X is read once and Y written once.
+//
+// Stands in for SpatialSoftmaxForwardKernelFunctor (src/ATen/native/xpu/sycl/
+// SoftMaxKernels.cpp:725-950) and SpatialSoftmaxBackwardKernelFunctor
+// (:1387-1564), which walk the D rows three times (max, sum, output) from
+// global memory; the dispatch they sit behind is :1721-1736.  D too large for
+// the registers takes the multi-pass kernels at the end of this file, which do
+// the same walk.
+#pragma once
+#include "device/pack.hpp"
+#include "device/reduce.hpp"
+#include "launch.hpp"
+#include "softmax_kernels.hpp"
+
+namespace rownorm {
+
+// LDS floats for column_allreduce in a BLOCK-thread workgroup of E-element packs.
+template <int BLOCK, int E>
+struct column_lds_floats {
+  static constexpr int value = 2 * (BLOCK / 64) * 64 * E;
+};
+
+// Thread layout of one workgroup: threadIdx.x = (group * TY + ty) * TX + tx.
+struct StridedLayout {
+  int tx_log2, ty_log2;
+};
+
+// All-reduce of the E values of every lane over the TY threads of its group
+// that share tx (TX, TY powers of two, TX <= 64, TX * TY <= BLOCK).  Fixed
+// order; every thread of the workgroup must call it (it holds a barrier when
+// a group spans several wavefronts).
+template <int BLOCK, int E, class Op>
+__device__ __forceinline__ void column_allreduce(float (&v)[E], StridedLayout lay, float* lds,
+                                                 int& phase) {
+  const int TX = 1 << lay.tx_log2;
+  const int GT = TX << lay.ty_log2;  // threads per group
+  const int span = GT < 64 ? GT : 64;
+  for (int off = TX; off < span; off <<= 1) {
+#pragma unroll
+    for (int i = 0; i < E; ++i) v[i] = Op::apply(v[i], __shfl_xor(v[i], off, 64));
+  }
+  constexpr int NW = BLOCK / 64;
+  if (GT > 64) {  // uniform over the workgroup
+    const int lane = threadIdx.x & 63;
+    const int wave = threadIdx.x >> 6;
+    const int wpg = GT >> 6;  // wavefronts per group
+    float* buf = lds + phase * (NW * 64 * E);
+    if (lane < TX) {
+#pragma unroll
+      for (int i = 0; i < E; ++i) buf[(wave * 64 + lane) * E + i] = v[i];
+    }
+    __syncthreads();
+    const int tx = lane & (TX - 1);
+    const int w0 = wave & ~(wpg - 1);
+#pragma unroll
+    for (int i = 0; i < E; ++i) {
+      float acc = buf[(w0 * 64 + tx) * E + i];
+      for (int w = 1; w < wpg; ++w) acc = Op::apply(acc, buf[((w0 + w) * 64 + tx) * E + i]);
+      v[i] = acc;
+    }
+    phase ^= 1;
+  }
+}
+
+// The tile a thread works on in one iteration of its workgroup.
+struct StridedTile {
+  int64_t slab;  // element offset of the [D, inner] slab
+  int e0;        // first inner element of this lane's pack (== inner when out of range)
+  int ty, TY;
+  bool valid;    // false: the group has run out of tiles; nothing is loaded or stored
+};
+
+template <int BLOCK, int E>
+__device__ __forceinline__ StridedTile strided_tile(int64_t t0, int64_t ntiles, int64_t xtiles,
+                                                    int D, int inner, StridedLayout lay) {
+  const int TX = 1 << lay.tx_log2;
+  const int tx = threadIdx.x & (TX - 1);
+  const int rest = threadIdx.x >> lay.tx_log2;
+  StridedTile r;
+  r.TY = 1 << lay.ty_log2;
+  r.ty = rest & (r.TY - 1);
+  const int64_t t = t0 + (rest >> lay.ty_log2);
+  r.valid = t < ntiles;
+  const int64_t tc = r.valid ? t : 0;
+  const int64_t o = tc / xtiles;
+  const int64_t xt = tc - o * xtiles;
+  r.slab = o * (int64_t)D * (int64_t)inner;
+  const int64_t e = (xt * TX + tx) * (int64_t)E;
+  r.e0 = e < inner ? (int)e : inner;
+  return r;
+}
+
+// Tiles a workgroup takes per iteration, and the tile count of the problem.
+template <int BLOCK>
+__device__ __forceinline__ int groups_per_block(StridedLayout lay) {
+  return BLOCK >> (lay.tx_log2 + lay.ty_log2);
+}
+
+template <class TI, class TO, int V, int BLOCK, bool FAST>
+__global__ void __launch_bounds__(BLOCK)
+softmax_strided_fwd_kernel(const TI* __restrict__ x, TO* __restrict__ y, int64_t outer, int D,
+                           int inner, StridedLayout lay, int flags) {
+  constexpr int E = elems_per_pack<TI>::value;
+  constexpr bool PRECISE = sizeof(TO) == 4;
+  __shared__ float red[column_lds_floats<BLOCK, E>::value];
+  int phase = 0;
+  const bool is_log = (flags & kSoftmaxLog) != 0;
+  const bool is_safe = (flags & kSoftmaxSafe) != 0;
+  const int64_t xtiles = (((inner + E - 1) / E) + (1 << lay.tx_log2) - 1) >> lay.tx_log2;
+  const int64_t ntiles = outer * xtiles;
+  const int NG = groups_per_block<BLOCK>(lay);
+  for (int64_t t0 = (int64_t)blockIdx.x * NG; t0 < ntiles; t0 += (int64_t)gridDim.x * NG) {
+    const StridedTile tile = strided_tile<BLOCK, E>(t0, ntiles, xtiles, D, inner, lay);
+    const int ty = tile.ty, TY = tile.TY;
+    float xf[V][E];
+#pragma unroll
+    for (int k = 0; k < V; ++k) {
+      const int d = ty + k * TY;
+      const bool ok = tile.valid && d < D;
+      const TI* row = x + tile.slab + (int64_t)(ok ? d : 0) * inner;
+      const Pack<TI, E> p = row_load<TI, E, true, FAST>(row, tile.e0, inner, ok, -INFINITY);
+#pragma unroll
+      for (int i = 0; i < E; ++i) xf[k][i] = p.get(i);
+    }
+    float mx[E], sum[E];
+#pragma unroll
+    for (int i = 0; i < E; ++i) {
+      mx[i] = -INFINITY;
+#pragma unroll
+      for (int k = 0; k < V; ++k) mx[i] = fmaxf(mx[i], xf[k][i]);
+    }
+    column_allreduce<BLOCK, E, MaxOp>(mx, lay, red, phase);
+#pragma unroll
+    for (int i = 0; i < E; ++i) {
+      sum[i] = 0.0f;
+#pragma unroll
+      for (int k = 0; k < V; ++k) {
+        if (is_log) {
+          xf[k][i] -= mx[i];
+          sum[i] += row_exp<PRECISE>(xf[k][i]);
+        } else {
+          xf[k][i] = row_exp<PRECISE>(xf[k][i] - mx[i]);
+          sum[i] += xf[k][i];
+        }
+      }
+    }
+    column_allreduce<BLOCK, E, SumOp>(sum, lay, red, phase);
+    float kf[E];
+    bool zero[E];
+#pragma unroll
+    for (int i = 0; i < E; ++i) {
+      kf[i] = is_log ? logf(sum[i]) : 1.0f / sum[i];
+      zero[i] = is_safe && mx[i] == -INFINITY;
+    }
+#pragma unroll
+    for (int k = 0; k < V; ++k) {
+      const int d = ty + k * TY;
+      const bool ok = tile.valid && d < D;
+      Pack<TO, E> o;
+#pragma unroll
+      for (int i = 0; i < E; ++i) {
+        const float v = is_log ? xf[k][i] - kf[i] : xf[k][i] * kf[i];
+        o.set(i, zero[i] ? 0.0f : v);
+      }
+      TO* row = y + tile.slab + (int64_t)(ok ? d : 0) * inner;
+      row_store<TO, E, true, FAST>(row, tile.e0, inner, ok, o);
+    }
+  }
+}
+
+// TG: dtype of grad and of the saved output y; TO: dtype of the input gradient.
+template <class TG, class TO, int V, int BLOCK, bool FAST>
+__global__ void __launch_bounds__(BLOCK)
+softmax_strided_bwd_kernel(const TG* __restrict__ grad, const TG* __restrict__ y,
+                           TO* __restrict__ gi, int64_t outer, int D, int inner, StridedLayout lay,
+                           int flags) {
+  constexpr int E = elems_per_pack<TG>::value;
+  constexpr bool PRECISE = sizeof(TO) == 4 && sizeof(TG) == 4;
+  __shared__ float red[column_lds_floats<BLOCK, E>::value];
+  int phase = 0;
+  const bool is_log = (flags & kSoftmaxLog) != 0;
+  const int64_t xtiles = (((inner + E - 1) / E) + (1 << lay.tx_log2) - 1) >> lay.tx_log2;
+  const int64_t ntiles = outer * xtiles;
+  const int NG = groups_per_block<BLOCK>(lay);
+  for (int64_t t0 = (int64_t)blockIdx.x * NG; t0 < ntiles; t0 += (int64_t)gridDim.x * NG) {
+    const StridedTile tile = strided_tile<BLOCK, E>(t0, ntiles, xtiles, D, inner, lay);
+    const int ty = tile.ty, TY = tile.TY;
+    Pack<TG, E> pg[V], py[V];
+#pragma unroll
+    for (int k = 0; k < V; ++k) {
+      const int d = ty + k * TY;
+      const bool ok = tile.valid && d < D;
+      const int64_t off = tile.slab + (int64_t)(ok ? d : 0) * inner;
+      pg[k] = row_load<TG, E, true, FAST>(grad + off, tile.e0, inner, ok, 0.0f);
+      py[k] = row_load<TG, E, true, FAST>(y + off, tile.e0, inner, ok, 0.0f);
+    }
+    float sum[E];
+#pragma unroll
+    for (int i = 0; i < E; ++i) {
+      sum[i] = 0.0f;
+#pragma unroll
+      for (int k = 0; k < V; ++k)
+        sum[i] = is_log ? sum[i] + pg[k].get(i) : fmaf(py[k].get(i), pg[k].get(i), sum[i]);
+    }
+    column_allreduce<BLOCK, E, SumOp>(sum, lay, red, phase);
+#pragma unroll
+    for (int k = 0; k < V; ++k) {
+      const int d = ty + k * TY;
+      const bool ok = tile.valid && d < D;
+      Pack<TO, E> o;
+#pragma unroll
+      for (int i = 0; i < E; ++i) {
+        const float g = pg[k].get(i), yv = py[k].get(i);
+        o.set(i, is_log ? g - row_exp<PRECISE>(yv) * sum[i] : yv * (g - sum[i]));
+      }
+      TO* row = gi + tile.slab + (int64_t)(ok ? d : 0) * inner;
+      row_store<TO, E, true, FAST>(row, tile.e0, inner, ok, o);
+    }
+  }
+}
+
+// D beyond the register budget: same tiling, the D rows are walked three times
+// (forward) or twice (backward) from memory.
+template <class TI, class TO, int BLOCK>
+__global__ void __launch_bounds__(BLOCK)
+softmax_strided_fwd_stream_kernel(const TI* __restrict__ x, TO* __restrict__ y, int64_t outer,
+                                  int D, int inner, StridedLayout lay, int flags) {
+  constexpr int E = elems_per_pack<TI>::value;
+  constexpr bool PRECISE = sizeof(TO) == 4;
+  __shared__ float red[column_lds_floats<BLOCK, E>::value];
+  int phase = 0;
+  const bool is_log = (flags & kSoftmaxLog) != 0;
+  const bool is_safe = (flags & kSoftmaxSafe) != 0;
+  const int64_t xtiles = (((inner + E - 1) / E) + (1 << lay.tx_log2) - 1) >> lay.tx_log2;
+  const int64_t ntiles = outer * xtiles;
+  const int NG = groups_per_block<BLOCK>(lay);
+  for (int64_t t0 = (int64_t)blockIdx.x * NG; t0 < ntiles; t0 += (int64_t)gridDim.x * NG) {
+    const StridedTile tile = strided_tile<BLOCK, E>(t0, ntiles, xtiles, D, inner, lay);
+    const int ty = tile.ty, TY = tile.TY;
+    const TI* xs = x + tile.slab;
+    TO* ys = y + tile.slab;
+    float mx[E], sum[E];
+#pragma unroll
+    for (int i = 0; i < E; ++i) mx[i] = -INFINITY;
+    for (int d = ty; d < D; d += TY) {
+      const Pack<TI, E> p =
+          load_row_pack<TI, E, false>(xs + (int64_t)d * inner, tile.e0, inner, tile.valid, -INFINITY);
+#pragma unroll
+      for (int i = 0; i < E; ++i) mx[i] = fmaxf(mx[i], p.get(i));
+    }
+    column_allreduce<BLOCK, E, MaxOp>(mx, lay, red, phase);
+#pragma unroll
+    for (int i = 0; i < E; ++i) sum[i] = 0.0f;
+    for (int d = ty; d < D; d += TY) {
+      const Pack<TI, E> p =
+          load_row_pack<TI, E, false>(xs + (int64_t)d * inner, tile.e0, inner, tile.valid, -INFINITY);
+#pragma unroll
+      for (int i = 0; i < E; ++i) sum[i] += row_exp<PRECISE>(p.get(i) - mx[i]);
+    }
+    column_allreduce<BLOCK, E, SumOp>(sum, lay, red, phase);
+    float kf[E];
+#pragma unroll
+    for (int i = 0; i < E; ++i) kf[i] = is_log ? logf(sum[i]) : 1.0f / sum[i];
+    for (int d = ty; d < D; d += TY) {
+      const Pack<TI, E> p =
+          load_row_pack<TI, E, true>(xs + (int64_t)d * inner, tile.e0, inner, tile.valid, -INFINITY);
+      Pack<TO, E> o;
+#pragma unroll
+      for (int i = 0; i < E; ++i) {
+        const float dlt = p.get(i) - mx[i];
+        const float v = is_log ? dlt - kf[i] : row_exp<PRECISE>(dlt) * kf[i];
+        o.set(i, (is_safe && mx[i] == -INFINITY) ? 0.0f : v);
+      }
+      store_row_pack<TO, E, true>(ys + (int64_t)d * inner, tile.e0, inner, tile.valid, o);
+    }
+  }
+}
+
+template <class TG, class TO, int BLOCK>
+__global__ void __launch_bounds__(BLOCK)
+softmax_strided_bwd_stream_kernel(const TG* __restrict__ grad, const TG* __restrict__ y,
+                                  TO* __restrict__ gi, int64_t outer, int D, int inner,
+                                  StridedLayout lay, int flags) {
+  constexpr int E = elems_per_pack<TG>::value;
+  constexpr bool PRECISE = sizeof(TO) == 4 && sizeof(TG) == 4;
+  __shared__ float red[column_lds_floats<BLOCK, E>::value];
+  int phase = 0;
+  const bool is_log = (flags & kSoftmaxLog) != 0;
+  const int64_t xtiles = (((inner + E - 1) / E) + (1 << lay.tx_log2) - 1) >> lay.tx_log2;
+  const int64_t ntiles = outer * xtiles;
+  const int NG = groups_per_block<BLOCK>(lay);
+  for (int64_t t0 = (int64_t)blockIdx.x * NG; t0 < ntiles; t0 += (int64_t)gridDim.x * NG) {
+    const StridedTile tile = strided_tile<BLOCK, E>(t0, ntiles, xtiles, D, inner, lay);
+    const int ty = tile.ty, TY = tile.TY;
+    const TG* gs = grad + tile.slab;
+    const TG* ys = y + tile.slab;
+    TO* os = gi + tile.slab;
+    float sum[E];
+#pragma unroll
+    for (int i = 0; i < E; ++i) sum[i] = 0.0f;
+    for (int d = ty; d < D; d += TY) {
+      const int64_t off = (int64_t)d * inner;
+      const Pack<TG, E> pg = load_row_pack<TG, E, false>(gs + off, tile.e0, inner, tile.valid, 0.0f);
+      if (is_log) {
+#pragma unroll
+        for (int i = 0; i < E; ++i) sum[i] += pg.get(i);
+      } else {
+        const Pack<TG, E> py = load_row_pack<TG, E, false>(ys + off, tile.e0, inner, tile.valid, 0.0f);
+#pragma unroll
+        for (int i = 0; i < E; ++i) sum[i] = fmaf(py.get(i), pg.get(i), sum[i]);
+      }
+    }
+    column_allreduce<BLOCK, E, SumOp>(sum, lay, red, phase);
+    for (int d = ty; d < D; d += TY) {
+      const int64_t off = (int64_t)d * inner;
+      const Pack<TG, E> pg = load_row_pack<TG, E, true>(gs + off, tile.e0, inner, tile.valid, 0.0f);
+      const Pack<TG, E> py = load_row_pack<TG, E, true>(ys + off, tile.e0, inner, tile.valid, 0.0f);
+      Pack<TO, E> o;
+#pragma unroll
+      for (int i = 0; i < E; ++i) {
+        const float g = pg.get(i), yv = py.get(i);
+        o.set(i, is_log ? g - row_exp<PRECISE>(yv) * sum[i] : yv * (g - sum[i]));
+      }
+      store_row_pack<TO, E, true>(os + off, tile.e0, inner, tile.valid, o);
+    }
+  }
+}
+
+}  // namespace rownorm
