@@ -58,7 +58,9 @@ typedef enum {
   ROWNORM_OP_SOFTMAX_BWD = 5,
   ROWNORM_OP_SOFTMAX_STRIDED_FWD = 6, /* mi355x_softmax_strided_fwd (override / strided_plan only) */
   ROWNORM_OP_SOFTMAX_STRIDED_BWD = 7,
-  ROWNORM_OP_COUNT = 8
+  ROWNORM_OP_GROUP_NORM_FWD = 8,      /* mi355x_group_norm_fwd (override / group_norm_plan only) */
+  ROWNORM_OP_GROUP_NORM_BWD = 9,
+  ROWNORM_OP_COUNT = 10
 } rownorm_op;
 
 /* `mode` of the strided softmax entry points. */
@@ -179,6 +181,44 @@ int mi355x_masked_softmax_bwd(const void* grad, const void* y, const void* mask,
                               int64_t rows, int64_t N, int64_t mask_rows, int64_t mask_row_div,
                               int64_t mask_row_stride, int64_t mask_row_mod, rownorm_dtype dtype,
                               void* stream);
+
+/* native_group_norm on a dense NCHW-contiguous [N, C, HxW] input with `groups`
+ * groups of C / groups channels.  Replaces group_norm_kernel
+ * (src/ATen/native/xpu/sycl/GroupNormKernels.h:17-28, GroupNormKernels.cpp:
+ * 364-530).  gamma/beta are [C] of w_dtype and may be NULL (1 / 0).  mean and
+ * rstd are [N * groups] of w_dtype -- x_dtype, or ROWNORM_F32 beside fp32
+ * weights -- as native_group_norm returns them; either may be NULL.  Pass
+ * w_dtype = x_dtype when there are no weights.  C must be a multiple of
+ * groups; N * groups < 2^31 and (C / groups) * HxW <= 2^30. */
+int mi355x_group_norm_fwd(const void* x, const void* gamma, const void* beta, void* y, void* mean,
+                          void* rstd, int64_t N, int64_t C, int64_t HxW, int64_t groups, float eps,
+                          rownorm_dtype x_dtype, rownorm_dtype w_dtype, void* stream);
+
+/* Bytes of device scratch mi355x_group_norm_bwd needs (0 when neither dgamma
+ * nor dbeta is wanted): two float32 [N, C] arrays of per-sample channel sums.
+ * The reference allocates the same two (ds, db) with at::empty
+ * (GroupNormKernels.cpp:1398-1399). */
+size_t mi355x_group_norm_bwd_workspace_bytes(int64_t N, int64_t C, int64_t HxW, int64_t groups,
+                                             rownorm_dtype x_dtype, rownorm_dtype w_dtype,
+                                             int want_dgamma, int want_dbeta);
+
+/* native_group_norm_backward.  Replaces group_norm_backward_kernel
+ * (GroupNormKernels.h:30-42, GroupNormKernels.cpp:1353-1589).  mean/rstd are
+ * the forward's [N * groups] statistics in w_dtype.  dx, dgamma, dbeta may each
+ * be NULL (not computed); dgamma/dbeta are [C] of w_dtype, summed in float32 in
+ * a fixed order. */
+int mi355x_group_norm_bwd(const void* dy, const void* x, const void* mean, const void* rstd,
+                          const void* gamma, void* dx, void* dgamma, void* dbeta, void* workspace,
+                          size_t workspace_bytes, int64_t N, int64_t C, int64_t HxW,
+                          int64_t groups, rownorm_dtype x_dtype, rownorm_dtype w_dtype,
+                          void* stream);
+
+/* Launch layout of a GroupNorm call (no launch): one row is one (n, group)
+ * slab of (C / groups) * HxW elements; `reserved` is 1 when HxW is a whole
+ * number of 16-byte packs (per-pack weight lookup, channel sums fused into the
+ * backward); partial_rows is N for the backward. */
+int mi355x_group_norm_plan(int backward, int64_t N, int64_t C, int64_t HxW, int64_t groups,
+                           rownorm_dtype x_dtype, rownorm_plan* out);
 
 /* _softmax / _log_softmax / _safe_softmax over a dimension that is not
  * innermost: the dense tensor is viewed as [outer, dim_size, inner] and each of

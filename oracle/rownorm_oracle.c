@@ -6,6 +6,7 @@
  *   src/ATen/native/xpu/sycl/LayerNormKernels.cpp
  *   src/ATen/native/xpu/sycl/Norm.h
  *   src/ATen/native/xpu/sycl/SoftMaxKernels.cpp
+ *   src/ATen/native/xpu/sycl/GroupNormKernels.cpp
  *   src/ATen/native/xpu/sycl/SharedReduceOps.h
  * It is the checker the GPU kernels are compared against.  Only the test
  * suite, the smoke check and the bench's CPU-baseline leg may load it; the
@@ -25,7 +26,9 @@
  * (4) invariants (sum softmax = 1, sum softmax-backward = 0, dbeta of a
  * sum() loss = row count, constant row -> beta), (5) for the masked and
  * safe softmax variants, the plain functions applied to the unmasked
- * elements alone.  No function is "parity unpinned".
+ * elements alone, (6) for GroupNorm, the LayerNorm functions applied to each
+ * (sample, group) slab with the per-channel weights expanded per element.
+ * No function is "parity unpinned".
  *
  * All arrays are dense row-major float32; low-precision inputs are passed
  * already widened to float32 (exactly representable), outputs are returned
@@ -34,6 +37,7 @@
 #include <math.h>
 #include <stddef.h>
 #include <stdint.h>
+#include <stdlib.h>
 
 /* ------------------------------------------------------------------ */
 /* Welford accumulator: SharedReduceOps.h:31-102 (WelfordData/WelfordOps) */
@@ -322,4 +326,96 @@ void oracle_masked_softmax_bwd(const float* g, const float* y,
     for (int64_t j = 0; j < N; ++j)
       o[j] = mr[j] ? 0.0f : (float)((double)yr[j] * ((double)gr[j] - s));
   }
+}
+
+/* native_group_norm on NCHW-contiguous [N, C, HxW] with G groups of D = C/G
+ * channels.  GroupNormKernels.cpp:72-133 (row moments over the D*HxW elements
+ * of a group, biased variance, rstd = 1/sqrt(var + eps)) and :220-260, :351-357
+ * (y = x*a + b with a = rstd*gamma[c], b = beta[c] - a*mean).  mean/rstd are
+ * [N, G]; gamma/beta may be NULL. */
+void oracle_group_norm_fwd(const float* x, const float* gamma,
+                           const float* beta, float* y, float* mean,
+                           float* rstd, int64_t N, int64_t C, int64_t HxW,
+                           int64_t G, double eps) {
+  const int64_t D = G ? C / G : 0;
+  const int64_t L = D * HxW;
+  for (int64_t r = 0; r < N * G; ++r) {
+    const float* xr = x + r * L;
+    double mu, var;
+    oracle_welford_moments(xr, L, &mu, &var);
+    const double rs = 1.0 / sqrt(var + eps);
+    if (mean) mean[r] = (float)mu;
+    if (rstd) rstd[r] = (float)rs;
+    const int64_t g = r % G;
+    for (int64_t p = 0; p < L; ++p) {
+      const int64_t c = g * D + p / HxW;
+      const double a = rs * (gamma ? (double)gamma[c] : 1.0);
+      const double b = (beta ? (double)beta[c] : 0.0) - a * mu;
+      y[r * L + p] = (float)((double)xr[p] * a + b);
+    }
+  }
+}
+
+/* native_group_norm_backward, in the reference's own form:
+ * ds[n,c] = sum_hw dy*x, db[n,c] = sum_hw dy (GroupNormKernels.cpp:955-975);
+ * per (n,g): ds_sum = sum_c ds*gamma, db_sum = sum_c db*gamma,
+ * c2 = (db_sum*mean - ds_sum)*rstd^3/(D*HxW), c3 = -c2*mean - db_sum*rstd/(D*HxW),
+ * dx = rstd*gamma[c]*dy + c2*x + c3 (:1133-1160, :1081-1086);
+ * dgamma[c] = sum_n (ds - db*mean)*rstd, dbeta[c] = sum_n db (:1195-1215).
+ * mean/rstd are the saved [N, G] statistics.  Any output may be NULL. */
+void oracle_group_norm_bwd(const float* dy, const float* x, const float* mean,
+                           const float* rstd, const float* gamma, float* dx,
+                           float* dgamma, float* dbeta, int64_t N, int64_t C,
+                           int64_t HxW, int64_t G) {
+  const int64_t D = G ? C / G : 0;
+  const int64_t L = D * HxW;
+  for (int64_t c = 0; c < C; ++c) {
+    if (dgamma) dgamma[c] = 0;
+    if (dbeta) dbeta[c] = 0;
+  }
+  if (N == 0 || L == 0) return;
+  double* dgs = (double*)calloc((size_t)C, sizeof(double));
+  double* dbs = (double*)calloc((size_t)C, sizeof(double));
+  double* ds = (double*)malloc((size_t)(D ? D : 1) * sizeof(double));
+  double* db = (double*)malloc((size_t)(D ? D : 1) * sizeof(double));
+  for (int64_t r = 0; r < N * G; ++r) {
+    const int64_t g = r % G;
+    const double mu = mean[r], rs = rstd[r];
+    double ds_sum = 0, db_sum = 0;
+    for (int64_t d = 0; d < D; ++d) {
+      double a = 0, b = 0;
+      for (int64_t h = 0; h < HxW; ++h) {
+        const int64_t i = r * L + d * HxW + h;
+        a += (double)dy[i] * (double)x[i];
+        b += (double)dy[i];
+      }
+      ds[d] = a;
+      db[d] = b;
+      const double ga = gamma ? (double)gamma[g * D + d] : 1.0;
+      ds_sum += a * ga;
+      db_sum += b * ga;
+      dgs[g * D + d] += (a - b * mu) * rs;
+      dbs[g * D + d] += b;
+    }
+    if (dx) {
+      const double s = 1.0 / (double)L;
+      const double c2 = (db_sum * mu - ds_sum) * rs * rs * rs * s;
+      const double c3 = -c2 * mu - db_sum * rs * s;
+      for (int64_t d = 0; d < D; ++d) {
+        const double c1 = rs * (gamma ? (double)gamma[g * D + d] : 1.0);
+        for (int64_t h = 0; h < HxW; ++h) {
+          const int64_t i = r * L + d * HxW + h;
+          dx[i] = (float)(c1 * (double)dy[i] + c2 * (double)x[i] + c3);
+        }
+      }
+    }
+  }
+  for (int64_t c = 0; c < C; ++c) {
+    if (dgamma) dgamma[c] = (float)dgs[c];
+    if (dbeta) dbeta[c] = (float)dbs[c];
+  }
+  free(dgs);
+  free(dbs);
+  free(ds);
+  free(db);
 }

@@ -46,6 +46,12 @@ def lib():
         L.oracle_rms_norm_bwd.argtypes = [_f32p, _f32p, _f32p, _f32p, _f32p, _f32p, _f64p, _i64, _i64]
         L.oracle_softmax_fwd.argtypes = [_f32p, _f32p, _i64, _i64, ctypes.c_int]
         L.oracle_softmax_bwd.argtypes = [_f32p, _f32p, _f32p, _i64, _i64, ctypes.c_int]
+        L.oracle_group_norm_fwd.argtypes = [_f32p, _f32p, _f32p, _f32p, _f32p, _f32p, _i64, _i64,
+                                            _i64, _i64, ctypes.c_double]
+        L.oracle_group_norm_bwd.argtypes = [_f32p, _f32p, _f32p, _f32p, _f32p, _f32p, _f32p, _f32p,
+                                            _i64, _i64, _i64, _i64]
+        L.oracle_group_norm_fwd.restype = None
+        L.oracle_group_norm_bwd.restype = None
         _u8p = ctypes.POINTER(ctypes.c_uint8)
         L.oracle_safe_softmax_fwd.argtypes = [_f32p, _f32p, _i64, _i64]
         L.oracle_masked_softmax_fwd.argtypes = [_f32p, _u8p, _f32p, _i64, _i64]
@@ -206,3 +212,36 @@ def masked_softmax_bwd(grad, y, mask):
         m, mp = _mask_bytes(mask, y.shape)
         lib().oracle_masked_softmax_bwd(_p(grad), _p(y), mp, _p(gi), y.size // N, N)
     return gi
+
+
+def _nchw(x):
+    N, C = x.shape[0], x.shape[1]
+    HxW = int(np.prod(x.shape[2:], dtype=np.int64)) if x.ndim > 2 else 1
+    return N, C, HxW
+
+
+def group_norm_fwd(x, groups, gamma=None, beta=None, eps=1e-5):
+    """native_group_norm on [N, C, *] -> (y, mean[N, groups], rstd[N, groups])."""
+    x = _c(x)
+    N, C, HxW = _nchw(x)
+    gamma, beta = _c(gamma), _c(beta)
+    y = np.empty_like(x)
+    mean = np.zeros((N, groups), np.float32)
+    rstd = np.zeros((N, groups), np.float32)
+    if x.size:
+        lib().oracle_group_norm_fwd(_p(x), _p(gamma), _p(beta), _p(y), _p(mean), _p(rstd), N, C, HxW,
+                                    groups, float(eps))
+    return y, mean, rstd
+
+
+def group_norm_bwd(dy, x, groups, mean, rstd, gamma=None, mask=(True, True, True)):
+    """native_group_norm_backward -> (dx, dgamma, dbeta), None where the mask is False."""
+    x, dy = _c(x), _c(dy)
+    N, C, HxW = _nchw(x)
+    mean, rstd, gamma = _c(mean).reshape(-1), _c(rstd).reshape(-1), _c(gamma)
+    dx = np.empty_like(x) if mask[0] else None
+    dg = np.zeros(C, np.float32) if mask[1] else None
+    db = np.zeros(C, np.float32) if mask[2] else None
+    lib().oracle_group_norm_bwd(_p(dy), _p(x), _p(mean), _p(rstd), _p(gamma), _p(dx), _p(dg), _p(db),
+                                N, C, HxW, groups)
+    return dx, dg, db

@@ -122,6 +122,46 @@ def main():
     path = os.path.join(HERE, "aten_cpu_golden.npz")
     np.savez_compressed(path, **store)
     print("wrote", path, os.path.getsize(path), "bytes,", len(store), "arrays")
+    group_norm_vectors()
+
+
+# (N, C, spatial shape, groups): channel size a whole number of 16-byte packs, a ragged one,
+# the 2-d input (one element per channel), one group, one channel per group
+GN_SHAPES = [(3, 8, (4, 8), 2), (2, 6, (5,), 3), (5, 12, (), 4), (2, 4, (3, 3), 1), (2, 6, (16,), 6)]
+
+
+def group_norm_vectors():
+    """tests/golden/aten_cpu_group_norm.npz: native_group_norm / native_group_norm_backward of
+    the CPU kernels, unmixed and (16-bit rows, float32 weights) mixed, eps 1e-5."""
+    torch.manual_seed(0)
+    store = {"meta/torch_version": np.frombuffer(torch.__version__.encode(), dtype=np.uint8)}
+    for dname, dt in DTYPES.items():
+        for (N, C, sp, G) in GN_SHAPES:
+            g = torch.Generator().manual_seed(2000 + C)
+            HxW = int(np.prod(sp)) if sp else 1
+            case = "%s_%dx%dx%dg%d" % (dname, N, C, HxW, G)
+            x = (0.5 + torch.randn((N, C) + sp, generator=g)).to(dt)
+            dy = torch.randn((N, C) + sp, generator=g).to(dt)
+            gamma = (1 + 0.1 * torch.randn(C, generator=g)).to(dt)
+            beta = (0.1 * torch.randn(C, generator=g)).to(dt)
+            for k, v in (("x", x), ("dy", dy), ("gamma", gamma), ("beta", beta)):
+                put(store, case + "/" + k, v)
+            variants = [("gn", gamma, beta)]
+            if dt != torch.float32:
+                variants.append(("gnmix", gamma.float(), beta.float()))
+            for pre, gk, bk in variants:
+                y, mean, rstd = torch.ops.aten.native_group_norm(x, gk, bk, N, C, HxW, G, 1e-5)
+                put(store, case + "/%s_y" % pre, y)
+                put(store, case + "/%s_mean" % pre, mean)
+                put(store, case + "/%s_rstd" % pre, rstd)
+                dx, dg, db = torch.ops.aten.native_group_norm_backward(
+                    dy, x, mean, rstd, gk, N, C, HxW, G, [True, True, True])
+                put(store, case + "/%s_dx" % pre, dx)
+                put(store, case + "/%s_dgamma" % pre, dg)
+                put(store, case + "/%s_dbeta" % pre, db)
+    path = os.path.join(HERE, "aten_cpu_group_norm.npz")
+    np.savez_compressed(path, **store)
+    print("wrote", path, os.path.getsize(path), "bytes,", len(store), "arrays")
 
 
 if __name__ == "__main__":

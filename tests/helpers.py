@@ -90,10 +90,10 @@ def causal_scores(B, H, T, seed, dtype=torch.bfloat16):
     return s.to(dtype)
 
 
-def load_golden():
-    """tests/golden/aten_cpu_golden.npz as {case: {name: torch tensor}} with the stored dtypes."""
+def load_golden(name="aten_cpu_golden.npz"):
+    """tests/golden/<name> as {case: {name: torch tensor}} with the stored dtypes."""
     import os
-    path = os.path.join(os.path.dirname(os.path.abspath(__file__)), "golden", "aten_cpu_golden.npz")
+    path = os.path.join(os.path.dirname(os.path.abspath(__file__)), "golden", name)
     z = np.load(path, allow_pickle=False)
     cases = {}
     for key in z.files:

@@ -213,3 +213,39 @@ def test_strided_softmax_validation_and_plans(cabi):
     cabi.set_override(cabi.OP_SOFTMAX_STRIDED_FWD, -1)
     assert cabi.strided_plan(0, 4, 5, 4096, cabi.BF16)["resident"] == 0
     cabi.clear_overrides()
+
+
+def test_group_norm_validation_and_plans(cabi):
+    L = cabi.lib()
+    one, null = ctypes.c_void_p(256), None
+    f = lambda N, C, HxW, G, xd=0, wd=0, x=one: L.mi355x_group_norm_fwd(x, null, null, one, null, null, N, C, HxW,
+                                                                        G, 1e-5, xd, wd, null)
+    assert f(2, 6, 4, 3, xd=cabi.F32, wd=cabi.BF16) == -1        # weights narrower than the rows
+    assert f(2, 6, 4, 4) == -2                                   # C not a multiple of groups
+    assert f(2, 6, 4, 0) == -2 and f(-1, 6, 4, 3) == -2
+    assert f(1 << 30, 8, 4, 4) == -2                             # N * groups beyond 2^31
+    assert f(1, 4, 1 << 30, 2) == -2                             # a group row beyond 2^30 elements
+    assert f(0, 6, 4, 3, x=null) == 0 and f(2, 6, 0, 3, x=null) == 0 and f(2, 0, 4, 3, x=null) == 0
+    assert f(2, 6, 4, 3, x=null) == -3
+    b = L.mi355x_group_norm_bwd
+    assert b(one, one, one, one, null, one, one, one, null, 0, 2, 6, 4, 3, 0, 0, null) == -4   # no workspace
+    assert b(one, one, null, one, null, one, null, null, null, 0, 2, 6, 4, 3, 0, 0, null) == -3  # no mean
+    assert b(one, one, one, one, null, null, null, null, null, 0, 2, 6, 4, 3, 0, 0, null) == 0  # nothing asked
+    assert L.mi355x_group_norm_bwd_workspace_bytes(2, 6, 4, 3, 0, 0, 1, 0) == 2 * 2 * 6 * 4
+    assert L.mi355x_group_norm_bwd_workspace_bytes(2, 6, 4, 3, 0, 0, 0, 0) == 0
+    for dt, E in ((cabi.F32, 4), (cabi.BF16, 8)):
+        for (N, C, HxW, G) in ((2, 4, 1, 2), (256, 32, 16, 4), (4, 64, 1024, 32), (2, 320, 4096, 32),
+                               (3, 6, 5, 3), (1, 4, 1 << 17, 2), (1, 8, 1 << 20, 2)):
+            for bwd in (0, 1):
+                p = cabi.group_norm_plan(bwd, N, C, HxW, G, dt)
+                Lrow = (C // G) * HxW
+                assert p["uniform"] == int(HxW % E == 0)
+                assert p["grid_blocks"] >= 1
+                if p["resident"]:
+                    assert p["lanes_per_row"] * p["packs_per_lane"] * E >= Lrow
+                    assert p["grid_blocks"] == -(-(N * G) // p["rows_per_block"])
+                else:
+                    assert Lrow > 8192
+    # the diffusion-UNet shape keeps its 40960-element rows in registers
+    assert cabi.group_norm_plan(0, 2, 320, 4096, 32, cabi.BF16)["resident"] == 1
+    assert cabi.group_norm_plan(1, 2, 320, 4096, 32, cabi.BF16)["resident"] == 1

@@ -21,6 +21,8 @@ def test_ops_are_registered_with_the_reference_schemas(ops):
         "_log_softmax": "(Tensor self, int dim, bool half_to_float) -> Tensor",
         "_softmax_backward_data": "(Tensor grad_output, Tensor output, int dim, ScalarType input_dtype) -> Tensor",
         "_log_softmax_backward_data": "(Tensor grad_output, Tensor output, int dim, ScalarType input_dtype) -> Tensor",
+        "native_group_norm": "(Tensor input, Tensor? weight, Tensor? bias, int N, int C, int HxW, int group, float eps) -> (Tensor, Tensor, Tensor)",
+        "native_group_norm_backward": "(Tensor grad_out, Tensor input, Tensor mean, Tensor rstd, Tensor? weight, int N, int C, int HxW, int group, bool[3] output_mask) -> (Tensor, Tensor, Tensor)",
         "_safe_softmax": "(Tensor self, int dim, ScalarType? dtype=None) -> Tensor",
         "_masked_softmax": "(Tensor self, Tensor mask, int? dim=None, int? mask_type=None) -> Tensor",
         "_masked_softmax_backward": "(Tensor grad_output, Tensor output, Tensor mask, int? dim=None) -> Tensor",
@@ -62,6 +64,9 @@ def test_cpu_tensors_are_rejected_loudly(ops):
         lambda: ops._softmax_backward_data(x, x, -1, torch.float32),
         lambda: ops._log_softmax_backward_data(x, x, -1, torch.float32),
         lambda: ops._safe_softmax(x, -1),
+        lambda: ops.native_group_norm(x, None, None, 4, 8, 1, 2, 1e-5),
+        lambda: ops.native_group_norm_backward(x, x, m[:, :1].expand(4, 2), r.expand(4, 2), None, 4, 8, 1, 2,
+                                               [True, False, False]),
         lambda: ops._masked_softmax(x, x > 0, -1, 2),
         lambda: ops._masked_softmax_backward(x, x, x > 0, -1),
     ]
@@ -106,3 +111,18 @@ def test_masked_softmax_argument_errors(ops):
         ops._masked_softmax(x, ok[0, 0], -1, 1)  # [T, T] is not a key-padding mask
     with pytest.raises(RuntimeError, match="Mask shape should match input"):
         ops._masked_softmax(x, ok[:, 0, 0], -1, 0)  # [B, T] is not a src mask
+
+
+def test_group_norm_argument_errors_match_aten(ops):
+    x = torch.randn(2, 6, 4)
+    cases = [
+        lambda m: m.native_group_norm(x, None, None, 2, 6, 4, 4, 1e-5),              # C % groups
+        lambda m: m.native_group_norm(x, torch.randn(5), None, 2, 6, 4, 3, 1e-5),     # weight size
+        lambda m: m.native_group_norm(x, None, None, 2, 6, 4, 0, 1e-5),              # no groups
+        lambda m: m.native_group_norm_backward(x.half(), x, torch.zeros(2, 3), torch.ones(2, 3), None, 2, 6, 4,
+                                               3, [True, False, False]),              # dY dtype
+    ]
+    for fn in cases:
+        assert _aten_message(lambda: fn(ops)) == _aten_message(lambda: fn(torch.ops.aten))
+    with pytest.raises(RuntimeError, match="Expected bias to be a vector of size equal to the number of channels"):
+        ops.native_group_norm(x, None, torch.randn(7), 2, 6, 4, 3, 1e-5)

@@ -53,7 +53,7 @@ from . import cabi  # noqa: E402  (ctypes layer; loads the kernel library on fir
 
 def override_aten_ops():
     """Explicit opt-in: route the aten ops of this family to the MI355X kernels for GPU tensors,
-    so ``F.layer_norm`` / ``F.rms_norm`` / ``F.softmax`` / ``F.log_softmax``,
+    so ``F.layer_norm`` / ``F.rms_norm`` / ``F.group_norm`` / ``F.softmax`` / ``F.log_softmax``,
     ``torch._masked_softmax`` / ``torch._safe_softmax`` and their autograd formulas run them.
     PyTorch warns about overriding existing kernels; that is why this is never done at import.  float64 inputs are rejected by the kernels after the override."""
     import torch
@@ -69,6 +69,8 @@ def override_aten_ops():
     lib.impl("_log_softmax", m._log_softmax.default, "CUDA")
     lib.impl("_softmax_backward_data", m._softmax_backward_data.default, "CUDA")
     lib.impl("_log_softmax_backward_data", m._log_softmax_backward_data.default, "CUDA")
+    lib.impl("native_group_norm", m.native_group_norm.default, "CUDA")
+    lib.impl("native_group_norm_backward", m.native_group_norm_backward.default, "CUDA")
     lib.impl("_safe_softmax", m._safe_softmax.default, "CUDA")
     lib.impl("_masked_softmax", m._masked_softmax.default, "CUDA")
     lib.impl("_masked_softmax_backward", m._masked_softmax_backward.default, "CUDA")

@@ -14,6 +14,7 @@ F32, F16, BF16 = 0, 1, 2
 OP_LAYER_NORM_FWD, OP_LAYER_NORM_BWD, OP_RMS_NORM_FWD, OP_RMS_NORM_BWD = 0, 1, 2, 3
 OP_SOFTMAX_FWD, OP_SOFTMAX_BWD = 4, 5
 OP_SOFTMAX_STRIDED_FWD, OP_SOFTMAX_STRIDED_BWD = 6, 7
+OP_GROUP_NORM_FWD, OP_GROUP_NORM_BWD = 8, 9
 SOFTMAX, LOG_SOFTMAX, SAFE_SOFTMAX = 0, 1, 2
 
 EXPORTED_SYMBOLS = (
@@ -22,7 +23,9 @@ EXPORTED_SYMBOLS = (
     "mi355x_rms_norm_bwd_workspace_bytes", "mi355x_rms_norm_bwd", "mi355x_softmax_fwd",
     "mi355x_softmax_bwd", "mi355x_safe_softmax_fwd", "mi355x_masked_softmax_fwd",
     "mi355x_masked_softmax_bwd", "mi355x_softmax_strided_fwd", "mi355x_softmax_strided_bwd",
-    "mi355x_softmax_strided_plan", "mi355x_rownorm_plan", "mi355x_rownorm_set_override",
+    "mi355x_softmax_strided_plan", "mi355x_group_norm_fwd",
+    "mi355x_group_norm_bwd_workspace_bytes", "mi355x_group_norm_bwd", "mi355x_group_norm_plan",
+    "mi355x_rownorm_plan", "mi355x_rownorm_set_override",
 )
 
 
@@ -73,6 +76,16 @@ def lib():
                                                  _vp]
         L.mi355x_softmax_strided_plan.argtypes = [_int, _i64, _i64, _i64, _int,
                                                   ctypes.POINTER(Plan)]
+        L.mi355x_group_norm_fwd.argtypes = [_vp, _vp, _vp, _vp, _vp, _vp, _i64, _i64, _i64, _i64, _f,
+                                            _int, _int, _vp]
+        L.mi355x_group_norm_bwd_workspace_bytes.restype = ctypes.c_size_t
+        L.mi355x_group_norm_bwd_workspace_bytes.argtypes = [_i64, _i64, _i64, _i64, _int, _int,
+                                                            _int, _int]
+        L.mi355x_group_norm_bwd.argtypes = [_vp, _vp, _vp, _vp, _vp, _vp, _vp, _vp, _vp,
+                                            ctypes.c_size_t, _i64, _i64, _i64, _i64, _int, _int,
+                                            _vp]
+        L.mi355x_group_norm_plan.argtypes = [_int, _i64, _i64, _i64, _i64, _int,
+                                             ctypes.POINTER(Plan)]
         L.mi355x_rownorm_plan.argtypes = [_int, _i64, _i64, _int, _int, ctypes.POINTER(Plan)]
         L.mi355x_rownorm_set_override.argtypes = [_int, _int, _int, _int, _int]
         for name in ("mi355x_layer_norm_fwd", "mi355x_rms_norm_fwd", "mi355x_layer_norm_bwd",
@@ -80,6 +93,7 @@ def lib():
                      "mi355x_safe_softmax_fwd", "mi355x_masked_softmax_fwd",
                      "mi355x_masked_softmax_bwd", "mi355x_softmax_strided_fwd",
                      "mi355x_softmax_strided_bwd", "mi355x_softmax_strided_plan",
+                     "mi355x_group_norm_fwd", "mi355x_group_norm_bwd", "mi355x_group_norm_plan",
                      "mi355x_rownorm_plan", "mi355x_rownorm_set_override"):
             getattr(L, name).restype = _int
         _lib = L
@@ -121,8 +135,17 @@ def strided_plan(backward, outer, dim_size, inner, dtype=F32):
     return p.as_dict()
 
 
+def group_norm_plan(backward, N, C, HxW, groups, dtype=F32):
+    p = Plan()
+    _check(lib().mi355x_group_norm_plan(int(backward), N, C, HxW, groups, dtype, ctypes.byref(p)),
+           "group_norm_plan")
+    d = p.as_dict()
+    d["uniform"] = p.reserved
+    return d
+
+
 def clear_overrides():
-    for op in range(8):
+    for op in range(10):
         set_override(op)
 
 
@@ -354,3 +377,52 @@ def softmax_strided_bwd(grad, y, dim, mode=SOFTMAX, gi_dtype=None, gi=None):
                                             dtype_code(grad.dtype), dtype_code(gi.dtype), mode,
                                             _stream()), "softmax_strided_bwd")
     return gi
+
+
+def _nchw(x):
+    N, C = x.shape[0], x.shape[1]
+    HxW = 1
+    for s in x.shape[2:]:
+        HxW *= s
+    return N, C, HxW
+
+
+def group_norm_fwd(x, gamma, beta, groups, eps, y=None, mean=None, rstd=None):
+    """-> (y, mean[N, groups], rstd[N, groups]); x is a dense [N, C, *]; the statistics come in
+    the weight dtype (the input dtype when there are no weights)."""
+    import torch
+    _gpu(x, gamma, beta)
+    N, C, HxW = _nchw(x)
+    sdt = gamma.dtype if gamma is not None else (beta.dtype if beta is not None else x.dtype)
+    y = torch.empty_like(x) if y is None else y
+    mean = torch.empty(N, groups, dtype=sdt, device=x.device) if mean is None else mean
+    rstd = torch.empty(N, groups, dtype=sdt, device=x.device) if rstd is None else rstd
+    _check(lib().mi355x_group_norm_fwd(_ptr(x), _ptr(gamma), _ptr(beta), _ptr(y), _ptr(mean),
+                                       _ptr(rstd), N, C, HxW, groups, eps, dtype_code(x.dtype),
+                                       dtype_code(sdt), _stream()), "group_norm_fwd")
+    return y, mean, rstd
+
+
+def group_norm_bwd(dy, x, mean, rstd, gamma, groups, want=(True, True, True), dx=None,
+                   dgamma=None, dbeta=None, workspace=None):
+    import torch
+    _gpu(dy, x, mean, rstd, gamma)
+    N, C, HxW = _nchw(x)
+    wdt = mean.dtype
+    if want[0] and dx is None:
+        dx = torch.empty_like(x)
+    if want[1] and dgamma is None:
+        dgamma = torch.empty(C, dtype=wdt, device=x.device)
+    if want[2] and dbeta is None:
+        dbeta = torch.empty(C, dtype=wdt, device=x.device)
+    xd, wd = dtype_code(x.dtype), dtype_code(wdt)
+    nbytes = lib().mi355x_group_norm_bwd_workspace_bytes(N, C, HxW, groups, xd, wd,
+                                                         int(dgamma is not None),
+                                                         int(dbeta is not None))
+    if workspace is None and nbytes:
+        workspace = torch.empty(nbytes, dtype=torch.uint8, device=x.device)
+    _check(lib().mi355x_group_norm_bwd(_ptr(dy), _ptr(x), _ptr(mean), _ptr(rstd), _ptr(gamma),
+                                       _ptr(dx), _ptr(dgamma), _ptr(dbeta), _ptr(workspace),
+                                       0 if workspace is None else workspace.numel(), N, C, HxW,
+                                       groups, xd, wd, _stream()), "group_norm_bwd")
+    return dx, dgamma, dbeta

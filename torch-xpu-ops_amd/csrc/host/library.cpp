@@ -8,6 +8,7 @@
 // opt-in done from Python.
 #include <torch/library.h>
 
+#include "group_norm_ops.h"
 #include "norm_ops.h"
 #include "softmax_ops.h"
 
@@ -63,5 +64,15 @@ TORCH_LIBRARY(mi355x, m) {
       "_masked_softmax_backward(Tensor grad_output, Tensor output, Tensor mask, int? dim=None) "
       "-> Tensor",
       &mi355x::_masked_softmax_backward);
+  m.def(
+      "native_group_norm(Tensor input, Tensor? weight, Tensor? bias, int N, int C, int HxW, "
+      "int group, float eps) -> (Tensor, Tensor, Tensor)",
+      &mi355x::native_group_norm);
+  m.def(
+      "native_group_norm_backward(Tensor grad_out, Tensor input, Tensor mean, Tensor rstd, "
+      "Tensor? weight, int N, int C, int HxW, int group, bool[3] output_mask) -> "
+      "(Tensor, Tensor, Tensor)",
+      &mi355x::native_group_norm_backward);
+  m.def("install_group_norm_dispatch_stubs() -> ()", &mi355x::install_group_norm_dispatch_stubs);
   m.def("install_layer_norm_dispatch_stubs() -> ()", &mi355x::install_layer_norm_dispatch_stubs);
 }

@@ -36,6 +36,16 @@ extern template int launch_softmax_bwd<float, float>(const Plan&, const SoftmaxB
 extern template int launch_softmax_bwd<f16, f16>(const Plan&, const SoftmaxBwdArgs&, hipStream_t);
 extern template int launch_softmax_bwd<bf16, bf16>(const Plan&, const SoftmaxBwdArgs&, hipStream_t);
 extern template int launch_softmax_bwd<float, f16>(const Plan&, const SoftmaxBwdArgs&, hipStream_t);
+extern template int launch_group_norm_fwd<float, float>(const Plan&, const GroupNormFwdArgs&, hipStream_t);
+extern template int launch_group_norm_fwd<f16, f16>(const Plan&, const GroupNormFwdArgs&, hipStream_t);
+extern template int launch_group_norm_fwd<f16, float>(const Plan&, const GroupNormFwdArgs&, hipStream_t);
+extern template int launch_group_norm_fwd<bf16, bf16>(const Plan&, const GroupNormFwdArgs&, hipStream_t);
+extern template int launch_group_norm_fwd<bf16, float>(const Plan&, const GroupNormFwdArgs&, hipStream_t);
+extern template int launch_group_norm_bwd<float, float>(const Plan&, const GroupNormBwdArgs&, hipStream_t);
+extern template int launch_group_norm_bwd<f16, f16>(const Plan&, const GroupNormBwdArgs&, hipStream_t);
+extern template int launch_group_norm_bwd<f16, float>(const Plan&, const GroupNormBwdArgs&, hipStream_t);
+extern template int launch_group_norm_bwd<bf16, bf16>(const Plan&, const GroupNormBwdArgs&, hipStream_t);
+extern template int launch_group_norm_bwd<bf16, float>(const Plan&, const GroupNormBwdArgs&, hipStream_t);
 extern template int launch_softmax_strided_fwd<float, float>(const StridedPlan&, const SoftmaxStridedFwdArgs&, hipStream_t);
 extern template int launch_softmax_strided_fwd<f16, f16>(const StridedPlan&, const SoftmaxStridedFwdArgs&, hipStream_t);
 extern template int launch_softmax_strided_fwd<bf16, bf16>(const StridedPlan&, const SoftmaxStridedFwdArgs&, hipStream_t);
@@ -236,6 +246,34 @@ int softmax_bwd(const void* grad, const void* y, const void* mask, void* gi, int
                            : launch_softmax_bwd<float, float>(plan, a, s);
 }
 
+// Shape of a GroupNorm call as the kernels see it; returns 0 or an error code.
+struct GroupDims {
+  int64_t rows = 0;  // N * groups
+  int64_t L = 0;     // (C / groups) * HxW
+  int64_t D = 0;
+};
+
+int group_dims(int64_t N, int64_t C, int64_t HxW, int64_t groups, GroupDims* out) {
+  if (N < 0 || C < 0 || HxW < 0 || groups <= 0) return ROWNORM_ERR_SHAPE;
+  if (C % groups != 0) return ROWNORM_ERR_SHAPE;
+  GroupDims d;
+  d.D = C / groups;
+  if (C >= (int64_t(1) << 31) || HxW > kMaxN || d.D > kMaxN) return ROWNORM_ERR_SHAPE;
+  d.L = d.D * HxW;
+  if (d.L > kMaxN) return ROWNORM_ERR_SHAPE;
+  if (N >= (int64_t(1) << 31) / groups) return ROWNORM_ERR_SHAPE;
+  d.rows = N * groups;
+  *out = d;
+  return 0;
+}
+
+// The general kernels are taken whenever a pack could straddle two channels.
+int group_plan(OpClass oc, int op, const GroupDims& d, int64_t HxW, int esize, Plan* plan) {
+  const int E = 16 / esize;
+  return make_plan(oc, d.rows, d.L, esize, current_num_cus(), g_override[op], false, plan,
+                   HxW % E != 0);
+}
+
 int softmax_mode_flags(int mode, bool forward, int* flags) {
   switch (mode) {
     case ROWNORM_SOFTMAX: *flags = 0; return 0;
@@ -351,6 +389,95 @@ int mi355x_masked_softmax_bwd(const void* grad, const void* y, const void* mask,
   return softmax_bwd(grad, y, mask, gi, rows, N,
                      MaskRows{mask_rows, mask_row_div, mask_row_stride, mask_row_mod}, (int)dtype,
                      (int)dtype, 0, stream);
+}
+
+int mi355x_group_norm_fwd(const void* x, const void* gamma, const void* beta, void* y, void* mean,
+                          void* rstd, int64_t N, int64_t C, int64_t HxW, int64_t groups, float eps,
+                          rownorm_dtype x_dtype, rownorm_dtype w_dtype, void* stream) {
+  const int xd = (int)x_dtype, wd = (int)w_dtype;
+  if (!norm_dtypes_ok(xd, wd)) return ROWNORM_ERR_DTYPE;
+  GroupDims d;
+  if (int e = group_dims(N, C, HxW, groups, &d)) return e;
+  if (d.rows == 0 || d.L == 0) return 0;
+  if (!x || !y) return ROWNORM_ERR_NULL;
+  Plan plan;
+  if (int e = group_plan(OC_GROUP_FWD, ROWNORM_OP_GROUP_NORM_FWD, d, HxW, esize_of(xd), &plan))
+    return e;
+  GroupNormFwdArgs a{x,      gamma,      beta,     y,          mean,        rstd,
+                     d.rows, (int)d.L, (int)HxW, (int)d.D, (int)groups, eps};
+  hipStream_t s = (hipStream_t)stream;
+  if (xd == ROWNORM_F32) return launch_group_norm_fwd<float, float>(plan, a, s);
+  if (xd == ROWNORM_F16)
+    return wd == ROWNORM_F32 ? launch_group_norm_fwd<f16, float>(plan, a, s)
+                             : launch_group_norm_fwd<f16, f16>(plan, a, s);
+  return wd == ROWNORM_F32 ? launch_group_norm_fwd<bf16, float>(plan, a, s)
+                           : launch_group_norm_fwd<bf16, bf16>(plan, a, s);
+}
+
+size_t mi355x_group_norm_bwd_workspace_bytes(int64_t N, int64_t C, int64_t HxW, int64_t groups,
+                                             rownorm_dtype x_dtype, rownorm_dtype w_dtype,
+                                             int want_dgamma, int want_dbeta) {
+  GroupDims d;
+  if (!norm_dtypes_ok((int)x_dtype, (int)w_dtype) || group_dims(N, C, HxW, groups, &d)) return 0;
+  if (d.rows == 0 || d.L == 0 || !(want_dgamma || want_dbeta)) return 0;
+  return (size_t)N * (size_t)C * sizeof(float) * 2;
+}
+
+int mi355x_group_norm_bwd(const void* dy, const void* x, const void* mean, const void* rstd,
+                          const void* gamma, void* dx, void* dgamma, void* dbeta, void* workspace,
+                          size_t workspace_bytes, int64_t N, int64_t C, int64_t HxW,
+                          int64_t groups, rownorm_dtype x_dtype, rownorm_dtype w_dtype,
+                          void* stream) {
+  const int xd = (int)x_dtype, wd = (int)w_dtype;
+  if (!norm_dtypes_ok(xd, wd)) return ROWNORM_ERR_DTYPE;
+  GroupDims d;
+  if (int e = group_dims(N, C, HxW, groups, &d)) return e;
+  if (d.rows == 0 || d.L == 0) return 0;
+  const bool want_cols = dgamma != nullptr || dbeta != nullptr;
+  if (!dx && !want_cols) return 0;
+  if (!dy || !x || !mean || !rstd) return ROWNORM_ERR_NULL;
+  Plan plan;
+  if (int e = group_plan(OC_GROUP_BWD, ROWNORM_OP_GROUP_NORM_BWD, d, HxW, esize_of(xd), &plan))
+    return e;
+  float* part_dg = nullptr;
+  float* part_db = nullptr;
+  if (want_cols) {
+    const size_t one = (size_t)N * (size_t)C * sizeof(float);
+    if (!workspace || workspace_bytes < 2 * one) return ROWNORM_ERR_WORKSPACE;
+    part_dg = (float*)workspace;
+    part_db = (float*)((char*)workspace + one);
+  }
+  GroupNormBwdArgs a{dy,      x,       mean,   rstd,     gamma,    dx,       dgamma,     dbeta,
+                     part_dg, part_db, d.rows, (int)d.L, (int)HxW, (int)d.D, (int)groups};
+  hipStream_t s = (hipStream_t)stream;
+  if (xd == ROWNORM_F32) return launch_group_norm_bwd<float, float>(plan, a, s);
+  if (xd == ROWNORM_F16)
+    return wd == ROWNORM_F32 ? launch_group_norm_bwd<f16, float>(plan, a, s)
+                             : launch_group_norm_bwd<f16, f16>(plan, a, s);
+  return wd == ROWNORM_F32 ? launch_group_norm_bwd<bf16, float>(plan, a, s)
+                           : launch_group_norm_bwd<bf16, bf16>(plan, a, s);
+}
+
+int mi355x_group_norm_plan(int backward, int64_t N, int64_t C, int64_t HxW, int64_t groups,
+                           rownorm_dtype x_dtype, rownorm_plan* out) {
+  if (!out) return ROWNORM_ERR_NULL;
+  if (esize_of((int)x_dtype) == 0) return ROWNORM_ERR_DTYPE;
+  GroupDims d;
+  if (int e = group_dims(N, C, HxW, groups, &d)) return e;
+  Plan plan;
+  if (int e = group_plan(backward ? OC_GROUP_BWD : OC_GROUP_FWD,
+                         backward ? ROWNORM_OP_GROUP_NORM_BWD : ROWNORM_OP_GROUP_NORM_FWD, d, HxW,
+                         esize_of((int)x_dtype), &plan))
+    return e;
+  out->resident = plan.resident ? 1 : 0;
+  out->lanes_per_row = plan.G;
+  out->packs_per_lane = plan.V;
+  out->block_threads = plan.block;
+  out->rows_per_block = plan.rpb;
+  out->reserved = plan.fast ? 1 : 0;
+  out->grid_blocks = plan.grid;
+  out->partial_rows = backward ? N : 0;
+  return 0;
 }
 
 int mi355x_softmax_strided_fwd(const void* x, void* y, int64_t outer, int64_t dim_size,

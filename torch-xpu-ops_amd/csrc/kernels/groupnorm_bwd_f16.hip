@@ -1,0 +1,5 @@
+// GroupNorm backward kernels, fp16 rows, fp16 weights.
+#include "groupnorm_launch.hpp"
+namespace rownorm {
+template int launch_group_norm_bwd<f16, f16>(const Plan&, const GroupNormBwdArgs&, hipStream_t);
+}  // namespace rownorm

@@ -1,0 +1,444 @@
+// GroupNorm forward and backward kernels for gfx950 (wave64), NCHW-contiguous input.
+//
+// X is [N, C, HxW]; with `groups` groups of D = C / groups channels each, the
+// (n, g) slab of L = D * HxW contiguous elements is one row of a dense
+// [N * groups, L] matrix, normalized like a LayerNorm row, and the affine
+// weights are per channel: element p of row (n, g) uses channel g * D + p / HxW.
+// The row layout is that of the LayerNorm kernels (G lanes share a row, V
+// 16-byte packs per lane, BLOCK / G rows per workgroup), so X is read once and
+// Y written once; the backward reads dY and X once, writes dX once and leaves
+// the per-(n, channel) sums of dY * xhat and dY in an fp32 [N, C] workspace that
+// colsum_finalize_kernel adds up over n.
+//
+// UNIFORM: HxW is a whole number of packs, so every pack lies in one channel
+// (one weight lookup per pack, branch-free row access, channel sums fused into
+// the backward through an LDS staging area).  Otherwise the channel is looked
+// up per element, row access is the general one, and the channel sums come
+// from gn_channel_sums_kernel, which reads dY and X a second time.
+//
+// What these stand in for in the reference (src/ATen/native/xpu/sycl/
+// GroupNormKernels.cpp): GNRowwiseMomentsFunctor / ...VectorizedFunctor
+// (:72-218) + ComputeFusedParamsFunctor (:220-260) + the elementwise
+// GroupNormFunctor pass (:351-357, :446-496), three launches that read X
+// twice; and for the backward ComputeInternalGradients[Vectorized]Functor
+// (:943-1072), ComputeBackwardFusedParamsFunctor (:1088-1165), the elementwise
+// dX pass (:1081-1086, :1476-1520) and GammaBetaBackward[Plain]Functor
+// (:1167-1351), which read dY and X twice.  Formulas (same file):
+//   y  = (x - mean) * rstd * gamma[c] + beta[c]
+//   ds[n,c] = sum_hw dy * x,  db[n,c] = sum_hw dy                       (:955-975)
+//   dx = rstd*gamma[c]*dy + c2*x + c3 with
+//        c2 = (sum_c db*gamma * mean - sum_c ds*gamma) * rstd^3 / L,
+//        c3 = -c2 * mean - sum_c db*gamma * rstd / L                    (:1133-1160)
+//   dgamma[c] = sum_n (ds - db * mean) * rstd,  dbeta[c] = sum_n db     (:1195-1215)
+// Here dx is evaluated in the equivalent LayerNorm form
+//   dx = (rstd / L) * (L * g - xhat * s2 - s1),  g = dy * gamma[c],
+//   s1 = sum g, s2 = sum g * xhat, xhat = (x - mean) * rstd,
+// which does not cancel when mean is large against the spread.
+//
+// mean and rstd are stored in the weight dtype WT (the row dtype when the
+// weights share it, fp32 beside fp32 weights), as native_group_norm returns them.
+#pragma once
+#include <type_traits>
+
+#include "device/pack.hpp"
+#include "device/reduce.hpp"
+
+namespace rownorm {
+
+struct GroupShape {
+  int L;        // elements per (n, g) row: D * HxW
+  int HxW;      // elements per channel
+  int D;        // channels per group
+  int groups;   // groups per sample
+};
+
+// Channel (index into gamma/beta) of element p of row `g` (p is clamped into the row).
+__device__ __forceinline__ int gn_channel(const GroupShape& s, int g, int p) {
+  const int pc = p < s.L ? p : s.L - 1;
+  return g * s.D + (int)((unsigned)pc / (unsigned)s.HxW);
+}
+
+template <class WT>
+__device__ __forceinline__ float gn_weight(const WT* w, int ch, float dflt) {
+  return w ? (float)w[ch] : dflt;
+}
+
+// ---------------------------------------------------------------------------
+// Forward, row resident in registers.  Statistics as in the LayerNorm kernel:
+// mean0 = sum(x)/L, centred sums over the registers, mean = mean0 + s1/L,
+// var = (s2 - s1*s1/L)/L; y uses (x - mean0) - s1/L so that a constant row
+// gives beta bit for bit.
+template <class T, class WT, int G, int V, int BLOCK, bool UNIFORM>
+__global__ void __launch_bounds__(BLOCK)
+gn_fwd_resident_kernel(const T* __restrict__ x, const WT* __restrict__ gamma,
+                       const WT* __restrict__ beta, T* __restrict__ y, WT* __restrict__ mean,
+                       WT* __restrict__ rstd, int64_t rows, GroupShape s, float eps) {
+  constexpr int E = elems_per_pack<T>::value;
+  constexpr int RPB = BLOCK / G;
+  __shared__ float red[reduce_lds_floats<G, BLOCK, 2>::value];
+  int phase = 0;
+  const int slot = threadIdx.x / G;
+  const int lane = threadIdx.x % G;
+  const float fL = (float)s.L;
+  const bool exact = s.L == G * V * E;
+  const int64_t nrb = (rows + RPB - 1) / RPB;
+  for (int64_t rb = blockIdx.x; rb < nrb; rb += gridDim.x) {
+    const int64_t row = rb * RPB + slot;
+    const bool ok = RPB == 1 ? true : row < rows;
+    const int64_t rowc = ok ? row : 0;
+    const int g = (int)((uint32_t)rowc % (uint32_t)s.groups);
+    const T* xr = x + rowc * (int64_t)s.L;
+    Pack<T, E> xp[V];
+#pragma unroll
+    for (int c = 0; c < V; ++c)
+      xp[c] = row_load<T, E, true, UNIFORM>(xr, (c * G + lane) * E, s.L, ok, 0.0f);
+    float acc0[1] = {0.0f};
+#pragma unroll
+    for (int c = 0; c < V; ++c)
+#pragma unroll
+      for (int i = 0; i < E; ++i) acc0[0] += xp[c].get(i);
+    group_allreduce<G, BLOCK, 1, SumOp>(acc0, red, phase);
+    const float mean0 = acc0[0] / fL;
+    float acc[2] = {0.0f, 0.0f};
+    auto centred_sums = [&](auto masked) {
+      constexpr bool MASKED = decltype(masked)::value;
+#pragma unroll
+      for (int c = 0; c < V; ++c) {
+        keep_packed(xp[c]);
+        const int nvalid = ok ? s.L - (c * G + lane) * E : 0;
+#pragma unroll
+        for (int i = 0; i < E; ++i) {
+          float d = xp[c].get(i) - mean0;
+          if constexpr (MASKED) d = (i < nvalid) ? d : 0.0f;
+          acc[0] += d;
+          acc[1] = fmaf(d, d, acc[1]);
+        }
+      }
+    };
+    if (exact)
+      centred_sums(std::false_type{});
+    else
+      centred_sums(std::true_type{});
+    group_allreduce<G, BLOCK, 2, SumOp>(acc, red, phase);
+    const float m1 = acc[0] / fL;
+    const float var = fmaxf((acc[1] - acc[0] * m1) / fL, 0.0f);
+    const float rs = 1.0f / sqrtf(var + eps);
+    T* yr = y + row * (int64_t)s.L;
+#pragma unroll
+    for (int c = 0; c < V; ++c) {
+      keep_packed(xp[c]);
+      const int e0 = (c * G + lane) * E;
+      Pack<T, E> o;
+      if constexpr (UNIFORM) {
+        const int ch = gn_channel(s, g, e0);
+        const float ga = gn_weight(gamma, ch, 1.0f) * rs;
+        const float be = gn_weight(beta, ch, 0.0f);
+#pragma unroll
+        for (int i = 0; i < E; ++i) o.set(i, ((xp[c].get(i) - mean0) - m1) * ga + be);
+      } else {
+#pragma unroll
+        for (int i = 0; i < E; ++i) {
+          const int ch = gn_channel(s, g, e0 + i);
+          const float ga = gn_weight(gamma, ch, 1.0f) * rs;
+          o.set(i, ((xp[c].get(i) - mean0) - m1) * ga + gn_weight(beta, ch, 0.0f));
+        }
+      }
+      row_store<T, E, true, UNIFORM>(yr, e0, s.L, ok, o);
+    }
+    if (ok && lane == 0) {
+      if (mean) mean[row] = (WT)(mean0 + m1);
+      if (rstd) rstd[row] = (WT)rs;
+    }
+  }
+}
+
+// Forward for rows too long for the registers: one workgroup per row, three
+// passes over the row (sum, centred sums, normalize).
+template <class T, class WT, int BLOCK>
+__global__ void __launch_bounds__(BLOCK)
+gn_fwd_stream_kernel(const T* __restrict__ x, const WT* __restrict__ gamma,
+                     const WT* __restrict__ beta, T* __restrict__ y, WT* __restrict__ mean,
+                     WT* __restrict__ rstd, int64_t rows, GroupShape s, float eps) {
+  constexpr int E = elems_per_pack<T>::value;
+  __shared__ float red[reduce_lds_floats<BLOCK, BLOCK, 2>::value];
+  int phase = 0;
+  const float fL = (float)s.L;
+  const int npacks = (s.L + E - 1) / E;
+  for (int64_t row = blockIdx.x; row < rows; row += gridDim.x) {
+    const int g = (int)((uint32_t)row % (uint32_t)s.groups);
+    const T* xr = x + row * (int64_t)s.L;
+    T* yr = y + row * (int64_t)s.L;
+    float acc0[1] = {0.0f};
+    for (int pk = threadIdx.x; pk < npacks; pk += BLOCK) {
+      const Pack<T, E> p = load_row_pack<T, E, false>(xr, pk * E, s.L, true, 0.0f);
+#pragma unroll
+      for (int i = 0; i < E; ++i) acc0[0] += p.get(i);
+    }
+    group_allreduce<BLOCK, BLOCK, 1, SumOp>(acc0, red, phase);
+    const float mean0 = acc0[0] / fL;
+    float acc[2] = {0.0f, 0.0f};
+    for (int pk = threadIdx.x; pk < npacks; pk += BLOCK) {
+      const Pack<T, E> p = load_row_pack<T, E, false>(xr, pk * E, s.L, true, 0.0f);
+      const int nvalid = s.L - pk * E;
+#pragma unroll
+      for (int i = 0; i < E; ++i) {
+        const float d = i < nvalid ? p.get(i) - mean0 : 0.0f;
+        acc[0] += d;
+        acc[1] = fmaf(d, d, acc[1]);
+      }
+    }
+    group_allreduce<BLOCK, BLOCK, 2, SumOp>(acc, red, phase);
+    const float m1 = acc[0] / fL;
+    const float var = fmaxf((acc[1] - acc[0] * m1) / fL, 0.0f);
+    const float rs = 1.0f / sqrtf(var + eps);
+    for (int pk = threadIdx.x; pk < npacks; pk += BLOCK) {
+      const int e0 = pk * E;
+      const Pack<T, E> p = load_row_pack<T, E, true>(xr, e0, s.L, true, 0.0f);
+      Pack<T, E> o;
+#pragma unroll
+      for (int i = 0; i < E; ++i) {
+        const int ch = gn_channel(s, g, e0 + i);
+        const float ga = gn_weight(gamma, ch, 1.0f) * rs;
+        o.set(i, ((p.get(i) - mean0) - m1) * ga + gn_weight(beta, ch, 0.0f));
+      }
+      store_row_pack<T, E, true>(yr, e0, s.L, true, o);
+    }
+    if (threadIdx.x == 0) {
+      if (mean) mean[row] = (WT)(mean0 + m1);
+      if (rstd) rstd[row] = (WT)rs;
+    }
+  }
+}
+
+// ---------------------------------------------------------------------------
+// Backward, rows resident in registers.  With UNIFORM and a workspace, each
+// lane parks the sums of dy*xhat and dy over each of its packs in LDS; after a
+// barrier the channels of the row are summed from there in a fixed order (TPC
+// lanes per channel, then a butterfly) and written to part_dg / part_db [N, C].
+template <int G, int V, int BLOCK, bool UNIFORM>
+struct gn_stage_floats {
+  static constexpr int value = UNIFORM ? 2 * BLOCK * V : 1;
+};
+
+template <class T, class WT, int G, int V, int BLOCK, bool UNIFORM>
+__global__ void __launch_bounds__(BLOCK)
+gn_bwd_resident_kernel(const T* __restrict__ dy, const T* __restrict__ x,
+                       const WT* __restrict__ mean, const WT* __restrict__ rstd,
+                       const WT* __restrict__ gamma, T* __restrict__ dx,
+                       float* __restrict__ part_dg, float* __restrict__ part_db, int64_t rows,
+                       GroupShape s, int tpc_log2) {
+  constexpr int E = elems_per_pack<T>::value;
+  constexpr int RPB = BLOCK / G;
+  __shared__ float red[reduce_lds_floats<G, BLOCK, 2>::value];
+  __shared__ float stage[gn_stage_floats<G, V, BLOCK, UNIFORM>::value];
+  int phase = 0;
+  const int slot = threadIdx.x / G;
+  const int lane = threadIdx.x % G;
+  const float fL = (float)s.L;
+  const bool want_cols = UNIFORM && part_dg != nullptr;  // uniform over the grid
+  const int64_t nrb = (rows + RPB - 1) / RPB;
+  for (int64_t rb = blockIdx.x; rb < nrb; rb += gridDim.x) {
+    const int64_t row = rb * RPB + slot;
+    const bool ok = RPB == 1 ? true : row < rows;
+    const int64_t rowc = ok ? row : 0;
+    const int g = (int)((uint32_t)rowc % (uint32_t)s.groups);
+    const float mu = (float)mean[rowc];
+    const float rs = (float)rstd[rowc];
+    Pack<T, E> xp[V], dp[V];
+#pragma unroll
+    for (int c = 0; c < V; ++c) {
+      const int e0 = (c * G + lane) * E;
+      xp[c] = row_load<T, E, true, UNIFORM>(x + rowc * (int64_t)s.L, e0, s.L, ok, 0.0f);
+      dp[c] = row_load<T, E, true, UNIFORM>(dy + rowc * (int64_t)s.L, e0, s.L, ok, 0.0f);
+    }
+    float acc[2] = {0.0f, 0.0f};
+    float* st = stage + slot * (UNIFORM ? 2 * G * V : 0);
+#pragma unroll
+    for (int c = 0; c < V; ++c) {
+      const int e0 = (c * G + lane) * E;
+      if constexpr (UNIFORM) {
+        const float ga = gn_weight(gamma, gn_channel(s, g, e0), 1.0f);
+        float pdg = 0.0f, pdb = 0.0f;
+#pragma unroll
+        for (int i = 0; i < E; ++i) {
+          const float gy = dp[c].get(i);
+          pdb += gy;
+          pdg = fmaf(gy, xp[c].get(i) - mu, pdg);
+        }
+        // zero-filled packs (row slot or pack out of range) add nothing
+        acc[0] = fmaf(pdb, ga, acc[0]);
+        acc[1] = fmaf(pdg * rs, ga, acc[1]);
+        if (want_cols) {
+          st[2 * (c * G + lane)] = pdg * rs;
+          st[2 * (c * G + lane) + 1] = pdb;
+        }
+      } else {
+#pragma unroll
+        for (int i = 0; i < E; ++i) {
+          const float ga = gn_weight(gamma, gn_channel(s, g, e0 + i), 1.0f);
+          const float gv = dp[c].get(i) * ga;
+          acc[0] += gv;
+          acc[1] = fmaf(gv, (xp[c].get(i) - mu) * rs, acc[1]);
+        }
+      }
+    }
+    group_allreduce<G, BLOCK, 2, SumOp>(acc, red, phase);
+    if (dx != nullptr) {
+      T* dr = dx + row * (int64_t)s.L;
+      const float s1 = acc[0], s2 = acc[1];
+      const float term1 = rs / fL;
+#pragma unroll
+      for (int c = 0; c < V; ++c) {
+        keep_packed(xp[c]);
+        keep_packed(dp[c]);
+        const int e0 = (c * G + lane) * E;
+        float gu = 1.0f;
+        if constexpr (UNIFORM) gu = gn_weight(gamma, gn_channel(s, g, e0), 1.0f);
+        Pack<T, E> o;
+#pragma unroll
+        for (int i = 0; i < E; ++i) {
+          const float ga = UNIFORM ? gu : gn_weight(gamma, gn_channel(s, g, e0 + i), 1.0f);
+          const float xh = (xp[c].get(i) - mu) * rs;
+          float f = fL * (dp[c].get(i) * ga);
+          f -= xh * s2;
+          f -= s1;
+          o.set(i, f * term1);
+        }
+        row_store<T, E, true, UNIFORM>(dr, e0, s.L, ok, o);
+      }
+    }
+    if constexpr (UNIFORM) {
+      if (want_cols) {
+        __syncthreads();
+        // channel d of the row owns packs [d * S, (d + 1) * S), S = HxW / E
+        const int S = s.HxW / E;
+        const int TPC = 1 << tpc_log2;  // lanes per channel, power of two <= min(G, 64)
+        const int sub = lane & (TPC - 1);
+        const int cpi = G >> tpc_log2;  // channels per iteration of the slot
+        for (int d0 = 0; d0 < s.D; d0 += cpi) {
+          const int d = d0 + (lane >> tpc_log2);
+          float ag = 0.0f, ab = 0.0f;
+          if (d < s.D) {
+            for (int q = d * S + sub; q < (d + 1) * S; q += TPC) {
+              ag += st[2 * q];
+              ab += st[2 * q + 1];
+            }
+          }
+          for (int off = TPC >> 1; off > 0; off >>= 1) {
+            ag += __shfl_xor(ag, off, 64);
+            ab += __shfl_xor(ab, off, 64);
+          }
+          if (ok && d < s.D && sub == 0) {
+            const int64_t n = row / s.groups;
+            const int64_t o = n * ((int64_t)s.groups * s.D) + (int64_t)g * s.D + d;
+            part_dg[o] = ag;
+            if (part_db) part_db[o] = ab;
+          }
+        }
+        __syncthreads();  // the staging area is reused by the next row
+      }
+    }
+  }
+}
+
+// Backward dX for rows too long for the registers: one workgroup per row, two
+// passes (row sums, then dX).
+template <class T, class WT, int BLOCK>
+__global__ void __launch_bounds__(BLOCK)
+gn_bwd_stream_dx_kernel(const T* __restrict__ dy, const T* __restrict__ x,
+                        const WT* __restrict__ mean, const WT* __restrict__ rstd,
+                        const WT* __restrict__ gamma, T* __restrict__ dx, int64_t rows,
+                        GroupShape s) {
+  constexpr int E = elems_per_pack<T>::value;
+  __shared__ float red[reduce_lds_floats<BLOCK, BLOCK, 2>::value];
+  int phase = 0;
+  const float fL = (float)s.L;
+  const int npacks = (s.L + E - 1) / E;
+  for (int64_t row = blockIdx.x; row < rows; row += gridDim.x) {
+    const int g = (int)((uint32_t)row % (uint32_t)s.groups);
+    const float mu = (float)mean[row], rs = (float)rstd[row];
+    const T* xr = x + row * (int64_t)s.L;
+    const T* gr = dy + row * (int64_t)s.L;
+    T* dr = dx + row * (int64_t)s.L;
+    float acc[2] = {0.0f, 0.0f};
+    for (int pk = threadIdx.x; pk < npacks; pk += BLOCK) {
+      const int e0 = pk * E;
+      const Pack<T, E> px = load_row_pack<T, E, false>(xr, e0, s.L, true, 0.0f);
+      const Pack<T, E> pd = load_row_pack<T, E, false>(gr, e0, s.L, true, 0.0f);
+#pragma unroll
+      for (int i = 0; i < E; ++i) {
+        const float gv = pd.get(i) * gn_weight(gamma, gn_channel(s, g, e0 + i), 1.0f);
+        acc[0] += gv;
+        acc[1] = fmaf(gv, (px.get(i) - mu) * rs, acc[1]);
+      }
+    }
+    group_allreduce<BLOCK, BLOCK, 2, SumOp>(acc, red, phase);
+    const float s1 = acc[0], s2 = acc[1], term1 = rs / fL;
+    for (int pk = threadIdx.x; pk < npacks; pk += BLOCK) {
+      const int e0 = pk * E;
+      const Pack<T, E> px = load_row_pack<T, E, true>(xr, e0, s.L, true, 0.0f);
+      const Pack<T, E> pd = load_row_pack<T, E, true>(gr, e0, s.L, true, 0.0f);
+      Pack<T, E> o;
+#pragma unroll
+      for (int i = 0; i < E; ++i) {
+        const float ga = gn_weight(gamma, gn_channel(s, g, e0 + i), 1.0f);
+        float f = fL * (pd.get(i) * ga);
+        f -= ((px.get(i) - mu) * rs) * s2;
+        f -= s1;
+        o.set(i, f * term1);
+      }
+      store_row_pack<T, E, true>(dr, e0, s.L, true, o);
+    }
+  }
+}
+
+// Per-(n, channel) sums of dy*xhat and dy for the cases the fused path does not
+// cover: LANES lanes (a power of two <= 64) walk one channel row of HxW
+// contiguous elements; a wavefront holds 64 / LANES such rows.
+template <class T, class WT, int BLOCK>
+__global__ void __launch_bounds__(BLOCK)
+gn_channel_sums_kernel(const T* __restrict__ dy, const T* __restrict__ x,
+                       const WT* __restrict__ mean, const WT* __restrict__ rstd,
+                       float* __restrict__ part_dg, float* __restrict__ part_db, int64_t nc_rows,
+                       GroupShape s, int lanes_log2) {
+  constexpr int E = elems_per_pack<T>::value;
+  const int LANES = 1 << lanes_log2;
+  const int sub = threadIdx.x & (LANES - 1);
+  const int rpb = BLOCK >> lanes_log2;  // channel rows per workgroup iteration
+  const int npacks = (s.HxW + E - 1) / E;
+  const int C = s.groups * s.D;
+  const int64_t nrb = (nc_rows + rpb - 1) / rpb;
+  for (int64_t rb = blockIdx.x; rb < nrb; rb += gridDim.x) {
+    const int64_t r = rb * rpb + (threadIdx.x >> lanes_log2);  // n * C + c
+    const bool ok = r < nc_rows;
+    const int64_t rc = ok ? r : 0;
+    const int64_t n = rc / C;
+    const int c = (int)(rc - n * C);
+    const int64_t srow = n * s.groups + c / s.D;
+    const float mu = (float)mean[srow], rs = (float)rstd[srow];
+    const T* xr = x + rc * (int64_t)s.HxW;
+    const T* gr = dy + rc * (int64_t)s.HxW;
+    float ag = 0.0f, ab = 0.0f;
+    for (int pk = sub; pk < npacks; pk += LANES) {
+      const Pack<T, E> px = load_row_pack<T, E, true>(xr, pk * E, s.HxW, ok, 0.0f);
+      const Pack<T, E> pd = load_row_pack<T, E, true>(gr, pk * E, s.HxW, ok, 0.0f);
+      const int nvalid = s.HxW - pk * E;
+#pragma unroll
+      for (int i = 0; i < E; ++i) {
+        const float gy = pd.get(i);
+        ab += gy;
+        ag = fmaf(gy, i < nvalid ? px.get(i) - mu : 0.0f, ag);
+      }
+    }
+    for (int off = LANES >> 1; off > 0; off >>= 1) {
+      ag += __shfl_xor(ag, off, 64);
+      ab += __shfl_xor(ab, off, 64);
+    }
+    if (ok && sub == 0) {
+      part_dg[r] = ag * rs;
+      if (part_db) part_db[r] = ab;
+    }
+  }
+}
+
+}  // namespace rownorm

@@ -1,0 +1,144 @@
+// Host dispatch of the GroupNorm kernels: plan -> template instance.
+#pragma once
+#include "groupnorm_kernels.hpp"
+#include "launch.hpp"
+#include "norm_kernels.hpp"  // colsum_finalize_kernel
+
+namespace rownorm {
+
+inline GroupShape group_shape(int L, int HxW, int D, int groups) { return GroupShape{L, HxW, D, groups}; }
+
+template <class T, class WT>
+struct GroupNormFwdCtx {
+  const Plan& plan;
+  const GroupNormFwdArgs& a;
+  hipStream_t stream;
+};
+
+template <class T, class WT, bool UNIFORM>
+struct GroupNormFwdLauncher {
+  template <int G, int V, int BLOCK>
+  struct At {
+    static bool run(const GroupNormFwdCtx<T, WT>& c) {
+      if constexpr (variant_built(OC_GROUP_FWD, sizeof(T), G, V, UNIFORM) &&
+                    block_built(OC_GROUP_FWD, G, BLOCK)) {
+        if (c.plan.G == G && c.plan.V == V && c.plan.block == BLOCK) {
+          hipLaunchKernelGGL((gn_fwd_resident_kernel<T, WT, G, V, BLOCK, UNIFORM>),
+                             dim3((unsigned)c.plan.grid), dim3(BLOCK), 0, c.stream,
+                             (const T*)c.a.x, (const WT*)c.a.gamma, (const WT*)c.a.beta,
+                             (T*)c.a.y, (WT*)c.a.mean, (WT*)c.a.rstd, c.a.rows,
+                             group_shape(c.a.L, c.a.HxW, c.a.D, c.a.groups), c.a.eps);
+          return true;
+        }
+      }
+      return false;
+    }
+  };
+};
+
+template <class T, class WT>
+int launch_group_norm_fwd(const Plan& plan, const GroupNormFwdArgs& a, hipStream_t stream) {
+  if (plan.resident) {
+    GroupNormFwdCtx<T, WT> ctx{plan, a, stream};
+    const bool launched =
+        plan.fast ? launch_variant<GroupNormFwdLauncher<T, WT, true>::template At>(ctx)
+                  : launch_variant<GroupNormFwdLauncher<T, WT, false>::template At>(ctx);
+    if (!launched) return (int)hipErrorInvalidConfiguration;
+  } else {
+    hipLaunchKernelGGL((gn_fwd_stream_kernel<T, WT, kStreamBlock>), dim3((unsigned)plan.grid),
+                       dim3(kStreamBlock), 0, stream, (const T*)a.x, (const WT*)a.gamma,
+                       (const WT*)a.beta, (T*)a.y, (WT*)a.mean, (WT*)a.rstd, a.rows,
+                       group_shape(a.L, a.HxW, a.D, a.groups), a.eps);
+  }
+  return (int)hipGetLastError();
+}
+
+template <class T, class WT>
+struct GroupNormBwdCtx {
+  const Plan& plan;
+  const GroupNormBwdArgs& a;
+  int tpc_log2;
+  hipStream_t stream;
+};
+
+template <class T, class WT, bool UNIFORM>
+struct GroupNormBwdLauncher {
+  template <int G, int V, int BLOCK>
+  struct At {
+    static bool run(const GroupNormBwdCtx<T, WT>& c) {
+      if constexpr (variant_built(OC_GROUP_BWD, sizeof(T), G, V, UNIFORM) &&
+                    block_built(OC_GROUP_BWD, G, BLOCK)) {
+        if (c.plan.G == G && c.plan.V == V && c.plan.block == BLOCK) {
+          hipLaunchKernelGGL((gn_bwd_resident_kernel<T, WT, G, V, BLOCK, UNIFORM>),
+                             dim3((unsigned)c.plan.grid), dim3(BLOCK), 0, c.stream,
+                             (const T*)c.a.dy, (const T*)c.a.x, (const WT*)c.a.mean,
+                             (const WT*)c.a.rstd, (const WT*)c.a.gamma, (T*)c.a.dx, c.a.part_dg,
+                             c.a.part_db, c.a.rows,
+                             group_shape(c.a.L, c.a.HxW, c.a.D, c.a.groups), c.tpc_log2);
+          return true;
+        }
+      }
+      return false;
+    }
+  };
+};
+
+// Lanes that share one channel in the fused channel sums: as many as the row
+// group has to spare for its D channels, at most a wavefront, at most the packs
+// of a channel.
+inline int gn_tpc_log2(int G, int D, int packs_per_channel) {
+  int tpc = G / pow2_ceil(D);
+  if (tpc > 64) tpc = 64;
+  while (tpc > 1 && tpc > packs_per_channel) tpc >>= 1;
+  if (tpc < 1) tpc = 1;
+  return log2_of_pow2(tpc);
+}
+
+template <class T, class WT>
+int launch_group_norm_bwd(const Plan& plan, const GroupNormBwdArgs& a, hipStream_t stream) {
+  constexpr int E = elems_per_pack<T>::value;
+  const bool want_cols = a.part_dg != nullptr;
+  const bool fused_cols = plan.resident && plan.fast;  // channel sums come out of the dX kernel
+  const GroupShape shape = group_shape(a.L, a.HxW, a.D, a.groups);
+  if (plan.resident) {
+    if (a.dx != nullptr || (want_cols && fused_cols)) {
+      GroupNormBwdCtx<T, WT> ctx{plan, a, 0, stream};
+      if (plan.fast) ctx.tpc_log2 = gn_tpc_log2(plan.G, a.D, a.HxW / E);
+      const bool launched =
+          plan.fast ? launch_variant<GroupNormBwdLauncher<T, WT, true>::template At>(ctx)
+                    : launch_variant<GroupNormBwdLauncher<T, WT, false>::template At>(ctx);
+      if (!launched) return (int)hipErrorInvalidConfiguration;
+    }
+  } else if (a.dx != nullptr) {
+    hipLaunchKernelGGL((gn_bwd_stream_dx_kernel<T, WT, kStreamBlock>), dim3((unsigned)plan.grid),
+                       dim3(kStreamBlock), 0, stream, (const T*)a.dy, (const T*)a.x,
+                       (const WT*)a.mean, (const WT*)a.rstd, (const WT*)a.gamma, (T*)a.dx, a.rows,
+                       shape);
+  }
+  int err = (int)hipGetLastError();
+  if (err != 0 || !want_cols) return err;
+  const int64_t N = a.rows / a.groups;
+  const int C = a.groups * a.D;
+  if (!fused_cols) {
+    constexpr int CB = 256;
+    const int packs = (a.HxW + E - 1) / E;
+    const int lanes = packs >= 64 ? 64 : pow2_ceil(packs);
+    const int64_t nc_rows = N * C;
+    const int rpb = CB / lanes;
+    int64_t grid = (nc_rows + rpb - 1) / rpb;
+    if (grid > (1 << 22)) grid = 1 << 22;
+    hipLaunchKernelGGL((gn_channel_sums_kernel<T, WT, CB>), dim3((unsigned)grid), dim3(CB), 0,
+                       stream, (const T*)a.dy, (const T*)a.x, (const WT*)a.mean,
+                       (const WT*)a.rstd, a.part_dg, a.part_db, nc_rows, shape,
+                       log2_of_pow2(lanes));
+    err = (int)hipGetLastError();
+    if (err != 0) return err;
+  }
+  const unsigned gx = (unsigned)((C + kFinalizeCols - 1) / kFinalizeCols);
+  hipLaunchKernelGGL((colsum_finalize_kernel<WT>), dim3(gx, 2), dim3(1024), 0, stream,
+                     (const float*)a.part_dg, (const float*)a.part_db, (WT*)a.dgamma,
+                     (WT*)a.dbeta, (int)N, C);
+  return (int)hipGetLastError();
+}
+
+}  // namespace rownorm

@@ -79,6 +79,34 @@ struct SoftmaxStridedBwdArgs {
   int flags;
 };
 
+// GroupNorm on [N, C, HxW] with C = groups * D: rows = N * groups rows of L = D * HxW.
+struct GroupNormFwdArgs {
+  const void* x;
+  const void* gamma;
+  const void* beta;
+  void* y;
+  void* mean;  // [rows], weight dtype
+  void* rstd;
+  int64_t rows;
+  int L, HxW, D, groups;
+  float eps;
+};
+
+struct GroupNormBwdArgs {
+  const void* dy;
+  const void* x;
+  const void* mean;
+  const void* rstd;
+  const void* gamma;
+  void* dx;
+  void* dgamma;
+  void* dbeta;
+  float* part_dg;  // [N, C] fp32 each, or null when neither dgamma nor dbeta is wanted
+  float* part_db;
+  int64_t rows;
+  int L, HxW, D, groups;
+};
+
 // All return 0 or a hipError_t value.
 template <class T, class WT, bool RMS>
 int launch_norm_fwd(const Plan& plan, const NormFwdArgs& a, hipStream_t stream);
@@ -89,6 +117,10 @@ int launch_softmax_fwd(const Plan& plan, const SoftmaxFwdArgs& a, hipStream_t st
 template <class TG, class TO>
 int launch_softmax_bwd(const Plan& plan, const SoftmaxBwdArgs& a, hipStream_t stream);
 
+template <class T, class WT>
+int launch_group_norm_fwd(const Plan& plan, const GroupNormFwdArgs& a, hipStream_t stream);
+template <class T, class WT>
+int launch_group_norm_bwd(const Plan& plan, const GroupNormBwdArgs& a, hipStream_t stream);
 template <class TI, class TO>
 int launch_softmax_strided_fwd(const StridedPlan& plan, const SoftmaxStridedFwdArgs& a,
                                hipStream_t stream);

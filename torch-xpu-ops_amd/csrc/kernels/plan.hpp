@@ -21,7 +21,14 @@
 
 namespace rownorm {
 
-enum OpClass { OC_NORM_FWD = 0, OC_NORM_BWD = 1, OC_SOFTMAX_FWD = 2, OC_SOFTMAX_BWD = 3 };
+enum OpClass {
+  OC_NORM_FWD = 0,
+  OC_NORM_BWD = 1,
+  OC_SOFTMAX_FWD = 2,
+  OC_SOFTMAX_BWD = 3,
+  OC_GROUP_FWD = 4,  // GroupNorm: rows are (sample, group) slabs, no per-column registers
+  OC_GROUP_BWD = 5
+};
 
 struct Override {
   int G = 0, V = 0, block = 0, bpc = 0;  // 0 = automatic; G = -1 = force the streaming kernel
@@ -55,6 +62,10 @@ constexpr int v_max(OpClass oc, int esize, int G) {
     case OC_NORM_BWD: v = esize == 4 ? 8 : 4; break;
     case OC_SOFTMAX_FWD: v = esize == 4 ? 16 : 8; break;
     case OC_SOFTMAX_BWD: v = esize == 4 ? 16 : 8; break;
+    // GroupNorm lanes hold the row (and dY) only, no weights or column sums, so
+    // 16-bit rows keep 8 packs a lane at 1024 lanes (128 VGPRs); fp32 rows halve
+    case OC_GROUP_FWD: return esize == 4 ? (G >= 1024 ? 8 : 16) : 8;
+    case OC_GROUP_BWD: return esize == 4 ? (G >= 1024 ? 4 : 8) : 8;
   }
   if (G >= 1024 && v > 1) v /= 2;
   return v;
@@ -66,7 +77,7 @@ constexpr int v_max(OpClass oc, int esize, int G) {
 //                   of the dgamma/dbeta reduction;
 //   softmax         512 at least.
 constexpr int block_threads(OpClass oc, int G) {
-  const int floor_threads = oc == OC_NORM_FWD ? 256 : 512;
+  const int floor_threads = (oc == OC_NORM_FWD || oc == OC_GROUP_FWD) ? 256 : 512;
   return G <= floor_threads ? floor_threads : G;
 }
 
@@ -117,12 +128,13 @@ inline int pow2_ceil(int64_t v) {
 }
 
 // Returns 0, or -5 (ROWNORM_ERR_OVERRIDE) when a forced variant cannot hold the row.
+// force_general: take the general (ragged-row) kernels even when N % E == 0.
 inline int make_plan(OpClass oc, int64_t M, int64_t N, int esize, int num_cus, const Override& ov,
-                     bool want_cols, Plan* out) {
+                     bool want_cols, Plan* out, bool force_general = false) {
   Plan p;
   const int E = 16 / esize;
   const int64_t packs = (N + E - 1) / E;
-  p.fast = (N % E) == 0;
+  p.fast = (N % E) == 0 && !force_general;
   if (num_cus <= 0) num_cus = 256;
   bool stream = ov.G < 0;
   if (!stream) {
