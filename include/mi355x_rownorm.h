@@ -194,8 +194,10 @@ int mi355x_group_norm_fwd(const void* x, const void* gamma, const void* beta, vo
                           void* rstd, int64_t N, int64_t C, int64_t HxW, int64_t groups, float eps,
                           rownorm_dtype x_dtype, rownorm_dtype w_dtype, void* stream);
 
-/* Bytes of device scratch mi355x_group_norm_bwd needs (0 when neither dgamma
- * nor dbeta is wanted): two float32 [N, C] arrays of per-sample channel sums.
+/* Bytes of device scratch mi355x_group_norm_bwd needs: two float32 [N, C]
+ * arrays of per-sample channel sums; 0 when neither dgamma nor dbeta is wanted
+ * and a (sample, group) row fits the registers (longer rows get dX from the
+ * channel sums, so they always need the scratch).
  * The reference allocates the same two (ds, db) with at::empty
  * (GroupNormKernels.cpp:1398-1399). */
 size_t mi355x_group_norm_bwd_workspace_bytes(int64_t N, int64_t C, int64_t HxW, int64_t groups,

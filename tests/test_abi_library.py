@@ -233,6 +233,9 @@ def test_group_norm_validation_and_plans(cabi):
     assert b(one, one, one, one, null, null, null, null, null, 0, 2, 6, 4, 3, 0, 0, null) == 0  # nothing asked
     assert L.mi355x_group_norm_bwd_workspace_bytes(2, 6, 4, 3, 0, 0, 1, 0) == 2 * 2 * 6 * 4
     assert L.mi355x_group_norm_bwd_workspace_bytes(2, 6, 4, 3, 0, 0, 0, 0) == 0
+    # rows too long for the registers need the channel sums for dX alone
+    assert L.mi355x_group_norm_bwd_workspace_bytes(1, 4, 1 << 20, 2, 0, 0, 0, 0) == 2 * 1 * 4 * 4
+    assert b(one, one, one, one, null, one, null, null, null, 0, 1, 4, 1 << 20, 2, 0, 0, null) == -4
     for dt, E in ((cabi.F32, 4), (cabi.BF16, 8)):
         for (N, C, HxW, G) in ((2, 4, 1, 2), (256, 32, 16, 4), (4, 64, 1024, 32), (2, 320, 4096, 32),
                                (3, 6, 5, 3), (1, 4, 1 << 17, 2), (1, 8, 1 << 20, 2)):

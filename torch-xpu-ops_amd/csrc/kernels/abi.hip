@@ -419,7 +419,14 @@ size_t mi355x_group_norm_bwd_workspace_bytes(int64_t N, int64_t C, int64_t HxW, 
                                              int want_dgamma, int want_dbeta) {
   GroupDims d;
   if (!norm_dtypes_ok((int)x_dtype, (int)w_dtype) || group_dims(N, C, HxW, groups, &d)) return 0;
-  if (d.rows == 0 || d.L == 0 || !(want_dgamma || want_dbeta)) return 0;
+  if (d.rows == 0 || d.L == 0) return 0;
+  if (!(want_dgamma || want_dbeta)) {
+    // rows too long for the registers compute dX from the channel sums
+    Plan plan;
+    if (group_plan(OC_GROUP_BWD, ROWNORM_OP_GROUP_NORM_BWD, d, HxW, esize_of((int)x_dtype), &plan))
+      return 0;
+    if (plan.resident) return 0;
+  }
   return (size_t)N * (size_t)C * sizeof(float) * 2;
 }
 
@@ -441,7 +448,7 @@ int mi355x_group_norm_bwd(const void* dy, const void* x, const void* mean, const
     return e;
   float* part_dg = nullptr;
   float* part_db = nullptr;
-  if (want_cols) {
+  if (want_cols || (!plan.resident && dx)) {
     const size_t one = (size_t)N * (size_t)C * sizeof(float);
     if (!workspace || workspace_bytes < 2 * one) return ROWNORM_ERR_WORKSPACE;
     part_dg = (float*)workspace;

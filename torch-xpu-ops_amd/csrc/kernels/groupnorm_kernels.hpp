@@ -14,7 +14,9 @@
 // (one weight lookup per pack, branch-free row access, channel sums fused into
 // the backward through an LDS staging area).  Otherwise the channel is looked
 // up per element, row access is the general one, and the channel sums come
-// from gn_channel_sums_kernel, which reads dY and X a second time.
+// from gn_channel_sums_kernel, which reads dY and X a second time.  Rows too
+// long for the registers: the forward takes two passes over the row; the
+// backward computes the channel sums first and dX from them, element by element.
 //
 // What these stand in for in the reference (src/ATen/native/xpu/sycl/
 // GroupNormKernels.cpp): GNRowwiseMomentsFunctor / ...VectorizedFunctor
@@ -152,15 +154,20 @@ gn_fwd_resident_kernel(const T* __restrict__ x, const WT* __restrict__ gamma,
   }
 }
 
-// Forward for rows too long for the registers: one workgroup per row, three
-// passes over the row (sum, centred sums, normalize).
+// Forward for rows too long for the registers: one workgroup per row, two
+// passes over the row (statistics, normalize).  Each thread sums its elements
+// shifted by the first one it sees, (x - k), (x - k)^2, which gives its own
+// count / mean / M2 without cancellation; the threads' triples are then merged
+// with the pairwise formula of WelfordOps::combine (src/ATen/native/xpu/sycl/
+// SharedReduceOps.h:71-88) written as two block sums: mean = k0 + sum n_t *
+// (mean_t - k0) / L, M2 = sum M2_t + n_t * (mean_t - mean)^2.
 template <class T, class WT, int BLOCK>
 __global__ void __launch_bounds__(BLOCK)
 gn_fwd_stream_kernel(const T* __restrict__ x, const WT* __restrict__ gamma,
                      const WT* __restrict__ beta, T* __restrict__ y, WT* __restrict__ mean,
                      WT* __restrict__ rstd, int64_t rows, GroupShape s, float eps) {
   constexpr int E = elems_per_pack<T>::value;
-  __shared__ float red[reduce_lds_floats<BLOCK, BLOCK, 2>::value];
+  __shared__ float red[reduce_lds_floats<BLOCK, BLOCK, 1>::value];
   int phase = 0;
   const float fL = (float)s.L;
   const int npacks = (s.L + E - 1) / E;
@@ -168,29 +175,35 @@ gn_fwd_stream_kernel(const T* __restrict__ x, const WT* __restrict__ gamma,
     const int g = (int)((uint32_t)row % (uint32_t)s.groups);
     const T* xr = x + row * (int64_t)s.L;
     T* yr = y + row * (int64_t)s.L;
-    float acc0[1] = {0.0f};
+    float k = 0.0f, s1 = 0.0f, s2 = 0.0f, cnt = 0.0f;
+    bool first = true;
     for (int pk = threadIdx.x; pk < npacks; pk += BLOCK) {
       const Pack<T, E> p = load_row_pack<T, E, false>(xr, pk * E, s.L, true, 0.0f);
-#pragma unroll
-      for (int i = 0; i < E; ++i) acc0[0] += p.get(i);
-    }
-    group_allreduce<BLOCK, BLOCK, 1, SumOp>(acc0, red, phase);
-    const float mean0 = acc0[0] / fL;
-    float acc[2] = {0.0f, 0.0f};
-    for (int pk = threadIdx.x; pk < npacks; pk += BLOCK) {
-      const Pack<T, E> p = load_row_pack<T, E, false>(xr, pk * E, s.L, true, 0.0f);
+      if (first) {
+        k = p.get(0);
+        first = false;
+      }
       const int nvalid = s.L - pk * E;
 #pragma unroll
       for (int i = 0; i < E; ++i) {
-        const float d = i < nvalid ? p.get(i) - mean0 : 0.0f;
-        acc[0] += d;
-        acc[1] = fmaf(d, d, acc[1]);
+        const float d = i < nvalid ? p.get(i) - k : 0.0f;
+        s1 += d;
+        s2 = fmaf(d, d, s2);
       }
+      cnt += (float)(nvalid < E ? nvalid : E);
     }
-    group_allreduce<BLOCK, BLOCK, 2, SumOp>(acc, red, phase);
-    const float m1 = acc[0] / fL;
-    const float var = fmaxf((acc[1] - acc[0] * m1) / fL, 0.0f);
-    const float rs = 1.0f / sqrtf(var + eps);
+    const float mean_t = cnt > 0.0f ? k + s1 / cnt : 0.0f;
+    const float m2_t = cnt > 0.0f ? fmaxf(s2 - s1 * (s1 / cnt), 0.0f) : 0.0f;
+    // summed relative to the row's first element, so a constant row gets its
+    // constant back exactly
+    const float k0 = (float)xr[0];
+    float a[1] = {cnt * (mean_t - k0)};
+    group_allreduce<BLOCK, BLOCK, 1, SumOp>(a, red, phase);
+    const float mu = k0 + a[0] / fL;
+    const float dm = mean_t - mu;
+    float b[1] = {m2_t + cnt * dm * dm};
+    group_allreduce<BLOCK, BLOCK, 1, SumOp>(b, red, phase);
+    const float rs = 1.0f / sqrtf(fmaxf(b[0] / fL, 0.0f) + eps);
     for (int pk = threadIdx.x; pk < npacks; pk += BLOCK) {
       const int e0 = pk * E;
       const Pack<T, E> p = load_row_pack<T, E, true>(xr, e0, s.L, true, 0.0f);
@@ -199,12 +212,12 @@ gn_fwd_stream_kernel(const T* __restrict__ x, const WT* __restrict__ gamma,
       for (int i = 0; i < E; ++i) {
         const int ch = gn_channel(s, g, e0 + i);
         const float ga = gn_weight(gamma, ch, 1.0f) * rs;
-        o.set(i, ((p.get(i) - mean0) - m1) * ga + gn_weight(beta, ch, 0.0f));
+        o.set(i, (p.get(i) - mu) * ga + gn_weight(beta, ch, 0.0f));
       }
       store_row_pack<T, E, true>(yr, e0, s.L, true, o);
     }
     if (threadIdx.x == 0) {
-      if (mean) mean[row] = (WT)(mean0 + m1);
+      if (mean) mean[row] = (WT)mu;
       if (rstd) rstd[row] = (WT)rs;
     }
   }
@@ -341,47 +354,58 @@ gn_bwd_resident_kernel(const T* __restrict__ dy, const T* __restrict__ x,
   }
 }
 
-// Backward dX for rows too long for the registers: one workgroup per row, two
-// passes (row sums, then dX).
+// Backward dX for rows too long for the registers, from the per-(n, channel)
+// sums that gn_channel_sums_kernel left in part_dg / part_db: every workgroup
+// takes one chunk of BLOCK * CHUNK_PACKS packs of one row, rebuilds the row's
+// s1 = sum_c gamma*db and s2 = sum_c gamma*dg from the D channel sums (the
+// reference's ComputeBackwardFusedParamsFunctor, GroupNormKernels.cpp:
+// 1088-1165) and then works element by element, so a few very long rows still
+// spread over the whole machine.
+constexpr int kGnChunkPacks = 8;
+
 template <class T, class WT, int BLOCK>
 __global__ void __launch_bounds__(BLOCK)
-gn_bwd_stream_dx_kernel(const T* __restrict__ dy, const T* __restrict__ x,
-                        const WT* __restrict__ mean, const WT* __restrict__ rstd,
-                        const WT* __restrict__ gamma, T* __restrict__ dx, int64_t rows,
-                        GroupShape s) {
+gn_bwd_dx_from_sums_kernel(const T* __restrict__ dy, const T* __restrict__ x,
+                           const WT* __restrict__ mean, const WT* __restrict__ rstd,
+                           const WT* __restrict__ gamma, const float* __restrict__ part_dg,
+                           const float* __restrict__ part_db, T* __restrict__ dx, int64_t rows,
+                           GroupShape s, int chunks_per_row) {
   constexpr int E = elems_per_pack<T>::value;
   __shared__ float red[reduce_lds_floats<BLOCK, BLOCK, 2>::value];
   int phase = 0;
   const float fL = (float)s.L;
-  const int npacks = (s.L + E - 1) / E;
-  for (int64_t row = blockIdx.x; row < rows; row += gridDim.x) {
+  const int64_t ntiles = rows * chunks_per_row;
+  const bool uniform = (s.HxW % E) == 0;
+  for (int64_t t = blockIdx.x; t < ntiles; t += gridDim.x) {
+    const int64_t row = t / chunks_per_row;
+    const int chunk = (int)(t - row * chunks_per_row);
     const int g = (int)((uint32_t)row % (uint32_t)s.groups);
+    const int64_t n = row / s.groups;
     const float mu = (float)mean[row], rs = (float)rstd[row];
-    const T* xr = x + row * (int64_t)s.L;
-    const T* gr = dy + row * (int64_t)s.L;
-    T* dr = dx + row * (int64_t)s.L;
+    const int64_t c0 = n * ((int64_t)s.groups * s.D) + (int64_t)g * s.D;
     float acc[2] = {0.0f, 0.0f};
-    for (int pk = threadIdx.x; pk < npacks; pk += BLOCK) {
-      const int e0 = pk * E;
-      const Pack<T, E> px = load_row_pack<T, E, false>(xr, e0, s.L, true, 0.0f);
-      const Pack<T, E> pd = load_row_pack<T, E, false>(gr, e0, s.L, true, 0.0f);
-#pragma unroll
-      for (int i = 0; i < E; ++i) {
-        const float gv = pd.get(i) * gn_weight(gamma, gn_channel(s, g, e0 + i), 1.0f);
-        acc[0] += gv;
-        acc[1] = fmaf(gv, (px.get(i) - mu) * rs, acc[1]);
-      }
+    for (int d = threadIdx.x; d < s.D; d += BLOCK) {
+      const float ga = gn_weight(gamma, g * s.D + d, 1.0f);
+      acc[0] = fmaf(part_db[c0 + d], ga, acc[0]);
+      acc[1] = fmaf(part_dg[c0 + d], ga, acc[1]);
     }
     group_allreduce<BLOCK, BLOCK, 2, SumOp>(acc, red, phase);
     const float s1 = acc[0], s2 = acc[1], term1 = rs / fL;
-    for (int pk = threadIdx.x; pk < npacks; pk += BLOCK) {
-      const int e0 = pk * E;
+    const T* xr = x + row * (int64_t)s.L;
+    const T* gr = dy + row * (int64_t)s.L;
+    T* dr = dx + row * (int64_t)s.L;
+#pragma unroll
+    for (int k = 0; k < kGnChunkPacks; ++k) {
+      const int64_t pk = ((int64_t)chunk * kGnChunkPacks + k) * BLOCK + threadIdx.x;
+      const int64_t e64 = pk * E;
+      const int e0 = e64 < s.L ? (int)e64 : s.L;
       const Pack<T, E> px = load_row_pack<T, E, true>(xr, e0, s.L, true, 0.0f);
       const Pack<T, E> pd = load_row_pack<T, E, true>(gr, e0, s.L, true, 0.0f);
+      const float gu = gn_weight(gamma, gn_channel(s, g, e0), 1.0f);
       Pack<T, E> o;
 #pragma unroll
       for (int i = 0; i < E; ++i) {
-        const float ga = gn_weight(gamma, gn_channel(s, g, e0 + i), 1.0f);
+        const float ga = uniform ? gu : gn_weight(gamma, gn_channel(s, g, e0 + i), 1.0f);
         float f = fL * (pd.get(i) * ga);
         f -= ((px.get(i) - mu) * rs) * s2;
         f -= s1;
@@ -393,8 +417,9 @@ gn_bwd_stream_dx_kernel(const T* __restrict__ dy, const T* __restrict__ x,
 }
 
 // Per-(n, channel) sums of dy*xhat and dy for the cases the fused path does not
-// cover: LANES lanes (a power of two <= 64) walk one channel row of HxW
-// contiguous elements; a wavefront holds 64 / LANES such rows.
+// cover.  LANES lanes walk one channel row of HxW contiguous elements: a power
+// of two up to 64 (a wavefront then holds 64 / LANES rows, reduced with
+// shuffles), or the whole workgroup for long channel rows (reduced through LDS).
 template <class T, class WT, int BLOCK>
 __global__ void __launch_bounds__(BLOCK)
 gn_channel_sums_kernel(const T* __restrict__ dy, const T* __restrict__ x,
@@ -402,7 +427,10 @@ gn_channel_sums_kernel(const T* __restrict__ dy, const T* __restrict__ x,
                        float* __restrict__ part_dg, float* __restrict__ part_db, int64_t nc_rows,
                        GroupShape s, int lanes_log2) {
   constexpr int E = elems_per_pack<T>::value;
+  __shared__ float red[reduce_lds_floats<BLOCK, BLOCK, 2>::value];
+  int phase = 0;
   const int LANES = 1 << lanes_log2;
+  const bool whole_block = LANES == BLOCK;  // uniform
   const int sub = threadIdx.x & (LANES - 1);
   const int rpb = BLOCK >> lanes_log2;  // channel rows per workgroup iteration
   const int npacks = (s.HxW + E - 1) / E;
@@ -418,7 +446,7 @@ gn_channel_sums_kernel(const T* __restrict__ dy, const T* __restrict__ x,
     const float mu = (float)mean[srow], rs = (float)rstd[srow];
     const T* xr = x + rc * (int64_t)s.HxW;
     const T* gr = dy + rc * (int64_t)s.HxW;
-    float ag = 0.0f, ab = 0.0f;
+    float acc[2] = {0.0f, 0.0f};
     for (int pk = sub; pk < npacks; pk += LANES) {
       const Pack<T, E> px = load_row_pack<T, E, true>(xr, pk * E, s.HxW, ok, 0.0f);
       const Pack<T, E> pd = load_row_pack<T, E, true>(gr, pk * E, s.HxW, ok, 0.0f);
@@ -426,17 +454,21 @@ gn_channel_sums_kernel(const T* __restrict__ dy, const T* __restrict__ x,
 #pragma unroll
       for (int i = 0; i < E; ++i) {
         const float gy = pd.get(i);
-        ab += gy;
-        ag = fmaf(gy, i < nvalid ? px.get(i) - mu : 0.0f, ag);
+        acc[1] += gy;
+        acc[0] = fmaf(gy, i < nvalid ? px.get(i) - mu : 0.0f, acc[0]);
       }
     }
-    for (int off = LANES >> 1; off > 0; off >>= 1) {
-      ag += __shfl_xor(ag, off, 64);
-      ab += __shfl_xor(ab, off, 64);
+    if (whole_block) {
+      group_allreduce<BLOCK, BLOCK, 2, SumOp>(acc, red, phase);
+    } else {
+      for (int off = LANES >> 1; off > 0; off >>= 1) {
+        acc[0] += __shfl_xor(acc[0], off, 64);
+        acc[1] += __shfl_xor(acc[1], off, 64);
+      }
     }
     if (ok && sub == 0) {
-      part_dg[r] = ag * rs;
-      if (part_db) part_db[r] = ab;
+      part_dg[r] = acc[0] * rs;
+      if (part_db) part_db[r] = acc[1];
     }
   }
 }

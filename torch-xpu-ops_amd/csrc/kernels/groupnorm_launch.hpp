@@ -97,32 +97,19 @@ inline int gn_tpc_log2(int G, int D, int packs_per_channel) {
 template <class T, class WT>
 int launch_group_norm_bwd(const Plan& plan, const GroupNormBwdArgs& a, hipStream_t stream) {
   constexpr int E = elems_per_pack<T>::value;
-  const bool want_cols = a.part_dg != nullptr;
+  const bool want_cols = a.dgamma != nullptr || a.dbeta != nullptr;
   const bool fused_cols = plan.resident && plan.fast;  // channel sums come out of the dX kernel
+  // rows too long for the registers get dX from the channel sums, wanted or not
+  const bool need_sums = want_cols || (!plan.resident && a.dx != nullptr);
   const GroupShape shape = group_shape(a.L, a.HxW, a.D, a.groups);
-  if (plan.resident) {
-    if (a.dx != nullptr || (want_cols && fused_cols)) {
-      GroupNormBwdCtx<T, WT> ctx{plan, a, 0, stream};
-      if (plan.fast) ctx.tpc_log2 = gn_tpc_log2(plan.G, a.D, a.HxW / E);
-      const bool launched =
-          plan.fast ? launch_variant<GroupNormBwdLauncher<T, WT, true>::template At>(ctx)
-                    : launch_variant<GroupNormBwdLauncher<T, WT, false>::template At>(ctx);
-      if (!launched) return (int)hipErrorInvalidConfiguration;
-    }
-  } else if (a.dx != nullptr) {
-    hipLaunchKernelGGL((gn_bwd_stream_dx_kernel<T, WT, kStreamBlock>), dim3((unsigned)plan.grid),
-                       dim3(kStreamBlock), 0, stream, (const T*)a.dy, (const T*)a.x,
-                       (const WT*)a.mean, (const WT*)a.rstd, (const WT*)a.gamma, (T*)a.dx, a.rows,
-                       shape);
-  }
-  int err = (int)hipGetLastError();
-  if (err != 0 || !want_cols) return err;
   const int64_t N = a.rows / a.groups;
   const int C = a.groups * a.D;
-  if (!fused_cols) {
+  int err = 0;
+  if (need_sums && !fused_cols) {
     constexpr int CB = 256;
     const int packs = (a.HxW + E - 1) / E;
-    const int lanes = packs >= 64 ? 64 : pow2_ceil(packs);
+    // long channel rows take a whole workgroup each
+    const int lanes = packs >= 8 * CB ? CB : (packs >= 64 ? 64 : pow2_ceil(packs));
     const int64_t nc_rows = N * C;
     const int rpb = CB / lanes;
     int64_t grid = (nc_rows + rpb - 1) / rpb;
@@ -134,6 +121,30 @@ int launch_group_norm_bwd(const Plan& plan, const GroupNormBwdArgs& a, hipStream
     err = (int)hipGetLastError();
     if (err != 0) return err;
   }
+  if (plan.resident) {
+    if (a.dx != nullptr || (want_cols && fused_cols)) {
+      GroupNormBwdArgs k = a;
+      if (!want_cols || !fused_cols) k.part_dg = k.part_db = nullptr;
+      GroupNormBwdCtx<T, WT> ctx{plan, k, 0, stream};
+      if (plan.fast) ctx.tpc_log2 = gn_tpc_log2(plan.G, a.D, a.HxW / E);
+      const bool launched =
+          plan.fast ? launch_variant<GroupNormBwdLauncher<T, WT, true>::template At>(ctx)
+                    : launch_variant<GroupNormBwdLauncher<T, WT, false>::template At>(ctx);
+      if (!launched) return (int)hipErrorInvalidConfiguration;
+    }
+  } else if (a.dx != nullptr) {
+    constexpr int DB = 256;
+    const int64_t chunk_elems = (int64_t)DB * kGnChunkPacks * E;
+    const int chunks = (int)((a.L + chunk_elems - 1) / chunk_elems);
+    int64_t grid = a.rows * chunks;
+    if (grid > (1 << 24)) grid = 1 << 24;
+    hipLaunchKernelGGL((gn_bwd_dx_from_sums_kernel<T, WT, DB>), dim3((unsigned)grid), dim3(DB), 0,
+                       stream, (const T*)a.dy, (const T*)a.x, (const WT*)a.mean,
+                       (const WT*)a.rstd, (const WT*)a.gamma, (const float*)a.part_dg,
+                       (const float*)a.part_db, (T*)a.dx, a.rows, shape, chunks);
+  }
+  err = (int)hipGetLastError();
+  if (err != 0 || !want_cols) return err;
   const unsigned gx = (unsigned)((C + kFinalizeCols - 1) / kFinalizeCols);
   hipLaunchKernelGGL((colsum_finalize_kernel<WT>), dim3(gx, 2), dim3(1024), 0, stream,
                      (const float*)a.part_dg, (const float*)a.part_db, (WT*)a.dgamma,

@@ -101,7 +101,7 @@ struct GroupNormBwdArgs {
   void* dx;
   void* dgamma;
   void* dbeta;
-  float* part_dg;  // [N, C] fp32 each, or null when neither dgamma nor dbeta is wanted
+  float* part_dg;  // [N, C] fp32 each; null when the call needs no channel sums
   float* part_db;
   int64_t rows;
   int L, HxW, D, groups;
