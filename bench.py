@@ -294,6 +294,45 @@ def per_op_table(torch, cabi, L, dev, stream, P):
                                                   1, BF, stream)) for s in sets])
     del sets, full
     torch.cuda.empty_cache()
+
+    # softmax over a non-innermost dimension: class scores [256, 21, 128*128] over dim 1
+    O, D, I = 256, 21, 128 * 128
+    sets = [(torch.randn(O, D, I, device=dev).bfloat16(), torch.randn(O, D, I, device=dev).bfloat16(),
+             torch.empty(O, D, I, device=dev, dtype=torch.bfloat16),
+             torch.empty(O, D, I, device=dev, dtype=torch.bfloat16)) for _ in range(4)]
+    add("_softmax dim=1 fwd bf16 [256,21,16384]", 2 * O * D * I * 2,
+        [(lambda s=s: L.mi355x_softmax_strided_fwd(P(s[0]), P(s[2]), O, D, I, BF, BF, 0, stream))
+         for s in sets])
+    add("_softmax dim=1 bwd bf16 [256,21,16384]", 3 * O * D * I * 2,
+        [(lambda s=s: L.mi355x_softmax_strided_bwd(P(s[1]), P(s[2]), P(s[3]), O, D, I, BF, BF, 0,
+                                                   stream)) for s in sets])
+    del sets
+
+    # GroupNorm: a diffusion-UNet block, [64, 320, 64, 64] bf16, 32 groups (rows of 40960 elements)
+    Nb, C, HW, Gr = 64, 320, 64 * 64, 32
+    g = (1 + 0.1 * torch.randn(C, device=dev)).bfloat16()
+    b = (0.1 * torch.randn(C, device=dev)).bfloat16()
+    sets = []
+    for _ in range(3):
+        x = torch.randn(Nb, C, HW, device=dev).bfloat16()
+        s = (x, torch.randn(Nb, C, HW, device=dev).bfloat16(), torch.empty_like(x),
+             torch.empty(Nb, Gr, device=dev, dtype=torch.bfloat16),
+             torch.empty(Nb, Gr, device=dev, dtype=torch.bfloat16), torch.empty_like(x),
+             torch.empty_like(g), torch.empty_like(g))
+        L.mi355x_group_norm_fwd(P(s[0]), P(g), P(b), P(s[2]), P(s[3]), P(s[4]), Nb, C, HW, Gr, 1e-5,
+                                BF, BF, stream)
+        sets.append(s)
+    nws = L.mi355x_group_norm_bwd_workspace_bytes(Nb, C, HW, Gr, BF, BF, 1, 1)
+    ws = torch.empty(max(nws, 1), dtype=torch.uint8, device=dev)
+    add("native_group_norm fwd bf16 [64,320,64,64] g32", 2 * Nb * C * HW * 2 + 2 * C * 2 + 2 * Nb * Gr * 2,
+        [(lambda s=s: L.mi355x_group_norm_fwd(P(s[0]), P(g), P(b), P(s[2]), P(s[3]), P(s[4]), Nb, C,
+                                              HW, Gr, 1e-5, BF, BF, stream)) for s in sets])
+    add("native_group_norm bwd bf16 [64,320,64,64] g32", 3 * Nb * C * HW * 2 + 3 * C * 2 + 2 * Nb * Gr * 2,
+        [(lambda s=s: L.mi355x_group_norm_bwd(P(s[1]), P(s[0]), P(s[3]), P(s[4]), P(g), P(s[5]),
+                                              P(s[6]), P(s[7]), P(ws), nws, Nb, C, HW, Gr, BF, BF,
+                                              stream)) for s in sets])
+    del sets
+    torch.cuda.empty_cache()
     return rows
 
 

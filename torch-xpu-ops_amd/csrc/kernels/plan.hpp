@@ -108,9 +108,13 @@ constexpr int default_bpc(OpClass oc, int block) {
 
 // Which (G, V) kernels exist in the library.  Kept in one place so the
 // dispatcher, the planner and the forced-variant check agree.
+constexpr bool is_group_class(OpClass oc) { return oc == OC_GROUP_FWD || oc == OC_GROUP_BWD; }
+
 constexpr bool variant_built(OpClass oc, int esize, int G, int V, bool fast) {
-  if (G < kMinG || G > kMaxG || (G & (G - 1)) || V < 1 || V > kMaxV || (V & (V - 1)))
-    return false;
+  if (G < kMinG || G > kMaxG || (G & (G - 1)) || V < 1 || V > kMaxV) return false;
+  // GroupNorm rows that need all 1024 lanes take exactly the packs they have
+  // (a 40960-element bf16 row is 5 packs a lane, not 8): V need not be a power of two
+  if (V & (V - 1)) return is_group_class(oc) && fast && G == kMaxG && V <= v_max(oc, esize, G);
   if (V > v_max(oc, esize, G)) return false;
   if (!fast) return V == v_pref(oc, esize);
 #ifdef ROWNORM_TUNE_WIDE
@@ -150,6 +154,8 @@ inline int make_plan(OpClass oc, int64_t M, int64_t N, int esize, int num_cus, c
       V = ov.V;
     } else {
       V = pow2_ceil((packs + G - 1) / G);
+      if (is_group_class(oc) && p.fast && G == kMaxG && (packs + G - 1) / G <= kMaxV)
+        V = (int)((packs + G - 1) / G);
       if (!p.fast && V < v_pref(oc, esize)) V = v_pref(oc, esize);
     }
     const bool holds = (int64_t)G * V >= packs;
@@ -201,8 +207,8 @@ inline int make_plan(OpClass oc, int64_t M, int64_t N, int esize, int num_cus, c
 //
 // A group of TX * TY threads owns one tile: TX lanes along `inner` (one 16-byte
 // pack each) by TY threads along D, each holding V packs, so the registers
-// cover D <= TY * V rows.  The rule: V = 8 packs a lane (fewer when D is
-// smaller; 4 for the 16-bit backward of D <= 32), TY = the power of two that then covers D, and TX = as many lanes
+// cover D <= TY * V rows.  The rule: at most 8 packs a lane (4 for the 16-bit
+// backward of D <= 32), TY = the power of two that then covers D, V = ceil(D / TY), and TX = as many lanes
 // as a row of `inner` has packs, capped so that a group is one wavefront where
 // that leaves at least 8 lanes (128-byte segments) per row, and 256 threads
 // otherwise.  A group of one wavefront reduces with shuffles alone.  D beyond
@@ -234,12 +240,16 @@ inline int make_strided_plan(bool backward, int64_t outer, int64_t D, int64_t in
   p.block = kStridedBlock;
   if (num_cus <= 0) num_cus = 256;
   const int px = packs >= 64 ? 64 : pow2_ceil(packs);  // lanes a row of `inner` can use
-  int V = ov.V > 0 ? ov.V : (D >= kStridedMaxV ? kStridedMaxV : pow2_ceil(D));
-  // measured: the 16-bit backward (two packed rows per lane) runs faster with 4
-  // packs a lane while a wavefront still covers D
-  if (ov.V == 0 && backward && esize == 2 && D > 4 && D <= 32) V = 4;
-  if (V < 1 || V > kStridedMaxV || (V & (V - 1))) return -5;
-  const int64_t ty_need = pow2_ceil((D + V - 1) / V);
+  // packs a lane may hold: 8, or 4 for the 16-bit backward (two packed rows per
+  // lane) while a wavefront still covers D -- measured faster
+  int vcap = kStridedMaxV;
+  if (backward && esize == 2 && D > 4 && D <= 32) vcap = 4;
+  if (ov.V > 0) vcap = ov.V;
+  if (vcap < 1 || vcap > kStridedMaxV) return -5;
+  // TY = the power of two that covers D with at most vcap rows a thread; V = the
+  // rows a thread then really has (not rounded up: D = 21 is 4 x 6, not 4 x 8)
+  const int64_t ty_need = pow2_ceil((D + vcap - 1) / vcap);
+  int V = ov.V > 0 ? ov.V : (int)((D + ty_need - 1) / ty_need);
   int TX = 0, TY = 0;
   // rows are never cut below 4 lanes (64 bytes) to make room for a larger D
   const int ty_max = kStridedBlock / (px < 4 ? px : 4);
@@ -266,7 +276,7 @@ inline int make_strided_plan(bool backward, int64_t outer, int64_t D, int64_t in
     // one group per workgroup; few lanes along inner, fewer still while the
     // problem has less than two workgroups per compute unit
     TX = px < 8 ? px : 8;
-    while (TX > 2 && outer * ((packs + TX - 1) / TX) < 2 * (int64_t)num_cus) TX >>= 1;
+    while (TX > 4 && outer * ((packs + TX - 1) / TX) < 2 * (int64_t)num_cus) TX >>= 1;
     TY = kStridedBlock / TX;
     V = 0;
   }

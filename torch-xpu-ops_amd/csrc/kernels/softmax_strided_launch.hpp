@@ -17,7 +17,11 @@ bool launch_strided_fwd_f(const StridedPlan& p, const SoftmaxStridedFwdArgs& a, 
   switch (p.V) {
     case 1: launch_strided_fwd_v<TI, TO, 1, FAST>(p, a, s); return true;
     case 2: launch_strided_fwd_v<TI, TO, 2, FAST>(p, a, s); return true;
+    case 3: launch_strided_fwd_v<TI, TO, 3, FAST>(p, a, s); return true;
     case 4: launch_strided_fwd_v<TI, TO, 4, FAST>(p, a, s); return true;
+    case 5: launch_strided_fwd_v<TI, TO, 5, FAST>(p, a, s); return true;
+    case 6: launch_strided_fwd_v<TI, TO, 6, FAST>(p, a, s); return true;
+    case 7: launch_strided_fwd_v<TI, TO, 7, FAST>(p, a, s); return true;
     case 8: launch_strided_fwd_v<TI, TO, 8, FAST>(p, a, s); return true;
   }
   return false;
@@ -52,7 +56,11 @@ bool launch_strided_bwd_f(const StridedPlan& p, const SoftmaxStridedBwdArgs& a, 
   switch (p.V) {
     case 1: launch_strided_bwd_v<TG, TO, 1, FAST>(p, a, s); return true;
     case 2: launch_strided_bwd_v<TG, TO, 2, FAST>(p, a, s); return true;
+    case 3: launch_strided_bwd_v<TG, TO, 3, FAST>(p, a, s); return true;
     case 4: launch_strided_bwd_v<TG, TO, 4, FAST>(p, a, s); return true;
+    case 5: launch_strided_bwd_v<TG, TO, 5, FAST>(p, a, s); return true;
+    case 6: launch_strided_bwd_v<TG, TO, 6, FAST>(p, a, s); return true;
+    case 7: launch_strided_bwd_v<TG, TO, 7, FAST>(p, a, s); return true;
     case 8: launch_strided_bwd_v<TG, TO, 8, FAST>(p, a, s); return true;
   }
   return false;
