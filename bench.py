@@ -71,7 +71,7 @@ def main():
     P = lambda t: ctypes.c_void_p(t.data_ptr()) if t is not None else None  # noqa: E731
     BF, F32 = cabi.BF16, cabi.F32
 
-    # ---- workload: BASELINE config 2 ------------------------------------------------------
+    # ---- workload: benchmark configuration 2 ------------------------------------------------------
     M, N, eps = 16384, 4096, 1e-6
     fwd_bytes = 2 * M * N * 2 + N * 2 + M * 4
     bwd_bytes = 3 * M * N * 2 + M * 4 + 2 * N * 2
@@ -150,7 +150,7 @@ def main():
         "dtype": "bf16",
         "data": "synthetic",
         "config": {"workload": "_fused_rms_norm forward+backward, bf16 [16384, 4096], bf16 weight "
-                               "[4096], eps 1e-6 (BASELINE config 2)",
+                               "[4096], eps 1e-6 (benchmark configuration 2)",
                    "algorithmic_bytes_per_step": fwd_bytes + bwd_bytes,
                    "buffer_sets_rotated": nsets},
         "roofline": {
@@ -196,7 +196,7 @@ def _time_rotating(torch, fns, iters=30, warm=5):
 
 
 def per_op_table(torch, cabi, L, dev, stream, P):
-    """Every op of the family at its BASELINE configuration: avg microseconds per call (HIP events
+    """Every op of the family at its benchmark configuration: avg microseconds per call (HIP events
     over 30 back-to-back calls rotating over buffer sets), algorithmic GB/s, fraction of 8 TB/s."""
     BF, F32 = cabi.BF16, cabi.F32
     rows = []

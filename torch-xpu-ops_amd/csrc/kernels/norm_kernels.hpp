@@ -581,26 +581,25 @@ colsum_finalize_kernel(const float* __restrict__ part0, const float* __restrict_
   if (part == nullptr || out == nullptr) return;  // uniform per workgroup
   const int cq = threadIdx.x % CQ, rl = threadIdx.x / CQ;
   const int col0 = blockIdx.x * kFinalizeCols + cq * 4;
+  // U partial rows per thread are requested before any of them is used, so the
+  // 512 partial rows of a full-machine backward cost one memory round trip
+  constexpr int U = 8;
   float a[4] = {0.0f, 0.0f, 0.0f, 0.0f};
-  float b[4] = {0.0f, 0.0f, 0.0f, 0.0f};
-  int p = rl;
-  for (; p + RL < P; p += 2 * RL) {
-    const Pack<float, 4> v0 = load_row_pack<float, 4, false>(part + (int64_t)p * N, col0, N, true, 0.0f);
-    const Pack<float, 4> v1 =
-        load_row_pack<float, 4, false>(part + (int64_t)(p + RL) * N, col0, N, true, 0.0f);
+  for (int p0 = rl; p0 < P; p0 += U * RL) {
+    Pack<float, 4> v[U];
 #pragma unroll
-    for (int i = 0; i < 4; ++i) {
-      a[i] += v0.get(i);
-      b[i] += v1.get(i);
+    for (int u = 0; u < U; ++u) {
+      const int p = p0 + u * RL;
+      v[u] = load_row_pack<float, 4, false>(part + (int64_t)(p < P ? p : 0) * N, col0, N, p < P,
+                                            0.0f);
     }
-  }
-  if (p < P) {
-    const Pack<float, 4> v0 = load_row_pack<float, 4, false>(part + (int64_t)p * N, col0, N, true, 0.0f);
 #pragma unroll
-    for (int i = 0; i < 4; ++i) a[i] += v0.get(i);
+    for (int u = 0; u < U; ++u)
+#pragma unroll
+      for (int i = 0; i < 4; ++i) a[i] += v[u].get(i);
   }
 #pragma unroll
-  for (int i = 0; i < 4; ++i) tile[rl][cq * 4 + i] = a[i] + b[i];
+  for (int i = 0; i < 4; ++i) tile[rl][cq * 4 + i] = a[i];
   __syncthreads();
   if (threadIdx.x < kFinalizeCols) {
     const int col = blockIdx.x * kFinalizeCols + threadIdx.x;
