@@ -181,7 +181,7 @@ def main():
     print(json.dumps(out))
 
 
-def _time_rotating(torch, fns, iters=30, warm=5):
+def _time_rotating(torch, fns, iters=60, warm=30):
     n = len(fns)
     for i in range(warm):
         fns[i % n]()
@@ -197,7 +197,8 @@ def _time_rotating(torch, fns, iters=30, warm=5):
 
 def per_op_table(torch, cabi, L, dev, stream, P):
     """Every op of the family at its benchmark configuration: avg microseconds per call (HIP events
-    over 30 back-to-back calls rotating over buffer sets), algorithmic GB/s, fraction of 8 TB/s."""
+    over 60 back-to-back calls, after 30 untimed ones, rotating over buffer sets), algorithmic GB/s,
+    fraction of 8 TB/s."""
     BF, F32 = cabi.BF16, cabi.F32
     rows = []
 

@@ -67,7 +67,7 @@ __device__ __forceinline__ float gn_weight(const WT* w, int ch, float dflt) {
 
 // ---------------------------------------------------------------------------
 // Forward, row resident in registers.  Statistics as in the LayerNorm kernel:
-// mean0 = sum(x)/L, centred sums over the registers, mean = mean0 + s1/L,
+// a centre mean0, centred sums over the registers, mean = mean0 + s1/L,
 // var = (s2 - s1*s1/L)/L; y uses (x - mean0) - s1/L so that a constant row
 // gives beta bit for bit.
 template <class T, class WT, int G, int V, int BLOCK, bool UNIFORM>
@@ -94,13 +94,24 @@ gn_fwd_resident_kernel(const T* __restrict__ x, const WT* __restrict__ gamma,
 #pragma unroll
     for (int c = 0; c < V; ++c)
       xp[c] = row_load<T, E, true, UNIFORM>(xr, (c * G + lane) * E, s.L, ok, 0.0f);
-    float acc0[1] = {0.0f};
+    // centre of the sums: fp32 rows take the row mean (a reduction round of its
+    // own, exact for any data); 16-bit rows take the median of the row's first
+    // three elements, which every lane reads for itself, so the statistics need
+    // one round (see the LayerNorm forward for the error argument)
+    float mean0;
+    if constexpr (sizeof(T) == 2) {
+      const Pack<T, E> head = load_row_pack<T, E, false>(xr, 0, s.L, true, 0.0f);
+      const float a = head.get(0), b = head.get(1), c3 = head.get(2);
+      mean0 = fmaxf(fminf(a, b), fminf(fmaxf(a, b), c3));
+    } else {
+      float acc0[1] = {0.0f};
 #pragma unroll
-    for (int c = 0; c < V; ++c)
+      for (int c = 0; c < V; ++c)
 #pragma unroll
-      for (int i = 0; i < E; ++i) acc0[0] += xp[c].get(i);
-    group_allreduce<G, BLOCK, 1, SumOp>(acc0, red, phase);
-    const float mean0 = acc0[0] / fL;
+        for (int i = 0; i < E; ++i) acc0[0] += xp[c].get(i);
+      group_allreduce<G, BLOCK, 1, SumOp>(acc0, red, phase);
+      mean0 = acc0[0] / fL;
+    }
     float acc[2] = {0.0f, 0.0f};
     auto centred_sums = [&](auto masked) {
       constexpr bool MASKED = decltype(masked)::value;
