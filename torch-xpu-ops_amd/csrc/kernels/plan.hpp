@@ -112,9 +112,13 @@ constexpr bool is_group_class(OpClass oc) { return oc == OC_GROUP_FWD || oc == O
 
 constexpr bool variant_built(OpClass oc, int esize, int G, int V, bool fast) {
   if (G < kMinG || G > kMaxG || (G & (G - 1)) || V < 1 || V > kMaxV) return false;
-  // GroupNorm rows that need all 1024 lanes take exactly the packs they have
-  // (a 40960-element bf16 row is 5 packs a lane, not 8): V need not be a power of two
-  if (V & (V - 1)) return is_group_class(oc) && fast && G == kMaxG && V <= v_max(oc, esize, G);
+  // GroupNorm rows take the packs they have, not the next power of two (a
+  // 40960-element bf16 row is 1024 lanes x 5 packs, not x 8): 3 or 5 packs a
+  // lane from one wavefront up, anything up to the budget at 1024 lanes
+  if (V & (V - 1)) {
+    if (!is_group_class(oc) || !fast || V > v_max(oc, esize, G)) return false;
+    return G == kMaxG || (G >= 64 && (V == 3 || V == 5));
+  }
   if (V > v_max(oc, esize, G)) return false;
   if (!fast) return V == v_pref(oc, esize);
 #ifdef ROWNORM_TUNE_WIDE
@@ -150,12 +154,26 @@ inline int make_plan(OpClass oc, int64_t M, int64_t N, int esize, int num_cus, c
       if (G < kMinG) G = kMinG;
       if (G > kMaxG) G = kMaxG;
     }
+    // GroupNorm rows of a wavefront or more (measured): about 5 packs a lane on
+    // as few lanes as that allows, and exactly the packs the row has
+    bool group_exact = false;
+    if (is_group_class(oc) && p.fast && ov.G == 0 && ov.V == 0) {
+      int Gg = pow2_ceil((packs + 4) / 5);
+      if (Gg > kMaxG) Gg = kMaxG;
+      if (Gg >= 64) {
+        int Vg = (int)((packs + Gg - 1) / Gg);
+        while (Vg < kMaxV && !variant_built(oc, esize, Gg, Vg, true)) ++Vg;
+        if (variant_built(oc, esize, Gg, Vg, true)) {
+          G = Gg;
+          V = Vg;
+          group_exact = true;
+        }
+      }
+    }
     if (ov.V > 0) {
       V = ov.V;
-    } else {
+    } else if (!group_exact) {
       V = pow2_ceil((packs + G - 1) / G);
-      if (is_group_class(oc) && p.fast && G == kMaxG && (packs + G - 1) / G <= kMaxV)
-        V = (int)((packs + G - 1) / G);
       if (!p.fast && V < v_pref(oc, esize)) V = v_pref(oc, esize);
     }
     const bool holds = (int64_t)G * V >= packs;
