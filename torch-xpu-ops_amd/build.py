@@ -3,6 +3,8 @@
   lib/libmi355x_rownorm.so       HIP kernels + the extern "C" launcher ABI (include/mi355x_rownorm.h)
   lib/libmi355x_rownorm_aten.so  C++ host layer with the ATen operator signatures, registered
                                  as torch.ops.mi355x.*; links libtorch and the library above
+  lib/cabi_check                 torch-free test program that calls the C ABI on hipMalloc memory
+                                 (tests/native/cabi_check.cpp; needs only libdl + the HIP runtime)
 
 Run `python build.py` (or call build_all()).  Objects go to build/ (git-ignored); the .so files
 stay in-tree under lib/ so they travel with the source tree to the GPU machine.
@@ -21,6 +23,8 @@ LIB_DIR = os.path.join(HERE, "lib")
 OBJ_DIR = os.path.join(HERE, "build")
 KERNEL_LIB = os.path.join(LIB_DIR, "libmi355x_rownorm.so")
 HOST_LIB = os.path.join(LIB_DIR, "libmi355x_rownorm_aten.so")
+CABI_CHECK = os.path.join(LIB_DIR, "cabi_check")
+CABI_CHECK_SRC = os.path.join(ROOT, "tests", "native", "cabi_check.cpp")
 
 # Device numerics mirror the reference's flags (cmake/BuildFlags.cmake:111-160 there): no
 # fast-math, FMA contraction on, correctly rounded fp32 division and square root (hipcc's
@@ -79,10 +83,22 @@ def build_host(out=HOST_LIB, verbose=False):
     return out
 
 
+def build_cabi_check(out=CABI_CHECK, verbose=False):
+    """The torch-free caller of the C ABI (host code only: hipcc is used as the C++ compiler that
+    knows where the HIP runtime headers and library are)."""
+    msg = _run(["hipcc", "-O2", "-std=c++17", "-Wall", "-Wno-unused-command-line-argument",
+                "-D__HIP_PLATFORM_AMD__", "-x", "c++", CABI_CHECK_SRC, "-I/opt/rocm/include",
+                "-L/opt/rocm/lib", "-lamdhip64", "-ldl", "-Wl,-rpath,/opt/rocm/lib", "-o", out])
+    if verbose and msg.strip():
+        print(msg)
+    return out
+
+
 def build_all(verbose=False):
     build_kernels(verbose=verbose)
     build_host(verbose=verbose)
-    return KERNEL_LIB, HOST_LIB
+    build_cabi_check(verbose=verbose)
+    return KERNEL_LIB, HOST_LIB, CABI_CHECK
 
 
 if __name__ == "__main__":
