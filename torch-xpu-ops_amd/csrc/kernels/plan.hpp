@@ -60,7 +60,9 @@ constexpr int v_max(OpClass oc, int esize, int G) {
   switch (oc) {
     case OC_NORM_FWD: v = esize == 4 ? 16 : 8; break;
     case OC_NORM_BWD: v = esize == 4 ? 8 : 4; break;
-    case OC_SOFTMAX_FWD: v = esize == 4 ? 16 : 8; break;
+    // the forward keeps long rows in storage format: 16 packs a lane at any
+    // G (a 131072-element 16-bit row, a 65536-element fp32 row)
+    case OC_SOFTMAX_FWD: return 16;
     case OC_SOFTMAX_BWD: v = esize == 4 ? 16 : 8; break;
     // GroupNorm lanes hold the row (and dY) only, no weights or column sums, so
     // 16-bit rows keep 8 packs a lane at 1024 lanes (128 VGPRs); fp32 rows halve
@@ -116,10 +118,16 @@ constexpr bool variant_built(OpClass oc, int esize, int G, int V, bool fast) {
   // 40960-element bf16 row is 1024 lanes x 5 packs, not x 8): 3 or 5 packs a
   // lane from one wavefront up, anything up to the budget at 1024 lanes
   if (V & (V - 1)) {
-    if (!is_group_class(oc) || !fast || V > v_max(oc, esize, G)) return false;
+    if (!fast || V > v_max(oc, esize, G)) return false;
+    // softmax rows that need all 1024 lanes (vocabulary-sized) likewise
+    if (oc == OC_SOFTMAX_FWD || oc == OC_SOFTMAX_BWD) return G == kMaxG;
+    if (!is_group_class(oc)) return false;
     return G == kMaxG || (G >= 64 && (V == 3 || V == 5));
   }
   if (V > v_max(oc, esize, G)) return false;
+  // ragged rows: the general kernels exist for the preferred packs per lane only;
+  // longer ragged rows take the multi-pass kernels (measured faster for softmax
+  // at vocabulary sizes such as 50257 than a general kernel with more packs)
   if (!fast) return V == v_pref(oc, esize);
 #ifdef ROWNORM_TUNE_WIDE
   return true;
@@ -174,6 +182,10 @@ inline int make_plan(OpClass oc, int64_t M, int64_t N, int esize, int num_cus, c
       V = ov.V;
     } else if (!group_exact) {
       V = pow2_ceil((packs + G - 1) / G);
+      const int64_t v_exact = (packs + G - 1) / G;
+      if ((oc == OC_SOFTMAX_FWD || oc == OC_SOFTMAX_BWD) && p.fast && G == kMaxG &&
+          v_exact <= kMaxV && variant_built(oc, esize, G, (int)v_exact, true))
+        V = (int)v_exact;
       if (!p.fast && V < v_pref(oc, esize)) V = v_pref(oc, esize);
     }
     const bool holds = (int64_t)G * V >= packs;

@@ -43,6 +43,12 @@ __device__ __forceinline__ float row_exp(float v) {
     return __expf(v);
 }
 
+// Packs a thread of the multi-pass kernels requests before using the first.
+constexpr int kStreamUnroll = 2;
+
+// Rows of more than this many elements a lane are kept in storage format.
+constexpr int kSoftmaxWideElems = 32;
+
 struct MaskRef {
   const uint8_t* data;  // one byte per element, non-zero = masked out
   uint32_t div, mod;    // mask row of data row r: (r / div) * stride + r % mod
@@ -101,6 +107,51 @@ softmax_fwd_resident_kernel(const TI* __restrict__ x, TO* __restrict__ y, MaskRe
 #pragma unroll
     for (int c = 0; c < V; ++c)
       xp[c] = row_load<TI, E, true, FAST>(xr, (c * G + lane) * E, N, ok, -INFINITY);
+    if constexpr (V * E > kSoftmaxWideElems) {
+      // Long rows (a vocabulary-sized row is 16 packs a lane): the row stays in
+      // storage format and each of the three passes widens it again; softmax
+      // then evaluates exp twice per element, log_softmax still once.
+      if constexpr (MASKED) {
+        const uint8_t* mrow = mask_row_ptr(mask, rowc, N);
+#pragma unroll
+        for (int c = 0; c < V; ++c) {
+          const Pack<uint8_t, E> mk = load_mask_pack<E, FAST>(mrow, (c * G + lane) * E, N, ok);
+#pragma unroll
+          for (int i = 0; i < E; ++i)
+            if (mk.v[i]) xp[c].set(i, -INFINITY);
+        }
+      }
+      float mx[1] = {-INFINITY};
+#pragma unroll
+      for (int c = 0; c < V; ++c)
+#pragma unroll
+        for (int i = 0; i < E; ++i) mx[0] = fmaxf(mx[0], xp[c].get(i));
+      group_allreduce<G, BLOCK, 1, MaxOp>(mx, red, phase);
+      const float m = mx[0];
+      float sum[1] = {0.0f};
+#pragma unroll
+      for (int c = 0; c < V; ++c) {
+        keep_packed(xp[c]);
+#pragma unroll
+        for (int i = 0; i < E; ++i) sum[0] += row_exp<PRECISE>(xp[c].get(i) - m);
+      }
+      group_allreduce<G, BLOCK, 1, SumOp>(sum, red, phase);
+      const float k = is_log ? logf(sum[0]) : 1.0f / sum[0];
+      const bool zero_row = is_safe && m == -INFINITY;
+#pragma unroll
+      for (int c = 0; c < V; ++c) {
+        keep_packed(xp[c]);
+        Pack<TO, E> o;
+#pragma unroll
+        for (int i = 0; i < E; ++i) {
+          const float d = xp[c].get(i) - m;
+          const float v = is_log ? d - k : row_exp<PRECISE>(d) * k;
+          o.set(i, zero_row ? 0.0f : v);
+        }
+        row_store<TO, E, true, FAST>(yr, (c * G + lane) * E, N, ok, o);
+      }
+      continue;
+    }
     float xf[V][E];
 #pragma unroll
     for (int c = 0; c < V; ++c)
@@ -158,7 +209,12 @@ softmax_fwd_resident_kernel(const TI* __restrict__ x, TO* __restrict__ y, MaskRe
   }
 }
 
-// Rows too wide for registers: one workgroup per row, three streaming passes.
+// Rows too wide for registers: one workgroup per row, two passes over the row.
+// The first keeps a running maximum and a running sum of exp(x - maximum) per
+// thread, rescaling the sum whenever a pack raises the maximum; the threads'
+// pairs are merged with s * exp(m - M) after the block maximum M is known.  The
+// second pass writes the output.  (The reference's SoftmaxForwardKernelFunctor,
+// SoftMaxKernels.cpp:546-684, walks the row three times: max, sum, output.)
 template <class TI, class TO, int BLOCK, bool MASKED>
 __global__ void __launch_bounds__(BLOCK)
 softmax_fwd_stream_kernel(const TI* __restrict__ x, TO* __restrict__ y, MaskRef mask, int64_t M,
@@ -173,48 +229,77 @@ softmax_fwd_stream_kernel(const TI* __restrict__ x, TO* __restrict__ y, MaskRef 
   for (int64_t row = blockIdx.x; row < M; row += gridDim.x) {
     const TI* xr = x + row * (int64_t)N;
     TO* yr = y + row * (int64_t)N;
-    const uint8_t* mrow =
-        MASKED ? mask_row_ptr(mask, row, N) : nullptr;
-    // element i of pack pk, with the mask applied
+    const uint8_t* mrow = MASKED ? mask_row_ptr(mask, row, N) : nullptr;
+    // element i of a pack, with the mask applied
     auto masked_value = [&](const Pack<TI, E>& p, const Pack<uint8_t, E>& mk, int i) {
       const float v = p.get(i);
       if constexpr (MASKED) return mk.v[i] ? -INFINITY : v;
       return v;
     };
-    float mx[1] = {-INFINITY};
-    for (int pk = threadIdx.x; pk < npacks; pk += BLOCK) {
-      const Pack<TI, E> p = load_row_pack<TI, E, false>(xr, pk * E, N, true, -INFINITY);
-      Pack<uint8_t, E> mk;
-      if constexpr (MASKED) mk = load_mask_pack<E, false>(mrow, pk * E, N, true);
+    float m_t = -INFINITY, s_t = 0.0f;
+    // kStreamUnroll packs a thread are requested before the first is used
+    for (int pk0 = threadIdx.x; pk0 < npacks; pk0 += kStreamUnroll * BLOCK) {
+      Pack<TI, E> pv[kStreamUnroll];
+      Pack<uint8_t, E> mv[kStreamUnroll];
 #pragma unroll
-      for (int i = 0; i < E; ++i) mx[0] = fmaxf(mx[0], masked_value(p, mk, i));
+      for (int u = 0; u < kStreamUnroll; ++u) {
+        const int pk = pk0 + u * BLOCK;
+        pv[u] = load_row_pack<TI, E, false>(xr, pk * E, N, pk < npacks, -INFINITY);
+        if constexpr (MASKED) mv[u] = load_mask_pack<E, false>(mrow, pk * E, N, pk < npacks);
+      }
+#pragma unroll
+      for (int u = 0; u < kStreamUnroll; ++u) {
+        float v[E];
+        float pm = -INFINITY;
+#pragma unroll
+        for (int i = 0; i < E; ++i) {
+          v[i] = masked_value(pv[u], mv[u], i);
+          pm = fmaxf(pm, v[i]);
+        }
+        if (pm > m_t) {  // a new maximum: bring the sum so far to the new reference
+          s_t *= row_exp<PRECISE>(m_t - pm);
+          m_t = pm;
+        }
+        if (m_t > -INFINITY) {
+#pragma unroll
+          for (int i = 0; i < E; ++i) s_t += row_exp<PRECISE>(v[i] - m_t);
+        } else {
+          // nothing finite yet: a NaN element must still poison the row
+#pragma unroll
+          for (int i = 0; i < E; ++i) s_t += (v[i] != v[i]) ? v[i] : 0.0f;
+        }
+      }
     }
+    float mx[1] = {m_t};
     group_allreduce<BLOCK, BLOCK, 1, MaxOp>(mx, red, phase);
     const float m = mx[0];
-    float sum[1] = {0.0f};
-    for (int pk = threadIdx.x; pk < npacks; pk += BLOCK) {
-      const Pack<TI, E> p = load_row_pack<TI, E, false>(xr, pk * E, N, true, -INFINITY);
-      Pack<uint8_t, E> mk;
-      if constexpr (MASKED) mk = load_mask_pack<E, false>(mrow, pk * E, N, true);
-#pragma unroll
-      for (int i = 0; i < E; ++i) sum[0] += row_exp<PRECISE>(masked_value(p, mk, i) - m);
-    }
+    // exp(-inf - m) = 0 drops threads that saw nothing finite; a row with no
+    // finite element at all gives exp(NaN) = NaN, like the three-pass form
+    float sum[1] = {s_t == 0.0f ? (m == -INFINITY ? NAN : 0.0f) : s_t * row_exp<PRECISE>(m_t - m)};
     group_allreduce<BLOCK, BLOCK, 1, SumOp>(sum, red, phase);
     const float k = is_log ? logf(sum[0]) : 1.0f / sum[0];
     const bool zero_row = is_safe && m == -INFINITY;
-    for (int pk = threadIdx.x; pk < npacks; pk += BLOCK) {
-      const int e0 = pk * E;
-      const Pack<TI, E> p = load_row_pack<TI, E, true>(xr, e0, N, true, -INFINITY);
-      Pack<uint8_t, E> mk;
-      if constexpr (MASKED) mk = load_mask_pack<E, false>(mrow, e0, N, true);
-      Pack<TO, E> o;
+    for (int pk0 = threadIdx.x; pk0 < npacks; pk0 += kStreamUnroll * BLOCK) {
+      Pack<TI, E> pv[kStreamUnroll];
+      Pack<uint8_t, E> mv[kStreamUnroll];
 #pragma unroll
-      for (int i = 0; i < E; ++i) {
-        const float d = masked_value(p, mk, i) - m;
-        const float v = is_log ? d - k : row_exp<PRECISE>(d) * k;
-        o.set(i, zero_row ? 0.0f : v);
+      for (int u = 0; u < kStreamUnroll; ++u) {
+        const int pk = pk0 + u * BLOCK;
+        pv[u] = load_row_pack<TI, E, true>(xr, pk * E, N, pk < npacks, -INFINITY);
+        if constexpr (MASKED) mv[u] = load_mask_pack<E, false>(mrow, pk * E, N, pk < npacks);
       }
-      store_row_pack<TO, E, true>(yr, e0, N, true, o);
+#pragma unroll
+      for (int u = 0; u < kStreamUnroll; ++u) {
+        const int pk = pk0 + u * BLOCK;
+        Pack<TO, E> o;
+#pragma unroll
+        for (int i = 0; i < E; ++i) {
+          const float d = masked_value(pv[u], mv[u], i) - m;
+          const float v = is_log ? d - k : row_exp<PRECISE>(d) * k;
+          o.set(i, zero_row ? 0.0f : v);
+        }
+        store_row_pack<TO, E, true>(yr, pk * E, N, pk < npacks, o);
+      }
     }
   }
 }
@@ -299,6 +384,7 @@ __global__ void __launch_bounds__(BLOCK)
 softmax_bwd_stream_kernel(const TG* __restrict__ grad, const TG* __restrict__ y,
                           TO* __restrict__ gi, MaskRef mask, int64_t M, int N, int flags) {
   constexpr int E = elems_per_pack<TG>::value;
+  constexpr int U = kStreamUnroll;
   constexpr bool PRECISE = sizeof(TO) == 4 && sizeof(TG) == 4;
   __shared__ float red[reduce_lds_floats<BLOCK, BLOCK, 1>::value];
   int phase = 0;
@@ -308,43 +394,63 @@ softmax_bwd_stream_kernel(const TG* __restrict__ grad, const TG* __restrict__ y,
     const TG* gr = grad + row * (int64_t)N;
     const TG* yr = y + row * (int64_t)N;
     TO* outr = gi + row * (int64_t)N;
-    const uint8_t* mrow =
-        MASKED ? mask_row_ptr(mask, row, N) : nullptr;
+    const uint8_t* mrow = MASKED ? mask_row_ptr(mask, row, N) : nullptr;
     auto saved_output = [&](const Pack<TG, E>& p, const Pack<uint8_t, E>& mk, int i) {
       const float v = p.get(i);
       if constexpr (MASKED) return mk.v[i] ? 0.0f : v;
       return v;
     };
+    // first pass: sum(grad) for log_softmax (y is not read), sum(y * grad) otherwise
     float sum[1] = {0.0f};
-    for (int pk = threadIdx.x; pk < npacks; pk += BLOCK) {
-      const Pack<TG, E> pg = load_row_pack<TG, E, false>(gr, pk * E, N, true, 0.0f);
-      if (is_log) {
+    for (int pk0 = threadIdx.x; pk0 < npacks; pk0 += U * BLOCK) {
+      Pack<TG, E> pg[U], py[U];
+      Pack<uint8_t, E> mk[U];
 #pragma unroll
-        for (int i = 0; i < E; ++i) sum[0] += pg.get(i);
-      } else {
-        const Pack<TG, E> py = load_row_pack<TG, E, false>(yr, pk * E, N, true, 0.0f);
-        Pack<uint8_t, E> mk;
-        if constexpr (MASKED) mk = load_mask_pack<E, false>(mrow, pk * E, N, true);
+      for (int u = 0; u < U; ++u) {
+        const int pk = pk0 + u * BLOCK;
+        pg[u] = load_row_pack<TG, E, false>(gr, pk * E, N, pk < npacks, 0.0f);
+        if (!is_log) {
+          py[u] = load_row_pack<TG, E, false>(yr, pk * E, N, pk < npacks, 0.0f);
+          if constexpr (MASKED) mk[u] = load_mask_pack<E, false>(mrow, pk * E, N, pk < npacks);
+        }
+      }
 #pragma unroll
-        for (int i = 0; i < E; ++i) sum[0] = fmaf(saved_output(py, mk, i), pg.get(i), sum[0]);
+      for (int u = 0; u < U; ++u) {
+        if (is_log) {
+#pragma unroll
+          for (int i = 0; i < E; ++i) sum[0] += pg[u].get(i);
+        } else {
+#pragma unroll
+          for (int i = 0; i < E; ++i)
+            sum[0] = fmaf(saved_output(py[u], mk[u], i), pg[u].get(i), sum[0]);
+        }
       }
     }
     group_allreduce<BLOCK, BLOCK, 1, SumOp>(sum, red, phase);
     const float s = sum[0];
-    for (int pk = threadIdx.x; pk < npacks; pk += BLOCK) {
-      const int e0 = pk * E;
-      const Pack<TG, E> pg = load_row_pack<TG, E, true>(gr, e0, N, true, 0.0f);
-      const Pack<TG, E> py = load_row_pack<TG, E, true>(yr, e0, N, true, 0.0f);
-      Pack<uint8_t, E> mk;
-      if constexpr (MASKED) mk = load_mask_pack<E, false>(mrow, e0, N, true);
-      Pack<TO, E> o;
+    for (int pk0 = threadIdx.x; pk0 < npacks; pk0 += U * BLOCK) {
+      Pack<TG, E> pg[U], py[U];
+      Pack<uint8_t, E> mk[U];
 #pragma unroll
-      for (int i = 0; i < E; ++i) {
-        const float yv = saved_output(py, mk, i);
-        const float v = is_log ? pg.get(i) - row_exp<PRECISE>(yv) * s : yv * (pg.get(i) - s);
-        o.set(i, v);
+      for (int u = 0; u < U; ++u) {
+        const int pk = pk0 + u * BLOCK;
+        pg[u] = load_row_pack<TG, E, true>(gr, pk * E, N, pk < npacks, 0.0f);
+        py[u] = load_row_pack<TG, E, true>(yr, pk * E, N, pk < npacks, 0.0f);
+        if constexpr (MASKED) mk[u] = load_mask_pack<E, false>(mrow, pk * E, N, pk < npacks);
       }
-      store_row_pack<TO, E, true>(outr, e0, N, true, o);
+#pragma unroll
+      for (int u = 0; u < U; ++u) {
+        const int pk = pk0 + u * BLOCK;
+        Pack<TO, E> o;
+#pragma unroll
+        for (int i = 0; i < E; ++i) {
+          const float yv = saved_output(py[u], mk[u], i);
+          const float v =
+              is_log ? pg[u].get(i) - row_exp<PRECISE>(yv) * s : yv * (pg[u].get(i) - s);
+          o.set(i, v);
+        }
+        store_row_pack<TO, E, true>(outr, pk * E, N, pk < npacks, o);
+      }
     }
   }
 }
