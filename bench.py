@@ -296,6 +296,23 @@ def per_op_table(torch, cabi, L, dev, stream, P):
     del sets, full
     torch.cuda.empty_cache()
 
+    # log_softmax over a vocabulary, as cross_entropy calls it: Llama-2 (32000) and Llama-3
+    # (128256) vocabularies, bf16 logits
+    for R, N in ((8192, 32000), (4096, 128256)):
+        sets = []
+        for _ in range(2):
+            xv = torch.randn(R, N, device=dev).bfloat16()
+            sets.append((xv, torch.randn(R, N, device=dev).bfloat16(), torch.empty_like(xv),
+                         torch.empty_like(xv)))
+        add("_log_softmax fwd bf16 [%d,%d]" % (R, N), 2 * R * N * 2,
+            [(lambda s=s: L.mi355x_softmax_fwd(P(s[0]), P(s[2]), R, N, BF, BF, 1, stream))
+             for s in sets])
+        add("_log_softmax bwd bf16 [%d,%d]" % (R, N), 3 * R * N * 2,
+            [(lambda s=s: L.mi355x_softmax_bwd(P(s[1]), P(s[2]), P(s[3]), R, N, BF, BF, 1, stream))
+             for s in sets])
+        del sets
+        torch.cuda.empty_cache()
+
     # softmax over a non-innermost dimension: class scores [256, 21, 128*128] over dim 1
     O, D, I = 256, 21, 128 * 128
     sets = [(torch.randn(O, D, I, device=dev).bfloat16(), torch.randn(O, D, I, device=dev).bfloat16(),

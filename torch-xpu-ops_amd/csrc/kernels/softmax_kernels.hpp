@@ -47,7 +47,7 @@ __device__ __forceinline__ float row_exp(float v) {
 constexpr int kStreamUnroll = 2;
 
 // Rows of more than this many elements a lane are kept in storage format.
-constexpr int kSoftmaxWideElems = 32;
+constexpr int kSoftmaxWideElems = 16;
 
 struct MaskRef {
   const uint8_t* data;  // one byte per element, non-zero = masked out
