@@ -125,37 +125,32 @@ softmax_strided_fwd_kernel(const TI* __restrict__ x, TO* __restrict__ y, int64_t
   for (int64_t t0 = (int64_t)blockIdx.x * NG; t0 < ntiles; t0 += (int64_t)gridDim.x * NG) {
     const StridedTile tile = strided_tile<BLOCK, E>(t0, ntiles, xtiles, D, inner, lay);
     const int ty = tile.ty, TY = tile.TY;
-    float xf[V][E];
+    // the V packs stay in storage format; each pass widens them again (softmax
+    // then evaluates exp twice per element, which measured faster than holding
+    // V * E fp32 values a lane)
+    Pack<TI, E> xp[V];
 #pragma unroll
     for (int k = 0; k < V; ++k) {
       const int d = ty + k * TY;
       const bool ok = tile.valid && d < D;
       const TI* row = x + tile.slab + (int64_t)(ok ? d : 0) * inner;
-      const Pack<TI, E> p = row_load<TI, E, true, FAST>(row, tile.e0, inner, ok, -INFINITY);
-#pragma unroll
-      for (int i = 0; i < E; ++i) xf[k][i] = p.get(i);
+      xp[k] = row_load<TI, E, true, FAST>(row, tile.e0, inner, ok, -INFINITY);
     }
     float mx[E], sum[E];
 #pragma unroll
     for (int i = 0; i < E; ++i) {
       mx[i] = -INFINITY;
 #pragma unroll
-      for (int k = 0; k < V; ++k) mx[i] = fmaxf(mx[i], xf[k][i]);
+      for (int k = 0; k < V; ++k) mx[i] = fmaxf(mx[i], xp[k].get(i));
     }
     column_allreduce<BLOCK, E, MaxOp>(mx, lay, red, phase);
 #pragma unroll
-    for (int i = 0; i < E; ++i) {
-      sum[i] = 0.0f;
+    for (int i = 0; i < E; ++i) sum[i] = 0.0f;
 #pragma unroll
-      for (int k = 0; k < V; ++k) {
-        if (is_log) {
-          xf[k][i] -= mx[i];
-          sum[i] += row_exp<PRECISE>(xf[k][i]);
-        } else {
-          xf[k][i] = row_exp<PRECISE>(xf[k][i] - mx[i]);
-          sum[i] += xf[k][i];
-        }
-      }
+    for (int k = 0; k < V; ++k) {
+      keep_packed(xp[k]);
+#pragma unroll
+      for (int i = 0; i < E; ++i) sum[i] += row_exp<PRECISE>(xp[k].get(i) - mx[i]);
     }
     column_allreduce<BLOCK, E, SumOp>(sum, lay, red, phase);
     float kf[E];
@@ -167,12 +162,14 @@ softmax_strided_fwd_kernel(const TI* __restrict__ x, TO* __restrict__ y, int64_t
     }
 #pragma unroll
     for (int k = 0; k < V; ++k) {
+      keep_packed(xp[k]);
       const int d = ty + k * TY;
       const bool ok = tile.valid && d < D;
       Pack<TO, E> o;
 #pragma unroll
       for (int i = 0; i < E; ++i) {
-        const float v = is_log ? xf[k][i] - kf[i] : xf[k][i] * kf[i];
+        const float dv = xp[k].get(i) - mx[i];
+        const float v = is_log ? dv - kf[i] : row_exp<PRECISE>(dv) * kf[i];
         o.set(i, zero[i] ? 0.0f : v);
       }
       TO* row = y + tile.slab + (int64_t)(ok ? d : 0) * inner;
