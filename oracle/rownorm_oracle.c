@@ -282,7 +282,7 @@ void oracle_safe_softmax_fwd(const float* x, float* y, int64_t rows, int64_t N) 
 /* _masked_softmax over the last dimension; mask is [rows, N] bytes, non-zero
  * = leave the element out.  SoftMaxKernels.cpp:257-272 replaces masked
  * elements by -inf before the max; :331-332 turns a zero sum (every element
- * masked) into NaN. */
+ * masked, or -inf wherever the mask leaves one in) into a NaN row. */
 void oracle_masked_softmax_fwd(const float* x, const uint8_t* mask, float* y,
                                int64_t rows, int64_t N) {
   for (int64_t r = 0; r < rows; ++r) {
@@ -302,7 +302,7 @@ void oracle_masked_softmax_fwd(const float* x, const uint8_t* mask, float* y,
     for (int64_t j = 0; j < N; ++j)
       if (!mr[j]) s += exp((double)xr[j] - m);
     for (int64_t j = 0; j < N; ++j) {
-      if (!any || s == 0)
+      if (!any || s == 0 || m == -INFINITY)
         yr[j] = NAN;
       else
         yr[j] = mr[j] ? 0.0f : (float)(exp((double)xr[j] - m) / s);
@@ -311,7 +311,8 @@ void oracle_masked_softmax_fwd(const float* x, const uint8_t* mask, float* y,
 }
 
 /* _masked_softmax_backward: softmax backward with the saved output read as 0
- * at masked positions (SoftMaxKernels.cpp:991-1001), hence gi = 0 there. */
+ * at masked positions (SoftMaxKernels.cpp:991-1001), hence gi = 0 * (g - s)
+ * there: 0, or NaN when the row's unmasked outputs hold a NaN. */
 void oracle_masked_softmax_bwd(const float* g, const float* y,
                                const uint8_t* mask, float* gi, int64_t rows,
                                int64_t N) {
@@ -324,7 +325,7 @@ void oracle_masked_softmax_bwd(const float* g, const float* y,
     for (int64_t j = 0; j < N; ++j)
       if (!mr[j]) s += (double)yr[j] * (double)gr[j];
     for (int64_t j = 0; j < N; ++j)
-      o[j] = mr[j] ? 0.0f : (float)((double)yr[j] * ((double)gr[j] - s));
+      o[j] = (float)((mr[j] ? 0.0 : (double)yr[j]) * ((double)gr[j] - s));
   }
 }
 

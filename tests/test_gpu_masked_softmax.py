@@ -72,6 +72,27 @@ def test_masked_softmax_fwd_bwd(cabi, oracle, gpu, dtype, shape):
     _check_masked(cabi, oracle, gpu, x, grad, _mask(M, N, g), dtype, "full mask")
 
 
+@pytest.mark.parametrize("dtype", DTYPES, ids=str)
+def test_nan_output_poisons_its_backward_row(cabi, oracle, gpu, dtype):
+    """A row whose unmasked inputs are all -inf comes out NaN, and its backward is NaN at the
+    masked positions too: 0 * (g - NaN), as SoftMaxKernels.cpp:991-1047 evaluates it."""
+    g = gen(43)
+    for (M, N) in ((6, 40), (5, 127), (4, 2048), (3, 4097)):
+        x = (3.0 * torch.randn(M, N, generator=g)).to(dtype)
+        grad = torch.randn(M, N, generator=g).to(dtype)
+        mask = torch.rand(M, N, generator=g) < 0.4
+        x[1] = torch.where(mask[1], x[1], torch.full_like(x[1], float("-inf")))
+        y = cabi.masked_softmax_fwd(x.to(gpu), mask.to(gpu))
+        assert_close(y, oracle.masked_softmax_fwd(to_np32(x), mask.numpy()), dtype, "y")
+        assert bool(torch.isnan(y[1]).all())
+        gi = cabi.masked_softmax_bwd(grad.to(gpu), y, mask.to(gpu))
+        ogi = oracle.masked_softmax_bwd(to_np32(grad), to_np32(y), mask.numpy())
+        assert_close(gi, ogi, dtype, "grad_input")
+        nan = torch.isnan(gi.cpu())
+        assert bool(nan[1].all()) and not bool(nan[[0] + list(range(2, M))].any())
+        assert bool(torch.equal(nan, torch.isnan(torch.from_numpy(ogi))))
+
+
 @pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16], ids=str)
 @pytest.mark.parametrize("T", [8, 33, 128, 257])
 def test_mask_layouts_under_attention_scores(cabi, oracle, gpu, dtype, T):

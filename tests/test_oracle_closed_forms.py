@@ -263,6 +263,14 @@ def test_masked_softmax_is_softmax_of_the_unmasked_elements(oracle):
     full = np.ones((M, N), bool)
     assert np.all(np.isnan(oracle.masked_softmax_fwd(x, full)))
     assert np.all(oracle.masked_softmax_bwd(g, y, full) == 0)
+    # a saved output that holds NaN (every unmasked input was -inf) poisons its whole row, the
+    # masked positions too: 0 * (g - NaN), as SoftMaxKernels.cpp:991-1047 evaluates it
+    xn = x.copy()
+    xn[3, ~mask[3]] = -np.inf
+    yn = oracle.masked_softmax_fwd(xn, mask)
+    assert np.all(np.isnan(yn[3]))
+    gn = oracle.masked_softmax_bwd(g, yn, mask)
+    assert np.all(np.isnan(gn[3])) and np.array_equal(gn[[0, 1, 2]], gi[[0, 1, 2]])
     # masking with the mask equals feeding -inf to the plain softmax
     xm = np.where(mask, -np.inf, x).astype(np.float32)
     np.testing.assert_array_equal(y, oracle.softmax_fwd(xm))
