@@ -175,6 +175,7 @@ def main():
 
     if not args.no_ops:
         out["ops"] = per_op_table(torch, cabi, L, dev, stream, P)
+        out["config5"] = stress_table(torch, cabi, L, dev, stream, P)
     del sets
     if not args.no_cpu:
         out["cpu_baseline"], out["cpu_aten"] = cpu_baselines(torch, M, N, eps, fwd_bytes + bwd_bytes)
@@ -352,6 +353,65 @@ def per_op_table(torch, cabi, L, dev, stream, P):
     del sets
     torch.cuda.empty_cache()
     return rows
+
+
+def stress_table(torch, cabi, L, dev, stream, P):
+    """Benchmark configuration 5 (the correctness configuration: irregular row lengths, every
+    tensor 2 elements into its buffer, so only 8-byte / 4-byte aligned): algorithmic GB/s of every
+    op, fp32 and fp16, forward and backward.  Reported, not held to the bandwidth target."""
+    F32, F16 = cabi.F32, cabi.F16
+    shapes = [(1 << 20, 64), (8192, 127), (8192, 4097), (8192, 5120), (8192, 16384)]
+    out = []
+
+    def off(numel, dtype):
+        buf = torch.empty(numel + 66, dtype=dtype, device=dev)
+        return buf[2:2 + numel]
+
+    for dtype, code, b in ((torch.float32, F32, 4), (torch.float16, F16, 2)):
+        res = {}
+        for (M, N) in shapes:
+            sets = []
+            for _ in range(2):
+                x = off(M * N, dtype).copy_(torch.randn(M * N, device=dev))
+                dy = off(M * N, dtype).copy_(torch.randn(M * N, device=dev))
+                sets.append(dict(x=x, dy=dy, y=off(M * N, dtype), dx=off(M * N, dtype),
+                                 mean=off(M, torch.float32), rstd=off(M, torch.float32),
+                                 dg=off(N, dtype), db=off(N, dtype)))
+            g = off(N, dtype).copy_(1 + 0.1 * torch.randn(N, device=dev))
+            bt = off(N, dtype).copy_(0.1 * torch.randn(N, device=dev))
+            nws = L.mi355x_layer_norm_bwd_workspace_bytes(M, N, code, code, 1, 1)
+            ws = torch.empty(max(nws, 1), dtype=torch.uint8, device=dev)
+            ops = {
+                "native_layer_norm fwd": (2 * M * N * b + 2 * N * b + 8 * M, lambda s: L.mi355x_layer_norm_fwd(
+                    P(s["x"]), P(g), P(bt), P(s["y"]), P(s["mean"]), P(s["rstd"]), M, N, 1e-5, code,
+                    code, stream)),
+                "native_layer_norm bwd": (3 * M * N * b + 8 * M + 3 * N * b, lambda s: L.mi355x_layer_norm_bwd(
+                    P(s["dy"]), P(s["x"]), P(s["mean"]), P(s["rstd"]), P(g), P(s["dx"]), P(s["dg"]),
+                    P(s["db"]), P(ws), nws, M, N, code, code, stream)),
+                "_fused_rms_norm fwd": (2 * M * N * b + N * b + 4 * M, lambda s: L.mi355x_rms_norm_fwd(
+                    P(s["x"]), P(g), P(s["y"]), P(s["rstd"]), M, N, 1e-6, code, code, stream)),
+                "_fused_rms_norm bwd": (3 * M * N * b + 4 * M + 2 * N * b, lambda s: L.mi355x_rms_norm_bwd(
+                    P(s["dy"]), P(s["x"]), P(s["rstd"]), P(g), P(s["dx"]), P(s["dg"]), P(ws), nws, M,
+                    N, code, code, stream)),
+                "_softmax fwd": (2 * M * N * b, lambda s: L.mi355x_softmax_fwd(
+                    P(s["x"]), P(s["y"]), M, N, code, code, 0, stream)),
+                "_softmax bwd": (3 * M * N * b, lambda s: L.mi355x_softmax_bwd(
+                    P(s["dy"]), P(s["y"]), P(s["dx"]), M, N, code, code, 0, stream)),
+                "_log_softmax fwd": (2 * M * N * b, lambda s: L.mi355x_softmax_fwd(
+                    P(s["x"]), P(s["y"]), M, N, code, code, 1, stream)),
+                "_log_softmax bwd": (3 * M * N * b, lambda s: L.mi355x_softmax_bwd(
+                    P(s["dy"]), P(s["y"]), P(s["dx"]), M, N, code, code, 1, stream)),
+            }
+            for name, (nbytes, fn) in ops.items():
+                us = _time_rotating(torch, [(lambda s=s, fn=fn: fn(s)) for s in sets], iters=30,
+                                    warm=10)
+                res.setdefault(name, []).append(round(nbytes / us / 1e3))
+            del sets
+        for name, gbs in res.items():
+            out.append({"op": name, "dtype": "fp32" if b == 4 else "fp16", "GB/s": gbs})
+        torch.cuda.empty_cache()
+    return {"rows_x_N": ["%dx%d" % sh for sh in shapes],
+            "layout": "every tensor starts 2 elements into its buffer", "ops": out}
 
 
 def cpu_baselines(torch, M, N, eps, step_bytes):

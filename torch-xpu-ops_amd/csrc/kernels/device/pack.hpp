@@ -95,39 +95,100 @@ __device__ __forceinline__ void keep_packed(Pack<T, E>& p) {
   }
 }
 
-// Loads the pack that starts at element `e0` of a row of `n` elements.  A pack
-// that lies wholly inside the row is one 128-bit load; the (at most one) pack
-// that straddles the end of the row is read element by element and padded with
-// `fill`; a pack wholly outside the row is all `fill`.
+// Loads the pack that starts at element `e0` of a row whose elements are
+// [lo, n) of `row`.  A pack that lies wholly inside the row is one 128-bit load;
+// a pack that straddles either end of the row is read element by element and
+// padded with `fill`; a pack wholly outside the row is all `fill`.  Nothing
+// outside [lo, n) is touched.  The element loads go to clamped addresses, all
+// valid, so they are independent of one another and of the padding: E requests
+// in flight and one wait, not a load-and-wait per element.
 template <class T, int E, bool STREAM>
 __device__ __forceinline__ Pack<T, E> load_row_pack(const T* row, int e0, int n, bool row_ok,
-                                                    float fill) {
-  if (row_ok && e0 + E <= n) {
+                                                    float fill, int lo = 0) {
+  if (row_ok && e0 >= lo && e0 + E <= n) {
     return STREAM ? Pack<T, E>::load_stream(row + e0) : Pack<T, E>::load(row + e0);
   }
   Pack<T, E> r = Pack<T, E>::splat(fill);
-  if (row_ok && e0 < n) {
+  if (row_ok && e0 < n && e0 + E > lo) {
+    T t[E];
+#pragma unroll
+    for (int i = 0; i < E; ++i) {
+      int j = e0 + i;
+      j = j < lo ? lo : j;
+      j = j >= n ? n - 1 : j;
+      t[i] = row[j];
+    }
 #pragma unroll
     for (int i = 0; i < E; ++i)
-      if (e0 + i < n) r.v[i] = row[e0 + i];
+      if (e0 + i >= lo && e0 + i < n) r.v[i] = t[i];
   }
   return r;
 }
 
+// The same for a row seen through a window whose packs are 16-byte aligned
+// (see window_head below), in two steps.  A pack that holds any element of the
+// row lies in that element's page, so it is read whole: one unconditional
+// 128-bit load, like the fast kernels', and a lane's loads are straight-line
+// code.  trim_window_pack then replaces the elements outside [lo, n) by `fill`;
+// callers run it over their packs after all of them have been requested.
+// `win` must be the window of a readable row even when `ok` is false (callers
+// clamp the row index); lo < E.
+template <class T, int E, bool STREAM>
+__device__ __forceinline__ Pack<T, E> load_window_pack(const T* win, int e0, int n, bool ok,
+                                                       float fill) {
+  const bool inb = ok && e0 < n;
+  const T* p = win + (inb ? e0 : 0);
+  Pack<T, E> r = STREAM ? Pack<T, E>::load_stream(p) : Pack<T, E>::load(p);
+  const Pack<T, E> f = Pack<T, E>::splat(fill);
+  if (!inb) r = f;
+  return r;
+}
+
+template <class T, int E>
+__device__ __forceinline__ void trim_window_pack(Pack<T, E>& r, int e0, int n, float fill,
+                                                 int lo) {
+  if (e0 < n && (e0 < lo || e0 + E > n)) {
+#pragma unroll
+    for (int i = 0; i < E; ++i)
+      if (e0 + i < lo || e0 + i >= n) r.v[i] = (T)fill;
+  }
+}
+
 template <class T, int E, bool STREAM>
 __device__ __forceinline__ void store_row_pack(T* row, int e0, int n, bool row_ok,
-                                               const Pack<T, E>& p) {
+                                               const Pack<T, E>& p, int lo = 0) {
   if (!row_ok) return;
-  if (e0 + E <= n) {
+  if (e0 >= lo && e0 + E <= n) {
     if (STREAM)
       p.store_stream(row + e0);
     else
       p.store(row + e0);
-  } else if (e0 < n) {
+  } else if (e0 < n && e0 + E > lo) {
 #pragma unroll
     for (int i = 0; i < E; ++i)
-      if (e0 + i < n) row[e0 + i] = p.v[i];
+      if (e0 + i >= lo && e0 + i < n) row[e0 + i] = p.v[i];
   }
+}
+
+// Ragged rows (a row length that is not a whole number of packs puts every row
+// at a different 2- or 4-byte alignment) are addressed through a window that
+// starts on a 16-byte boundary of `row`'s memory: the row's first element sits
+// `window_head(row)` elements into it.  Every whole pack of the window is then an
+// aligned 128-bit access (a 128-bit access at a 2-byte alignment costs about
+// twice as much), and only the window's first and last pack are moved element
+// by element.  Tensors that share the row index keep a constant alignment
+// relative to the window (the same one, when their base addresses are congruent
+// modulo 16 bytes).
+template <class T, int E>
+__device__ __forceinline__ int window_head(const T* row) {
+  return (int)((reinterpret_cast<uintptr_t>(row) / sizeof(T)) % (unsigned)E);
+}
+
+// Whether the packs of tensor `b` are 16-byte aligned in a window laid over the
+// same rows of tensor `a` (same element type, same row length).
+template <class T>
+__device__ __forceinline__ bool same_pack_alignment(const T* a, const T* b) {
+  return ((reinterpret_cast<uintptr_t>(a) ^ reinterpret_cast<uintptr_t>(b)) & 15u) == 0;
 }
 
 // Row accessors used by the register-resident kernels.
@@ -137,10 +198,14 @@ __device__ __forceinline__ void store_row_pack(T* row, int e0, int n, bool row_o
 // and the value is replaced by `fill` with a select -- so the V loads of a lane
 // are straight-line code that the hardware issues back to back.  `row` must
 // point at a readable row even when `ok` is false (callers clamp the index).
-// Otherwise: the general loader above (handles a pack that straddles the row
-// end element by element, at the price of a branch per pack).
+// Otherwise: the general loaders above -- `whole` (the row is seen through a
+// window of 16-byte aligned packs) picks the one that reads boundary packs in
+// full and leaves the trimming to the caller (row_trim), else a pack that
+// straddles an end of the row [lo, n) is read element by element, at the price
+// of a branch per pack.
 template <class T, int E, bool STREAM, bool FAST>
-__device__ __forceinline__ Pack<T, E> row_load(const T* row, int e0, int n, bool ok, float fill) {
+__device__ __forceinline__ Pack<T, E> row_load(const T* row, int e0, int n, bool ok, float fill,
+                                               int lo = 0, bool whole = false) {
   if constexpr (FAST) {
     const bool inb = e0 < n;
     const T* p = row + (inb ? e0 : 0);
@@ -149,12 +214,23 @@ __device__ __forceinline__ Pack<T, E> row_load(const T* row, int e0, int n, bool
     if (!(inb && ok)) r = f;
     return r;
   } else {
-    return load_row_pack<T, E, STREAM>(row, e0, n, ok, fill);
+    if (whole) return load_window_pack<T, E, STREAM>(row, e0, n, ok, fill);
+    return load_row_pack<T, E, STREAM>(row, e0, n, ok, fill, lo);
+  }
+}
+
+// After row_load(..., whole): `fill` for the elements of the pack outside [lo, n).
+template <class T, int E, bool FAST>
+__device__ __forceinline__ void row_trim(Pack<T, E>& r, int e0, int n, float fill, int lo,
+                                         bool whole) {
+  if constexpr (!FAST) {
+    if (whole) trim_window_pack<T, E>(r, e0, n, fill, lo);
   }
 }
 
 template <class T, int E, bool STREAM, bool FAST>
-__device__ __forceinline__ void row_store(T* row, int e0, int n, bool ok, const Pack<T, E>& p) {
+__device__ __forceinline__ void row_store(T* row, int e0, int n, bool ok, const Pack<T, E>& p,
+                                          int lo = 0) {
   if constexpr (FAST) {
     if (ok && e0 < n) {
       if (STREAM)
@@ -163,7 +239,7 @@ __device__ __forceinline__ void row_store(T* row, int e0, int n, bool ok, const 
         p.store(row + e0);
     }
   } else {
-    store_row_pack<T, E, STREAM>(row, e0, n, ok, p);
+    store_row_pack<T, E, STREAM>(row, e0, n, ok, p, lo);
   }
 }
 

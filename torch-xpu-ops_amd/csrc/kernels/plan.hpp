@@ -149,8 +149,11 @@ inline int make_plan(OpClass oc, int64_t M, int64_t N, int esize, int num_cus, c
                      bool want_cols, Plan* out, bool force_general = false) {
   Plan p;
   const int E = 16 / esize;
-  const int64_t packs = (N + E - 1) / E;
   p.fast = (N % E) == 0 && !force_general;
+  const bool softmax = oc == OC_SOFTMAX_FWD || oc == OC_SOFTMAX_BWD;
+  // the general softmax kernels address a row through the 16-byte aligned window
+  // that holds it, which starts up to E - 1 elements before the row
+  const int64_t packs = ((softmax && !p.fast ? N + E - 1 : N) + E - 1) / E;
   if (num_cus <= 0) num_cus = 256;
   bool stream = ov.G < 0;
   if (!stream) {
@@ -183,7 +186,7 @@ inline int make_plan(OpClass oc, int64_t M, int64_t N, int esize, int num_cus, c
     } else if (!group_exact) {
       V = pow2_ceil((packs + G - 1) / G);
       const int64_t v_exact = (packs + G - 1) / G;
-      if ((oc == OC_SOFTMAX_FWD || oc == OC_SOFTMAX_BWD) && p.fast && G == kMaxG &&
+      if (softmax && p.fast && G == kMaxG &&
           v_exact <= kMaxV && variant_built(oc, esize, G, (int)v_exact, true))
         V = (int)v_exact;
       if (!p.fast && V < v_pref(oc, esize)) V = v_pref(oc, esize);

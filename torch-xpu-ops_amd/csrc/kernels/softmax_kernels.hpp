@@ -29,6 +29,7 @@
 #include "device/pack.hpp"
 #include "device/reduce.hpp"
 #include "launch.hpp"
+#include <type_traits>
 
 namespace rownorm {
 
@@ -62,10 +63,11 @@ __device__ __forceinline__ const uint8_t* mask_row_ptr(const MaskRef& m, int64_t
   return m.data + mr * (int64_t)n;
 }
 
-// E mask bytes for the pack starting at element e0 of a mask row (fill: not masked).
+// E mask bytes for the pack starting at element e0 of a mask row whose elements are
+// [lo, n) of `mrow` (fill: not masked).
 template <int E, bool FAST>
 __device__ __forceinline__ Pack<uint8_t, E> load_mask_pack(const uint8_t* mrow, int e0, int n,
-                                                           bool ok) {
+                                                           bool ok, int lo = 0) {
   Pack<uint8_t, E> m;
   if constexpr (FAST) {
     const bool inb = e0 < n;
@@ -77,7 +79,7 @@ __device__ __forceinline__ Pack<uint8_t, E> load_mask_pack(const uint8_t* mrow, 
     if (ok) {
 #pragma unroll
       for (int i = 0; i < E; ++i)
-        if (e0 + i < n) m.v[i] = mrow[e0 + i];
+        if (e0 + i >= lo && e0 + i < n) m.v[i] = mrow[e0 + i];
     }
   }
   return m;
@@ -101,21 +103,28 @@ softmax_fwd_resident_kernel(const TI* __restrict__ x, TO* __restrict__ y, MaskRe
     const int64_t row = rb * RPB + slot;
     const bool ok = RPB == 1 ? true : row < M;
     const int64_t rowc = ok ? row : 0;
-    const TI* xr = x + rowc * (int64_t)N;
-    TO* yr = y + row * (int64_t)N;
+    // ragged rows go through the 16-byte aligned window that holds the row
+    const int h = FAST ? 0 : window_head<TI, E>(x + rowc * (int64_t)N);
+    const int nw = N + h;
+    const TI* xr = x + rowc * (int64_t)N - h;
+    TO* yr = y + row * (int64_t)N - h;
     Pack<TI, E> xp[V];
 #pragma unroll
     for (int c = 0; c < V; ++c)
-      xp[c] = row_load<TI, E, true, FAST>(xr, (c * G + lane) * E, N, ok, -INFINITY);
+      xp[c] = row_load<TI, E, true, FAST>(xr, (c * G + lane) * E, nw, ok, -INFINITY, h, true);
+#pragma unroll
+    for (int c = 0; c < V; ++c)
+      row_trim<TI, E, FAST>(xp[c], (c * G + lane) * E, nw, -INFINITY, h, true);
     if constexpr (V * E > kSoftmaxWideElems) {
       // Long rows (a vocabulary-sized row is 16 packs a lane): the row stays in
       // storage format and each of the three passes widens it again; softmax
       // then evaluates exp twice per element, log_softmax still once.
       if constexpr (MASKED) {
-        const uint8_t* mrow = mask_row_ptr(mask, rowc, N);
+        const uint8_t* mrow = mask_row_ptr(mask, rowc, N) - h;
 #pragma unroll
         for (int c = 0; c < V; ++c) {
-          const Pack<uint8_t, E> mk = load_mask_pack<E, FAST>(mrow, (c * G + lane) * E, N, ok);
+          const Pack<uint8_t, E> mk =
+              load_mask_pack<E, FAST>(mrow, (c * G + lane) * E, nw, ok, h);
 #pragma unroll
           for (int i = 0; i < E; ++i)
             if (mk.v[i]) xp[c].set(i, -INFINITY);
@@ -148,7 +157,7 @@ softmax_fwd_resident_kernel(const TI* __restrict__ x, TO* __restrict__ y, MaskRe
           const float v = is_log ? d - k : row_exp<PRECISE>(d) * k;
           o.set(i, zero_row ? 0.0f : v);
         }
-        row_store<TO, E, true, FAST>(yr, (c * G + lane) * E, N, ok, o);
+        row_store<TO, E, true, FAST>(yr, (c * G + lane) * E, nw, ok, o, h);
       }
       continue;
     }
@@ -158,10 +167,10 @@ softmax_fwd_resident_kernel(const TI* __restrict__ x, TO* __restrict__ y, MaskRe
 #pragma unroll
       for (int i = 0; i < E; ++i) xf[c][i] = xp[c].get(i);
     if constexpr (MASKED) {
-      const uint8_t* mrow = mask_row_ptr(mask, rowc, N);
+      const uint8_t* mrow = mask_row_ptr(mask, rowc, N) - h;
 #pragma unroll
       for (int c = 0; c < V; ++c) {
-        const Pack<uint8_t, E> mk = load_mask_pack<E, FAST>(mrow, (c * G + lane) * E, N, ok);
+        const Pack<uint8_t, E> mk = load_mask_pack<E, FAST>(mrow, (c * G + lane) * E, nw, ok, h);
 #pragma unroll
         for (int i = 0; i < E; ++i) xf[c][i] = mk.v[i] ? -INFINITY : xf[c][i];
       }
@@ -204,7 +213,7 @@ softmax_fwd_resident_kernel(const TI* __restrict__ x, TO* __restrict__ y, MaskRe
         const float v = is_log ? xf[c][i] - k : xf[c][i] * k;
         o.set(i, zero_row ? 0.0f : v);
       }
-      row_store<TO, E, true, FAST>(yr, e0, N, ok, o);
+      row_store<TO, E, true, FAST>(yr, e0, nw, ok, o, h);
     }
   }
 }
@@ -225,11 +234,14 @@ softmax_fwd_stream_kernel(const TI* __restrict__ x, TO* __restrict__ y, MaskRef 
   int phase = 0;
   const bool is_log = (flags & kSoftmaxLog) != 0;
   const bool is_safe = (flags & kSoftmaxSafe) != 0;
-  const int npacks = (N + E - 1) / E;
   for (int64_t row = blockIdx.x; row < M; row += gridDim.x) {
-    const TI* xr = x + row * (int64_t)N;
-    TO* yr = y + row * (int64_t)N;
-    const uint8_t* mrow = MASKED ? mask_row_ptr(mask, row, N) : nullptr;
+    // the 16-byte aligned window that holds the row: elements [h, nw) of it
+    const int h = window_head<TI, E>(x + row * (int64_t)N);
+    const int nw = N + h;
+    const int npacks = (nw + E - 1) / E;
+    const TI* xr = x + row * (int64_t)N - h;
+    TO* yr = y + row * (int64_t)N - h;
+    const uint8_t* mrow = MASKED ? mask_row_ptr(mask, row, N) - h : nullptr;
     // element i of a pack, with the mask applied
     auto masked_value = [&](const Pack<TI, E>& p, const Pack<uint8_t, E>& mk, int i) {
       const float v = p.get(i);
@@ -244,11 +256,12 @@ softmax_fwd_stream_kernel(const TI* __restrict__ x, TO* __restrict__ y, MaskRef 
 #pragma unroll
       for (int u = 0; u < kStreamUnroll; ++u) {
         const int pk = pk0 + u * BLOCK;
-        pv[u] = load_row_pack<TI, E, false>(xr, pk * E, N, pk < npacks, -INFINITY);
-        if constexpr (MASKED) mv[u] = load_mask_pack<E, false>(mrow, pk * E, N, pk < npacks);
+        pv[u] = load_window_pack<TI, E, false>(xr, pk * E, nw, pk < npacks, -INFINITY);
+        if constexpr (MASKED) mv[u] = load_mask_pack<E, false>(mrow, pk * E, nw, pk < npacks, h);
       }
 #pragma unroll
       for (int u = 0; u < kStreamUnroll; ++u) {
+        trim_window_pack<TI, E>(pv[u], (pk0 + u * BLOCK) * E, nw, -INFINITY, h);
         float v[E];
         float pm = -INFINITY;
 #pragma unroll
@@ -285,8 +298,8 @@ softmax_fwd_stream_kernel(const TI* __restrict__ x, TO* __restrict__ y, MaskRef 
 #pragma unroll
       for (int u = 0; u < kStreamUnroll; ++u) {
         const int pk = pk0 + u * BLOCK;
-        pv[u] = load_row_pack<TI, E, true>(xr, pk * E, N, pk < npacks, -INFINITY);
-        if constexpr (MASKED) mv[u] = load_mask_pack<E, false>(mrow, pk * E, N, pk < npacks);
+        pv[u] = load_window_pack<TI, E, true>(xr, pk * E, nw, pk < npacks, -INFINITY);
+        if constexpr (MASKED) mv[u] = load_mask_pack<E, false>(mrow, pk * E, nw, pk < npacks, h);
       }
 #pragma unroll
       for (int u = 0; u < kStreamUnroll; ++u) {
@@ -298,7 +311,7 @@ softmax_fwd_stream_kernel(const TI* __restrict__ x, TO* __restrict__ y, MaskRef 
           const float v = is_log ? d - k : row_exp<PRECISE>(d) * k;
           o.set(i, zero_row ? 0.0f : v);
         }
-        store_row_pack<TO, E, true>(yr, pk * E, N, pk < npacks, o);
+        store_row_pack<TO, E, true>(yr, pk * E, nw, pk < npacks, o, h);
       }
     }
   }
@@ -318,20 +331,31 @@ softmax_bwd_resident_kernel(const TG* __restrict__ grad, const TG* __restrict__ 
   const int slot = threadIdx.x / G;
   const int lane = threadIdx.x % G;
   const bool is_log = (flags & kSoftmaxLog) != 0;
+  // y's packs are aligned like grad's when the two base addresses are congruent
+  const bool y_whole = same_pack_alignment(grad, y);
   const int64_t nrb = (M + RPB - 1) / RPB;
   for (int64_t rb = blockIdx.x; rb < nrb; rb += gridDim.x) {
     const int64_t row = rb * RPB + slot;
     const bool ok = RPB == 1 ? true : row < M;
     const int64_t rowc = ok ? row : 0;
-    const TG* gr = grad + rowc * (int64_t)N;
-    const TG* yr = y + rowc * (int64_t)N;
-    TO* outr = gi + row * (int64_t)N;
+    // ragged rows go through the 16-byte aligned window that holds the row of grad
+    const int h = FAST ? 0 : window_head<TG, E>(grad + rowc * (int64_t)N);
+    const int nw = N + h;
+    const TG* gr = grad + rowc * (int64_t)N - h;
+    const TG* yr = y + rowc * (int64_t)N - h;
+    TO* outr = gi + row * (int64_t)N - h;
     Pack<TG, E> pg[V], py[V];
 #pragma unroll
     for (int c = 0; c < V; ++c) {
       const int e0 = (c * G + lane) * E;
-      pg[c] = row_load<TG, E, true, FAST>(gr, e0, N, ok, 0.0f);
-      py[c] = row_load<TG, E, true, FAST>(yr, e0, N, ok, 0.0f);
+      pg[c] = row_load<TG, E, true, FAST>(gr, e0, nw, ok, 0.0f, h, true);
+      py[c] = row_load<TG, E, true, FAST>(yr, e0, nw, ok, 0.0f, h, y_whole);
+    }
+#pragma unroll
+    for (int c = 0; c < V; ++c) {
+      const int e0 = (c * G + lane) * E;
+      row_trim<TG, E, FAST>(pg[c], e0, nw, 0.0f, h, true);
+      row_trim<TG, E, FAST>(py[c], e0, nw, 0.0f, h, y_whole);
     }
     float gf[V][E], yf[V][E];
 #pragma unroll
@@ -342,10 +366,10 @@ softmax_bwd_resident_kernel(const TG* __restrict__ grad, const TG* __restrict__ 
         yf[c][i] = py[c].get(i);
       }
     if constexpr (MASKED) {
-      const uint8_t* mrow = mask_row_ptr(mask, rowc, N);
+      const uint8_t* mrow = mask_row_ptr(mask, rowc, N) - h;
 #pragma unroll
       for (int c = 0; c < V; ++c) {
-        const Pack<uint8_t, E> mk = load_mask_pack<E, FAST>(mrow, (c * G + lane) * E, N, ok);
+        const Pack<uint8_t, E> mk = load_mask_pack<E, FAST>(mrow, (c * G + lane) * E, nw, ok, h);
 #pragma unroll
         for (int i = 0; i < E; ++i) yf[c][i] = mk.v[i] ? 0.0f : yf[c][i];
       }
@@ -374,7 +398,7 @@ softmax_bwd_resident_kernel(const TG* __restrict__ grad, const TG* __restrict__ 
                                : yf[c][i] * (gf[c][i] - s);
         o.set(i, v);
       }
-      row_store<TO, E, true, FAST>(outr, e0, N, ok, o);
+      row_store<TO, E, true, FAST>(outr, e0, nw, ok, o, h);
     }
   }
 }
@@ -389,12 +413,22 @@ softmax_bwd_stream_kernel(const TG* __restrict__ grad, const TG* __restrict__ y,
   __shared__ float red[reduce_lds_floats<BLOCK, BLOCK, 1>::value];
   int phase = 0;
   const bool is_log = (flags & kSoftmaxLog) != 0;
-  const int npacks = (N + E - 1) / E;
+  const bool y_whole = same_pack_alignment(grad, y);
+  // a pack of y: whole when it is aligned like grad's, else element by element at the row ends
+  auto load_y = [&](const TG* yr, int e0, int nw, bool in_row, int h, auto stream_tag) {
+    constexpr bool STREAM = decltype(stream_tag)::value;
+    return y_whole ? load_window_pack<TG, E, STREAM>(yr, e0, nw, in_row, 0.0f)
+                   : load_row_pack<TG, E, STREAM>(yr, e0, nw, in_row, 0.0f, h);
+  };
   for (int64_t row = blockIdx.x; row < M; row += gridDim.x) {
-    const TG* gr = grad + row * (int64_t)N;
-    const TG* yr = y + row * (int64_t)N;
-    TO* outr = gi + row * (int64_t)N;
-    const uint8_t* mrow = MASKED ? mask_row_ptr(mask, row, N) : nullptr;
+    // the 16-byte aligned window that holds the row of grad: elements [h, nw) of it
+    const int h = window_head<TG, E>(grad + row * (int64_t)N);
+    const int nw = N + h;
+    const int npacks = (nw + E - 1) / E;
+    const TG* gr = grad + row * (int64_t)N - h;
+    const TG* yr = y + row * (int64_t)N - h;
+    TO* outr = gi + row * (int64_t)N - h;
+    const uint8_t* mrow = MASKED ? mask_row_ptr(mask, row, N) - h : nullptr;
     auto saved_output = [&](const Pack<TG, E>& p, const Pack<uint8_t, E>& mk, int i) {
       const float v = p.get(i);
       if constexpr (MASKED) return mk.v[i] ? 0.0f : v;
@@ -408,14 +442,16 @@ softmax_bwd_stream_kernel(const TG* __restrict__ grad, const TG* __restrict__ y,
 #pragma unroll
       for (int u = 0; u < U; ++u) {
         const int pk = pk0 + u * BLOCK;
-        pg[u] = load_row_pack<TG, E, false>(gr, pk * E, N, pk < npacks, 0.0f);
+        pg[u] = load_window_pack<TG, E, false>(gr, pk * E, nw, pk < npacks, 0.0f);
         if (!is_log) {
-          py[u] = load_row_pack<TG, E, false>(yr, pk * E, N, pk < npacks, 0.0f);
-          if constexpr (MASKED) mk[u] = load_mask_pack<E, false>(mrow, pk * E, N, pk < npacks);
+          py[u] = load_y(yr, pk * E, nw, pk < npacks, h, std::false_type{});
+          if constexpr (MASKED) mk[u] = load_mask_pack<E, false>(mrow, pk * E, nw, pk < npacks, h);
         }
       }
 #pragma unroll
       for (int u = 0; u < U; ++u) {
+        trim_window_pack<TG, E>(pg[u], (pk0 + u * BLOCK) * E, nw, 0.0f, h);
+        if (!is_log && y_whole) trim_window_pack<TG, E>(py[u], (pk0 + u * BLOCK) * E, nw, 0.0f, h);
         if (is_log) {
 #pragma unroll
           for (int i = 0; i < E; ++i) sum[0] += pg[u].get(i);
@@ -434,9 +470,9 @@ softmax_bwd_stream_kernel(const TG* __restrict__ grad, const TG* __restrict__ y,
 #pragma unroll
       for (int u = 0; u < U; ++u) {
         const int pk = pk0 + u * BLOCK;
-        pg[u] = load_row_pack<TG, E, true>(gr, pk * E, N, pk < npacks, 0.0f);
-        py[u] = load_row_pack<TG, E, true>(yr, pk * E, N, pk < npacks, 0.0f);
-        if constexpr (MASKED) mk[u] = load_mask_pack<E, false>(mrow, pk * E, N, pk < npacks);
+        pg[u] = load_window_pack<TG, E, true>(gr, pk * E, nw, pk < npacks, 0.0f);
+        py[u] = load_y(yr, pk * E, nw, pk < npacks, h, std::true_type{});
+        if constexpr (MASKED) mk[u] = load_mask_pack<E, false>(mrow, pk * E, nw, pk < npacks, h);
       }
 #pragma unroll
       for (int u = 0; u < U; ++u) {
@@ -449,7 +485,7 @@ softmax_bwd_stream_kernel(const TG* __restrict__ grad, const TG* __restrict__ y,
               is_log ? pg[u].get(i) - row_exp<PRECISE>(yv) * s : yv * (pg[u].get(i) - s);
           o.set(i, v);
         }
-        store_row_pack<TO, E, true>(outr, pk * E, N, pk < npacks, o);
+        store_row_pack<TO, E, true>(outr, pk * E, nw, pk < npacks, o, h);
       }
     }
   }
