@@ -132,13 +132,23 @@ norm_fwd_resident_kernel(const T* __restrict__ x, const WT* __restrict__ gamma,
         const float k = fmaxf(fminf(a, b), fminf(fmaxf(a, b), c3));
         mean0[r] = k;
         acc[2 * r] = acc[2 * r + 1] = 0.0f;
+        if constexpr (FAST) {
+          // a pack lies wholly inside or wholly outside the row: the ones outside
+          // become k (a value of the row, so exact in T) and add nothing
+          if (!exact) {
+            const Pack<T, E> kp = Pack<T, E>::splat(k);
+#pragma unroll
+            for (int c = 0; c < V; ++c)
+              if ((c * G + lane) * E >= N) xp[r][c] = kp;
+          }
+        }
 #pragma unroll
         for (int c = 0; c < V; ++c) {
           const int nvalid = ok[r] ? N - (c * G + lane) * E : 0;
 #pragma unroll
           for (int i = 0; i < E; ++i) {
             float d = xp[r][c].get(i) - k;
-            if (!exact) d = (i < nvalid) ? d : 0.0f;
+            if constexpr (!FAST) d = (i < nvalid) ? d : 0.0f;
             acc[2 * r] += d;
             acc[2 * r + 1] = fmaf(d, d, acc[2 * r + 1]);
           }
@@ -164,11 +174,12 @@ norm_fwd_resident_kernel(const T* __restrict__ x, const WT* __restrict__ gamma,
       group_allreduce<G, BLOCK, R, SumOp>(acc0, red, phase);
       float acc[2 * R];
       // MASKED: some packs reach past the row end; their elements must not count.
+#pragma unroll
+      for (int r = 0; r < R; ++r) mean0[r] = acc0[r] / fN;
       auto centred_sums = [&](auto masked) {
         constexpr bool MASKED = decltype(masked)::value;
 #pragma unroll
         for (int r = 0; r < R; ++r) {
-          mean0[r] = acc0[r] / fN;
           acc[2 * r] = acc[2 * r + 1] = 0.0f;
 #pragma unroll
           for (int c = 0; c < V; ++c) {
@@ -184,10 +195,20 @@ norm_fwd_resident_kernel(const T* __restrict__ x, const WT* __restrict__ gamma,
           }
         }
       };
-      if (exact)
+      if (exact) {
         centred_sums(std::false_type{});
-      else
+      } else if constexpr (FAST && sizeof(T) == 4) {
+        // a pack lies wholly inside or wholly outside the row: the ones outside
+        // become mean0 and add nothing
+#pragma unroll
+        for (int r = 0; r < R; ++r)
+#pragma unroll
+          for (int c = 0; c < V; ++c)
+            if ((c * G + lane) * E >= N) xp[r][c] = Pack<T, E>::splat(mean0[r]);
+        centred_sums(std::false_type{});
+      } else {
         centred_sums(std::true_type{});
+      }
       group_allreduce<G, BLOCK, 2 * R, SumOp>(acc, red, phase);
 #pragma unroll
       for (int r = 0; r < R; ++r) {

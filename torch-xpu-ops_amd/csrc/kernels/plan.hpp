@@ -145,8 +145,10 @@ inline int pow2_ceil(int64_t v) {
 
 // Returns 0, or -5 (ROWNORM_ERR_OVERRIDE) when a forced variant cannot hold the row.
 // force_general: take the general (ragged-row) kernels even when N % E == 0.
+// layer_norm: the norm op is LayerNorm (statistics of two sums, beta), not RMSNorm.
 inline int make_plan(OpClass oc, int64_t M, int64_t N, int esize, int num_cus, const Override& ov,
-                     bool want_cols, Plan* out, bool force_general = false) {
+                     bool want_cols, Plan* out, bool force_general = false,
+                     bool layer_norm = false) {
   Plan p;
   const int E = 16 / esize;
   p.fast = (N % E) == 0 && !force_general;
@@ -164,6 +166,17 @@ inline int make_plan(OpClass oc, int64_t M, int64_t N, int esize, int num_cus, c
       G = pow2_ceil((packs + v_pref(oc, esize) - 1) / v_pref(oc, esize));
       if (G < kMinG) G = kMinG;
       if (G > kMaxG) G = kMaxG;
+      // 16-bit norm rows, measured at 16384 rows: a row group of 1024 lanes (16
+      // wavefronts around every reduction) loses to 512 lanes with four packs
+      // each in the forward (LayerNorm 160 -> 124 us at N = 10240, RMSNorm 2-4 %)
+      // and in the LayerNorm backward (250 -> 217 us); the RMSNorm backward keeps
+      // 1024 lanes (192 vs 205 us).  The forward also halves the lanes of a row
+      // that fills at most three quarters of them (N = 5120, 6144: 5-10 %).
+      if (esize == 2 && p.fast && ov.V == 0) {
+        const bool fwd = oc == OC_NORM_FWD;
+        if ((fwd || (oc == OC_NORM_BWD && layer_norm)) && packs > 1024 && packs <= 2048) G = 512;
+        if (fwd && packs > 512 && packs <= 768) G = 256;
+      }
     }
     // GroupNorm rows of a wavefront or more (measured): about 5 packs a lane on
     // as few lanes as that allows, and exactly the packs the row has
