@@ -128,7 +128,7 @@ int norm_fwd(const void* x, const void* gamma, const void* beta, void* y, float*
   Plan plan;
   const int op = RMS ? ROWNORM_OP_RMS_NORM_FWD : ROWNORM_OP_LAYER_NORM_FWD;
   if (int e = make_plan(OC_NORM_FWD, M, N, esize_of(xd), current_num_cus(), g_override[op],
-                        false, &plan, false, !RMS))
+                        false, &plan, false, !RMS, esize_of(wd) > esize_of(xd)))
     return e;
   NormFwdArgs a{x, gamma, RMS ? nullptr : beta, y, RMS ? nullptr : mean, rstd, M, (int)N, eps};
   hipStream_t s = (hipStream_t)stream;
@@ -144,7 +144,7 @@ size_t norm_bwd_workspace(int op, int64_t M, int64_t N, int xd, int wd, int npar
   if (!norm_dtypes_ok(xd, wd) || shape_check(M, N) || M == 0 || N == 0 || nparts == 0) return 0;
   Plan plan;
   if (make_plan(OC_NORM_BWD, M, N, esize_of(xd), current_num_cus(), g_override[op], true, &plan,
-                false, op == ROWNORM_OP_LAYER_NORM_BWD))
+                false, op == ROWNORM_OP_LAYER_NORM_BWD, esize_of(wd) > esize_of(xd)))
     return 0;
   return (size_t)plan.partial_rows * (size_t)N * sizeof(float) * (size_t)nparts;
 }
@@ -163,7 +163,7 @@ int norm_bwd(const void* dy, const void* x, const float* mean, const float* rstd
   Plan plan;
   const int op = RMS ? ROWNORM_OP_RMS_NORM_BWD : ROWNORM_OP_LAYER_NORM_BWD;
   if (int e = make_plan(OC_NORM_BWD, M, N, esize_of(xd), current_num_cus(), g_override[op],
-                        want_cols, &plan, false, !RMS))
+                        want_cols, &plan, false, !RMS, esize_of(wd) > esize_of(xd)))
     return e;
   float* part_dg = nullptr;
   float* part_db = nullptr;
@@ -561,7 +561,6 @@ int mi355x_softmax_strided_plan(int backward, int64_t outer, int64_t dim_size, i
 
 int mi355x_rownorm_plan(rownorm_op op, int64_t M, int64_t N, rownorm_dtype x_dtype,
                         rownorm_dtype w_dtype, rownorm_plan* out) {
-  (void)w_dtype;
   if ((int)op < 0 || (int)op > ROWNORM_OP_SOFTMAX_BWD) return ROWNORM_ERR_SHAPE;
   if (!out) return ROWNORM_ERR_NULL;
   if (esize_of((int)x_dtype) == 0) return ROWNORM_ERR_DTYPE;
@@ -570,7 +569,8 @@ int mi355x_rownorm_plan(rownorm_op op, int64_t M, int64_t N, rownorm_dtype x_dty
   const OpClass oc = class_of((int)op);
   const bool layer_norm = op == ROWNORM_OP_LAYER_NORM_FWD || op == ROWNORM_OP_LAYER_NORM_BWD;
   if (int e = make_plan(oc, M, N, esize_of((int)x_dtype), current_num_cus(), g_override[(int)op],
-                        oc == OC_NORM_BWD, &plan, false, layer_norm))
+                        oc == OC_NORM_BWD, &plan, false, layer_norm,
+                        esize_of((int)w_dtype) > esize_of((int)x_dtype)))
     return e;
   out->resident = plan.resident ? 1 : 0;
   out->lanes_per_row = plan.G;

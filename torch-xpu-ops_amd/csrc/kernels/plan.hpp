@@ -14,8 +14,12 @@
 // If V exceeds the per-op register budget V_max the multi-pass streaming
 // kernel is used instead.  Rows whose length is a whole number of packs take
 // the branch-free "fast" kernels; ragged rows (N % E != 0) take the general
-// ones, which exist for V = V_pref only.  Workgroup size and grid size per op
-// class are set by block_threads() and default_bpc() below.
+// ones, which exist for V = V_pref only.  Measured exceptions for rows that
+// leave many of those lanes idle (hidden sizes that are not powers of two) or
+// that would take 1024 lanes: norm_layout() and the softmax / GroupNorm rules
+// in make_plan() pick three or five packs a lane, or fewer lanes.  Workgroup
+// size and grid size per op class are set by block_threads() and default_bpc()
+// below.
 #pragma once
 #include <stdint.h>
 
@@ -120,8 +124,12 @@ constexpr bool variant_built(OpClass oc, int esize, int G, int V, bool fast) {
   if (V & (V - 1)) {
     if (!fast || V > v_max(oc, esize, G)) return false;
     // softmax rows that need all 1024 lanes (vocabulary-sized) likewise
+    // (and the 16-bit forward takes three packs a lane where that fits better)
+    if (oc == OC_SOFTMAX_FWD && esize == 2) return G == kMaxG || (G >= 64 && V == 3);
     if (oc == OC_SOFTMAX_FWD || oc == OC_SOFTMAX_BWD) return G == kMaxG;
-    if (!is_group_class(oc)) return false;
+    // LayerNorm / RMSNorm rows of hidden sizes such as 5120, 6144, 10240, 12288
+    // (640, 768, 1280, 1536 16-bit packs): 3 or 5 packs a lane
+    if (!is_group_class(oc)) return G >= 64 && (V == 3 || V == 5);
     return G == kMaxG || (G >= 64 && (V == 3 || V == 5));
   }
   if (V > v_max(oc, esize, G)) return false;
@@ -143,12 +151,65 @@ inline int pow2_ceil(int64_t v) {
   return p;
 }
 
+// LayerNorm / RMSNorm rows that the power-of-two rule serves badly (measured on
+// MI355X at 16384 rows; "slots" = lanes x preferred packs of that rule):
+//  * a 16-bit row of 1025..2048 packs would take 1024 lanes, 16 wavefronts around
+//    every reduction: 512 lanes with 3 or 4 packs each are faster in the forward
+//    (LayerNorm 160 -> 116 us at N = 10240, RMSNorm 2-4 %) and in the LayerNorm
+//    backward (250 -> 206 us); the RMSNorm backward gains only with 3 packs
+//    (N = 12288: 222 -> 212 us) and keeps 1024 lanes beyond 1536 packs;
+//  * a row that fills at most three quarters of the slots takes three packs on a
+//    quarter of the slots' lanes instead: hidden sizes such as 1536, 3072, 6144,
+//    12288 fit exactly, 2560, 5120, 10240 to 83 % (16-bit forward 3-14 %, fp32
+//    LayerNorm backward 5-15 %).  The 16-bit backward below 1024 packs is the
+//    exception: its column sums want the lanes (N = 5120: 96 vs 109 us); so is
+//    the LayerNorm forward with fp32 weights below 512 lanes;
+//  * fp32 LayerNorm forward rows of 2049..2560 packs: 512 lanes x 5 (N = 10240:
+//    261 -> 222 us).
+// Returns false where the general rule stands.
+inline bool norm_layout(OpClass oc, int esize, int64_t packs, bool layer_norm, bool wide_weights,
+                        int* G_out, int* V_out) {
+  const int vp = v_pref(oc, esize);
+  int G2 = pow2_ceil((packs + vp - 1) / vp);
+  if (G2 < kMinG) G2 = kMinG;
+  if (G2 > kMaxG) G2 = kMaxG;
+  const int64_t slots = (int64_t)G2 * vp;
+  if (packs > slots) return false;
+  const bool fwd = oc == OC_NORM_FWD;
+  const bool sparse = packs * 4 <= slots * 3;
+  int G = 0, V = 0;
+  if (esize == 2) {
+    if (G2 == kMaxG) {
+      if (sparse) {
+        G = 512, V = 3;
+      } else if (fwd || layer_norm) {
+        G = 512, V = 4;
+      }
+    } else if (fwd && sparse && !(layer_norm && wide_weights && G2 < 512)) {
+      // (fp32 gamma and beta beside 16-bit rows: three packs of each are 48
+      // registers, and below 512 lanes the two-pack layout stays ahead)
+      G = G2 / 2, V = 3;
+    }
+  } else {
+    if (fwd && layer_norm && G2 == kMaxG && packs <= 2560) {
+      G = 512, V = 5;
+    } else if (sparse) {
+      G = G2, V = 3;
+    }
+  }
+  if (G == 0 || (int64_t)G * V < packs || !variant_built(oc, esize, G, V, true)) return false;
+  *G_out = G;
+  *V_out = V;
+  return true;
+}
+
 // Returns 0, or -5 (ROWNORM_ERR_OVERRIDE) when a forced variant cannot hold the row.
 // force_general: take the general (ragged-row) kernels even when N % E == 0.
 // layer_norm: the norm op is LayerNorm (statistics of two sums, beta), not RMSNorm.
+// wide_weights: fp32 gamma/beta beside 16-bit rows.
 inline int make_plan(OpClass oc, int64_t M, int64_t N, int esize, int num_cus, const Override& ov,
                      bool want_cols, Plan* out, bool force_general = false,
-                     bool layer_norm = false) {
+                     bool layer_norm = false, bool wide_weights = false) {
   Plan p;
   const int E = 16 / esize;
   p.fast = (N % E) == 0 && !force_general;
@@ -166,21 +227,22 @@ inline int make_plan(OpClass oc, int64_t M, int64_t N, int esize, int num_cus, c
       G = pow2_ceil((packs + v_pref(oc, esize) - 1) / v_pref(oc, esize));
       if (G < kMinG) G = kMinG;
       if (G > kMaxG) G = kMaxG;
-      // 16-bit norm rows, measured at 16384 rows: a row group of 1024 lanes (16
-      // wavefronts around every reduction) loses to 512 lanes with four packs
-      // each in the forward (LayerNorm 160 -> 124 us at N = 10240, RMSNorm 2-4 %)
-      // and in the LayerNorm backward (250 -> 217 us); the RMSNorm backward keeps
-      // 1024 lanes (192 vs 205 us).  The forward also halves the lanes of a row
-      // that fills at most three quarters of them (N = 5120, 6144: 5-10 %).
-      if (esize == 2 && p.fast && ov.V == 0) {
-        const bool fwd = oc == OC_NORM_FWD;
-        if ((fwd || (oc == OC_NORM_BWD && layer_norm)) && packs > 1024 && packs <= 2048) G = 512;
-        if (fwd && packs > 512 && packs <= 768) G = 256;
-      }
     }
     // GroupNorm rows of a wavefront or more (measured): about 5 packs a lane on
     // as few lanes as that allows, and exactly the packs the row has
     bool group_exact = false;
+    if ((oc == OC_NORM_FWD || oc == OC_NORM_BWD) && p.fast && ov.G == 0 && ov.V == 0)
+      group_exact = norm_layout(oc, esize, packs, layer_norm, wide_weights, &G, &V);
+    // 16-bit softmax forward (its exp makes it the arithmetic-heavy one): a row
+    // that fills at most three quarters of the two-pack slots takes three packs
+    // on half the lanes (N = 5120: 62 -> 56 us, 10240: 120 -> 110 us at 16384 rows)
+    if (oc == OC_SOFTMAX_FWD && esize == 2 && p.fast && ov.G == 0 && ov.V == 0 && G >= 128 &&
+        packs <= (int64_t)G * 2 && packs * 4 <= (int64_t)G * 2 * 3 &&
+        variant_built(oc, esize, G / 2, 3, true)) {
+      G /= 2;
+      V = 3;
+      group_exact = true;
+    }
     if (is_group_class(oc) && p.fast && ov.G == 0 && ov.V == 0) {
       int Gg = pow2_ceil((packs + 4) / 5);
       if (Gg > kMaxG) Gg = kMaxG;
