@@ -214,9 +214,9 @@ inline int make_plan(OpClass oc, int64_t M, int64_t N, int esize, int num_cus, c
   const int E = 16 / esize;
   p.fast = (N % E) == 0 && !force_general;
   const bool softmax = oc == OC_SOFTMAX_FWD || oc == OC_SOFTMAX_BWD;
-  // the general softmax kernels address a row through the 16-byte aligned window
-  // that holds it, which starts up to E - 1 elements before the row
-  const int64_t packs = ((softmax && !p.fast ? N + E - 1 : N) + E - 1) / E;
+  // the general softmax kernels address a 16-bit row through the 16-byte aligned
+  // window that holds it, which starts up to E - 1 elements before the row
+  const int64_t packs = ((softmax && !p.fast && esize == 2 ? N + E - 1 : N) + E - 1) / E;
   if (num_cus <= 0) num_cus = 256;
   bool stream = ov.G < 0;
   if (!stream) {

@@ -44,6 +44,28 @@ __device__ __forceinline__ float row_exp(float v) {
     return __expf(v);
 }
 
+// Whether ragged rows of T are addressed through the 16-byte aligned window that
+// holds them (window_head in device/pack.hpp).  16-bit rows: every ragged row
+// starts 2-byte aligned, where a 128-bit access costs about twice an aligned
+// one.  fp32 rows start 4-byte aligned, where it costs the same, and the
+// window's second element-wise row end only slowed them (N = 4097: 4.9 -> 4.3
+// TB/s), so they are addressed from the row start.
+template <class T>
+constexpr bool softmax_row_window() {
+  return sizeof(T) == 2;
+}
+
+// A pack of a row of the multi-pass kernels: whole from the aligned window (to
+// be trimmed), or through the general loader from the row start.
+template <class T, int E, bool STREAM, bool WINDOW>
+__device__ __forceinline__ Pack<T, E> stream_load(const T* row, int e0, int n, bool in_row,
+                                                  float fill, int lo) {
+  if constexpr (WINDOW)
+    return load_window_pack<T, E, STREAM>(row, e0, n, in_row, fill);
+  else
+    return load_row_pack<T, E, STREAM>(row, e0, n, in_row, fill, lo);
+}
+
 // Packs a thread of the multi-pass kernels requests before using the first.
 constexpr int kStreamUnroll = 2;
 
@@ -92,6 +114,7 @@ softmax_fwd_resident_kernel(const TI* __restrict__ x, TO* __restrict__ y, MaskRe
   constexpr int E = elems_per_pack<TI>::value;
   constexpr int RPB = BLOCK / G;
   constexpr bool PRECISE = sizeof(TO) == 4;
+  constexpr bool WINDOW = !FAST && softmax_row_window<TI>();
   __shared__ float red[reduce_lds_floats<G, BLOCK, 1>::value];
   int phase = 0;
   const int slot = threadIdx.x / G;
@@ -103,18 +126,18 @@ softmax_fwd_resident_kernel(const TI* __restrict__ x, TO* __restrict__ y, MaskRe
     const int64_t row = rb * RPB + slot;
     const bool ok = RPB == 1 ? true : row < M;
     const int64_t rowc = ok ? row : 0;
-    // ragged rows go through the 16-byte aligned window that holds the row
-    const int h = FAST ? 0 : window_head<TI, E>(x + rowc * (int64_t)N);
+    // ragged 16-bit rows go through the 16-byte aligned window that holds the row
+    const int h = WINDOW ? window_head<TI, E>(x + rowc * (int64_t)N) : 0;
     const int nw = N + h;
     const TI* xr = x + rowc * (int64_t)N - h;
     TO* yr = y + row * (int64_t)N - h;
     Pack<TI, E> xp[V];
 #pragma unroll
     for (int c = 0; c < V; ++c)
-      xp[c] = row_load<TI, E, true, FAST>(xr, (c * G + lane) * E, nw, ok, -INFINITY, h, true);
+      xp[c] = row_load<TI, E, true, FAST>(xr, (c * G + lane) * E, nw, ok, -INFINITY, h, WINDOW);
 #pragma unroll
     for (int c = 0; c < V; ++c)
-      row_trim<TI, E, FAST>(xp[c], (c * G + lane) * E, nw, -INFINITY, h, true);
+      row_trim<TI, E, FAST>(xp[c], (c * G + lane) * E, nw, -INFINITY, h, WINDOW);
     if constexpr (V * E > kSoftmaxWideElems) {
       // Long rows (a vocabulary-sized row is 16 packs a lane): the row stays in
       // storage format and each of the three passes widens it again; softmax
@@ -230,13 +253,14 @@ softmax_fwd_stream_kernel(const TI* __restrict__ x, TO* __restrict__ y, MaskRef 
                           int N, int flags) {
   constexpr int E = elems_per_pack<TI>::value;
   constexpr bool PRECISE = sizeof(TO) == 4;
+  constexpr bool WINDOW = softmax_row_window<TI>();
   __shared__ float red[reduce_lds_floats<BLOCK, BLOCK, 1>::value];
   int phase = 0;
   const bool is_log = (flags & kSoftmaxLog) != 0;
   const bool is_safe = (flags & kSoftmaxSafe) != 0;
   for (int64_t row = blockIdx.x; row < M; row += gridDim.x) {
-    // the 16-byte aligned window that holds the row: elements [h, nw) of it
-    const int h = window_head<TI, E>(x + row * (int64_t)N);
+    // 16-bit rows: the 16-byte aligned window that holds the row, elements [h, nw) of it
+    const int h = WINDOW ? window_head<TI, E>(x + row * (int64_t)N) : 0;
     const int nw = N + h;
     const int npacks = (nw + E - 1) / E;
     const TI* xr = x + row * (int64_t)N - h;
@@ -256,12 +280,12 @@ softmax_fwd_stream_kernel(const TI* __restrict__ x, TO* __restrict__ y, MaskRef 
 #pragma unroll
       for (int u = 0; u < kStreamUnroll; ++u) {
         const int pk = pk0 + u * BLOCK;
-        pv[u] = load_window_pack<TI, E, false>(xr, pk * E, nw, pk < npacks, -INFINITY);
+        pv[u] = stream_load<TI, E, false, WINDOW>(xr, pk * E, nw, pk < npacks, -INFINITY, h);
         if constexpr (MASKED) mv[u] = load_mask_pack<E, false>(mrow, pk * E, nw, pk < npacks, h);
       }
 #pragma unroll
       for (int u = 0; u < kStreamUnroll; ++u) {
-        trim_window_pack<TI, E>(pv[u], (pk0 + u * BLOCK) * E, nw, -INFINITY, h);
+        if constexpr (WINDOW) trim_window_pack<TI, E>(pv[u], (pk0 + u * BLOCK) * E, nw, -INFINITY, h);
         float v[E];
         float pm = -INFINITY;
 #pragma unroll
@@ -298,7 +322,7 @@ softmax_fwd_stream_kernel(const TI* __restrict__ x, TO* __restrict__ y, MaskRef 
 #pragma unroll
       for (int u = 0; u < kStreamUnroll; ++u) {
         const int pk = pk0 + u * BLOCK;
-        pv[u] = load_window_pack<TI, E, true>(xr, pk * E, nw, pk < npacks, -INFINITY);
+        pv[u] = stream_load<TI, E, true, WINDOW>(xr, pk * E, nw, pk < npacks, -INFINITY, h);
         if constexpr (MASKED) mv[u] = load_mask_pack<E, false>(mrow, pk * E, nw, pk < npacks, h);
       }
 #pragma unroll
@@ -326,20 +350,21 @@ softmax_bwd_resident_kernel(const TG* __restrict__ grad, const TG* __restrict__ 
   constexpr int E = elems_per_pack<TG>::value;
   constexpr int RPB = BLOCK / G;
   constexpr bool PRECISE = sizeof(TO) == 4 && sizeof(TG) == 4;
+  constexpr bool WINDOW = !FAST && softmax_row_window<TG>();
   __shared__ float red[reduce_lds_floats<G, BLOCK, 1>::value];
   int phase = 0;
   const int slot = threadIdx.x / G;
   const int lane = threadIdx.x % G;
   const bool is_log = (flags & kSoftmaxLog) != 0;
   // y's packs are aligned like grad's when the two base addresses are congruent
-  const bool y_whole = same_pack_alignment(grad, y);
+  const bool y_whole = WINDOW && same_pack_alignment(grad, y);
   const int64_t nrb = (M + RPB - 1) / RPB;
   for (int64_t rb = blockIdx.x; rb < nrb; rb += gridDim.x) {
     const int64_t row = rb * RPB + slot;
     const bool ok = RPB == 1 ? true : row < M;
     const int64_t rowc = ok ? row : 0;
-    // ragged rows go through the 16-byte aligned window that holds the row of grad
-    const int h = FAST ? 0 : window_head<TG, E>(grad + rowc * (int64_t)N);
+    // ragged 16-bit rows go through the 16-byte aligned window that holds the row of grad
+    const int h = WINDOW ? window_head<TG, E>(grad + rowc * (int64_t)N) : 0;
     const int nw = N + h;
     const TG* gr = grad + rowc * (int64_t)N - h;
     const TG* yr = y + rowc * (int64_t)N - h;
@@ -348,13 +373,13 @@ softmax_bwd_resident_kernel(const TG* __restrict__ grad, const TG* __restrict__ 
 #pragma unroll
     for (int c = 0; c < V; ++c) {
       const int e0 = (c * G + lane) * E;
-      pg[c] = row_load<TG, E, true, FAST>(gr, e0, nw, ok, 0.0f, h, true);
+      pg[c] = row_load<TG, E, true, FAST>(gr, e0, nw, ok, 0.0f, h, WINDOW);
       py[c] = row_load<TG, E, true, FAST>(yr, e0, nw, ok, 0.0f, h, y_whole);
     }
 #pragma unroll
     for (int c = 0; c < V; ++c) {
       const int e0 = (c * G + lane) * E;
-      row_trim<TG, E, FAST>(pg[c], e0, nw, 0.0f, h, true);
+      row_trim<TG, E, FAST>(pg[c], e0, nw, 0.0f, h, WINDOW);
       row_trim<TG, E, FAST>(py[c], e0, nw, 0.0f, h, y_whole);
     }
     float gf[V][E], yf[V][E];
@@ -410,10 +435,11 @@ softmax_bwd_stream_kernel(const TG* __restrict__ grad, const TG* __restrict__ y,
   constexpr int E = elems_per_pack<TG>::value;
   constexpr int U = kStreamUnroll;
   constexpr bool PRECISE = sizeof(TO) == 4 && sizeof(TG) == 4;
+  constexpr bool WINDOW = softmax_row_window<TG>();
   __shared__ float red[reduce_lds_floats<BLOCK, BLOCK, 1>::value];
   int phase = 0;
   const bool is_log = (flags & kSoftmaxLog) != 0;
-  const bool y_whole = same_pack_alignment(grad, y);
+  const bool y_whole = WINDOW && same_pack_alignment(grad, y);
   // a pack of y: whole when it is aligned like grad's, else element by element at the row ends
   auto load_y = [&](const TG* yr, int e0, int nw, bool in_row, int h, auto stream_tag) {
     constexpr bool STREAM = decltype(stream_tag)::value;
@@ -421,8 +447,8 @@ softmax_bwd_stream_kernel(const TG* __restrict__ grad, const TG* __restrict__ y,
                    : load_row_pack<TG, E, STREAM>(yr, e0, nw, in_row, 0.0f, h);
   };
   for (int64_t row = blockIdx.x; row < M; row += gridDim.x) {
-    // the 16-byte aligned window that holds the row of grad: elements [h, nw) of it
-    const int h = window_head<TG, E>(grad + row * (int64_t)N);
+    // 16-bit rows: the 16-byte aligned window that holds the row of grad, elements [h, nw) of it
+    const int h = WINDOW ? window_head<TG, E>(grad + row * (int64_t)N) : 0;
     const int nw = N + h;
     const int npacks = (nw + E - 1) / E;
     const TG* gr = grad + row * (int64_t)N - h;
@@ -442,7 +468,7 @@ softmax_bwd_stream_kernel(const TG* __restrict__ grad, const TG* __restrict__ y,
 #pragma unroll
       for (int u = 0; u < U; ++u) {
         const int pk = pk0 + u * BLOCK;
-        pg[u] = load_window_pack<TG, E, false>(gr, pk * E, nw, pk < npacks, 0.0f);
+        pg[u] = stream_load<TG, E, false, WINDOW>(gr, pk * E, nw, pk < npacks, 0.0f, h);
         if (!is_log) {
           py[u] = load_y(yr, pk * E, nw, pk < npacks, h, std::false_type{});
           if constexpr (MASKED) mk[u] = load_mask_pack<E, false>(mrow, pk * E, nw, pk < npacks, h);
@@ -450,7 +476,7 @@ softmax_bwd_stream_kernel(const TG* __restrict__ grad, const TG* __restrict__ y,
       }
 #pragma unroll
       for (int u = 0; u < U; ++u) {
-        trim_window_pack<TG, E>(pg[u], (pk0 + u * BLOCK) * E, nw, 0.0f, h);
+        if constexpr (WINDOW) trim_window_pack<TG, E>(pg[u], (pk0 + u * BLOCK) * E, nw, 0.0f, h);
         if (!is_log && y_whole) trim_window_pack<TG, E>(py[u], (pk0 + u * BLOCK) * E, nw, 0.0f, h);
         if (is_log) {
 #pragma unroll
@@ -470,7 +496,7 @@ softmax_bwd_stream_kernel(const TG* __restrict__ grad, const TG* __restrict__ y,
 #pragma unroll
       for (int u = 0; u < U; ++u) {
         const int pk = pk0 + u * BLOCK;
-        pg[u] = load_window_pack<TG, E, true>(gr, pk * E, nw, pk < npacks, 0.0f);
+        pg[u] = stream_load<TG, E, true, WINDOW>(gr, pk * E, nw, pk < npacks, 0.0f, h);
         py[u] = load_y(yr, pk * E, nw, pk < npacks, h, std::true_type{});
         if constexpr (MASKED) mk[u] = load_mask_pack<E, false>(mrow, pk * E, nw, pk < npacks, h);
       }
