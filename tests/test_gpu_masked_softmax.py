@@ -150,9 +150,16 @@ def test_safe_softmax(cabi, oracle, gpu, dtype):
         assert bool((yc[0] == 0).all())
         if M > 2:
             assert bool(torch.isnan(yc[2]).all())
-        # every other row is bit-identical to plain softmax
+        # every other row is plain softmax: NaN rows are NaN in both, and the values agree to
+        # one unit in the last place (the two code paths may round the last multiply and the
+        # conversion to 16 bits in one step or in two)
         plain = cabi.softmax_fwd(x.to(gpu)).cpu()
-        assert torch.equal(yc[1:].view(torch.uint8), plain[1:].view(torch.uint8))
+        assert torch.equal(torch.isnan(yc[1:]), torch.isnan(plain[1:]))
+        if M > 1:
+            ibits = torch.int32 if dtype == torch.float32 else torch.int16
+            ulps = (yc[1:].nan_to_num(nan=0.0).view(ibits).to(torch.int64) -
+                    plain[1:].nan_to_num(nan=0.0).view(ibits).to(torch.int64)).abs().max()
+            assert int(ulps) <= (0 if dtype == torch.float32 else 1), (dtype, M, N, int(ulps))
     # half input with a float result
     x = torch.randn(5, 300, generator=g).half()
     x[4] = float("-inf")

@@ -66,6 +66,14 @@ __device__ __forceinline__ Pack<T, E> stream_load(const T* row, int e0, int n, b
     return load_row_pack<T, E, STREAM>(row, e0, n, in_row, fill, lo);
 }
 
+// The kernels serve softmax and log_softmax (and the "safe" variant) from one
+// instance, told apart by run-time flags that are uniform over the launch.  Each
+// arm of such a choice opens with this marker: an empty volatile asm cannot be
+// speculated, so the compiler keeps one scalar branch around the arm instead
+// of computing both formulas for every element and selecting (which evaluated
+// the exponential in log_softmax's output pass and in softmax's backward too).
+#define ROWNORM_UNIFORM_ARM(tag) asm volatile("; " tag)
+
 // Packs a thread of the multi-pass kernels requests before using the first.
 constexpr int kStreamUnroll = 2;
 
@@ -168,19 +176,41 @@ softmax_fwd_resident_kernel(const TI* __restrict__ x, TO* __restrict__ y, MaskRe
         for (int i = 0; i < E; ++i) sum[0] += row_exp<PRECISE>(xp[c].get(i) - m);
       }
       group_allreduce<G, BLOCK, 1, SumOp>(sum, red, phase);
-      const float k = is_log ? logf(sum[0]) : 1.0f / sum[0];
-      const bool zero_row = is_safe && m == -INFINITY;
+      if (is_log) {
+        ROWNORM_UNIFORM_ARM("log_softmax: x - max - log(sum)");
+        const float k = logf(sum[0]);
 #pragma unroll
-      for (int c = 0; c < V; ++c) {
-        keep_packed(xp[c]);
-        Pack<TO, E> o;
+        for (int c = 0; c < V; ++c) {
+          keep_packed(xp[c]);
+          Pack<TO, E> o;
 #pragma unroll
-        for (int i = 0; i < E; ++i) {
-          const float d = xp[c].get(i) - m;
-          const float v = is_log ? d - k : row_exp<PRECISE>(d) * k;
-          o.set(i, zero_row ? 0.0f : v);
+          for (int i = 0; i < E; ++i) o.set(i, (xp[c].get(i) - m) - k);
+          row_store<TO, E, true, FAST>(yr, (c * G + lane) * E, nw, ok, o, h);
         }
-        row_store<TO, E, true, FAST>(yr, (c * G + lane) * E, nw, ok, o, h);
+      } else if (is_safe) {
+        ROWNORM_UNIFORM_ARM("safe softmax: zeros for a row without a finite element");
+        const float k = 1.0f / sum[0];
+        const bool zero_row = m == -INFINITY;
+#pragma unroll
+        for (int c = 0; c < V; ++c) {
+          keep_packed(xp[c]);
+          Pack<TO, E> o;
+#pragma unroll
+          for (int i = 0; i < E; ++i)
+            o.set(i, zero_row ? 0.0f : row_exp<PRECISE>(xp[c].get(i) - m) * k);
+          row_store<TO, E, true, FAST>(yr, (c * G + lane) * E, nw, ok, o, h);
+        }
+      } else {
+        ROWNORM_UNIFORM_ARM("softmax: exp(x - max) / sum");
+        const float k = 1.0f / sum[0];
+#pragma unroll
+        for (int c = 0; c < V; ++c) {
+          keep_packed(xp[c]);
+          Pack<TO, E> o;
+#pragma unroll
+          for (int i = 0; i < E; ++i) o.set(i, row_exp<PRECISE>(xp[c].get(i) - m) * k);
+          row_store<TO, E, true, FAST>(yr, (c * G + lane) * E, nw, ok, o, h);
+        }
       }
       continue;
     }
@@ -206,8 +236,10 @@ softmax_fwd_resident_kernel(const TI* __restrict__ x, TO* __restrict__ y, MaskRe
     group_allreduce<G, BLOCK, 1, MaxOp>(mx, red, phase);
     const float m = mx[0];
     float sum[1] = {0.0f};
+    // (no arm markers here: both arms evaluate exp(x - max) and differ in what
+    // they keep, which the compiler turns into one shared body by itself)
     if (is_log) {
-      // keep x - m; the exponentials are only needed for the sum
+      // keep x - max; the exponentials only feed the sum
 #pragma unroll
       for (int c = 0; c < V; ++c)
 #pragma unroll
@@ -225,18 +257,37 @@ softmax_fwd_resident_kernel(const TI* __restrict__ x, TO* __restrict__ y, MaskRe
         }
     }
     group_allreduce<G, BLOCK, 1, SumOp>(sum, red, phase);
-    const float k = is_log ? logf(sum[0]) : 1.0f / sum[0];
-    const bool zero_row = is_safe && m == -INFINITY;  // no finite element in the row
+    if (is_log) {
+      ROWNORM_UNIFORM_ARM("log_softmax: (x - max) - log(sum)");
+      const float k = logf(sum[0]);
 #pragma unroll
-    for (int c = 0; c < V; ++c) {
-      const int e0 = (c * G + lane) * E;
-      Pack<TO, E> o;
+      for (int c = 0; c < V; ++c) {
+        Pack<TO, E> o;
 #pragma unroll
-      for (int i = 0; i < E; ++i) {
-        const float v = is_log ? xf[c][i] - k : xf[c][i] * k;
-        o.set(i, zero_row ? 0.0f : v);
+        for (int i = 0; i < E; ++i) o.set(i, xf[c][i] - k);
+        row_store<TO, E, true, FAST>(yr, (c * G + lane) * E, nw, ok, o, h);
       }
-      row_store<TO, E, true, FAST>(yr, e0, nw, ok, o, h);
+    } else if (is_safe) {
+      ROWNORM_UNIFORM_ARM("safe softmax: zeros for a row without a finite element");
+      const float k = 1.0f / sum[0];
+      const bool zero_row = m == -INFINITY;
+#pragma unroll
+      for (int c = 0; c < V; ++c) {
+        Pack<TO, E> o;
+#pragma unroll
+        for (int i = 0; i < E; ++i) o.set(i, zero_row ? 0.0f : xf[c][i] * k);
+        row_store<TO, E, true, FAST>(yr, (c * G + lane) * E, nw, ok, o, h);
+      }
+    } else {
+      ROWNORM_UNIFORM_ARM("softmax: exp(x - max) * (1 / sum)");
+      const float k = 1.0f / sum[0];
+#pragma unroll
+      for (int c = 0; c < V; ++c) {
+        Pack<TO, E> o;
+#pragma unroll
+        for (int i = 0; i < E; ++i) o.set(i, xf[c][i] * k);
+        row_store<TO, E, true, FAST>(yr, (c * G + lane) * E, nw, ok, o, h);
+      }
     }
   }
 }
@@ -329,11 +380,17 @@ softmax_fwd_stream_kernel(const TI* __restrict__ x, TO* __restrict__ y, MaskRef 
       for (int u = 0; u < kStreamUnroll; ++u) {
         const int pk = pk0 + u * BLOCK;
         Pack<TO, E> o;
+        if (is_log) {
+          ROWNORM_UNIFORM_ARM("log_softmax");
 #pragma unroll
-        for (int i = 0; i < E; ++i) {
-          const float d = masked_value(pv[u], mv[u], i) - m;
-          const float v = is_log ? d - k : row_exp<PRECISE>(d) * k;
-          o.set(i, zero_row ? 0.0f : v);
+          for (int i = 0; i < E; ++i) o.set(i, (masked_value(pv[u], mv[u], i) - m) - k);
+        } else {
+          ROWNORM_UNIFORM_ARM("softmax");
+#pragma unroll
+          for (int i = 0; i < E; ++i) {
+            const float v = row_exp<PRECISE>(masked_value(pv[u], mv[u], i) - m) * k;
+            o.set(i, zero_row ? 0.0f : v);
+          }
         }
         store_row_pack<TO, E, true>(yr, pk * E, nw, pk < npacks, o, h);
       }
@@ -401,11 +458,13 @@ softmax_bwd_resident_kernel(const TG* __restrict__ grad, const TG* __restrict__ 
     }
     float sum[1] = {0.0f};
     if (is_log) {
+      ROWNORM_UNIFORM_ARM("log_softmax backward: sum of grad");
 #pragma unroll
       for (int c = 0; c < V; ++c)
 #pragma unroll
         for (int i = 0; i < E; ++i) sum[0] += gf[c][i];
     } else {
+      ROWNORM_UNIFORM_ARM("softmax backward: sum of y * grad");
 #pragma unroll
       for (int c = 0; c < V; ++c)
 #pragma unroll
@@ -413,17 +472,24 @@ softmax_bwd_resident_kernel(const TG* __restrict__ grad, const TG* __restrict__ 
     }
     group_allreduce<G, BLOCK, 1, SumOp>(sum, red, phase);
     const float s = sum[0];
+    if (is_log) {
+      ROWNORM_UNIFORM_ARM("log_softmax backward: grad - exp(y) * sum");
 #pragma unroll
-    for (int c = 0; c < V; ++c) {
-      const int e0 = (c * G + lane) * E;
-      Pack<TO, E> o;
+      for (int c = 0; c < V; ++c) {
+        Pack<TO, E> o;
 #pragma unroll
-      for (int i = 0; i < E; ++i) {
-        const float v = is_log ? gf[c][i] - row_exp<PRECISE>(yf[c][i]) * s
-                               : yf[c][i] * (gf[c][i] - s);
-        o.set(i, v);
+        for (int i = 0; i < E; ++i) o.set(i, gf[c][i] - row_exp<PRECISE>(yf[c][i]) * s);
+        row_store<TO, E, true, FAST>(outr, (c * G + lane) * E, nw, ok, o, h);
       }
-      row_store<TO, E, true, FAST>(outr, e0, nw, ok, o, h);
+    } else {
+      ROWNORM_UNIFORM_ARM("softmax backward: y * (grad - sum)");
+#pragma unroll
+      for (int c = 0; c < V; ++c) {
+        Pack<TO, E> o;
+#pragma unroll
+        for (int i = 0; i < E; ++i) o.set(i, yf[c][i] * (gf[c][i] - s));
+        row_store<TO, E, true, FAST>(outr, (c * G + lane) * E, nw, ok, o, h);
+      }
     }
   }
 }
@@ -479,9 +545,11 @@ softmax_bwd_stream_kernel(const TG* __restrict__ grad, const TG* __restrict__ y,
         if constexpr (WINDOW) trim_window_pack<TG, E>(pg[u], (pk0 + u * BLOCK) * E, nw, 0.0f, h);
         if (!is_log && y_whole) trim_window_pack<TG, E>(py[u], (pk0 + u * BLOCK) * E, nw, 0.0f, h);
         if (is_log) {
+          ROWNORM_UNIFORM_ARM("log_softmax backward: sum of grad");
 #pragma unroll
           for (int i = 0; i < E; ++i) sum[0] += pg[u].get(i);
         } else {
+          ROWNORM_UNIFORM_ARM("softmax backward: sum of y * grad");
 #pragma unroll
           for (int i = 0; i < E; ++i)
             sum[0] = fmaf(saved_output(py[u], mk[u], i), pg[u].get(i), sum[0]);
@@ -504,12 +572,16 @@ softmax_bwd_stream_kernel(const TG* __restrict__ grad, const TG* __restrict__ y,
       for (int u = 0; u < U; ++u) {
         const int pk = pk0 + u * BLOCK;
         Pack<TO, E> o;
+        if (is_log) {
+          ROWNORM_UNIFORM_ARM("log_softmax backward");
 #pragma unroll
-        for (int i = 0; i < E; ++i) {
-          const float yv = saved_output(py[u], mk[u], i);
-          const float v =
-              is_log ? pg[u].get(i) - row_exp<PRECISE>(yv) * s : yv * (pg[u].get(i) - s);
-          o.set(i, v);
+          for (int i = 0; i < E; ++i)
+            o.set(i, pg[u].get(i) - row_exp<PRECISE>(saved_output(py[u], mk[u], i)) * s);
+        } else {
+          ROWNORM_UNIFORM_ARM("softmax backward");
+#pragma unroll
+          for (int i = 0; i < E; ++i)
+            o.set(i, saved_output(py[u], mk[u], i) * (pg[u].get(i) - s));
         }
         store_row_pack<TO, E, true>(outr, pk * E, nw, pk < npacks, o, h);
       }
