@@ -153,27 +153,58 @@ softmax_strided_fwd_kernel(const TI* __restrict__ x, TO* __restrict__ y, int64_t
       for (int i = 0; i < E; ++i) sum[i] += row_exp<PRECISE>(xp[k].get(i) - mx[i]);
     }
     column_allreduce<BLOCK, E, SumOp>(sum, lay, red, phase);
+    // one scalar branch per run-time variant (see ROWNORM_UNIFORM_ARM)
     float kf[E];
-    bool zero[E];
+    if (is_log) {
+      ROWNORM_UNIFORM_ARM("log_softmax over a strided dimension");
 #pragma unroll
-    for (int i = 0; i < E; ++i) {
-      kf[i] = is_log ? logf(sum[i]) : 1.0f / sum[i];
-      zero[i] = is_safe && mx[i] == -INFINITY;
-    }
+      for (int i = 0; i < E; ++i) kf[i] = logf(sum[i]);
 #pragma unroll
-    for (int k = 0; k < V; ++k) {
-      keep_packed(xp[k]);
-      const int d = ty + k * TY;
-      const bool ok = tile.valid && d < D;
-      Pack<TO, E> o;
+      for (int k = 0; k < V; ++k) {
+        keep_packed(xp[k]);
+        const int d = ty + k * TY;
+        const bool ok = tile.valid && d < D;
+        Pack<TO, E> o;
+#pragma unroll
+        for (int i = 0; i < E; ++i) o.set(i, (xp[k].get(i) - mx[i]) - kf[i]);
+        TO* row = y + tile.slab + (int64_t)(ok ? d : 0) * inner;
+        row_store<TO, E, true, FAST>(row, tile.e0, inner, ok, o);
+      }
+    } else if (is_safe) {
+      ROWNORM_UNIFORM_ARM("safe softmax over a strided dimension");
+      bool zero[E];
 #pragma unroll
       for (int i = 0; i < E; ++i) {
-        const float dv = xp[k].get(i) - mx[i];
-        const float v = is_log ? dv - kf[i] : row_exp<PRECISE>(dv) * kf[i];
-        o.set(i, zero[i] ? 0.0f : v);
+        kf[i] = 1.0f / sum[i];
+        zero[i] = mx[i] == -INFINITY;
       }
-      TO* row = y + tile.slab + (int64_t)(ok ? d : 0) * inner;
-      row_store<TO, E, true, FAST>(row, tile.e0, inner, ok, o);
+#pragma unroll
+      for (int k = 0; k < V; ++k) {
+        keep_packed(xp[k]);
+        const int d = ty + k * TY;
+        const bool ok = tile.valid && d < D;
+        Pack<TO, E> o;
+#pragma unroll
+        for (int i = 0; i < E; ++i)
+          o.set(i, zero[i] ? 0.0f : row_exp<PRECISE>(xp[k].get(i) - mx[i]) * kf[i]);
+        TO* row = y + tile.slab + (int64_t)(ok ? d : 0) * inner;
+        row_store<TO, E, true, FAST>(row, tile.e0, inner, ok, o);
+      }
+    } else {
+      ROWNORM_UNIFORM_ARM("softmax over a strided dimension");
+#pragma unroll
+      for (int i = 0; i < E; ++i) kf[i] = 1.0f / sum[i];
+#pragma unroll
+      for (int k = 0; k < V; ++k) {
+        keep_packed(xp[k]);
+        const int d = ty + k * TY;
+        const bool ok = tile.valid && d < D;
+        Pack<TO, E> o;
+#pragma unroll
+        for (int i = 0; i < E; ++i) o.set(i, row_exp<PRECISE>(xp[k].get(i) - mx[i]) * kf[i]);
+        TO* row = y + tile.slab + (int64_t)(ok ? d : 0) * inner;
+        row_store<TO, E, true, FAST>(row, tile.e0, inner, ok, o);
+      }
     }
   }
 }
@@ -206,25 +237,46 @@ softmax_strided_bwd_kernel(const TG* __restrict__ grad, const TG* __restrict__ y
     }
     float sum[E];
 #pragma unroll
-    for (int i = 0; i < E; ++i) {
-      sum[i] = 0.0f;
+    for (int i = 0; i < E; ++i) sum[i] = 0.0f;
+    if (is_log) {
+      ROWNORM_UNIFORM_ARM("log_softmax backward over a strided dimension: sum of grad");
 #pragma unroll
-      for (int k = 0; k < V; ++k)
-        sum[i] = is_log ? sum[i] + pg[k].get(i) : fmaf(py[k].get(i), pg[k].get(i), sum[i]);
+      for (int i = 0; i < E; ++i)
+#pragma unroll
+        for (int k = 0; k < V; ++k) sum[i] += pg[k].get(i);
+    } else {
+      ROWNORM_UNIFORM_ARM("softmax backward over a strided dimension: sum of y * grad");
+#pragma unroll
+      for (int i = 0; i < E; ++i)
+#pragma unroll
+        for (int k = 0; k < V; ++k) sum[i] = fmaf(py[k].get(i), pg[k].get(i), sum[i]);
     }
     column_allreduce<BLOCK, E, SumOp>(sum, lay, red, phase);
+    if (is_log) {
+      ROWNORM_UNIFORM_ARM("log_softmax backward over a strided dimension");
 #pragma unroll
-    for (int k = 0; k < V; ++k) {
-      const int d = ty + k * TY;
-      const bool ok = tile.valid && d < D;
-      Pack<TO, E> o;
+      for (int k = 0; k < V; ++k) {
+        const int d = ty + k * TY;
+        const bool ok = tile.valid && d < D;
+        Pack<TO, E> o;
 #pragma unroll
-      for (int i = 0; i < E; ++i) {
-        const float g = pg[k].get(i), yv = py[k].get(i);
-        o.set(i, is_log ? g - row_exp<PRECISE>(yv) * sum[i] : yv * (g - sum[i]));
+        for (int i = 0; i < E; ++i)
+          o.set(i, pg[k].get(i) - row_exp<PRECISE>(py[k].get(i)) * sum[i]);
+        TO* row = gi + tile.slab + (int64_t)(ok ? d : 0) * inner;
+        row_store<TO, E, true, FAST>(row, tile.e0, inner, ok, o);
       }
-      TO* row = gi + tile.slab + (int64_t)(ok ? d : 0) * inner;
-      row_store<TO, E, true, FAST>(row, tile.e0, inner, ok, o);
+    } else {
+      ROWNORM_UNIFORM_ARM("softmax backward over a strided dimension");
+#pragma unroll
+      for (int k = 0; k < V; ++k) {
+        const int d = ty + k * TY;
+        const bool ok = tile.valid && d < D;
+        Pack<TO, E> o;
+#pragma unroll
+        for (int i = 0; i < E; ++i) o.set(i, py[k].get(i) * (pg[k].get(i) - sum[i]));
+        TO* row = gi + tile.slab + (int64_t)(ok ? d : 0) * inner;
+        row_store<TO, E, true, FAST>(row, tile.e0, inner, ok, o);
+      }
     }
   }
 }
@@ -275,11 +327,17 @@ softmax_strided_fwd_stream_kernel(const TI* __restrict__ x, TO* __restrict__ y, 
       const Pack<TI, E> p =
           load_row_pack<TI, E, true>(xs + (int64_t)d * inner, tile.e0, inner, tile.valid, -INFINITY);
       Pack<TO, E> o;
+      if (is_log) {
+        ROWNORM_UNIFORM_ARM("log_softmax");
 #pragma unroll
-      for (int i = 0; i < E; ++i) {
-        const float dlt = p.get(i) - mx[i];
-        const float v = is_log ? dlt - kf[i] : row_exp<PRECISE>(dlt) * kf[i];
-        o.set(i, (is_safe && mx[i] == -INFINITY) ? 0.0f : v);
+        for (int i = 0; i < E; ++i) o.set(i, (p.get(i) - mx[i]) - kf[i]);
+      } else {
+        ROWNORM_UNIFORM_ARM("softmax");
+#pragma unroll
+        for (int i = 0; i < E; ++i) {
+          const float v = row_exp<PRECISE>(p.get(i) - mx[i]) * kf[i];
+          o.set(i, (is_safe && mx[i] == -INFINITY) ? 0.0f : v);
+        }
       }
       store_row_pack<TO, E, true>(ys + (int64_t)d * inner, tile.e0, inner, tile.valid, o);
     }
@@ -326,10 +384,14 @@ softmax_strided_bwd_stream_kernel(const TG* __restrict__ grad, const TG* __restr
       const Pack<TG, E> pg = load_row_pack<TG, E, true>(gs + off, tile.e0, inner, tile.valid, 0.0f);
       const Pack<TG, E> py = load_row_pack<TG, E, true>(ys + off, tile.e0, inner, tile.valid, 0.0f);
       Pack<TO, E> o;
+      if (is_log) {
+        ROWNORM_UNIFORM_ARM("log_softmax backward");
 #pragma unroll
-      for (int i = 0; i < E; ++i) {
-        const float g = pg.get(i), yv = py.get(i);
-        o.set(i, is_log ? g - row_exp<PRECISE>(yv) * sum[i] : yv * (g - sum[i]));
+        for (int i = 0; i < E; ++i) o.set(i, pg.get(i) - row_exp<PRECISE>(py.get(i)) * sum[i]);
+      } else {
+        ROWNORM_UNIFORM_ARM("softmax backward");
+#pragma unroll
+        for (int i = 0; i < E; ++i) o.set(i, py.get(i) * (pg.get(i) - sum[i]));
       }
       store_row_pack<TO, E, true>(os + off, tile.e0, inner, tile.valid, o);
     }
