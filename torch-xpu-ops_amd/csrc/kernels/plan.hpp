@@ -122,7 +122,11 @@ constexpr bool variant_built(OpClass oc, int esize, int G, int V, bool fast) {
   // 40960-element bf16 row is 1024 lanes x 5 packs, not x 8): 3 or 5 packs a
   // lane from one wavefront up, anything up to the budget at 1024 lanes
   if (V & (V - 1)) {
-    if (!fast || V > v_max(oc, esize, G)) return false;
+    // ragged 16-bit softmax rows just above a power of two (N = 4097: 514 packs of
+    // the aligned window) take three packs on half the lanes as well
+    if (!fast)
+      return (oc == OC_SOFTMAX_FWD || oc == OC_SOFTMAX_BWD) && esize == 2 && G >= 64 && V == 3;
+    if (V > v_max(oc, esize, G)) return false;
     // softmax rows that need all 1024 lanes (vocabulary-sized) likewise
     // (and the 16-bit forward takes three packs a lane where that fits better)
     if (oc == OC_SOFTMAX_FWD && esize == 2) return G == kMaxG || (G >= 64 && V == 3);
@@ -233,12 +237,13 @@ inline int make_plan(OpClass oc, int64_t M, int64_t N, int esize, int num_cus, c
     bool group_exact = false;
     if ((oc == OC_NORM_FWD || oc == OC_NORM_BWD) && p.fast && ov.G == 0 && ov.V == 0)
       group_exact = norm_layout(oc, esize, packs, layer_norm, wide_weights, &G, &V);
-    // 16-bit softmax forward (its exp makes it the arithmetic-heavy one): a row
-    // that fills at most three quarters of the two-pack slots takes three packs
-    // on half the lanes (N = 5120: 62 -> 56 us, 10240: 120 -> 110 us at 16384 rows)
-    if (oc == OC_SOFTMAX_FWD && esize == 2 && p.fast && ov.G == 0 && ov.V == 0 && G >= 128 &&
-        packs <= (int64_t)G * 2 && packs * 4 <= (int64_t)G * 2 * 3 &&
-        variant_built(oc, esize, G / 2, 3, true)) {
+    // 16-bit softmax forward (its exp makes it the arithmetic-heavy one) and ragged
+    // 16-bit softmax rows in both directions: a row that fills at most three
+    // quarters of the two-pack slots takes three packs on half the lanes
+    // (N = 5120: 62 -> 56 us, 10240: 120 -> 110 us at 16384 rows)
+    if (softmax && esize == 2 && (oc == OC_SOFTMAX_FWD || !p.fast) && ov.G == 0 && ov.V == 0 &&
+        G >= 128 && packs <= (int64_t)G * 2 && packs * 4 <= (int64_t)G * 2 * 3 &&
+        variant_built(oc, esize, G / 2, 3, p.fast)) {
       G /= 2;
       V = 3;
       group_exact = true;
