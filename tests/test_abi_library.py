@@ -158,6 +158,44 @@ def test_plan_picks_resident_kernels_for_the_llama_shapes(cabi):
     assert cabi.plan(cabi.OP_SOFTMAX_FWD, 4, 1 << 20, cabi.F32, cabi.F32)["resident"] == 0
 
 
+def test_plan_layouts_for_hidden_sizes_that_are_not_powers_of_two(cabi):
+    """(lanes per row, packs per lane) of the measured exceptions to the power-of-two rule."""
+    def lay(op, N, dt, wdt=None):
+        p = cabi.plan(op, 16384, N, dt, dt if wdt is None else wdt)
+        assert p["resident"] == 1
+        return p["lanes_per_row"], p["packs_per_lane"]
+    BF, F32 = cabi.BF16, cabi.F32
+    LF, LB, RF, RB = (cabi.OP_LAYER_NORM_FWD, cabi.OP_LAYER_NORM_BWD, cabi.OP_RMS_NORM_FWD,
+                      cabi.OP_RMS_NORM_BWD)
+    # powers of two keep the rule: 2 packs (16-bit) / 4 packs (fp32) a lane
+    assert lay(RF, 4096, BF) == (256, 2) and lay(RB, 4096, BF) == (256, 2)
+    assert lay(LF, 8192, BF, F32) == (512, 2) and lay(LB, 8192, BF, F32) == (512, 2)
+    assert lay(LF, 1024, F32) == (64, 4)
+    # rows that fill at most 3/4 of the slots: three packs on fewer lanes (forward)
+    for N, want in ((1536, (64, 3)), (3072, (128, 3)), (5120, (256, 3)), (6144, (256, 3))):
+        assert lay(LF, N, BF) == want and lay(RF, N, BF) == want
+        assert lay(cabi.OP_SOFTMAX_FWD, N, BF) == want
+    assert lay(LF, 7168, BF) == (512, 2)                       # fills 7/8: the rule stands
+    assert lay(LB, 5120, BF) == (512, 2) and lay(RB, 5120, BF) == (512, 2)  # 16-bit backward keeps its lanes
+    assert lay(LF, 3072, BF, F32) == (256, 2)                  # fp32 weights below 512 lanes
+    assert lay(LF, 5120, BF, F32) == (256, 3)
+    assert lay(cabi.OP_SOFTMAX_BWD, 5120, BF) == (512, 2)
+    # 16-bit norm rows beyond 8192 elements: 512 lanes, not 1024
+    assert lay(LF, 10240, BF) == (512, 3) and lay(LB, 10240, BF) == (512, 3)
+    assert lay(RF, 12288, BF) == (512, 3) and lay(RB, 12288, BF) == (512, 3)
+    assert lay(LF, 16384, BF) == (512, 4) and lay(LB, 16384, BF) == (512, 4)
+    assert lay(RF, 16384, BF) == (512, 4) and lay(RB, 16384, BF) == (1024, 2)
+    assert lay(LF, 32768, BF) == (1024, 4)
+    # fp32 rows
+    assert lay(LF, 5120, F32) == (512, 3) and lay(LB, 5120, F32) == (512, 3)
+    assert lay(LF, 10240, F32) == (512, 5) and lay(RF, 10240, F32) == (1024, 3)
+    assert lay(LB, 10240, F32) == (1024, 3) and lay(LB, 16384, F32) == (1024, 4)
+    # ragged 16-bit softmax rows (the aligned window adds up to 7 elements in front)
+    assert lay(cabi.OP_SOFTMAX_FWD, 4097, cabi.F16) == (256, 3)
+    assert lay(cabi.OP_SOFTMAX_BWD, 4097, cabi.F16) == (256, 3)
+    assert lay(cabi.OP_SOFTMAX_FWD, 4097, F32) == (512, 4)
+
+
 def test_forced_variants(cabi):
     cabi.set_override(cabi.OP_SOFTMAX_FWD, -1)
     assert cabi.plan(cabi.OP_SOFTMAX_FWD, 64, 2048, cabi.BF16, cabi.BF16)["resident"] == 0

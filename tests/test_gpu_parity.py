@@ -18,7 +18,10 @@ pytestmark = pytest.mark.gpu
 DTYPES = [torch.float32, torch.float16, torch.bfloat16]
 # rows x normalized size: tiny, odd, power-of-two, wider than one wavefront / one workgroup
 SHAPES = [(1, 1), (3, 8), (7, 64), (5, 127), (64, 256), (33, 1024), (17, 2048), (9, 4097),
-          (12, 4096), (4, 5120), (6, 8192), (3, 16384), (2, 40000)]
+          (12, 4096), (4, 5120), (6, 8192), (3, 16384), (2, 40000),
+          # hidden sizes that are not powers of two: 3 or 5 packs a lane, 512 lanes beyond 8192
+          (10, 1536), (5, 2560), (7, 3072), (6, 6144), (5, 7168), (4, 10240), (5, 12288),
+          (3, 14336), (3, 20480)]
 
 
 def _mk(M, N, dtype, seed, wdtype=None):
