@@ -194,6 +194,9 @@ def test_plan_layouts_for_hidden_sizes_that_are_not_powers_of_two(cabi):
     assert lay(cabi.OP_SOFTMAX_FWD, 4097, cabi.F16) == (256, 3)
     assert lay(cabi.OP_SOFTMAX_BWD, 4097, cabi.F16) == (256, 3)
     assert lay(cabi.OP_SOFTMAX_FWD, 4097, F32) == (512, 4)
+    # ragged 16-bit norm rows: three packs in the forward, the rule in the backward
+    assert lay(LF, 4097, cabi.F16) == (256, 3) and lay(RF, 4097, BF) == (256, 3)
+    assert lay(LB, 4097, cabi.F16) == (512, 2)
 
 
 def test_forced_variants(cabi):

@@ -14,7 +14,8 @@
 // If V exceeds the per-op register budget V_max the multi-pass streaming
 // kernel is used instead.  Rows whose length is a whole number of packs take
 // the branch-free "fast" kernels; ragged rows (N % E != 0) take the general
-// ones, which exist for V = V_pref only.  Measured exceptions for rows that
+// ones, which exist for V = V_pref only (and three packs for 16-bit softmax and
+// the 16-bit norm forward).  Measured exceptions for rows that
 // leave many of those lanes idle (hidden sizes that are not powers of two) or
 // that would take 1024 lanes: norm_layout() and the softmax / GroupNorm rules
 // in make_plan() pick three or five packs a lane, or fewer lanes.  Workgroup
@@ -122,10 +123,11 @@ constexpr bool variant_built(OpClass oc, int esize, int G, int V, bool fast) {
   // 40960-element bf16 row is 1024 lanes x 5 packs, not x 8): 3 or 5 packs a
   // lane from one wavefront up, anything up to the budget at 1024 lanes
   if (V & (V - 1)) {
-    // ragged 16-bit softmax rows just above a power of two (N = 4097: 514 packs of
+    // ragged 16-bit rows just above a power of two (softmax N = 4097: 514 packs of
     // the aligned window) take three packs on half the lanes as well
     if (!fast)
-      return (oc == OC_SOFTMAX_FWD || oc == OC_SOFTMAX_BWD) && esize == 2 && G >= 64 && V == 3;
+      return (oc == OC_SOFTMAX_FWD || oc == OC_SOFTMAX_BWD || oc == OC_NORM_FWD) && esize == 2 &&
+             G >= 64 && V == 3;
     if (V > v_max(oc, esize, G)) return false;
     // softmax rows that need all 1024 lanes (vocabulary-sized) likewise
     // (and the 16-bit forward takes three packs a lane where that fits better)
@@ -237,11 +239,13 @@ inline int make_plan(OpClass oc, int64_t M, int64_t N, int esize, int num_cus, c
     bool group_exact = false;
     if ((oc == OC_NORM_FWD || oc == OC_NORM_BWD) && p.fast && ov.G == 0 && ov.V == 0)
       group_exact = norm_layout(oc, esize, packs, layer_norm, wide_weights, &G, &V);
-    // 16-bit softmax forward (its exp makes it the arithmetic-heavy one) and ragged
-    // 16-bit softmax rows in both directions: a row that fills at most three
-    // quarters of the two-pack slots takes three packs on half the lanes
-    // (N = 5120: 62 -> 56 us, 10240: 120 -> 110 us at 16384 rows)
-    if (softmax && esize == 2 && (oc == OC_SOFTMAX_FWD || !p.fast) && ov.G == 0 && ov.V == 0 &&
+    // 16-bit softmax forward (its exp makes it the arithmetic-heavy one), ragged
+    // 16-bit softmax rows in both directions and ragged 16-bit norm forward rows:
+    // a row that fills at most three quarters of the two-pack slots takes three
+    // packs on half the lanes (softmax N = 5120: 62 -> 56 us, 10240: 120 -> 110 us
+    // at 16384 rows; LayerNorm N = 4097: 60 -> 52 us at 8192 rows)
+    if (((softmax && (oc == OC_SOFTMAX_FWD || !p.fast)) || (oc == OC_NORM_FWD && !p.fast)) &&
+        esize == 2 && ov.G == 0 && ov.V == 0 &&
         G >= 128 && packs <= (int64_t)G * 2 && packs * 4 <= (int64_t)G * 2 * 3 &&
         variant_built(oc, esize, G / 2, 3, p.fast)) {
       G /= 2;
