@@ -15,8 +15,10 @@ prints ONE JSON line (see the keys below).  `roofline` covers the dominant opera
 one mi355x_rms_norm_bwd call (norm_bwd_resident_kernel + colsum_finalize_kernel), timed with a
 HIP event pair per call on the launch stream over a second run of the same K steps.  `cpu_baseline` is the scalar C oracle
 (oracle/, a port of the same arithmetic) timed on one host core; `cpu_aten` is PyTorch's CPU ATen
-path (the parity target) on all host cores.  `ops` lists every op of the family at its
-Llama-class configuration (informational, measured after the timed region).
+path (the parity target) on all host cores.  `stock_pytorch_rocm` is the same step through the
+kernels PyTorch-ROCm ships, on the same GPU.  `ops` lists every op of the family at its
+Llama-class configuration and `config5` the irregular shapes of configuration 5 (all
+informational, measured after the timed region).
 """
 import argparse
 import ctypes
@@ -174,12 +176,63 @@ def main():
             pass
 
     if not args.no_ops:
+        out["stock_pytorch_rocm"] = stock_step(torch, sets, w, M, N, eps, fwd_bytes + bwd_bytes)
         out["ops"] = per_op_table(torch, cabi, L, dev, stream, P)
         out["config5"] = stress_table(torch, cabi, L, dev, stream, P)
     del sets
     if not args.no_cpu:
         out["cpu_baseline"], out["cpu_aten"] = cpu_baselines(torch, M, N, eps, fwd_bytes + bwd_bytes)
     print(json.dumps(out))
+
+
+def stock_step(torch, sets, w, M, N, eps, step_bytes):
+    """The same forward+backward step through the kernels PyTorch-ROCm ships, for comparison
+    only: aten::_fused_rms_norm and aten::_fused_rms_norm_backward called directly on the same
+    buffers (F.rms_norm + autograd where those ops are missing); algorithmic GB/s of the step,
+    HIP events over 20 steps after 5 untimed ones."""
+    aten = torch.ops.aten
+    direct = hasattr(aten, "_fused_rms_norm") and hasattr(aten, "_fused_rms_norm_backward")
+    xs = [s["x"] for s in sets[:2]]
+    if not direct:
+        wr = w.clone().requires_grad_()
+        xs = [x.clone().requires_grad_() for x in xs]
+
+    def step(i):
+        x, dy = xs[i % len(xs)], sets[i % len(xs)]["dy"]
+        if direct:
+            y, rstd = aten._fused_rms_norm(x, [N], w, eps)
+            aten._fused_rms_norm_backward(dy, x, [N], rstd, w, [True, True])
+        else:
+            x.grad = None
+            wr.grad = None
+            torch.nn.functional.rms_norm(x, (N,), wr, eps).backward(dy)
+
+    try:
+        step(0)
+    except Exception:  # the ops exist but have no GPU kernel in this build
+        if not direct:
+            raise
+        direct = False
+        wr = w.clone().requires_grad_()
+        xs = [x.clone().requires_grad_() for x in xs]
+    for i in range(5):
+        step(i)
+    torch.cuda.synchronize()
+    a, b = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+    a.record()
+    for i in range(20):
+        step(i)
+    b.record()
+    torch.cuda.synchronize()
+    ms = a.elapsed_time(b) / 20
+    del xs
+    torch.cuda.empty_cache()
+    return {"value": round(step_bytes / (ms * 1e-3) / 1e9, 1), "unit": "GB/s",
+            "ms_per_step": round(ms, 5),
+            "what": "torch %s on the same GPU, same shapes: %s" % (
+                torch.__version__,
+                "aten::_fused_rms_norm + aten::_fused_rms_norm_backward" if direct
+                else "F.rms_norm + autograd backward (with autograd's own bookkeeping)")}
 
 
 def _time_rotating(torch, fns, iters=60, warm=30):
