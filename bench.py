@@ -252,15 +252,27 @@ def _time_rotating(torch, fns, iters=60, warm=30):
 def per_op_table(torch, cabi, L, dev, stream, P):
     """Every op of the family at its benchmark configuration: avg microseconds per call (HIP events
     over 60 back-to-back calls, after 30 untimed ones, rotating over buffer sets), algorithmic GB/s,
-    fraction of 8 TB/s."""
+    fraction of 8 TB/s; `stock_us` = the same call through the kernel PyTorch-ROCm ships (20
+    calls after 5), for comparison."""
     BF, F32 = cabi.BF16, cabi.F32
     rows = []
 
-    def add(name, nbytes, fns):
+    def add(name, nbytes, fns, stock=None, stock_note=None):
         us = _time_rotating(torch, fns)
         gbs = nbytes / us / 1e3
-        rows.append({"op": name, "us": round(us, 2), "GB/s": round(gbs, 1),
-                     "frac": round(gbs / HBM_PEAK_GBS, 4)})
+        row = {"op": name, "us": round(us, 2), "GB/s": round(gbs, 1),
+               "frac": round(gbs / HBM_PEAK_GBS, 4)}
+        if stock is not None:
+            # the same call through the kernel PyTorch-ROCm ships (its outputs are allocated
+            # by its caching allocator inside the call), for comparison only
+            try:
+                row["stock_us"] = round(_time_rotating(torch, stock, iters=20, warm=5), 2)
+            except Exception as e:  # an op without a GPU kernel in this torch build
+                row["stock_us"] = None
+                row["stock_error"] = type(e).__name__
+            if stock_note:
+                row["stock_note"] = stock_note
+        rows.append(row)
 
     # C1: native_layer_norm forward fp32 [4096, 1024] (32 MiB: cache resident, informational)
     M, N = 4096, 1024
@@ -270,7 +282,8 @@ def per_op_table(torch, cabi, L, dev, stream, P):
              torch.empty(M, device=dev), torch.empty(M, device=dev)) for _ in range(16)]
     add("C1 native_layer_norm fwd fp32 [4096,1024]", 2 * M * N * 4 + 2 * N * 4 + 2 * M * 4,
         [(lambda s=s: L.mi355x_layer_norm_fwd(P(s[0]), P(g), P(b), P(s[1]), P(s[2]), P(s[3]), M, N,
-                                              1e-5, F32, F32, stream)) for s in sets])
+                                              1e-5, F32, F32, stream)) for s in sets],
+        stock=[(lambda s=s: torch.ops.aten.native_layer_norm(s[0], [N], g, b, 1e-5)) for s in sets])
     del sets
 
     # C2: _fused_rms_norm bf16 [16384, 4096]
@@ -285,10 +298,14 @@ def per_op_table(torch, cabi, L, dev, stream, P):
     ws = torch.empty(max(nws, 1), dtype=torch.uint8, device=dev)
     add("C2 _fused_rms_norm fwd bf16 [16384,4096]", 2 * M * N * 2 + N * 2 + M * 4,
         [(lambda s=s: L.mi355x_rms_norm_fwd(P(s[0]), P(w), P(s[2]), P(s[3]), M, N, 1e-6, BF, BF,
-                                            stream)) for s in sets])
+                                            stream)) for s in sets],
+        stock=[(lambda s=s: torch.ops.aten._fused_rms_norm(s[0], [N], w, 1e-6)) for s in sets])
+    r2 = [s[3].view(M, 1) for s in sets]
     add("C2 _fused_rms_norm bwd bf16 [16384,4096]", 3 * M * N * 2 + M * 4 + 2 * N * 2,
         [(lambda s=s: L.mi355x_rms_norm_bwd(P(s[1]), P(s[0]), P(s[3]), P(w), P(s[4]), P(s[5]),
-                                            P(ws), nws, M, N, BF, BF, stream)) for s in sets])
+                                            P(ws), nws, M, N, BF, BF, stream)) for s in sets],
+        stock=[(lambda s=s, r=r: torch.ops.aten._fused_rms_norm_backward(
+            s[1], s[0], [N], r, w, [True, True])) for s, r in zip(sets, r2)])
     del sets
 
     # C4: native_layer_norm bf16 rows, fp32 gamma/beta [16384, 8192]
@@ -306,13 +323,20 @@ def per_op_table(torch, cabi, L, dev, stream, P):
         sets.append(s)
     nws = L.mi355x_layer_norm_bwd_workspace_bytes(M, N, BF, F32, 1, 1)
     ws = torch.empty(max(nws, 1), dtype=torch.uint8, device=dev)
+    g16, b16 = g.bfloat16(), b.bfloat16()
+    note16 = "bf16 gamma/beta: the stock kernel takes no fp32 weights beside bf16 rows"
     add("C4 native_layer_norm fwd bf16/fp32w [16384,8192]", 2 * M * N * 2 + 2 * N * 4 + 2 * M * 4,
         [(lambda s=s: L.mi355x_layer_norm_fwd(P(s[0]), P(g), P(b), P(s[2]), P(s[3]), P(s[4]), M, N,
-                                              1e-5, BF, F32, stream)) for s in sets])
+                                              1e-5, BF, F32, stream)) for s in sets],
+        stock=[(lambda s=s: torch.ops.aten.native_layer_norm(s[0], [N], g16, b16, 1e-5))
+               for s in sets], stock_note=note16)
     add("C4 native_layer_norm bwd bf16/fp32w [16384,8192]", 3 * M * N * 2 + 2 * M * 4 + 3 * N * 4,
         [(lambda s=s: L.mi355x_layer_norm_bwd(P(s[1]), P(s[0]), P(s[3]), P(s[4]), P(g), P(s[5]),
                                               P(s[6]), P(s[7]), P(ws), nws, M, N, BF, F32, stream))
-         for s in sets])
+         for s in sets],
+        stock=[(lambda s=s: torch.ops.aten.native_layer_norm_backward(
+            s[1], s[0], [N], s[3].view(M, 1), s[4].view(M, 1), g16, b16, [True, True, True]))
+            for s in sets], stock_note=note16)
     del sets
 
     # C3: softmax / log_softmax bf16 [4, 32, 2048, 2048] with a causal -inf mask
@@ -327,10 +351,13 @@ def per_op_table(torch, cabi, L, dev, stream, P):
     for is_log, nm in ((0, "_softmax"), (1, "_log_softmax")):
         add("C3 %s fwd bf16 [4,32,2048,2048]" % nm, 2 * R * N * 2,
             [(lambda s=s: L.mi355x_softmax_fwd(P(s[0]), P(s[2]), R, N, BF, BF, is_log, stream))
-             for s in sets])
+             for s in sets],
+            stock=[(lambda s=s: getattr(torch.ops.aten, nm)(s[0], -1, False)) for s in sets])
         add("C3 %s bwd bf16 [4,32,2048,2048]" % nm, 3 * R * N * 2,
             [(lambda s=s: L.mi355x_softmax_bwd(P(s[1]), P(s[2]), P(s[3]), R, N, BF, BF, is_log,
-                                               stream)) for s in sets])
+                                               stream)) for s in sets],
+            stock=[(lambda s=s: getattr(torch.ops.aten, nm + "_backward_data")(
+                s[1], s[2], -1, torch.bfloat16)) for s in sets])
     # the same scores through _safe_softmax, and through _masked_softmax with the causal mask
     # as a [T, T] bool tensor read in place and as a full-shape bool tensor
     add("C3 _safe_softmax fwd bf16 [4,32,2048,2048]", 2 * R * N * 2,
@@ -360,10 +387,13 @@ def per_op_table(torch, cabi, L, dev, stream, P):
                          torch.empty_like(xv)))
         add("_log_softmax fwd bf16 [%d,%d]" % (R, N), 2 * R * N * 2,
             [(lambda s=s: L.mi355x_softmax_fwd(P(s[0]), P(s[2]), R, N, BF, BF, 1, stream))
-             for s in sets])
+             for s in sets],
+            stock=[(lambda s=s: torch.ops.aten._log_softmax(s[0], -1, False)) for s in sets])
         add("_log_softmax bwd bf16 [%d,%d]" % (R, N), 3 * R * N * 2,
             [(lambda s=s: L.mi355x_softmax_bwd(P(s[1]), P(s[2]), P(s[3]), R, N, BF, BF, 1, stream))
-             for s in sets])
+             for s in sets],
+            stock=[(lambda s=s: torch.ops.aten._log_softmax_backward_data(
+                s[1], s[2], -1, torch.bfloat16)) for s in sets])
         del sets
         torch.cuda.empty_cache()
 
@@ -374,10 +404,13 @@ def per_op_table(torch, cabi, L, dev, stream, P):
              torch.empty(O, D, I, device=dev, dtype=torch.bfloat16)) for _ in range(4)]
     add("_softmax dim=1 fwd bf16 [256,21,16384]", 2 * O * D * I * 2,
         [(lambda s=s: L.mi355x_softmax_strided_fwd(P(s[0]), P(s[2]), O, D, I, BF, BF, 0, stream))
-         for s in sets])
+         for s in sets],
+        stock=[(lambda s=s: torch.ops.aten._softmax(s[0], 1, False)) for s in sets])
     add("_softmax dim=1 bwd bf16 [256,21,16384]", 3 * O * D * I * 2,
         [(lambda s=s: L.mi355x_softmax_strided_bwd(P(s[1]), P(s[2]), P(s[3]), O, D, I, BF, BF, 0,
-                                                   stream)) for s in sets])
+                                                   stream)) for s in sets],
+        stock=[(lambda s=s: torch.ops.aten._softmax_backward_data(s[1], s[2], 1, torch.bfloat16))
+               for s in sets])
     del sets
 
     # GroupNorm: a diffusion-UNet block, [64, 320, 64, 64] bf16, 32 groups (rows of 40960 elements)
@@ -398,11 +431,15 @@ def per_op_table(torch, cabi, L, dev, stream, P):
     ws = torch.empty(max(nws, 1), dtype=torch.uint8, device=dev)
     add("native_group_norm fwd bf16 [64,320,64,64] g32", 2 * Nb * C * HW * 2 + 2 * C * 2 + 2 * Nb * Gr * 2,
         [(lambda s=s: L.mi355x_group_norm_fwd(P(s[0]), P(g), P(b), P(s[2]), P(s[3]), P(s[4]), Nb, C,
-                                              HW, Gr, 1e-5, BF, BF, stream)) for s in sets])
+                                              HW, Gr, 1e-5, BF, BF, stream)) for s in sets],
+        stock=[(lambda s=s: torch.ops.aten.native_group_norm(s[0], g, b, Nb, C, HW, Gr, 1e-5))
+               for s in sets])
     add("native_group_norm bwd bf16 [64,320,64,64] g32", 3 * Nb * C * HW * 2 + 3 * C * 2 + 2 * Nb * Gr * 2,
         [(lambda s=s: L.mi355x_group_norm_bwd(P(s[1]), P(s[0]), P(s[3]), P(s[4]), P(g), P(s[5]),
                                               P(s[6]), P(s[7]), P(ws), nws, Nb, C, HW, Gr, BF, BF,
-                                              stream)) for s in sets])
+                                              stream)) for s in sets],
+        stock=[(lambda s=s: torch.ops.aten.native_group_norm_backward(
+            s[1], s[0], s[3], s[4], g, Nb, C, HW, Gr, [True, True, True])) for s in sets])
     del sets
     torch.cuda.empty_cache()
     return rows
