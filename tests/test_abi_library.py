@@ -199,6 +199,20 @@ def test_plan_layouts_for_hidden_sizes_that_are_not_powers_of_two(cabi):
     assert lay(LB, 4097, cabi.F16) == (512, 2)
 
 
+def test_forward_grid_grows_with_the_row_count(cabi):
+    """The norm forward keeps a workgroup to about 2 (RMSNorm) / 4 (LayerNorm) row blocks, twice
+    that with fp32 weights beside 16-bit rows, once the rows outgrow four resident grids."""
+    BF, F32 = cabi.BF16, cabi.F32
+    grid = lambda op, M, N, wd=BF: cabi.plan(op, M, N, BF, wd)["grid_blocks"]
+    assert grid(cabi.OP_RMS_NORM_FWD, 16384, 4096) == 8192       # 256 CUs x 32: the floor
+    assert grid(cabi.OP_LAYER_NORM_FWD, 16384, 8192, F32) == 4096
+    assert grid(cabi.OP_RMS_NORM_FWD, 65536, 4096) == 32768
+    assert grid(cabi.OP_LAYER_NORM_FWD, 65536, 4096) == 16384
+    assert grid(cabi.OP_LAYER_NORM_FWD, 65536, 4096, F32) == 8192
+    assert grid(cabi.OP_RMS_NORM_FWD, 262144, 2048) == 65536     # two rows a workgroup iteration
+    assert grid(cabi.OP_RMS_NORM_BWD, 262144, 4096) == 512       # backward: one partial row each
+
+
 def test_forced_variants(cabi):
     cabi.set_override(cabi.OP_SOFTMAX_FWD, -1)
     assert cabi.plan(cabi.OP_SOFTMAX_FWD, 64, 2048, cabi.BF16, cabi.BF16)["resident"] == 0

@@ -103,7 +103,8 @@ constexpr bool block_built(OpClass oc, int G, int block) {
 // workgroup.  Forward: four times as many workgroups as fit on the machine at
 // once, so that they drift out of phase (a grid that is exactly resident runs
 // its load and store phases in lockstep and loses 5-10% bandwidth) while each
-// still amortizes its weight loads over several rows.  Backward: every
+// still amortizes its weight loads over several rows (make_plan() grows this
+// grid with the row count).  Backward: every
 // workgroup emits one partial row of the dgamma/dbeta reduction, so the grid
 // is just what is resident at 1024 threads per CU.  Softmax has no per-column
 // state: one workgroup per row block.
@@ -302,7 +303,19 @@ inline int make_plan(OpClass oc, int64_t M, int64_t N, int esize, int num_cus, c
   const int64_t nrb = (M + p.rpb - 1) / p.rpb;
   const int bpc = ov.bpc > 0 ? ov.bpc : default_bpc(oc, p.block);
   int64_t grid = (int64_t)num_cus * bpc;
+  // The norm forward beyond a few tens of thousands of rows (measured on bf16 rows
+  // of 2048..8192 elements, 65536 and 262144 rows): a workgroup that walks more
+  // than a handful of row blocks loses bandwidth (32 iterations: 65 % against
+  // 76 %), one that walks too few reloads gamma/beta too often.  The grid grows
+  // with the row count so that a workgroup makes about 2 (RMSNorm) or 4
+  // (LayerNorm) iterations, twice that with fp32 weights beside 16-bit rows.
+  if (oc == OC_NORM_FWD && p.resident && ov.bpc == 0) {
+    const int iters = (layer_norm ? 4 : 2) * (wide_weights ? 2 : 1);
+    const int64_t want = (nrb + iters - 1) / iters;
+    if (grid < want) grid = want;
+  }
   if (grid > nrb) grid = nrb;
+  if (grid > 0x7fffffff) grid = 0x7fffffff;
   if (grid < 1) grid = 1;
   p.grid = grid;
   p.partial_rows = 0;
