@@ -199,6 +199,24 @@ def test_plan_layouts_for_hidden_sizes_that_are_not_powers_of_two(cabi):
     assert lay(LB, 4097, cabi.F16) == (512, 2)
 
 
+def test_group_norm_rows_take_512_lanes_while_two_workgroups_fit(cabi):
+    """GroupNorm rows that would spread over 1024 lanes take 512 lanes with 6..10 (forward) or 6..7
+    (backward) packs each; beyond that 1024 lanes with exactly the packs the row has."""
+    BF, F32 = cabi.BF16, cabi.F32
+    def lay(bwd, C, dt):  # [64, C, 64, 64] in 32 groups
+        p = cabi.group_norm_plan(bwd, 64, C, 4096, 32, dt)
+        return (p["lanes_per_row"], p["packs_per_lane"]) if p["resident"] else None
+    assert lay(0, 160, BF) == (512, 5) and lay(1, 160, BF) == (512, 5)
+    assert lay(0, 192, BF) == (512, 6) and lay(1, 192, BF) == (512, 6)
+    assert lay(0, 224, BF) == (512, 7) and lay(1, 224, BF) == (512, 7)
+    assert lay(0, 256, BF) == (512, 8) and lay(1, 256, BF) == (1024, 4)
+    assert lay(0, 320, BF) == (512, 10) and lay(1, 320, BF) == (1024, 5)
+    assert lay(0, 352, BF) == (1024, 6) and lay(1, 352, BF) == (1024, 6)
+    assert lay(0, 96, F32) == (512, 6) and lay(1, 96, F32) == (512, 6)
+    assert lay(0, 160, F32) == (512, 10) and lay(1, 128, F32) == (1024, 4)
+    assert lay(0, 352, F32) == (1024, 11) and lay(0, 384, F32) is None and lay(1, 160, F32) is None
+
+
 def test_forward_grid_grows_with_the_row_count(cabi):
     """The norm forward keeps a workgroup to about 2 (RMSNorm) / 4 (LayerNorm) row blocks, twice
     that with fp32 weights beside 16-bit rows, once the rows outgrow four resident grids."""

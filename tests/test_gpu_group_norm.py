@@ -23,7 +23,11 @@ DTYPES = [torch.float32, torch.float16, torch.bfloat16]
 SHAPES = [(2, 4, (), 2), (64, 32, (), 4), (256, 32, (), 4), (64, 32, (16,), 4), (256, 32, (4, 4), 4),
           (3, 6, (5,), 3), (2, 6, (7, 3), 2), (4, 64, (32, 32), 32), (2, 320, (16, 16), 32),
           (1, 8, (127,), 1), (3, 10, (4097,), 5), (2, 8, (64, 129), 2), (1, 4, (1 << 17,), 2),
-          (2, 6, (1,), 6), (5, 5, (5,), 1)]
+          (2, 6, (1,), 6), (5, 5, (5,), 1),
+          # rows of 6..10 packs a lane on 512 lanes (16-bit: L = 24576 .. 40960; fp32: 12288 ..
+          # 20480) and an fp32 row of 11 packs a lane on 1024 lanes
+          (2, 12, (64, 64), 2), (2, 14, (64, 64), 2), (2, 18, (64, 64), 2), (1, 20, (64, 64), 2),
+          (2, 12, (2048,), 2), (2, 14, (2048,), 2), (1, 20, (2048,), 2), (1, 22, (64, 64), 2)]
 CASES = load_golden("aten_cpu_group_norm.npz")
 
 

@@ -44,6 +44,7 @@
 
 #include "device/pack.hpp"
 #include "device/reduce.hpp"
+#include "plan.hpp"
 
 namespace rownorm {
 
@@ -53,6 +54,14 @@ struct GroupShape {
   int D;        // channels per group
   int groups;   // groups per sample
 };
+
+// Wavefronts per SIMD a resident kernel is compiled for (the second argument of
+// __launch_bounds__): the 512-lane layouts with 6 packs or more that the
+// planner prefers to 1024 lanes must leave room for two workgroups a compute
+// unit, i.e. 4 wavefronts per SIMD, 128 VGPRs a lane.
+constexpr int gn_min_waves(int G, int V, int max_v) {
+  return (G == 512 && V > 5 && V <= max_v) ? 4 : 1;
+}
 
 // Channel (index into gamma/beta) of element p of row `g` (p is clamped into the row).
 __device__ __forceinline__ int gn_channel(const GroupShape& s, int g, int p) {
@@ -71,7 +80,7 @@ __device__ __forceinline__ float gn_weight(const WT* w, int ch, float dflt) {
 // var = (s2 - s1*s1/L)/L; y uses (x - mean0) - s1/L so that a constant row
 // gives beta bit for bit.
 template <class T, class WT, int G, int V, int BLOCK, bool UNIFORM>
-__global__ void __launch_bounds__(BLOCK)
+__global__ void __launch_bounds__(BLOCK, gn_min_waves(G, V, group_half_lanes_max_v(OC_GROUP_FWD)))
 gn_fwd_resident_kernel(const T* __restrict__ x, const WT* __restrict__ gamma,
                        const WT* __restrict__ beta, T* __restrict__ y, WT* __restrict__ mean,
                        WT* __restrict__ rstd, int64_t rows, GroupShape s, float eps) {
@@ -245,7 +254,7 @@ struct gn_stage_floats {
 };
 
 template <class T, class WT, int G, int V, int BLOCK, bool UNIFORM>
-__global__ void __launch_bounds__(BLOCK)
+__global__ void __launch_bounds__(BLOCK, gn_min_waves(G, V, group_half_lanes_max_v(OC_GROUP_BWD)))
 gn_bwd_resident_kernel(const T* __restrict__ dy, const T* __restrict__ x,
                        const WT* __restrict__ mean, const WT* __restrict__ rstd,
                        const WT* __restrict__ gamma, T* __restrict__ dx,

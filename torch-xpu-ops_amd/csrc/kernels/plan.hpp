@@ -70,8 +70,10 @@ constexpr int v_max(OpClass oc, int esize, int G) {
     case OC_SOFTMAX_FWD: return 16;
     case OC_SOFTMAX_BWD: v = esize == 4 ? 16 : 8; break;
     // GroupNorm lanes hold the row (and dY) only, no weights or column sums, so
-    // 16-bit rows keep 8 packs a lane at 1024 lanes (128 VGPRs); fp32 rows halve
-    case OC_GROUP_FWD: return esize == 4 ? (G >= 1024 ? 8 : 16) : 8;
+    // 16-bit rows keep 8 packs a lane at 1024 lanes (128 VGPRs) and 10 at 512
+    // lanes (two workgroups a compute unit); the fp32 forward holds 11 at 1024
+    // lanes without spilling, the fp32 backward 4
+    case OC_GROUP_FWD: return esize == 4 ? (G >= 1024 ? 11 : 16) : (G == 512 ? 10 : 8);
     case OC_GROUP_BWD: return esize == 4 ? (G >= 1024 ? 4 : 8) : 8;
   }
   if (G >= 1024 && v > 1) v /= 2;
@@ -118,6 +120,15 @@ constexpr int default_bpc(OpClass oc, int block) {
 // dispatcher, the planner and the forced-variant check agree.
 constexpr bool is_group_class(OpClass oc) { return oc == OC_GROUP_FWD || oc == OC_GROUP_BWD; }
 
+// GroupNorm rows that would spread over 1024 lanes (one workgroup a compute
+// unit, whose load, reduce and store phases then run one after the other) take
+// 512 lanes with twice the packs instead while two such workgroups fit a compute
+// unit's registers (128 VGPRs a lane): up to 10 packs forward, 7 backward.
+// Measured on [64, C, 64, 64] in 32 groups: bf16 forward 71 -> 62 us (C = 320),
+// 57 -> 47 us (224); backward 76 -> 63 us (192), 88 -> 71 us (224); fp32
+// backward 66 -> 59 us (96).  Eight packs backward spill and gain nothing.
+constexpr int group_half_lanes_max_v(OpClass oc) { return oc == OC_GROUP_FWD ? 10 : 7; }
+
 constexpr bool variant_built(OpClass oc, int esize, int G, int V, bool fast) {
   if (G < kMinG || G > kMaxG || (G & (G - 1)) || V < 1 || V > kMaxV) return false;
   // GroupNorm rows take the packs they have, not the next power of two (a
@@ -137,7 +148,9 @@ constexpr bool variant_built(OpClass oc, int esize, int G, int V, bool fast) {
     // LayerNorm / RMSNorm rows of hidden sizes such as 5120, 6144, 10240, 12288
     // (640, 768, 1280, 1536 16-bit packs): 3 or 5 packs a lane
     if (!is_group_class(oc)) return G >= 64 && (V == 3 || V == 5);
-    return G == kMaxG || (G >= 64 && (V == 3 || V == 5));
+    // (and 6..10 packs on 512 lanes, which make_plan() prefers to 1024 lanes)
+    return G == kMaxG || (G >= 64 && (V == 3 || V == 5)) ||
+           (G == 512 && V <= group_half_lanes_max_v(oc));
   }
   if (V > v_max(oc, esize, G)) return false;
   // ragged rows: the general kernels exist for the preferred packs per lane only;
@@ -258,6 +271,11 @@ inline int make_plan(OpClass oc, int64_t M, int64_t N, int esize, int num_cus, c
       if (Gg > kMaxG) Gg = kMaxG;
       if (Gg >= 64) {
         int Vg = (int)((packs + Gg - 1) / Gg);
+        if (Gg == kMaxG && packs <= 512 * (int64_t)group_half_lanes_max_v(oc) &&
+            variant_built(oc, esize, 512, (int)((packs + 511) / 512), true)) {
+          Gg = 512;
+          Vg = (int)((packs + 511) / 512);
+        }
         while (Vg < kMaxV && !variant_built(oc, esize, Gg, Vg, true)) ++Vg;
         if (variant_built(oc, esize, Gg, Vg, true)) {
           G = Gg;
