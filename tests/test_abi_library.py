@@ -224,6 +224,9 @@ def test_forward_grid_grows_with_the_row_count(cabi):
     grid = lambda op, M, N, wd=BF: cabi.plan(op, M, N, BF, wd)["grid_blocks"]
     assert grid(cabi.OP_RMS_NORM_FWD, 16384, 4096) == 8192       # 256 CUs x 32: the floor
     assert grid(cabi.OP_LAYER_NORM_FWD, 16384, 8192, F32) == 4096
+    assert grid(cabi.OP_LAYER_NORM_FWD, 16384, 4096) == 8192
+    assert grid(cabi.OP_LAYER_NORM_FWD, 16384, 4096, F32) == 4096  # fp32 weights: half the floor
+    assert grid(cabi.OP_RMS_NORM_FWD, 16384, 4096, F32) == 8192
     assert grid(cabi.OP_RMS_NORM_FWD, 65536, 4096) == 32768
     assert grid(cabi.OP_LAYER_NORM_FWD, 65536, 4096) == 16384
     assert grid(cabi.OP_LAYER_NORM_FWD, 65536, 4096, F32) == 8192

@@ -319,7 +319,14 @@ inline int make_plan(OpClass oc, int64_t M, int64_t N, int esize, int num_cus, c
     p.rpb = 1;
   }
   const int64_t nrb = (M + p.rpb - 1) / p.rpb;
-  const int bpc = ov.bpc > 0 ? ov.bpc : default_bpc(oc, p.block);
+  int bpc = ov.bpc > 0 ? ov.bpc : default_bpc(oc, p.block);
+  // LayerNorm forward with fp32 gamma/beta beside 16-bit rows: every workgroup
+  // loads twice the weight bytes, so 256-thread workgroups take half the grid
+  // (16384 rows of bf16: N = 4096 53.0 -> 50.7 us, 5120 64.4 -> 62.0 us, 6144
+  // 75.7 -> 73.3 us; RMSNorm and 512-thread workgroups measured no gain)
+  if (ov.bpc == 0 && oc == OC_NORM_FWD && p.resident && layer_norm && wide_weights &&
+      p.block == 256)
+    bpc /= 2;
   int64_t grid = (int64_t)num_cus * bpc;
   // The norm forward beyond a few tens of thousands of rows (measured on bf16 rows
   // of 2048..8192 elements, 65536 and 262144 rows): a workgroup that walks more
