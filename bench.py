@@ -461,7 +461,7 @@ def stress_table(torch, cabi, L, dev, stream, P):
         res = {}
         for (M, N) in shapes:
             sets = []
-            for _ in range(2):
+            for _ in range(4):  # 4 x (x, dy, y, dx) outgrows the 256 MB Infinity Cache at every shape
                 x = off(M * N, dtype).copy_(torch.randn(M * N, device=dev))
                 dy = off(M * N, dtype).copy_(torch.randn(M * N, device=dev))
                 sets.append(dict(x=x, dy=dy, y=off(M * N, dtype), dx=off(M * N, dtype),

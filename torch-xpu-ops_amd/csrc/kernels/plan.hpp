@@ -15,7 +15,7 @@
 // kernel is used instead.  Rows whose length is a whole number of packs take
 // the branch-free "fast" kernels; ragged rows (N % E != 0) take the general
 // ones, which exist for V = V_pref only (and three packs for 16-bit softmax and
-// the 16-bit norm forward).  Measured exceptions for rows that
+// the 16-bit norms).  Measured exceptions for rows that
 // leave many of those lanes idle (hidden sizes that are not powers of two) or
 // that would take 1024 lanes: norm_layout() and the softmax / GroupNorm rules
 // in make_plan() pick three or five packs a lane, or fewer lanes.  Workgroup
@@ -138,7 +138,7 @@ constexpr bool variant_built(OpClass oc, int esize, int G, int V, bool fast) {
     // ragged 16-bit rows just above a power of two (softmax N = 4097: 514 packs of
     // the aligned window) take three packs on half the lanes as well
     if (!fast)
-      return (oc == OC_SOFTMAX_FWD || oc == OC_SOFTMAX_BWD || oc == OC_NORM_FWD) && esize == 2 &&
+      return (oc == OC_SOFTMAX_FWD || oc == OC_SOFTMAX_BWD || oc == OC_NORM_FWD || oc == OC_NORM_BWD) && esize == 2 &&
              G >= 64 && V == 3;
     if (V > v_max(oc, esize, G)) return false;
     // softmax rows that need all 1024 lanes (vocabulary-sized) likewise
@@ -254,11 +254,15 @@ inline int make_plan(OpClass oc, int64_t M, int64_t N, int esize, int num_cus, c
     if ((oc == OC_NORM_FWD || oc == OC_NORM_BWD) && p.fast && ov.G == 0 && ov.V == 0)
       group_exact = norm_layout(oc, esize, packs, layer_norm, wide_weights, &G, &V);
     // 16-bit softmax forward (its exp makes it the arithmetic-heavy one), ragged
-    // 16-bit softmax rows in both directions and ragged 16-bit norm forward rows:
+    // 16-bit softmax rows in both directions and ragged 16-bit norm rows:
     // a row that fills at most three quarters of the two-pack slots takes three
     // packs on half the lanes (softmax N = 5120: 62 -> 56 us, 10240: 120 -> 110 us
-    // at 16384 rows; LayerNorm N = 4097: 60 -> 52 us at 8192 rows)
-    if (((softmax && (oc == OC_SOFTMAX_FWD || !p.fast)) || (oc == OC_NORM_FWD && !p.fast)) &&
+    // at 16384 rows; at 8192 rows LayerNorm N = 4097: forward 60 -> 52 us, backward
+    // 89 -> 77 us, RMSNorm backward 84 -> 69 us; the RMSNorm backward from 1024
+    // lanes is the exception, N = 8193: 116 us against 123 us)
+    const bool ragged_norm = !p.fast && (oc == OC_NORM_FWD ||
+                                         (oc == OC_NORM_BWD && (layer_norm || G < kMaxG)));
+    if (((softmax && (oc == OC_SOFTMAX_FWD || !p.fast)) || ragged_norm) &&
         esize == 2 && ov.G == 0 && ov.V == 0 &&
         G >= 128 && packs <= (int64_t)G * 2 && packs * 4 <= (int64_t)G * 2 * 3 &&
         variant_built(oc, esize, G / 2, 3, p.fast)) {
