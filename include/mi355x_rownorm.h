@@ -79,7 +79,8 @@ typedef struct {
   int32_t packs_per_lane;  /* V: 16-byte packs each lane holds per row */
   int32_t block_threads;   /* threads per workgroup */
   int32_t rows_per_block;  /* rows a workgroup handles per iteration: block_threads / lanes_per_row */
-  int32_t reserved;
+  int32_t reserved;        /* mi355x_rownorm_plan: workgroups a row is split over (norm ops, few very
+                              long rows), else 0; mi355x_group_norm_plan: 1 when every pack lies in one channel */
   int64_t grid_blocks;     /* workgroups launched (persistent, grid-stride over rows) */
   int64_t partial_rows;    /* rows of the fp32 [partial_rows, N] column-sum workspace (backward only) */
 } rownorm_plan;
@@ -91,16 +92,22 @@ int mi355x_rownorm_abi_version(void);
 
 /* native_layer_norm forward.  Replaces layer_norm_kernel(X, gamma, beta, M, N, eps, Y*, mean*, rstd*)
  * (LayerNormKernels.h:19-28).  gamma/beta may be NULL (treated as 1 / 0,
- * LayerNormKernels.cpp:281-285); mean/rstd may be NULL (not written).
+ * LayerNormKernels.cpp:281-285); mean/rstd may be NULL (not written; a few
+ * rows far too long for the registers are then not split over workgroups).
  * w_dtype is the dtype of gamma and beta: equal to x_dtype, or ROWNORM_F32
  * with a 16-bit x (mixed precision, a CPU-ATen feature the reference lacks). */
 int mi355x_layer_norm_fwd(const void* x, const void* gamma, const void* beta, void* y,
                           float* mean, float* rstd, int64_t M, int64_t N, float eps,
                           rownorm_dtype x_dtype, rownorm_dtype w_dtype, void* stream);
 
-/* Bytes of scratch mi355x_layer_norm_bwd needs for this call (0 when neither
- * dgamma nor dbeta is wanted).  Replaces the at::empty/at::zeros scratch the
- * reference allocates inside its entry point (LayerNormKernels.cpp:1255-1264). */
+/* Bytes of scratch mi355x_layer_norm_bwd takes for this call.  Replaces the
+ * at::empty/at::zeros scratch the reference allocates inside its entry point
+ * (LayerNormKernels.cpp:1255-1264, Norm.h:263-283).  Two parts: the fp32 column
+ * sums behind dgamma/dbeta (0 when neither is wanted; a shorter workspace is
+ * ROWNORM_ERR_WORKSPACE), and, for a few rows far too long for the registers,
+ * the partial sums of the split-row dX (the regime of Norm.h:632-812), which
+ * follow the column sums.  A workspace that holds the first part only is
+ * accepted: every row's dX then stays on one workgroup. */
 size_t mi355x_layer_norm_bwd_workspace_bytes(int64_t M, int64_t N, rownorm_dtype x_dtype,
                                              rownorm_dtype w_dtype, int want_dgamma,
                                              int want_dbeta);

@@ -120,7 +120,9 @@ def dtype_code(dt):
 def plan(op, M, N, x_dtype=F32, w_dtype=F32):
     p = Plan()
     _check(lib().mi355x_rownorm_plan(op, M, N, x_dtype, w_dtype, ctypes.byref(p)), "plan")
-    return p.as_dict()
+    d = p.as_dict()
+    d["row_chunks"] = p.reserved  # workgroups a row is split over (0: not split)
+    return d
 
 
 def set_override(op, lanes_per_row=0, packs_per_lane=0, block_threads=0, blocks_per_cu=0):

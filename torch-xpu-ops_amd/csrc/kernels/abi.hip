@@ -140,13 +140,19 @@ int norm_fwd(const void* x, const void* gamma, const void* beta, void* y, float*
                            : launch_norm_fwd<bf16, bf16, RMS>(plan, a, s);
 }
 
+// Bytes of the [M, split, 2] fp32 partial sums of the split-row backward (0: not split).
+size_t split_bytes(const Plan& plan, int64_t M) {
+  return plan.split > 1 ? (size_t)M * (size_t)plan.split * 2 * sizeof(float) : 0;
+}
+
 size_t norm_bwd_workspace(int op, int64_t M, int64_t N, int xd, int wd, int nparts) {
-  if (!norm_dtypes_ok(xd, wd) || shape_check(M, N) || M == 0 || N == 0 || nparts == 0) return 0;
+  if (!norm_dtypes_ok(xd, wd) || shape_check(M, N) || M == 0 || N == 0) return 0;
   Plan plan;
-  if (make_plan(OC_NORM_BWD, M, N, esize_of(xd), current_num_cus(), g_override[op], true, &plan,
-                false, op == ROWNORM_OP_LAYER_NORM_BWD, esize_of(wd) > esize_of(xd)))
+  if (make_plan(OC_NORM_BWD, M, N, esize_of(xd), current_num_cus(), g_override[op], nparts > 0,
+                &plan, false, op == ROWNORM_OP_LAYER_NORM_BWD, esize_of(wd) > esize_of(xd)))
     return 0;
-  return (size_t)plan.partial_rows * (size_t)N * sizeof(float) * (size_t)nparts;
+  return (size_t)plan.partial_rows * (size_t)N * sizeof(float) * (size_t)nparts +
+         split_bytes(plan, M);
 }
 
 template <bool RMS>
@@ -167,14 +173,19 @@ int norm_bwd(const void* dy, const void* x, const float* mean, const float* rstd
     return e;
   float* part_dg = nullptr;
   float* part_db = nullptr;
+  size_t need = 0;
   if (want_cols) {
     const size_t one = (size_t)plan.partial_rows * (size_t)N * sizeof(float);
-    const size_t need = one * (RMS ? 1 : 2);
+    need = one * (RMS ? 1 : 2);
     if (!workspace || workspace_bytes < need) return ROWNORM_ERR_WORKSPACE;
     part_dg = (float*)workspace;
     part_db = RMS ? nullptr : (float*)((char*)workspace + one);
   }
   NormBwdArgs a{dy, x, mean, rstd, gamma, dx, dgamma, dbeta, part_dg, part_db, M, (int)N};
+  // the split-row dX takes its partial sums behind the column sums when the
+  // caller brought the room for them; without it a row stays on one workgroup
+  if (dx && workspace && split_bytes(plan, M) > 0 && workspace_bytes >= need + split_bytes(plan, M))
+    a.split_ws = (float*)((char*)workspace + need);
   hipStream_t s = (hipStream_t)stream;
   if (xd == ROWNORM_F32) return launch_norm_bwd<float, float, RMS>(plan, a, s);
   if (xd == ROWNORM_F16)
@@ -577,7 +588,7 @@ int mi355x_rownorm_plan(rownorm_op op, int64_t M, int64_t N, rownorm_dtype x_dty
   out->packs_per_lane = plan.V;
   out->block_threads = plan.block;
   out->rows_per_block = plan.rpb;
-  out->reserved = 0;
+  out->reserved = plan.split > 1 ? plan.split : 0;
   out->grid_blocks = plan.grid;
   out->partial_rows = plan.partial_rows;
   return 0;

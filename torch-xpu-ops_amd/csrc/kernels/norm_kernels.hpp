@@ -28,6 +28,7 @@
 #include <type_traits>
 
 #include "device/pack.hpp"
+#include "plan.hpp"
 #include "device/reduce.hpp"
 
 namespace rownorm {
@@ -337,6 +338,127 @@ norm_fwd_stream_kernel(const T* __restrict__ x, const WT* __restrict__ gamma,
 }
 
 // ---------------------------------------------------------------------------
+// Split-row forward: few rows, each far beyond the registers (the regime of the
+// reference's split-row kernels, Norm.h:632-812).  A row is cut into `chunks`
+// chunks of `chunk_packs` packs; workgroup (chunk, row) of the first launch sums
+// its chunk, a second launch adds a row's partial sums in a fixed order and
+// writes mean / rstd, a third normalizes chunk by chunk.  The partial sums cross
+// the launches in the first bytes of the row's own Y, which the third launch
+// overwrites afterwards: no workspace, and the result does not depend on which
+// workgroup runs when.  LayerNorm sums (x - k), (x - k)^2 with k the median of
+// the row's first three elements, as the resident 16-bit kernel does.
+template <class T>
+__device__ __forceinline__ float* split_row_scratch(T* y_row) {
+  return reinterpret_cast<float*>((reinterpret_cast<uintptr_t>(y_row) + 3) & ~uintptr_t(3));
+}
+
+template <class T>
+__device__ __forceinline__ float split_row_centre(const T* xr, int N) {
+  const float a = (float)xr[0], b = (float)xr[N > 1 ? 1 : 0], c = (float)xr[N > 2 ? 2 : 0];
+  return fmaxf(fminf(a, b), fminf(fmaxf(a, b), c));
+}
+
+template <class T, int BLOCK, bool RMS>
+__global__ void __launch_bounds__(BLOCK)
+norm_fwd_split_sums_kernel(const T* __restrict__ x, T* __restrict__ y, int N,
+                           int64_t chunk_packs) {
+  constexpr int E = elems_per_pack<T>::value;
+  __shared__ float red[reduce_lds_floats<BLOCK, BLOCK, 2>::value];
+  int phase = 0;
+  const int64_t row = blockIdx.y;
+  const T* xr = x + row * (int64_t)N;
+  const int64_t npacks = ((int64_t)N + E - 1) / E;
+  const int64_t p0 = (int64_t)blockIdx.x * chunk_packs;
+  const int64_t p1 = p0 + chunk_packs < npacks ? p0 + chunk_packs : npacks;
+  const float k = RMS ? 0.0f : split_row_centre(xr, N);
+  float acc[2] = {0.0f, 0.0f};
+  for (int64_t pk = p0 + threadIdx.x; pk < p1; pk += BLOCK) {
+    const int e0 = (int)(pk * E);
+    const Pack<T, E> p = load_row_pack<T, E, false>(xr, e0, N, true, 0.0f);
+    const int nvalid = N - e0;
+#pragma unroll
+    for (int i = 0; i < E; ++i) {
+      const float d = (i < nvalid) ? p.get(i) - k : 0.0f;
+      acc[0] += d;
+      acc[1] = fmaf(d, d, acc[1]);
+    }
+  }
+  group_allreduce<BLOCK, BLOCK, 2, SumOp>(acc, red, phase);
+  if (threadIdx.x == 0) {
+    float* sc = split_row_scratch(y + row * (int64_t)N);
+    sc[2 * blockIdx.x] = acc[0];
+    sc[2 * blockIdx.x + 1] = acc[1];
+  }
+}
+
+// One wavefront per row: lane l adds partial sums l, l + 64, ... and a butterfly
+// adds the lanes, the same order on every run.
+template <class T, bool RMS>
+__global__ void __launch_bounds__(64)
+norm_fwd_split_stats_kernel(const T* __restrict__ x, T* __restrict__ y,
+                            float* __restrict__ mean, float* __restrict__ rstd, int N, int chunks,
+                            float eps) {
+  const int64_t row = blockIdx.x;
+  const float* sc = split_row_scratch(y + row * (int64_t)N);
+  float s1 = 0.0f, s2 = 0.0f;
+  for (int c = threadIdx.x; c < chunks; c += 64) {
+    s1 += sc[2 * c];
+    s2 += sc[2 * c + 1];
+  }
+  s1 = wave_group_allreduce<64, SumOp>(s1);
+  s2 = wave_group_allreduce<64, SumOp>(s2);
+  if (threadIdx.x == 0) {
+    const float fN = (float)N;
+    if constexpr (RMS) {
+      rstd[row] = 1.0f / sqrtf(s2 / fN + eps);
+    } else {
+      const float k = split_row_centre(x + row * (int64_t)N, N);
+      const float m1 = s1 / fN;
+      const float var = fmaxf((s2 - s1 * m1) / fN, 0.0f);
+      mean[row] = k + m1;
+      rstd[row] = 1.0f / sqrtf(var + eps);
+    }
+  }
+}
+
+template <class T, class WT, int BLOCK, bool RMS>
+__global__ void __launch_bounds__(BLOCK)
+norm_fwd_split_apply_kernel(const T* __restrict__ x, const WT* __restrict__ gamma,
+                            const WT* __restrict__ beta, T* __restrict__ y,
+                            const float* __restrict__ mean, const float* __restrict__ rstd, int N,
+                            int64_t chunk_packs) {
+  constexpr int E = elems_per_pack<T>::value;
+  const int64_t row = blockIdx.y;
+  const T* xr = x + row * (int64_t)N;
+  T* yr = y + row * (int64_t)N;
+  const int64_t npacks = ((int64_t)N + E - 1) / E;
+  const int64_t p0 = (int64_t)blockIdx.x * chunk_packs;
+  const int64_t p1 = p0 + chunk_packs < npacks ? p0 + chunk_packs : npacks;
+  const float mu = RMS ? 0.0f : mean[row];
+  const float rs = rstd[row];
+  for (int64_t pk = p0 + threadIdx.x; pk < p1; pk += BLOCK) {
+    const int e0 = (int)(pk * E);
+    const Pack<T, E> p = load_row_pack<T, E, true>(xr, e0, N, true, 0.0f);
+    const Pack<WT, E> pg = gamma ? load_row_pack<WT, E, false>(gamma, e0, N, true, 1.0f)
+                                 : Pack<WT, E>::splat(1.0f);
+    Pack<WT, E> pb = Pack<WT, E>::zero();
+    if constexpr (!RMS)
+      if (beta) pb = load_row_pack<WT, E, false>(beta, e0, N, true, 0.0f);
+    Pack<T, E> o;
+#pragma unroll
+    for (int i = 0; i < E; ++i) {
+      float v;
+      if constexpr (RMS)
+        v = (p.get(i) * rs) * pg.get(i);
+      else
+        v = ((p.get(i) - mu) * rs) * pg.get(i) + pb.get(i);
+      o.set(i, v);
+    }
+    store_row_pack<T, E, true>(yr, e0, N, true, o);
+  }
+}
+
+// ---------------------------------------------------------------------------
 // Backward, rows resident in registers: X and dY are read once, dX written
 // once, and each lane keeps the dgamma/dbeta sums of its own columns in fp32
 // registers over all the rows its workgroup visits.  At the end the BLOCK/G
@@ -586,6 +708,95 @@ norm_bwd_stream_dx_kernel(const T* __restrict__ dy, const T* __restrict__ x,
   }
 }
 
+// Split-row backward dX (see the split-row forward): workgroup (chunk, row) of
+// the first launch leaves its chunk's s1 = sum dy*gamma and s2 = sum dy*gamma*xhat
+// in split_ws[row][chunk]; every workgroup of the second launch adds its row's
+// partial sums in the same fixed order and writes dX for its chunk.
+template <class T, class WT, int BLOCK, bool RMS>
+__global__ void __launch_bounds__(BLOCK)
+norm_bwd_split_sums_kernel(const T* __restrict__ dy, const T* __restrict__ x,
+                           const float* __restrict__ mean, const float* __restrict__ rstd,
+                           const WT* __restrict__ gamma, float* __restrict__ split_ws, int N,
+                           int64_t chunk_packs) {
+  constexpr int E = elems_per_pack<T>::value;
+  __shared__ float red[reduce_lds_floats<BLOCK, BLOCK, 2>::value];
+  int phase = 0;
+  const int64_t row = blockIdx.y;
+  const T* xr = x + row * (int64_t)N;
+  const T* gr = dy + row * (int64_t)N;
+  const int64_t npacks = ((int64_t)N + E - 1) / E;
+  const int64_t p0 = (int64_t)blockIdx.x * chunk_packs;
+  const int64_t p1 = p0 + chunk_packs < npacks ? p0 + chunk_packs : npacks;
+  const float mu = RMS ? 0.0f : mean[row];
+  const float rs = rstd[row];
+  float acc[2] = {0.0f, 0.0f};
+  for (int64_t pk = p0 + threadIdx.x; pk < p1; pk += BLOCK) {
+    const int e0 = (int)(pk * E);
+    const Pack<T, E> px = load_row_pack<T, E, false>(xr, e0, N, true, 0.0f);
+    const Pack<T, E> pd = load_row_pack<T, E, false>(gr, e0, N, true, 0.0f);
+    const Pack<WT, E> pg = gamma ? load_row_pack<WT, E, false>(gamma, e0, N, true, 1.0f)
+                                 : Pack<WT, E>::splat(1.0f);
+#pragma unroll
+    for (int i = 0; i < E; ++i) {
+      const float g = pd.get(i) * pg.get(i);
+      acc[0] += g;
+      acc[1] = fmaf(g, (px.get(i) - mu) * rs, acc[1]);
+    }
+  }
+  group_allreduce<BLOCK, BLOCK, 2, SumOp>(acc, red, phase);
+  if (threadIdx.x == 0) {
+    float* sc = split_ws + (row * gridDim.x + blockIdx.x) * 2;
+    sc[0] = acc[0];
+    sc[1] = acc[1];
+  }
+}
+
+template <class T, class WT, int BLOCK, bool RMS>
+__global__ void __launch_bounds__(BLOCK)
+norm_bwd_split_dx_kernel(const T* __restrict__ dy, const T* __restrict__ x,
+                         const float* __restrict__ mean, const float* __restrict__ rstd,
+                         const WT* __restrict__ gamma, const float* __restrict__ split_ws,
+                         T* __restrict__ dx, int N, int64_t chunk_packs) {
+  constexpr int E = elems_per_pack<T>::value;
+  static_assert(BLOCK >= kSplitMaxChunks, "one thread per partial sum");
+  __shared__ float red[reduce_lds_floats<BLOCK, BLOCK, 2>::value];
+  int phase = 0;
+  const int64_t row = blockIdx.y;
+  const T* xr = x + row * (int64_t)N;
+  const T* gr = dy + row * (int64_t)N;
+  T* dr = dx + row * (int64_t)N;
+  const int64_t npacks = ((int64_t)N + E - 1) / E;
+  const int64_t p0 = (int64_t)blockIdx.x * chunk_packs;
+  const int64_t p1 = p0 + chunk_packs < npacks ? p0 + chunk_packs : npacks;
+  const float mu = RMS ? 0.0f : mean[row];
+  const float rs = rstd[row];
+  float acc[2] = {0.0f, 0.0f};
+  if (threadIdx.x < gridDim.x) {
+    const float* sc = split_ws + (row * gridDim.x + threadIdx.x) * 2;
+    acc[0] = sc[0];
+    acc[1] = sc[1];
+  }
+  group_allreduce<BLOCK, BLOCK, 2, SumOp>(acc, red, phase);
+  const float fN = (float)N;
+  const float term1 = rs / fN;
+  for (int64_t pk = p0 + threadIdx.x; pk < p1; pk += BLOCK) {
+    const int e0 = (int)(pk * E);
+    const Pack<T, E> px = load_row_pack<T, E, true>(xr, e0, N, true, 0.0f);
+    const Pack<T, E> pd = load_row_pack<T, E, true>(gr, e0, N, true, 0.0f);
+    const Pack<WT, E> pg = gamma ? load_row_pack<WT, E, false>(gamma, e0, N, true, 1.0f)
+                                 : Pack<WT, E>::splat(1.0f);
+    Pack<T, E> o;
+#pragma unroll
+    for (int i = 0; i < E; ++i) {
+      float f = fN * (pd.get(i) * pg.get(i));
+      f -= ((px.get(i) - mu) * rs) * acc[1];
+      if constexpr (!RMS) f -= acc[0];
+      o.set(i, f * term1);
+    }
+    store_row_pack<T, E, true>(dr, e0, N, true, o);
+  }
+}
+
 // Column sums for rows too wide for registers: workgroup (bx, by) owns the
 // BLOCK*E columns starting at bx*BLOCK*E and the rows by, by+gridDim.y, ...;
 // it writes row `by` of the [gridDim.y, N] partial buffers.
@@ -672,6 +883,33 @@ colsum_finalize_kernel(const float* __restrict__ part0, const float* __restrict_
     }
     if (col < N) out[col] = (WT)((s0 + s1) + (s2 + s3));
   }
+}
+
+// The same sum for a handful of partial rows under very many columns (few, very
+// long rows): a thread owns 4 adjacent columns and walks the P rows itself, so
+// a workgroup of 256 threads covers 1024 columns and nothing crosses lanes.
+constexpr int kFinalizeFlatRows = 16;
+constexpr int kFinalizeFlatCols = 1024;
+
+template <class WT>
+__global__ void __launch_bounds__(256)
+colsum_finalize_flat_kernel(const float* __restrict__ part0, const float* __restrict__ part1,
+                            WT* __restrict__ out0, WT* __restrict__ out1, int P, int N) {
+  const float* part = blockIdx.y == 0 ? part0 : part1;
+  WT* out = blockIdx.y == 0 ? out0 : out1;
+  if (part == nullptr || out == nullptr) return;  // uniform per workgroup
+  const int col0 = (blockIdx.x * 256 + threadIdx.x) * 4;
+  if (col0 >= N) return;
+  float a[4] = {0.0f, 0.0f, 0.0f, 0.0f};
+  for (int p = 0; p < P; ++p) {
+    const Pack<float, 4> v = load_row_pack<float, 4, false>(part + (int64_t)p * N, col0, N, true,
+                                                           0.0f);
+#pragma unroll
+    for (int i = 0; i < 4; ++i) a[i] += v.get(i);
+  }
+#pragma unroll
+  for (int i = 0; i < 4; ++i)
+    if (col0 + i < N) out[col0 + i] = (WT)a[i];
 }
 
 }  // namespace rownorm

@@ -32,6 +32,19 @@ struct NormFwdLauncher {
   };
 };
 
+// The split-row forward keeps a row's partial sums in the first bytes of the
+// row's Y and hands the statistics to its last launch through mean / rstd: it
+// needs those outputs, and a Y that does not overlap X.
+template <class T, bool RMS>
+inline bool norm_fwd_can_split(const Plan& plan, const NormFwdArgs& a) {
+  if (plan.split <= 1 || a.M > 65535 || a.rstd == nullptr || (!RMS && a.mean == nullptr))
+    return false;
+  const char* xb = (const char*)a.x;
+  const char* yb = (const char*)a.y;
+  const int64_t bytes = a.M * (int64_t)a.N * (int64_t)sizeof(T);
+  return yb + bytes <= xb || xb + bytes <= yb;
+}
+
 template <class T, class WT, bool RMS>
 int launch_norm_fwd(const Plan& plan, const NormFwdArgs& a, hipStream_t stream) {
   if (plan.resident) {
@@ -40,6 +53,17 @@ int launch_norm_fwd(const Plan& plan, const NormFwdArgs& a, hipStream_t stream) 
         plan.fast ? launch_variant<NormFwdLauncher<T, WT, RMS, true>::template At>(ctx)
                   : launch_variant<NormFwdLauncher<T, WT, RMS, false>::template At>(ctx);
     if (!launched) return (int)hipErrorInvalidConfiguration;
+  } else if (norm_fwd_can_split<T, RMS>(plan, a)) {
+    const dim3 grid((unsigned)plan.split, (unsigned)a.M);
+    hipLaunchKernelGGL((norm_fwd_split_sums_kernel<T, kStreamBlock, RMS>), grid,
+                       dim3(kStreamBlock), 0, stream, (const T*)a.x, (T*)a.y, a.N,
+                       plan.chunk_packs);
+    hipLaunchKernelGGL((norm_fwd_split_stats_kernel<T, RMS>), dim3((unsigned)a.M), dim3(64), 0,
+                       stream, (const T*)a.x, (T*)a.y, a.mean, a.rstd, a.N, plan.split, a.eps);
+    hipLaunchKernelGGL((norm_fwd_split_apply_kernel<T, WT, kStreamBlock, RMS>), grid,
+                       dim3(kStreamBlock), 0, stream, (const T*)a.x, (const WT*)a.gamma,
+                       (const WT*)a.beta, (T*)a.y, (const float*)a.mean, (const float*)a.rstd,
+                       a.N, plan.chunk_packs);
   } else {
     hipLaunchKernelGGL((norm_fwd_stream_kernel<T, WT, kStreamBlock, RMS>),
                        dim3((unsigned)plan.grid), dim3(kStreamBlock), 0, stream, (const T*)a.x,
@@ -88,7 +112,16 @@ int launch_norm_bwd(const Plan& plan, const NormBwdArgs& a, hipStream_t stream) 
     if (!launched) return (int)hipErrorInvalidConfiguration;
   } else {
     constexpr int E = elems_per_pack<T>::value;
-    if (a.dx != nullptr) {
+    if (a.dx != nullptr && a.split_ws != nullptr && plan.split > 1 && a.M <= 65535) {
+      const dim3 grid((unsigned)plan.split, (unsigned)a.M);
+      hipLaunchKernelGGL((norm_bwd_split_sums_kernel<T, WT, kStreamBlock, RMS>), grid,
+                         dim3(kStreamBlock), 0, stream, (const T*)a.dy, (const T*)a.x, a.mean,
+                         a.rstd, (const WT*)a.gamma, a.split_ws, a.N, plan.chunk_packs);
+      hipLaunchKernelGGL((norm_bwd_split_dx_kernel<T, WT, kStreamBlock, RMS>), grid,
+                         dim3(kStreamBlock), 0, stream, (const T*)a.dy, (const T*)a.x, a.mean,
+                         a.rstd, (const WT*)a.gamma, (const float*)a.split_ws, (T*)a.dx, a.N,
+                         plan.chunk_packs);
+    } else if (a.dx != nullptr) {
       hipLaunchKernelGGL((norm_bwd_stream_dx_kernel<T, WT, kStreamBlock, RMS>),
                          dim3((unsigned)plan.grid), dim3(kStreamBlock), 0, stream,
                          (const T*)a.dy, (const T*)a.x, a.mean, a.rstd, (const WT*)a.gamma,
@@ -105,6 +138,13 @@ int launch_norm_bwd(const Plan& plan, const NormBwdArgs& a, hipStream_t stream) 
   }
   int err = (int)hipGetLastError();
   if (err != 0 || !want_cols) return err;
+  if (!plan.resident && plan.partial_rows <= kFinalizeFlatRows) {
+    const unsigned gx = (unsigned)((a.N + kFinalizeFlatCols - 1) / kFinalizeFlatCols);
+    hipLaunchKernelGGL((colsum_finalize_flat_kernel<WT>), dim3(gx, RMS ? 1 : 2), dim3(256), 0,
+                       stream, (const float*)a.part_dg, (const float*)a.part_db, (WT*)a.dgamma,
+                       (WT*)a.dbeta, (int)plan.partial_rows, a.N);
+    return (int)hipGetLastError();
+  }
   const unsigned gx = (unsigned)((a.N + kFinalizeCols - 1) / kFinalizeCols);
   hipLaunchKernelGGL((colsum_finalize_kernel<WT>), dim3(gx, RMS ? 1 : 2), dim3(1024), 0, stream,
                      (const float*)a.part_dg, (const float*)a.part_db, (WT*)a.dgamma,

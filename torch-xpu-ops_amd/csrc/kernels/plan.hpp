@@ -36,7 +36,9 @@ enum OpClass {
 };
 
 struct Override {
-  int G = 0, V = 0, block = 0, bpc = 0;  // 0 = automatic; G = -1 = force the streaming kernel
+  // 0 = automatic; G = -1 = force the streaming kernel, and then V = 1 keeps every
+  // row on one workgroup, V > 1 splits every row over V workgroups (norm ops)
+  int G = 0, V = 0, block = 0, bpc = 0;
 };
 
 struct Plan {
@@ -45,12 +47,21 @@ struct Plan {
   int G = 0, V = 0, block = 0, rpb = 0;
   int64_t grid = 0;
   int64_t partial_rows = 0;
+  // Split-row path of the norm ops (few rows, each far too long for registers):
+  // a row is cut into `split` chunks of `chunk_packs` packs, one workgroup each;
+  // 0 or 1 = one workgroup per row.
+  int split = 0;
+  int64_t chunk_packs = 0;
 };
 
 constexpr int kMinG = 8;
 constexpr int kMaxG = 1024;
 constexpr int kMaxV = 16;
 constexpr int kStreamBlock = 1024;
+// Split-row path: a chunk is a whole number of workgroup strides and at least
+// four of them (32768 16-bit elements); a row is cut into at most 1024 chunks.
+constexpr int kSplitMinStrides = 4;
+constexpr int kSplitMaxChunks = 1024;
 
 // Preferred packs per lane: what the G ladder aims for.
 // Measured on MI355X: 16 elements a lane (two 16-bit packs, four fp32 packs)
@@ -354,8 +365,37 @@ inline int make_plan(OpClass oc, int64_t M, int64_t N, int esize, int num_cus, c
     if (p.resident) {
       p.partial_rows = grid;
     } else {
-      int64_t pr = M < 64 ? M : 64;
+      // enough partial rows that the column-sum grid (256 lanes, one pack each,
+      // across; partial rows down) gives a compute unit about four workgroups
+      const int64_t across = (packs + 255) / 256;
+      int64_t pr = (4 * (int64_t)num_cus + across - 1) / across;
+      if (pr > 64) pr = 64;
+      if (pr > M) pr = M;
       p.partial_rows = pr < 1 ? 1 : pr;
+    }
+  }
+  // Rows beyond the registers, and too few of them to give every compute unit a
+  // workgroup (the regime of the reference's split-row kernels, Norm.h:632-812):
+  // cut each row into chunks so that about four workgroups per compute unit
+  // exist.  The partial sums of a row cross workgroups through memory, in a fixed
+  // order, between two launches.
+  if ((oc == OC_NORM_FWD || oc == OC_NORM_BWD) && !p.resident) {
+    const int64_t min_chunk = (int64_t)kSplitMinStrides * kStreamBlock;
+    int64_t want = 1;
+    if (ov.G < 0 && ov.V > 0)
+      want = ov.V;
+    else if (M < 2 * (int64_t)num_cus)
+      want = (4 * (int64_t)num_cus + M - 1) / M;
+    if (want > kSplitMaxChunks) want = kSplitMaxChunks;
+    if (want > 1) {
+      int64_t cp = (packs + want - 1) / want;
+      cp = (cp + kStreamBlock - 1) / kStreamBlock * kStreamBlock;
+      if (cp < min_chunk && !(ov.G < 0 && ov.V > 0)) cp = min_chunk;
+      const int64_t chunks = (packs + cp - 1) / cp;
+      if (chunks > 1) {
+        p.split = (int)chunks;
+        p.chunk_packs = cp;
+      }
     }
   }
   *out = p;
