@@ -140,9 +140,10 @@ int norm_fwd(const void* x, const void* gamma, const void* beta, void* y, float*
                            : launch_norm_fwd<bf16, bf16, RMS>(plan, a, s);
 }
 
-// Bytes of the [M, split, 2] fp32 partial sums of the split-row backward (0: not split).
+// Bytes of the [M, split, 2] fp32 partial sums of the split-row backward and the
+// [M, 2] row totals behind them (0: not split).
 size_t split_bytes(const Plan& plan, int64_t M) {
-  return plan.split > 1 ? (size_t)M * (size_t)plan.split * 2 * sizeof(float) : 0;
+  return plan.split > 1 ? (size_t)M * ((size_t)plan.split + 1) * 2 * sizeof(float) : 0;
 }
 
 size_t norm_bwd_workspace(int op, int64_t M, int64_t N, int xd, int wd, int nparts) {

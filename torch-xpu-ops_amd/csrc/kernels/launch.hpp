@@ -34,7 +34,7 @@ struct NormBwdArgs {
   float* part_db;
   int64_t M;
   int N;
-  float* split_ws = nullptr;  // [M, plan.split, 2] fp32 for the split-row path, or null: not split
+  float* split_ws = nullptr;  // [M, plan.split + 1, 2] fp32 for the split-row path, or null: not split
 };
 
 constexpr int kSoftmaxLog = 1;   // log_softmax instead of softmax

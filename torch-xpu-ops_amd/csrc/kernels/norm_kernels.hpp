@@ -797,6 +797,93 @@ norm_bwd_split_dx_kernel(const T* __restrict__ dy, const T* __restrict__ x,
   }
 }
 
+// Split-row backward when dgamma / dbeta are wanted as well: one wavefront per
+// row adds the row's chunk sums in a fixed order into totals[row] = {s1, s2} ...
+template <int DUMMY = 0>
+__global__ void __launch_bounds__(64)
+norm_bwd_split_totals_kernel(const float* __restrict__ split_ws, float* __restrict__ totals,
+                             int chunks) {
+  const int64_t row = blockIdx.x;
+  const float* sc = split_ws + row * (int64_t)chunks * 2;
+  float s1 = 0.0f, s2 = 0.0f;
+  for (int c = threadIdx.x; c < chunks; c += 64) {
+    s1 += sc[2 * c];
+    s2 += sc[2 * c + 1];
+  }
+  s1 = wave_group_allreduce<64, SumOp>(s1);
+  s2 = wave_group_allreduce<64, SumOp>(s2);
+  if (threadIdx.x == 0) {
+    totals[2 * row] = s1;
+    totals[2 * row + 1] = s2;
+  }
+}
+
+// ... and workgroup (bx, by) owns the BLOCK*E columns starting at bx*BLOCK*E and
+// the rows by, by+gridDim.y, ...: it writes their dX and keeps the column sums
+// of its strip, so X and dY are read once more, not twice (row `by` of the
+// [gridDim.y, N] partial buffers, like the column-sum kernel below).  U rows are
+// requested before any of them is used.
+template <class T, class WT, int BLOCK, bool RMS>
+__global__ void __launch_bounds__(BLOCK)
+norm_bwd_split_dx_colsum_kernel(const T* __restrict__ dy, const T* __restrict__ x,
+                                const float* __restrict__ mean, const float* __restrict__ rstd,
+                                const WT* __restrict__ gamma, const float* __restrict__ totals,
+                                T* __restrict__ dx, float* __restrict__ part_dg,
+                                float* __restrict__ part_db, int64_t M, int N) {
+  constexpr int E = elems_per_pack<T>::value;
+  constexpr int U = 4;
+  const int64_t e0l = ((int64_t)blockIdx.x * BLOCK + threadIdx.x) * E;
+  if (e0l >= N) return;  // no barrier below
+  const int e0 = (int)e0l;
+  const Pack<WT, E> pg = gamma ? load_row_pack<WT, E, false>(gamma, e0, N, true, 1.0f)
+                               : Pack<WT, E>::splat(1.0f);
+  const float fN = (float)N;
+  float dg[E], db[E];
+#pragma unroll
+  for (int i = 0; i < E; ++i) dg[i] = db[i] = 0.0f;
+  for (int64_t row0 = blockIdx.y; row0 < M; row0 += (int64_t)gridDim.y * U) {
+    Pack<T, E> px[U], pd[U];
+    float mu[U], rs[U], s1[U], s2[U];
+    bool ok[U];
+#pragma unroll
+    for (int u = 0; u < U; ++u) {
+      const int64_t row = row0 + (int64_t)u * gridDim.y;
+      ok[u] = row < M;
+      const int64_t rc = ok[u] ? row : row0;
+      px[u] = load_row_pack<T, E, true>(x + rc * (int64_t)N, e0, N, true, 0.0f);
+      pd[u] = load_row_pack<T, E, true>(dy + rc * (int64_t)N, e0, N, true, 0.0f);
+      mu[u] = RMS ? 0.0f : mean[rc];
+      rs[u] = rstd[rc];
+      s1[u] = totals[2 * rc];
+      s2[u] = totals[2 * rc + 1];
+    }
+#pragma unroll
+    for (int u = 0; u < U; ++u) {
+      if (!ok[u]) continue;
+      const int64_t row = row0 + (int64_t)u * gridDim.y;
+      const float term1 = rs[u] / fN;
+      Pack<T, E> o;
+#pragma unroll
+      for (int i = 0; i < E; ++i) {
+        const float xh = (px[u].get(i) - mu[u]) * rs[u];
+        float f = fN * (pd[u].get(i) * pg.get(i));
+        f -= xh * s2[u];
+        if constexpr (!RMS) f -= s1[u];
+        o.set(i, f * term1);
+        dg[i] = fmaf(pd[u].get(i), xh, dg[i]);
+        db[i] += pd[u].get(i);
+      }
+      store_row_pack<T, E, true>(dx + row * (int64_t)N, e0, N, true, o);
+    }
+  }
+#pragma unroll
+  for (int i = 0; i < E; ++i)
+    if (e0 + i < N) {
+      part_dg[(int64_t)blockIdx.y * N + e0 + i] = dg[i];
+      if constexpr (!RMS) part_db[(int64_t)blockIdx.y * N + e0 + i] = db[i];
+    }
+}
+
 // Column sums for rows too wide for registers: workgroup (bx, by) owns the
 // BLOCK*E columns starting at bx*BLOCK*E and the rows by, by+gridDim.y, ...;
 // it writes row `by` of the [gridDim.y, N] partial buffers.

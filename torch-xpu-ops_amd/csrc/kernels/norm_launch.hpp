@@ -112,22 +112,37 @@ int launch_norm_bwd(const Plan& plan, const NormBwdArgs& a, hipStream_t stream) 
     if (!launched) return (int)hipErrorInvalidConfiguration;
   } else {
     constexpr int E = elems_per_pack<T>::value;
+    bool cols_done = false;
     if (a.dx != nullptr && a.split_ws != nullptr && plan.split > 1 && a.M <= 65535) {
       const dim3 grid((unsigned)plan.split, (unsigned)a.M);
       hipLaunchKernelGGL((norm_bwd_split_sums_kernel<T, WT, kStreamBlock, RMS>), grid,
                          dim3(kStreamBlock), 0, stream, (const T*)a.dy, (const T*)a.x, a.mean,
                          a.rstd, (const WT*)a.gamma, a.split_ws, a.N, plan.chunk_packs);
-      hipLaunchKernelGGL((norm_bwd_split_dx_kernel<T, WT, kStreamBlock, RMS>), grid,
-                         dim3(kStreamBlock), 0, stream, (const T*)a.dy, (const T*)a.x, a.mean,
-                         a.rstd, (const WT*)a.gamma, (const float*)a.split_ws, (T*)a.dx, a.N,
-                         plan.chunk_packs);
+      if (want_cols) {
+        // dX and the column sums in one more pass over X and dY
+        constexpr int CB = 256;
+        float* totals = a.split_ws + a.M * (int64_t)plan.split * 2;
+        hipLaunchKernelGGL((norm_bwd_split_totals_kernel<0>), dim3((unsigned)a.M), dim3(64), 0,
+                           stream, (const float*)a.split_ws, totals, plan.split);
+        const unsigned gx = (unsigned)((a.N + CB * E - 1) / (CB * E));
+        hipLaunchKernelGGL((norm_bwd_split_dx_colsum_kernel<T, WT, CB, RMS>),
+                           dim3(gx, (unsigned)plan.partial_rows), dim3(CB), 0, stream,
+                           (const T*)a.dy, (const T*)a.x, a.mean, a.rstd, (const WT*)a.gamma,
+                           (const float*)totals, (T*)a.dx, a.part_dg, a.part_db, a.M, a.N);
+        cols_done = true;
+      } else {
+        hipLaunchKernelGGL((norm_bwd_split_dx_kernel<T, WT, kStreamBlock, RMS>), grid,
+                           dim3(kStreamBlock), 0, stream, (const T*)a.dy, (const T*)a.x, a.mean,
+                           a.rstd, (const WT*)a.gamma, (const float*)a.split_ws, (T*)a.dx, a.N,
+                           plan.chunk_packs);
+      }
     } else if (a.dx != nullptr) {
       hipLaunchKernelGGL((norm_bwd_stream_dx_kernel<T, WT, kStreamBlock, RMS>),
                          dim3((unsigned)plan.grid), dim3(kStreamBlock), 0, stream,
                          (const T*)a.dy, (const T*)a.x, a.mean, a.rstd, (const WT*)a.gamma,
                          (T*)a.dx, a.M, a.N);
     }
-    if (want_cols) {
+    if (want_cols && !cols_done) {
       constexpr int CB = 256;
       const unsigned gx = (unsigned)((a.N + CB * E - 1) / (CB * E));
       hipLaunchKernelGGL((norm_bwd_stream_colsum_kernel<T, CB, RMS>),
