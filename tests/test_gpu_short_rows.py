@@ -1,0 +1,62 @@
+"""Short LayerNorm / RMSNorm rows (at most one wavefront of 16-byte packs): the one-pack-a-lane
+layouts on 8..64 lanes that the backward always takes and the forward takes for tensors that do
+not start on a 128-byte line, through the extern "C" ABI against the CPU oracle.  Tolerances as
+everywhere: float32 rtol = atol = 1e-5; 16-bit atol 1e-2, rtol 1.6e-2."""
+import pytest
+import torch
+
+from helpers import assert_close, colsum_slack, gen, offset_view, to_np32
+
+pytestmark = pytest.mark.gpu
+
+DTYPES = [torch.float32, torch.float16, torch.bfloat16]
+# whole packs only (the ragged-row kernels keep their own layout): 4 fp32 / 8 16-bit elements
+LENGTHS = [8, 16, 24, 32, 64, 96, 128, 200, 256, 264, 384, 512]
+
+
+@pytest.mark.parametrize("dtype", DTYPES, ids=str)
+@pytest.mark.parametrize("offset", [0, 2, 8, 32], ids=lambda o: "off%d" % o)
+def test_short_rows_match_the_oracle(cabi, oracle, gpu, dtype, offset):
+    code = cabi.dtype_code(dtype)
+    E = 16 // torch.empty(0, dtype=dtype).element_size()
+    for N in LENGTHS:
+        if N % E:
+            continue
+        M = 1031  # not a multiple of any rows-per-workgroup count
+        print("case short rows", dtype, offset, (M, N), flush=True)
+        packs = N // E
+        pb = cabi.plan(cabi.OP_LAYER_NORM_BWD, M, N, code, code)
+        if packs <= 64:
+            assert pb["packs_per_lane"] == 1 and pb["lanes_per_row"] >= packs, pb
+        g = gen(900 + N)
+        x = (0.5 + torch.randn(M, N, generator=g)).to(dtype)
+        x[3] = 1.5  # a constant row
+        dy = torch.randn(M, N, generator=g).to(dtype)
+        gamma = (1 + 0.1 * torch.randn(N, generator=g)).to(dtype)
+        beta = (0.1 * torch.randn(N, generator=g)).to(dtype)
+        place = (lambda t: offset_view(t.to(gpu), offset)) if offset else (lambda t: t.to(gpu))
+        xg, dyg, gg, bg = place(x), place(dy), place(gamma), place(beta)
+        out = lambda: place(torch.empty(M, N, dtype=dtype))  # noqa: E731
+        y, mean, rstd = cabi.layer_norm_fwd(xg, gg, bg, 1e-5, y=out())
+        oy, om, orr = oracle.layer_norm_fwd(to_np32(x), (N,), to_np32(gamma), to_np32(beta), 1e-5)
+        assert_close(y, oy, dtype, "layer_norm y N=%d" % N)
+        assert_close(mean, om.reshape(-1), dtype, "mean N=%d" % N)
+        assert_close(rstd, orr.reshape(-1), dtype, "rstd N=%d" % N)
+        assert torch.equal(y[3].cpu(), beta)
+        dx, dg, db = cabi.layer_norm_bwd(dyg, xg, mean, rstd, gg, dx=out())
+        odx, odg, odb = oracle.layer_norm_bwd(to_np32(dy), to_np32(x), (N,), to_np32(mean),
+                                              to_np32(rstd), to_np32(gamma))
+        xhat = (x.float() - mean.cpu().reshape(M, 1)) * rstd.cpu().reshape(M, 1)
+        sl_g, sl_b = colsum_slack(dy.float() * xhat), colsum_slack(dy.float())
+        assert_close(dx, odx, dtype, "layer_norm dx N=%d" % N)
+        assert_close(dg, odg, dtype, "dgamma N=%d" % N, slack=sl_g)
+        assert_close(db, odb, dtype, "dbeta N=%d" % N, slack=sl_b)
+        ry, rr = cabi.rms_norm_fwd(xg, gg, 1e-6, y=out())
+        roy, ror = oracle.rms_norm_fwd(to_np32(x), (N,), to_np32(gamma), 1e-6)
+        assert_close(ry, roy, dtype, "rms_norm y N=%d" % N)
+        assert_close(rr, ror.reshape(-1), dtype, "rms rstd N=%d" % N)
+        rdx, rdg = cabi.rms_norm_bwd(dyg, xg, rr, gg, dx=out())
+        rodx, rodg = oracle.rms_norm_bwd(to_np32(dy), to_np32(x), (N,), to_np32(rr), to_np32(gamma))
+        assert_close(rdx, rodx, dtype, "rms_norm dx N=%d" % N)
+        assert_close(rdg, rodg, dtype, "rms dgamma N=%d" % N,
+                     slack=colsum_slack(dy.float() * x.float() * rr.cpu().reshape(M, 1)))

@@ -127,8 +127,9 @@ int norm_fwd(const void* x, const void* gamma, const void* beta, void* y, float*
   if (!x || !y) return ROWNORM_ERR_NULL;
   Plan plan;
   const int op = RMS ? ROWNORM_OP_RMS_NORM_FWD : ROWNORM_OP_LAYER_NORM_FWD;
+  const bool off_line = (((uintptr_t)x | (uintptr_t)y) & 127u) != 0;
   if (int e = make_plan(OC_NORM_FWD, M, N, esize_of(xd), current_num_cus(), g_override[op],
-                        false, &plan, false, !RMS, esize_of(wd) > esize_of(xd)))
+                        false, &plan, false, !RMS, esize_of(wd) > esize_of(xd), off_line))
     return e;
   NormFwdArgs a{x, gamma, RMS ? nullptr : beta, y, RMS ? nullptr : mean, rstd, M, (int)N, eps};
   hipStream_t s = (hipStream_t)stream;

@@ -172,6 +172,8 @@ constexpr bool variant_built(OpClass oc, int esize, int G, int V, bool fast) {
   return true;
 #else
   if (G == kMinG) return V <= v_pref(oc, esize);
+  // short norm rows take one pack a lane on up to one wavefront (see make_plan())
+  if ((oc == OC_NORM_FWD || oc == OC_NORM_BWD) && G <= 64 && V == 1) return true;
   return V >= v_pref(oc, esize);
 #endif
 }
@@ -238,9 +240,10 @@ inline bool norm_layout(OpClass oc, int esize, int64_t packs, bool layer_norm, b
 // force_general: take the general (ragged-row) kernels even when N % E == 0.
 // layer_norm: the norm op is LayerNorm (statistics of two sums, beta), not RMSNorm.
 // wide_weights: fp32 gamma/beta beside 16-bit rows.
+// off_line: a tensor of the call does not start on a 128-byte cache line.
 inline int make_plan(OpClass oc, int64_t M, int64_t N, int esize, int num_cus, const Override& ov,
                      bool want_cols, Plan* out, bool force_general = false,
-                     bool layer_norm = false, bool wide_weights = false) {
+                     bool layer_norm = false, bool wide_weights = false, bool off_line = false) {
   Plan p;
   const int E = 16 / esize;
   p.fast = (N % E) == 0 && !force_general;
@@ -264,6 +267,24 @@ inline int make_plan(OpClass oc, int64_t M, int64_t N, int esize, int num_cus, c
     bool group_exact = false;
     if ((oc == OC_NORM_FWD || oc == OC_NORM_BWD) && p.fast && ov.G == 0 && ov.V == 0)
       group_exact = norm_layout(oc, esize, packs, layer_norm, wide_weights, &G, &V);
+    // Norm rows of at most one wavefront of packs: with one pack a lane, a load
+    // instruction of a wavefront covers one contiguous span of 64 packs (several
+    // whole rows), while with V packs a lane it covers 64/G separate pieces of
+    // G packs, and every piece that does not start on a cache line touches one
+    // line more: 2 instead of 1 at G = 8.  Measured at 2^25 elements (fp32; rows
+    // of 64 / 128 / 256 elements that start 8 bytes into a line): LayerNorm
+    // forward 160 / 139 / 109 -> 105 / 104 / 105 us, backward 238 / 221 / 178 ->
+    // 157 / 156 / 158 us; fp16 rows of 128 elements 78 -> 56 us and 125 -> 83 us.
+    // On line-aligned rows the backward gains 4-5 % as well (its column sums take
+    // a quarter of the registers), the LayerNorm forward loses 5 %: the forward
+    // takes this layout for rows off the line only.
+    if ((oc == OC_NORM_FWD || oc == OC_NORM_BWD) && p.fast && ov.G == 0 && ov.V == 0 &&
+        packs <= 64 && (oc == OC_NORM_BWD || off_line)) {
+      G = pow2_ceil(packs);
+      if (G < kMinG) G = kMinG;
+      V = 1;
+      group_exact = true;
+    }
     // 16-bit softmax forward (its exp makes it the arithmetic-heavy one), ragged
     // 16-bit softmax rows in both directions and ragged 16-bit norm rows:
     // a row that fills at most three quarters of the two-pack slots takes three
