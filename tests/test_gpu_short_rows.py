@@ -60,3 +60,34 @@ def test_short_rows_match_the_oracle(cabi, oracle, gpu, dtype, offset):
         assert_close(rdx, rodx, dtype, "rms_norm dx N=%d" % N)
         assert_close(rdg, rodg, dtype, "rms dgamma N=%d" % N,
                      slack=colsum_slack(dy.float() * x.float() * rr.cpu().reshape(M, 1)))
+
+
+@pytest.mark.parametrize("dtype", DTYPES, ids=str)
+@pytest.mark.parametrize("offset", [0, 2, 8, 32], ids=lambda o: "off%d" % o)
+def test_short_softmax_rows_match_the_oracle(cabi, oracle, gpu, dtype, offset):
+    """softmax / log_softmax forward and backward take the same layout for tensors off a line;
+    masked entries (-inf), a fully masked row and the float16 -> float32 output included."""
+    E = 16 // torch.empty(0, dtype=dtype).element_size()
+    for N in LENGTHS:
+        if N % E:
+            continue
+        M = 1031
+        print("case short softmax rows", dtype, offset, (M, N), flush=True)
+        g = gen(950 + N)
+        x = (3 * torch.randn(M, N, generator=g)).to(dtype)
+        x[5, N // 2:] = float("-inf")
+        x[7] = float("-inf")
+        grad = torch.randn(M, N, generator=g).to(dtype)
+        place = (lambda t: offset_view(t.to(gpu), offset)) if offset else (lambda t: t.to(gpu))
+        xg, gg = place(x), place(grad)
+        for is_log in (False, True):
+            y = cabi.softmax_fwd(xg, is_log, y=place(torch.empty(M, N, dtype=dtype)))
+            assert_close(y, oracle.softmax_fwd(to_np32(x), is_log), dtype,
+                         "softmax y N=%d log=%d" % (N, is_log))
+            gi = cabi.softmax_bwd(gg, y, is_log, gi=place(torch.empty(M, N, dtype=dtype)))
+            assert_close(gi, oracle.softmax_bwd(to_np32(grad), to_np32(y), is_log), dtype,
+                         "softmax grad_input N=%d log=%d" % (N, is_log))
+            if dtype == torch.float16:
+                y32 = cabi.softmax_fwd(xg, is_log, y=place(torch.empty(M, N)))
+                assert_close(y32, oracle.softmax_fwd(to_np32(x), is_log), torch.float32,
+                             "softmax float16 -> float32 N=%d log=%d" % (N, is_log))

@@ -226,8 +226,10 @@ int softmax_fwd(const void* x, const void* mask, void* y, int64_t rows, int64_t 
   if (mask)
     if (int e = mask_check(mr, rows)) return e;
   Plan plan;
+  const bool off_line = (((uintptr_t)x | (uintptr_t)y) & 127u) != 0;
   if (int e = make_plan(OC_SOFTMAX_FWD, rows, N, esize_of(id), current_num_cus(),
-                        g_override[ROWNORM_OP_SOFTMAX_FWD], false, &plan))
+                        g_override[ROWNORM_OP_SOFTMAX_FWD], false, &plan, false, false, false,
+                        off_line))
     return e;
   SoftmaxFwdArgs a{x,    y, (const uint8_t*)mask, (uint32_t)mr.div, (uint32_t)mr.mod, mr.stride,
                    rows, (int)N, flags};
@@ -248,8 +250,10 @@ int softmax_bwd(const void* grad, const void* y, const void* mask, void* gi, int
   if (mask)
     if (int e = mask_check(mr, rows)) return e;
   Plan plan;
+  const bool off_line = (((uintptr_t)grad | (uintptr_t)y | (uintptr_t)gi) & 127u) != 0;
   if (int e = make_plan(OC_SOFTMAX_BWD, rows, N, esize_of(gd), current_num_cus(),
-                        g_override[ROWNORM_OP_SOFTMAX_BWD], false, &plan))
+                        g_override[ROWNORM_OP_SOFTMAX_BWD], false, &plan, false, false, false,
+                        off_line))
     return e;
   SoftmaxBwdArgs a{grad, y, gi, (const uint8_t*)mask, (uint32_t)mr.div, (uint32_t)mr.mod,
                    mr.stride, rows, (int)N, flags};
