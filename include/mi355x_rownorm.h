@@ -260,7 +260,7 @@ int mi355x_softmax_strided_plan(int backward, int64_t outer, int64_t dim_size, i
  * device (no launch; needs no GPU when the device query fails: 256 compute
  * units are assumed).  x_dtype is the row dtype, w_dtype the weight dtype
  * (ignored by the softmax ops).  The strided softmax ops have their own query above.
- * The norm forwards also look at their pointers: this reports the layout for
+ * The norm forwards and the softmax ops also look at their pointers: this reports the layout for
  * tensors that start on a 128-byte line; rows of at most 64 packs in tensors
  * that do not take one pack a lane (lanes_per_row = packs rounded up to a
  * power of two). */
