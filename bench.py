@@ -442,6 +442,35 @@ def per_op_table(torch, cabi, L, dev, stream, P):
             s[1], s[0], s[3], s[4], g, Nb, C, HW, Gr, [True, True, True])) for s in sets])
     del sets
     torch.cuda.empty_cache()
+
+    # few very long rows: every row is split over workgroups (the reference's split-row regime)
+    M, N = 8, 1 << 22
+    w = (1 + 0.1 * torch.randn(N, device=dev)).bfloat16()
+    b = (0.1 * torch.randn(N, device=dev)).bfloat16()
+    sets = []
+    for _ in range(4):
+        x = torch.randn(M, N, device=dev).bfloat16()
+        s = (x, torch.randn(M, N, device=dev).bfloat16(), torch.empty_like(x),
+             torch.empty(M, device=dev), torch.empty(M, device=dev), torch.empty_like(x),
+             torch.empty_like(w), torch.empty_like(w))
+        L.mi355x_layer_norm_fwd(P(s[0]), P(w), P(b), P(s[2]), P(s[3]), P(s[4]), M, N, 1e-5, BF, BF,
+                                stream)
+        sets.append(s)
+    nws = L.mi355x_layer_norm_bwd_workspace_bytes(M, N, BF, BF, 1, 1)
+    ws = torch.empty(max(nws, 1), dtype=torch.uint8, device=dev)
+    add("native_layer_norm fwd bf16 [8,4194304] (rows split)", 2 * M * N * 2 + 2 * N * 2 + 2 * M * 4,
+        [(lambda s=s: L.mi355x_layer_norm_fwd(P(s[0]), P(w), P(b), P(s[2]), P(s[3]), P(s[4]), M, N,
+                                              1e-5, BF, BF, stream)) for s in sets],
+        stock=[(lambda s=s: torch.ops.aten.native_layer_norm(s[0], [N], w, b, 1e-5)) for s in sets])
+    add("native_layer_norm bwd bf16 [8,4194304] (rows split)", 3 * M * N * 2 + 2 * M * 4 + 3 * N * 2,
+        [(lambda s=s: L.mi355x_layer_norm_bwd(P(s[1]), P(s[0]), P(s[3]), P(s[4]), P(w), P(s[5]),
+                                              P(s[6]), P(s[7]), P(ws), nws, M, N, BF, BF, stream))
+         for s in sets],
+        stock=[(lambda s=s: torch.ops.aten.native_layer_norm_backward(
+            s[1], s[0], [N], s[3].view(M, 1), s[4].view(M, 1), w, b, [True, True, True]))
+               for s in sets])
+    del sets
+    torch.cuda.empty_cache()
     return rows
 
 
