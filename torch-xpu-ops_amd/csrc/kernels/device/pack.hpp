@@ -110,6 +110,9 @@ __device__ __forceinline__ Pack<T, E> load_row_pack(const T* row, int e0, int n,
   }
   Pack<T, E> r = Pack<T, E>::splat(fill);
   if (row_ok && e0 < n && e0 + E > lo) {
+    // the index arithmetic of this rare path stays inside it: computed ahead of
+    // the row loop it would hold registers in every lane for the whole kernel
+    asm volatile("" : "+v"(e0));
     T t[E];
 #pragma unroll
     for (int i = 0; i < E; ++i) {
@@ -164,6 +167,7 @@ __device__ __forceinline__ void store_row_pack(T* row, int e0, int n, bool row_o
     else
       p.store(row + e0);
   } else if (e0 < n && e0 + E > lo) {
+    asm volatile("" : "+v"(e0));  // as in load_row_pack
 #pragma unroll
     for (int i = 0; i < E; ++i)
       if (e0 + i >= lo && e0 + i < n) row[e0 + i] = p.v[i];
