@@ -436,8 +436,8 @@ softmax_bwd_resident_kernel(const TG* __restrict__ grad, const TG* __restrict__ 
 #pragma unroll
     for (int c = 0; c < V; ++c) {
       const int e0 = (c * G + lane) * E;
-      row_trim<TG, E, FAST>(pg[c], e0, nw, 0.0f, h, WINDOW);
-      row_trim<TG, E, FAST>(py[c], e0, nw, 0.0f, h, y_whole);
+      row_trim<TG, E, FAST, true>(pg[c], e0, nw, 0.0f, h, WINDOW);
+      row_trim<TG, E, FAST, true>(py[c], e0, nw, 0.0f, h, y_whole);
     }
     float gf[V][E], yf[V][E];
 #pragma unroll
