@@ -45,7 +45,8 @@ enum {
   ROWNORM_ERR_SHAPE = -2,     /* negative size, or N beyond 2^30 elements */
   ROWNORM_ERR_NULL = -3,      /* a required pointer is NULL */
   ROWNORM_ERR_WORKSPACE = -4, /* workspace missing or smaller than *_workspace_bytes() */
-  ROWNORM_ERR_OVERRIDE = -5   /* a forced variant cannot run this shape */
+  ROWNORM_ERR_OVERRIDE = -5,  /* a forced variant cannot run this shape */
+  ROWNORM_ERR_SCRATCH_LIMIT = -6 /* mi355x_rms_norm_bwd_static: the call needs more than the static scratch */
 };
 
 /* Operation ids for mi355x_rownorm_plan / mi355x_rownorm_set_override. */
@@ -138,6 +139,26 @@ int mi355x_rms_norm_bwd(const void* dy, const void* x, const float* rstd, const 
                         void* dx, void* dgamma, void* workspace, size_t workspace_bytes,
                         int64_t M, int64_t N, rownorm_dtype x_dtype, rownorm_dtype w_dtype,
                         void* stream);
+
+/* mi355x_rms_norm_bwd for callers that cannot allocate device memory: code
+ * under HIP graph capture, tight serving loops, harnesses that forbid
+ * hipMalloc.  It has no counterpart in the reference, whose entry point
+ * allocates its scratch itself (LayerNormKernels.cpp:1255-1264).  Same
+ * arguments and results as mi355x_rms_norm_bwd (bit for bit, given the full
+ * workspace) minus the workspace: the fp32 partial rows live in a 16 MiB array
+ * inside the library's device image, one copy per GPU, held until the process
+ * ends.  A call that would need more (mi355x_rms_norm_bwd_workspace_bytes()
+ * above mi355x_rms_norm_bwd_static_limit_bytes(): on 256 compute units that is
+ * N > 8192 with 512-lane layouts) fails with ROWNORM_ERR_SCRATCH_LIMIT and
+ * launches nothing.  Calls no hipMalloc / hipFree and no allocating library
+ * routine.  Every call on one GPU shares that GPU's array: calls that overlap
+ * in time on one GPU (two streams, two threads) race; calls on one stream are
+ * ordered and safe.  Nothing in the array has to start at zero: each launch
+ * writes every partial row before its second stage reads it. */
+size_t mi355x_rms_norm_bwd_static_limit_bytes(void);
+int mi355x_rms_norm_bwd_static(const void* dy, const void* x, const float* rstd,
+                               const void* gamma, void* dx, void* dgamma, int64_t M, int64_t N,
+                               rownorm_dtype x_dtype, rownorm_dtype w_dtype, void* stream);
 
 /* _softmax / _log_softmax over the innermost dimension of a dense [rows, N]
  * tensor.  Replaces _softmax_kernel / _log_softmax_kernel (SoftMaxKernels.h:19-29)

@@ -1,0 +1,103 @@
+"""mi355x_rms_norm_bwd_static -- the entry point for callers that cannot allocate device memory
+(HIP graph capture, serving loops): the RMSNorm backward with its scratch in a static device array
+of the library.  Through the extern "C" ABI, against mi355x_rms_norm_bwd given the full workspace
+(bit for bit: same kernels, same fixed summation order) and against the CPU oracle (16-bit: atol
+1e-2, rtol 1.6e-2; float32: rtol = atol = 1e-5), on two calls in a row, the second one smaller so
+that it finds the first call's partial rows in the scratch."""
+import ctypes
+
+import pytest
+import torch
+
+from helpers import assert_close, colsum_slack, gen, to_np32
+
+pytestmark = pytest.mark.gpu
+
+
+def _inputs(M, N, dtype, wdtype, seed, gpu):
+    g = gen(seed)
+    x = torch.randn(M, N, generator=g).to(dtype)
+    dy = torch.randn(M, N, generator=g).to(dtype)
+    w = (1 + 0.02 * torch.randn(N, generator=g)).to(wdtype)
+    return x.to(gpu), dy.to(gpu), w.to(gpu)
+
+
+def _both(cabi, x, dy, w, want_dx=True, want_dw=True):
+    """-> ((dx, dw) of the static entry point, (dx, dw) of the allocating one), each on its own
+    pre-filled output buffers."""
+    M, N = x.shape
+    _, rstd = cabi.rms_norm_fwd(x, w, 1e-6)
+    dx_s = torch.full_like(x, 7.0) if want_dx else None
+    dw_s = torch.full_like(w, 7.0) if want_dw else None
+    # the first launch of a kernel loads its code object (and with it the static array) into
+    # device memory; after that a call must leave the free device memory exactly as it found it
+    cabi.rms_norm_bwd_static(dy, x, rstd, w, dx_s, dw_s, w_dtype=w.dtype)
+    for t in (dx_s, dw_s):
+        if t is not None:
+            t.fill_(7.0)
+    torch.cuda.synchronize()
+    free_before = torch.cuda.mem_get_info()[0]
+    cabi.rms_norm_bwd_static(dy, x, rstd, w, dx_s, dw_s, w_dtype=w.dtype)
+    torch.cuda.synchronize()
+    assert torch.cuda.mem_get_info()[0] == free_before  # no device memory was taken
+    dx_r, dw_r = cabi.rms_norm_bwd(dy, x, rstd, w, want=(want_dx, want_dw), w_dtype=w.dtype)
+    return rstd, (dx_s, dw_s), (dx_r, dw_r)
+
+
+def _check_oracle(oracle, x, dy, w, rstd, got, dtype):
+    N = x.shape[1]
+    odx, odw = oracle.rms_norm_bwd(to_np32(dy), to_np32(x), (N,), to_np32(rstd), to_np32(w))
+    if got[0] is not None:
+        assert_close(got[0], odx, dtype, "static dx")
+    if got[1] is not None:
+        # a float32 column sum over all rows carries its own rounding (helpers.colsum_slack)
+        sl = None
+        if dtype == torch.float32:
+            sl = colsum_slack(dy.cpu().double() * x.cpu().double() * rstd.cpu().double().reshape(-1, 1))
+        assert_close(got[1], odw, got[1].dtype, "static dweight", slack=sl)
+
+
+@pytest.mark.parametrize("dtype,wdtype", [(torch.bfloat16, torch.bfloat16),
+                                          (torch.float16, torch.float32),
+                                          (torch.float32, torch.float32)], ids=str)
+def test_two_calls_in_a_row_second_smaller(cabi, oracle, gpu, dtype, wdtype):
+    for (M, N, seed) in ((2048, 4096, 91), (300, 1000, 92)):
+        print("case static scratch", dtype, wdtype, (M, N), flush=True)
+        x, dy, w = _inputs(M, N, dtype, wdtype, seed, gpu)
+        rstd, got, ref = _both(cabi, x, dy, w)
+        assert torch.equal(got[0], ref[0]) and torch.equal(got[1], ref[1])
+        _check_oracle(oracle, x, dy, w, rstd, got, dtype)
+
+
+def test_split_rows_and_partial_requests(cabi, oracle, gpu):
+    # a few very long rows: the split-row partial sums sit behind the column sums in the scratch
+    print("case static scratch split rows", flush=True)
+    x, dy, w = _inputs(2, 300000, torch.bfloat16, torch.bfloat16, 93, gpu)
+    p = cabi.plan(cabi.OP_RMS_NORM_BWD, 2, 300000, cabi.BF16, cabi.BF16)
+    assert p["row_chunks"] > 1
+    rstd, got, ref = _both(cabi, x, dy, w)
+    assert torch.equal(got[0], ref[0]) and torch.equal(got[1], ref[1])
+    _check_oracle(oracle, x, dy, w, rstd, got, torch.bfloat16)
+    # then a smaller resident call, dX only and dweight only
+    x, dy, w = _inputs(512, 2048, torch.bfloat16, torch.bfloat16, 94, gpu)
+    for want in ((True, False), (False, True)):
+        rstd, got, ref = _both(cabi, x, dy, w, *want)
+        for a, b in zip(got, ref):
+            assert (a is None and b is None) or torch.equal(a, b)
+        _check_oracle(oracle, x, dy, w, rstd, got, torch.bfloat16)
+
+
+def test_limit_is_an_error_before_any_launch(cabi, gpu):
+    L = cabi.lib()
+    limit = L.mi355x_rms_norm_bwd_static_limit_bytes()
+    assert limit == 16 << 20
+    M, N = 16384, 12288  # 512 partial rows of 12288 floats: 24 MiB
+    need = L.mi355x_rms_norm_bwd_workspace_bytes(M, N, cabi.BF16, cabi.BF16, 1)
+    assert need > limit
+    one = ctypes.c_void_p(256)  # never dereferenced
+    assert L.mi355x_rms_norm_bwd_static(one, one, one, one, one, one, M, N, cabi.BF16, cabi.BF16,
+                                        None) == -6
+    assert "static" in cabi.error_string(-6)
+    # dX alone needs no scratch at that size: accepted (nothing launched here: empty problem)
+    assert L.mi355x_rms_norm_bwd_static(one, one, one, one, one, None, 0, N, cabi.BF16, cabi.BF16,
+                                        None) == 0

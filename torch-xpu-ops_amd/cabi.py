@@ -20,7 +20,8 @@ SOFTMAX, LOG_SOFTMAX, SAFE_SOFTMAX = 0, 1, 2
 EXPORTED_SYMBOLS = (
     "mi355x_rownorm_error_string", "mi355x_rownorm_abi_version", "mi355x_layer_norm_fwd",
     "mi355x_layer_norm_bwd_workspace_bytes", "mi355x_layer_norm_bwd", "mi355x_rms_norm_fwd",
-    "mi355x_rms_norm_bwd_workspace_bytes", "mi355x_rms_norm_bwd", "mi355x_softmax_fwd",
+    "mi355x_rms_norm_bwd_workspace_bytes", "mi355x_rms_norm_bwd",
+    "mi355x_rms_norm_bwd_static_limit_bytes", "mi355x_rms_norm_bwd_static", "mi355x_softmax_fwd",
     "mi355x_softmax_bwd", "mi355x_safe_softmax_fwd", "mi355x_masked_softmax_fwd",
     "mi355x_masked_softmax_bwd", "mi355x_softmax_strided_fwd", "mi355x_softmax_strided_bwd",
     "mi355x_softmax_strided_plan", "mi355x_group_norm_fwd",
@@ -64,6 +65,10 @@ def lib():
                                             ctypes.c_size_t, _i64, _i64, _int, _int, _vp]
         L.mi355x_rms_norm_bwd.argtypes = [_vp, _vp, _vp, _vp, _vp, _vp, _vp, ctypes.c_size_t,
                                           _i64, _i64, _int, _int, _vp]
+        L.mi355x_rms_norm_bwd_static_limit_bytes.restype = ctypes.c_size_t
+        L.mi355x_rms_norm_bwd_static_limit_bytes.argtypes = []
+        L.mi355x_rms_norm_bwd_static.argtypes = [_vp, _vp, _vp, _vp, _vp, _vp, _i64, _i64, _int,
+                                                 _int, _vp]
         L.mi355x_softmax_fwd.argtypes = [_vp, _vp, _i64, _i64, _int, _int, _int, _vp]
         L.mi355x_softmax_bwd.argtypes = [_vp, _vp, _vp, _i64, _i64, _int, _int, _int, _vp]
         L.mi355x_safe_softmax_fwd.argtypes = [_vp, _vp, _i64, _i64, _int, _int, _vp]
@@ -89,7 +94,8 @@ def lib():
         L.mi355x_rownorm_plan.argtypes = [_int, _i64, _i64, _int, _int, ctypes.POINTER(Plan)]
         L.mi355x_rownorm_set_override.argtypes = [_int, _int, _int, _int, _int]
         for name in ("mi355x_layer_norm_fwd", "mi355x_rms_norm_fwd", "mi355x_layer_norm_bwd",
-                     "mi355x_rms_norm_bwd", "mi355x_softmax_fwd", "mi355x_softmax_bwd",
+                     "mi355x_rms_norm_bwd", "mi355x_rms_norm_bwd_static", "mi355x_softmax_fwd",
+                     "mi355x_softmax_bwd",
                      "mi355x_safe_softmax_fwd", "mi355x_masked_softmax_fwd",
                      "mi355x_masked_softmax_bwd", "mi355x_softmax_strided_fwd",
                      "mi355x_softmax_strided_bwd", "mi355x_softmax_strided_plan",
@@ -252,6 +258,19 @@ def rms_norm_bwd(dy, x, rstd, gamma, n_norm_dims=1, want=(True, True), w_dtype=N
                                      _ptr(dgamma), _ptr(workspace),
                                      0 if workspace is None else workspace.numel(), M, N, xd, wd,
                                      _stream()), "rms_norm_bwd")
+    return dx, dgamma
+
+
+def rms_norm_bwd_static(dy, x, rstd, gamma, dx, dgamma, n_norm_dims=1, w_dtype=None):
+    """mi355x_rms_norm_bwd_static: the caller brings every output (either may be None = not
+    wanted); the scratch is the library's own static device array, nothing is allocated."""
+    _gpu(dy, x, rstd, gamma, dx, dgamma)
+    M, N = _rows(x, n_norm_dims)
+    wdt = w_dtype if w_dtype is not None else (
+        dgamma.dtype if dgamma is not None else (gamma.dtype if gamma is not None else x.dtype))
+    _check(lib().mi355x_rms_norm_bwd_static(_ptr(dy), _ptr(x), _ptr(rstd), _ptr(gamma), _ptr(dx),
+                                            _ptr(dgamma), M, N, dtype_code(x.dtype),
+                                            dtype_code(wdt), _stream()), "rms_norm_bwd_static")
     return dx, dgamma
 
 

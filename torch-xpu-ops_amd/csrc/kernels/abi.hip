@@ -88,6 +88,35 @@ int current_num_cus() {
 // Forced variants for tests and tuning (process-global, see the header).
 Override g_override[ROWNORM_OP_COUNT];
 
+// Device-resident scratch of mi355x_rms_norm_bwd_static: the fp32 partial rows of
+// the dgamma reduction (and the split-row partial sums behind them) for callers
+// that may not allocate.  Every GPU the library runs on holds its own copy of
+// the array, at its own address, until the process ends.  The name below is a
+// host-side stand-in only; host code uses the per-device address that
+// hipGetSymbolAddress reports (static_scratch()).
+constexpr size_t kStaticScratchBytes = size_t(16) << 20;
+static __device__ __align__(256) __attribute__((used)) unsigned char scratch[kStaticScratchBytes];
+std::atomic<void*> g_scratch_ptr[kMaxDevices];
+
+// The current device's address of `scratch`, looked up once per device.
+// Returns 0, a positive hipError_t, or ROWNORM_ERR_SHAPE for a device ordinal
+// beyond the table.
+int static_scratch(void** out) {
+  int dev = 0;
+  hipError_t e = hipGetDevice(&dev);
+  if (e != hipSuccess) return (int)e;
+  if (dev < 0 || dev >= kMaxDevices) return ROWNORM_ERR_SHAPE;
+  void* p = g_scratch_ptr[dev].load(std::memory_order_acquire);
+  if (p == nullptr) {
+    e = hipGetSymbolAddress(&p, HIP_SYMBOL(scratch));
+    if (e != hipSuccess) return (int)e;
+    if (p == nullptr) return (int)hipErrorInvalidSymbol;
+    g_scratch_ptr[dev].store(p, std::memory_order_release);
+  }
+  *out = p;
+  return 0;
+}
+
 int esize_of(int dt) {
   switch (dt) {
     case ROWNORM_F32: return 4;
@@ -321,6 +350,8 @@ const char* mi355x_rownorm_error_string(int code) {
     case ROWNORM_ERR_NULL: return "mi355x_rownorm: a required pointer is NULL";
     case ROWNORM_ERR_WORKSPACE: return "mi355x_rownorm: workspace missing or too small";
     case ROWNORM_ERR_OVERRIDE: return "mi355x_rownorm: forced variant cannot run this shape";
+    case ROWNORM_ERR_SCRATCH_LIMIT:
+      return "mi355x_rownorm: the call needs more scratch than the library's static 16 MiB";
   }
   if (code > 0) return hipGetErrorString((hipError_t)code);
   return "mi355x_rownorm: unknown error code";
@@ -369,6 +400,26 @@ int mi355x_rms_norm_bwd(const void* dy, const void* x, const float* rstd, const 
                         void* stream) {
   return norm_bwd<true>(dy, x, nullptr, rstd, gamma, dx, dgamma, nullptr, workspace,
                         workspace_bytes, M, N, (int)x_dtype, (int)w_dtype, stream);
+}
+
+size_t mi355x_rms_norm_bwd_static_limit_bytes(void) { return kStaticScratchBytes; }
+
+int mi355x_rms_norm_bwd_static(const void* dy, const void* x, const float* rstd,
+                               const void* gamma, void* dx, void* dgamma, int64_t M, int64_t N,
+                               rownorm_dtype x_dtype, rownorm_dtype w_dtype, void* stream) {
+  if (!norm_dtypes_ok((int)x_dtype, (int)w_dtype)) return ROWNORM_ERR_DTYPE;
+  if (int e = shape_check(M, N)) return e;
+  if (M == 0 || N == 0 || (!dx && !dgamma)) return 0;
+  // What the allocating entry point would be given in full: the column-sum
+  // partial rows and, for a few very long rows, the split-row partial sums.
+  const size_t need = norm_bwd_workspace(ROWNORM_OP_RMS_NORM_BWD, M, N, (int)x_dtype,
+                                         (int)w_dtype, dgamma ? 1 : 0);
+  if (need > kStaticScratchBytes) return ROWNORM_ERR_SCRATCH_LIMIT;
+  void* ws = nullptr;
+  if (need > 0)
+    if (int e = static_scratch(&ws)) return e;
+  return norm_bwd<true>(dy, x, nullptr, rstd, gamma, dx, dgamma, nullptr, ws, need, M, N,
+                        (int)x_dtype, (int)w_dtype, stream);
 }
 
 int mi355x_softmax_fwd(const void* x, void* y, int64_t rows, int64_t N, rownorm_dtype in_dtype,
