@@ -74,7 +74,7 @@ def test_forced_chunk_counts_against_one_workgroup_per_row(cabi, oracle, gpu, dt
     ops = (cabi.OP_LAYER_NORM_FWD, cabi.OP_LAYER_NORM_BWD, cabi.OP_RMS_NORM_FWD, cabi.OP_RMS_NORM_BWD)
     code = cabi.dtype_code(dtype)
     try:
-        for (M, N, shift) in ((5, 20000, 0.0), (3, 33333, 3.0), (4, 8192 * 3 + 1, -2.0)):
+        for (M, N, shift) in ((5, 40000, 0.0), (3, 33333, 3.0), (4, 8192 * 3 + 1, -2.0)):
             x, dy, gamma, beta = _mk(M, N, dtype, 82, shift)
             results = {}
             for chunks in (1, 2, 3, 7):

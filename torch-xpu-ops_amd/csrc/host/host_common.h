@@ -23,6 +23,20 @@ inline rownorm_dtype to_rownorm_dtype(at::ScalarType t, const char* op) {
   }
 }
 
+// float64 is outside what the MI355X kernels compute (float32 accumulation): the
+// operator level hands such calls to the kernels PyTorch-ROCm itself ships, with
+// one warning per process, in the way the reference hands what it lacks to
+// another backend (src/ATen/native/xpu/XPUFallback.cpp:59-69).  The reference
+// itself accumulates float64 in double (sycl/LayerNormKernels.cpp:1418-1438).
+inline bool delegated_dtype(const at::Tensor& t) {
+  return t.defined() && t.is_cuda() && t.scalar_type() == at::kDouble;
+}
+
+inline void warn_delegated(const char* op) {
+  TORCH_WARN_ONCE("mi355x: float64 tensors are delegated to the stock PyTorch-ROCm kernels (first "
+                  "seen in ", op, "); the MI355X kernels compute float32, float16 and bfloat16");
+}
+
 inline void check_gpu(const at::Tensor& t, const char* op, const char* name) {
   TORCH_CHECK(t.is_cuda(), op, ": expected `", name,
               "` on a HIP GPU device, but it is on ", t.device(),

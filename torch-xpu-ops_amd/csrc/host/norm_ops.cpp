@@ -4,6 +4,10 @@
 #include "norm_ops.h"
 
 #include <ATen/native/layer_norm.h>
+#include <ATen/ops/_fused_rms_norm_backward_cuda_dispatch.h>
+#include <ATen/ops/_fused_rms_norm_cuda_dispatch.h>
+#include <ATen/ops/native_layer_norm_backward_cuda_dispatch.h>
+#include <ATen/ops/native_layer_norm_cuda_dispatch.h>
 #include <limits>
 
 #include "host_common.h"
@@ -208,6 +212,10 @@ std::tuple<Tensor, Tensor, Tensor> native_layer_norm(const Tensor& input,
                                                      const std::optional<Tensor>& bias_opt,
                                                      double epsilon) {
   static const char* op = "mi355x::native_layer_norm";
+  if (delegated_dtype(input)) {
+    warn_delegated(op);
+    return at::cuda::native_layer_norm(input, normalized_shape, weight_opt, bias_opt, epsilon);
+  }
   const Tensor weight = defined_or_empty(weight_opt);
   const Tensor bias = defined_or_empty(bias_opt);
   check_same_device(input, weight, op, "weight");
@@ -222,7 +230,13 @@ std::tuple<Tensor, Tensor, Tensor> native_layer_norm(const Tensor& input,
   Tensor Y = contiguous_like(X);
   Tensor mean = at::empty({M}, X.options().dtype(at::kFloat));
   Tensor rstd = at::empty({M}, X.options().dtype(at::kFloat));
-  if (M > 0) layer_norm_kernel(X, gamma, beta, M, N, epsilon, &Y, &mean, &rstd);
+  if (M > 0 && N > 0) {
+    layer_norm_kernel(X, gamma, beta, M, N, epsilon, &Y, &mean, &rstd);
+  } else if (M > 0) {
+    // rows of no elements: what the CPU kernel's formulas give, mean 0 and rstd NaN
+    mean.zero_();
+    rstd.fill_(std::numeric_limits<float>::quiet_NaN());
+  }
   const auto stat_shape = stat_shape_of(input, normalized_shape.size());
   return std::make_tuple(std::move(Y), mean.view(stat_shape), rstd.view(stat_shape));
 }
@@ -235,6 +249,11 @@ std::tuple<Tensor, Tensor, Tensor> native_layer_norm_backward(
     const Tensor& mean, const Tensor& rstd, const std::optional<Tensor>& weight_opt,
     const std::optional<Tensor>& bias_opt, std::array<bool, 3> grad_input_mask) {
   static const char* op = "mi355x::native_layer_norm_backward";
+  if (delegated_dtype(input)) {
+    warn_delegated(op);
+    return at::cuda::native_layer_norm_backward(grad_output, input, normalized_shape, mean, rstd,
+                                                weight_opt, bias_opt, grad_input_mask);
+  }
   const Tensor weight = defined_or_empty(weight_opt);
   const Tensor bias = defined_or_empty(bias_opt);
   check_same_device(input, grad_output, op, "grad_out");
@@ -267,6 +286,10 @@ std::tuple<Tensor, Tensor> _fused_rms_norm(const Tensor& input, at::IntArrayRef 
                                            const std::optional<Tensor>& weight_opt,
                                            std::optional<double> eps_opt) {
   static const char* op = "mi355x::_fused_rms_norm";
+  if (delegated_dtype(input)) {
+    warn_delegated(op);
+    return at::cuda::_fused_rms_norm(input, normalized_shape, weight_opt, eps_opt);
+  }
   const Tensor weight = defined_or_empty(weight_opt);
   check_same_device(input, weight, op, "weight");
   const auto [M, N] =
@@ -279,7 +302,11 @@ std::tuple<Tensor, Tensor> _fused_rms_norm(const Tensor& input, at::IntArrayRef 
   const double eps = eps_opt.value_or((double)std::numeric_limits<float>::epsilon());
   Tensor Y = contiguous_like(X);
   Tensor rstd = at::empty({M}, X.options().dtype(at::kFloat));
-  if (M > 0) rms_norm_kernel(X, gamma, M, N, eps, &Y, &rstd);
+  if (M > 0 && N > 0) {
+    rms_norm_kernel(X, gamma, M, N, eps, &Y, &rstd);
+  } else if (M > 0) {
+    rstd.fill_(std::numeric_limits<float>::quiet_NaN());  // the mean of no squares, as on the CPU
+  }
   return std::make_tuple(std::move(Y), rstd.view(stat_shape_of(input, normalized_shape.size())));
 }
 
@@ -290,6 +317,11 @@ std::tuple<Tensor, Tensor> _fused_rms_norm_backward(const Tensor& dY, const Tens
                                                     const std::optional<Tensor>& weight_opt,
                                                     std::array<bool, 2> grad_input_mask) {
   static const char* op = "mi355x::_fused_rms_norm_backward";
+  if (delegated_dtype(input)) {
+    warn_delegated(op);
+    return at::cuda::_fused_rms_norm_backward(dY, input, normalized_shape, rstd, weight_opt,
+                                              grad_input_mask);
+  }
   const Tensor weight = defined_or_empty(weight_opt);
   check_same_device(input, dY, op, "grad_out");
   check_same_device(input, rstd, op, "rstd");
@@ -312,20 +344,59 @@ std::tuple<Tensor, Tensor> _fused_rms_norm_backward(const Tensor& dY, const Tens
 // ---- ATen dispatch stubs -------------------------------------------------------
 
 namespace {
+
+// The GPU slot of one of ATen's DispatchStub objects.  A DispatchStub is a
+// standard-layout class whose only non-static data member is its
+// DispatchStubImpl, so the object's address is that member's address; the
+// class has a setter for the slot but no getter, and uninstalling needs the
+// previous value.
+template <class Stub>
+void*& gpu_slot(Stub& stub) {
+  return reinterpret_cast<at::native::DispatchStubImpl*>(&stub)->cuda_dispatch_ptr;
+}
+
+struct SavedStubs {
+  bool installed = false;
+  void* forward = nullptr;
+  void* backward = nullptr;
+};
+SavedStubs g_layer_norm_saved;
+
 void stub_forward(const Tensor& X, const Tensor& gamma, const Tensor& beta, int64_t M, int64_t N,
                   double eps, Tensor* Y, Tensor* mean, Tensor* rstd) {
+  if (delegated_dtype(X) && g_layer_norm_saved.forward != nullptr) {
+    warn_delegated("LayerNormKernel");
+    return reinterpret_cast<at::native::forward_fn>(g_layer_norm_saved.forward)(
+        X, gamma, beta, M, N, eps, Y, mean, rstd);
+  }
   layer_norm_kernel(X, gamma, beta, M, N, eps, Y, mean, rstd);
 }
 void stub_backward(const Tensor& dY, const Tensor& X, const Tensor& mean, const Tensor& rstd,
                    const Tensor& gamma, int64_t M, int64_t N, Tensor* dX, Tensor* dgamma,
                    Tensor* dbeta) {
+  if (delegated_dtype(X) && g_layer_norm_saved.backward != nullptr) {
+    warn_delegated("LayerNormBackwardKernel");
+    return reinterpret_cast<at::native::backward_fn>(g_layer_norm_saved.backward)(
+        dY, X, mean, rstd, gamma, M, N, dX, dgamma, dbeta);
+  }
   layer_norm_backward_kernel(dY, X, mean, rstd, gamma, M, N, dX, dgamma, dbeta);
 }
 }  // namespace
 
 void install_layer_norm_dispatch_stubs() {
+  if (g_layer_norm_saved.installed) return;
+  g_layer_norm_saved.forward = gpu_slot(at::native::LayerNormKernel);
+  g_layer_norm_saved.backward = gpu_slot(at::native::LayerNormBackwardKernel);
+  g_layer_norm_saved.installed = true;
   at::native::LayerNormKernel.set_cuda_dispatch_ptr(&stub_forward);
   at::native::LayerNormBackwardKernel.set_cuda_dispatch_ptr(&stub_backward);
+}
+
+void uninstall_layer_norm_dispatch_stubs() {
+  if (!g_layer_norm_saved.installed) return;
+  gpu_slot(at::native::LayerNormKernel) = g_layer_norm_saved.forward;
+  gpu_slot(at::native::LayerNormBackwardKernel) = g_layer_norm_saved.backward;
+  g_layer_norm_saved = SavedStubs{};
 }
 
 }  // namespace mi355x

@@ -43,6 +43,11 @@ std::tuple<at::Tensor, at::Tensor> _fused_rms_norm_backward(
 // Points ATen's own LayerNormKernel / LayerNormBackwardKernel dispatch stubs at
 // the kernels above for GPU tensors (what REGISTER_XPU_DISPATCH does at load
 // time in LayerNorm.cpp:198-201 of the reference).  Explicit, never at import.
+// ATen callers that go through the stubs (nested-tensor layer_norm is one) then
+// run these kernels; float64 calls are passed on to the kernels that were
+// registered before.  uninstall_* puts the previous kernels back.  Not
+// synchronized with concurrent calls of the ops: install at start-up.
 void install_layer_norm_dispatch_stubs();
+void uninstall_layer_norm_dispatch_stubs();
 
 }  // namespace mi355x

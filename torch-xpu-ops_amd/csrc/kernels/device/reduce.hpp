@@ -96,4 +96,30 @@ __device__ __forceinline__ void group_allreduce(float (&v)[K], float* lds, int& 
   }
 }
 
+// Sum of two float64 values per thread over the workgroup, added in a fixed
+// order; the result is valid in thread 0 only.
+template <int BLOCK>
+__device__ __forceinline__ void block_sum2_f64(double& a, double& b, double* lds) {
+#pragma unroll
+  for (int off = 32; off > 0; off >>= 1) {
+    a += __shfl_down(a, off, 64);
+    b += __shfl_down(b, off, 64);
+  }
+  const int wave = threadIdx.x >> 6;
+  if ((threadIdx.x & 63) == 0) {
+    lds[2 * wave] = a;
+    lds[2 * wave + 1] = b;
+  }
+  __syncthreads();
+  if (threadIdx.x == 0) {
+    a = lds[0];
+    b = lds[1];
+#pragma unroll
+    for (int w = 1; w < BLOCK / 64; ++w) {
+      a += lds[2 * w];
+      b += lds[2 * w + 1];
+    }
+  }
+}
+
 }  // namespace rownorm

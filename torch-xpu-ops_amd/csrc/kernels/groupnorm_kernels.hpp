@@ -143,7 +143,8 @@ gn_fwd_resident_kernel(const T* __restrict__ x, const WT* __restrict__ gamma,
       centred_sums(std::true_type{});
     group_allreduce<G, BLOCK, 2, SumOp>(acc, red, phase);
     const float m1 = acc[0] / fL;
-    const float var = fmaxf((acc[1] - acc[0] * m1) / fL, 0.0f);
+    float var = (acc[1] - acc[0] * m1) / fL;
+    var = var < 0.0f ? 0.0f : var;  // a select, not v_max_f32: a NaN row keeps NaN statistics
     const float rs = 1.0f / sqrtf(var + eps);
     T* yr = y + row * (int64_t)s.L;
 #pragma unroll
@@ -168,62 +169,60 @@ gn_fwd_resident_kernel(const T* __restrict__ x, const WT* __restrict__ gamma,
       row_store<T, E, true, UNIFORM>(yr, e0, s.L, ok, o);
     }
     if (ok && lane == 0) {
-      if (mean) mean[row] = (WT)(mean0 + m1);
+      if (mean) mean[row] = (WT)(rs == rs ? mean0 + m1 : rs);  // NaN variance: NaN mean
       if (rstd) rstd[row] = (WT)rs;
     }
   }
 }
 
 // Forward for rows too long for the registers: one workgroup per row, two
-// passes over the row (statistics, normalize).  Each thread sums its elements
-// shifted by the first one it sees, (x - k), (x - k)^2, which gives its own
-// count / mean / M2 without cancellation; the threads' triples are then merged
-// with the pairwise formula of WelfordOps::combine (src/ATen/native/xpu/sycl/
-// SharedReduceOps.h:71-88) written as two block sums: mean = k0 + sum n_t *
-// (mean_t - k0) / L, M2 = sum M2_t + n_t * (mean_t - mean)^2.
+// passes over the row (statistics, normalize).  The statistics are the sums of
+// (x - k) and (x - k)^2 in float64, k = the row's first element: float32 and
+// 16-bit values and their differences are exact in float64, and with 53-bit
+// sums s2 - s1*s1/L keeps its accuracy however far k lies from the row (a zero
+// head before a row around 1000 cost rstd 8e-6 with per-thread float32 sums).
+// It stands in for the Welford merge of the reference (WelfordOps::combine,
+// src/ATen/native/xpu/sycl/SharedReduceOps.h:71-88).  The mean goes to the
+// normalize pass as float(mean) plus the remainder, so the rounding of the
+// saved statistic never enters y; on a constant row x - k is exactly zero.
 template <class T, class WT, int BLOCK>
 __global__ void __launch_bounds__(BLOCK)
 gn_fwd_stream_kernel(const T* __restrict__ x, const WT* __restrict__ gamma,
                      const WT* __restrict__ beta, T* __restrict__ y, WT* __restrict__ mean,
                      WT* __restrict__ rstd, int64_t rows, GroupShape s, float eps) {
   constexpr int E = elems_per_pack<T>::value;
-  __shared__ float red[reduce_lds_floats<BLOCK, BLOCK, 1>::value];
-  int phase = 0;
-  const float fL = (float)s.L;
+  __shared__ double red[2 * (BLOCK / 64)];
+  __shared__ float stat[3];
   const int npacks = (s.L + E - 1) / E;
   for (int64_t row = blockIdx.x; row < rows; row += gridDim.x) {
     const int g = (int)((uint32_t)row % (uint32_t)s.groups);
     const T* xr = x + row * (int64_t)s.L;
     T* yr = y + row * (int64_t)s.L;
-    float k = 0.0f, s1 = 0.0f, s2 = 0.0f, cnt = 0.0f;
-    bool first = true;
+    const double k = (double)(float)xr[0];
+    double s1 = 0.0, s2 = 0.0;
     for (int pk = threadIdx.x; pk < npacks; pk += BLOCK) {
       const Pack<T, E> p = load_row_pack<T, E, false>(xr, pk * E, s.L, true, 0.0f);
-      if (first) {
-        k = p.get(0);
-        first = false;
-      }
       const int nvalid = s.L - pk * E;
 #pragma unroll
       for (int i = 0; i < E; ++i) {
-        const float d = i < nvalid ? p.get(i) - k : 0.0f;
+        const double d = i < nvalid ? (double)p.get(i) - k : 0.0;
         s1 += d;
-        s2 = fmaf(d, d, s2);
+        s2 = fma(d, d, s2);
       }
-      cnt += (float)(nvalid < E ? nvalid : E);
     }
-    const float mean_t = cnt > 0.0f ? k + s1 / cnt : 0.0f;
-    const float m2_t = cnt > 0.0f ? fmaxf(s2 - s1 * (s1 / cnt), 0.0f) : 0.0f;
-    // summed relative to the row's first element, so a constant row gets its
-    // constant back exactly
-    const float k0 = (float)xr[0];
-    float a[1] = {cnt * (mean_t - k0)};
-    group_allreduce<BLOCK, BLOCK, 1, SumOp>(a, red, phase);
-    const float mu = k0 + a[0] / fL;
-    const float dm = mean_t - mu;
-    float b[1] = {m2_t + cnt * dm * dm};
-    group_allreduce<BLOCK, BLOCK, 1, SumOp>(b, red, phase);
-    const float rs = 1.0f / sqrtf(fmaxf(b[0] / fL, 0.0f) + eps);
+    block_sum2_f64<BLOCK>(s1, s2, red);
+    if (threadIdx.x == 0) {
+      const double dL = (double)s.L;
+      const double m1 = s1 / dL;
+      const double mu = k + m1;
+      double var = (s2 - s1 * m1) / dL;
+      var = var < 0.0 ? 0.0 : var;  // a select: a NaN row keeps NaN statistics
+      stat[0] = (float)mu;
+      stat[1] = (float)(mu - (double)stat[0]);
+      stat[2] = (float)(1.0 / sqrt(var + (double)eps));
+    }
+    __syncthreads();
+    const float hi = stat[0], lo = stat[1], rs = stat[2];
     for (int pk = threadIdx.x; pk < npacks; pk += BLOCK) {
       const int e0 = pk * E;
       const Pack<T, E> p = load_row_pack<T, E, true>(xr, e0, s.L, true, 0.0f);
@@ -232,12 +231,12 @@ gn_fwd_stream_kernel(const T* __restrict__ x, const WT* __restrict__ gamma,
       for (int i = 0; i < E; ++i) {
         const int ch = gn_channel(s, g, e0 + i);
         const float ga = gn_weight(gamma, ch, 1.0f) * rs;
-        o.set(i, (p.get(i) - mu) * ga + gn_weight(beta, ch, 0.0f));
+        o.set(i, ((p.get(i) - hi) - lo) * ga + gn_weight(beta, ch, 0.0f));
       }
       store_row_pack<T, E, true>(yr, e0, s.L, true, o);
     }
     if (threadIdx.x == 0) {
-      if (mean) mean[row] = (WT)mu;
+      if (mean) mean[row] = (WT)(rs == rs ? hi : rs);  // NaN variance: NaN mean
       if (rstd) rstd[row] = (WT)rs;
     }
   }

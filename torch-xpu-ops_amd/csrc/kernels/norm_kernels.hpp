@@ -159,7 +159,8 @@ norm_fwd_resident_kernel(const T* __restrict__ x, const WT* __restrict__ gamma,
 #pragma unroll
       for (int r = 0; r < R; ++r) {
         m1[r] = acc[2 * r] / fN;
-        const float var = fmaxf((acc[2 * r + 1] - acc[2 * r] * m1[r]) / fN, 0.0f);
+        float var = (acc[2 * r + 1] - acc[2 * r] * m1[r]) / fN;
+        var = var < 0.0f ? 0.0f : var;  // a select, not v_max_f32: a NaN row keeps NaN statistics
         rs[r] = 1.0f / sqrtf(var + eps);
       }
     } else {
@@ -214,7 +215,8 @@ norm_fwd_resident_kernel(const T* __restrict__ x, const WT* __restrict__ gamma,
 #pragma unroll
       for (int r = 0; r < R; ++r) {
         m1[r] = acc[2 * r] / fN;
-        const float var = fmaxf((acc[2 * r + 1] - acc[2 * r] * m1[r]) / fN, 0.0f);
+        float var = (acc[2 * r + 1] - acc[2 * r] * m1[r]) / fN;
+        var = var < 0.0f ? 0.0f : var;  // a select, not v_max_f32: a NaN row keeps NaN statistics
         rs[r] = 1.0f / sqrtf(var + eps);
       }
     }
@@ -248,17 +250,30 @@ norm_fwd_resident_kernel(const T* __restrict__ x, const WT* __restrict__ gamma,
       }
       if (ok[r] && lane == 0) {
         if constexpr (!RMS)
-          if (mean) mean[row0 + r] = mean0[r] + m1[r];
+          // (a row with an inf element has NaN variance; its mean is NaN as well, as the
+          // Welford recurrence of the CPU kernel gives)
+          if (mean) mean[row0 + r] = rs[r] == rs[r] ? mean0[r] + m1[r] : rs[r];
         if (rstd) rstd[row0 + r] = rs[r];
       }
     }
   }
 }
 
+// The centre the long-row kernels shift their sums by: the median of the row's
+// first three elements, the same value in every workgroup that works on the row.
+template <class T>
+__device__ __forceinline__ float split_row_centre(const T* xr, int N) {
+  const float a = (float)xr[0], b = (float)xr[N > 1 ? 1 : 0], c = (float)xr[N > 2 ? 2 : 0];
+  return fmaxf(fminf(a, b), fminf(fmaxf(a, b), c));
+}
+
 // ---------------------------------------------------------------------------
 // Forward for rows too wide to hold in registers: one workgroup per row, the
-// row is streamed from memory three times (sum, centred sums, normalize); the
-// second and third pass hit L2 / Infinity Cache for any realistic row.
+// row is streamed from memory twice (statistics, normalize); the second pass
+// hits L2 / Infinity Cache for any realistic row.  LayerNorm sums (x - k) and
+// (x - k)^2 in float64, k = the median of the row's first three elements (see
+// the split-row kernels below for why float64); RMSNorm sums x^2 in float32,
+// where nothing cancels.
 template <class T, class WT, int BLOCK, bool RMS>
 __global__ void __launch_bounds__(BLOCK)
 norm_fwd_stream_kernel(const T* __restrict__ x, const WT* __restrict__ gamma,
@@ -267,13 +282,17 @@ norm_fwd_stream_kernel(const T* __restrict__ x, const WT* __restrict__ gamma,
                        float eps) {
   constexpr int E = elems_per_pack<T>::value;
   __shared__ float red[reduce_lds_floats<BLOCK, BLOCK, 2>::value];
+  __shared__ double red64[RMS ? 1 : 2 * (BLOCK / 64)];
+  __shared__ float stat[3];
   int phase = 0;
   const float fN = (float)N;
   const int npacks = (N + E - 1) / E;
   for (int64_t row = blockIdx.x; row < M; row += gridDim.x) {
     const T* xr = x + row * (int64_t)N;
     T* yr = y + row * (int64_t)N;
-    float mu = 0.0f, rs;
+    // mean = hi + lo: the saved statistic and the remainder of the float64 mean, kept
+    // apart so that the rounding of the saved mean never enters y
+    float hi = 0.0f, lo = 0.0f, rs;
     if constexpr (RMS) {
       float acc[1] = {0.0f};
       for (int pk = threadIdx.x; pk < npacks; pk += BLOCK) {
@@ -284,30 +303,33 @@ norm_fwd_stream_kernel(const T* __restrict__ x, const WT* __restrict__ gamma,
       group_allreduce<BLOCK, BLOCK, 1, SumOp>(acc, red, phase);
       rs = 1.0f / sqrtf(acc[0] / fN + eps);
     } else {
-      float acc0[1] = {0.0f};
-      for (int pk = threadIdx.x; pk < npacks; pk += BLOCK) {
-        const Pack<T, E> p = load_row_pack<T, E, false>(xr, pk * E, N, true, 0.0f);
-#pragma unroll
-        for (int i = 0; i < E; ++i) acc0[0] += p.get(i);
-      }
-      group_allreduce<BLOCK, BLOCK, 1, SumOp>(acc0, red, phase);
-      const float mean0 = acc0[0] / fN;
-      float acc[2] = {0.0f, 0.0f};
+      const double k = (double)split_row_centre(xr, N);
+      double s1 = 0.0, s2 = 0.0;
       for (int pk = threadIdx.x; pk < npacks; pk += BLOCK) {
         const Pack<T, E> p = load_row_pack<T, E, false>(xr, pk * E, N, true, 0.0f);
         const int nvalid = N - pk * E;
 #pragma unroll
         for (int i = 0; i < E; ++i) {
-          const float d = (i < nvalid) ? p.get(i) - mean0 : 0.0f;
-          acc[0] += d;
-          acc[1] = fmaf(d, d, acc[1]);
+          const double d = (i < nvalid) ? (double)p.get(i) - k : 0.0;
+          s1 += d;
+          s2 = fma(d, d, s2);
         }
       }
-      group_allreduce<BLOCK, BLOCK, 2, SumOp>(acc, red, phase);
-      const float m1 = acc[0] / fN;
-      mu = mean0 + m1;
-      const float var = fmaxf((acc[1] - acc[0] * m1) / fN, 0.0f);
-      rs = 1.0f / sqrtf(var + eps);
+      block_sum2_f64<BLOCK>(s1, s2, red64);
+      if (threadIdx.x == 0) {
+        const double dN = (double)N;
+        const double m1 = s1 / dN;
+        const double mu = k + m1;
+        double var = (s2 - s1 * m1) / dN;
+        var = var < 0.0 ? 0.0 : var;  // a select: a NaN row keeps NaN statistics
+        stat[0] = (float)mu;
+        stat[1] = (float)(mu - (double)stat[0]);
+        stat[2] = (float)(1.0 / sqrt(var + (double)eps));
+      }
+      __syncthreads();
+      hi = stat[0];
+      lo = stat[1];
+      rs = stat[2];
     }
     for (int pk = threadIdx.x; pk < npacks; pk += BLOCK) {
       const int e0 = pk * E;
@@ -324,38 +346,62 @@ norm_fwd_stream_kernel(const T* __restrict__ x, const WT* __restrict__ gamma,
         if constexpr (RMS)
           v = (p.get(i) * rs) * pg.get(i);
         else
-          v = ((p.get(i) - mu) * rs) * pg.get(i) + pb.get(i);
+          v = (((p.get(i) - hi) - lo) * rs) * pg.get(i) + pb.get(i);
         o.set(i, v);
       }
       store_row_pack<T, E, true>(yr, e0, N, true, o);
     }
     if (threadIdx.x == 0) {
       if constexpr (!RMS)
-        if (mean) mean[row] = mu;
+        if (mean) mean[row] = rs == rs ? hi : rs;  // NaN variance: NaN mean
       if (rstd) rstd[row] = rs;
     }
+    // stat[] is rewritten for the next row only after every thread has passed the
+    // barrier inside the next block sum, i.e. after it has read this row's values
   }
 }
 
 // ---------------------------------------------------------------------------
 // Split-row forward: few rows, each far beyond the registers (the regime of the
 // reference's split-row kernels, Norm.h:632-812).  A row is cut into `chunks`
-// chunks of `chunk_packs` packs; workgroup (chunk, row) of the first launch sums
-// its chunk, a second launch adds a row's partial sums in a fixed order and
-// writes mean / rstd, a third normalizes chunk by chunk.  The partial sums cross
-// the launches in the first bytes of the row's own Y, which the third launch
-// overwrites afterwards: no workspace, and the result does not depend on which
-// workgroup runs when.  LayerNorm sums (x - k), (x - k)^2 with k the median of
-// the row's first three elements, as the resident 16-bit kernel does.
-template <class T>
-__device__ __forceinline__ float* split_row_scratch(T* y_row) {
-  return reinterpret_cast<float*>((reinterpret_cast<uintptr_t>(y_row) + 3) & ~uintptr_t(3));
-}
+// chunks of `chunk_packs` packs (the last one takes the remainder as well, at
+// most one workgroup stride more); workgroup (chunk, row) of the first launch
+// sums its chunk, a second launch adds a row's partial sums in a fixed order and
+// writes mean / rstd, a third normalizes chunk by chunk.
+//
+// Statistics.  The partial sums are sum(x - k) and sum((x - k)^2) accumulated in
+// float64, k = the median of the row's first three elements (float32 and 16-bit
+// values and their differences are exact in float64).  With 53-bit sums the
+// subtraction s2 - s1*s1/N keeps 1e-10 of relative accuracy even when k lies a
+// thousand standard deviations from the row (a padded head, outlier features),
+// which single-precision shifted sums do not: rows of 3e5 elements around 100
+// whose first three elements are 0 gave rstd 1e-4 off in float32.  It plays the
+// part of the reference's Welford merge across work-groups (WelfordOps::combine,
+// SharedReduceOps.h:71-88) with no division per element and no more passes over
+// X.  The second launch forms mean = k + s1/N in float64 and splits it into
+// hi = float(mean), which is the saved statistic, and lo = float(mean - hi); the
+// third launch evaluates (x - hi) - lo, so the rounding of the saved mean never
+// enters y, as in the resident kernel.  On a constant row x - k is exactly zero:
+// mean is the constant and y is beta bit for bit.
+//
+// The partial sums and `lo` cross the launches in the first bytes of the chunk's
+// own piece of Y (24 bytes, 8-byte aligned; every chunk is at least 1024 packs),
+// which only that chunk's workgroup of the third launch overwrites, after it has
+// read `lo`: no workspace, and no workgroup waits for another.
+constexpr int kSplitSlotBytes = 24;
 
 template <class T>
-__device__ __forceinline__ float split_row_centre(const T* xr, int N) {
-  const float a = (float)xr[0], b = (float)xr[N > 1 ? 1 : 0], c = (float)xr[N > 2 ? 2 : 0];
-  return fmaxf(fminf(a, b), fminf(fmaxf(a, b), c));
+__device__ __forceinline__ double* split_chunk_slot(T* y_row, int64_t first_pack) {
+  constexpr int E = elems_per_pack<T>::value;
+  return reinterpret_cast<double*>(
+      (reinterpret_cast<uintptr_t>(y_row + first_pack * E) + 7) & ~uintptr_t(7));
+}
+
+// The packs [p0, p1) of chunk `chunk` out of `chunks`.
+__device__ __forceinline__ void split_chunk_range(int chunk, int chunks, int64_t chunk_packs,
+                                                  int64_t npacks, int64_t* p0, int64_t* p1) {
+  *p0 = (int64_t)chunk * chunk_packs;
+  *p1 = chunk == chunks - 1 ? npacks : *p0 + chunk_packs;
 }
 
 template <class T, int BLOCK, bool RMS>
@@ -363,62 +409,74 @@ __global__ void __launch_bounds__(BLOCK)
 norm_fwd_split_sums_kernel(const T* __restrict__ x, T* __restrict__ y, int N,
                            int64_t chunk_packs) {
   constexpr int E = elems_per_pack<T>::value;
-  __shared__ float red[reduce_lds_floats<BLOCK, BLOCK, 2>::value];
-  int phase = 0;
+  __shared__ double red[2 * (BLOCK / 64)];
   const int64_t row = blockIdx.y;
   const T* xr = x + row * (int64_t)N;
   const int64_t npacks = ((int64_t)N + E - 1) / E;
-  const int64_t p0 = (int64_t)blockIdx.x * chunk_packs;
-  const int64_t p1 = p0 + chunk_packs < npacks ? p0 + chunk_packs : npacks;
-  const float k = RMS ? 0.0f : split_row_centre(xr, N);
-  float acc[2] = {0.0f, 0.0f};
+  int64_t p0, p1;
+  split_chunk_range(blockIdx.x, gridDim.x, chunk_packs, npacks, &p0, &p1);
+  const double k = RMS ? 0.0 : (double)split_row_centre(xr, N);
+  double s1 = 0.0, s2 = 0.0;
   for (int64_t pk = p0 + threadIdx.x; pk < p1; pk += BLOCK) {
     const int e0 = (int)(pk * E);
     const Pack<T, E> p = load_row_pack<T, E, false>(xr, e0, N, true, 0.0f);
     const int nvalid = N - e0;
 #pragma unroll
     for (int i = 0; i < E; ++i) {
-      const float d = (i < nvalid) ? p.get(i) - k : 0.0f;
-      acc[0] += d;
-      acc[1] = fmaf(d, d, acc[1]);
+      const double d = (i < nvalid) ? (double)p.get(i) - k : 0.0;
+      if constexpr (!RMS) s1 += d;
+      s2 = fma(d, d, s2);
     }
   }
-  group_allreduce<BLOCK, BLOCK, 2, SumOp>(acc, red, phase);
+  block_sum2_f64<BLOCK>(s1, s2, red);
   if (threadIdx.x == 0) {
-    float* sc = split_row_scratch(y + row * (int64_t)N);
-    sc[2 * blockIdx.x] = acc[0];
-    sc[2 * blockIdx.x + 1] = acc[1];
+    double* slot = split_chunk_slot(y + row * (int64_t)N, p0);
+    slot[0] = s1;
+    slot[1] = s2;
   }
 }
 
-// One wavefront per row: lane l adds partial sums l, l + 64, ... and a butterfly
-// adds the lanes, the same order on every run.
+// One wavefront per row: lane l adds the partial sums of chunks l, l + 64, ...
+// and a fixed tree adds the lanes, the same order on every run.
 template <class T, bool RMS>
 __global__ void __launch_bounds__(64)
 norm_fwd_split_stats_kernel(const T* __restrict__ x, T* __restrict__ y,
                             float* __restrict__ mean, float* __restrict__ rstd, int N, int chunks,
-                            float eps) {
+                            int64_t chunk_packs, float eps) {
   const int64_t row = blockIdx.x;
-  const float* sc = split_row_scratch(y + row * (int64_t)N);
-  float s1 = 0.0f, s2 = 0.0f;
+  T* yr = y + row * (int64_t)N;
+  double s1 = 0.0, s2 = 0.0;
   for (int c = threadIdx.x; c < chunks; c += 64) {
-    s1 += sc[2 * c];
-    s2 += sc[2 * c + 1];
+    const double* slot = split_chunk_slot(yr, (int64_t)c * chunk_packs);
+    s1 += slot[0];
+    s2 += slot[1];
   }
-  s1 = wave_group_allreduce<64, SumOp>(s1);
-  s2 = wave_group_allreduce<64, SumOp>(s2);
-  if (threadIdx.x == 0) {
-    const float fN = (float)N;
-    if constexpr (RMS) {
-      rstd[row] = 1.0f / sqrtf(s2 / fN + eps);
-    } else {
-      const float k = split_row_centre(x + row * (int64_t)N, N);
-      const float m1 = s1 / fN;
-      const float var = fmaxf((s2 - s1 * m1) / fN, 0.0f);
-      mean[row] = k + m1;
-      rstd[row] = 1.0f / sqrtf(var + eps);
+#pragma unroll
+  for (int off = 32; off > 0; off >>= 1) {
+    s1 += __shfl_down(s1, off, 64);
+    s2 += __shfl_down(s2, off, 64);
+  }
+  s1 = __shfl(s1, 0, 64);
+  s2 = __shfl(s2, 0, 64);
+  const double dN = (double)N;
+  float lo = 0.0f;
+  if constexpr (RMS) {
+    if (threadIdx.x == 0) rstd[row] = (float)(1.0 / sqrt(s2 / dN + (double)eps));
+  } else {
+    const double m1 = s1 / dN;
+    const double mu = (double)split_row_centre(x + row * (int64_t)N, N) + m1;
+    double var = (s2 - s1 * m1) / dN;
+    var = var < 0.0 ? 0.0 : var;  // (a select: NaN stays NaN)
+    const float hi = (float)mu;
+    lo = (float)(mu - (double)hi);
+    if (threadIdx.x == 0) {
+      mean[row] = var == var ? hi : (float)var;  // NaN variance (a NaN or inf element): NaN mean
+      rstd[row] = (float)(1.0 / sqrt(var + (double)eps));
     }
   }
+  if constexpr (!RMS)
+    for (int c = threadIdx.x; c < chunks; c += 64)
+      *reinterpret_cast<float*>(split_chunk_slot(yr, (int64_t)c * chunk_packs)) = lo;
 }
 
 template <class T, class WT, int BLOCK, bool RMS>
@@ -432,10 +490,13 @@ norm_fwd_split_apply_kernel(const T* __restrict__ x, const WT* __restrict__ gamm
   const T* xr = x + row * (int64_t)N;
   T* yr = y + row * (int64_t)N;
   const int64_t npacks = ((int64_t)N + E - 1) / E;
-  const int64_t p0 = (int64_t)blockIdx.x * chunk_packs;
-  const int64_t p1 = p0 + chunk_packs < npacks ? p0 + chunk_packs : npacks;
-  const float mu = RMS ? 0.0f : mean[row];
+  int64_t p0, p1;
+  split_chunk_range(blockIdx.x, gridDim.x, chunk_packs, npacks, &p0, &p1);
+  const float hi = RMS ? 0.0f : mean[row];
   const float rs = rstd[row];
+  // the low part of the mean sits where this workgroup is about to write y
+  const float lo = RMS ? 0.0f : *reinterpret_cast<const float*>(split_chunk_slot(yr, p0));
+  __syncthreads();
   for (int64_t pk = p0 + threadIdx.x; pk < p1; pk += BLOCK) {
     const int e0 = (int)(pk * E);
     const Pack<T, E> p = load_row_pack<T, E, true>(xr, e0, N, true, 0.0f);
@@ -451,7 +512,7 @@ norm_fwd_split_apply_kernel(const T* __restrict__ x, const WT* __restrict__ gamm
       if constexpr (RMS)
         v = (p.get(i) * rs) * pg.get(i);
       else
-        v = ((p.get(i) - mu) * rs) * pg.get(i) + pb.get(i);
+        v = (((p.get(i) - hi) - lo) * rs) * pg.get(i) + pb.get(i);
       o.set(i, v);
     }
     store_row_pack<T, E, true>(yr, e0, N, true, o);
@@ -725,8 +786,8 @@ norm_bwd_split_sums_kernel(const T* __restrict__ dy, const T* __restrict__ x,
   const T* xr = x + row * (int64_t)N;
   const T* gr = dy + row * (int64_t)N;
   const int64_t npacks = ((int64_t)N + E - 1) / E;
-  const int64_t p0 = (int64_t)blockIdx.x * chunk_packs;
-  const int64_t p1 = p0 + chunk_packs < npacks ? p0 + chunk_packs : npacks;
+  int64_t p0, p1;
+  split_chunk_range(blockIdx.x, gridDim.x, chunk_packs, npacks, &p0, &p1);
   const float mu = RMS ? 0.0f : mean[row];
   const float rs = rstd[row];
   float acc[2] = {0.0f, 0.0f};
@@ -766,8 +827,8 @@ norm_bwd_split_dx_kernel(const T* __restrict__ dy, const T* __restrict__ x,
   const T* gr = dy + row * (int64_t)N;
   T* dr = dx + row * (int64_t)N;
   const int64_t npacks = ((int64_t)N + E - 1) / E;
-  const int64_t p0 = (int64_t)blockIdx.x * chunk_packs;
-  const int64_t p1 = p0 + chunk_packs < npacks ? p0 + chunk_packs : npacks;
+  int64_t p0, p1;
+  split_chunk_range(blockIdx.x, gridDim.x, chunk_packs, npacks, &p0, &p1);
   const float mu = RMS ? 0.0f : mean[row];
   const float rs = rstd[row];
   float acc[2] = {0.0f, 0.0f};

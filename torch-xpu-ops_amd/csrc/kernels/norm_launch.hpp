@@ -32,9 +32,9 @@ struct NormFwdLauncher {
   };
 };
 
-// The split-row forward keeps a row's partial sums in the first bytes of the
-// row's Y and hands the statistics to its last launch through mean / rstd: it
-// needs those outputs, and a Y that does not overlap X.
+// The split-row forward keeps a chunk's partial sums in the first bytes of the
+// chunk's piece of Y and hands the statistics to its last launch through mean /
+// rstd: it needs those outputs, and a Y that does not overlap X.
 template <class T, bool RMS>
 inline bool norm_fwd_can_split(const Plan& plan, const NormFwdArgs& a) {
   if (plan.split <= 1 || a.M > 65535 || a.rstd == nullptr || (!RMS && a.mean == nullptr))
@@ -59,7 +59,8 @@ int launch_norm_fwd(const Plan& plan, const NormFwdArgs& a, hipStream_t stream) 
                        dim3(kStreamBlock), 0, stream, (const T*)a.x, (T*)a.y, a.N,
                        plan.chunk_packs);
     hipLaunchKernelGGL((norm_fwd_split_stats_kernel<T, RMS>), dim3((unsigned)a.M), dim3(64), 0,
-                       stream, (const T*)a.x, (T*)a.y, a.mean, a.rstd, a.N, plan.split, a.eps);
+                       stream, (const T*)a.x, (T*)a.y, a.mean, a.rstd, a.N, plan.split,
+                       plan.chunk_packs, a.eps);
     hipLaunchKernelGGL((norm_fwd_split_apply_kernel<T, WT, kStreamBlock, RMS>), grid,
                        dim3(kStreamBlock), 0, stream, (const T*)a.x, (const WT*)a.gamma,
                        (const WT*)a.beta, (T*)a.y, (const float*)a.mean, (const float*)a.rstd,

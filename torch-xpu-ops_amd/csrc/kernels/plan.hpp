@@ -418,7 +418,11 @@ inline int make_plan(OpClass oc, int64_t M, int64_t N, int esize, int num_cus, c
       int64_t cp = (packs + want - 1) / want;
       cp = (cp + kStreamBlock - 1) / kStreamBlock * kStreamBlock;
       if (cp < min_chunk && !(ov.G < 0 && ov.V > 0)) cp = min_chunk;
-      const int64_t chunks = (packs + cp - 1) / cp;
+      int64_t chunks = (packs + cp - 1) / cp;
+      // a remainder of less than one workgroup stride joins the chunk before it, so
+      // every chunk holds at least kStreamBlock packs (the forward keeps a chunk's
+      // partial sums in the first bytes of the chunk's own output)
+      if (chunks > 1 && packs - (chunks - 1) * cp < kStreamBlock) --chunks;
       if (chunks > 1) {
         p.split = (int)chunks;
         p.chunk_packs = cp;
