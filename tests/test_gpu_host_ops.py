@@ -171,11 +171,95 @@ def test_softmax_half_to_float(ops, gpu):
 
 
 def test_unsupported_dtype_is_an_error_not_a_fallback(ops, gpu):
-    x = torch.randn(4, 8, dtype=torch.float64, device=gpu)
-    with pytest.raises(RuntimeError, match="not implemented by the MI355X kernels"):
-        ops.native_layer_norm(x, [8], None, None, 1e-5)
+    x = torch.randint(0, 5, (4, 8), dtype=torch.int32, device=gpu)
     with pytest.raises(RuntimeError, match="not implemented by the MI355X kernels"):
         ops._softmax(x, -1, False)
+    xc = torch.randn(4, 8, dtype=torch.complex64, device=gpu)
+    with pytest.raises(RuntimeError, match="not implemented by the MI355X kernels"):
+        ops._softmax(xc, -1, False)
+
+
+def test_zero_width_rows_have_defined_statistics(ops, gpu):
+    """M > 0 rows of no elements: nothing is launched, and the saved statistics are what the CPU
+    kernel's formulas give on an empty row (mean 0, rstd NaN), not uninitialised memory."""
+    x = torch.empty(3, 0, device=gpu)
+    y, mean, rstd = ops.native_layer_norm(x, [0], None, None, 1e-5)
+    cy, cm, cr = torch.ops.aten.native_layer_norm(x.cpu(), [0], None, None, 1e-5)
+    assert y.shape == (3, 0) and mean.shape == cm.shape and rstd.shape == cr.shape
+    assert torch.equal(mean.cpu(), cm) and bool(torch.isnan(rstd).all()) and bool(torch.isnan(cr).all())
+    y, rstd = ops._fused_rms_norm(x, [0], None, 1e-5)
+    _, cr = torch.ops.aten._fused_rms_norm(x.cpu(), [0], None, 1e-5)
+    assert y.shape == (3, 0) and rstd.shape == cr.shape
+    assert bool(torch.isnan(rstd).all()) and bool(torch.isnan(cr).all())
+    xg = torch.empty(2, 4, 0, device=gpu)
+    y, mean, rstd = ops.native_group_norm(xg, None, None, 2, 4, 0, 2, 1e-5)
+    _, cm, cr = torch.ops.aten.native_group_norm(xg.cpu(), None, None, 2, 4, 0, 2, 1e-5)
+    assert y.shape == (2, 4, 0) and mean.shape == (2, 2)
+    assert torch.equal(mean.cpu(), cm) and bool(torch.isnan(rstd).all()) and bool(torch.isnan(cr).all())
+
+
+def test_float64_is_delegated_to_the_stock_kernels(pkg, ops, gpu):
+    """The kernels accumulate in float32 and do not take float64; the reference computes float64
+    in double (sycl/LayerNormKernels.cpp:1418-1438, sycl/SoftMaxKernels.cpp:2125-2178).  The host
+    layer hands float64 GPU tensors to the kernels PyTorch-ROCm ships (the idea of
+    src/ATen/native/xpu/XPUFallback.cpp:59-69), so that after the aten override everything that
+    worked before still works and gives the same bits."""
+    import warnings
+    g = gen(60)
+    x = torch.randn(6, 5, 64, generator=g, dtype=torch.float64).to(gpu)
+    w = torch.randn(64, generator=g, dtype=torch.float64).to(gpu)
+    b = torch.randn(64, generator=g, dtype=torch.float64).to(gpu)
+    dy = torch.randn(6, 5, 64, generator=g, dtype=torch.float64).to(gpu)
+    xn = torch.randn(4, 8, 6, 6, generator=g, dtype=torch.float64).to(gpu)
+    wn = torch.randn(8, generator=g, dtype=torch.float64).to(gpu)
+    mask = (torch.rand(6, 5, 64, generator=g) < 0.3).to(gpu)
+
+    def everything():
+        out = []
+        for fn in (lambda t: F.layer_norm(t, (64,), w, b, 1e-5),
+                   lambda t: F.rms_norm(t, (64,), w, 1e-6),
+                   lambda t: F.softmax(t, -1), lambda t: F.softmax(t, 1),
+                   lambda t: F.log_softmax(t, -1), lambda t: F.log_softmax(t, 0),
+                   lambda t: torch._masked_softmax(t, mask, -1, 2),
+                   lambda t: torch.ops.aten._safe_softmax(t, -1)):
+            xs = x.detach().clone().requires_grad_()
+            y = fn(xs)
+            y.backward(dy)
+            out += [y.detach(), xs.grad]
+        xs = xn.detach().clone().requires_grad_()
+        y = F.group_norm(xs, 2, wn, wn, 1e-5)
+        y.backward(torch.ones_like(y))
+        out += [y.detach(), xs.grad]
+        o = torch.empty_like(x)
+        torch.softmax(x, -1, out=o)
+        out.append(o)
+        return out
+
+    pkg.restore_aten_ops()
+    stock = everything()
+    with warnings.catch_warnings():
+        warnings.simplefilter("ignore")
+        pkg.override_aten_ops()
+        ours = everything()
+    assert len(stock) == len(ours)
+    for a, r in zip(ours, stock):
+        assert a.dtype == torch.float64 and torch.equal(a, r)
+    # and the operators called directly
+    y, mean, rstd = ops.native_layer_norm(x, [64], w, b, 1e-5)
+    sy, sm, sr = torch.ops.aten.native_layer_norm.default(x, [64], w, b, 1e-5)
+    assert y.dtype == torch.float64 and torch.equal(y, sy) and torch.equal(rstd, sr)
+    ref = F.layer_norm(x.cpu(), (64,), w.cpu(), b.cpu(), 1e-5)
+    assert float((y.cpu() - ref).abs().max()) < 1e-12  # float64 accuracy, not float32
+    # restore really restores: float32 goes back to the stock kernels, and forth again
+    x32 = x.float()
+    over = F.softmax(x32, -1)
+    pkg.restore_aten_ops()
+    stock32 = F.softmax(x32, -1)
+    with warnings.catch_warnings():
+        warnings.simplefilter("ignore")
+        pkg.override_aten_ops()
+    assert torch.equal(F.softmax(x32, -1), over)
+    assert_close(over, stock32, torch.float32, "override vs stock softmax")
 
 
 def test_aten_override_runs_autograd_end_to_end(pkg, gpu):

@@ -12,6 +12,8 @@ Two layers are exposed:
   * ``cabi``  -- ctypes bindings of the ``extern "C"`` launcher ABI (include/mi355x_rownorm.h),
                  taking torch tensors only as device memory.
 There is no CPU path and no fallback: if the compiled libraries are missing the import raises.
+(float64 GPU tensors, which these float32-accumulating kernels do not compute, are passed on by
+the host layer to the kernels PyTorch-ROCm ships.)
 """
 import os
 
@@ -55,7 +57,10 @@ def override_aten_ops():
     """Explicit opt-in: route the aten ops of this family to the MI355X kernels for GPU tensors,
     so ``F.layer_norm`` / ``F.rms_norm`` / ``F.group_norm`` / ``F.softmax`` / ``F.log_softmax``,
     ``torch._masked_softmax`` / ``torch._safe_softmax`` and their autograd formulas run them.
-    PyTorch warns about overriding existing kernels; that is why this is never done at import.  float64 inputs are rejected by the kernels after the override."""
+    PyTorch warns about overriding existing kernels; that is why this is never done at import.
+    float64 GPU tensors are handed on to the kernels PyTorch-ROCm itself ships (one warning per
+    process), so code that worked before the override keeps working.  ``restore_aten_ops()``
+    undoes the override."""
     import torch
     if _state["aten_lib"] is not None:
         return _state["aten_lib"]
@@ -76,3 +81,12 @@ def override_aten_ops():
     lib.impl("_masked_softmax_backward", m._masked_softmax_backward.default, "CUDA")
     _state["aten_lib"] = lib
     return lib
+
+
+def restore_aten_ops():
+    """Drops the registrations made by ``override_aten_ops()``: the aten ops go back to the kernels
+    PyTorch-ROCm ships.  A no-op when nothing is overridden."""
+    lib = _state["aten_lib"]
+    if lib is not None:
+        lib._destroy()
+        _state["aten_lib"] = None

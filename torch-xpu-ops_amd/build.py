@@ -74,7 +74,7 @@ def build_host(out=HOST_LIB, verbose=False):
            "-I" + os.path.join(tdir, "include"),
            "-I" + os.path.join(tdir, "include", "torch", "csrc", "api", "include"),
            "-I/opt/rocm/include", "-I" + os.path.join(ROOT, "include")] + srcs + [
-           "-L" + os.path.join(tdir, "lib"), "-ltorch", "-ltorch_cpu", "-lc10", "-lc10_hip",
+           "-L" + os.path.join(tdir, "lib"), "-ltorch", "-ltorch_cpu", "-ltorch_hip", "-lc10", "-lc10_hip",
            "-L" + LIB_DIR, "-lmi355x_rownorm",
            "-Wl,-rpath," + os.path.join(tdir, "lib"), "-Wl,-rpath,$ORIGIN", "-o", out]
     msg = _run(cmd)

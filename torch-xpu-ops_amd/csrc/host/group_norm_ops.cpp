@@ -6,6 +6,9 @@
 #include "group_norm_ops.h"
 
 #include <ATen/native/group_norm.h>
+#include <ATen/ops/native_group_norm_backward_cuda_dispatch.h>
+#include <ATen/ops/native_group_norm_cuda_dispatch.h>
+#include <limits>
 
 #include "host_common.h"
 
@@ -39,6 +42,21 @@ at::ScalarType to_scalar_type(rownorm_dtype d) {
   return d == ROWNORM_F32 ? at::kFloat : d == ROWNORM_F16 ? at::kHalf : at::kBFloat16;
 }
 
+// The GPU slot of one of ATen's DispatchStub objects (a standard-layout class
+// whose only non-static data member is its DispatchStubImpl; it has a setter
+// for the slot but no getter, and uninstalling needs the previous value).
+template <class Stub>
+void*& gpu_slot(Stub& stub) {
+  return reinterpret_cast<at::native::DispatchStubImpl*>(&stub)->cuda_dispatch_ptr;
+}
+
+struct SavedStubs {
+  bool installed = false;
+  void* forward = nullptr;
+  void* backward = nullptr;
+};
+SavedStubs g_group_norm_saved;
+
 }  // namespace
 
 // group_norm_kernel, GroupNormKernels.cpp:499-530 (checks at :377-379).
@@ -46,6 +64,13 @@ void group_norm_kernel(const Tensor& X, const Tensor& gamma, const Tensor& beta,
                        int64_t C, int64_t HxW, int64_t group, double eps, Tensor& Y, Tensor& mean,
                        Tensor& rstd) {
   static const char* op = "mi355x::group_norm_kernel";
+  if (delegated_dtype(X) && g_group_norm_saved.forward != nullptr) {
+    // reached through ATen's GroupNormKernel stub: pass float64 on to the kernel
+    // that was registered before
+    warn_delegated(op);
+    return reinterpret_cast<at::native::forward_fn>(g_group_norm_saved.forward)(
+        X, gamma, beta, N, C, HxW, group, eps, Y, mean, rstd);
+  }
   check_gpu(X, op, "X");
   TORCH_CHECK(X.numel() == N * C * HxW, op, ": X does not hold N*C*HxW elements");
   TORCH_CHECK(!gamma.defined() || gamma.numel() == C, op, ": gamma must hold C elements");
@@ -56,6 +81,12 @@ void group_norm_kernel(const Tensor& X, const Tensor& gamma, const Tensor& beta,
   if (N == 0) return;
   const rownorm_dtype xd = to_rownorm_dtype(X.scalar_type(), op);
   const rownorm_dtype sd = stat_dtype(X, gamma, beta, op);
+  if (C == 0 || HxW == 0) {
+    // groups of no elements: what the CPU kernel's formulas give, mean 0 and rstd NaN
+    if (mean.defined()) mean.zero_();
+    if (rstd.defined()) rstd.fill_(std::numeric_limits<double>::quiet_NaN());
+    return;
+  }
   for (const Tensor* t : {&mean, &rstd}) {
     if (t->defined()) {
       TORCH_CHECK(t->is_contiguous() && t->numel() == N * group &&
@@ -82,6 +113,11 @@ void group_norm_backward_kernel(const Tensor& dY, const Tensor& X, const Tensor&
                                 int64_t HxW, int64_t group, Tensor& dX, Tensor& dgamma,
                                 Tensor& dbeta) {
   static const char* op = "mi355x::group_norm_backward_kernel";
+  if (delegated_dtype(X) && g_group_norm_saved.backward != nullptr) {
+    warn_delegated(op);
+    return reinterpret_cast<at::native::backward_fn>(g_group_norm_saved.backward)(
+        dY, X, mean, rstd, gamma, N, C, HxW, group, dX, dgamma, dbeta);
+  }
   check_gpu(X, op, "X");
   check_same_device(X, dY, op, "dY");
   TORCH_CHECK(dY.numel() == N * C * HxW && X.numel() == N * C * HxW, op,
@@ -145,6 +181,10 @@ std::tuple<Tensor, Tensor, Tensor> native_group_norm(const Tensor& X,
                                                      int64_t N, int64_t C, int64_t HxW,
                                                      int64_t group, double eps) {
   static const char* op = "mi355x::native_group_norm";
+  if (delegated_dtype(X)) {
+    warn_delegated(op);
+    return at::cuda::native_group_norm(X, weight_opt, bias_opt, N, C, HxW, group, eps);
+  }
   const Tensor gamma = defined_or_empty(weight_opt);
   const Tensor beta = defined_or_empty(bias_opt);
   TORCH_CHECK(group > 0, "Expected num groups to be greater than 0, got ", group);
@@ -180,6 +220,11 @@ std::tuple<Tensor, Tensor, Tensor> native_group_norm_backward(
     const std::optional<Tensor>& weight_opt, int64_t N, int64_t C, int64_t HxW, int64_t group,
     std::array<bool, 3> output_mask) {
   static const char* op = "mi355x::native_group_norm_backward";
+  if (delegated_dtype(X)) {
+    warn_delegated(op);
+    return at::cuda::native_group_norm_backward(dY, X, mean, rstd, weight_opt, N, C, HxW, group,
+                                                output_mask);
+  }
   const Tensor gamma = defined_or_empty(weight_opt);
   TORCH_CHECK(X.scalar_type() == dY.scalar_type(), "Expected scalar types of X and dY are same.");
   check_gpu(X, op, "input");
@@ -196,8 +241,19 @@ std::tuple<Tensor, Tensor, Tensor> native_group_norm_backward(
 }
 
 void install_group_norm_dispatch_stubs() {
+  if (g_group_norm_saved.installed) return;
+  g_group_norm_saved.forward = gpu_slot(at::native::GroupNormKernel);
+  g_group_norm_saved.backward = gpu_slot(at::native::GroupNormBackwardKernel);
+  g_group_norm_saved.installed = true;
   at::native::GroupNormKernel.set_cuda_dispatch_ptr(&group_norm_kernel);
   at::native::GroupNormBackwardKernel.set_cuda_dispatch_ptr(&group_norm_backward_kernel);
+}
+
+void uninstall_group_norm_dispatch_stubs() {
+  if (!g_group_norm_saved.installed) return;
+  gpu_slot(at::native::GroupNormKernel) = g_group_norm_saved.forward;
+  gpu_slot(at::native::GroupNormBackwardKernel) = g_group_norm_saved.backward;
+  g_group_norm_saved = SavedStubs{};
 }
 
 }  // namespace mi355x

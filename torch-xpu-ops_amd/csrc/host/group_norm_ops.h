@@ -33,7 +33,11 @@ std::tuple<at::Tensor, at::Tensor, at::Tensor> native_group_norm_backward(
 
 // Points ATen's GroupNormKernel / GroupNormBackwardKernel dispatch stubs at the
 // kernel entries above for GPU tensors: REGISTER_XPU_DISPATCH in
-// GroupNorm.cpp:19-23 of the reference.  Explicit, never at import.
+// GroupNorm.cpp:19-23 of the reference.  Explicit, never at import.  ATen's own
+// native_group_norm host function then reaches these kernels; float64 calls are
+// passed on to the kernels that were registered before.  uninstall_* puts the
+// previous kernels back.  Not synchronized with concurrent calls of the ops.
 void install_group_norm_dispatch_stubs();
+void uninstall_group_norm_dispatch_stubs();
 
 }  // namespace mi355x

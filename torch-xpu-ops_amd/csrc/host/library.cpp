@@ -75,4 +75,8 @@ TORCH_LIBRARY(mi355x, m) {
       &mi355x::native_group_norm_backward);
   m.def("install_group_norm_dispatch_stubs() -> ()", &mi355x::install_group_norm_dispatch_stubs);
   m.def("install_layer_norm_dispatch_stubs() -> ()", &mi355x::install_layer_norm_dispatch_stubs);
+  m.def("uninstall_group_norm_dispatch_stubs() -> ()",
+        &mi355x::uninstall_group_norm_dispatch_stubs);
+  m.def("uninstall_layer_norm_dispatch_stubs() -> ()",
+        &mi355x::uninstall_layer_norm_dispatch_stubs);
 }

@@ -10,6 +10,13 @@
 
 #include <ATen/WrapDimUtils.h>
 #include <ATen/native/Resize.h>
+#include <ATen/ops/_log_softmax_backward_data_cuda_dispatch.h>
+#include <ATen/ops/_log_softmax_cuda_dispatch.h>
+#include <ATen/ops/_masked_softmax_backward_cuda_dispatch.h>
+#include <ATen/ops/_masked_softmax_cuda_dispatch.h>
+#include <ATen/ops/_safe_softmax_native.h>
+#include <ATen/ops/_softmax_backward_data_cuda_dispatch.h>
+#include <ATen/ops/_softmax_cuda_dispatch.h>
 
 #include "host_common.h"
 
@@ -176,6 +183,11 @@ Tensor _safe_softmax_kernel(const Tensor& self, int64_t dim, bool half_to_float)
 // kernel, any other dtype request converts the input first.
 Tensor _safe_softmax(const Tensor& self, int64_t dim, std::optional<at::ScalarType> dtype) {
   check_gpu(self, "mi355x::_safe_softmax", "self");
+  if (delegated_dtype(self) || (self.is_cuda() && dtype == at::kDouble)) {
+    // ATen's composite formula; the softmax inside it comes back here and is delegated
+    warn_delegated("mi355x::_safe_softmax");
+    return at::native::_safe_softmax(self, dim, dtype);
+  }
   if (self.scalar_type() == at::kHalf && dtype == at::kFloat)
     return _safe_softmax_kernel(self, dim, true);
   const Tensor converted = dtype.has_value() ? self.toType(dtype.value()) : self;
@@ -284,10 +296,18 @@ Tensor masked_softmax_backward_kernel(const Tensor& grad_, const Tensor& output_
 // masked_softmax_xpu / masked_softmax_backward_xpu, SoftMax.cpp:112-126.
 Tensor _masked_softmax(const Tensor& self, const Tensor& mask, std::optional<int64_t> dim,
                        std::optional<int64_t> mask_type) {
+  if (delegated_dtype(self)) {
+    warn_delegated("mi355x::_masked_softmax");
+    return at::cuda::_masked_softmax(self, mask, dim, mask_type);
+  }
   return masked_softmax_kernel(self, mask, dim, mask_type);
 }
 Tensor _masked_softmax_backward(const Tensor& grad_output, const Tensor& output,
                                 const Tensor& mask, std::optional<int64_t> dim) {
+  if (delegated_dtype(grad_output)) {
+    warn_delegated("mi355x::_masked_softmax_backward");
+    return at::cuda::_masked_softmax_backward(grad_output, output, mask, dim);
+  }
   return masked_softmax_backward_kernel(grad_output, output, mask, dim);
 }
 
@@ -311,23 +331,39 @@ void _log_softmax_backward_kernel(const Tensor& grad, const Tensor& output, int6
 }
 
 Tensor _softmax(const Tensor& self, int64_t dim, bool half_to_float) {
+  if (delegated_dtype(self)) {
+    warn_delegated("mi355x::_softmax");
+    return at::cuda::_softmax(self, dim, half_to_float);
+  }
   check_gpu(self, "mi355x::_softmax", "self");
   Tensor out = alloc_forward_output(self, half_to_float);
   _softmax_kernel(self, dim, half_to_float, out);
   return out;
 }
 Tensor _log_softmax(const Tensor& self, int64_t dim, bool half_to_float) {
+  if (delegated_dtype(self)) {
+    warn_delegated("mi355x::_log_softmax");
+    return at::cuda::_log_softmax(self, dim, half_to_float);
+  }
   check_gpu(self, "mi355x::_log_softmax", "self");
   Tensor out = alloc_forward_output(self, half_to_float);
   _log_softmax_kernel(self, dim, half_to_float, out);
   return out;
 }
 Tensor& _softmax_out(const Tensor& self, int64_t dim, bool half_to_float, Tensor& out) {
+  if (delegated_dtype(self)) {
+    warn_delegated("mi355x::_softmax.out");
+    return at::cuda::_softmax_out(out, self, dim, half_to_float);
+  }
   at::native::resize_output(out, self.sizes());
   _softmax_kernel(self, dim, half_to_float, out);
   return out;
 }
 Tensor& _log_softmax_out(const Tensor& self, int64_t dim, bool half_to_float, Tensor& out) {
+  if (delegated_dtype(self)) {
+    warn_delegated("mi355x::_log_softmax.out");
+    return at::cuda::_log_softmax_out(out, self, dim, half_to_float);
+  }
   at::native::resize_output(out, self.sizes());
   _log_softmax_kernel(self, dim, half_to_float, out);
   return out;
@@ -335,6 +371,10 @@ Tensor& _log_softmax_out(const Tensor& self, int64_t dim, bool half_to_float, Te
 
 Tensor _softmax_backward_data(const Tensor& grad_output, const Tensor& output, int64_t dim,
                               at::ScalarType input_dtype) {
+  if (delegated_dtype(grad_output)) {
+    warn_delegated("mi355x::_softmax_backward_data");
+    return at::cuda::_softmax_backward_data(grad_output, output, dim, input_dtype);
+  }
   const bool h2f = backward_half_to_float(grad_output, input_dtype);
   check_gpu(grad_output, "mi355x::_softmax_backward_data", "grad_output");
   Tensor gi = at::empty_like(grad_output, grad_output.options().dtype(input_dtype),
@@ -344,6 +384,10 @@ Tensor _softmax_backward_data(const Tensor& grad_output, const Tensor& output, i
 }
 Tensor _log_softmax_backward_data(const Tensor& grad_output, const Tensor& output, int64_t dim,
                                   at::ScalarType input_dtype) {
+  if (delegated_dtype(grad_output)) {
+    warn_delegated("mi355x::_log_softmax_backward_data");
+    return at::cuda::_log_softmax_backward_data(grad_output, output, dim, input_dtype);
+  }
   const bool h2f = backward_half_to_float(grad_output, input_dtype);
   check_gpu(grad_output, "mi355x::_log_softmax_backward_data", "grad_output");
   Tensor gi = at::empty_like(grad_output, grad_output.options().dtype(input_dtype),
@@ -353,6 +397,10 @@ Tensor _log_softmax_backward_data(const Tensor& grad_output, const Tensor& outpu
 }
 Tensor& _softmax_backward_data_out(const Tensor& grad_output, const Tensor& output, int64_t dim,
                                    at::ScalarType input_dtype, Tensor& grad_input) {
+  if (delegated_dtype(grad_output)) {
+    warn_delegated("mi355x::_softmax_backward_data.out");
+    return at::cuda::_softmax_backward_data_out(grad_input, grad_output, output, dim, input_dtype);
+  }
   const bool h2f = backward_half_to_float(grad_output, input_dtype);
   at::native::resize_output(grad_input, grad_output.sizes());
   _softmax_backward_kernel(grad_output, output, dim, h2f, grad_input);
@@ -361,6 +409,11 @@ Tensor& _softmax_backward_data_out(const Tensor& grad_output, const Tensor& outp
 Tensor& _log_softmax_backward_data_out(const Tensor& grad_output, const Tensor& output,
                                        int64_t dim, at::ScalarType input_dtype,
                                        Tensor& grad_input) {
+  if (delegated_dtype(grad_output)) {
+    warn_delegated("mi355x::_log_softmax_backward_data.out");
+    return at::cuda::_log_softmax_backward_data_out(grad_input, grad_output, output, dim,
+                                                    input_dtype);
+  }
   const bool h2f = backward_half_to_float(grad_output, input_dtype);
   at::native::resize_output(grad_input, grad_output.sizes());
   _log_softmax_backward_kernel(grad_output, output, dim, h2f, grad_input);
