@@ -21,7 +21,13 @@
  *    argument (nothing was launched), or a positive hipError_t value when a
  *    launch failed.  mi355x_rownorm_error_string() renders either.
  *  - M == 0 or N == 0 is a successful no-op, like the `if (M > 0)` guards in
- *    LayerNorm.cpp:77,236,301 and `numel() > 0` in SoftMaxKernels.cpp:2150.
+ *    LayerNorm.cpp:77,236,301 and `numel() > 0` in SoftMaxKernels.cpp:2150
+ *    (mean / rstd are not written then; the host layer fills them).
+ *  - `eps` is a float where the reference's kernel entries take a double
+ *    (LayerNormKernels.h:25): every supported dtype accumulates in float32, and
+ *    the reference converts eps to that accumulate type before use
+ *    (LayerNormKernels.cpp:1434), so nothing is lost; float64 rows are not
+ *    computed here at all (the host layer passes them to the stock kernels).
  */
 #ifndef MI355X_ROWNORM_H_
 #define MI355X_ROWNORM_H_
@@ -288,12 +294,23 @@ int mi355x_softmax_strided_plan(int backward, int64_t outer, int64_t dim_size, i
 int mi355x_rownorm_plan(rownorm_op op, int64_t M, int64_t N, rownorm_dtype x_dtype,
                         rownorm_dtype w_dtype, rownorm_plan* out);
 
+/* The same query for tensors that do NOT all start on a 128-byte line
+ * (off_line != 0), which is what the norm forwards and the softmax ops see
+ * through their pointers: rows of at most 64 packs then take one pack a lane.
+ * off_line == 0 is mi355x_rownorm_plan. */
+int mi355x_rownorm_plan_at(rownorm_op op, int64_t M, int64_t N, rownorm_dtype x_dtype,
+                           rownorm_dtype w_dtype, int off_line, rownorm_plan* out);
+
 /* Test and tuning hook: force lanes_per_row / packs_per_lane / threads per
  * workgroup / workgroups per compute unit for one op (0 keeps the automatic
- * choice for that field; lanes_per_row == -1 forces the multi-pass kernel).  Process-global and not
- * synchronized with concurrent calls; production callers never use it.  A
- * call whose shape the forced variant cannot hold fails with
- * ROWNORM_ERR_OVERRIDE instead of silently choosing another. */
+ * choice for that field; lanes_per_row == -1 forces the multi-pass kernel).  Process-global;
+ * the four fields of an op are stored as one atomic word, so a call that runs
+ * while another thread changes the override uses the old or the new variant,
+ * never a mix.  Production callers never use it: with no override set (the
+ * state a process starts in) every entry point is re-entrant and reads no
+ * mutable global state.  A call whose shape the forced variant cannot hold
+ * fails with ROWNORM_ERR_OVERRIDE instead of silently choosing another, and so
+ * does a field outside 0..65535. */
 int mi355x_rownorm_set_override(rownorm_op op, int lanes_per_row, int packs_per_lane,
                                 int block_threads, int blocks_per_cu);
 

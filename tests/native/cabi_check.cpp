@@ -46,6 +46,7 @@ DECL(mi355x_group_norm_bwd_workspace_bytes);
 DECL(mi355x_group_norm_bwd);
 DECL(mi355x_group_norm_plan);
 DECL(mi355x_rownorm_plan);
+DECL(mi355x_rownorm_plan_at);
 DECL(mi355x_rownorm_set_override);
 
 static int failures = 0;
@@ -91,6 +92,7 @@ static bool load_all(void* lib) {
   LOAD(mi355x_group_norm_bwd);
   LOAD(mi355x_group_norm_plan);
   LOAD(mi355x_rownorm_plan);
+  LOAD(mi355x_rownorm_plan_at);
   LOAD(mi355x_rownorm_set_override);
   return ok;
 }

@@ -144,6 +144,44 @@ def test_plan_invariants(cabi, op, dt):
                 assert p["partial_rows"] == 0
 
 
+def test_plan_query_for_tensors_off_a_cache_line(cabi):
+    """The norm forwards and the softmax ops look at their pointers: rows of at most 64 packs in
+    tensors off a 128-byte line take one pack a lane.  mi355x_rownorm_plan_at reports that layout;
+    the norm backward takes it everywhere."""
+    for op in (cabi.OP_LAYER_NORM_FWD, cabi.OP_RMS_NORM_FWD, cabi.OP_SOFTMAX_FWD,
+               cabi.OP_SOFTMAX_BWD):
+        for dt, E in ((cabi.F32, 4), (cabi.F16, 8)):
+            for packs in (9, 16, 33, 64):
+                on = cabi.plan(op, 4096, packs * E, dt, dt)
+                off = cabi.plan(op, 4096, packs * E, dt, dt, off_line=True)
+                assert on["packs_per_lane"] > 1, (op, dt, packs, on)
+                assert off["packs_per_lane"] == 1 and off["lanes_per_row"] >= packs, (op, off)
+            # longer rows do not change
+            assert cabi.plan(op, 4096, 65 * E * 2, dt, dt) == cabi.plan(op, 4096, 65 * E * 2, dt, dt,
+                                                                        off_line=True)
+    for op in (cabi.OP_LAYER_NORM_BWD, cabi.OP_RMS_NORM_BWD):
+        assert cabi.plan(op, 4096, 256, cabi.F32, cabi.F32) == \
+            cabi.plan(op, 4096, 256, cabi.F32, cabi.F32, off_line=True)
+        assert cabi.plan(op, 4096, 256, cabi.F32, cabi.F32)["packs_per_lane"] == 1
+
+
+def test_override_fields_are_range_checked(cabi):
+    L = cabi.lib()
+    assert L.mi355x_rownorm_set_override(cabi.OP_SOFTMAX_FWD, 70000, 0, 0, 0) == -5
+    assert L.mi355x_rownorm_set_override(cabi.OP_SOFTMAX_FWD, 0, -1, 0, 0) == -5
+    assert L.mi355x_rownorm_set_override(cabi.OP_SOFTMAX_FWD, -2, 0, 0, 0) == -5
+    assert L.mi355x_rownorm_set_override(99, 0, 0, 0, 0) == -2
+    # a forced variant round-trips through the packed word, the multi-pass marker (-1) included
+    cabi.set_override(cabi.OP_LAYER_NORM_FWD, -1, 5)
+    p = cabi.plan(cabi.OP_LAYER_NORM_FWD, 4, 300000, cabi.F32, cabi.F32)
+    assert p["resident"] == 0 and p["row_chunks"] == 5, p
+    cabi.set_override(cabi.OP_LAYER_NORM_FWD, 512, 4, 512, 3)
+    p = cabi.plan(cabi.OP_LAYER_NORM_FWD, 16384, 16384, cabi.BF16, cabi.BF16)
+    assert (p["lanes_per_row"], p["packs_per_lane"], p["block_threads"]) == (512, 4, 512), p
+    assert p["grid_blocks"] == 3 * 256
+    cabi.clear_overrides()
+
+
 def test_plan_picks_resident_kernels_for_the_llama_shapes(cabi):
     for op, M, N, dt in ((cabi.OP_LAYER_NORM_FWD, 4096, 1024, cabi.F32),
                          (cabi.OP_RMS_NORM_FWD, 16384, 4096, cabi.BF16),

@@ -28,6 +28,12 @@ def test_short_rows_match_the_oracle(cabi, oracle, gpu, dtype, offset):
         pb = cabi.plan(cabi.OP_LAYER_NORM_BWD, M, N, code, code)
         if packs <= 64:
             assert pb["packs_per_lane"] == 1 and pb["lanes_per_row"] >= packs, pb
+            # the forward looks at its pointers: off a 128-byte line it takes the same layout,
+            # and the plan query reports that when told so
+            off_line = (offset * (16 // E)) % 128 != 0
+            pf = cabi.plan(cabi.OP_LAYER_NORM_FWD, M, N, code, code, off_line=off_line)
+            assert (pf["packs_per_lane"] == 1 and pf["lanes_per_row"] >= packs) == (
+                off_line or packs <= 8), (offset, pf)
         g = gen(900 + N)
         x = (0.5 + torch.randn(M, N, generator=g)).to(dtype)
         x[3] = 1.5  # a constant row

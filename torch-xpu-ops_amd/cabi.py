@@ -26,7 +26,7 @@ EXPORTED_SYMBOLS = (
     "mi355x_masked_softmax_bwd", "mi355x_softmax_strided_fwd", "mi355x_softmax_strided_bwd",
     "mi355x_softmax_strided_plan", "mi355x_group_norm_fwd",
     "mi355x_group_norm_bwd_workspace_bytes", "mi355x_group_norm_bwd", "mi355x_group_norm_plan",
-    "mi355x_rownorm_plan", "mi355x_rownorm_set_override",
+    "mi355x_rownorm_plan", "mi355x_rownorm_plan_at", "mi355x_rownorm_set_override",
 )
 
 
@@ -92,6 +92,8 @@ def lib():
         L.mi355x_group_norm_plan.argtypes = [_int, _i64, _i64, _i64, _i64, _int,
                                              ctypes.POINTER(Plan)]
         L.mi355x_rownorm_plan.argtypes = [_int, _i64, _i64, _int, _int, ctypes.POINTER(Plan)]
+        L.mi355x_rownorm_plan_at.argtypes = [_int, _i64, _i64, _int, _int, _int,
+                                             ctypes.POINTER(Plan)]
         L.mi355x_rownorm_set_override.argtypes = [_int, _int, _int, _int, _int]
         for name in ("mi355x_layer_norm_fwd", "mi355x_rms_norm_fwd", "mi355x_layer_norm_bwd",
                      "mi355x_rms_norm_bwd", "mi355x_rms_norm_bwd_static", "mi355x_softmax_fwd",
@@ -100,7 +102,8 @@ def lib():
                      "mi355x_masked_softmax_bwd", "mi355x_softmax_strided_fwd",
                      "mi355x_softmax_strided_bwd", "mi355x_softmax_strided_plan",
                      "mi355x_group_norm_fwd", "mi355x_group_norm_bwd", "mi355x_group_norm_plan",
-                     "mi355x_rownorm_plan", "mi355x_rownorm_set_override"):
+                     "mi355x_rownorm_plan", "mi355x_rownorm_plan_at",
+                     "mi355x_rownorm_set_override"):
             getattr(L, name).restype = _int
         _lib = L
     return _lib
@@ -123,9 +126,11 @@ def dtype_code(dt):
         raise RuntimeError("dtype %s is not implemented by the MI355X kernels" % dt)
 
 
-def plan(op, M, N, x_dtype=F32, w_dtype=F32):
+def plan(op, M, N, x_dtype=F32, w_dtype=F32, off_line=False):
+    """The launch layout of a call; off_line: its tensors do not all start on a 128-byte line."""
     p = Plan()
-    _check(lib().mi355x_rownorm_plan(op, M, N, x_dtype, w_dtype, ctypes.byref(p)), "plan")
+    _check(lib().mi355x_rownorm_plan_at(op, M, N, x_dtype, w_dtype, int(off_line),
+                                        ctypes.byref(p)), "plan")
     d = p.as_dict()
     d["row_chunks"] = p.reserved  # workgroups a row is split over (0: not split)
     return d

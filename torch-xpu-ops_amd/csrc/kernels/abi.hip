@@ -85,8 +85,28 @@ int current_num_cus() {
   return v;
 }
 
-// Forced variants for tests and tuning (process-global, see the header).
-Override g_override[ROWNORM_OP_COUNT];
+// Forced variants for tests and tuning (process-global, see the header).  One
+// 64-bit atomic per op holds the four fields, so a call that runs while another
+// thread sets an override sees the old or the new variant, never a mix.
+std::atomic<uint64_t> g_override_bits[ROWNORM_OP_COUNT];
+
+uint64_t pack_override(const Override& o) {
+  return (uint64_t)(uint16_t)(int16_t)o.G | ((uint64_t)(uint16_t)o.V << 16) |
+         ((uint64_t)(uint16_t)o.block << 32) | ((uint64_t)(uint16_t)o.bpc << 48);
+}
+
+struct OverrideTable {
+  Override operator[](int op) const {
+    const uint64_t b = g_override_bits[op].load(std::memory_order_relaxed);
+    Override o;
+    o.G = (int16_t)(uint16_t)(b & 0xffff);
+    o.V = (int)((b >> 16) & 0xffff);
+    o.block = (int)((b >> 32) & 0xffff);
+    o.bpc = (int)((b >> 48) & 0xffff);
+    return o;
+  }
+};
+const OverrideTable g_override;
 
 // Device-resident scratch of mi355x_rms_norm_bwd_static: the fp32 partial rows of
 // the dgamma reduction (and the split-row partial sums behind them) for callers
@@ -627,8 +647,8 @@ int mi355x_softmax_strided_plan(int backward, int64_t outer, int64_t dim_size, i
   return 0;
 }
 
-int mi355x_rownorm_plan(rownorm_op op, int64_t M, int64_t N, rownorm_dtype x_dtype,
-                        rownorm_dtype w_dtype, rownorm_plan* out) {
+int mi355x_rownorm_plan_at(rownorm_op op, int64_t M, int64_t N, rownorm_dtype x_dtype,
+                           rownorm_dtype w_dtype, int off_line, rownorm_plan* out) {
   if ((int)op < 0 || (int)op > ROWNORM_OP_SOFTMAX_BWD) return ROWNORM_ERR_SHAPE;
   if (!out) return ROWNORM_ERR_NULL;
   if (esize_of((int)x_dtype) == 0) return ROWNORM_ERR_DTYPE;
@@ -636,9 +656,11 @@ int mi355x_rownorm_plan(rownorm_op op, int64_t M, int64_t N, rownorm_dtype x_dty
   Plan plan;
   const OpClass oc = class_of((int)op);
   const bool layer_norm = op == ROWNORM_OP_LAYER_NORM_FWD || op == ROWNORM_OP_LAYER_NORM_BWD;
+  // the norm backward does not look at its pointers
+  const bool off = off_line != 0 && oc != OC_NORM_BWD;
   if (int e = make_plan(oc, M, N, esize_of((int)x_dtype), current_num_cus(), g_override[(int)op],
                         oc == OC_NORM_BWD, &plan, false, layer_norm,
-                        esize_of((int)w_dtype) > esize_of((int)x_dtype)))
+                        esize_of((int)w_dtype) > esize_of((int)x_dtype), off))
     return e;
   out->resident = plan.resident ? 1 : 0;
   out->lanes_per_row = plan.G;
@@ -651,15 +673,24 @@ int mi355x_rownorm_plan(rownorm_op op, int64_t M, int64_t N, rownorm_dtype x_dty
   return 0;
 }
 
+int mi355x_rownorm_plan(rownorm_op op, int64_t M, int64_t N, rownorm_dtype x_dtype,
+                        rownorm_dtype w_dtype, rownorm_plan* out) {
+  return mi355x_rownorm_plan_at(op, M, N, x_dtype, w_dtype, 0, out);
+}
+
 int mi355x_rownorm_set_override(rownorm_op op, int lanes_per_row, int packs_per_lane,
                                 int block_threads, int blocks_per_cu) {
   if ((int)op < 0 || (int)op >= ROWNORM_OP_COUNT) return ROWNORM_ERR_SHAPE;
+  if (lanes_per_row < -1 || lanes_per_row > 0x7fff || packs_per_lane < 0 ||
+      packs_per_lane > 0xffff || block_threads < 0 || block_threads > 0xffff ||
+      blocks_per_cu < 0 || blocks_per_cu > 0xffff)
+    return ROWNORM_ERR_OVERRIDE;
   Override o;
   o.G = lanes_per_row;
   o.V = packs_per_lane;
   o.block = block_threads;
   o.bpc = blocks_per_cu;
-  g_override[(int)op] = o;
+  g_override_bits[(int)op].store(pack_override(o), std::memory_order_relaxed);
   return 0;
 }
 
