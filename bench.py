@@ -347,6 +347,43 @@ def per_op_table(torch, cabi, L, dev, stream, P, only=None, iters=60, warm=30):
             s[1], s[0], [N], r, w, [True, True])) for s, r in zip(sets, r2)])
     del sets
 
+    # the residual add fused into the norm (h = x + res written once, y = norm(h)), same shape:
+    # 4 tensors move instead of the 5 of an add followed by the norm; and the output cast fused
+    # into a float32 norm (y written as bf16)
+    sets = []
+    for _ in range(3):
+        x = torch.randn(M, N, device=dev).bfloat16()
+        sets.append((x, torch.randn(M, N, device=dev).bfloat16(), torch.empty_like(x),
+                     torch.empty_like(x), torch.empty(M, device=dev),
+                     torch.randn(M, N, device=dev).bfloat16(), torch.randn(M, N, device=dev).bfloat16(),
+                     torch.empty_like(x), torch.empty_like(w)))
+    add("add + _fused_rms_norm fwd bf16 [16384,4096] (h and y written)",
+        4 * M * N * 2 + N * 2 + M * 4,
+        [(lambda s=s: L.mi355x_add_rms_norm_fwd(P(s[0]), P(s[1]), P(w), P(s[2]), P(s[3]), P(s[4]), M,
+                                                N, 1e-6, BF, BF, BF, stream)) for s in sets],
+        stock=[(lambda s=s: torch.ops.aten._fused_rms_norm(s[0] + s[1], [N], w, 1e-6))
+               for s in sets], stock_note="stock: an elementwise add, then aten::_fused_rms_norm")
+    for s in sets:
+        L.mi355x_add_rms_norm_fwd(P(s[0]), P(s[1]), P(w), P(s[2]), P(s[3]), P(s[4]), M, N, 1e-6, BF,
+                                  BF, BF, stream)
+    add("add + _fused_rms_norm bwd bf16 [16384,4096] (dh = norm bwd + residual grad)",
+        4 * M * N * 2 + M * 4 + 2 * N * 2,
+        [(lambda s=s: L.mi355x_add_rms_norm_bwd(P(s[5]), P(s[6]), P(s[2]), P(s[4]), P(w), P(s[7]),
+                                                P(s[8]), P(ws), nws, M, N, BF, BF, stream))
+         for s in sets])
+    del sets
+    x32 = [torch.randn(M, N, device=dev) for _ in range(3)]
+    w32 = 1 + 0.02 * torch.randn(N, device=dev)
+    y16 = torch.empty(M, N, device=dev, dtype=torch.bfloat16)
+    r32 = torch.empty(M, device=dev)
+    add("_fused_rms_norm fwd fp32 rows -> bf16 y [16384,4096] (cast fused)",
+        M * N * 4 + M * N * 2 + N * 4 + M * 4,
+        [(lambda x=x: L.mi355x_add_rms_norm_fwd(P(x), None, P(w32), None, P(y16), P(r32), M, N, 1e-6,
+                                                F32, F32, BF, stream)) for x in x32],
+        stock=[(lambda x=x: torch.ops.aten._fused_rms_norm(x, [N], w32, 1e-6)[0].bfloat16())
+               for x in x32], stock_note="stock: aten::_fused_rms_norm in float32, then a cast")
+    del x32, y16
+
     # C4: native_layer_norm bf16 rows, fp32 gamma/beta [16384, 8192]
     M, N = 16384, 8192
     g = 1 + 0.1 * torch.randn(N, device=dev)

@@ -146,6 +146,47 @@ int mi355x_rms_norm_bwd(const void* dy, const void* x, const float* rstd, const 
                         int64_t M, int64_t N, rownorm_dtype x_dtype, rownorm_dtype w_dtype,
                         void* stream);
 
+/* Fused residual add -> norm (-> output cast), forward.  The step that precedes
+ * the norm in a transformer block, h = x + residual, is formed in float32,
+ * rounded once to x_dtype -- exactly what an elementwise add of the two tensors
+ * gives -- written to `h` and normalized in the same pass: one read of x, one of
+ * residual, one write of h and one of y, where an add followed by the norm reads
+ * three tensors and writes two.  The reference has no such operator (its
+ * forward, VectorizedLayerNormKernelFunctor in LayerNormKernels.cpp:469-586,
+ * starts from the summed row); results equal the reference's norm applied to
+ * that sum.  x, residual and h share x_dtype and the shape [M, N]; h may be the
+ * memory of x or of residual (the usual in-place update of the residual
+ * stream), y may not overlap them.  residual == NULL: no add, h is not touched
+ * (may be NULL): the plain norm with the output cast.
+ * y_dtype: x_dtype, or ROWNORM_F16 / ROWNORM_BF16 for float32 rows (a float32
+ * residual stream feeding a 16-bit matrix multiply): y is rounded once, from
+ * the float32 result.  Other arguments as mi355x_layer_norm_fwd /
+ * mi355x_rms_norm_fwd. */
+int mi355x_add_layer_norm_fwd(const void* x, const void* residual, const void* gamma,
+                              const void* beta, void* h, void* y, float* mean, float* rstd,
+                              int64_t M, int64_t N, float eps, rownorm_dtype x_dtype,
+                              rownorm_dtype w_dtype, rownorm_dtype y_dtype, void* stream);
+int mi355x_add_rms_norm_fwd(const void* x, const void* residual, const void* gamma, void* h,
+                            void* y, float* rstd, int64_t M, int64_t N, float eps,
+                            rownorm_dtype x_dtype, rownorm_dtype w_dtype, rownorm_dtype y_dtype,
+                            void* stream);
+
+/* Backward of the fused add -> norm.  h is the saved sum (the row that was
+ * normalized), dy the gradient of y (x_dtype: the backward has no cast), dh_in
+ * the gradient that reaches h by the residual path (NULL: none).  dh = the norm's
+ * input gradient + dh_in, added in float32 and rounded once; it is the gradient
+ * of both x and residual.  dh may be the memory of dh_in.  Workspace as for
+ * mi355x_layer_norm_bwd / mi355x_rms_norm_bwd (same *_workspace_bytes). */
+int mi355x_add_layer_norm_bwd(const void* dy, const void* dh_in, const void* h, const float* mean,
+                              const float* rstd, const void* gamma, void* dh, void* dgamma,
+                              void* dbeta, void* workspace, size_t workspace_bytes, int64_t M,
+                              int64_t N, rownorm_dtype x_dtype, rownorm_dtype w_dtype,
+                              void* stream);
+int mi355x_add_rms_norm_bwd(const void* dy, const void* dh_in, const void* h, const float* rstd,
+                            const void* gamma, void* dh, void* dgamma, void* workspace,
+                            size_t workspace_bytes, int64_t M, int64_t N, rownorm_dtype x_dtype,
+                            rownorm_dtype w_dtype, void* stream);
+
 /* mi355x_rms_norm_bwd for callers that cannot allocate device memory: code
  * under HIP graph capture, tight serving loops, harnesses that forbid
  * hipMalloc.  It has no counterpart in the reference, whose entry point

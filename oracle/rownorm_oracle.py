@@ -157,6 +157,64 @@ def rms_norm_bwd(dy, x, normalized_shape, rstd, gamma=None, mask=(True, True)):
     return dx, None if dg is None else dg.reshape(tuple(normalized_shape))
 
 
+def round_to(a, dtype):
+    """float32 values rounded to the storage format `dtype` ("f32", "f16" or "bf16") with round to
+    nearest even, returned as float32: what a store of the accumulate type into a tensor of that
+    dtype does.  bfloat16 keeps the top 16 bits of the float32 pattern; NaN stays NaN."""
+    a = np.ascontiguousarray(a, dtype=np.float32)
+    if dtype == "f32":
+        return a.copy()
+    if dtype == "f16":
+        with np.errstate(over="ignore"):
+            return a.astype(np.float16).astype(np.float32)
+    if dtype != "bf16":
+        raise ValueError("dtype must be f32, f16 or bf16, got %r" % (dtype,))
+    bits = a.view(np.uint32).astype(np.uint64)
+    rounded = ((bits + 0x7FFF + ((bits >> 16) & 1)) & 0xFFFF0000).astype(np.uint32)
+    out = rounded.view(np.float32).copy()
+    out[np.isnan(a)] = np.nan
+    return out
+
+
+def residual_sum(x, residual, dtype):
+    """h = x + residual as the fused add -> norm operators form it: the float32 sum of the two
+    rows rounded once to the row dtype (an elementwise add of two tensors of that dtype)."""
+    return round_to(_c(x) + _c(residual), dtype)
+
+
+def add_layer_norm_fwd(x, residual, normalized_shape, gamma=None, beta=None, eps=1e-5, dtype="f32"):
+    """Fused residual add -> LayerNorm: the pinned layer_norm_fwd applied to residual_sum().
+    -> (y, h, mean, rstd).  The reference has no fused operator; its forward starts from the
+    summed row (VectorizedLayerNormKernelFunctor, LayerNormKernels.cpp:469-586)."""
+    h = residual_sum(x, residual, dtype)
+    y, mean, rstd = layer_norm_fwd(h, normalized_shape, gamma, beta, eps)
+    return y, h, mean, rstd
+
+
+def add_rms_norm_fwd(x, residual, normalized_shape, gamma=None, eps=None, dtype="f32"):
+    """Fused residual add -> RMSNorm -> (y, h, rstd)."""
+    h = residual_sum(x, residual, dtype)
+    y, rstd = rms_norm_fwd(h, normalized_shape, gamma, eps)
+    return y, h, rstd
+
+
+def add_layer_norm_bwd(dy, dh_in, h, normalized_shape, mean, rstd, gamma=None,
+                       mask=(True, True, True)):
+    """Backward of the fused add -> LayerNorm: the norm's input gradient plus the gradient that
+    reaches h by the residual path (None: none), summed in float64.  -> (dh, dgamma, dbeta)."""
+    dx, dg, db = layer_norm_bwd(dy, h, normalized_shape, mean, rstd, gamma, mask)
+    if dx is not None and dh_in is not None:
+        dx = (dx.astype(np.float64) + _c(dh_in).astype(np.float64)).astype(np.float32)
+    return dx, dg, db
+
+
+def add_rms_norm_bwd(dy, dh_in, h, normalized_shape, rstd, gamma=None, mask=(True, True)):
+    dx, dg = rms_norm_bwd(dy, h, normalized_shape, rstd, gamma, mask)
+    if dx is not None and dh_in is not None:
+        dx = (dx.astype(np.float64) + _c(dh_in).astype(np.float64)).astype(np.float32)
+    return dx, dg
+
+
 def softmax_fwd(x, is_log=False):
     """_softmax / _log_softmax over the last dimension."""
     x = _c(x)

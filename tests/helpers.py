@@ -135,3 +135,26 @@ def rowsum_slack(terms, weight):
     w = torch.as_tensor(weight).to(torch.float64).abs()
     w = torch.where(torch.isfinite(w), w, torch.zeros_like(w))
     return w * (16.0 * EPS32 * t.pow(2).sum(-1, keepdim=True).sqrt())
+
+
+def assert_same_arithmetic(a, b, what, max_fraction=1e-3):
+    """Two kernel instances that evaluate the same formulas on the same values: the results are
+    equal except where the compiler contracted a multiply-add in one instance and not in the other,
+    which moves a result by at most one unit in the last place of its dtype.  Asserts that every
+    element is equal or adjacent and that at most `max_fraction` of them (or two) differ; NaN / inf
+    positions must agree."""
+    assert a.dtype == b.dtype and a.shape == b.shape, (what, a.dtype, b.dtype, a.shape, b.shape)
+    if torch.equal(a, b):
+        return
+    af, bf = a.detach().double().cpu().reshape(-1), b.detach().double().cpu().reshape(-1)
+    fin = torch.isfinite(af) & torch.isfinite(bf)
+    assert torch.equal(torch.isnan(af), torch.isnan(bf)) and torch.equal(af[~fin & ~torch.isnan(af)],
+                                                                         bf[~fin & ~torch.isnan(bf)]), what
+    d = (af[fin] - bf[fin]).abs()
+    ulp = torch.finfo(a.dtype).eps * torch.maximum(af[fin].abs(), bf[fin].abs()).clamp_min(
+        torch.finfo(a.dtype).tiny)
+    assert bool((d <= ulp).all()), "%s: results more than one ulp apart (max %.3g ulp)" % (
+        what, float((d / ulp).max()))
+    ndiff = int((d > 0).sum())
+    assert ndiff <= max(2, max_fraction * d.numel()), "%s: %d of %d elements differ" % (
+        what, ndiff, d.numel())

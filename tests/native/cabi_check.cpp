@@ -33,6 +33,10 @@ DECL(mi355x_rms_norm_bwd_workspace_bytes);
 DECL(mi355x_rms_norm_bwd);
 DECL(mi355x_rms_norm_bwd_static_limit_bytes);
 DECL(mi355x_rms_norm_bwd_static);
+DECL(mi355x_add_layer_norm_fwd);
+DECL(mi355x_add_rms_norm_fwd);
+DECL(mi355x_add_layer_norm_bwd);
+DECL(mi355x_add_rms_norm_bwd);
 DECL(mi355x_softmax_fwd);
 DECL(mi355x_softmax_bwd);
 DECL(mi355x_safe_softmax_fwd);
@@ -79,6 +83,10 @@ static bool load_all(void* lib) {
   LOAD(mi355x_rms_norm_bwd);
   LOAD(mi355x_rms_norm_bwd_static_limit_bytes);
   LOAD(mi355x_rms_norm_bwd_static);
+  LOAD(mi355x_add_layer_norm_fwd);
+  LOAD(mi355x_add_rms_norm_fwd);
+  LOAD(mi355x_add_layer_norm_bwd);
+  LOAD(mi355x_add_rms_norm_bwd);
   LOAD(mi355x_softmax_fwd);
   LOAD(mi355x_softmax_bwd);
   LOAD(mi355x_safe_softmax_fwd);

@@ -162,7 +162,7 @@ def test_config4_layer_norm_fwd_bwd_bf16_fp32_weights(cabi, oracle, gpu):
 
 
 STRESS = [(1 << 20, 64), (8192, 127), (8192, 4097), (8192, 5120), (8192, 16384)]
-ORACLE_ROWS = 192  # rows checked against the float64 oracle (row 0 is the constant row)
+ORACLE_ROWS = None  # every row is checked against the float64 oracle (row 0 is the constant row)
 
 
 @pytest.mark.parametrize("dtype", [torch.float32, torch.float16], ids=str)

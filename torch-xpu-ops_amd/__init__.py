@@ -9,6 +9,8 @@ Two layers are exposed:
   * ``ops``   -- ``torch.ops.mi355x.*``: the C++ host layer with the ATen operator signatures
                  (native_layer_norm, native_layer_norm_backward, _fused_rms_norm,
                  _fused_rms_norm_backward, _softmax, _log_softmax and their backward ops).
+  * ``fused`` -- ``add_rms_norm`` / ``add_layer_norm``: the residual add fused into the norm, with
+                 autograd (``torch.ops.mi355x.add_rms_norm`` & co. underneath).
   * ``cabi``  -- ctypes bindings of the ``extern "C"`` launcher ABI (include/mi355x_rownorm.h),
                  taking torch tensors only as device memory.
 There is no CPU path and no fallback: if the compiled libraries are missing the import raises.
@@ -51,6 +53,7 @@ class _LazyOps(object):
 ops = _LazyOps()
 
 from . import cabi  # noqa: E402  (ctypes layer; loads the kernel library on first use)
+from . import fused  # noqa: E402  (fused residual add -> norm with autograd)
 
 
 def override_aten_ops():

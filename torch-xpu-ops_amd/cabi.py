@@ -21,7 +21,9 @@ EXPORTED_SYMBOLS = (
     "mi355x_rownorm_error_string", "mi355x_rownorm_abi_version", "mi355x_layer_norm_fwd",
     "mi355x_layer_norm_bwd_workspace_bytes", "mi355x_layer_norm_bwd", "mi355x_rms_norm_fwd",
     "mi355x_rms_norm_bwd_workspace_bytes", "mi355x_rms_norm_bwd",
-    "mi355x_rms_norm_bwd_static_limit_bytes", "mi355x_rms_norm_bwd_static", "mi355x_softmax_fwd",
+    "mi355x_rms_norm_bwd_static_limit_bytes", "mi355x_rms_norm_bwd_static",
+    "mi355x_add_layer_norm_fwd", "mi355x_add_rms_norm_fwd", "mi355x_add_layer_norm_bwd",
+    "mi355x_add_rms_norm_bwd", "mi355x_softmax_fwd",
     "mi355x_softmax_bwd", "mi355x_safe_softmax_fwd", "mi355x_masked_softmax_fwd",
     "mi355x_masked_softmax_bwd", "mi355x_softmax_strided_fwd", "mi355x_softmax_strided_bwd",
     "mi355x_softmax_strided_plan", "mi355x_group_norm_fwd",
@@ -69,6 +71,14 @@ def lib():
         L.mi355x_rms_norm_bwd_static_limit_bytes.argtypes = []
         L.mi355x_rms_norm_bwd_static.argtypes = [_vp, _vp, _vp, _vp, _vp, _vp, _i64, _i64, _int,
                                                  _int, _vp]
+        L.mi355x_add_layer_norm_fwd.argtypes = [_vp, _vp, _vp, _vp, _vp, _vp, _vp, _vp, _i64, _i64,
+                                                _f, _int, _int, _int, _vp]
+        L.mi355x_add_rms_norm_fwd.argtypes = [_vp, _vp, _vp, _vp, _vp, _vp, _i64, _i64, _f, _int,
+                                              _int, _int, _vp]
+        L.mi355x_add_layer_norm_bwd.argtypes = [_vp, _vp, _vp, _vp, _vp, _vp, _vp, _vp, _vp, _vp,
+                                                ctypes.c_size_t, _i64, _i64, _int, _int, _vp]
+        L.mi355x_add_rms_norm_bwd.argtypes = [_vp, _vp, _vp, _vp, _vp, _vp, _vp, _vp,
+                                              ctypes.c_size_t, _i64, _i64, _int, _int, _vp]
         L.mi355x_softmax_fwd.argtypes = [_vp, _vp, _i64, _i64, _int, _int, _int, _vp]
         L.mi355x_softmax_bwd.argtypes = [_vp, _vp, _vp, _i64, _i64, _int, _int, _int, _vp]
         L.mi355x_safe_softmax_fwd.argtypes = [_vp, _vp, _i64, _i64, _int, _int, _vp]
@@ -96,7 +106,9 @@ def lib():
                                              ctypes.POINTER(Plan)]
         L.mi355x_rownorm_set_override.argtypes = [_int, _int, _int, _int, _int]
         for name in ("mi355x_layer_norm_fwd", "mi355x_rms_norm_fwd", "mi355x_layer_norm_bwd",
-                     "mi355x_rms_norm_bwd", "mi355x_rms_norm_bwd_static", "mi355x_softmax_fwd",
+                     "mi355x_rms_norm_bwd", "mi355x_rms_norm_bwd_static",
+                     "mi355x_add_layer_norm_fwd", "mi355x_add_rms_norm_fwd",
+                     "mi355x_add_layer_norm_bwd", "mi355x_add_rms_norm_bwd", "mi355x_softmax_fwd",
                      "mi355x_softmax_bwd",
                      "mi355x_safe_softmax_fwd", "mi355x_masked_softmax_fwd",
                      "mi355x_masked_softmax_bwd", "mi355x_softmax_strided_fwd",
@@ -277,6 +289,90 @@ def rms_norm_bwd_static(dy, x, rstd, gamma, dx, dgamma, n_norm_dims=1, w_dtype=N
                                             _ptr(dgamma), M, N, dtype_code(x.dtype),
                                             dtype_code(wdt), _stream()), "rms_norm_bwd_static")
     return dx, dgamma
+
+
+def add_layer_norm_fwd(x, residual, gamma, beta, eps, n_norm_dims=1, y_dtype=None, h=None, y=None,
+                       mean=None, rstd=None):
+    """Fused residual add -> LayerNorm (-> cast): -> (y, h, mean[M], rstd[M]) with h = x + residual
+    (pass h=residual to update the residual stream in place).  residual=None: the plain norm with
+    the output cast (h comes back None)."""
+    import torch
+    _gpu(x, residual, gamma, beta, h, y)
+    M, N = _rows(x, n_norm_dims)
+    if residual is not None and h is None:
+        h = torch.empty_like(x)
+    y = torch.empty(x.shape, dtype=y_dtype or x.dtype, device=x.device) if y is None else y
+    mean = torch.empty(M, dtype=torch.float32, device=x.device) if mean is None else mean
+    rstd = torch.empty(M, dtype=torch.float32, device=x.device) if rstd is None else rstd
+    _check(lib().mi355x_add_layer_norm_fwd(_ptr(x), _ptr(residual), _ptr(gamma), _ptr(beta),
+                                           _ptr(h), _ptr(y), _ptr(mean), _ptr(rstd), M, N, eps,
+                                           dtype_code(x.dtype), _wd(x, gamma, beta),
+                                           dtype_code(y.dtype), _stream()), "add_layer_norm_fwd")
+    return y, h, mean, rstd
+
+
+def add_rms_norm_fwd(x, residual, gamma, eps, n_norm_dims=1, y_dtype=None, h=None, y=None,
+                     rstd=None):
+    """Fused residual add -> RMSNorm (-> cast): -> (y, h, rstd[M])."""
+    import torch
+    _gpu(x, residual, gamma, h, y)
+    M, N = _rows(x, n_norm_dims)
+    if residual is not None and h is None:
+        h = torch.empty_like(x)
+    y = torch.empty(x.shape, dtype=y_dtype or x.dtype, device=x.device) if y is None else y
+    rstd = torch.empty(M, dtype=torch.float32, device=x.device) if rstd is None else rstd
+    _check(lib().mi355x_add_rms_norm_fwd(_ptr(x), _ptr(residual), _ptr(gamma), _ptr(h), _ptr(y),
+                                         _ptr(rstd), M, N, eps, dtype_code(x.dtype), _wd(x, gamma),
+                                         dtype_code(y.dtype), _stream()), "add_rms_norm_fwd")
+    return y, h, rstd
+
+
+def add_layer_norm_bwd(dy, dh_in, h, mean, rstd, gamma, n_norm_dims=1, want=(True, True, True),
+                       w_dtype=None, dh=None, dgamma=None, dbeta=None, workspace=None):
+    """Backward of the fused add -> LayerNorm: -> (dh, dgamma, dbeta); dh = the norm's input
+    gradient + dh_in (None: nothing to add) is the gradient of both x and residual."""
+    import torch
+    _gpu(dy, dh_in, h, mean, rstd, gamma)
+    M, N = _rows(h, n_norm_dims)
+    wdt = w_dtype if w_dtype is not None else (gamma.dtype if gamma is not None else h.dtype)
+    if want[0] and dh is None:
+        dh = torch.empty_like(h)
+    if want[1] and dgamma is None:
+        dgamma = torch.empty(N, dtype=wdt, device=h.device)
+    if want[2] and dbeta is None:
+        dbeta = torch.empty(N, dtype=wdt, device=h.device)
+    xd, wd = dtype_code(h.dtype), dtype_code(wdt)
+    nbytes = lib().mi355x_layer_norm_bwd_workspace_bytes(M, N, xd, wd, int(dgamma is not None),
+                                                         int(dbeta is not None))
+    if workspace is None and nbytes:
+        workspace = torch.empty(nbytes, dtype=torch.uint8, device=h.device)
+    _check(lib().mi355x_add_layer_norm_bwd(_ptr(dy), _ptr(dh_in), _ptr(h), _ptr(mean), _ptr(rstd),
+                                           _ptr(gamma), _ptr(dh), _ptr(dgamma), _ptr(dbeta),
+                                           _ptr(workspace),
+                                           0 if workspace is None else workspace.numel(), M, N, xd,
+                                           wd, _stream()), "add_layer_norm_bwd")
+    return dh, dgamma, dbeta
+
+
+def add_rms_norm_bwd(dy, dh_in, h, rstd, gamma, n_norm_dims=1, want=(True, True), w_dtype=None,
+                     dh=None, dgamma=None, workspace=None):
+    import torch
+    _gpu(dy, dh_in, h, rstd, gamma)
+    M, N = _rows(h, n_norm_dims)
+    wdt = w_dtype if w_dtype is not None else (gamma.dtype if gamma is not None else h.dtype)
+    if want[0] and dh is None:
+        dh = torch.empty_like(h)
+    if want[1] and dgamma is None:
+        dgamma = torch.empty(N, dtype=wdt, device=h.device)
+    xd, wd = dtype_code(h.dtype), dtype_code(wdt)
+    nbytes = lib().mi355x_rms_norm_bwd_workspace_bytes(M, N, xd, wd, int(dgamma is not None))
+    if workspace is None and nbytes:
+        workspace = torch.empty(nbytes, dtype=torch.uint8, device=h.device)
+    _check(lib().mi355x_add_rms_norm_bwd(_ptr(dy), _ptr(dh_in), _ptr(h), _ptr(rstd), _ptr(gamma),
+                                         _ptr(dh), _ptr(dgamma), _ptr(workspace),
+                                         0 if workspace is None else workspace.numel(), M, N, xd, wd,
+                                         _stream()), "add_rms_norm_bwd")
+    return dh, dgamma
 
 
 def softmax_fwd(x, is_log=False, out_dtype=None, y=None):

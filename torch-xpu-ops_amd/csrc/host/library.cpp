@@ -8,6 +8,7 @@
 // opt-in done from Python.
 #include <torch/library.h>
 
+#include "fused_ops.h"
 #include "group_norm_ops.h"
 #include "norm_ops.h"
 #include "softmax_ops.h"
@@ -73,6 +74,32 @@ TORCH_LIBRARY(mi355x, m) {
       "Tensor? weight, int N, int C, int HxW, int group, bool[3] output_mask) -> "
       "(Tensor, Tensor, Tensor)",
       &mi355x::native_group_norm_backward);
+  // fused residual add -> norm (-> cast): new operator surface, not aten ops
+  m.def(
+      "add_layer_norm(Tensor input, Tensor residual, int[] normalized_shape, Tensor? weight, "
+      "Tensor? bias, float eps, ScalarType? out_dtype=None) -> (Tensor, Tensor, Tensor, Tensor)",
+      &mi355x::add_layer_norm);
+  m.def(
+      "add_layer_norm_(Tensor input, Tensor(a!) residual, int[] normalized_shape, Tensor? weight, "
+      "Tensor? bias, float eps, ScalarType? out_dtype=None) -> (Tensor, Tensor, Tensor)",
+      &mi355x::add_layer_norm_);
+  m.def(
+      "add_layer_norm_backward(Tensor grad_y, Tensor? grad_h, Tensor h, int[] normalized_shape, "
+      "Tensor mean, Tensor rstd, Tensor? weight, Tensor? bias, bool[3] output_mask) -> "
+      "(Tensor, Tensor, Tensor)",
+      &mi355x::add_layer_norm_backward);
+  m.def(
+      "add_rms_norm(Tensor input, Tensor residual, int[] normalized_shape, Tensor? weight, "
+      "float? eps, ScalarType? out_dtype=None) -> (Tensor, Tensor, Tensor)",
+      &mi355x::add_rms_norm);
+  m.def(
+      "add_rms_norm_(Tensor input, Tensor(a!) residual, int[] normalized_shape, Tensor? weight, "
+      "float? eps, ScalarType? out_dtype=None) -> (Tensor, Tensor)",
+      &mi355x::add_rms_norm_);
+  m.def(
+      "add_rms_norm_backward(Tensor grad_y, Tensor? grad_h, Tensor h, int[] normalized_shape, "
+      "Tensor rstd, Tensor? weight, bool[2] output_mask) -> (Tensor, Tensor)",
+      &mi355x::add_rms_norm_backward);
   m.def("install_group_norm_dispatch_stubs() -> ()", &mi355x::install_group_norm_dispatch_stubs);
   m.def("install_layer_norm_dispatch_stubs() -> ()", &mi355x::install_layer_norm_dispatch_stubs);
   m.def("uninstall_group_norm_dispatch_stubs() -> ()",

@@ -28,6 +28,34 @@ extern template int launch_norm_bwd<bf16, bf16, false>(const Plan&, const NormBw
 extern template int launch_norm_bwd<bf16, bf16, true>(const Plan&, const NormBwdArgs&, hipStream_t);
 extern template int launch_norm_bwd<bf16, float, false>(const Plan&, const NormBwdArgs&, hipStream_t);
 extern template int launch_norm_bwd<bf16, float, true>(const Plan&, const NormBwdArgs&, hipStream_t);
+extern template int launch_norm_fwd<bf16, bf16, false, bf16, true>(const Plan&, const NormFwdArgs&, hipStream_t);
+extern template int launch_norm_bwd<bf16, bf16, false, true>(const Plan&, const NormBwdArgs&, hipStream_t);
+extern template int launch_norm_fwd<bf16, bf16, true, bf16, true>(const Plan&, const NormFwdArgs&, hipStream_t);
+extern template int launch_norm_bwd<bf16, bf16, true, true>(const Plan&, const NormBwdArgs&, hipStream_t);
+extern template int launch_norm_fwd<bf16, float, false, bf16, true>(const Plan&, const NormFwdArgs&, hipStream_t);
+extern template int launch_norm_bwd<bf16, float, false, true>(const Plan&, const NormBwdArgs&, hipStream_t);
+extern template int launch_norm_fwd<bf16, float, true, bf16, true>(const Plan&, const NormFwdArgs&, hipStream_t);
+extern template int launch_norm_bwd<bf16, float, true, true>(const Plan&, const NormBwdArgs&, hipStream_t);
+extern template int launch_norm_fwd<f16, f16, false, f16, true>(const Plan&, const NormFwdArgs&, hipStream_t);
+extern template int launch_norm_bwd<f16, f16, false, true>(const Plan&, const NormBwdArgs&, hipStream_t);
+extern template int launch_norm_fwd<f16, f16, true, f16, true>(const Plan&, const NormFwdArgs&, hipStream_t);
+extern template int launch_norm_bwd<f16, f16, true, true>(const Plan&, const NormBwdArgs&, hipStream_t);
+extern template int launch_norm_fwd<f16, float, false, f16, true>(const Plan&, const NormFwdArgs&, hipStream_t);
+extern template int launch_norm_bwd<f16, float, false, true>(const Plan&, const NormBwdArgs&, hipStream_t);
+extern template int launch_norm_fwd<f16, float, true, f16, true>(const Plan&, const NormFwdArgs&, hipStream_t);
+extern template int launch_norm_bwd<f16, float, true, true>(const Plan&, const NormBwdArgs&, hipStream_t);
+extern template int launch_norm_fwd<float, float, false, float, true>(const Plan&, const NormFwdArgs&, hipStream_t);
+extern template int launch_norm_bwd<float, float, false, true>(const Plan&, const NormBwdArgs&, hipStream_t);
+extern template int launch_norm_fwd<float, float, true, float, true>(const Plan&, const NormFwdArgs&, hipStream_t);
+extern template int launch_norm_bwd<float, float, true, true>(const Plan&, const NormBwdArgs&, hipStream_t);
+extern template int launch_norm_fwd<float, float, false, bf16, false>(const Plan&, const NormFwdArgs&, hipStream_t);
+extern template int launch_norm_fwd<float, float, true, bf16, false>(const Plan&, const NormFwdArgs&, hipStream_t);
+extern template int launch_norm_fwd<float, float, false, bf16, true>(const Plan&, const NormFwdArgs&, hipStream_t);
+extern template int launch_norm_fwd<float, float, true, bf16, true>(const Plan&, const NormFwdArgs&, hipStream_t);
+extern template int launch_norm_fwd<float, float, false, f16, false>(const Plan&, const NormFwdArgs&, hipStream_t);
+extern template int launch_norm_fwd<float, float, true, f16, false>(const Plan&, const NormFwdArgs&, hipStream_t);
+extern template int launch_norm_fwd<float, float, false, f16, true>(const Plan&, const NormFwdArgs&, hipStream_t);
+extern template int launch_norm_fwd<float, float, true, f16, true>(const Plan&, const NormFwdArgs&, hipStream_t);
 extern template int launch_softmax_fwd<float, float>(const Plan&, const SoftmaxFwdArgs&, hipStream_t);
 extern template int launch_softmax_fwd<f16, f16>(const Plan&, const SoftmaxFwdArgs&, hipStream_t);
 extern template int launch_softmax_fwd<bf16, bf16>(const Plan&, const SoftmaxFwdArgs&, hipStream_t);
@@ -167,27 +195,53 @@ int shape_check(int64_t M, int64_t N) {
   return 0;
 }
 
+// res / h: the fused residual add (both null: plain norm of x).  yd: dtype of y.
 template <bool RMS>
-int norm_fwd(const void* x, const void* gamma, const void* beta, void* y, float* mean,
-             float* rstd, int64_t M, int64_t N, float eps, int xd, int wd, void* stream) {
-  if (!norm_dtypes_ok(xd, wd)) return ROWNORM_ERR_DTYPE;
+int norm_fwd(const void* x, const void* res, const void* gamma, const void* beta, void* h,
+             void* y, float* mean, float* rstd, int64_t M, int64_t N, float eps, int xd, int wd,
+             int yd, void* stream) {
+  if (!norm_dtypes_ok(xd, wd) || esize_of(yd) == 0) return ROWNORM_ERR_DTYPE;
+  if (!(yd == xd || xd == ROWNORM_F32)) return ROWNORM_ERR_DTYPE;  // only float32 rows are cast
   if (int e = shape_check(M, N)) return e;
   if (M == 0 || N == 0) return 0;
-  if (!x || !y) return ROWNORM_ERR_NULL;
+  if (!x || !y || (res != nullptr && h == nullptr)) return ROWNORM_ERR_NULL;
+  const bool add = res != nullptr;
   Plan plan;
   const int op = RMS ? ROWNORM_OP_RMS_NORM_FWD : ROWNORM_OP_LAYER_NORM_FWD;
-  const bool off_line = (((uintptr_t)x | (uintptr_t)y) & 127u) != 0;
+  uintptr_t bits = (uintptr_t)x | (uintptr_t)y;
+  if (add) bits |= (uintptr_t)res | (uintptr_t)h;
+  const bool off_line = (bits & 127u) != 0;
   if (int e = make_plan(OC_NORM_FWD, M, N, esize_of(xd), current_num_cus(), g_override[op],
                         false, &plan, false, !RMS, esize_of(wd) > esize_of(xd), off_line))
     return e;
   NormFwdArgs a{x, gamma, RMS ? nullptr : beta, y, RMS ? nullptr : mean, rstd, M, (int)N, eps};
+  if (add) {
+    a.res = res;
+    a.h = h;
+  }
   hipStream_t s = (hipStream_t)stream;
-  if (xd == ROWNORM_F32) return launch_norm_fwd<float, float, RMS>(plan, a, s);
-  if (xd == ROWNORM_F16)
-    return wd == ROWNORM_F32 ? launch_norm_fwd<f16, float, RMS>(plan, a, s)
-                             : launch_norm_fwd<f16, f16, RMS>(plan, a, s);
-  return wd == ROWNORM_F32 ? launch_norm_fwd<bf16, float, RMS>(plan, a, s)
-                           : launch_norm_fwd<bf16, bf16, RMS>(plan, a, s);
+  if (xd == ROWNORM_F32) {
+    if (yd == ROWNORM_BF16)
+      return add ? launch_norm_fwd<float, float, RMS, bf16, true>(plan, a, s)
+                 : launch_norm_fwd<float, float, RMS, bf16, false>(plan, a, s);
+    if (yd == ROWNORM_F16)
+      return add ? launch_norm_fwd<float, float, RMS, f16, true>(plan, a, s)
+                 : launch_norm_fwd<float, float, RMS, f16, false>(plan, a, s);
+    return add ? launch_norm_fwd<float, float, RMS, float, true>(plan, a, s)
+               : launch_norm_fwd<float, float, RMS>(plan, a, s);
+  }
+  if (xd == ROWNORM_F16) {
+    if (wd == ROWNORM_F32)
+      return add ? launch_norm_fwd<f16, float, RMS, f16, true>(plan, a, s)
+                 : launch_norm_fwd<f16, float, RMS>(plan, a, s);
+    return add ? launch_norm_fwd<f16, f16, RMS, f16, true>(plan, a, s)
+               : launch_norm_fwd<f16, f16, RMS>(plan, a, s);
+  }
+  if (wd == ROWNORM_F32)
+    return add ? launch_norm_fwd<bf16, float, RMS, bf16, true>(plan, a, s)
+               : launch_norm_fwd<bf16, float, RMS>(plan, a, s);
+  return add ? launch_norm_fwd<bf16, bf16, RMS, bf16, true>(plan, a, s)
+             : launch_norm_fwd<bf16, bf16, RMS>(plan, a, s);
 }
 
 // Bytes of the [M, split, 2] fp32 partial sums of the split-row backward and the
@@ -206,10 +260,12 @@ size_t norm_bwd_workspace(int op, int64_t M, int64_t N, int xd, int wd, int npar
          split_bytes(plan, M);
 }
 
+// dres: the gradient reaching the normalized row by the residual path, added to dx (or null).
 template <bool RMS>
 int norm_bwd(const void* dy, const void* x, const float* mean, const float* rstd,
              const void* gamma, void* dx, void* dgamma, void* dbeta, void* workspace,
-             size_t workspace_bytes, int64_t M, int64_t N, int xd, int wd, void* stream) {
+             size_t workspace_bytes, int64_t M, int64_t N, int xd, int wd, void* stream,
+             const void* dres = nullptr) {
   if (!norm_dtypes_ok(xd, wd)) return ROWNORM_ERR_DTYPE;
   if (int e = shape_check(M, N)) return e;
   if (M == 0 || N == 0) return 0;
@@ -238,6 +294,15 @@ int norm_bwd(const void* dy, const void* x, const float* mean, const float* rstd
   if (dx && workspace && split_bytes(plan, M) > 0 && workspace_bytes >= need + split_bytes(plan, M))
     a.split_ws = (float*)((char*)workspace + need);
   hipStream_t s = (hipStream_t)stream;
+  if (dres != nullptr && dx != nullptr) {
+    a.dres = dres;
+    if (xd == ROWNORM_F32) return launch_norm_bwd<float, float, RMS, true>(plan, a, s);
+    if (xd == ROWNORM_F16)
+      return wd == ROWNORM_F32 ? launch_norm_bwd<f16, float, RMS, true>(plan, a, s)
+                               : launch_norm_bwd<f16, f16, RMS, true>(plan, a, s);
+    return wd == ROWNORM_F32 ? launch_norm_bwd<bf16, float, RMS, true>(plan, a, s)
+                             : launch_norm_bwd<bf16, bf16, RMS, true>(plan, a, s);
+  }
   if (xd == ROWNORM_F32) return launch_norm_bwd<float, float, RMS>(plan, a, s);
   if (xd == ROWNORM_F16)
     return wd == ROWNORM_F32 ? launch_norm_bwd<f16, float, RMS>(plan, a, s)
@@ -382,15 +447,48 @@ int mi355x_rownorm_abi_version(void) { return 1; }
 int mi355x_layer_norm_fwd(const void* x, const void* gamma, const void* beta, void* y,
                           float* mean, float* rstd, int64_t M, int64_t N, float eps,
                           rownorm_dtype x_dtype, rownorm_dtype w_dtype, void* stream) {
-  return norm_fwd<false>(x, gamma, beta, y, mean, rstd, M, N, eps, (int)x_dtype, (int)w_dtype,
-                         stream);
+  return norm_fwd<false>(x, nullptr, gamma, beta, nullptr, y, mean, rstd, M, N, eps, (int)x_dtype,
+                         (int)w_dtype, (int)x_dtype, stream);
+}
+
+int mi355x_add_layer_norm_fwd(const void* x, const void* residual, const void* gamma,
+                              const void* beta, void* h, void* y, float* mean, float* rstd,
+                              int64_t M, int64_t N, float eps, rownorm_dtype x_dtype,
+                              rownorm_dtype w_dtype, rownorm_dtype y_dtype, void* stream) {
+  return norm_fwd<false>(x, residual, gamma, beta, h, y, mean, rstd, M, N, eps, (int)x_dtype,
+                         (int)w_dtype, (int)y_dtype, stream);
+}
+
+int mi355x_add_rms_norm_fwd(const void* x, const void* residual, const void* gamma, void* h,
+                            void* y, float* rstd, int64_t M, int64_t N, float eps,
+                            rownorm_dtype x_dtype, rownorm_dtype w_dtype, rownorm_dtype y_dtype,
+                            void* stream) {
+  return norm_fwd<true>(x, residual, gamma, nullptr, h, y, nullptr, rstd, M, N, eps,
+                        (int)x_dtype, (int)w_dtype, (int)y_dtype, stream);
+}
+
+int mi355x_add_layer_norm_bwd(const void* dy, const void* dh_in, const void* h, const float* mean,
+                              const float* rstd, const void* gamma, void* dh, void* dgamma,
+                              void* dbeta, void* workspace, size_t workspace_bytes, int64_t M,
+                              int64_t N, rownorm_dtype x_dtype, rownorm_dtype w_dtype,
+                              void* stream) {
+  return norm_bwd<false>(dy, h, mean, rstd, gamma, dh, dgamma, dbeta, workspace, workspace_bytes,
+                         M, N, (int)x_dtype, (int)w_dtype, stream, dh_in);
+}
+
+int mi355x_add_rms_norm_bwd(const void* dy, const void* dh_in, const void* h, const float* rstd,
+                            const void* gamma, void* dh, void* dgamma, void* workspace,
+                            size_t workspace_bytes, int64_t M, int64_t N, rownorm_dtype x_dtype,
+                            rownorm_dtype w_dtype, void* stream) {
+  return norm_bwd<true>(dy, h, nullptr, rstd, gamma, dh, dgamma, nullptr, workspace,
+                        workspace_bytes, M, N, (int)x_dtype, (int)w_dtype, stream, dh_in);
 }
 
 int mi355x_rms_norm_fwd(const void* x, const void* gamma, void* y, float* rstd, int64_t M,
                         int64_t N, float eps, rownorm_dtype x_dtype, rownorm_dtype w_dtype,
                         void* stream) {
-  return norm_fwd<true>(x, gamma, nullptr, y, nullptr, rstd, M, N, eps, (int)x_dtype,
-                        (int)w_dtype, stream);
+  return norm_fwd<true>(x, nullptr, gamma, nullptr, nullptr, y, nullptr, rstd, M, N, eps,
+                        (int)x_dtype, (int)w_dtype, (int)x_dtype, stream);
 }
 
 size_t mi355x_layer_norm_bwd_workspace_bytes(int64_t M, int64_t N, rownorm_dtype x_dtype,

@@ -19,6 +19,10 @@ struct NormFwdArgs {
   int64_t M;
   int N;
   float eps;
+  // fused residual add: the row that is normalized is h = x + res, written to h
+  // (both null: plain norm of x)
+  const void* res = nullptr;
+  void* h = nullptr;
 };
 
 struct NormBwdArgs {
@@ -35,6 +39,7 @@ struct NormBwdArgs {
   int64_t M;
   int N;
   float* split_ws = nullptr;  // [M, plan.split + 1, 2] fp32 for the split-row path, or null: not split
+  const void* dres = nullptr;  // gradient reaching the normalized row by the residual path, added to dx
 };
 
 constexpr int kSoftmaxLog = 1;   // log_softmax instead of softmax
@@ -109,9 +114,11 @@ struct GroupNormBwdArgs {
 };
 
 // All return 0 or a hipError_t value.
-template <class T, class WT, bool RMS>
+// TY: element type of y (T, or a 16-bit type for float32 rows); ADD: a.res / a.h
+// are given (forward), a.dres is given (backward).
+template <class T, class WT, bool RMS, class TY = T, bool ADD = false>
 int launch_norm_fwd(const Plan& plan, const NormFwdArgs& a, hipStream_t stream);
-template <class T, class WT, bool RMS>
+template <class T, class WT, bool RMS, bool ADD = false>
 int launch_norm_bwd(const Plan& plan, const NormBwdArgs& a, hipStream_t stream);
 template <class TI, class TO>
 int launch_softmax_fwd(const Plan& plan, const SoftmaxFwdArgs& a, hipStream_t stream);

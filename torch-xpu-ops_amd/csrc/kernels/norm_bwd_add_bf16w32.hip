@@ -1,0 +1,7 @@
+// LayerNorm / RMSNorm bwd kernels that add the gradient of the residual path to dx, rows bf16,
+// weights float.
+#include "norm_launch.hpp"
+namespace rownorm {
+template int launch_norm_bwd<bf16, float, false, true>(const Plan&, const NormBwdArgs&, hipStream_t);
+template int launch_norm_bwd<bf16, float, true, true>(const Plan&, const NormBwdArgs&, hipStream_t);
+}  // namespace rownorm

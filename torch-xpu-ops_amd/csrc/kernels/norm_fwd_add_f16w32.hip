@@ -1,0 +1,7 @@
+// LayerNorm / RMSNorm fwd kernels with the residual add fused in (h = x + res is written and
+// normalized), rows f16, weights float.
+#include "norm_launch.hpp"
+namespace rownorm {
+template int launch_norm_fwd<f16, float, false, f16, true>(const Plan&, const NormFwdArgs&, hipStream_t);
+template int launch_norm_fwd<f16, float, true, f16, true>(const Plan&, const NormFwdArgs&, hipStream_t);
+}  // namespace rownorm

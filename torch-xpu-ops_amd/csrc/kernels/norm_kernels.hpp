@@ -50,10 +50,20 @@ namespace rownorm {
 // library is built with R = 1: on MI355X R = 2 measured only 1-3% faster at
 // G >= 256 (and slower in the backward, whose two-row body needs over 150
 // VGPRs), not worth twice the kernels.
-template <class T, class WT, int G, int V, int BLOCK, int R, bool RMS, bool FAST>
+//
+// ADD: the row that is normalized is h = x + res (the residual stream of a
+// transformer block), formed in float32 and rounded once to T, exactly what an
+// elementwise add of the two tensors gives; h is written out (one read of x,
+// one of res, one write of h and one of y instead of the three reads and two
+// writes of an add followed by a norm).  h may be the memory of x or of res: a
+// lane stores its h packs after the statistics, when every lane of the row has
+// read what it needs.  TY: the element type of y (the output cast fused into the
+// store; T unless a float32 row is written out in 16 bits).
+template <class T, class WT, int G, int V, int BLOCK, int R, bool RMS, bool FAST, class TY = T,
+          bool ADD = false>
 __global__ void __launch_bounds__(BLOCK)
-norm_fwd_resident_kernel(const T* __restrict__ x, const WT* __restrict__ gamma,
-                         const WT* __restrict__ beta, T* __restrict__ y,
+norm_fwd_resident_kernel(const T* __restrict__ x, const T* res, const WT* __restrict__ gamma,
+                         const WT* __restrict__ beta, T* h, TY* __restrict__ y,
                          float* __restrict__ mean, float* __restrict__ rstd, int64_t M, int N,
                          float eps) {
   constexpr int E = elems_per_pack<T>::value;
@@ -92,6 +102,17 @@ norm_fwd_resident_kernel(const T* __restrict__ x, const WT* __restrict__ gamma,
 #pragma unroll
       for (int c = 0; c < V; ++c)
         xp[r][c] = row_load<T, E, true, FAST>(xr, (c * G + lane) * E, N, ok[r], 0.0f);
+      if constexpr (ADD) {
+        const T* rr = res + (ok[r] ? row0 + r : 0) * (int64_t)N;
+        Pack<T, E> rp[V];
+#pragma unroll
+        for (int c = 0; c < V; ++c)
+          rp[c] = row_load<T, E, true, FAST>(rr, (c * G + lane) * E, N, ok[r], 0.0f);
+#pragma unroll
+        for (int c = 0; c < V; ++c)
+#pragma unroll
+          for (int i = 0; i < E; ++i) xp[r][c].set(i, xp[r][c].get(i) + rp[c].get(i));
+      }
     }
 
     float mean0[R], m1[R], rs[R];
@@ -128,7 +149,14 @@ norm_fwd_resident_kernel(const T* __restrict__ x, const WT* __restrict__ gamma,
 #pragma unroll
       for (int r = 0; r < R; ++r) {
         const T* xr = x + (ok[r] ? row0 + r : 0) * (int64_t)N;
-        const Pack<T, E> head = load_row_pack<T, E, false>(xr, 0, N, true, 0.0f);
+        Pack<T, E> head = load_row_pack<T, E, false>(xr, 0, N, true, 0.0f);
+        if constexpr (ADD) {
+          // the head of h, formed as the lane that owns it forms it
+          const Pack<T, E> rh = load_row_pack<T, E, false>(
+              res + (ok[r] ? row0 + r : 0) * (int64_t)N, 0, N, true, 0.0f);
+#pragma unroll
+          for (int i = 0; i < 3; ++i) head.set(i, head.get(i) + rh.get(i));
+        }
         const float a = head.get(0), b = head.get(1), c3 = head.get(2);
         const float k = fmaxf(fminf(a, b), fminf(fmaxf(a, b), c3));
         mean0[r] = k;
@@ -228,15 +256,18 @@ norm_fwd_resident_kernel(const T* __restrict__ x, const WT* __restrict__ gamma,
     // element; it measured slower: fewer wavefronts stay resident.)
 #pragma unroll
     for (int r = 0; r < R; ++r) {
-      T* yr = y + (row0 + r) * (int64_t)N;
+      TY* yr = y + (row0 + r) * (int64_t)N;
 #pragma unroll
       for (int c = 0; c < V; ++c) {
         keep_packed(xp[r][c]);
+        if constexpr (ADD)
+          row_store<T, E, true, FAST>(h + (row0 + r) * (int64_t)N, (c * G + lane) * E, N, ok[r],
+                                      xp[r][c]);
         if constexpr (!kWideWeights) {
           keep_packed(gp[c]);
           if constexpr (!RMS) keep_packed(bp[c]);
         }
-        Pack<T, E> o;
+        Pack<TY, E> o;
 #pragma unroll
         for (int i = 0; i < E; ++i) {
           float v;
@@ -246,7 +277,7 @@ norm_fwd_resident_kernel(const T* __restrict__ x, const WT* __restrict__ gamma,
             v = (((xp[r][c].get(i) - mean0[r]) - m1[r]) * rs[r]) * gp[c].get(i) + bp[c].get(i);
           o.set(i, v);
         }
-        row_store<T, E, true, FAST>(yr, (c * G + lane) * E, N, ok[r], o);
+        row_store<TY, E, true, FAST>(yr, (c * G + lane) * E, N, ok[r], o);
       }
       if (ok[r] && lane == 0) {
         if constexpr (!RMS)
@@ -261,10 +292,30 @@ norm_fwd_resident_kernel(const T* __restrict__ x, const WT* __restrict__ gamma,
 
 // The centre the long-row kernels shift their sums by: the median of the row's
 // first three elements, the same value in every workgroup that works on the row.
+// With a residual row `rr` (may be null) the row is h = x + res rounded to T.
 template <class T>
-__device__ __forceinline__ float split_row_centre(const T* xr, int N) {
-  const float a = (float)xr[0], b = (float)xr[N > 1 ? 1 : 0], c = (float)xr[N > 2 ? 2 : 0];
+__device__ __forceinline__ float split_row_centre(const T* xr, const T* rr, int N) {
+  const int i1 = N > 1 ? 1 : 0, i2 = N > 2 ? 2 : 0;
+  float a = (float)xr[0], b = (float)xr[i1], c = (float)xr[i2];
+  if (rr != nullptr) {
+    a = (float)(T)(a + (float)rr[0]);
+    b = (float)(T)(b + (float)rr[i1]);
+    c = (float)(T)(c + (float)rr[i2]);
+  }
   return fmaxf(fminf(a, b), fminf(fmaxf(a, b), c));
+}
+
+// One pack of the row the long-row kernels normalize: x, or x + res (formed in
+// float32, rounded once to T) when a residual row is given.
+template <class T, int E, bool STREAM>
+__device__ __forceinline__ Pack<T, E> load_sum_pack(const T* xr, const T* rr, int e0, int n) {
+  Pack<T, E> p = load_row_pack<T, E, STREAM>(xr, e0, n, true, 0.0f);
+  if (rr != nullptr) {
+    const Pack<T, E> q = load_row_pack<T, E, STREAM>(rr, e0, n, true, 0.0f);
+#pragma unroll
+    for (int i = 0; i < E; ++i) p.set(i, p.get(i) + q.get(i));
+  }
+  return p;
 }
 
 // ---------------------------------------------------------------------------
@@ -274,10 +325,12 @@ __device__ __forceinline__ float split_row_centre(const T* xr, int N) {
 // (x - k)^2 in float64, k = the median of the row's first three elements (see
 // the split-row kernels below for why float64); RMSNorm sums x^2 in float32,
 // where nothing cancels.
-template <class T, class WT, int BLOCK, bool RMS>
+// res / h (null, or both given): the row is h = x + res, written out in the
+// second pass (see the resident kernel); TY: the element type of y.
+template <class T, class WT, int BLOCK, bool RMS, class TY = T>
 __global__ void __launch_bounds__(BLOCK)
-norm_fwd_stream_kernel(const T* __restrict__ x, const WT* __restrict__ gamma,
-                       const WT* __restrict__ beta, T* __restrict__ y,
+norm_fwd_stream_kernel(const T* __restrict__ x, const T* res, const WT* __restrict__ gamma,
+                       const WT* __restrict__ beta, T* h, TY* __restrict__ y,
                        float* __restrict__ mean, float* __restrict__ rstd, int64_t M, int N,
                        float eps) {
   constexpr int E = elems_per_pack<T>::value;
@@ -289,24 +342,25 @@ norm_fwd_stream_kernel(const T* __restrict__ x, const WT* __restrict__ gamma,
   const int npacks = (N + E - 1) / E;
   for (int64_t row = blockIdx.x; row < M; row += gridDim.x) {
     const T* xr = x + row * (int64_t)N;
-    T* yr = y + row * (int64_t)N;
+    const T* rr = res ? res + row * (int64_t)N : nullptr;
+    TY* yr = y + row * (int64_t)N;
     // mean = hi + lo: the saved statistic and the remainder of the float64 mean, kept
     // apart so that the rounding of the saved mean never enters y
     float hi = 0.0f, lo = 0.0f, rs;
     if constexpr (RMS) {
       float acc[1] = {0.0f};
       for (int pk = threadIdx.x; pk < npacks; pk += BLOCK) {
-        const Pack<T, E> p = load_row_pack<T, E, false>(xr, pk * E, N, true, 0.0f);
+        const Pack<T, E> p = load_sum_pack<T, E, false>(xr, rr, pk * E, N);
 #pragma unroll
         for (int i = 0; i < E; ++i) acc[0] = fmaf(p.get(i), p.get(i), acc[0]);
       }
       group_allreduce<BLOCK, BLOCK, 1, SumOp>(acc, red, phase);
       rs = 1.0f / sqrtf(acc[0] / fN + eps);
     } else {
-      const double k = (double)split_row_centre(xr, N);
+      const double k = (double)split_row_centre(xr, rr, N);
       double s1 = 0.0, s2 = 0.0;
       for (int pk = threadIdx.x; pk < npacks; pk += BLOCK) {
-        const Pack<T, E> p = load_row_pack<T, E, false>(xr, pk * E, N, true, 0.0f);
+        const Pack<T, E> p = load_sum_pack<T, E, false>(xr, rr, pk * E, N);
         const int nvalid = N - pk * E;
 #pragma unroll
         for (int i = 0; i < E; ++i) {
@@ -331,15 +385,19 @@ norm_fwd_stream_kernel(const T* __restrict__ x, const WT* __restrict__ gamma,
       lo = stat[1];
       rs = stat[2];
     }
+    // (h may lie on top of x or res: the block reduction above is a barrier, so every
+    // thread has finished the first pass before any of h is written; a thread then
+    // reads and writes the same elements)
     for (int pk = threadIdx.x; pk < npacks; pk += BLOCK) {
       const int e0 = pk * E;
-      const Pack<T, E> p = load_row_pack<T, E, true>(xr, e0, N, true, 0.0f);
+      const Pack<T, E> p = load_sum_pack<T, E, true>(xr, rr, e0, N);
+      if (rr != nullptr) store_row_pack<T, E, true>(h + row * (int64_t)N, e0, N, true, p);
       const Pack<WT, E> pg = gamma ? load_row_pack<WT, E, false>(gamma, e0, N, true, 1.0f)
                                    : Pack<WT, E>::splat(1.0f);
       Pack<WT, E> pb = Pack<WT, E>::zero();
       if constexpr (!RMS)
         if (beta) pb = load_row_pack<WT, E, false>(beta, e0, N, true, 0.0f);
-      Pack<T, E> o;
+      Pack<TY, E> o;
 #pragma unroll
       for (int i = 0; i < E; ++i) {
         float v;
@@ -349,7 +407,7 @@ norm_fwd_stream_kernel(const T* __restrict__ x, const WT* __restrict__ gamma,
           v = (((p.get(i) - hi) - lo) * rs) * pg.get(i) + pb.get(i);
         o.set(i, v);
       }
-      store_row_pack<T, E, true>(yr, e0, N, true, o);
+      store_row_pack<TY, E, true>(yr, e0, N, true, o);
     }
     if (threadIdx.x == 0) {
       if constexpr (!RMS)
@@ -390,11 +448,14 @@ norm_fwd_stream_kernel(const T* __restrict__ x, const WT* __restrict__ gamma,
 // read `lo`: no workspace, and no workgroup waits for another.
 constexpr int kSplitSlotBytes = 24;
 
-template <class T>
-__device__ __forceinline__ double* split_chunk_slot(T* y_row, int64_t first_pack) {
-  constexpr int E = elems_per_pack<T>::value;
+// `elems_per_chunk_pack`: elements of the row per pack (of the row type, whatever the
+// element type of y).
+template <class TY>
+__device__ __forceinline__ double* split_chunk_slot(TY* y_row, int64_t first_pack,
+                                                    int elems_per_chunk_pack) {
   return reinterpret_cast<double*>(
-      (reinterpret_cast<uintptr_t>(y_row + first_pack * E) + 7) & ~uintptr_t(7));
+      (reinterpret_cast<uintptr_t>(y_row + first_pack * elems_per_chunk_pack) + 7) &
+      ~uintptr_t(7));
 }
 
 // The packs [p0, p1) of chunk `chunk` out of `chunks`.
@@ -404,22 +465,23 @@ __device__ __forceinline__ void split_chunk_range(int chunk, int chunks, int64_t
   *p1 = chunk == chunks - 1 ? npacks : *p0 + chunk_packs;
 }
 
-template <class T, int BLOCK, bool RMS>
+template <class T, int BLOCK, bool RMS, class TY = T>
 __global__ void __launch_bounds__(BLOCK)
-norm_fwd_split_sums_kernel(const T* __restrict__ x, T* __restrict__ y, int N,
+norm_fwd_split_sums_kernel(const T* __restrict__ x, const T* res, TY* __restrict__ y, int N,
                            int64_t chunk_packs) {
   constexpr int E = elems_per_pack<T>::value;
   __shared__ double red[2 * (BLOCK / 64)];
   const int64_t row = blockIdx.y;
   const T* xr = x + row * (int64_t)N;
+  const T* rr = res ? res + row * (int64_t)N : nullptr;
   const int64_t npacks = ((int64_t)N + E - 1) / E;
   int64_t p0, p1;
   split_chunk_range(blockIdx.x, gridDim.x, chunk_packs, npacks, &p0, &p1);
-  const double k = RMS ? 0.0 : (double)split_row_centre(xr, N);
+  const double k = RMS ? 0.0 : (double)split_row_centre(xr, rr, N);
   double s1 = 0.0, s2 = 0.0;
   for (int64_t pk = p0 + threadIdx.x; pk < p1; pk += BLOCK) {
     const int e0 = (int)(pk * E);
-    const Pack<T, E> p = load_row_pack<T, E, false>(xr, e0, N, true, 0.0f);
+    const Pack<T, E> p = load_sum_pack<T, E, false>(xr, rr, e0, N);
     const int nvalid = N - e0;
 #pragma unroll
     for (int i = 0; i < E; ++i) {
@@ -430,7 +492,7 @@ norm_fwd_split_sums_kernel(const T* __restrict__ x, T* __restrict__ y, int N,
   }
   block_sum2_f64<BLOCK>(s1, s2, red);
   if (threadIdx.x == 0) {
-    double* slot = split_chunk_slot(y + row * (int64_t)N, p0);
+    double* slot = split_chunk_slot(y + row * (int64_t)N, p0, E);
     slot[0] = s1;
     slot[1] = s2;
   }
@@ -438,16 +500,17 @@ norm_fwd_split_sums_kernel(const T* __restrict__ x, T* __restrict__ y, int N,
 
 // One wavefront per row: lane l adds the partial sums of chunks l, l + 64, ...
 // and a fixed tree adds the lanes, the same order on every run.
-template <class T, bool RMS>
+template <class T, bool RMS, class TY = T>
 __global__ void __launch_bounds__(64)
-norm_fwd_split_stats_kernel(const T* __restrict__ x, T* __restrict__ y,
+norm_fwd_split_stats_kernel(const T* __restrict__ x, const T* res, TY* __restrict__ y,
                             float* __restrict__ mean, float* __restrict__ rstd, int N, int chunks,
                             int64_t chunk_packs, float eps) {
+  constexpr int E = elems_per_pack<T>::value;
   const int64_t row = blockIdx.x;
-  T* yr = y + row * (int64_t)N;
+  TY* yr = y + row * (int64_t)N;
   double s1 = 0.0, s2 = 0.0;
   for (int c = threadIdx.x; c < chunks; c += 64) {
-    const double* slot = split_chunk_slot(yr, (int64_t)c * chunk_packs);
+    const double* slot = split_chunk_slot(yr, (int64_t)c * chunk_packs, E);
     s1 += slot[0];
     s2 += slot[1];
   }
@@ -464,7 +527,8 @@ norm_fwd_split_stats_kernel(const T* __restrict__ x, T* __restrict__ y,
     if (threadIdx.x == 0) rstd[row] = (float)(1.0 / sqrt(s2 / dN + (double)eps));
   } else {
     const double m1 = s1 / dN;
-    const double mu = (double)split_row_centre(x + row * (int64_t)N, N) + m1;
+    const double mu = (double)split_row_centre(x + row * (int64_t)N,
+                                               res ? res + row * (int64_t)N : nullptr, N) + m1;
     double var = (s2 - s1 * m1) / dN;
     var = var < 0.0 ? 0.0 : var;  // (a select: NaN stays NaN)
     const float hi = (float)mu;
@@ -476,36 +540,38 @@ norm_fwd_split_stats_kernel(const T* __restrict__ x, T* __restrict__ y,
   }
   if constexpr (!RMS)
     for (int c = threadIdx.x; c < chunks; c += 64)
-      *reinterpret_cast<float*>(split_chunk_slot(yr, (int64_t)c * chunk_packs)) = lo;
+      *reinterpret_cast<float*>(split_chunk_slot(yr, (int64_t)c * chunk_packs, E)) = lo;
 }
 
-template <class T, class WT, int BLOCK, bool RMS>
+template <class T, class WT, int BLOCK, bool RMS, class TY = T>
 __global__ void __launch_bounds__(BLOCK)
-norm_fwd_split_apply_kernel(const T* __restrict__ x, const WT* __restrict__ gamma,
-                            const WT* __restrict__ beta, T* __restrict__ y,
+norm_fwd_split_apply_kernel(const T* __restrict__ x, const T* res, const WT* __restrict__ gamma,
+                            const WT* __restrict__ beta, T* h, TY* __restrict__ y,
                             const float* __restrict__ mean, const float* __restrict__ rstd, int N,
                             int64_t chunk_packs) {
   constexpr int E = elems_per_pack<T>::value;
   const int64_t row = blockIdx.y;
   const T* xr = x + row * (int64_t)N;
-  T* yr = y + row * (int64_t)N;
+  const T* rr = res ? res + row * (int64_t)N : nullptr;
+  TY* yr = y + row * (int64_t)N;
   const int64_t npacks = ((int64_t)N + E - 1) / E;
   int64_t p0, p1;
   split_chunk_range(blockIdx.x, gridDim.x, chunk_packs, npacks, &p0, &p1);
   const float hi = RMS ? 0.0f : mean[row];
   const float rs = rstd[row];
   // the low part of the mean sits where this workgroup is about to write y
-  const float lo = RMS ? 0.0f : *reinterpret_cast<const float*>(split_chunk_slot(yr, p0));
+  const float lo = RMS ? 0.0f : *reinterpret_cast<const float*>(split_chunk_slot(yr, p0, E));
   __syncthreads();
   for (int64_t pk = p0 + threadIdx.x; pk < p1; pk += BLOCK) {
     const int e0 = (int)(pk * E);
-    const Pack<T, E> p = load_row_pack<T, E, true>(xr, e0, N, true, 0.0f);
+    const Pack<T, E> p = load_sum_pack<T, E, true>(xr, rr, e0, N);
+    if (rr != nullptr) store_row_pack<T, E, true>(h + row * (int64_t)N, e0, N, true, p);
     const Pack<WT, E> pg = gamma ? load_row_pack<WT, E, false>(gamma, e0, N, true, 1.0f)
                                  : Pack<WT, E>::splat(1.0f);
     Pack<WT, E> pb = Pack<WT, E>::zero();
     if constexpr (!RMS)
       if (beta) pb = load_row_pack<WT, E, false>(beta, e0, N, true, 0.0f);
-    Pack<T, E> o;
+    Pack<TY, E> o;
 #pragma unroll
     for (int i = 0; i < E; ++i) {
       float v;
@@ -515,7 +581,7 @@ norm_fwd_split_apply_kernel(const T* __restrict__ x, const WT* __restrict__ gamm
         v = (((p.get(i) - hi) - lo) * rs) * pg.get(i) + pb.get(i);
       o.set(i, v);
     }
-    store_row_pack<T, E, true>(yr, e0, N, true, o);
+    store_row_pack<TY, E, true>(yr, e0, N, true, o);
   }
 }
 
@@ -530,11 +596,17 @@ norm_fwd_split_apply_kernel(const T* __restrict__ x, const WT* __restrict__ gamm
 //   s1 = sum dy*gamma            s2 = sum dy*gamma*xhat       xhat = (x-mean)*rstd
 //   dx = (rstd/N) * (N*gamma*dy - xhat*s2 - s1)               (RMS: mean = 0, no s1)
 //   dgamma[j] = sum_rows dy*xhat   dbeta[j] = sum_rows dy
-template <class T, class WT, int G, int V, int BLOCK, int R, bool RMS, bool FAST>
+//
+// ADD: dres, the gradient that reaches the normalized row by another path (the
+// residual stream: the row was h = x + res and the loss also depends on h
+// directly), is added to dx in float32 before the one rounding of the store.
+// dres may be the memory of dx.
+template <class T, class WT, int G, int V, int BLOCK, int R, bool RMS, bool FAST,
+          bool ADD = false>
 __global__ void __launch_bounds__(BLOCK)
-norm_bwd_resident_kernel(const T* __restrict__ dy, const T* __restrict__ x,
+norm_bwd_resident_kernel(const T* __restrict__ dy, const T* __restrict__ x, const T* dres,
                          const float* __restrict__ mean, const float* __restrict__ rstd,
-                         const WT* __restrict__ gamma, T* __restrict__ dx,
+                         const WT* __restrict__ gamma, T* dx,
                          float* __restrict__ part_dg, float* __restrict__ part_db, int64_t M,
                          int N) {
   constexpr int E = elems_per_pack<T>::value;
@@ -625,6 +697,13 @@ norm_bwd_resident_kernel(const T* __restrict__ dy, const T* __restrict__ x,
         const float b = RMS ? 0.0f : s1 * term1;
         const float ra = rs[r] * a;
         const float cc = mu[r] * ra - b;
+        Pack<T, E> up[ADD ? V : 1];
+        if constexpr (ADD) {
+#pragma unroll
+          for (int c = 0; c < V; ++c)
+            up[c] = row_load<T, E, true, FAST>(dres + (ok[r] ? row0 + r : 0) * (int64_t)N,
+                                               (c * G + lane) * E, N, ok[r], 0.0f);
+        }
 #pragma unroll
         for (int c = 0; c < V; ++c) {
           keep_packed(xp[r][c]);
@@ -645,6 +724,7 @@ norm_bwd_resident_kernel(const T* __restrict__ dy, const T* __restrict__ x,
               if constexpr (!RMS) f -= s1;
               f *= term1;
             }
+            if constexpr (ADD) f += up[c].get(i);
             o.set(i, f);
           }
           row_store<T, E, true, FAST>(dr, (c * G + lane) * E, N, ok[r], o);
@@ -720,9 +800,9 @@ norm_bwd_resident_kernel(const T* __restrict__ dy, const T* __restrict__ x,
 // streaming passes over X and dY (sums, then dX).
 template <class T, class WT, int BLOCK, bool RMS>
 __global__ void __launch_bounds__(BLOCK)
-norm_bwd_stream_dx_kernel(const T* __restrict__ dy, const T* __restrict__ x,
+norm_bwd_stream_dx_kernel(const T* __restrict__ dy, const T* __restrict__ x, const T* dres,
                           const float* __restrict__ mean, const float* __restrict__ rstd,
-                          const WT* __restrict__ gamma, T* __restrict__ dx, int64_t M, int N) {
+                          const WT* __restrict__ gamma, T* dx, int64_t M, int N) {
   constexpr int E = elems_per_pack<T>::value;
   __shared__ float red[reduce_lds_floats<BLOCK, BLOCK, 2>::value];
   int phase = 0;
@@ -756,13 +836,15 @@ norm_bwd_stream_dx_kernel(const T* __restrict__ dy, const T* __restrict__ x,
       const Pack<T, E> pd = load_row_pack<T, E, true>(gr, e0, N, true, 0.0f);
       const Pack<WT, E> pg = gamma ? load_row_pack<WT, E, false>(gamma, e0, N, true, 1.0f)
                                    : Pack<WT, E>::splat(1.0f);
+      Pack<T, E> pu = Pack<T, E>::zero();  // the gradient from the residual path, if any
+      if (dres != nullptr) pu = load_row_pack<T, E, true>(dres + row * (int64_t)N, e0, N, true, 0.0f);
       Pack<T, E> o;
 #pragma unroll
       for (int i = 0; i < E; ++i) {
         float f = fN * (pd.get(i) * pg.get(i));
         f -= ((px.get(i) - mu) * rs) * acc[1];
         if constexpr (!RMS) f -= acc[0];
-        o.set(i, f * term1);
+        o.set(i, f * term1 + pu.get(i));
       }
       store_row_pack<T, E, true>(dr, e0, N, true, o);
     }
@@ -814,10 +896,10 @@ norm_bwd_split_sums_kernel(const T* __restrict__ dy, const T* __restrict__ x,
 
 template <class T, class WT, int BLOCK, bool RMS>
 __global__ void __launch_bounds__(BLOCK)
-norm_bwd_split_dx_kernel(const T* __restrict__ dy, const T* __restrict__ x,
+norm_bwd_split_dx_kernel(const T* __restrict__ dy, const T* __restrict__ x, const T* dres,
                          const float* __restrict__ mean, const float* __restrict__ rstd,
                          const WT* __restrict__ gamma, const float* __restrict__ split_ws,
-                         T* __restrict__ dx, int N, int64_t chunk_packs) {
+                         T* dx, int N, int64_t chunk_packs) {
   constexpr int E = elems_per_pack<T>::value;
   static_assert(BLOCK >= kSplitMaxChunks, "one thread per partial sum");
   __shared__ float red[reduce_lds_floats<BLOCK, BLOCK, 2>::value];
@@ -846,13 +928,15 @@ norm_bwd_split_dx_kernel(const T* __restrict__ dy, const T* __restrict__ x,
     const Pack<T, E> pd = load_row_pack<T, E, true>(gr, e0, N, true, 0.0f);
     const Pack<WT, E> pg = gamma ? load_row_pack<WT, E, false>(gamma, e0, N, true, 1.0f)
                                  : Pack<WT, E>::splat(1.0f);
+    Pack<T, E> pu = Pack<T, E>::zero();
+    if (dres != nullptr) pu = load_row_pack<T, E, true>(dres + row * (int64_t)N, e0, N, true, 0.0f);
     Pack<T, E> o;
 #pragma unroll
     for (int i = 0; i < E; ++i) {
       float f = fN * (pd.get(i) * pg.get(i));
       f -= ((px.get(i) - mu) * rs) * acc[1];
       if constexpr (!RMS) f -= acc[0];
-      o.set(i, f * term1);
+      o.set(i, f * term1 + pu.get(i));
     }
     store_row_pack<T, E, true>(dr, e0, N, true, o);
   }
@@ -887,9 +971,10 @@ norm_bwd_split_totals_kernel(const float* __restrict__ split_ws, float* __restri
 template <class T, class WT, int BLOCK, bool RMS>
 __global__ void __launch_bounds__(BLOCK)
 norm_bwd_split_dx_colsum_kernel(const T* __restrict__ dy, const T* __restrict__ x,
-                                const float* __restrict__ mean, const float* __restrict__ rstd,
-                                const WT* __restrict__ gamma, const float* __restrict__ totals,
-                                T* __restrict__ dx, float* __restrict__ part_dg,
+                                const T* dres, const float* __restrict__ mean,
+                                const float* __restrict__ rstd, const WT* __restrict__ gamma,
+                                const float* __restrict__ totals, T* dx,
+                                float* __restrict__ part_dg,
                                 float* __restrict__ part_db, int64_t M, int N) {
   constexpr int E = elems_per_pack<T>::value;
   constexpr int U = 4;
@@ -903,7 +988,7 @@ norm_bwd_split_dx_colsum_kernel(const T* __restrict__ dy, const T* __restrict__ 
 #pragma unroll
   for (int i = 0; i < E; ++i) dg[i] = db[i] = 0.0f;
   for (int64_t row0 = blockIdx.y; row0 < M; row0 += (int64_t)gridDim.y * U) {
-    Pack<T, E> px[U], pd[U];
+    Pack<T, E> px[U], pd[U], pu[U];
     float mu[U], rs[U], s1[U], s2[U];
     bool ok[U];
 #pragma unroll
@@ -913,6 +998,9 @@ norm_bwd_split_dx_colsum_kernel(const T* __restrict__ dy, const T* __restrict__ 
       const int64_t rc = ok[u] ? row : row0;
       px[u] = load_row_pack<T, E, true>(x + rc * (int64_t)N, e0, N, true, 0.0f);
       pd[u] = load_row_pack<T, E, true>(dy + rc * (int64_t)N, e0, N, true, 0.0f);
+      pu[u] = Pack<T, E>::zero();
+      if (dres != nullptr)
+        pu[u] = load_row_pack<T, E, true>(dres + rc * (int64_t)N, e0, N, true, 0.0f);
       mu[u] = RMS ? 0.0f : mean[rc];
       rs[u] = rstd[rc];
       s1[u] = totals[2 * rc];
@@ -930,7 +1018,7 @@ norm_bwd_split_dx_colsum_kernel(const T* __restrict__ dy, const T* __restrict__ 
         float f = fN * (pd[u].get(i) * pg.get(i));
         f -= xh * s2[u];
         if constexpr (!RMS) f -= s1[u];
-        o.set(i, f * term1);
+        o.set(i, f * term1 + pu[u].get(i));
         dg[i] = fmaf(pd[u].get(i), xh, dg[i]);
         db[i] += pd[u].get(i);
       }

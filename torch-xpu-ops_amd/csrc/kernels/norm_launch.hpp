@@ -12,7 +12,7 @@ struct NormFwdCtx {
   hipStream_t stream;
 };
 
-template <class T, class WT, bool RMS, bool FAST>
+template <class T, class WT, bool RMS, bool FAST, class TY, bool ADD>
 struct NormFwdLauncher {
   template <int G, int V, int BLOCK>
   struct At {
@@ -20,10 +20,11 @@ struct NormFwdLauncher {
       if constexpr (variant_built(OC_NORM_FWD, sizeof(T), G, V, FAST) &&
                     block_built(OC_NORM_FWD, G, BLOCK)) {
         if (c.plan.G == G && c.plan.V == V && c.plan.block == BLOCK) {
-          hipLaunchKernelGGL((norm_fwd_resident_kernel<T, WT, G, V, BLOCK, 1, RMS, FAST>),
-                             dim3((unsigned)c.plan.grid), dim3(BLOCK), 0, c.stream,
-                             (const T*)c.a.x, (const WT*)c.a.gamma, (const WT*)c.a.beta,
-                             (T*)c.a.y, c.a.mean, c.a.rstd, c.a.M, c.a.N, c.a.eps);
+          hipLaunchKernelGGL(
+              (norm_fwd_resident_kernel<T, WT, G, V, BLOCK, 1, RMS, FAST, TY, ADD>),
+              dim3((unsigned)c.plan.grid), dim3(BLOCK), 0, c.stream, (const T*)c.a.x,
+              (const T*)c.a.res, (const WT*)c.a.gamma, (const WT*)c.a.beta, (T*)c.a.h,
+              (TY*)c.a.y, c.a.mean, c.a.rstd, c.a.M, c.a.N, c.a.eps);
           return true;
         }
       }
@@ -32,44 +33,54 @@ struct NormFwdLauncher {
   };
 };
 
+inline bool regions_disjoint(const void* a, int64_t abytes, const void* b, int64_t bbytes) {
+  if (a == nullptr || b == nullptr) return true;
+  const char* pa = (const char*)a;
+  const char* pb = (const char*)b;
+  return pa + abytes <= pb || pb + bbytes <= pa;
+}
+
 // The split-row forward keeps a chunk's partial sums in the first bytes of the
 // chunk's piece of Y and hands the statistics to its last launch through mean /
-// rstd: it needs those outputs, and a Y that does not overlap X.
-template <class T, bool RMS>
+// rstd: it needs those outputs, and a Y that overlaps none of X, res and h.
+template <class T, class TY, bool RMS>
 inline bool norm_fwd_can_split(const Plan& plan, const NormFwdArgs& a) {
   if (plan.split <= 1 || a.M > 65535 || a.rstd == nullptr || (!RMS && a.mean == nullptr))
     return false;
-  const char* xb = (const char*)a.x;
-  const char* yb = (const char*)a.y;
-  const int64_t bytes = a.M * (int64_t)a.N * (int64_t)sizeof(T);
-  return yb + bytes <= xb || xb + bytes <= yb;
+  const int64_t elems = a.M * (int64_t)a.N;
+  const int64_t ybytes = elems * (int64_t)sizeof(TY), xbytes = elems * (int64_t)sizeof(T);
+  return regions_disjoint(a.y, ybytes, a.x, xbytes) && regions_disjoint(a.y, ybytes, a.res, xbytes) &&
+         regions_disjoint(a.y, ybytes, a.h, xbytes);
 }
 
-template <class T, class WT, bool RMS>
+template <class T, class WT, bool RMS, class TY, bool ADD>
 int launch_norm_fwd(const Plan& plan, const NormFwdArgs& a, hipStream_t stream) {
+  const T* res = ADD ? (const T*)a.res : nullptr;
+  T* h = ADD ? (T*)a.h : nullptr;
   if (plan.resident) {
     NormFwdCtx<T, WT, RMS> ctx{plan, a, stream};
     const bool launched =
-        plan.fast ? launch_variant<NormFwdLauncher<T, WT, RMS, true>::template At>(ctx)
-                  : launch_variant<NormFwdLauncher<T, WT, RMS, false>::template At>(ctx);
+        plan.fast
+            ? launch_variant<NormFwdLauncher<T, WT, RMS, true, TY, ADD>::template At>(ctx)
+            : launch_variant<NormFwdLauncher<T, WT, RMS, false, TY, ADD>::template At>(ctx);
     if (!launched) return (int)hipErrorInvalidConfiguration;
-  } else if (norm_fwd_can_split<T, RMS>(plan, a)) {
+  } else if (norm_fwd_can_split<T, TY, RMS>(plan, a)) {
     const dim3 grid((unsigned)plan.split, (unsigned)a.M);
-    hipLaunchKernelGGL((norm_fwd_split_sums_kernel<T, kStreamBlock, RMS>), grid,
-                       dim3(kStreamBlock), 0, stream, (const T*)a.x, (T*)a.y, a.N,
+    hipLaunchKernelGGL((norm_fwd_split_sums_kernel<T, kStreamBlock, RMS, TY>), grid,
+                       dim3(kStreamBlock), 0, stream, (const T*)a.x, res, (TY*)a.y, a.N,
                        plan.chunk_packs);
-    hipLaunchKernelGGL((norm_fwd_split_stats_kernel<T, RMS>), dim3((unsigned)a.M), dim3(64), 0,
-                       stream, (const T*)a.x, (T*)a.y, a.mean, a.rstd, a.N, plan.split,
+    hipLaunchKernelGGL((norm_fwd_split_stats_kernel<T, RMS, TY>), dim3((unsigned)a.M), dim3(64), 0,
+                       stream, (const T*)a.x, res, (TY*)a.y, a.mean, a.rstd, a.N, plan.split,
                        plan.chunk_packs, a.eps);
-    hipLaunchKernelGGL((norm_fwd_split_apply_kernel<T, WT, kStreamBlock, RMS>), grid,
-                       dim3(kStreamBlock), 0, stream, (const T*)a.x, (const WT*)a.gamma,
-                       (const WT*)a.beta, (T*)a.y, (const float*)a.mean, (const float*)a.rstd,
-                       a.N, plan.chunk_packs);
+    hipLaunchKernelGGL((norm_fwd_split_apply_kernel<T, WT, kStreamBlock, RMS, TY>), grid,
+                       dim3(kStreamBlock), 0, stream, (const T*)a.x, res, (const WT*)a.gamma,
+                       (const WT*)a.beta, h, (TY*)a.y, (const float*)a.mean,
+                       (const float*)a.rstd, a.N, plan.chunk_packs);
   } else {
-    hipLaunchKernelGGL((norm_fwd_stream_kernel<T, WT, kStreamBlock, RMS>),
+    hipLaunchKernelGGL((norm_fwd_stream_kernel<T, WT, kStreamBlock, RMS, TY>),
                        dim3((unsigned)plan.grid), dim3(kStreamBlock), 0, stream, (const T*)a.x,
-                       (const WT*)a.gamma, (const WT*)a.beta, (T*)a.y, a.mean, a.rstd, a.M, a.N,
-                       a.eps);
+                       res, (const WT*)a.gamma, (const WT*)a.beta, h, (TY*)a.y, a.mean, a.rstd,
+                       a.M, a.N, a.eps);
   }
   return (int)hipGetLastError();
 }
@@ -81,7 +92,7 @@ struct NormBwdCtx {
   hipStream_t stream;
 };
 
-template <class T, class WT, bool RMS, bool FAST>
+template <class T, class WT, bool RMS, bool FAST, bool ADD>
 struct NormBwdLauncher {
   template <int G, int V, int BLOCK>
   struct At {
@@ -89,11 +100,11 @@ struct NormBwdLauncher {
       if constexpr (variant_built(OC_NORM_BWD, sizeof(T), G, V, FAST) &&
                     block_built(OC_NORM_BWD, G, BLOCK)) {
         if (c.plan.G == G && c.plan.V == V && c.plan.block == BLOCK) {
-          hipLaunchKernelGGL((norm_bwd_resident_kernel<T, WT, G, V, BLOCK, 1, RMS, FAST>),
+          hipLaunchKernelGGL((norm_bwd_resident_kernel<T, WT, G, V, BLOCK, 1, RMS, FAST, ADD>),
                              dim3((unsigned)c.plan.grid), dim3(BLOCK), 0, c.stream,
-                             (const T*)c.a.dy, (const T*)c.a.x, c.a.mean, c.a.rstd,
-                             (const WT*)c.a.gamma, (T*)c.a.dx, c.a.part_dg, c.a.part_db, c.a.M,
-                             c.a.N);
+                             (const T*)c.a.dy, (const T*)c.a.x, (const T*)c.a.dres, c.a.mean,
+                             c.a.rstd, (const WT*)c.a.gamma, (T*)c.a.dx, c.a.part_dg,
+                             c.a.part_db, c.a.M, c.a.N);
           return true;
         }
       }
@@ -102,14 +113,15 @@ struct NormBwdLauncher {
   };
 };
 
-template <class T, class WT, bool RMS>
+template <class T, class WT, bool RMS, bool ADD>
 int launch_norm_bwd(const Plan& plan, const NormBwdArgs& a, hipStream_t stream) {
   const bool want_cols = a.part_dg != nullptr;
+  const T* dres = ADD ? (const T*)a.dres : nullptr;
   if (plan.resident) {
     NormBwdCtx<T, WT, RMS> ctx{plan, a, stream};
     const bool launched =
-        plan.fast ? launch_variant<NormBwdLauncher<T, WT, RMS, true>::template At>(ctx)
-                  : launch_variant<NormBwdLauncher<T, WT, RMS, false>::template At>(ctx);
+        plan.fast ? launch_variant<NormBwdLauncher<T, WT, RMS, true, ADD>::template At>(ctx)
+                  : launch_variant<NormBwdLauncher<T, WT, RMS, false, ADD>::template At>(ctx);
     if (!launched) return (int)hipErrorInvalidConfiguration;
   } else {
     constexpr int E = elems_per_pack<T>::value;
@@ -128,20 +140,21 @@ int launch_norm_bwd(const Plan& plan, const NormBwdArgs& a, hipStream_t stream) 
         const unsigned gx = (unsigned)((a.N + CB * E - 1) / (CB * E));
         hipLaunchKernelGGL((norm_bwd_split_dx_colsum_kernel<T, WT, CB, RMS>),
                            dim3(gx, (unsigned)plan.partial_rows), dim3(CB), 0, stream,
-                           (const T*)a.dy, (const T*)a.x, a.mean, a.rstd, (const WT*)a.gamma,
-                           (const float*)totals, (T*)a.dx, a.part_dg, a.part_db, a.M, a.N);
+                           (const T*)a.dy, (const T*)a.x, dres, a.mean, a.rstd,
+                           (const WT*)a.gamma, (const float*)totals, (T*)a.dx, a.part_dg,
+                           a.part_db, a.M, a.N);
         cols_done = true;
       } else {
         hipLaunchKernelGGL((norm_bwd_split_dx_kernel<T, WT, kStreamBlock, RMS>), grid,
-                           dim3(kStreamBlock), 0, stream, (const T*)a.dy, (const T*)a.x, a.mean,
-                           a.rstd, (const WT*)a.gamma, (const float*)a.split_ws, (T*)a.dx, a.N,
-                           plan.chunk_packs);
+                           dim3(kStreamBlock), 0, stream, (const T*)a.dy, (const T*)a.x, dres,
+                           a.mean, a.rstd, (const WT*)a.gamma, (const float*)a.split_ws,
+                           (T*)a.dx, a.N, plan.chunk_packs);
       }
     } else if (a.dx != nullptr) {
       hipLaunchKernelGGL((norm_bwd_stream_dx_kernel<T, WT, kStreamBlock, RMS>),
                          dim3((unsigned)plan.grid), dim3(kStreamBlock), 0, stream,
-                         (const T*)a.dy, (const T*)a.x, a.mean, a.rstd, (const WT*)a.gamma,
-                         (T*)a.dx, a.M, a.N);
+                         (const T*)a.dy, (const T*)a.x, dres, a.mean, a.rstd,
+                         (const WT*)a.gamma, (T*)a.dx, a.M, a.N);
     }
     if (want_cols && !cols_done) {
       constexpr int CB = 256;
