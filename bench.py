@@ -54,8 +54,8 @@ def main():
     ap.add_argument("--no-cpu", action="store_true", help="skip the CPU baselines")
     ap.add_argument("--only-op", default=None, metavar="TEXT",
                     help="profiling aid: run only the rows of the per-op table whose name contains "
-                         "TEXT (--steps calls each after --warmup untimed ones) and print them; "
-                         "no timed step, no baselines")
+                         "TEXT (several alternatives separated by '|'; --steps calls each after "
+                         "--warmup untimed ones) and print them; no timed step, no baselines")
     ap.add_argument("--calibrate-copy", action="store_true",
                     help="also run a plain 256 MiB device copy 10 times (torch copy_), the "
                          "known-size kernel that FETCH_SIZE / WRITE_SIZE readings are scaled by")
@@ -294,7 +294,7 @@ def per_op_table(torch, cabi, L, dev, stream, P, only=None, iters=60, warm=30):
 
     def add(name, nbytes, fns, stock=None, stock_note=None):
         if only is not None:
-            if only not in name:
+            if not any(t in name for t in only.split("|")):
                 return
             stock = None
         us = _time_rotating(torch, fns, iters=iters, warm=warm)

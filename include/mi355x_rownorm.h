@@ -320,7 +320,9 @@ int mi355x_softmax_strided_bwd(const void* grad, const void* y, void* gi, int64_
  * lanes_per_row is the number of lanes along `inner` (one 16-byte pack each),
  * rows_per_block the number of threads along dim_size that share one such
  * lane position, packs_per_lane the dim_size rows each of those holds;
- * resident == 0 means the multi-pass kernel. */
+ * resident == 0 means the multi-pass kernels, and then `reserved` is the number
+ * of chunks the dim_size rows of a tile are cut into, one workgroup each (0: not
+ * cut; the cut needs an output that does not overlap an input). */
 int mi355x_softmax_strided_plan(int backward, int64_t outer, int64_t dim_size, int64_t inner,
                                 rownorm_dtype dtype, rownorm_plan* out);
 

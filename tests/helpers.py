@@ -128,6 +128,17 @@ def colsum_slack(terms):
     return 16.0 * EPS32 * t.pow(2).sum(0).sqrt()
 
 
+def xhat_slack(dy, mean, rstd):
+    """Allowance for a float32 dgamma beside 16-bit rows.  The 16-bit backward kernels form the
+    normalized element as fma(x, rstd, -mean * rstd) (one instruction an element less than
+    (x - mean) * rstd): each term of the column sum then carries the float32 rounding of
+    mean * rstd, 2^-24 * |mean * rstd|, times |dy|.  That is far below a 16-bit unit of x itself,
+    and only shows against the float32 tolerance where a column's terms cancel or the row has no
+    spread at all (N = 1: rstd = 1 / sqrt(eps))."""
+    mr = (torch.as_tensor(mean).double().cpu() * torch.as_tensor(rstd).double().cpu()).abs()
+    return 2.0 * EPS32 * (torch.as_tensor(dy).double().cpu().abs() * mr.reshape(-1, 1)).sum(0)
+
+
 def rowsum_slack(terms, weight):
     """Allowance for an output of the form weight * (float32 sum of `terms` over a row): the sum's
     rounding, 16 * 2^-24 * ||terms||_2 per row, times |weight| per element."""

@@ -159,3 +159,90 @@ def test_host_ops_use_the_strided_kernels_for_every_dim(ops, gpu):
         out = torch.empty(4, 18, 10, 6, dtype=dtype, device=gpu).transpose(0, 1).contiguous().transpose(0, 1)
         ops._softmax.out(xt, 1, False, out=out)
         assert_close(out, torch.ops.aten._softmax(x.float().transpose(1, 3), 1, False), dtype, "out=")
+
+
+@pytest.mark.parametrize("dtype", DTYPES, ids=str)
+def test_many_rows_few_columns_are_split_over_workgroups(cabi, oracle, gpu, dtype):
+    """D in the thousands under too few columns to fill the machine (the reference's own
+    micro-benchmark, test/microbench/softmax.py:17: softmax over dim 0 of [8192, 64] and
+    [8192, 8192]): the D rows of a tile are cut into chunks, one workgroup each, and the per-column
+    maxima and sums cross three launches inside the output tensor.  Forced chunk counts, a ragged
+    inner size, misaligned tensors, masked and NaN columns, the float16 -> float32 output; the
+    in-place call falls back to one workgroup a tile."""
+    dt = cabi.dtype_code(dtype)
+    g = gen(66)
+    ops = (cabi.OP_SOFTMAX_STRIDED_FWD, cabi.OP_SOFTMAX_STRIDED_BWD)
+    try:
+        for shape in ((1, 8192, 64), (2, 2500, 37), (1, 1100, 520), (3, 2300, 8)):
+            outer, D, inner = shape
+            x = (3.0 * torch.randn(shape, generator=g)).to(dtype)
+            x[0, D // 3:, 0] = float("-inf")      # a masked tail
+            x[0, :, 1] = float("-inf")            # a fully masked column
+            x[0, D // 2, 2] = float("nan")        # a NaN poisons its column
+            grad = torch.randn(shape, generator=g).to(dtype)
+            xg, gg = offset_view(x.to(gpu), 1), offset_view(grad.to(gpu), 3)
+            for chunks in (0, 1, 2, 5):
+                for op in ops:
+                    cabi.set_override(op, -1 if chunks else 0, chunks)
+                p = cabi.strided_plan(False, outer, D, inner, dt)
+                assert p["resident"] == 0
+                if chunks:
+                    assert (p["dim_chunks"] > 1) == (chunks > 1), (chunks, p)
+                else:
+                    assert p["dim_chunks"] > 1, p  # the planner's own choice for these shapes
+                print("case split strided", dtype, shape, chunks, p["dim_chunks"], flush=True)
+                for mode, is_log in ((cabi.SOFTMAX, False), (cabi.LOG_SOFTMAX, True)):
+                    y = cabi.softmax_strided_fwd(xg, 1, mode, y=offset_view(torch.empty_like(xg), 2))
+                    oy = _along(lambda a: oracle.softmax_fwd(a, is_log), to_np32(x), 1)
+                    assert_close(y, oy, dtype, "split y chunks=%d log=%d" % (chunks, is_log))
+                    gi = cabi.softmax_strided_bwd(gg, y, 1, mode,
+                                                  gi=offset_view(torch.empty_like(gg), 2))
+                    ogi = np.moveaxis(oracle.softmax_bwd(
+                        np.ascontiguousarray(np.moveaxis(to_np32(grad), 1, -1)),
+                        np.ascontiguousarray(np.moveaxis(to_np32(y), 1, -1)), is_log), -1, 1)
+                    yc, g32 = y.cpu().float().movedim(1, -1), grad.float().movedim(1, -1)
+                    sl = None
+                    if dtype == torch.float32:
+                        sl = (rowsum_slack(g32, torch.exp(yc)) if is_log
+                              else rowsum_slack(yc * g32, yc)).movedim(-1, 1)
+                    assert_close(gi, ogi, dtype, "split gi chunks=%d log=%d" % (chunks, is_log),
+                                 slack=sl)
+                ys = cabi.softmax_strided_fwd(xg, 1, cabi.SAFE_SOFTMAX)
+                assert_close(ys, _along(oracle.safe_softmax_fwd, to_np32(x), 1), dtype, "split safe y")
+                assert bool((ys[0, :, 1] == 0).all())
+                if dtype == torch.float16:
+                    y32 = cabi.softmax_strided_fwd(xg, 1, cabi.SOFTMAX, out_dtype=torch.float32)
+                    assert_close(y32, _along(oracle.softmax_fwd, to_np32(x), 1), torch.float32,
+                                 "split float16 -> float32 y")
+                    g32g = grad.float().to(gpu)
+                    gi16 = cabi.softmax_strided_bwd(g32g, y32, 1, cabi.SOFTMAX,
+                                                    gi_dtype=torch.float16)
+                    assert_close(gi16, cabi.softmax_strided_bwd(g32g, y32, 1, cabi.SOFTMAX),
+                                 torch.float16, "split float32 -> float16 gi")
+            cabi.clear_overrides()
+            # in place: the output is the input, so the values cannot travel in it
+            xin = x.to(gpu).clone()
+            cabi.softmax_strided_fwd(xin, 1, cabi.SOFTMAX, y=xin)
+            assert_close(xin, _along(oracle.softmax_fwd, to_np32(x), 1), dtype, "in place y")
+    finally:
+        cabi.clear_overrides()
+
+
+def test_dim0_of_a_square_matrix_against_the_last_dim_kernels(cabi, gpu):
+    """softmax over dim 0 of [8192, 8192] bf16 (test/microbench/softmax.py:17 in the reference)
+    equals softmax over the last dim of the transpose, computed by the innermost-dimension kernels,
+    within the 16-bit tolerance; forward and backward."""
+    H = W = 8192
+    g = gen(67)
+    x = (2.0 * torch.randn(H, W, generator=g)).bfloat16().to(gpu)
+    grad = torch.randn(H, W, generator=g).bfloat16().to(gpu)
+    p = cabi.strided_plan(False, 1, H, W, cabi.BF16)
+    assert p["resident"] == 0 and p["dim_chunks"] > 1, p
+    y = cabi.softmax_strided_fwd(x, 0)
+    yt = cabi.softmax_fwd(x.t().contiguous())
+    assert_close(y, yt.t(), torch.bfloat16, "dim 0 y vs last-dim kernel")
+    gi = cabi.softmax_strided_bwd(grad, y, 0)
+    git = cabi.softmax_bwd(grad.t().contiguous(), y.t().contiguous())
+    assert_close(gi, git.t(), torch.bfloat16, "dim 0 gi vs last-dim kernel")
+    colsum = y.float().sum(0)
+    assert_close(colsum, torch.ones_like(colsum), torch.bfloat16, "columns sum to 1")

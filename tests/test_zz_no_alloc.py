@@ -52,7 +52,7 @@ def _check_oracle(oracle, x, dy, w, rstd, got, dtype):
     if got[1] is not None:
         # a float32 column sum over all rows carries its own rounding (helpers.colsum_slack)
         sl = None
-        if dtype == torch.float32:
+        if got[1].dtype == torch.float32:
             sl = colsum_slack(dy.cpu().double() * x.cpu().double() * rstd.cpu().double().reshape(-1, 1))
         assert_close(got[1], odw, got[1].dtype, "static dweight", slack=sl)
 

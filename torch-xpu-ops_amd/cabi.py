@@ -157,7 +157,9 @@ def strided_plan(backward, outer, dim_size, inner, dtype=F32):
     p = Plan()
     _check(lib().mi355x_softmax_strided_plan(int(backward), outer, dim_size, inner, dtype,
                                              ctypes.byref(p)), "strided_plan")
-    return p.as_dict()
+    d = p.as_dict()
+    d["dim_chunks"] = p.reserved  # workgroups the dim_size rows of a tile are split over (0: not split)
+    return d
 
 
 def group_norm_plan(backward, N, C, HxW, groups, dtype=F32):

@@ -739,7 +739,7 @@ int mi355x_softmax_strided_plan(int backward, int64_t outer, int64_t dim_size, i
   out->packs_per_lane = plan.V;
   out->block_threads = plan.block;
   out->rows_per_block = 1 << plan.ty_log2;
-  out->reserved = 0;
+  out->reserved = plan.chunks > 1 ? plan.chunks : 0;
   out->grid_blocks = plan.grid;
   out->partial_rows = 0;
   return 0;

@@ -122,4 +122,31 @@ __device__ __forceinline__ void block_sum2_f64(double& a, double& b, double* lds
   }
 }
 
+// The per-row scalar arithmetic (sum / N, 1 / sqrt(var + eps)) is evaluated by
+// every lane of the row, and an IEEE float32 division or square root is about
+// ten VALU instructions: with 16 elements a lane, the two divisions, the square
+// root and the reciprocal of a LayerNorm row were a sixth of all the vector
+// instructions of the 16-bit forward, a kernel that runs the vector ALU at
+// 60 % while it streams from HBM.  16-bit rows therefore multiply by 1 / N
+// (rounded once, outside the row loop) and take the hardware reciprocal square
+// root (v_rsq_f32, one ulp): both move mean / rstd by a float32 ulp, four
+// orders of magnitude inside the 16-bit tolerance, and change nothing on a
+// constant row (the sums are exactly zero there).  float32 rows keep the
+// correctly rounded division and square root.
+template <class T>
+__device__ __forceinline__ float row_mean_of(float sum, float fN, float inv_n) {
+  if constexpr (sizeof(T) == 2)
+    return sum * inv_n;
+  else
+    return sum / fN;
+}
+
+template <class T>
+__device__ __forceinline__ float row_rstd_of(float v) {
+  if constexpr (sizeof(T) == 2)
+    return __builtin_amdgcn_rsqf(v);
+  else
+    return 1.0f / sqrtf(v);
+}
+
 }  // namespace rownorm

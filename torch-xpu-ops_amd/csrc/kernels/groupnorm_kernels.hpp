@@ -91,6 +91,7 @@ gn_fwd_resident_kernel(const T* __restrict__ x, const WT* __restrict__ gamma,
   const int slot = threadIdx.x / G;
   const int lane = threadIdx.x % G;
   const float fL = (float)s.L;
+  const float inv_l = 1.0f / fL;
   const bool exact = s.L == G * V * E;
   const int64_t nrb = (rows + RPB - 1) / RPB;
   for (int64_t rb = blockIdx.x; rb < nrb; rb += gridDim.x) {
@@ -142,10 +143,10 @@ gn_fwd_resident_kernel(const T* __restrict__ x, const WT* __restrict__ gamma,
     else
       centred_sums(std::true_type{});
     group_allreduce<G, BLOCK, 2, SumOp>(acc, red, phase);
-    const float m1 = acc[0] / fL;
-    float var = (acc[1] - acc[0] * m1) / fL;
+    const float m1 = row_mean_of<T>(acc[0], fL, inv_l);
+    float var = row_mean_of<T>(acc[1] - acc[0] * m1, fL, inv_l);
     var = var < 0.0f ? 0.0f : var;  // a select, not v_max_f32: a NaN row keeps NaN statistics
-    const float rs = 1.0f / sqrtf(var + eps);
+    const float rs = row_rstd_of<T>(var + eps);
     T* yr = y + row * (int64_t)s.L;
 #pragma unroll
     for (int c = 0; c < V; ++c) {

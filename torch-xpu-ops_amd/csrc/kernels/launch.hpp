@@ -113,6 +113,13 @@ struct GroupNormBwdArgs {
   int L, HxW, D, groups;
 };
 
+inline bool regions_disjoint(const void* a, int64_t abytes, const void* b, int64_t bbytes) {
+  if (a == nullptr || b == nullptr) return true;
+  const char* pa = (const char*)a;
+  const char* pb = (const char*)b;
+  return pa + abytes <= pb || pb + bbytes <= pa;
+}
+
 // All return 0 or a hipError_t value.
 // TY: element type of y (T, or a 16-bit type for float32 rows); ADD: a.res / a.h
 // are given (forward), a.dres is given (backward).

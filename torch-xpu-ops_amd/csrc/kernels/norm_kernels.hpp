@@ -74,6 +74,7 @@ norm_fwd_resident_kernel(const T* __restrict__ x, const T* res, const WT* __rest
   const int slot = threadIdx.x / G;
   const int lane = threadIdx.x % G;
   const float fN = (float)N;
+  const float inv_n = 1.0f / fN;
 
   // gamma/beta of this lane's columns stay in registers for all rows: widened to
   // fp32 once when they are few, otherwise in storage format and widened per row.
@@ -132,7 +133,7 @@ norm_fwd_resident_kernel(const T* __restrict__ x, const T* res, const WT* __rest
       group_allreduce<G, BLOCK, R, SumOp>(acc, red, phase);
 #pragma unroll
       for (int r = 0; r < R; ++r) {
-        rs[r] = 1.0f / sqrtf(acc[r] / fN + eps);
+        rs[r] = row_rstd_of<T>(row_mean_of<T>(acc[r], fN, inv_n) + eps);
         mean0[r] = m1[r] = 0.0f;
       }
     } else if constexpr (sizeof(T) == 2) {
@@ -186,10 +187,10 @@ norm_fwd_resident_kernel(const T* __restrict__ x, const T* res, const WT* __rest
       group_allreduce<G, BLOCK, 2 * R, SumOp>(acc, red, phase);
 #pragma unroll
       for (int r = 0; r < R; ++r) {
-        m1[r] = acc[2 * r] / fN;
-        float var = (acc[2 * r + 1] - acc[2 * r] * m1[r]) / fN;
+        m1[r] = row_mean_of<T>(acc[2 * r], fN, inv_n);
+        float var = row_mean_of<T>(acc[2 * r + 1] - acc[2 * r] * m1[r], fN, inv_n);
         var = var < 0.0f ? 0.0f : var;  // a select, not v_max_f32: a NaN row keeps NaN statistics
-        rs[r] = 1.0f / sqrtf(var + eps);
+        rs[r] = row_rstd_of<T>(var + eps);
       }
     } else {
       float acc0[R];
@@ -242,10 +243,10 @@ norm_fwd_resident_kernel(const T* __restrict__ x, const T* res, const WT* __rest
       group_allreduce<G, BLOCK, 2 * R, SumOp>(acc, red, phase);
 #pragma unroll
       for (int r = 0; r < R; ++r) {
-        m1[r] = acc[2 * r] / fN;
-        float var = (acc[2 * r + 1] - acc[2 * r] * m1[r]) / fN;
+        m1[r] = row_mean_of<T>(acc[2 * r], fN, inv_n);
+        float var = row_mean_of<T>(acc[2 * r + 1] - acc[2 * r] * m1[r], fN, inv_n);
         var = var < 0.0f ? 0.0f : var;  // a select, not v_max_f32: a NaN row keeps NaN statistics
-        rs[r] = 1.0f / sqrtf(var + eps);
+        rs[r] = row_rstd_of<T>(var + eps);
       }
     }
 
@@ -254,6 +255,9 @@ norm_fwd_resident_kernel(const T* __restrict__ x, const T* res, const WT* __rest
     // bit) and the rounding of mean0 + m1 to one float never enters y.  (Keeping
     // x - mean0 in fp32 registers from the previous pass would save two VALU ops an
     // element; it measured slower: fewer wavefronts stay resident.)
+    float nm1rs[R];
+#pragma unroll
+    for (int r = 0; r < R; ++r) nm1rs[r] = -m1[r] * rs[r];
 #pragma unroll
     for (int r = 0; r < R; ++r) {
       TY* yr = y + (row0 + r) * (int64_t)N;
@@ -273,6 +277,10 @@ norm_fwd_resident_kernel(const T* __restrict__ x, const T* res, const WT* __rest
           float v;
           if constexpr (RMS)
             v = (xp[r][c].get(i) * rs[r]) * gp[c].get(i);
+          else if constexpr (sizeof(T) == 2)
+            // (x - mean0) * rs - m1 * rs in one FMA: one instruction fewer an element;
+            // on a constant row x - mean0 and m1 are exactly zero, so y is still beta
+            v = fmaf(xp[r][c].get(i) - mean0[r], rs[r], nm1rs[r]) * gp[c].get(i) + bp[c].get(i);
           else
             v = (((xp[r][c].get(i) - mean0[r]) - m1[r]) * rs[r]) * gp[c].get(i) + bp[c].get(i);
           o.set(i, v);
@@ -355,7 +363,7 @@ norm_fwd_stream_kernel(const T* __restrict__ x, const T* res, const WT* __restri
         for (int i = 0; i < E; ++i) acc[0] = fmaf(p.get(i), p.get(i), acc[0]);
       }
       group_allreduce<BLOCK, BLOCK, 1, SumOp>(acc, red, phase);
-      rs = 1.0f / sqrtf(acc[0] / fN + eps);
+      rs = 1.0f / sqrtf(acc[0] / fN + eps);  // once a row of >= 32 Ki elements: exact
     } else {
       const double k = (double)split_row_centre(xr, rr, N);
       double s1 = 0.0, s2 = 0.0;
@@ -619,6 +627,7 @@ norm_bwd_resident_kernel(const T* __restrict__ dy, const T* __restrict__ x, cons
   const int slot = threadIdx.x / G;
   const int lane = threadIdx.x % G;
   const float fN = (float)N;
+  const float inv_n = 1.0f / fN;
   const bool want_cols = part_dg != nullptr;  // uniform
   constexpr bool kWideWeights = V * E <= 16;  // few weights: widen to fp32 once, not per row
 
@@ -692,7 +701,7 @@ norm_bwd_resident_kernel(const T* __restrict__ dy, const T* __restrict__ x, cons
         // use the regrouped rs*g - x*(rs*a) + (mu*rs*a - b), a = s2*rs/N,
         // b = s1*rs/N: two FMAs, rounding far below a 16-bit ulp.
         const float s1 = acc[2 * r], s2 = acc[2 * r + 1];
-        const float term1 = rs[r] / fN;
+        const float term1 = row_mean_of<T>(rs[r], fN, inv_n);
         const float a = s2 * term1;
         const float b = RMS ? 0.0f : s1 * term1;
         const float ra = rs[r] * a;

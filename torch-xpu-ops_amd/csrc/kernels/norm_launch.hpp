@@ -33,13 +33,6 @@ struct NormFwdLauncher {
   };
 };
 
-inline bool regions_disjoint(const void* a, int64_t abytes, const void* b, int64_t bbytes) {
-  if (a == nullptr || b == nullptr) return true;
-  const char* pa = (const char*)a;
-  const char* pb = (const char*)b;
-  return pa + abytes <= pb || pb + bbytes <= pa;
-}
-
 // The split-row forward keeps a chunk's partial sums in the first bytes of the
 // chunk's piece of Y and hands the statistics to its last launch through mean /
 // rstd: it needs those outputs, and a Y that overlaps none of X, res and h.

@@ -448,7 +448,12 @@ struct StridedPlan {
   bool fast = true;  // inner % E == 0
   int tx_log2 = 0, ty_log2 = 0, V = 0, block = 0;
   int64_t grid = 0;
+  // multi-pass kernels with too few tiles for the machine: the D rows are cut into
+  // `chunks` chunks of `chunk_rows` rows, one workgroup each (0 or 1: not split)
+  int chunks = 0, chunk_rows = 0;
 };
+
+constexpr int kStridedSplitUnroll = 4;  // rows a lane of the split kernels requests at a time
 
 constexpr int kStridedBlock = 256;
 constexpr int kStridedMaxV = 8;
@@ -460,7 +465,8 @@ inline int log2_of_pow2(int v) {
 }
 
 // Override: G = lanes along inner (power of two 1..64; -1 forces the multi-pass
-// kernel), V = packs per lane.  Returns 0 or -5.
+// kernel, and then V = 1 keeps all D rows of a tile on one workgroup, V > 1 cuts
+// them into that many chunks), V = packs per lane.  Returns 0 or -5.
 inline int make_strided_plan(bool backward, int64_t outer, int64_t D, int64_t inner, int esize,
                              int num_cus, const Override& ov, StridedPlan* out) {
   StridedPlan p;
@@ -474,12 +480,12 @@ inline int make_strided_plan(bool backward, int64_t outer, int64_t D, int64_t in
   // lane) while a wavefront still covers D -- measured faster
   int vcap = kStridedMaxV;
   if (backward && esize == 2 && D > 4 && D <= 32) vcap = 4;
-  if (ov.V > 0) vcap = ov.V;
+  if (ov.V > 0 && ov.G >= 0) vcap = ov.V;
   if (vcap < 1 || vcap > kStridedMaxV) return -5;
   // TY = the power of two that covers D with at most vcap rows a thread; V = the
   // rows a thread then really has (not rounded up: D = 21 is 4 x 6, not 4 x 8)
   const int64_t ty_need = pow2_ceil((D + vcap - 1) / vcap);
-  int V = ov.V > 0 ? ov.V : (int)((D + ty_need - 1) / ty_need);
+  int V = (ov.V > 0 && ov.G >= 0) ? ov.V : (int)((D + ty_need - 1) / ty_need);
   int TX = 0, TY = 0;
   // rows are never cut below 4 lanes (64 bytes) to make room for a larger D
   const int ty_max = kStridedBlock / (px < 4 ? px : 4);
@@ -499,16 +505,43 @@ inline int make_strided_plan(bool backward, int64_t outer, int64_t D, int64_t in
       if (ov.G > 0 || ov.V > 0) return -5;
       stream = true;
     }
-  } else if (ov.G > 0 || ov.V > 0) {
+  } else if (ov.G > 0 || (ov.V > 0 && ov.G >= 0)) {
     return -5;
   }
   if (stream) {
-    // one group per workgroup; few lanes along inner, fewer still while the
-    // problem has less than two workgroups per compute unit
+    // one group per workgroup, rows of up to 8 lanes (128 bytes)
     TX = px < 8 ? px : 8;
-    while (TX > 4 && outer * ((packs + TX - 1) / TX) < 2 * (int64_t)num_cus) TX >>= 1;
     TY = kStridedBlock / TX;
     V = 0;
+    // Too few tiles to fill the machine (softmax over dim 0 of [8192, 8192] is 128
+    // tiles): cut the D rows into chunks of whole TY * unroll strides so that
+    // about four workgroups per compute unit exist; a short remainder joins the
+    // chunk before it.
+    const int64_t tiles = outer * ((packs + TX - 1) / TX);
+    const int64_t min_rows = (int64_t)TY * kStridedSplitUnroll;
+    int64_t want = 1;
+    if (ov.G < 0 && ov.V > 0)
+      want = ov.V;
+    else if (tiles < 2 * (int64_t)num_cus)
+      want = (4 * (int64_t)num_cus + tiles - 1) / tiles;
+    if (want > 1) {
+      int64_t rows = (D + want - 1) / want;
+      rows = (rows + TY - 1) / TY * TY;
+      if (rows < min_rows && !(ov.G < 0 && ov.V > 0)) rows = min_rows;
+      int64_t chunks = (D + rows - 1) / rows;
+      if (chunks > 1 && D - (chunks - 1) * rows < TY) --chunks;
+      if (chunks > 65535) chunks = 1;
+      if (chunks > 1) {
+        p.chunks = (int)chunks;
+        p.chunk_rows = (int)rows;
+      }
+    }
+    if (p.chunks <= 1 && !(ov.G < 0 && ov.V > 0)) {
+      // not split: fewer lanes along inner while the problem has less than two
+      // workgroups per compute unit
+      while (TX > 4 && outer * ((packs + TX - 1) / TX) < 2 * (int64_t)num_cus) TX >>= 1;
+      TY = kStridedBlock / TX;
+    }
   }
   p.resident = !stream;
   p.tx_log2 = log2_of_pow2(TX);
