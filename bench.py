@@ -56,6 +56,9 @@ def main():
                     help="profiling aid: run only the rows of the per-op table whose name contains "
                          "TEXT (several alternatives separated by '|'; --steps calls each after "
                          "--warmup untimed ones) and print them; no timed step, no baselines")
+    ap.add_argument("--width-sweep", action="store_true",
+                    help="print only the hidden-size sweep of the norms (with --only-op: the rows "
+                         "whose name contains TEXT)")
     ap.add_argument("--calibrate-copy", action="store_true",
                     help="also run a plain 256 MiB device copy 10 times (torch copy_), the "
                          "known-size kernel that FETCH_SIZE / WRITE_SIZE readings are scaled by")
@@ -102,11 +105,16 @@ def main():
         return L.mi355x_rms_norm_bwd(P(s["dy"]), P(s["x"]), P(s["rstd"]), P(w), P(s["dx"]),
                                      P(s["dw"]), P(ws), ws_bytes, M, N, BF, BF, stream)
 
+    if args.width_sweep:
+        print(json.dumps({"norm_width_sweep": width_sweep_table(torch, cabi, L, dev, stream, P,
+                                                                only=args.only_op)}))
+        return
     if args.only_op is not None:
         if args.calibrate_copy:
             calibrate_copy(torch, dev)
         rows = per_op_table(torch, cabi, L, dev, stream, P, only=args.only_op,
                             iters=args.steps, warm=args.warmup)
+        rows += reference_microbench_table(torch, cabi, L, dev, stream, P, only=args.only_op)
         print(json.dumps({"ops": rows, "steps": args.steps, "warmup": args.warmup}))
         return
 
@@ -202,6 +210,7 @@ def main():
         worst = min(llama, key=lambda r: r["frac"])
         out["min_frac_llama_ops"] = {"frac": worst["frac"], "op": worst["op"], "target": 0.70,
                                      "ops_counted": len(llama)}
+        out["norm_width_sweep"] = width_sweep_table(torch, cabi, L, dev, stream, P)
         out["reference_microbench"] = reference_microbench_table(torch, cabi, L, dev, stream, P)
         out["config5"] = stress_table(torch, cabi, L, dev, stream, P)
     del sets
@@ -550,7 +559,72 @@ def per_op_table(torch, cabi, L, dev, stream, P, only=None, iters=60, warm=30):
     return rows
 
 
-def reference_microbench_table(torch, cabi, L, dev, stream, P):
+def width_sweep_table(torch, cabi, L, dev, stream, P, only=None):
+    """LayerNorm and RMSNorm forward and backward over the hidden sizes of the Llama-class models
+    (4096 ... 12288, 16384 tokens, bf16 rows; bf16 weights, and float32 weights for LayerNorm):
+    avg microseconds per call (60 back-to-back calls after 30, three buffer sets), algorithmic GB/s
+    and the fraction of 8 TB/s.  `min_frac` of the returned dict is the worst of them."""
+    BF, F32 = cabi.BF16, cabi.F32
+    bf16 = torch.bfloat16
+    M = 16384
+    rows = []
+    for N in (4096, 5120, 6144, 8192, 10240, 12288):
+        sets = []
+        for _ in range(3):
+            x = torch.randn(M, N, device=dev).to(bf16)
+            sets.append((x, torch.randn(M, N, device=dev).to(bf16), torch.empty_like(x),
+                         torch.empty(M, device=dev), torch.empty(M, device=dev)))
+        for wname, wd, wt in (("bf16w", BF, bf16), ("fp32w", F32, torch.float32)):
+            g = (1 + 0.1 * torch.randn(N, device=dev)).to(wt)
+            b = (0.1 * torch.randn(N, device=dev)).to(wt)
+            dg, db = torch.empty_like(g), torch.empty_like(g)
+            wb = g.element_size()
+            nws = max(L.mi355x_layer_norm_bwd_workspace_bytes(M, N, BF, wd, 1, 1),
+                      L.mi355x_rms_norm_bwd_workspace_bytes(M, N, BF, wd, 1))
+            ws = torch.empty(max(nws, 1), dtype=torch.uint8, device=dev)
+            ops = [
+                ("layer_norm fwd", 2 * M * N * 2 + 2 * N * wb + 8 * M,
+                 lambda s: L.mi355x_layer_norm_fwd(P(s[0]), P(g), P(b), P(s[2]), P(s[3]), P(s[4]), M,
+                                                   N, 1e-5, BF, wd, stream)),
+                ("layer_norm bwd", 3 * M * N * 2 + 8 * M + 3 * N * wb,
+                 lambda s: L.mi355x_layer_norm_bwd(P(s[1]), P(s[0]), P(s[3]), P(s[4]), P(g), P(s[2]),
+                                                   P(dg), P(db), P(ws), nws, M, N, BF, wd, stream)),
+            ]
+            if wd == BF:
+                ops += [
+                    ("rms_norm fwd", 2 * M * N * 2 + N * wb + 4 * M,
+                     lambda s: L.mi355x_rms_norm_fwd(P(s[0]), P(g), P(s[2]), P(s[4]), M, N, 1e-6, BF,
+                                                     wd, stream)),
+                    ("rms_norm bwd", 3 * M * N * 2 + 4 * M + 2 * N * wb,
+                     lambda s: L.mi355x_rms_norm_bwd(P(s[1]), P(s[0]), P(s[4]), P(g), P(s[2]), P(dg),
+                                                     P(ws), nws, M, N, BF, wd, stream)),
+                ]
+            for name, nbytes, fn in ops:
+                tag = "%s bf16/%s [%d,%d]" % (name, wname, M, N)
+                if only is not None and not any(t in tag for t in only.split("|")):
+                    continue
+                # the statistics the backward reads come from the forward of the same kind
+                for s_ in sets:
+                    if name.startswith("layer_norm"):
+                        L.mi355x_layer_norm_fwd(P(s_[0]), P(g), P(b), P(s_[2]), P(s_[3]), P(s_[4]), M,
+                                                N, 1e-5, BF, wd, stream)
+                    else:
+                        L.mi355x_rms_norm_fwd(P(s_[0]), P(g), P(s_[2]), P(s_[4]), M, N, 1e-6, BF, wd,
+                                              stream)
+                us = _time_rotating(torch, [(lambda s_=s_: fn(s_)) for s_ in sets])
+                rows.append({"op": tag, "us": round(us, 2), "GB/s": round(nbytes / us / 1e3, 1),
+                             "frac": round(nbytes / us / 1e3 / HBM_PEAK_GBS, 4)})
+            del ws
+        del sets
+        torch.cuda.empty_cache()
+    out = {"rows": rows}
+    if rows:
+        worst = min(rows, key=lambda r: r["frac"])
+        out["min_frac"] = {"frac": worst["frac"], "op": worst["op"], "target": 0.70}
+    return out
+
+
+def reference_microbench_table(torch, cabi, L, dev, stream, P, only=None):
     """The shapes of the reference's own micro-benchmarks for this path, bf16, forward and
     backward: test/microbench/layer_norm.py:17-22 (nn.LayerNorm over the trailing dimensions:
     rows x normalized size = 1 x 1024, 2 x 1310720, 512 x 401408, 128 x 9834496) and
@@ -561,14 +635,18 @@ def reference_microbench_table(torch, cabi, L, dev, stream, P):
     rows = []
 
     def add(name, nbytes, fn, stock, iters):
+        if only is not None and not any(t in name for t in only.split("|")):
+            return
         us = _time_rotating(torch, [fn], iters=iters, warm=max(2, iters // 4))
         row = {"op": name, "us": round(us, 2), "GB/s": round(nbytes / us / 1e3, 1),
                "frac": round(nbytes / us / 1e3 / HBM_PEAK_GBS, 4)}
-        try:
-            row["stock_us"] = round(_time_rotating(torch, [stock], iters=max(3, iters // 4), warm=2), 2)
-        except Exception as e:
-            row["stock_us"] = None
-            row["stock_error"] = type(e).__name__
+        if only is None:
+            try:
+                row["stock_us"] = round(_time_rotating(torch, [stock], iters=max(3, iters // 4),
+                                                       warm=2), 2)
+            except Exception as e:
+                row["stock_us"] = None
+                row["stock_error"] = type(e).__name__
         rows.append(row)
 
     for shape, nshape in (((1, 1024), (1024,)), ((2, 4096, 320), (4096, 320)),
@@ -580,6 +658,10 @@ def reference_microbench_table(torch, cabi, L, dev, stream, P):
         for d in shape:
             M *= d
         M //= N
+        tag = "LayerNorm %s over %s bf16" % ("x".join(map(str, shape)), "x".join(map(str, nshape)))
+        if only is not None and not any(t in tag + " fwd" or t in tag + " bwd"
+                                        for t in only.split("|")):
+            continue
         x = torch.randn(M, N, device=dev, dtype=bf16)
         dy = torch.randn(M, N, device=dev, dtype=bf16)
         g = torch.ones(N, device=dev, dtype=bf16)
@@ -590,7 +672,6 @@ def reference_microbench_table(torch, cabi, L, dev, stream, P):
         nws = L.mi355x_layer_norm_bwd_workspace_bytes(M, N, BF, BF, 1, 1)
         ws = torch.empty(max(nws, 1), dtype=torch.uint8, device=dev)
         iters = 40 if M * N < (1 << 28) else 8
-        tag = "LayerNorm %s over %s bf16" % ("x".join(map(str, shape)), "x".join(map(str, nshape)))
         add(tag + " fwd", 2 * M * N * 2 + 2 * N * 2 + 8 * M,
             lambda: L.mi355x_layer_norm_fwd(P(x), P(g), P(b), P(y), P(mean), P(rstd), M, N, 1e-5, BF,
                                             BF, stream),
@@ -604,6 +685,10 @@ def reference_microbench_table(torch, cabi, L, dev, stream, P):
         torch.cuda.empty_cache()
 
     for (H, W) in ((8192, 8192), (64, 8192), (8192, 64)):
+        if only is not None and not any(t in "Softmax %dx%d dim 0 bf16 fwd bwd" % (H, W) or
+                                        t in "Softmax %dx%d dim 1 bf16 fwd bwd" % (H, W)
+                                        for t in only.split("|")):
+            continue
         x = torch.randn(H, W, device=dev, dtype=bf16)
         gr = torch.randn(H, W, device=dev, dtype=bf16)
         y, gi = torch.empty_like(x), torch.empty_like(x)

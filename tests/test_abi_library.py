@@ -214,7 +214,8 @@ def test_plan_layouts_for_hidden_sizes_that_are_not_powers_of_two(cabi):
         assert lay(LF, N, BF) == want and lay(RF, N, BF) == want
         assert lay(cabi.OP_SOFTMAX_FWD, N, BF) == want
     assert lay(LF, 7168, BF) == (512, 2)                       # fills 7/8: the rule stands
-    assert lay(LB, 5120, BF) == (512, 2) and lay(RB, 5120, BF) == (512, 2)  # 16-bit backward keeps its lanes
+    assert lay(LB, 5120, BF) == (256, 3) and lay(RB, 6144, BF) == (256, 3)  # and the 16-bit backward from 513 packs
+    assert lay(LB, 3072, BF) == (256, 2) and lay(RB, 2560, BF) == (256, 2)  # which keeps its lanes below
     assert lay(LF, 3072, BF, F32) == (256, 2)                  # fp32 weights below 512 lanes
     assert lay(LF, 5120, BF, F32) == (256, 3)
     assert lay(cabi.OP_SOFTMAX_BWD, 5120, BF) == (512, 2)

@@ -91,12 +91,19 @@ def test_limit_is_an_error_before_any_launch(cabi, gpu):
     L = cabi.lib()
     limit = L.mi355x_rms_norm_bwd_static_limit_bytes()
     assert limit == 16 << 20
-    M, N = 16384, 12288  # 512 partial rows of 12288 floats: 24 MiB
-    need = L.mi355x_rms_norm_bwd_workspace_bytes(M, N, cabi.BF16, cabi.BF16, 1)
-    assert need > limit
+    # the launch plans of this build stay within the limit (at most 512 partial rows of 8192
+    # floats, or 256 of 16384: 16 MiB); a forced grid of four workgroups a compute unit does not
+    M, N = 16384, 8192
+    assert L.mi355x_rms_norm_bwd_workspace_bytes(M, N, cabi.BF16, cabi.BF16, 1) <= limit
     one = ctypes.c_void_p(256)  # never dereferenced
-    assert L.mi355x_rms_norm_bwd_static(one, one, one, one, one, one, M, N, cabi.BF16, cabi.BF16,
-                                        None) == -6
+    try:
+        cabi.set_override(cabi.OP_RMS_NORM_BWD, 0, 0, 0, 4)
+        need = L.mi355x_rms_norm_bwd_workspace_bytes(M, N, cabi.BF16, cabi.BF16, 1)
+        assert need > limit
+        assert L.mi355x_rms_norm_bwd_static(one, one, one, one, one, one, M, N, cabi.BF16,
+                                            cabi.BF16, None) == -6
+    finally:
+        cabi.clear_overrides()
     assert "static" in cabi.error_string(-6)
     # dX alone needs no scratch at that size: accepted (nothing launched here: empty problem)
     assert L.mi355x_rms_norm_bwd_static(one, one, one, one, one, None, 0, N, cabi.BF16, cabi.BF16,

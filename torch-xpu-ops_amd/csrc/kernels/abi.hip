@@ -245,9 +245,13 @@ int norm_fwd(const void* x, const void* res, const void* gamma, const void* beta
 }
 
 // Bytes of the [M, split, 2] fp32 partial sums of the split-row backward and the
-// [M, 2] row totals behind them (0: not split).
-size_t split_bytes(const Plan& plan, int64_t M) {
-  return plan.split > 1 ? (size_t)M * ((size_t)plan.split + 1) * 2 * sizeof(float) : 0;
+// [M, 2] row totals behind them; rows that stay on one workgroup but not in its
+// registers keep their [M, 2] row sums there when the column sums are wanted as
+// well (dX and the column sums then share one pass over X and dY).  0: neither.
+size_t split_bytes(const Plan& plan, int64_t M, bool want_cols) {
+  if (plan.resident) return 0;
+  if (plan.split > 1) return (size_t)M * ((size_t)plan.split + 1) * 2 * sizeof(float);
+  return want_cols ? (size_t)M * 2 * sizeof(float) : 0;
 }
 
 size_t norm_bwd_workspace(int op, int64_t M, int64_t N, int xd, int wd, int nparts) {
@@ -257,7 +261,7 @@ size_t norm_bwd_workspace(int op, int64_t M, int64_t N, int xd, int wd, int npar
                 &plan, false, op == ROWNORM_OP_LAYER_NORM_BWD, esize_of(wd) > esize_of(xd)))
     return 0;
   return (size_t)plan.partial_rows * (size_t)N * sizeof(float) * (size_t)nparts +
-         split_bytes(plan, M);
+         split_bytes(plan, M, nparts > 0);
 }
 
 // dres: the gradient reaching the normalized row by the residual path, added to dx (or null).
@@ -291,7 +295,8 @@ int norm_bwd(const void* dy, const void* x, const float* mean, const float* rstd
   NormBwdArgs a{dy, x, mean, rstd, gamma, dx, dgamma, dbeta, part_dg, part_db, M, (int)N};
   // the split-row dX takes its partial sums behind the column sums when the
   // caller brought the room for them; without it a row stays on one workgroup
-  if (dx && workspace && split_bytes(plan, M) > 0 && workspace_bytes >= need + split_bytes(plan, M))
+  if (dx && workspace && split_bytes(plan, M, want_cols) > 0 &&
+      workspace_bytes >= need + split_bytes(plan, M, want_cols))
     a.split_ws = (float*)((char*)workspace + need);
   hipStream_t s = (hipStream_t)stream;
   if (dres != nullptr && dx != nullptr) {

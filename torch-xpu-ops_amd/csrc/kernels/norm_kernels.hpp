@@ -609,6 +609,10 @@ norm_fwd_split_apply_kernel(const T* __restrict__ x, const T* res, const WT* __r
 // residual stream: the row was h = x + res and the loss also depends on h
 // directly), is added to dx in float32 before the one rounding of the store.
 // dres may be the memory of dx.
+//
+// PF (norm_bwd_prefetches()): the rows of the next iteration are requested
+// before the arithmetic, the reduction and the stores of the current one, and
+// wait in registers of their own.
 template <class T, class WT, int G, int V, int BLOCK, int R, bool RMS, bool FAST,
           bool ADD = false>
 __global__ void __launch_bounds__(BLOCK)
@@ -630,6 +634,7 @@ norm_bwd_resident_kernel(const T* __restrict__ dy, const T* __restrict__ x, cons
   const float inv_n = 1.0f / fN;
   const bool want_cols = part_dg != nullptr;  // uniform
   constexpr bool kWideWeights = V * E <= 16;  // few weights: widen to fp32 once, not per row
+  constexpr bool PF = R == 1 && norm_bwd_prefetches((int)sizeof(T), G, V, FAST, RMS);
 
   Pack<WT, E> gp[V];
   float dg[V][E];
@@ -647,26 +652,50 @@ norm_bwd_resident_kernel(const T* __restrict__ dy, const T* __restrict__ x, cons
   }
 
   const int64_t nrb = (M + RPI - 1) / RPI;
-  for (int64_t rb = blockIdx.x; rb < nrb; rb += gridDim.x) {
-    const int64_t row0 = (rb * RPB + slot) * R;
-    bool ok[R];
-    float mu[R], rs[R];
-    // A row slot past the end of the tensor gets all-zero x and dy, so it adds
-    // nothing to the column sums; its dx is not stored.
-    Pack<T, E> xp[R][V], dp[R][V];
+  // A row slot past the end of the tensor gets all-zero x and dy, so it adds
+  // nothing to the column sums; its dx is not stored.
+  bool ok[R];
+  float mu[R], rs[R];
+  Pack<T, E> xp[R][V], dp[R][V];
+  auto fetch = [&](int64_t rb, bool (&fok)[R], float (&fmu)[R], float (&frs)[R],
+                   Pack<T, E> (&fx)[R][V], Pack<T, E> (&fd)[R][V]) {
+    const int64_t frow0 = (rb * RPB + slot) * R;
+    if (PF && rb >= nrb) {  // uniform: nothing left to request (the values are never used)
+#pragma unroll
+      for (int r = 0; r < R; ++r) {
+        fok[r] = false;
+        fmu[r] = frs[r] = 0.0f;
+#pragma unroll
+        for (int c = 0; c < V; ++c) fx[r][c] = fd[r][c] = Pack<T, E>::zero();
+      }
+      return;
+    }
 #pragma unroll
     for (int r = 0; r < R; ++r) {
-      ok[r] = (RPI == 1) ? true : row0 + r < M;
-      const int64_t rowc = ok[r] ? row0 + r : 0;
-      mu[r] = RMS ? 0.0f : mean[rowc];
-      rs[r] = rstd[rowc];
+      fok[r] = (RPI == 1 && !PF) ? true : (rb < nrb && frow0 + r < M);
+      const int64_t rowc = fok[r] ? frow0 + r : 0;
+      fmu[r] = RMS ? 0.0f : mean[rowc];
+      frs[r] = rstd[rowc];
 #pragma unroll
       for (int c = 0; c < V; ++c) {
         const int e0 = (c * G + lane) * E;
-        xp[r][c] = row_load<T, E, true, FAST>(x + rowc * (int64_t)N, e0, N, ok[r], 0.0f);
-        dp[r][c] = row_load<T, E, true, FAST>(dy + rowc * (int64_t)N, e0, N, ok[r], 0.0f);
+        fx[r][c] = row_load<T, E, true, FAST>(x + rowc * (int64_t)N, e0, N, fok[r], 0.0f);
+        fd[r][c] = row_load<T, E, true, FAST>(dy + rowc * (int64_t)N, e0, N, fok[r], 0.0f);
       }
     }
+  };
+  if constexpr (PF) fetch(blockIdx.x, ok, mu, rs, xp, dp);
+  for (int64_t rb = blockIdx.x; rb < nrb; rb += gridDim.x) {
+    const int64_t row0 = (rb * RPB + slot) * R;
+    // PF: the rows of the next iteration are requested before this iteration's
+    // arithmetic, reduction and stores, and wait in registers of their own
+    bool okn[PF ? R : 1];
+    float mun[PF ? R : 1], rsn[PF ? R : 1];
+    Pack<T, E> xn[PF ? R : 1][PF ? V : 1], dn[PF ? R : 1][PF ? V : 1];
+    if constexpr (PF)
+      fetch(rb + gridDim.x, okn, mun, rsn, xn, dn);
+    else
+      fetch(rb, ok, mu, rs, xp, dp);
     float acc[2 * R];
 #pragma unroll
     for (int r = 0; r < R; ++r) {
@@ -737,6 +766,19 @@ norm_bwd_resident_kernel(const T* __restrict__ dy, const T* __restrict__ x, cons
             o.set(i, f);
           }
           row_store<T, E, true, FAST>(dr, (c * G + lane) * E, N, ok[r], o);
+        }
+      }
+    }
+    if constexpr (PF) {
+#pragma unroll
+      for (int r = 0; r < R; ++r) {
+        ok[r] = okn[r];
+        mu[r] = mun[r];
+        rs[r] = rsn[r];
+#pragma unroll
+        for (int c = 0; c < V; ++c) {
+          xp[r][c] = xn[r][c];
+          dp[r][c] = dn[r][c];
         }
       }
     }

@@ -119,17 +119,24 @@ int launch_norm_bwd(const Plan& plan, const NormBwdArgs& a, hipStream_t stream) 
   } else {
     constexpr int E = elems_per_pack<T>::value;
     bool cols_done = false;
-    if (a.dx != nullptr && a.split_ws != nullptr && plan.split > 1 && a.M <= 65535) {
-      const dim3 grid((unsigned)plan.split, (unsigned)a.M);
+    // the row sums s1, s2 go through memory when a row is split over workgroups,
+    // and also when it is not but the column sums are wanted: dX and the column
+    // sums then share the second pass over X and dY (two passes, not three)
+    const int chunks = plan.split > 1 ? plan.split : 1;
+    if (a.dx != nullptr && a.split_ws != nullptr && (chunks > 1 || want_cols) && a.M <= 65535) {
+      const dim3 grid((unsigned)chunks, (unsigned)a.M);
       hipLaunchKernelGGL((norm_bwd_split_sums_kernel<T, WT, kStreamBlock, RMS>), grid,
                          dim3(kStreamBlock), 0, stream, (const T*)a.dy, (const T*)a.x, a.mean,
                          a.rstd, (const WT*)a.gamma, a.split_ws, a.N, plan.chunk_packs);
       if (want_cols) {
         // dX and the column sums in one more pass over X and dY
         constexpr int CB = 256;
-        float* totals = a.split_ws + a.M * (int64_t)plan.split * 2;
-        hipLaunchKernelGGL((norm_bwd_split_totals_kernel<0>), dim3((unsigned)a.M), dim3(64), 0,
-                           stream, (const float*)a.split_ws, totals, plan.split);
+        float* totals = a.split_ws;  // one chunk a row: its sums are the totals
+        if (chunks > 1) {
+          totals = a.split_ws + a.M * (int64_t)chunks * 2;
+          hipLaunchKernelGGL((norm_bwd_split_totals_kernel<0>), dim3((unsigned)a.M), dim3(64), 0,
+                             stream, (const float*)a.split_ws, totals, chunks);
+        }
         const unsigned gx = (unsigned)((a.N + CB * E - 1) / (CB * E));
         hipLaunchKernelGGL((norm_bwd_split_dx_colsum_kernel<T, WT, CB, RMS>),
                            dim3(gx, (unsigned)plan.partial_rows), dim3(CB), 0, stream,

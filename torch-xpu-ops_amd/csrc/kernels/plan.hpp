@@ -101,6 +101,24 @@ constexpr int block_threads(OpClass oc, int G) {
   return G <= floor_threads ? floor_threads : G;
 }
 
+// Whether the resident norm backward requests the rows of its next iteration
+// ahead of the current one's arithmetic.  That costs V * 8 registers a lane for
+// 16-bit rows.  The two-pack layouts sit just under 128 registers, which keeps
+// two 512-thread workgroups on a compute unit, and lose more to a lost
+// workgroup than they gain (bf16 [16384, 4096] LayerNorm 78 -> 85 us; with the
+// dgamma/dbeta sums moved to LDS to make room, read-add-write 128 bits at a
+// time, 78 -> 82 us, and with LDS float atomics ten times that); from three packs
+// a lane the kernel holds one workgroup a compute unit anyway and has the
+// registers to spare (N = 10240: LayerNorm 208 -> 185 us, RMSNorm 189 -> 176 us;
+// with one workgroup a compute unit in the grid as well, see make_plan(), 173
+// and 169 us).  The two-pack LayerNorm, whose two sets of column sums make it
+// the slower one, gains a little from the prefetch on one workgroup a compute
+// unit up to 256 lanes (N = 2048: 44.6 -> 43.3 us, 4096: 78 -> 75 us) and loses a
+// little on 512 (N = 7168: 128 -> 130 us, 8192: 142 -> 144 us).
+constexpr bool norm_bwd_prefetches(int esize, int G, int V, bool fast, bool rms) {
+  return fast && esize == 2 && (V >= 3 || (V == 2 && !rms && G <= 256));
+}
+
 // Workgroup sizes a G-lane variant is compiled for.
 constexpr bool block_built(OpClass oc, int G, int block) {
   if (block < G || block < 256 || block > 1024 || (block & (block - 1))) return false;
@@ -196,12 +214,14 @@ inline int pow2_ceil(int64_t v) {
 //  * a row that fills at most three quarters of the slots takes three packs on a
 //    quarter of the slots' lanes instead: hidden sizes such as 1536, 3072, 6144,
 //    12288 fit exactly, 2560, 5120, 10240 to 83 % (16-bit forward 3-14 %, fp32
-//    LayerNorm backward 5-15 %).  The 16-bit backward below 1024 packs is the
-//    exception: its column sums want the lanes (N = 5120: 96 vs 109 us); so is
-//    the LayerNorm forward with fp32 weights below 512 lanes;
+//    LayerNorm backward 5-15 %).  The LayerNorm forward with fp32 weights below
+//    512 lanes is the exception, and so is the 16-bit backward below 512 packs;
 //  * fp32 LayerNorm forward rows of 2049..2560 packs: 512 lanes x 5 (N = 10240:
 //    261 -> 222 us).
 // Returns false where the general rule stands.
+#ifndef ROWNORM_BWD_SPARSE_MIN_G2
+#define ROWNORM_BWD_SPARSE_MIN_G2 512
+#endif
 inline bool norm_layout(OpClass oc, int esize, int64_t packs, bool layer_norm, bool wide_weights,
                         int* G_out, int* V_out) {
   const int vp = v_pref(oc, esize);
@@ -223,6 +243,11 @@ inline bool norm_layout(OpClass oc, int esize, int64_t packs, bool layer_norm, b
     } else if (fwd && sparse && !(layer_norm && wide_weights && G2 < 512)) {
       // (fp32 gamma and beta beside 16-bit rows: three packs of each are 48
       // registers, and below 512 lanes the two-pack layout stays ahead)
+      G = G2 / 2, V = 3;
+    } else if (!fwd && sparse && G2 >= ROWNORM_BWD_SPARSE_MIN_G2) {
+      // the backward with three packs a lane requests its next rows ahead:
+      // N = 5120: LayerNorm 95 -> 93 us, RMSNorm 92 -> 87 us; 6144: 112 -> 107 us
+      // and 108 -> 102 us
       G = G2 / 2, V = 3;
     }
   } else {
@@ -369,6 +394,12 @@ inline int make_plan(OpClass oc, int64_t M, int64_t N, int esize, int num_cus, c
   if (ov.bpc == 0 && oc == OC_NORM_FWD && p.resident && layer_norm && wide_weights &&
       p.block == 256)
     bpc /= 2;
+  // The backward that prefetches its next rows holds one workgroup a compute unit:
+  // a grid of that size halves the partial rows of the dgamma/dbeta reduction
+  // (bf16 [16384, 12288]: LayerNorm 222 -> 208 us, RMSNorm 210 -> 204 us)
+  if (ov.bpc == 0 && oc == OC_NORM_BWD && p.resident &&
+      norm_bwd_prefetches(esize, p.G, p.V, p.fast, !layer_norm))
+    bpc = 1;
   int64_t grid = (int64_t)num_cus * bpc;
   // The norm forward beyond a few tens of thousands of rows (measured on bf16 rows
   // of 2048..8192 elements, 65536 and 262144 rows): a workgroup that walks more
