@@ -660,16 +660,8 @@ norm_bwd_resident_kernel(const T* __restrict__ dy, const T* __restrict__ x, cons
   auto fetch = [&](int64_t rb, bool (&fok)[R], float (&fmu)[R], float (&frs)[R],
                    Pack<T, E> (&fx)[R][V], Pack<T, E> (&fd)[R][V]) {
     const int64_t frow0 = (rb * RPB + slot) * R;
-    if (PF && rb >= nrb) {  // uniform: nothing left to request (the values are never used)
-#pragma unroll
-      for (int r = 0; r < R; ++r) {
-        fok[r] = false;
-        fmu[r] = frs[r] = 0.0f;
-#pragma unroll
-        for (int c = 0; c < V; ++c) fx[r][c] = fd[r][c] = Pack<T, E>::zero();
-      }
-      return;
-    }
+    // (past the last row block the requests go to row 0 and are never used: a
+    // branch around them measured 10-15 % slower over the whole kernel)
 #pragma unroll
     for (int r = 0; r < R; ++r) {
       fok[r] = (RPI == 1 && !PF) ? true : (rb < nrb && frow0 + r < M);
