@@ -13,6 +13,7 @@
 // Here the access stays 128-bit wide for every pointer and only a row tail
 // shorter than one pack is moved element by element.
 #pragma once
+#include <type_traits>
 #include <hip/hip_runtime.h>
 #include <stdint.h>
 
@@ -176,6 +177,53 @@ __device__ __forceinline__ void store_row_pack(T* row, int e0, int n, bool row_o
 #pragma unroll
     for (int i = 0; i < E; ++i)
       if (e0 + i >= lo && e0 + i < n) row[e0 + i] = p.v[i];
+  }
+}
+
+// The packs p0 + t, p0 + t + BLOCK, ... below p1 of thread t, U at a time: the
+// loads of U packs are issued (`fetch`) before the first of them is used (`use`),
+// so a lane keeps U requests in flight instead of one.  Packs below `pfull` =
+// N / E lie wholly inside the row: for them the callbacks get std::true_type and
+// move plain 128-bit packs, straight-line code that the compiler can keep in
+// flight; a branch around a load (the ragged path of load_row_pack) stops that,
+// so only the last, ragged pack of a row (std::false_type) takes that path.
+//   fetch(pk, whole) -> data        use(pk, data, whole)
+template <int U, int BLOCK, class Fetch, class Use>
+__device__ __forceinline__ void for_packs(int64_t p0, int64_t p1, int64_t pfull, Fetch fetch,
+                                          Use use) {
+  const int64_t pe = p1 < pfull ? p1 : pfull;
+  int64_t pk = p0 + threadIdx.x;
+  using Data = decltype(fetch(pk, std::true_type{}));
+  for (; pk + (int64_t)(U - 1) * BLOCK < pe; pk += (int64_t)U * BLOCK) {
+    Data d[U];
+#pragma unroll
+    for (int u = 0; u < U; ++u) d[u] = fetch(pk + (int64_t)u * BLOCK, std::true_type{});
+#pragma unroll
+    for (int u = 0; u < U; ++u) use(pk + (int64_t)u * BLOCK, d[u], std::true_type{});
+  }
+  for (; pk < pe; pk += BLOCK) use(pk, fetch(pk, std::true_type{}), std::true_type{});
+  for (; pk < p1; pk += BLOCK) use(pk, fetch(pk, std::false_type{}), std::false_type{});
+}
+
+// One pack of a row of n elements at element e0: a plain 128-bit access when the
+// caller knows it lies inside the row (WHOLE), load_row_pack / store_row_pack otherwise.
+template <class T, int E, bool STREAM, bool WHOLE>
+__device__ __forceinline__ Pack<T, E> load_pack_of(const T* row, int64_t e0, int n, float fill) {
+  if constexpr (WHOLE)
+    return STREAM ? Pack<T, E>::load_stream(row + e0) : Pack<T, E>::load(row + e0);
+  else
+    return load_row_pack<T, E, STREAM>(row, (int)e0, n, true, fill);
+}
+
+template <class T, int E, bool STREAM, bool WHOLE>
+__device__ __forceinline__ void store_pack_of(T* row, int64_t e0, int n, const Pack<T, E>& p) {
+  if constexpr (WHOLE) {
+    if (STREAM)
+      p.store_stream(row + e0);
+    else
+      p.store(row + e0);
+  } else {
+    store_row_pack<T, E, STREAM>(row, (int)e0, n, true, p);
   }
 }
 

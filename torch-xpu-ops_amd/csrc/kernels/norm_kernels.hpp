@@ -313,17 +313,115 @@ __device__ __forceinline__ float split_row_centre(const T* xr, const T* rr, int 
   return fmaxf(fminf(a, b), fminf(fmaxf(a, b), c));
 }
 
-// One pack of the row the long-row kernels normalize: x, or x + res (formed in
-// float32, rounded once to T) when a residual row is given.
-template <class T, int E, bool STREAM>
-__device__ __forceinline__ Pack<T, E> load_sum_pack(const T* xr, const T* rr, int e0, int n) {
-  Pack<T, E> p = load_row_pack<T, E, STREAM>(xr, e0, n, true, 0.0f);
-  if (rr != nullptr) {
-    const Pack<T, E> q = load_row_pack<T, E, STREAM>(rr, e0, n, true, 0.0f);
+// Packs a lane of the long-row kernels requests before it uses the first.
+constexpr int kLongRowUnroll = 4;
+
+// What a lane of the long-row forward holds of one pack between request and use.
+template <class T, class WT, int E>
+struct LongRowIn {
+  Pack<T, E> x, r;   // the row and the residual row (r only with a residual)
+  Pack<WT, E> g, b;  // gamma, beta (output pass only)
+};
+
+// x, or x + res formed in float32 and rounded once to T.
+template <class T, int E, bool HASRES>
+__device__ __forceinline__ Pack<T, E> sum_pack_of(const Pack<T, E>& x, const Pack<T, E>& r) {
+  if constexpr (!HASRES) return x;
+  Pack<T, E> p;
 #pragma unroll
-    for (int i = 0; i < E; ++i) p.set(i, p.get(i) + q.get(i));
-  }
+  for (int i = 0; i < E; ++i) p.set(i, x.get(i) + r.get(i));
   return p;
+}
+
+// Adds sum(x - k) and sum((x - k)^2) of one pack (its first `nvalid` elements when
+// !WHOLE) to the float64 sums.  float32 rows: every term in float64, where the
+// differences are exact.  16-bit rows: x - k is exact in float32 already (unless
+// |k| is 2^16 times |x|), and the terms of a pack are added in float32 before they
+// join the float64 sums: a quarter of the float64 instructions (they made the
+// sums pass arithmetic-bound), and the rounding of a pack's sums -- 2^-24
+// relative, independent from pack to pack -- stays orders below the 16-bit
+// tolerance even when k lies a thousand standard deviations from the row.
+template <class T, int E, bool RMS, bool WHOLE>
+__device__ __forceinline__ void add_centred_sums(const Pack<T, E>& p, int nvalid, float kf,
+                                                 double kd, double& s1, double& s2) {
+  if constexpr (sizeof(T) == 2) {
+    float t1 = 0.0f, t2 = 0.0f;
+#pragma unroll
+    for (int i = 0; i < E; ++i) {
+      float d = p.get(i) - kf;
+      if constexpr (!WHOLE) d = (i < nvalid) ? d : 0.0f;
+      if constexpr (!RMS) t1 += d;
+      t2 = fmaf(d, d, t2);
+    }
+    if constexpr (!RMS) s1 += (double)t1;
+    s2 += (double)t2;
+  } else {
+#pragma unroll
+    for (int i = 0; i < E; ++i) {
+      double d = (double)p.get(i) - kd;
+      if constexpr (!WHOLE) d = (i < nvalid) ? d : 0.0;
+      if constexpr (!RMS) s1 += d;
+      s2 = fma(d, d, s2);
+    }
+  }
+}
+
+// sum(x - k), sum((x - k)^2) over the packs [p0, p1) of a thread (see for_packs).
+template <class T, int E, int BLOCK, bool RMS, bool HASRES>
+__device__ __forceinline__ void long_row_sums(const T* xr, const T* rr, int N, int64_t p0,
+                                              int64_t p1, float kf, double& s1, double& s2) {
+  const double kd = (double)kf;
+  for_packs<kLongRowUnroll, BLOCK>(
+      p0, p1, (int64_t)(N / E),
+      [&](int64_t pk, auto whole) {
+        constexpr bool W = decltype(whole)::value;
+        LongRowIn<T, T, E> d;
+        d.x = load_pack_of<T, E, false, W>(xr, pk * E, N, 0.0f);
+        if constexpr (HASRES) d.r = load_pack_of<T, E, false, W>(rr, pk * E, N, 0.0f);
+        return d;
+      },
+      [&](int64_t pk, const LongRowIn<T, T, E>& d, auto whole) {
+        constexpr bool W = decltype(whole)::value;
+        add_centred_sums<T, E, RMS, W>(sum_pack_of<T, E, HASRES>(d.x, d.r), N - (int)(pk * E), kf,
+                                       kd, s1, s2);
+      });
+}
+
+// y = gamma * ((x - hi) - lo) * rs + beta (RMSNorm: gamma * x * rs) over the packs
+// [p0, p1) of a thread; with a residual row the normalized row is h = x + res,
+// written out as well.
+template <class T, class WT, class TY, int E, int BLOCK, bool RMS, bool HASRES>
+__device__ __forceinline__ void long_row_apply(const T* xr, const T* rr, const WT* gamma,
+                                               const WT* beta, T* hr, TY* yr, int N, int64_t p0,
+                                               int64_t p1, float hi, float lo, float rs) {
+  const bool hg = gamma != nullptr, hb = !RMS && beta != nullptr;  // uniform over the launch
+  for_packs<kLongRowUnroll, BLOCK>(
+      p0, p1, (int64_t)(N / E),
+      [&](int64_t pk, auto whole) {
+        constexpr bool W = decltype(whole)::value;
+        LongRowIn<T, WT, E> d;
+        d.x = load_pack_of<T, E, true, W>(xr, pk * E, N, 0.0f);
+        if constexpr (HASRES) d.r = load_pack_of<T, E, true, W>(rr, pk * E, N, 0.0f);
+        d.g = hg ? load_pack_of<WT, E, false, W>(gamma, pk * E, N, 1.0f) : Pack<WT, E>::splat(1.0f);
+        d.b = hb ? load_pack_of<WT, E, false, W>(beta, pk * E, N, 0.0f) : Pack<WT, E>::zero();
+        return d;
+      },
+      [&](int64_t pk, const LongRowIn<T, WT, E>& d, auto whole) {
+        constexpr bool W = decltype(whole)::value;
+        const Pack<T, E> p = sum_pack_of<T, E, HASRES>(d.x, d.r);
+        if constexpr (HASRES) store_pack_of<T, E, true, W>(hr, pk * E, N, p);
+        Pack<TY, E> o;
+#pragma unroll
+        for (int i = 0; i < E; ++i) {
+          float v;
+          if constexpr (RMS)
+            v = (p.get(i) * rs) * d.g.get(i);
+          else
+            v = (((p.get(i) - hi) - lo) * rs) * d.g.get(i) + d.b.get(i);
+          o.set(i, v);
+        }
+        store_pack_of<TY, E, true, W>(yr, pk * E, N, o);
+      });
 }
 
 // ---------------------------------------------------------------------------
@@ -356,27 +454,23 @@ norm_fwd_stream_kernel(const T* __restrict__ x, const T* res, const WT* __restri
     // apart so that the rounding of the saved mean never enters y
     float hi = 0.0f, lo = 0.0f, rs;
     if constexpr (RMS) {
-      float acc[1] = {0.0f};
-      for (int pk = threadIdx.x; pk < npacks; pk += BLOCK) {
-        const Pack<T, E> p = load_sum_pack<T, E, false>(xr, rr, pk * E, N);
-#pragma unroll
-        for (int i = 0; i < E; ++i) acc[0] = fmaf(p.get(i), p.get(i), acc[0]);
-      }
+      // (float64 partial sums of float32 pack sums: see add_centred_sums)
+      double s1 = 0.0, s2 = 0.0;
+      if (rr != nullptr)
+        long_row_sums<T, E, BLOCK, true, true>(xr, rr, N, 0, npacks, 0.0f, s1, s2);
+      else
+        long_row_sums<T, E, BLOCK, true, false>(xr, rr, N, 0, npacks, 0.0f, s1, s2);
+      float acc[1] = {(float)s2};
       group_allreduce<BLOCK, BLOCK, 1, SumOp>(acc, red, phase);
       rs = 1.0f / sqrtf(acc[0] / fN + eps);  // once a row of >= 32 Ki elements: exact
     } else {
-      const double k = (double)split_row_centre(xr, rr, N);
+      const float kf = split_row_centre(xr, rr, N);
+      const double k = (double)kf;
       double s1 = 0.0, s2 = 0.0;
-      for (int pk = threadIdx.x; pk < npacks; pk += BLOCK) {
-        const Pack<T, E> p = load_sum_pack<T, E, false>(xr, rr, pk * E, N);
-        const int nvalid = N - pk * E;
-#pragma unroll
-        for (int i = 0; i < E; ++i) {
-          const double d = (i < nvalid) ? (double)p.get(i) - k : 0.0;
-          s1 += d;
-          s2 = fma(d, d, s2);
-        }
-      }
+      if (rr != nullptr)
+        long_row_sums<T, E, BLOCK, false, true>(xr, rr, N, 0, npacks, kf, s1, s2);
+      else
+        long_row_sums<T, E, BLOCK, false, false>(xr, rr, N, 0, npacks, kf, s1, s2);
       block_sum2_f64<BLOCK>(s1, s2, red64);
       if (threadIdx.x == 0) {
         const double dN = (double)N;
@@ -396,27 +490,13 @@ norm_fwd_stream_kernel(const T* __restrict__ x, const T* res, const WT* __restri
     // (h may lie on top of x or res: the block reduction above is a barrier, so every
     // thread has finished the first pass before any of h is written; a thread then
     // reads and writes the same elements)
-    for (int pk = threadIdx.x; pk < npacks; pk += BLOCK) {
-      const int e0 = pk * E;
-      const Pack<T, E> p = load_sum_pack<T, E, true>(xr, rr, e0, N);
-      if (rr != nullptr) store_row_pack<T, E, true>(h + row * (int64_t)N, e0, N, true, p);
-      const Pack<WT, E> pg = gamma ? load_row_pack<WT, E, false>(gamma, e0, N, true, 1.0f)
-                                   : Pack<WT, E>::splat(1.0f);
-      Pack<WT, E> pb = Pack<WT, E>::zero();
-      if constexpr (!RMS)
-        if (beta) pb = load_row_pack<WT, E, false>(beta, e0, N, true, 0.0f);
-      Pack<TY, E> o;
-#pragma unroll
-      for (int i = 0; i < E; ++i) {
-        float v;
-        if constexpr (RMS)
-          v = (p.get(i) * rs) * pg.get(i);
-        else
-          v = (((p.get(i) - hi) - lo) * rs) * pg.get(i) + pb.get(i);
-        o.set(i, v);
-      }
-      store_row_pack<TY, E, true>(yr, e0, N, true, o);
-    }
+    T* hr = rr != nullptr ? h + row * (int64_t)N : nullptr;
+    if (rr != nullptr)
+      long_row_apply<T, WT, TY, E, BLOCK, RMS, true>(xr, rr, gamma, beta, hr, yr, N, 0, npacks, hi,
+                                                     lo, rs);
+    else
+      long_row_apply<T, WT, TY, E, BLOCK, RMS, false>(xr, rr, gamma, beta, hr, yr, N, 0, npacks,
+                                                      hi, lo, rs);
     if (threadIdx.x == 0) {
       if constexpr (!RMS)
         if (mean) mean[row] = rs == rs ? hi : rs;  // NaN variance: NaN mean
@@ -485,19 +565,12 @@ norm_fwd_split_sums_kernel(const T* __restrict__ x, const T* res, TY* __restrict
   const int64_t npacks = ((int64_t)N + E - 1) / E;
   int64_t p0, p1;
   split_chunk_range(blockIdx.x, gridDim.x, chunk_packs, npacks, &p0, &p1);
-  const double k = RMS ? 0.0 : (double)split_row_centre(xr, rr, N);
+  const float kf = RMS ? 0.0f : split_row_centre(xr, rr, N);
   double s1 = 0.0, s2 = 0.0;
-  for (int64_t pk = p0 + threadIdx.x; pk < p1; pk += BLOCK) {
-    const int e0 = (int)(pk * E);
-    const Pack<T, E> p = load_sum_pack<T, E, false>(xr, rr, e0, N);
-    const int nvalid = N - e0;
-#pragma unroll
-    for (int i = 0; i < E; ++i) {
-      const double d = (i < nvalid) ? (double)p.get(i) - k : 0.0;
-      if constexpr (!RMS) s1 += d;
-      s2 = fma(d, d, s2);
-    }
-  }
+  if (rr != nullptr)
+    long_row_sums<T, E, BLOCK, RMS, true>(xr, rr, N, p0, p1, kf, s1, s2);
+  else
+    long_row_sums<T, E, BLOCK, RMS, false>(xr, rr, N, p0, p1, kf, s1, s2);
   block_sum2_f64<BLOCK>(s1, s2, red);
   if (threadIdx.x == 0) {
     double* slot = split_chunk_slot(y + row * (int64_t)N, p0, E);
@@ -570,27 +643,13 @@ norm_fwd_split_apply_kernel(const T* __restrict__ x, const T* res, const WT* __r
   // the low part of the mean sits where this workgroup is about to write y
   const float lo = RMS ? 0.0f : *reinterpret_cast<const float*>(split_chunk_slot(yr, p0, E));
   __syncthreads();
-  for (int64_t pk = p0 + threadIdx.x; pk < p1; pk += BLOCK) {
-    const int e0 = (int)(pk * E);
-    const Pack<T, E> p = load_sum_pack<T, E, true>(xr, rr, e0, N);
-    if (rr != nullptr) store_row_pack<T, E, true>(h + row * (int64_t)N, e0, N, true, p);
-    const Pack<WT, E> pg = gamma ? load_row_pack<WT, E, false>(gamma, e0, N, true, 1.0f)
-                                 : Pack<WT, E>::splat(1.0f);
-    Pack<WT, E> pb = Pack<WT, E>::zero();
-    if constexpr (!RMS)
-      if (beta) pb = load_row_pack<WT, E, false>(beta, e0, N, true, 0.0f);
-    Pack<TY, E> o;
-#pragma unroll
-    for (int i = 0; i < E; ++i) {
-      float v;
-      if constexpr (RMS)
-        v = (p.get(i) * rs) * pg.get(i);
-      else
-        v = (((p.get(i) - hi) - lo) * rs) * pg.get(i) + pb.get(i);
-      o.set(i, v);
-    }
-    store_row_pack<TY, E, true>(yr, e0, N, true, o);
-  }
+  T* hr = rr != nullptr ? h + row * (int64_t)N : nullptr;
+  if (rr != nullptr)
+    long_row_apply<T, WT, TY, E, BLOCK, RMS, true>(xr, rr, gamma, beta, hr, yr, N, p0, p1, hi, lo,
+                                                   rs);
+  else
+    long_row_apply<T, WT, TY, E, BLOCK, RMS, false>(xr, rr, gamma, beta, hr, yr, N, p0, p1, hi, lo,
+                                                    rs);
 }
 
 // ---------------------------------------------------------------------------
@@ -838,6 +897,76 @@ norm_bwd_resident_kernel(const T* __restrict__ dy, const T* __restrict__ x, cons
   }
 }
 
+// What a lane of the long-row backward holds of one pack between request and use.
+template <class T, class WT, int E>
+struct LongRowBwdIn {
+  Pack<T, E> x, dy, u;  // u: the gradient from the residual path (only with one)
+  Pack<WT, E> g;
+};
+
+// acc[0] += sum dy*gamma, acc[1] += sum dy*gamma*xhat over the packs [p0, p1) of a thread.
+template <class T, class WT, int E, int BLOCK, bool RMS>
+__device__ __forceinline__ void long_row_bwd_sums(const T* xr, const T* gr, const WT* gamma, int N,
+                                                  int64_t p0, int64_t p1, float mu, float rs,
+                                                  float (&acc)[2]) {
+  const bool hg = gamma != nullptr;  // uniform over the launch
+  for_packs<kLongRowUnroll, BLOCK>(
+      p0, p1, (int64_t)(N / E),
+      [&](int64_t pk, auto whole) {
+        constexpr bool W = decltype(whole)::value;
+        LongRowBwdIn<T, WT, E> d;
+        d.x = load_pack_of<T, E, false, W>(xr, pk * E, N, 0.0f);
+        d.dy = load_pack_of<T, E, false, W>(gr, pk * E, N, 0.0f);
+        d.g = hg ? load_pack_of<WT, E, false, W>(gamma, pk * E, N, 1.0f) : Pack<WT, E>::splat(1.0f);
+        return d;
+      },
+      [&](int64_t, const LongRowBwdIn<T, WT, E>& d, auto) {
+#pragma unroll
+        for (int i = 0; i < E; ++i) {
+          const float g = d.dy.get(i) * d.g.get(i);
+          acc[0] += g;
+          acc[1] = fmaf(g, (d.x.get(i) - mu) * rs, acc[1]);
+        }
+      });
+}
+
+// dx = (rs/N) * (N*gamma*dy - xhat*s2 - s1) (+ the residual path's gradient) over the
+// packs [p0, p1) of a thread.
+template <class T, class WT, int E, int BLOCK, bool RMS, bool HASRES>
+__device__ __forceinline__ void long_row_bwd_dx(const T* xr, const T* gr, const T* ur,
+                                                const WT* gamma, T* dr, int N, int64_t p0,
+                                                int64_t p1, float mu, float rs, float s1,
+                                                float s2) {
+  const bool hg = gamma != nullptr;  // uniform over the launch
+  const float fN = (float)N;
+  const float term1 = rs / fN;
+  for_packs<kLongRowUnroll, BLOCK>(
+      p0, p1, (int64_t)(N / E),
+      [&](int64_t pk, auto whole) {
+        constexpr bool W = decltype(whole)::value;
+        LongRowBwdIn<T, WT, E> d;
+        d.x = load_pack_of<T, E, true, W>(xr, pk * E, N, 0.0f);
+        d.dy = load_pack_of<T, E, true, W>(gr, pk * E, N, 0.0f);
+        if constexpr (HASRES) d.u = load_pack_of<T, E, true, W>(ur, pk * E, N, 0.0f);
+        d.g = hg ? load_pack_of<WT, E, false, W>(gamma, pk * E, N, 1.0f) : Pack<WT, E>::splat(1.0f);
+        return d;
+      },
+      [&](int64_t pk, const LongRowBwdIn<T, WT, E>& d, auto whole) {
+        constexpr bool W = decltype(whole)::value;
+        Pack<T, E> o;
+#pragma unroll
+        for (int i = 0; i < E; ++i) {
+          float f = fN * (d.dy.get(i) * d.g.get(i));
+          f -= ((d.x.get(i) - mu) * rs) * s2;
+          if constexpr (!RMS) f -= s1;
+          f *= term1;
+          if constexpr (HASRES) f += d.u.get(i);
+          o.set(i, f);
+        }
+        store_pack_of<T, E, true, W>(dr, pk * E, N, o);
+      });
+}
+
 // ---------------------------------------------------------------------------
 // Backward dX for rows too wide for registers: one workgroup per row, two
 // streaming passes over X and dY (sums, then dX).
@@ -849,7 +978,6 @@ norm_bwd_stream_dx_kernel(const T* __restrict__ dy, const T* __restrict__ x, con
   constexpr int E = elems_per_pack<T>::value;
   __shared__ float red[reduce_lds_floats<BLOCK, BLOCK, 2>::value];
   int phase = 0;
-  const float fN = (float)N;
   const int npacks = (N + E - 1) / E;
   for (int64_t row = blockIdx.x; row < M; row += gridDim.x) {
     const T* xr = x + row * (int64_t)N;
@@ -858,39 +986,14 @@ norm_bwd_stream_dx_kernel(const T* __restrict__ dy, const T* __restrict__ x, con
     const float mu = RMS ? 0.0f : mean[row];
     const float rs = rstd[row];
     float acc[2] = {0.0f, 0.0f};
-    for (int pk = threadIdx.x; pk < npacks; pk += BLOCK) {
-      const int e0 = pk * E;
-      const Pack<T, E> px = load_row_pack<T, E, false>(xr, e0, N, true, 0.0f);
-      const Pack<T, E> pd = load_row_pack<T, E, false>(gr, e0, N, true, 0.0f);
-      const Pack<WT, E> pg = gamma ? load_row_pack<WT, E, false>(gamma, e0, N, true, 1.0f)
-                                   : Pack<WT, E>::splat(1.0f);
-#pragma unroll
-      for (int i = 0; i < E; ++i) {
-        const float g = pd.get(i) * pg.get(i);
-        acc[0] += g;
-        acc[1] = fmaf(g, (px.get(i) - mu) * rs, acc[1]);
-      }
-    }
+    long_row_bwd_sums<T, WT, E, BLOCK, RMS>(xr, gr, gamma, N, 0, npacks, mu, rs, acc);
     group_allreduce<BLOCK, BLOCK, 2, SumOp>(acc, red, phase);
-    const float term1 = rs / fN;
-    for (int pk = threadIdx.x; pk < npacks; pk += BLOCK) {
-      const int e0 = pk * E;
-      const Pack<T, E> px = load_row_pack<T, E, true>(xr, e0, N, true, 0.0f);
-      const Pack<T, E> pd = load_row_pack<T, E, true>(gr, e0, N, true, 0.0f);
-      const Pack<WT, E> pg = gamma ? load_row_pack<WT, E, false>(gamma, e0, N, true, 1.0f)
-                                   : Pack<WT, E>::splat(1.0f);
-      Pack<T, E> pu = Pack<T, E>::zero();  // the gradient from the residual path, if any
-      if (dres != nullptr) pu = load_row_pack<T, E, true>(dres + row * (int64_t)N, e0, N, true, 0.0f);
-      Pack<T, E> o;
-#pragma unroll
-      for (int i = 0; i < E; ++i) {
-        float f = fN * (pd.get(i) * pg.get(i));
-        f -= ((px.get(i) - mu) * rs) * acc[1];
-        if constexpr (!RMS) f -= acc[0];
-        o.set(i, f * term1 + pu.get(i));
-      }
-      store_row_pack<T, E, true>(dr, e0, N, true, o);
-    }
+    if (dres != nullptr)
+      long_row_bwd_dx<T, WT, E, BLOCK, RMS, true>(xr, gr, dres + row * (int64_t)N, gamma, dr, N, 0,
+                                                  npacks, mu, rs, acc[0], acc[1]);
+    else
+      long_row_bwd_dx<T, WT, E, BLOCK, RMS, false>(xr, gr, nullptr, gamma, dr, N, 0, npacks, mu, rs,
+                                                   acc[0], acc[1]);
   }
 }
 
@@ -916,19 +1019,7 @@ norm_bwd_split_sums_kernel(const T* __restrict__ dy, const T* __restrict__ x,
   const float mu = RMS ? 0.0f : mean[row];
   const float rs = rstd[row];
   float acc[2] = {0.0f, 0.0f};
-  for (int64_t pk = p0 + threadIdx.x; pk < p1; pk += BLOCK) {
-    const int e0 = (int)(pk * E);
-    const Pack<T, E> px = load_row_pack<T, E, false>(xr, e0, N, true, 0.0f);
-    const Pack<T, E> pd = load_row_pack<T, E, false>(gr, e0, N, true, 0.0f);
-    const Pack<WT, E> pg = gamma ? load_row_pack<WT, E, false>(gamma, e0, N, true, 1.0f)
-                                 : Pack<WT, E>::splat(1.0f);
-#pragma unroll
-    for (int i = 0; i < E; ++i) {
-      const float g = pd.get(i) * pg.get(i);
-      acc[0] += g;
-      acc[1] = fmaf(g, (px.get(i) - mu) * rs, acc[1]);
-    }
-  }
+  long_row_bwd_sums<T, WT, E, BLOCK, RMS>(xr, gr, gamma, N, p0, p1, mu, rs, acc);
   group_allreduce<BLOCK, BLOCK, 2, SumOp>(acc, red, phase);
   if (threadIdx.x == 0) {
     float* sc = split_ws + (row * gridDim.x + blockIdx.x) * 2;
@@ -963,26 +1054,12 @@ norm_bwd_split_dx_kernel(const T* __restrict__ dy, const T* __restrict__ x, cons
     acc[1] = sc[1];
   }
   group_allreduce<BLOCK, BLOCK, 2, SumOp>(acc, red, phase);
-  const float fN = (float)N;
-  const float term1 = rs / fN;
-  for (int64_t pk = p0 + threadIdx.x; pk < p1; pk += BLOCK) {
-    const int e0 = (int)(pk * E);
-    const Pack<T, E> px = load_row_pack<T, E, true>(xr, e0, N, true, 0.0f);
-    const Pack<T, E> pd = load_row_pack<T, E, true>(gr, e0, N, true, 0.0f);
-    const Pack<WT, E> pg = gamma ? load_row_pack<WT, E, false>(gamma, e0, N, true, 1.0f)
-                                 : Pack<WT, E>::splat(1.0f);
-    Pack<T, E> pu = Pack<T, E>::zero();
-    if (dres != nullptr) pu = load_row_pack<T, E, true>(dres + row * (int64_t)N, e0, N, true, 0.0f);
-    Pack<T, E> o;
-#pragma unroll
-    for (int i = 0; i < E; ++i) {
-      float f = fN * (pd.get(i) * pg.get(i));
-      f -= ((px.get(i) - mu) * rs) * acc[1];
-      if constexpr (!RMS) f -= acc[0];
-      o.set(i, f * term1 + pu.get(i));
-    }
-    store_row_pack<T, E, true>(dr, e0, N, true, o);
-  }
+  if (dres != nullptr)
+    long_row_bwd_dx<T, WT, E, BLOCK, RMS, true>(xr, gr, dres + row * (int64_t)N, gamma, dr, N, p0,
+                                                p1, mu, rs, acc[0], acc[1]);
+  else
+    long_row_bwd_dx<T, WT, E, BLOCK, RMS, false>(xr, gr, nullptr, gamma, dr, N, p0, p1, mu, rs,
+                                                 acc[0], acc[1]);
 }
 
 // Split-row backward when dgamma / dbeta are wanted as well: one wavefront per
