@@ -197,7 +197,7 @@ def main():
         try:
             with open(traffic_file) as f:
                 out["roofline"]["traffic"] = json.load(f).get("hbm_bytes_per_launch")
-            out["roofline"]["traffic_source"] = "profiles/rms_norm_bf16_16384x4096_hbm_traffic.md"
+            out["roofline"]["traffic_source"] = "profiles/hbm_traffic_by_op.md"
         except Exception:
             pass
 
