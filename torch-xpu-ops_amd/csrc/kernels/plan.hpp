@@ -175,8 +175,10 @@ constexpr bool variant_built(OpClass oc, int esize, int G, int V, bool fast) {
     if (oc == OC_SOFTMAX_FWD && esize == 2) return G == kMaxG || (G >= 64 && V == 3);
     if (oc == OC_SOFTMAX_FWD || oc == OC_SOFTMAX_BWD) return G == kMaxG;
     // LayerNorm / RMSNorm rows of hidden sizes such as 5120, 6144, 10240, 12288
-    // (640, 768, 1280, 1536 16-bit packs): 3 or 5 packs a lane
-    if (!is_group_class(oc)) return G >= 64 && (V == 3 || V == 5);
+    // (640, 768, 1280, 1536 16-bit packs): 3 packs a lane; 5 on 512 lanes for the
+    // fp32 LayerNorm forward (see norm_layout())
+    if (!is_group_class(oc))
+      return G >= 64 && (V == 3 || (V == 5 && oc == OC_NORM_FWD && esize == 4 && G == 512));
     // (and 6..10 packs on 512 lanes, which make_plan() prefers to 1024 lanes)
     return G == kMaxG || (G >= 64 && (V == 3 || V == 5)) ||
            (G == 512 && V <= group_half_lanes_max_v(oc));
@@ -194,7 +196,13 @@ constexpr bool variant_built(OpClass oc, int esize, int G, int V, bool fast) {
   if ((oc == OC_NORM_FWD || oc == OC_NORM_BWD || oc == OC_SOFTMAX_FWD || oc == OC_SOFTMAX_BWD) &&
       G <= 64 && V == 1)
     return true;
-  return V >= v_pref(oc, esize);
+  if (is_group_class(oc) || G == kMaxG) return V >= v_pref(oc, esize);
+  // below the lane maximum make_plan() takes the preferred packs a lane (more lanes
+  // before more packs), with one measured exception: 16-bit norm rows of 1537..2048
+  // packs on 512 lanes x 4.  Other layouts are never selected and are not compiled
+  // (a third of the kernels otherwise).
+  if ((oc == OC_NORM_FWD || oc == OC_NORM_BWD) && esize == 2 && G == 512 && V == 4) return true;
+  return V == v_pref(oc, esize);
 #endif
 }
 
