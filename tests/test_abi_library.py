@@ -262,14 +262,19 @@ def test_group_norm_rows_take_512_lanes_while_two_workgroups_fit(cabi):
 
 def test_forward_grid_grows_with_the_row_count(cabi):
     """The norm forward keeps a workgroup to about 2 (RMSNorm) / 4 (LayerNorm) row blocks, twice
-    that with fp32 weights beside 16-bit rows, once the rows outgrow four resident grids."""
+    that with fp32 weights beside 16-bit rows, once the rows outgrow four resident grids; LayerNorm
+    with fp32 weights beside 16-bit rows takes a grid of two or three resident workgroups a compute
+    unit while that means at most 32 row blocks a workgroup."""
     BF, F32 = cabi.BF16, cabi.F32
     grid = lambda op, M, N, wd=BF: cabi.plan(op, M, N, BF, wd)["grid_blocks"]
     assert grid(cabi.OP_RMS_NORM_FWD, 16384, 4096) == 8192       # 256 CUs x 32: the floor
-    assert grid(cabi.OP_LAYER_NORM_FWD, 16384, 8192, F32) == 4096
     assert grid(cabi.OP_LAYER_NORM_FWD, 16384, 4096) == 8192
-    assert grid(cabi.OP_LAYER_NORM_FWD, 16384, 4096, F32) == 4096  # fp32 weights: half the floor
     assert grid(cabi.OP_RMS_NORM_FWD, 16384, 4096, F32) == 8192
+    assert grid(cabi.OP_LAYER_NORM_FWD, 16384, 8192, F32) == 512   # 256 CUs x two 512-thread workgroups
+    assert grid(cabi.OP_LAYER_NORM_FWD, 16384, 4096, F32) == 768   # x three 256-thread workgroups
+    assert grid(cabi.OP_LAYER_NORM_FWD, 300, 4096, F32) == 300     # never more workgroups than row blocks
+    assert grid(cabi.OP_LAYER_NORM_FWD, 24576, 4096, F32) == 768   # 32 row blocks a workgroup: the last
+    assert grid(cabi.OP_LAYER_NORM_FWD, 24577, 4096, F32) == 4096
     assert grid(cabi.OP_RMS_NORM_FWD, 65536, 4096) == 32768
     assert grid(cabi.OP_LAYER_NORM_FWD, 65536, 4096) == 16384
     assert grid(cabi.OP_LAYER_NORM_FWD, 65536, 4096, F32) == 8192
