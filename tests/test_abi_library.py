@@ -269,7 +269,9 @@ def test_forward_grid_grows_with_the_row_count(cabi):
     grid = lambda op, M, N, wd=BF: cabi.plan(op, M, N, BF, wd)["grid_blocks"]
     assert grid(cabi.OP_RMS_NORM_FWD, 16384, 4096) == 8192       # 256 CUs x 32: the floor
     assert grid(cabi.OP_LAYER_NORM_FWD, 16384, 4096) == 8192
-    assert grid(cabi.OP_RMS_NORM_FWD, 16384, 4096, F32) == 8192
+    assert grid(cabi.OP_RMS_NORM_FWD, 16384, 4096, F32) == 768     # fp32 weights: three resident workgroups
+    assert grid(cabi.OP_LAYER_NORM_FWD, 16384, 8192) == 512        # LayerNorm on 512 lanes: two
+    assert grid(cabi.OP_RMS_NORM_FWD, 16384, 8192) == 8192
     assert grid(cabi.OP_LAYER_NORM_FWD, 16384, 8192, F32) == 512   # 256 CUs x two 512-thread workgroups
     assert grid(cabi.OP_LAYER_NORM_FWD, 16384, 4096, F32) == 768   # x three 256-thread workgroups
     assert grid(cabi.OP_LAYER_NORM_FWD, 300, 4096, F32) == 300     # never more workgroups than row blocks

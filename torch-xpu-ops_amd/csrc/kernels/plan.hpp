@@ -419,23 +419,27 @@ inline int make_plan(OpClass oc, int64_t M, int64_t N, int esize, int num_cus, c
     const int iters = (layer_norm ? 4 : 2) * (wide_weights ? 2 : 1);
     const int64_t want = (nrb + iters - 1) / iters;
     if (grid < want) grid = want;
-    // LayerNorm with fp32 weights beside 16-bit rows, up to a few tens of thousands
-    // of rows: three 256-thread or two 512-thread workgroups a compute unit (four of
-    // 256 measured 6 % slower than three at N = 6144, where a lane holds three packs
-    // of each weight), all resident at once, each walking up to 32 row blocks -- the
-    // 2 * N * 4 bytes of weights are loaded once per 4..32 rows and no second wave of
-    // workgroups leaves a tail.  bf16 rows, grid-size sweeps at 2048 / 4096 / 16384
-    // rows: N = 4096 9.8 / 17.4 / 48.9 -> 8.2 / 13.5 / 46.0 us, N = 8192 17.7 / 33.2 / 93.3
-    // -> 14.2 / 24.3 / 88.6 us; 16384 rows of 5120 / 6144: 61.2 / 72.1 -> 58.9 / 67.6 us.
-    // Rows on fewer than 256 lanes (two row slots a workgroup) do not gain (N = 3072:
-    // 38.1 -> 40.0 us) and keep the grid above.  At 65536 rows and beyond (64+ row blocks a workgroup)
-    // it loses 3-10 % and the grid above stays.  With 16-bit weights, and for
-    // RMSNorm, the two regimes are within 2 % of each other at 16384 rows either
-    // way (and the residual-add forward, with twice the bytes in flight, loses 7 %
-    // on the small grid), so they keep the grid above.  Grids in between (6-8
+    // Up to a few tens of thousands of rows, fp32 weights beside 16-bit rows (and
+    // LayerNorm on 512 lanes with any weights) take the other regime: three
+    // 256-thread or two 512-thread workgroups a compute unit, all resident at once,
+    // each walking up to 32 row blocks -- the weights are loaded once per 4..32 rows
+    // and no second wave of workgroups leaves a tail.  Interleaved A/B runs, bf16
+    // rows, LayerNorm with fp32 weights at 2048 / 4096 / 16384 rows: N = 4096 9.8 /
+    // 17.4 / 48.9 -> 8.2 / 13.5 / 46.0 us, N = 8192 17.7 / 33.2 / 93.3 -> 14.2 / 24.3 /
+    // 88.6 us; 16384 rows of 5120 / 6144: 61.2 / 72.1 -> 58.9 / 67.6 us (four
+    // workgroups of 256 instead of three: 60.1 / 72.3 us).  RMSNorm with fp32 weights,
+    // 16384 rows: N = 5120 56.8 -> 54.8, 7168 80.0 -> 76.0, 8192 89.3 -> 85.3, 12288
+    // 135.2 -> 128.3 us.  LayerNorm with bf16 weights on 512 lanes: 7168 80.9 -> 77.4,
+    // 8192 89.2 -> 86.9, 12288 136.3 -> 131.6 us (10240: 115.3 -> 117.1).  With bf16
+    // weights on 256 lanes, and for RMSNorm with bf16 weights, the two regimes are
+    // within 1 % at 4096-6144 and the small grid loses 3 % at 10240; the
+    // residual-add forward, with twice the bytes in flight, loses 7 % on it: they
+    // keep the grid above.  Rows on fewer than 256 lanes (two row slots a workgroup)
+    // do not gain (N = 3072: 38.1 -> 40.0 us).  At 65536 rows and beyond (64+ row
+    // blocks a workgroup) the small grid loses 3-10 %.  Grids in between (6-8
     // workgroups a compute unit, where a second wave starts) were the slowest at
     // every row count.
-    if (layer_norm && wide_weights && p.block <= 512 && p.rpb == 1) {
+    if ((wide_weights || (layer_norm && p.block == 512)) && p.block <= 512 && p.rpb == 1) {
       const int64_t cap = (int64_t)num_cus * (p.block == 512 ? 2 : 3);
       if (nrb <= cap * 32) grid = cap;
     }
