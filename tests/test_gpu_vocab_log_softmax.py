@@ -1,0 +1,86 @@
+"""log_softmax backward on vocabulary-sized rows (the cross_entropy case): rows too long for both
+tensors in registers keep grad resident and stream y past it (log_softmax_bwd_grad_resident_kernel;
+the reference walks the row twice in LogSoftmaxBackward, src/ATen/native/xpu/sycl/
+SoftMaxKernels.cpp:991-1150).  Every packs-per-lane count of the kernel (5..16 for 16-bit rows,
+9..16 for float32 rows), with the row end inside and at the end of a lane's last pack, misaligned
+tensors and -inf / NaN entries, against the CPU oracle at the family's tolerances (float32
+rtol = atol = 1e-5; 16-bit atol 1e-2, rtol 1.6e-2) and against the multi-pass kernel forced on
+the same inputs."""
+import pytest
+import torch
+
+from helpers import assert_close, gen, offset_view, rowsum_slack, to_np32
+
+pytestmark = pytest.mark.gpu
+
+
+def _case(cabi, oracle, gpu, M, N, dtype, off, seed, gi_dtype=None):
+    g = gen(seed)
+    x = 2.0 * torch.randn(M, N, generator=g)
+    x[0, N // 3] = float("-inf")          # y = -inf, exp(y) = 0: the gradient passes through
+    grad = torch.randn(M, N, generator=g).to(dtype)
+    y = torch.log_softmax(x, -1).to(dtype)
+    put = (lambda t: offset_view(t.to(gpu), off)) if off else (lambda t: t.to(gpu))
+    yg, gg = put(y), put(grad)
+    p = cabi.plan(cabi.OP_SOFTMAX_BWD, M, N, cabi.dtype_code(dtype), cabi.dtype_code(dtype))
+    assert p["resident"] == 0
+    gi = cabi.softmax_bwd(gg, yg, True, gi_dtype=gi_dtype)
+    try:
+        cabi.set_override(cabi.OP_SOFTMAX_BWD, -1, 1)     # the multi-pass kernel
+        ref = cabi.softmax_bwd(gg, yg, True, gi_dtype=gi_dtype)
+    finally:
+        cabi.clear_overrides()
+    od = dtype if gi_dtype is None else gi_dtype
+    ogi = oracle.softmax_bwd(to_np32(grad), to_np32(y), True)
+    # float32: exp(y) * (a float32 sum over N terms) carries the sum's rounding (helpers.rowsum_slack)
+    sl = rowsum_slack(to_np32(grad), torch.exp(y.double())) if od == torch.float32 else None
+    what = "[%d, %d] %s off %d" % (M, N, dtype, off)
+    assert_close(gi, ogi, od, "grad-resident log_softmax backward " + what, slack=sl)
+    assert_close(ref, ogi, od, "multi-pass log_softmax backward " + what, slack=sl)
+    assert_close(gi, to_np32(ref), od, "grad-resident vs multi-pass " + what, slack=sl)
+
+
+@pytest.mark.parametrize("dtype", [torch.bfloat16, torch.float16], ids=str)
+def test_every_pack_count_16bit(cabi, oracle, gpu, dtype):
+    # packs a lane = ceil(N / 8192): 5 (one pack into the fifth round), 5 exactly, 6 .. 16
+    for i, N in enumerate((32776, 40960, 49144, 50304, 65536, 73728, 81912, 90112, 100000, 106496,
+                           114688, 122880, 128256, 131072)):
+        _case(cabi, oracle, gpu, 3, N, dtype, 0, 900 + i)
+    _case(cabi, oracle, gpu, 2, 50304, dtype, 3, 950)     # 6 bytes off 16-byte alignment
+    _case(cabi, oracle, gpu, 2, 128256, dtype, 1, 951)
+
+
+def test_every_pack_count_float32(cabi, oracle, gpu):
+    # float32 rows: 4 elements a pack, the two-tensor kernels end at 32768 elements
+    for i, N in enumerate((32772, 36864, 40000, 45056, 50304, 53248, 57344, 61440, 65536)):
+        _case(cabi, oracle, gpu, 2, N, torch.float32, 0, 960 + i)
+    _case(cabi, oracle, gpu, 2, 50304, torch.float32, 1, 970)
+
+
+def test_float32_grad_to_float16_gradient(cabi, oracle, gpu):
+    """half_to_float: float32 grad and y, float16 grad_input (SoftMax.cpp:72-100)."""
+    _case(cabi, oracle, gpu, 2, 50304, torch.float32, 0, 980, gi_dtype=torch.float16)
+
+
+def test_nan_poisons_its_row_only(cabi, gpu):
+    M, N = 3, 50304
+    y = torch.log_softmax(torch.randn(M, N, generator=gen(990)), -1).bfloat16()
+    grad = torch.randn(M, N, generator=gen(991)).bfloat16()
+    grad[1, 777] = float("nan")
+    gi = cabi.softmax_bwd(grad.to(gpu), y.to(gpu), True)
+    assert bool(torch.isnan(gi[1]).all())
+    assert bool(torch.isfinite(gi[0]).all()) and bool(torch.isfinite(gi[2]).all())
+
+
+def test_softmax_and_ragged_rows_keep_the_multi_pass_kernel(cabi, oracle, gpu):
+    """The kernel serves log_softmax on whole packs only; softmax and ragged rows of that length
+    still go through the multi-pass kernel and agree with the oracle."""
+    M = 2
+    for N, is_log in ((50304, False), (50257, True)):
+        g = gen(995)
+        x = torch.randn(M, N, generator=g)
+        grad = torch.randn(M, N, generator=g).bfloat16()
+        y = (torch.log_softmax(x, -1) if is_log else torch.softmax(x, -1)).bfloat16()
+        gi = cabi.softmax_bwd(grad.to(gpu), y.to(gpu), is_log)
+        assert_close(gi, oracle.softmax_bwd(to_np32(grad), to_np32(y), is_log), torch.bfloat16,
+                     "N=%d log=%d" % (N, is_log))

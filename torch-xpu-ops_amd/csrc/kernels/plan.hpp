@@ -52,6 +52,9 @@ struct Plan {
   // 0 or 1 = one workgroup per row.
   int split = 0;
   int64_t chunk_packs = 0;
+  // softmax backward of rows beyond the registers of two tensors: grad alone fits
+  // them (the log_softmax backward then keeps grad resident and streams y)
+  bool grad_resident = false;
 };
 
 constexpr int kMinG = 8;
@@ -492,6 +495,9 @@ inline int make_plan(OpClass oc, int64_t M, int64_t N, int esize, int num_cus, c
       }
     }
   }
+  if (oc == OC_SOFTMAX_BWD && !p.resident && p.fast && ov.G == 0 &&
+      packs <= (int64_t)kMaxG * kMaxV)
+    p.grad_resident = true;
   *out = p;
   return 0;
 }

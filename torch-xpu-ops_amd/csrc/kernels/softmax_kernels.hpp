@@ -494,6 +494,71 @@ softmax_bwd_resident_kernel(const TG* __restrict__ grad, const TG* __restrict__ 
   }
 }
 
+// log_softmax backward for rows beyond what the registers hold of TWO tensors
+// (vocabulary-sized rows under cross_entropy): gi = grad - exp(y) * sum(grad).  The
+// sum needs grad alone, so grad stays in the registers (V packs a lane on BLOCK
+// lanes, in storage format) and y is streamed past it, U packs at a time, the next
+// U requested before the current ones are used: every tensor crosses the memory
+// interface once, where the multi-pass kernel reads grad twice.  N is a whole
+// number of packs and V = ceil(packs / BLOCK) exactly, so only a lane's last pack
+// can lie beyond the row end (it is requested from the row's first pack and never
+// used) and the others sit at constant strides from the lane's first.
+constexpr int kGradResidentUnroll = 4;
+
+template <class TG, class TO, int V, int BLOCK>
+__global__ void __launch_bounds__(BLOCK)
+log_softmax_bwd_grad_resident_kernel(const TG* __restrict__ grad, const TG* __restrict__ y,
+                                     TO* __restrict__ gi, int64_t M, int N) {
+  constexpr int E = elems_per_pack<TG>::value;
+  constexpr int U = kGradResidentUnroll;
+  constexpr bool PRECISE = sizeof(TO) == 4 && sizeof(TG) == 4;
+  __shared__ float red[reduce_lds_floats<BLOCK, BLOCK, 1>::value];
+  int phase = 0;
+  const int lane = threadIdx.x;
+  const bool last_in = ((V - 1) * BLOCK + lane) * E < N;  // this lane's last pack lies in the row
+  for (int64_t row = blockIdx.x; row < M; row += gridDim.x) {
+    const TG* gr = grad + row * (int64_t)N + lane * E;
+    const TG* yr = y + row * (int64_t)N + lane * E;
+    TO* outr = gi + row * (int64_t)N + lane * E;
+    // element offset of pack c from the lane's first pack
+    auto off = [&](int c) { return (c < V - 1 || last_in) ? c * BLOCK * E : 0; };
+    Pack<TG, E> pg[V], py[U], pn[U];
+#pragma unroll
+    for (int c = 0; c < V; ++c) pg[c] = Pack<TG, E>::load_stream(gr + off(c));
+    auto request_y = [&](int c0, Pack<TG, E> (&dst)[U]) {
+#pragma unroll
+      for (int u = 0; u < U; ++u)
+        if (c0 + u < V) dst[u] = Pack<TG, E>::load_stream(yr + off(c0 + u));
+    };
+    request_y(0, pn);  // on its way while grad is summed
+    float sum[1] = {0.0f};
+    if (!last_in) pg[V - 1] = Pack<TG, E>::zero();
+#pragma unroll
+    for (int c = 0; c < V; ++c)
+#pragma unroll
+      for (int i = 0; i < E; ++i) sum[0] += pg[c].get(i);
+    group_allreduce<BLOCK, BLOCK, 1, SumOp>(sum, red, phase);
+    const float s = sum[0];
+#pragma unroll
+    for (int c0 = 0; c0 < V; c0 += U) {
+#pragma unroll
+      for (int u = 0; u < U; ++u) py[u] = pn[u];
+      if (c0 + U < V) request_y(c0 + U, pn);
+#pragma unroll
+      for (int u = 0; u < U; ++u) {
+        if (c0 + u < V) {
+          keep_packed(pg[c0 + u]);
+          Pack<TO, E> o;
+#pragma unroll
+          for (int i = 0; i < E; ++i)
+            o.set(i, pg[c0 + u].get(i) - row_exp<PRECISE>(py[u].get(i)) * s);
+          if (c0 + u < V - 1 || last_in) o.store_stream(outr + (c0 + u) * BLOCK * E);
+        }
+      }
+    }
+  }
+}
+
 template <class TG, class TO, int BLOCK, bool MASKED>
 __global__ void __launch_bounds__(BLOCK)
 softmax_bwd_stream_kernel(const TG* __restrict__ grad, const TG* __restrict__ y,

@@ -83,6 +83,40 @@ struct SoftmaxBwdLauncher {
   };
 };
 
+// log_softmax backward of rows too long for both tensors in registers but not for
+// grad alone: whole packs, at most 1024 lanes x 16 packs.  False: not this case.
+template <class TG, class TO, int V>
+inline void launch_grad_resident_v(const Plan& plan, const SoftmaxBwdArgs& a, hipStream_t stream) {
+  hipLaunchKernelGGL((log_softmax_bwd_grad_resident_kernel<TG, TO, V, kStreamBlock>),
+                     dim3((unsigned)plan.grid), dim3(kStreamBlock), 0, stream, (const TG*)a.grad,
+                     (const TG*)a.y, (TO*)a.gi, a.M, a.N);
+}
+
+template <class TG, class TO>
+inline bool launch_log_softmax_bwd_grad_resident(const Plan& plan, const SoftmaxBwdArgs& a,
+                                                 hipStream_t stream) {
+  constexpr int E = elems_per_pack<TG>::value;
+  if (!plan.grad_resident || !(a.flags & kSoftmaxLog) || a.N % E != 0) return false;
+  const int64_t packs = a.N / E;
+  switch ((int)((packs + kStreamBlock - 1) / kStreamBlock)) {
+    case 3: launch_grad_resident_v<TG, TO, 3>(plan, a, stream); return true;
+    case 4: launch_grad_resident_v<TG, TO, 4>(plan, a, stream); return true;
+    case 5: launch_grad_resident_v<TG, TO, 5>(plan, a, stream); return true;
+    case 6: launch_grad_resident_v<TG, TO, 6>(plan, a, stream); return true;
+    case 7: launch_grad_resident_v<TG, TO, 7>(plan, a, stream); return true;
+    case 8: launch_grad_resident_v<TG, TO, 8>(plan, a, stream); return true;
+    case 9: launch_grad_resident_v<TG, TO, 9>(plan, a, stream); return true;
+    case 10: launch_grad_resident_v<TG, TO, 10>(plan, a, stream); return true;
+    case 11: launch_grad_resident_v<TG, TO, 11>(plan, a, stream); return true;
+    case 12: launch_grad_resident_v<TG, TO, 12>(plan, a, stream); return true;
+    case 13: launch_grad_resident_v<TG, TO, 13>(plan, a, stream); return true;
+    case 14: launch_grad_resident_v<TG, TO, 14>(plan, a, stream); return true;
+    case 15: launch_grad_resident_v<TG, TO, 15>(plan, a, stream); return true;
+    case 16: launch_grad_resident_v<TG, TO, 16>(plan, a, stream); return true;
+  }
+  return false;
+}
+
 template <class TG, class TO, bool MASKED>
 int launch_softmax_bwd_m(const Plan& plan, const SoftmaxBwdArgs& a, hipStream_t stream) {
   if (plan.resident) {
@@ -91,6 +125,8 @@ int launch_softmax_bwd_m(const Plan& plan, const SoftmaxBwdArgs& a, hipStream_t 
         plan.fast ? launch_variant<SoftmaxBwdLauncher<TG, TO, true, MASKED>::template At>(ctx)
                   : launch_variant<SoftmaxBwdLauncher<TG, TO, false, MASKED>::template At>(ctx);
     if (!launched) return (int)hipErrorInvalidConfiguration;
+  } else if (!MASKED && launch_log_softmax_bwd_grad_resident<TG, TO>(plan, a, stream)) {
+    // (log_softmax rows of up to 16 packs a lane: grad resident, y streamed)
   } else {
     hipLaunchKernelGGL((softmax_bwd_stream_kernel<TG, TO, kStreamBlock, MASKED>),
                        dim3((unsigned)plan.grid), dim3(kStreamBlock), 0, stream,
