@@ -74,6 +74,10 @@ __device__ __forceinline__ Pack<T, E> stream_load(const T* row, int e0, int n, b
 // the exponential in log_softmax's output pass and in softmax's backward too).
 #define ROWNORM_UNIFORM_ARM(tag) asm volatile("; " tag)
 
+#ifndef ROWNORM_SOFTMAX_ONLINE_WIDE
+#define ROWNORM_SOFTMAX_ONLINE_WIDE 1
+#endif
+
 // Packs a thread of the multi-pass kernels requests before using the first.
 constexpr int kStreamUnroll = 2;
 
@@ -115,8 +119,20 @@ __device__ __forceinline__ Pack<uint8_t, E> load_mask_pack(const uint8_t* mrow, 
   return m;
 }
 
+// Wavefronts per SIMD the register budget of the resident forward is set for (the
+// second argument of __launch_bounds__ in HIP): eight, i.e. two 1024-thread
+// workgroups a compute unit and 64 registers, for 1024-lane rows of 5..8 packs a
+// lane; otherwise what the workgroup size implies.
+#ifndef ROWNORM_SOFTMAX_TWO_BLOCKS_MAX_V
+#define ROWNORM_SOFTMAX_TWO_BLOCKS_MAX_V 8
+#endif
+template <class TI, int G, int V, bool FAST, bool MASKED>
+constexpr int softmax_fwd_min_blocks() {
+  return (G == 1024 && FAST && !MASKED && V >= 5 && V <= ROWNORM_SOFTMAX_TWO_BLOCKS_MAX_V) ? 8 : 1;
+}
+
 template <class TI, class TO, int G, int V, int BLOCK, bool FAST, bool MASKED>
-__global__ void __launch_bounds__(BLOCK)
+__global__ void __launch_bounds__(BLOCK, (softmax_fwd_min_blocks<TI, G, V, FAST, MASKED>()))
 softmax_fwd_resident_kernel(const TI* __restrict__ x, TO* __restrict__ y, MaskRef mask, int64_t M,
                             int N, int flags) {
   constexpr int E = elems_per_pack<TI>::value;
@@ -162,20 +178,58 @@ softmax_fwd_resident_kernel(const TI* __restrict__ x, TO* __restrict__ y, MaskRe
         }
       }
       float mx[1] = {-INFINITY};
-#pragma unroll
-      for (int c = 0; c < V; ++c)
-#pragma unroll
-        for (int i = 0; i < E; ++i) mx[0] = fmaxf(mx[0], xp[c].get(i));
-      group_allreduce<G, BLOCK, 1, MaxOp>(mx, red, phase);
-      const float m = mx[0];
       float sum[1] = {0.0f};
+      float m;
+      if constexpr (ROWNORM_SOFTMAX_ONLINE_WIDE && !MASKED && FAST && V >= 8) {
+        // the lane's packs in two halves, each with its own maximum and sum of
+        // exp(x - maximum): the first half is worked on while the second is still
+        // arriving, and the exponentials no longer wait for the block maximum
+        constexpr int VA = V / 2;
+        float m_t = -INFINITY, s_t = 0.0f;
+        auto absorb = [&](auto c0, auto c1) {
+          float pm = -INFINITY;
 #pragma unroll
-      for (int c = 0; c < V; ++c) {
-        keep_packed(xp[c]);
+          for (int c = decltype(c0)::value; c < decltype(c1)::value; ++c)
 #pragma unroll
-        for (int i = 0; i < E; ++i) sum[0] += row_exp<PRECISE>(xp[c].get(i) - m);
+            for (int i = 0; i < E; ++i) pm = fmaxf(pm, xp[c].get(i));
+          const float nm = fmaxf(m_t, pm);
+          // (nothing finite yet: the reference is 0, against which -inf elements add 0
+          // and a NaN element still poisons the sum)
+          const float ref = nm == -INFINITY ? 0.0f : nm;
+          float acc = s_t * row_exp<PRECISE>(m_t - ref);
+#pragma unroll
+          for (int c = decltype(c0)::value; c < decltype(c1)::value; ++c) {
+            keep_packed(xp[c]);
+#pragma unroll
+            for (int i = 0; i < E; ++i) acc += row_exp<PRECISE>(xp[c].get(i) - ref);
+          }
+          s_t = acc;
+          m_t = nm;
+        };
+        absorb(std::integral_constant<int, 0>{}, std::integral_constant<int, VA>{});
+        absorb(std::integral_constant<int, VA>{}, std::integral_constant<int, V>{});
+        mx[0] = m_t;
+        group_allreduce<G, BLOCK, 1, MaxOp>(mx, red, phase);
+        m = mx[0];
+        // exp(-inf - m) = 0 drops lanes that saw nothing finite; a row with no finite
+        // element at all gives NaN, like the three-pass form
+        sum[0] = s_t == 0.0f ? (m == -INFINITY ? NAN : 0.0f) : s_t * row_exp<PRECISE>(m_t - m);
+        group_allreduce<G, BLOCK, 1, SumOp>(sum, red, phase);
+      } else {
+#pragma unroll
+        for (int c = 0; c < V; ++c)
+#pragma unroll
+          for (int i = 0; i < E; ++i) mx[0] = fmaxf(mx[0], xp[c].get(i));
+        group_allreduce<G, BLOCK, 1, MaxOp>(mx, red, phase);
+        m = mx[0];
+#pragma unroll
+        for (int c = 0; c < V; ++c) {
+          keep_packed(xp[c]);
+#pragma unroll
+          for (int i = 0; i < E; ++i) sum[0] += row_exp<PRECISE>(xp[c].get(i) - m);
+        }
+        group_allreduce<G, BLOCK, 1, SumOp>(sum, red, phase);
       }
-      group_allreduce<G, BLOCK, 1, SumOp>(sum, red, phase);
       if (is_log) {
         ROWNORM_UNIFORM_ARM("log_softmax: x - max - log(sum)");
         const float k = logf(sum[0]);
