@@ -398,18 +398,17 @@ softmax_fwd_stream_kernel(const TI* __restrict__ x, TO* __restrict__ y, MaskRef 
           v[i] = masked_value(pv[u], mv[u], i);
           pm = fmaxf(pm, v[i]);
         }
-        if (pm > m_t) {  // a new maximum: bring the sum so far to the new reference
-          s_t *= row_exp<PRECISE>(m_t - pm);
-          m_t = pm;
-        }
-        if (m_t > -INFINITY) {
+        // bring the sum so far to the new maximum and add the pack -- without a branch
+        // (a lane-divergent branch here costs registers and keeps loads from overlapping):
+        // while nothing finite has been seen the reference is 0, against which -inf
+        // elements add 0 and a NaN element still poisons the row
+        const float nm = fmaxf(m_t, pm);
+        const float ref = nm == -INFINITY ? 0.0f : nm;
+        float acc = s_t * row_exp<PRECISE>(m_t - ref);
 #pragma unroll
-          for (int i = 0; i < E; ++i) s_t += row_exp<PRECISE>(v[i] - m_t);
-        } else {
-          // nothing finite yet: a NaN element must still poison the row
-#pragma unroll
-          for (int i = 0; i < E; ++i) s_t += (v[i] != v[i]) ? v[i] : 0.0f;
-        }
+        for (int i = 0; i < E; ++i) acc += row_exp<PRECISE>(v[i] - ref);
+        s_t = acc;
+        m_t = nm;
       }
     }
     float mx[1] = {m_t};

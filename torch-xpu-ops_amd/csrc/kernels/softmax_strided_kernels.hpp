@@ -554,16 +554,14 @@ softmax_strided_split_partial_kernel(const TI* __restrict__ x, TO* __restrict__ 
         float nm = mx[i];
 #pragma unroll
         for (int u = 0; u < U; ++u) nm = fmaxf(nm, p[u].get(i));
-        if (nm != -INFINITY) {
-          float acc = sum[i] * row_exp<PRECISE>(mx[i] - nm);
+        // (no branch: while nothing finite has been seen the reference is 0, against
+        // which -inf elements add 0 and a NaN element, which fmaxf drops, still poisons
+        // the sum)
+        const float ref = nm == -INFINITY ? 0.0f : nm;
+        float acc = sum[i] * row_exp<PRECISE>(mx[i] - ref);
 #pragma unroll
-          for (int u = 0; u < U; ++u) acc += row_exp<PRECISE>(p[u].get(i) - nm);
-          sum[i] = acc;
-        } else {
-          // nothing finite yet; a NaN element (which fmaxf drops) must still poison the sum
-#pragma unroll
-          for (int u = 0; u < U; ++u) sum[i] += p[u].get(i) != p[u].get(i) ? p[u].get(i) : 0.0f;
-        }
+        for (int u = 0; u < U; ++u) acc += row_exp<PRECISE>(p[u].get(i) - ref);
+        sum[i] = acc;
         mx[i] = nm;
       }
     }
