@@ -27,7 +27,11 @@ SHAPES = [(2, 4, (), 2), (64, 32, (), 4), (256, 32, (), 4), (64, 32, (16,), 4), 
           # rows of 6..10 packs a lane on 512 lanes (16-bit: L = 24576 .. 40960; fp32: 12288 ..
           # 20480) and an fp32 row of 11 packs a lane on 1024 lanes
           (2, 12, (64, 64), 2), (2, 14, (64, 64), 2), (2, 18, (64, 64), 2), (1, 20, (64, 64), 2),
-          (2, 12, (2048,), 2), (2, 14, (2048,), 2), (1, 20, (2048,), 2), (1, 22, (64, 64), 2)]
+          (2, 12, (2048,), 2), (2, 14, (2048,), 2), (1, 20, (2048,), 2), (1, 22, (64, 64), 2),
+          # channels of 1, 3, 5, 125 and 1025 packs (the pack -> channel lookup multiplies by a
+          # rounded-up reciprocal of the packs per channel instead of dividing)
+          (4, 12, (8,), 3), (4, 12, (4,), 3), (3, 10, (24,), 5), (2, 6, (5, 8), 2), (2, 9, (1000,), 3),
+          (1, 6, (8200,), 2)]
 CASES = load_golden("aten_cpu_group_norm.npz")
 
 

@@ -96,6 +96,23 @@ __device__ __forceinline__ void keep_packed(Pack<T, E>& p) {
   }
 }
 
+// The lane index as a value the compiler cannot trace back to threadIdx, and
+// that exists only once `after` does: the pack offsets derived from it are then
+// computed where they are used (after a reduction, say) instead of ahead of the
+// row loop, where each would hold a register for the whole kernel.
+template <bool ON = true>
+__device__ __forceinline__ int lane_after(int lane, float& after) {
+  if constexpr (ON) asm volatile("" : "+v"(lane), "+v"(after));
+  return lane;
+}
+
+// The same at the top of a row loop, with nothing to wait for.
+template <bool ON = true>
+__device__ __forceinline__ int lane_again(int lane) {
+  if constexpr (ON) asm volatile("" : "+v"(lane));
+  return lane;
+}
+
 // Loads the pack that starts at element `e0` of a row whose elements are
 // [lo, n) of `row`.  A pack that lies wholly inside the row is one 128-bit load;
 // a pack that straddles either end of the row is read element by element and

@@ -53,6 +53,9 @@ struct GroupShape {
   int HxW;      // elements per channel
   int D;        // channels per group
   int groups;   // groups per sample
+  // rows whose channels are whole packs (HxW % E == 0), else both 0:
+  int packs;            // packs per row, L / E
+  unsigned pack_magic;  // ceil(2^31 / (HxW / E)), see gn_pack_channel
 };
 
 // Wavefronts per SIMD a resident kernel is compiled for (the second argument of
@@ -69,9 +72,19 @@ __device__ __forceinline__ int gn_channel(const GroupShape& s, int g, int p) {
   return g * s.D + (int)((unsigned)pc / (unsigned)s.HxW);
 }
 
+// Channel of pack `pk` of row `g` when every pack lies in one channel (pk is
+// clamped into the row).  pk / S for S = HxW / E packs per channel is
+// floor(2 * pk * ceil(2^31 / S) / 2^32), exact while pk * S < 2^31; the rows
+// held in registers have at most 2^14 packs.  A 32-bit division costs about
+// 25 instructions a pack, this costs 3.
+__device__ __forceinline__ int gn_pack_channel(const GroupShape& s, int g, int pk) {
+  const int pc = pk < s.packs ? pk : s.packs - 1;
+  return g * s.D + (int)__umulhi(2u * (unsigned)pc, s.pack_magic);
+}
+
 template <class WT>
 __device__ __forceinline__ float gn_weight(const WT* w, int ch, float dflt) {
-  return w ? (float)w[ch] : dflt;
+  return w ? (float)w[(unsigned)ch] : dflt;  // ch >= 0: a 32-bit offset from a scalar base
 }
 
 // ---------------------------------------------------------------------------
@@ -89,12 +102,17 @@ gn_fwd_resident_kernel(const T* __restrict__ x, const WT* __restrict__ gamma,
   __shared__ float red[reduce_lds_floats<G, BLOCK, 2>::value];
   int phase = 0;
   const int slot = threadIdx.x / G;
-  const int lane = threadIdx.x % G;
+  const int lane0 = threadIdx.x % G;
   const float fL = (float)s.L;
   const float inv_l = 1.0f / fL;
   const bool exact = s.L == G * V * E;
   const int64_t nrb = (rows + RPB - 1) / RPB;
   for (int64_t rb = blockIdx.x; rb < nrb; rb += gridDim.x) {
+    // opaque once a row, so that the V packs' offsets and channels are computed
+    // where they are used instead of being held in registers across the loop
+    // (see the backward)
+    int lane = lane0;
+    asm volatile("" : "+v"(lane));
     const int64_t row = rb * RPB + slot;
     const bool ok = RPB == 1 ? true : row < rows;
     const int64_t rowc = ok ? row : 0;
@@ -154,7 +172,7 @@ gn_fwd_resident_kernel(const T* __restrict__ x, const WT* __restrict__ gamma,
       const int e0 = (c * G + lane) * E;
       Pack<T, E> o;
       if constexpr (UNIFORM) {
-        const int ch = gn_channel(s, g, e0);
+        const int ch = gn_pack_channel(s, g, c * G + lane);
         const float ga = gn_weight(gamma, ch, 1.0f) * rs;
         const float be = gn_weight(beta, ch, 0.0f);
 #pragma unroll
@@ -266,11 +284,18 @@ gn_bwd_resident_kernel(const T* __restrict__ dy, const T* __restrict__ x,
   __shared__ float stage[gn_stage_floats<G, V, BLOCK, UNIFORM>::value];
   int phase = 0;
   const int slot = threadIdx.x / G;
-  const int lane = threadIdx.x % G;
+  const int lane0 = threadIdx.x % G;
   const float fL = (float)s.L;
   const bool want_cols = UNIFORM && part_dg != nullptr;  // uniform over the grid
   const int64_t nrb = (rows + RPB - 1) / RPB;
   for (int64_t rb = blockIdx.x; rb < nrb; rb += gridDim.x) {
+    // The lane index is made opaque once a row: the offsets, channels and LDS
+    // slots of the V packs derive from it, and the compiler would otherwise
+    // compute all of them before the loop and hold 3-4 registers a pack for the
+    // whole kernel (spilling at 7 and 8 packs).  Recomputing costs a few
+    // instructions a pack.
+    int lane = lane0;
+    asm volatile("" : "+v"(lane));
     const int64_t row = rb * RPB + slot;
     const bool ok = RPB == 1 ? true : row < rows;
     const int64_t rowc = ok ? row : 0;
@@ -285,12 +310,13 @@ gn_bwd_resident_kernel(const T* __restrict__ dy, const T* __restrict__ x,
       dp[c] = row_load<T, E, true, UNIFORM>(dy + rowc * (int64_t)s.L, e0, s.L, ok, 0.0f);
     }
     float acc[2] = {0.0f, 0.0f};
+    float gu[UNIFORM ? V : 1];  // the weight of each pack, looked up once a row
     float* st = stage + slot * (UNIFORM ? 2 * G * V : 0);
 #pragma unroll
     for (int c = 0; c < V; ++c) {
       const int e0 = (c * G + lane) * E;
       if constexpr (UNIFORM) {
-        const float ga = gn_weight(gamma, gn_channel(s, g, e0), 1.0f);
+        const float ga = gu[c] = gn_weight(gamma, gn_pack_channel(s, g, c * G + lane), 1.0f);
         float pdg = 0.0f, pdb = 0.0f;
 #pragma unroll
         for (int i = 0; i < E; ++i) {
@@ -320,22 +346,30 @@ gn_bwd_resident_kernel(const T* __restrict__ dy, const T* __restrict__ x,
       T* dr = dx + row * (int64_t)s.L;
       const float s1 = acc[0], s2 = acc[1];
       const float term1 = rs / fL;
+      // 16-bit rows with one weight a pack use the regrouped
+      // dy*(rs*gamma) - x*(rs*a) + (mu*rs*a - b), a = s2*rs/L, b = s1*rs/L: two
+      // FMAs an element, rounding far below a 16-bit ulp (as the LayerNorm backward)
+      const float ra = rs * (s2 * term1);
+      const float cc = mu * ra - s1 * term1;
 #pragma unroll
       for (int c = 0; c < V; ++c) {
         keep_packed(xp[c]);
         keep_packed(dp[c]);
         const int e0 = (c * G + lane) * E;
-        float gu = 1.0f;
-        if constexpr (UNIFORM) gu = gn_weight(gamma, gn_channel(s, g, e0), 1.0f);
+        const float gr = UNIFORM ? gu[c] * rs : 0.0f;
         Pack<T, E> o;
 #pragma unroll
         for (int i = 0; i < E; ++i) {
-          const float ga = UNIFORM ? gu : gn_weight(gamma, gn_channel(s, g, e0 + i), 1.0f);
-          const float xh = (xp[c].get(i) - mu) * rs;
-          float f = fL * (dp[c].get(i) * ga);
-          f -= xh * s2;
-          f -= s1;
-          o.set(i, f * term1);
+          if constexpr (UNIFORM && sizeof(T) == 2) {
+            o.set(i, fmaf(xp[c].get(i), -ra, fmaf(dp[c].get(i), gr, cc)));
+          } else {
+            const float ga = UNIFORM ? gu[c] : gn_weight(gamma, gn_channel(s, g, e0 + i), 1.0f);
+            const float xh = (xp[c].get(i) - mu) * rs;
+            float f = fL * (dp[c].get(i) * ga);
+            f -= xh * s2;
+            f -= s1;
+            o.set(i, f * term1);
+          }
         }
         row_store<T, E, true, UNIFORM>(dr, e0, s.L, ok, o);
       }

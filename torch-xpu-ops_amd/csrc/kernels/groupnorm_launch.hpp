@@ -6,7 +6,16 @@
 
 namespace rownorm {
 
-inline GroupShape group_shape(int L, int HxW, int D, int groups) { return GroupShape{L, HxW, D, groups}; }
+// E: elements per pack of the row dtype.
+inline GroupShape group_shape(int L, int HxW, int D, int groups, int E) {
+  GroupShape s{L, HxW, D, groups, 0, 0u};
+  if (HxW % E == 0) {
+    const uint64_t per_channel = (uint64_t)(HxW / E);
+    s.packs = L / E;
+    s.pack_magic = (unsigned)((((uint64_t)1 << 31) + per_channel - 1) / per_channel);
+  }
+  return s;
+}
 
 template <class T, class WT>
 struct GroupNormFwdCtx {
@@ -27,7 +36,7 @@ struct GroupNormFwdLauncher {
                              dim3((unsigned)c.plan.grid), dim3(BLOCK), 0, c.stream,
                              (const T*)c.a.x, (const WT*)c.a.gamma, (const WT*)c.a.beta,
                              (T*)c.a.y, (WT*)c.a.mean, (WT*)c.a.rstd, c.a.rows,
-                             group_shape(c.a.L, c.a.HxW, c.a.D, c.a.groups), c.a.eps);
+                             group_shape(c.a.L, c.a.HxW, c.a.D, c.a.groups, elems_per_pack<T>::value), c.a.eps);
           return true;
         }
       }
@@ -48,7 +57,7 @@ int launch_group_norm_fwd(const Plan& plan, const GroupNormFwdArgs& a, hipStream
     hipLaunchKernelGGL((gn_fwd_stream_kernel<T, WT, kStreamBlock>), dim3((unsigned)plan.grid),
                        dim3(kStreamBlock), 0, stream, (const T*)a.x, (const WT*)a.gamma,
                        (const WT*)a.beta, (T*)a.y, (WT*)a.mean, (WT*)a.rstd, a.rows,
-                       group_shape(a.L, a.HxW, a.D, a.groups), a.eps);
+                       group_shape(a.L, a.HxW, a.D, a.groups, elems_per_pack<T>::value), a.eps);
   }
   return (int)hipGetLastError();
 }
@@ -74,7 +83,7 @@ struct GroupNormBwdLauncher {
                              (const T*)c.a.dy, (const T*)c.a.x, (const WT*)c.a.mean,
                              (const WT*)c.a.rstd, (const WT*)c.a.gamma, (T*)c.a.dx, c.a.part_dg,
                              c.a.part_db, c.a.rows,
-                             group_shape(c.a.L, c.a.HxW, c.a.D, c.a.groups), c.tpc_log2);
+                             group_shape(c.a.L, c.a.HxW, c.a.D, c.a.groups, elems_per_pack<T>::value), c.tpc_log2);
           return true;
         }
       }
@@ -101,7 +110,7 @@ int launch_group_norm_bwd(const Plan& plan, const GroupNormBwdArgs& a, hipStream
   const bool fused_cols = plan.resident && plan.fast;  // channel sums come out of the dX kernel
   // rows too long for the registers get dX from the channel sums, wanted or not
   const bool need_sums = want_cols || (!plan.resident && a.dx != nullptr);
-  const GroupShape shape = group_shape(a.L, a.HxW, a.D, a.groups);
+  const GroupShape shape = group_shape(a.L, a.HxW, a.D, a.groups, elems_per_pack<T>::value);
   const int64_t N = a.rows / a.groups;
   const int C = a.groups * a.D;
   int err = 0;

@@ -121,11 +121,12 @@ __device__ __forceinline__ Pack<uint8_t, E> load_mask_pack(const uint8_t* mrow, 
 
 // Wavefronts per SIMD the register budget of the resident forward is set for (the
 // second argument of __launch_bounds__ in HIP): eight, i.e. two 1024-thread
-// workgroups a compute unit and 64 registers, for 1024-lane rows of 5..8 packs a
+// workgroups a compute unit and 64 registers, for 1024-lane rows of 5..9 packs a
 // lane; otherwise what the workgroup size implies.
 #ifndef ROWNORM_SOFTMAX_TWO_BLOCKS_MAX_V
-#define ROWNORM_SOFTMAX_TWO_BLOCKS_MAX_V 8
+#define ROWNORM_SOFTMAX_TWO_BLOCKS_MAX_V 9
 #endif
+constexpr int kSoftmaxFreshOffsetsMaxV = ROWNORM_SOFTMAX_TWO_BLOCKS_MAX_V;
 template <class TI, int G, int V, bool FAST, bool MASKED>
 constexpr int softmax_fwd_min_blocks() {
   return (G == 1024 && FAST && !MASKED && V >= 5 && V <= ROWNORM_SOFTMAX_TWO_BLOCKS_MAX_V) ? 8 : 1;
@@ -142,11 +143,21 @@ softmax_fwd_resident_kernel(const TI* __restrict__ x, TO* __restrict__ y, MaskRe
   __shared__ float red[reduce_lds_floats<G, BLOCK, 1>::value];
   int phase = 0;
   const int slot = threadIdx.x / G;
-  const int lane = threadIdx.x % G;
+  const int lane0 = threadIdx.x % G;
   const bool is_log = (flags & kSoftmaxLog) != 0;
   const bool is_safe = (flags & kSoftmaxSafe) != 0;
   const int64_t nrb = (M + RPB - 1) / RPB;
   for (int64_t rb = blockIdx.x; rb < nrb; rb += gridDim.x) {
+    // The lane index is made opaque once a row and again before the stores: the
+    // V pack offsets derive from it, and the compiler would otherwise compute
+    // them all before the loop and hold a register or two a pack for the whole
+    // kernel (at 8 and 9 packs a lane that decides whether two workgroups fit a
+    // compute unit: 65536-element bf16 rows 220 -> 188 us, 73728 258 -> 215 us;
+    // ragged rows drop from 94 to 54 registers).  From 10 packs a lane one
+    // workgroup a compute unit is the better layout for log_softmax, and there
+    // recomputing the offsets measured 1-2 % slower, so those keep them.
+    constexpr bool kFreshOffsets = !(FAST && G == 1024 && V > kSoftmaxFreshOffsetsMaxV);
+    const int lane = lane_again<kFreshOffsets>(lane0);
     const int64_t row = rb * RPB + slot;
     const bool ok = RPB == 1 ? true : row < M;
     const int64_t rowc = ok ? row : 0;
@@ -232,18 +243,20 @@ softmax_fwd_resident_kernel(const TI* __restrict__ x, TO* __restrict__ y, MaskRe
       }
       if (is_log) {
         ROWNORM_UNIFORM_ARM("log_softmax: x - max - log(sum)");
-        const float k = logf(sum[0]);
+        float k = logf(sum[0]);
+        const int ls = lane_after<kFreshOffsets>(lane0, k);
 #pragma unroll
         for (int c = 0; c < V; ++c) {
           keep_packed(xp[c]);
           Pack<TO, E> o;
 #pragma unroll
           for (int i = 0; i < E; ++i) o.set(i, (xp[c].get(i) - m) - k);
-          row_store<TO, E, true, FAST>(yr, (c * G + lane) * E, nw, ok, o, h);
+          row_store<TO, E, true, FAST>(yr, (c * G + ls) * E, nw, ok, o, h);
         }
       } else if (is_safe) {
         ROWNORM_UNIFORM_ARM("safe softmax: zeros for a row without a finite element");
-        const float k = 1.0f / sum[0];
+        float k = 1.0f / sum[0];
+        const int ls = lane_after<kFreshOffsets>(lane0, k);
         const bool zero_row = m == -INFINITY;
 #pragma unroll
         for (int c = 0; c < V; ++c) {
@@ -252,18 +265,19 @@ softmax_fwd_resident_kernel(const TI* __restrict__ x, TO* __restrict__ y, MaskRe
 #pragma unroll
           for (int i = 0; i < E; ++i)
             o.set(i, zero_row ? 0.0f : row_exp<PRECISE>(xp[c].get(i) - m) * k);
-          row_store<TO, E, true, FAST>(yr, (c * G + lane) * E, nw, ok, o, h);
+          row_store<TO, E, true, FAST>(yr, (c * G + ls) * E, nw, ok, o, h);
         }
       } else {
         ROWNORM_UNIFORM_ARM("softmax: exp(x - max) / sum");
-        const float k = 1.0f / sum[0];
+        float k = 1.0f / sum[0];
+        const int ls = lane_after<kFreshOffsets>(lane0, k);
 #pragma unroll
         for (int c = 0; c < V; ++c) {
           keep_packed(xp[c]);
           Pack<TO, E> o;
 #pragma unroll
           for (int i = 0; i < E; ++i) o.set(i, row_exp<PRECISE>(xp[c].get(i) - m) * k);
-          row_store<TO, E, true, FAST>(yr, (c * G + lane) * E, nw, ok, o, h);
+          row_store<TO, E, true, FAST>(yr, (c * G + ls) * E, nw, ok, o, h);
         }
       }
       continue;
@@ -313,34 +327,37 @@ softmax_fwd_resident_kernel(const TI* __restrict__ x, TO* __restrict__ y, MaskRe
     group_allreduce<G, BLOCK, 1, SumOp>(sum, red, phase);
     if (is_log) {
       ROWNORM_UNIFORM_ARM("log_softmax: (x - max) - log(sum)");
-      const float k = logf(sum[0]);
+      float k = logf(sum[0]);
+      const int ls = lane_after<kFreshOffsets>(lane0, k);
 #pragma unroll
       for (int c = 0; c < V; ++c) {
         Pack<TO, E> o;
 #pragma unroll
         for (int i = 0; i < E; ++i) o.set(i, xf[c][i] - k);
-        row_store<TO, E, true, FAST>(yr, (c * G + lane) * E, nw, ok, o, h);
+        row_store<TO, E, true, FAST>(yr, (c * G + ls) * E, nw, ok, o, h);
       }
     } else if (is_safe) {
       ROWNORM_UNIFORM_ARM("safe softmax: zeros for a row without a finite element");
-      const float k = 1.0f / sum[0];
+      float k = 1.0f / sum[0];
+      const int ls = lane_after<kFreshOffsets>(lane0, k);
       const bool zero_row = m == -INFINITY;
 #pragma unroll
       for (int c = 0; c < V; ++c) {
         Pack<TO, E> o;
 #pragma unroll
         for (int i = 0; i < E; ++i) o.set(i, zero_row ? 0.0f : xf[c][i] * k);
-        row_store<TO, E, true, FAST>(yr, (c * G + lane) * E, nw, ok, o, h);
+        row_store<TO, E, true, FAST>(yr, (c * G + ls) * E, nw, ok, o, h);
       }
     } else {
       ROWNORM_UNIFORM_ARM("softmax: exp(x - max) * (1 / sum)");
-      const float k = 1.0f / sum[0];
+      float k = 1.0f / sum[0];
+      const int ls = lane_after<kFreshOffsets>(lane0, k);
 #pragma unroll
       for (int c = 0; c < V; ++c) {
         Pack<TO, E> o;
 #pragma unroll
         for (int i = 0; i < E; ++i) o.set(i, xf[c][i] * k);
-        row_store<TO, E, true, FAST>(yr, (c * G + lane) * E, nw, ok, o, h);
+        row_store<TO, E, true, FAST>(yr, (c * G + ls) * E, nw, ok, o, h);
       }
     }
   }
@@ -464,12 +481,15 @@ softmax_bwd_resident_kernel(const TG* __restrict__ grad, const TG* __restrict__ 
   __shared__ float red[reduce_lds_floats<G, BLOCK, 1>::value];
   int phase = 0;
   const int slot = threadIdx.x / G;
-  const int lane = threadIdx.x % G;
+  const int lane0 = threadIdx.x % G;
   const bool is_log = (flags & kSoftmaxLog) != 0;
   // y's packs are aligned like grad's when the two base addresses are congruent
   const bool y_whole = WINDOW && same_pack_alignment(grad, y);
   const int64_t nrb = (M + RPB - 1) / RPB;
   for (int64_t rb = blockIdx.x; rb < nrb; rb += gridDim.x) {
+    // ragged rows: opaque once a row and again before the stores (see the forward;
+    // 8192 x 4097 bf16 49.6 -> 41.8 us); whole-pack rows measured 1 % slower with it
+    const int lane = lane_again<!FAST>(lane0);
     const int64_t row = rb * RPB + slot;
     const bool ok = RPB == 1 ? true : row < M;
     const int64_t rowc = ok ? row : 0;
@@ -524,7 +544,8 @@ softmax_bwd_resident_kernel(const TG* __restrict__ grad, const TG* __restrict__ 
         for (int i = 0; i < E; ++i) sum[0] = fmaf(yf[c][i], gf[c][i], sum[0]);
     }
     group_allreduce<G, BLOCK, 1, SumOp>(sum, red, phase);
-    const float s = sum[0];
+    float s = sum[0];
+    const int ls = lane_after<!FAST>(lane0, s);
     if (is_log) {
       ROWNORM_UNIFORM_ARM("log_softmax backward: grad - exp(y) * sum");
 #pragma unroll
@@ -532,7 +553,7 @@ softmax_bwd_resident_kernel(const TG* __restrict__ grad, const TG* __restrict__ 
         Pack<TO, E> o;
 #pragma unroll
         for (int i = 0; i < E; ++i) o.set(i, gf[c][i] - row_exp<PRECISE>(yf[c][i]) * s);
-        row_store<TO, E, true, FAST>(outr, (c * G + lane) * E, nw, ok, o, h);
+        row_store<TO, E, true, FAST>(outr, (c * G + ls) * E, nw, ok, o, h);
       }
     } else {
       ROWNORM_UNIFORM_ARM("softmax backward: y * (grad - sum)");
@@ -541,7 +562,7 @@ softmax_bwd_resident_kernel(const TG* __restrict__ grad, const TG* __restrict__ 
         Pack<TO, E> o;
 #pragma unroll
         for (int i = 0; i < E; ++i) o.set(i, yf[c][i] * (gf[c][i] - s));
-        row_store<TO, E, true, FAST>(outr, (c * G + lane) * E, nw, ok, o, h);
+        row_store<TO, E, true, FAST>(outr, (c * G + ls) * E, nw, ok, o, h);
       }
     }
   }
