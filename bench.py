@@ -16,7 +16,8 @@ one mi355x_rms_norm_bwd call (norm_bwd_resident_kernel + colsum_finalize_kernel)
 one HIP event pair on the launch stream around K back-to-back calls.  `cpu_baseline` is the scalar C oracle
 (oracle/, a port of the same arithmetic) timed on one host core; `cpu_aten` is PyTorch's CPU ATen
 path (the parity target) on all host cores.  `stock_pytorch_rocm` is the same step through the
-kernels PyTorch-ROCm ships, on the same GPU.  `ops` lists every op of the family at its
+kernels PyTorch-ROCm ships, on the same GPU; `device_copy` is what a plain device-to-device copy
+reaches at the same tensor sizes.  `ops` lists every op of the family at its
 Llama-class configuration, `min_frac_llama_ops` the worst of configurations 2-4 (the target is
 0.70), `reference_microbench` the shapes of the reference's own micro-benchmarks and `config5`
 the irregular shapes of configuration 5 (all informational, measured after the timed region).
@@ -203,6 +204,7 @@ def main():
 
     if not args.no_ops:
         out["stock_pytorch_rocm"] = stock_step(torch, sets, w, M, N, eps, fwd_bytes + bwd_bytes)
+        out["device_copy"] = device_copy_table(torch, dev, M, N)
         out["ops"] = per_op_table(torch, cabi, L, dev, stream, P)
         # the target of this operator family is one number: every op at its Llama-class bf16
         # configuration (2, 3 and 4) at or above 70 % of the HBM peak
@@ -227,6 +229,28 @@ def calibrate_copy(torch, dev):
     for _ in range(10):
         dst.copy_(src)
     torch.cuda.synchronize()
+
+
+def device_copy_table(torch, dev, M, N):
+    """What a plain device-to-device copy (torch's `copy_`) reaches on this GPU, measured like the
+    ops (HIP events over back-to-back calls, rotating over three buffer pairs): bytes read + bytes
+    written over time, at the size of the benchmark's tensor and at the sizes of the largest
+    tensors in the per-op table.  A copy is the simplest kernel with this family's traffic
+    pattern, so its rate says how much of the 8 TB/s peak a streaming kernel can get here."""
+    rows = []
+    for label, nelem in (("bf16 [%d, %d]" % (M, N), M * N), ("bf16 [16384, 8192]", 16384 * 8192),
+                         ("bf16 [4, 32, 2048, 2048]", 4 * 32 * 2048 * 2048)):
+        pairs = []
+        for _ in range(3):
+            src = torch.empty(nelem, dtype=torch.bfloat16, device=dev).normal_()
+            pairs.append((src, torch.empty_like(src)))
+        us = _time_rotating(torch, [(lambda s=s, d=d: d.copy_(s)) for s, d in pairs], iters=40, warm=10)
+        gbs = 2 * nelem * 2 / us / 1e3
+        rows.append({"tensor": label, "us": round(us, 2), "GB/s": round(gbs, 1),
+                     "frac": round(gbs / HBM_PEAK_GBS, 4)})
+        del pairs
+        torch.cuda.empty_cache()
+    return {"what": "torch copy_ of a tensor of that size: bytes read + written over time", "rows": rows}
 
 
 def stock_step(torch, sets, w, M, N, eps, step_bytes):
