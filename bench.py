@@ -585,14 +585,14 @@ def per_op_table(torch, cabi, L, dev, stream, P, only=None, iters=60, warm=30):
 
 def width_sweep_table(torch, cabi, L, dev, stream, P, only=None):
     """LayerNorm and RMSNorm forward and backward over the hidden sizes of the Llama-class models
-    (4096 ... 12288, 16384 tokens, bf16 rows; bf16 weights, and float32 weights for LayerNorm):
+    (4096 ... 16384, 16384 tokens, bf16 rows; bf16 weights, and float32 weights for LayerNorm):
     avg microseconds per call (60 back-to-back calls after 30, three buffer sets), algorithmic GB/s
     and the fraction of 8 TB/s.  `min_frac` of the returned dict is the worst of them."""
     BF, F32 = cabi.BF16, cabi.F32
     bf16 = torch.bfloat16
     M = 16384
     rows = []
-    for N in (4096, 5120, 6144, 8192, 10240, 12288):
+    for N in (4096, 5120, 6144, 8192, 10240, 12288, 16384):
         sets = []
         for _ in range(3):
             x = torch.randn(M, N, device=dev).to(bf16)

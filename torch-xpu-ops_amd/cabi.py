@@ -167,7 +167,7 @@ def group_norm_plan(backward, N, C, HxW, groups, dtype=F32):
     _check(lib().mi355x_group_norm_plan(int(backward), N, C, HxW, groups, dtype, ctypes.byref(p)),
            "group_norm_plan")
     d = p.as_dict()
-    d["uniform"] = p.reserved
+    d["uniform"] = p.reserved  # 1: every pack in one channel, 2: packs may straddle two, 0: general kernels
     return d
 
 

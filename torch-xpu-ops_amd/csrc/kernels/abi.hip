@@ -404,11 +404,12 @@ int group_dims(int64_t N, int64_t C, int64_t HxW, int64_t groups, GroupDims* out
   return 0;
 }
 
-// The general kernels are taken whenever a pack could straddle two channels.
+// The general kernels are taken when neither every pack lies in one channel nor
+// the straddling kernels apply (gn_mode, plan.hpp).
 int group_plan(OpClass oc, int op, const GroupDims& d, int64_t HxW, int esize, Plan* plan) {
   const int E = 16 / esize;
   return make_plan(oc, d.rows, d.L, esize, current_num_cus(), g_override[op], false, plan,
-                   HxW % E != 0);
+                   gn_mode(d.L, HxW, d.D, E) == kGnGeneral);
 }
 
 int softmax_mode_flags(int mode, bool forward, int* flags) {
@@ -673,7 +674,7 @@ int mi355x_group_norm_plan(int backward, int64_t N, int64_t C, int64_t HxW, int6
   out->packs_per_lane = plan.V;
   out->block_threads = plan.block;
   out->rows_per_block = plan.rpb;
-  out->reserved = plan.fast ? 1 : 0;
+  out->reserved = plan.fast ? gn_mode(d.L, HxW, d.D, 16 / esize_of((int)x_dtype)) : kGnGeneral;
   out->grid_blocks = plan.grid;
   out->partial_rows = backward ? N : 0;
   return 0;

@@ -10,12 +10,20 @@
 // the per-(n, channel) sums of dY * xhat and dY in an fp32 [N, C] workspace that
 // colsum_finalize_kernel adds up over n.
 //
-// UNIFORM: HxW is a whole number of packs, so every pack lies in one channel
-// (one weight lookup per pack, branch-free row access, channel sums fused into
-// the backward through an LDS staging area).  Otherwise the channel is looked
-// up per element, row access is the general one, and the channel sums come
-// from gn_channel_sums_kernel, which reads dY and X a second time.  Rows too
-// long for the registers: the forward takes two passes over the row; the
+// Three kinds of resident kernel (MODE):
+//   kGnUniform   HxW is a whole number of packs, so every pack lies in one
+//                channel: one weight lookup per pack, branch-free row access,
+//                channel sums fused into the backward through an LDS staging area.
+//   kGnStraddle  rows are whole packs (L % E == 0) but channels are not (7x7 and
+//                14x14 feature maps in 16 bits): a pack lies in one channel or
+//                straddles the border of two, so it looks up two weights and each
+//                element selects; row access and the fused channel sums as above,
+//                the part of a straddling pack that belongs to the next channel
+//                travels through a small LDS array of its own.
+//   kGnGeneral   anything else: the channel is looked up per element, row access
+//                is the general one, and the channel sums come from
+//                gn_channel_sums_kernel, which reads dY and X a second time.
+// Rows too long for the registers: the forward takes two passes over the row; the
 // backward computes the channel sums first and dX from them, element by element.
 //
 // What these stand in for in the reference (src/ATen/native/xpu/sycl/
@@ -56,7 +64,11 @@ struct GroupShape {
   // rows whose channels are whole packs (HxW % E == 0), else both 0:
   int packs;            // packs per row, L / E
   unsigned pack_magic;  // ceil(2^31 / (HxW / E)), see gn_pack_channel
+  // rows of whole packs whose channels are not (kGnStraddle), else 0:
+  unsigned elem_magic;  // ceil(2^32 / HxW), see gn_straddle
 };
+
+
 
 // Wavefronts per SIMD a resident kernel is compiled for (the second argument of
 // __launch_bounds__): the 512-lane layouts with 6 packs or more that the
@@ -82,6 +94,23 @@ __device__ __forceinline__ int gn_pack_channel(const GroupShape& s, int g, int p
   return g * s.D + (int)__umulhi(2u * (unsigned)pc, s.pack_magic);
 }
 
+// Where the pack at element e0 of a row lies among the channels when channels
+// are not whole packs: `ch` = channel (within the group) of its first element,
+// `bnd` = how many of its elements belong to that channel (>= E: all of them;
+// the others belong to channel ch + 1).  HxW >= E, so a pack meets one border
+// at most.  e0 / HxW is floor(e0 * ceil(2^32 / HxW) / 2^32), exact while
+// e0 * HxW < 2^32, and a register-resident row has at most 2^16 elements.
+struct GnStraddle {
+  int ch, bnd;
+};
+__device__ __forceinline__ GnStraddle gn_straddle(const GroupShape& s, int e0, int E) {
+  const int ec = e0 < s.L ? e0 : s.L - E;  // packs past the row end: any pack of the row
+  GnStraddle r;
+  r.ch = (int)__umulhi((unsigned)ec, s.elem_magic);
+  r.bnd = (r.ch + 1) * s.HxW - ec;
+  return r;
+}
+
 template <class WT>
 __device__ __forceinline__ float gn_weight(const WT* w, int ch, float dflt) {
   return w ? (float)w[(unsigned)ch] : dflt;  // ch >= 0: a 32-bit offset from a scalar base
@@ -92,13 +121,15 @@ __device__ __forceinline__ float gn_weight(const WT* w, int ch, float dflt) {
 // a centre mean0, centred sums over the registers, mean = mean0 + s1/L,
 // var = (s2 - s1*s1/L)/L; y uses (x - mean0) - s1/L so that a constant row
 // gives beta bit for bit.
-template <class T, class WT, int G, int V, int BLOCK, bool UNIFORM>
+template <class T, class WT, int G, int V, int BLOCK, int MODE>
 __global__ void __launch_bounds__(BLOCK, gn_min_waves(G, V, group_half_lanes_max_v(OC_GROUP_FWD)))
 gn_fwd_resident_kernel(const T* __restrict__ x, const WT* __restrict__ gamma,
                        const WT* __restrict__ beta, T* __restrict__ y, WT* __restrict__ mean,
                        WT* __restrict__ rstd, int64_t rows, GroupShape s, float eps) {
   constexpr int E = elems_per_pack<T>::value;
   constexpr int RPB = BLOCK / G;
+  constexpr bool UNIFORM = MODE != kGnGeneral;  // rows of whole packs: branch-free row access
+  constexpr bool STRADDLE = MODE == kGnStraddle;
   __shared__ float red[reduce_lds_floats<G, BLOCK, 2>::value];
   int phase = 0;
   const int slot = threadIdx.x / G;
@@ -171,7 +202,18 @@ gn_fwd_resident_kernel(const T* __restrict__ x, const WT* __restrict__ gamma,
       keep_packed(xp[c]);
       const int e0 = (c * G + lane) * E;
       Pack<T, E> o;
-      if constexpr (UNIFORM) {
+      if constexpr (STRADDLE) {
+        const GnStraddle w = gn_straddle(s, e0, E);
+        const int c0 = g * s.D + w.ch;
+        const int c1 = w.ch + 1 < s.D ? c0 + 1 : c0;
+        const float ga0 = gn_weight(gamma, c0, 1.0f) * rs, ga1 = gn_weight(gamma, c1, 1.0f) * rs;
+        const float be0 = gn_weight(beta, c0, 0.0f), be1 = gn_weight(beta, c1, 0.0f);
+#pragma unroll
+        for (int i = 0; i < E; ++i) {
+          const bool first = i < w.bnd;
+          o.set(i, ((xp[c].get(i) - mean0) - m1) * (first ? ga0 : ga1) + (first ? be0 : be1));
+        }
+      } else if constexpr (UNIFORM) {
         const int ch = gn_pack_channel(s, g, c * G + lane);
         const float ga = gn_weight(gamma, ch, 1.0f) * rs;
         const float be = gn_weight(beta, ch, 0.0f);
@@ -262,16 +304,25 @@ gn_fwd_stream_kernel(const T* __restrict__ x, const WT* __restrict__ gamma,
 }
 
 // ---------------------------------------------------------------------------
-// Backward, rows resident in registers.  With UNIFORM and a workspace, each
-// lane parks the sums of dy*xhat and dy over each of its packs in LDS; after a
-// barrier the channels of the row are summed from there in a fixed order (TPC
-// lanes per channel, then a butterfly) and written to part_dg / part_db [N, C].
-template <int G, int V, int BLOCK, bool UNIFORM>
+// Backward, rows resident in registers.  With rows of whole packs and a
+// workspace, each lane parks the sums of dy*xhat and dy over each of its packs
+// in LDS; after a barrier the channels of the row are summed from there in a
+// fixed order (TPC lanes per channel, then a butterfly) and written to part_dg /
+// part_db [N, C].  kGnStraddle: a pack parks the sums over its elements of its
+// first channel; what a straddling pack holds of the next channel goes to that
+// channel's slot of a second array (one straddling pack per channel border, so
+// one writer per slot), which the channel's fold adds when the channel does not
+// start on a pack.
+template <int G, int V, int BLOCK, int MODE>
 struct gn_stage_floats {
-  static constexpr int value = UNIFORM ? 2 * BLOCK * V : 1;
+  static constexpr int value = MODE != kGnGeneral ? 2 * BLOCK * V : 1;
+  // per row slot: two floats for each channel the slot's row can have
+  static constexpr int next_per_slot =
+      MODE == kGnStraddle ? 2 * (G * V < kGnStraddleMaxD ? G * V : kGnStraddleMaxD) : 0;
+  static constexpr int next_value = MODE == kGnStraddle ? (BLOCK / G) * next_per_slot : 1;
 };
 
-template <class T, class WT, int G, int V, int BLOCK, bool UNIFORM>
+template <class T, class WT, int G, int V, int BLOCK, int MODE>
 __global__ void __launch_bounds__(BLOCK, gn_min_waves(G, V, group_half_lanes_max_v(OC_GROUP_BWD)))
 gn_bwd_resident_kernel(const T* __restrict__ dy, const T* __restrict__ x,
                        const WT* __restrict__ mean, const WT* __restrict__ rstd,
@@ -280,8 +331,11 @@ gn_bwd_resident_kernel(const T* __restrict__ dy, const T* __restrict__ x,
                        GroupShape s, int tpc_log2) {
   constexpr int E = elems_per_pack<T>::value;
   constexpr int RPB = BLOCK / G;
+  constexpr bool UNIFORM = MODE != kGnGeneral;  // rows of whole packs, fused channel sums
+  constexpr bool STRADDLE = MODE == kGnStraddle;
   __shared__ float red[reduce_lds_floats<G, BLOCK, 2>::value];
-  __shared__ float stage[gn_stage_floats<G, V, BLOCK, UNIFORM>::value];
+  __shared__ float stage[gn_stage_floats<G, V, BLOCK, MODE>::value];
+  __shared__ float stage_next[gn_stage_floats<G, V, BLOCK, MODE>::next_value];
   int phase = 0;
   const int slot = threadIdx.x / G;
   const int lane0 = threadIdx.x % G;
@@ -311,11 +365,43 @@ gn_bwd_resident_kernel(const T* __restrict__ dy, const T* __restrict__ x,
     }
     float acc[2] = {0.0f, 0.0f};
     float gu[UNIFORM ? V : 1];  // the weight of each pack, looked up once a row
+    float gv[STRADDLE ? V : 1];  // kGnStraddle: the weight of the pack's second channel
+    int bnd[STRADDLE ? V : 1];   //              and the elements that belong to the first
     float* st = stage + slot * (UNIFORM ? 2 * G * V : 0);
+    float* sn = stage_next + slot * gn_stage_floats<G, V, BLOCK, MODE>::next_per_slot;
 #pragma unroll
     for (int c = 0; c < V; ++c) {
       const int e0 = (c * G + lane) * E;
-      if constexpr (UNIFORM) {
+      if constexpr (STRADDLE) {
+        const GnStraddle w = gn_straddle(s, e0, E);
+        const bool has_next = w.bnd < E && w.ch + 1 < s.D;
+        const float ga = gu[c] = gn_weight(gamma, g * s.D + w.ch, 1.0f);
+        const float gb = gv[c] = gn_weight(gamma, g * s.D + (has_next ? w.ch + 1 : w.ch), 1.0f);
+        bnd[c] = w.bnd;
+        float pdg = 0.0f, pdb = 0.0f, fdg = 0.0f, fdb = 0.0f;  // whole pack / first channel
+#pragma unroll
+        for (int i = 0; i < E; ++i) {
+          const float gy = dp[c].get(i);
+          const float t = gy * (xp[c].get(i) - mu);
+          pdb += gy;
+          pdg += t;
+          fdb += i < w.bnd ? gy : 0.0f;
+          fdg += i < w.bnd ? t : 0.0f;
+        }
+        // (a pack that lies in one channel adds the same terms to both pairs: the
+        // second channel's share is then exactly zero)
+        const float ndg = pdg - fdg, ndb = pdb - fdb;
+        acc[0] = fmaf(fdb, ga, fmaf(ndb, gb, acc[0]));
+        acc[1] = fmaf(fdg * rs, ga, fmaf(ndg * rs, gb, acc[1]));
+        if (want_cols) {
+          st[2 * (c * G + lane)] = fdg * rs;
+          st[2 * (c * G + lane) + 1] = fdb;
+          if (has_next && e0 < s.L) {
+            sn[2 * (w.ch + 1)] = ndg * rs;
+            sn[2 * (w.ch + 1) + 1] = ndb;
+          }
+        }
+      } else if constexpr (UNIFORM) {
         const float ga = gu[c] = gn_weight(gamma, gn_pack_channel(s, g, c * G + lane), 1.0f);
         float pdg = 0.0f, pdb = 0.0f;
 #pragma unroll
@@ -357,13 +443,17 @@ gn_bwd_resident_kernel(const T* __restrict__ dy, const T* __restrict__ x,
         keep_packed(dp[c]);
         const int e0 = (c * G + lane) * E;
         const float gr = UNIFORM ? gu[c] * rs : 0.0f;
+        const float gq = STRADDLE ? gv[c] * rs : 0.0f;
         Pack<T, E> o;
 #pragma unroll
         for (int i = 0; i < E; ++i) {
           if constexpr (UNIFORM && sizeof(T) == 2) {
-            o.set(i, fmaf(xp[c].get(i), -ra, fmaf(dp[c].get(i), gr, cc)));
+            const float gri = STRADDLE ? (i < bnd[c] ? gr : gq) : gr;
+            o.set(i, fmaf(xp[c].get(i), -ra, fmaf(dp[c].get(i), gri, cc)));
           } else {
-            const float ga = UNIFORM ? gu[c] : gn_weight(gamma, gn_channel(s, g, e0 + i), 1.0f);
+            const float ga = STRADDLE ? (i < bnd[c] ? gu[c] : gv[c])
+                             : UNIFORM ? gu[c]
+                                       : gn_weight(gamma, gn_channel(s, g, e0 + i), 1.0f);
             const float xh = (xp[c].get(i) - mu) * rs;
             float f = fL * (dp[c].get(i) * ga);
             f -= xh * s2;
@@ -377,7 +467,9 @@ gn_bwd_resident_kernel(const T* __restrict__ dy, const T* __restrict__ x,
     if constexpr (UNIFORM) {
       if (want_cols) {
         __syncthreads();
-        // channel d of the row owns packs [d * S, (d + 1) * S), S = HxW / E
+        // channel d of the row owns packs [d * S, (d + 1) * S), S = HxW / E; with
+        // straddling packs, the packs whose first element lies in it:
+        // [ceil(d * HxW / E), ceil((d + 1) * HxW / E))
         const int S = s.HxW / E;
         const int TPC = 1 << tpc_log2;  // lanes per channel, power of two <= min(G, 64)
         const int sub = lane & (TPC - 1);
@@ -386,9 +478,18 @@ gn_bwd_resident_kernel(const T* __restrict__ dy, const T* __restrict__ x,
           const int d = d0 + (lane >> tpc_log2);
           float ag = 0.0f, ab = 0.0f;
           if (d < s.D) {
-            for (int q = d * S + sub; q < (d + 1) * S; q += TPC) {
+            const int q0 = STRADDLE ? (d * s.HxW + E - 1) / E : d * S;
+            const int q1 = STRADDLE ? ((d + 1) * s.HxW + E - 1) / E : (d + 1) * S;
+            for (int q = q0 + sub; q < q1; q += TPC) {
               ag += st[2 * q];
               ab += st[2 * q + 1];
+            }
+            if constexpr (STRADDLE) {
+              // the channel starts inside a pack: that pack's share of it
+              if (sub == 0 && (d * s.HxW) % E != 0) {
+                ag += sn[2 * d];
+                ab += sn[2 * d + 1];
+              }
             }
           }
           for (int off = TPC >> 1; off > 0; off >>= 1) {

@@ -8,11 +8,14 @@ namespace rownorm {
 
 // E: elements per pack of the row dtype.
 inline GroupShape group_shape(int L, int HxW, int D, int groups, int E) {
-  GroupShape s{L, HxW, D, groups, 0, 0u};
-  if (HxW % E == 0) {
+  GroupShape s{L, HxW, D, groups, 0, 0u, 0u};
+  const int mode = gn_mode(L, HxW, D, E);
+  if (mode == kGnUniform) {
     const uint64_t per_channel = (uint64_t)(HxW / E);
     s.packs = L / E;
     s.pack_magic = (unsigned)((((uint64_t)1 << 31) + per_channel - 1) / per_channel);
+  } else if (mode == kGnStraddle) {
+    s.elem_magic = (unsigned)((((uint64_t)1 << 32) + (uint64_t)HxW - 1) / (uint64_t)HxW);
   }
   return s;
 }
@@ -24,15 +27,15 @@ struct GroupNormFwdCtx {
   hipStream_t stream;
 };
 
-template <class T, class WT, bool UNIFORM>
+template <class T, class WT, int MODE>
 struct GroupNormFwdLauncher {
   template <int G, int V, int BLOCK>
   struct At {
     static bool run(const GroupNormFwdCtx<T, WT>& c) {
-      if constexpr (variant_built(OC_GROUP_FWD, sizeof(T), G, V, UNIFORM) &&
+      if constexpr (variant_built(OC_GROUP_FWD, sizeof(T), G, V, MODE != kGnGeneral) &&
                     block_built(OC_GROUP_FWD, G, BLOCK)) {
         if (c.plan.G == G && c.plan.V == V && c.plan.block == BLOCK) {
-          hipLaunchKernelGGL((gn_fwd_resident_kernel<T, WT, G, V, BLOCK, UNIFORM>),
+          hipLaunchKernelGGL((gn_fwd_resident_kernel<T, WT, G, V, BLOCK, MODE>),
                              dim3((unsigned)c.plan.grid), dim3(BLOCK), 0, c.stream,
                              (const T*)c.a.x, (const WT*)c.a.gamma, (const WT*)c.a.beta,
                              (T*)c.a.y, (WT*)c.a.mean, (WT*)c.a.rstd, c.a.rows,
@@ -49,9 +52,11 @@ template <class T, class WT>
 int launch_group_norm_fwd(const Plan& plan, const GroupNormFwdArgs& a, hipStream_t stream) {
   if (plan.resident) {
     GroupNormFwdCtx<T, WT> ctx{plan, a, stream};
+    const int mode = plan.fast ? gn_mode(a.L, a.HxW, a.D, elems_per_pack<T>::value) : kGnGeneral;
     const bool launched =
-        plan.fast ? launch_variant<GroupNormFwdLauncher<T, WT, true>::template At>(ctx)
-                  : launch_variant<GroupNormFwdLauncher<T, WT, false>::template At>(ctx);
+        mode == kGnUniform    ? launch_variant<GroupNormFwdLauncher<T, WT, kGnUniform>::template At>(ctx)
+        : mode == kGnStraddle ? launch_variant<GroupNormFwdLauncher<T, WT, kGnStraddle>::template At>(ctx)
+                              : launch_variant<GroupNormFwdLauncher<T, WT, kGnGeneral>::template At>(ctx);
     if (!launched) return (int)hipErrorInvalidConfiguration;
   } else {
     hipLaunchKernelGGL((gn_fwd_stream_kernel<T, WT, kStreamBlock>), dim3((unsigned)plan.grid),
@@ -70,15 +75,15 @@ struct GroupNormBwdCtx {
   hipStream_t stream;
 };
 
-template <class T, class WT, bool UNIFORM>
+template <class T, class WT, int MODE>
 struct GroupNormBwdLauncher {
   template <int G, int V, int BLOCK>
   struct At {
     static bool run(const GroupNormBwdCtx<T, WT>& c) {
-      if constexpr (variant_built(OC_GROUP_BWD, sizeof(T), G, V, UNIFORM) &&
+      if constexpr (variant_built(OC_GROUP_BWD, sizeof(T), G, V, MODE != kGnGeneral) &&
                     block_built(OC_GROUP_BWD, G, BLOCK)) {
         if (c.plan.G == G && c.plan.V == V && c.plan.block == BLOCK) {
-          hipLaunchKernelGGL((gn_bwd_resident_kernel<T, WT, G, V, BLOCK, UNIFORM>),
+          hipLaunchKernelGGL((gn_bwd_resident_kernel<T, WT, G, V, BLOCK, MODE>),
                              dim3((unsigned)c.plan.grid), dim3(BLOCK), 0, c.stream,
                              (const T*)c.a.dy, (const T*)c.a.x, (const WT*)c.a.mean,
                              (const WT*)c.a.rstd, (const WT*)c.a.gamma, (T*)c.a.dx, c.a.part_dg,
@@ -136,9 +141,11 @@ int launch_group_norm_bwd(const Plan& plan, const GroupNormBwdArgs& a, hipStream
       if (!want_cols || !fused_cols) k.part_dg = k.part_db = nullptr;
       GroupNormBwdCtx<T, WT> ctx{plan, k, 0, stream};
       if (plan.fast) ctx.tpc_log2 = gn_tpc_log2(plan.G, a.D, a.HxW / E);
+      const int mode = plan.fast ? gn_mode(a.L, a.HxW, a.D, E) : kGnGeneral;
       const bool launched =
-          plan.fast ? launch_variant<GroupNormBwdLauncher<T, WT, true>::template At>(ctx)
-                    : launch_variant<GroupNormBwdLauncher<T, WT, false>::template At>(ctx);
+          mode == kGnUniform    ? launch_variant<GroupNormBwdLauncher<T, WT, kGnUniform>::template At>(ctx)
+          : mode == kGnStraddle ? launch_variant<GroupNormBwdLauncher<T, WT, kGnStraddle>::template At>(ctx)
+                                : launch_variant<GroupNormBwdLauncher<T, WT, kGnGeneral>::template At>(ctx);
       if (!launched) return (int)hipErrorInvalidConfiguration;
     }
   } else if (a.dx != nullptr) {

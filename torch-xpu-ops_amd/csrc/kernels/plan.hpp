@@ -152,6 +152,18 @@ constexpr int default_bpc(OpClass oc, int block) {
 // dispatcher, the planner and the forced-variant check agree.
 constexpr bool is_group_class(OpClass oc) { return oc == OC_GROUP_FWD || oc == OC_GROUP_BWD; }
 
+// Kinds of register-resident GroupNorm kernel (see groupnorm_kernels.hpp) and the
+// rule that picks one for a shape; E = elements per 16-byte pack of the row dtype.
+constexpr int kGnGeneral = 0, kGnUniform = 1, kGnStraddle = 2;
+// Channels per group up to which the straddling kernels are taken (their LDS
+// array for the parts of packs that belong to the next channel).
+constexpr int kGnStraddleMaxD = 64;
+constexpr int gn_mode(int64_t L, int64_t HxW, int64_t D, int E) {
+  if (HxW % E == 0) return kGnUniform;
+  if (L % E == 0 && HxW >= E && D <= kGnStraddleMaxD) return kGnStraddle;
+  return kGnGeneral;
+}
+
 // GroupNorm rows that would spread over 1024 lanes (one workgroup a compute
 // unit, whose load, reduce and store phases then run one after the other) take
 // 512 lanes with twice the packs instead while two such workgroups fit a compute
