@@ -55,6 +55,9 @@ struct Plan {
   // softmax backward of rows beyond the registers of two tensors: grad alone fits
   // them (the log_softmax backward then keeps grad resident and streams y)
   bool grad_resident = false;
+  // a layout was asked for by override: kernels chosen by other means than the
+  // layout (softmax of short ragged rows through LDS) stand back
+  bool forced = false;
 };
 
 constexpr int kMinG = 8;
@@ -297,6 +300,7 @@ inline int make_plan(OpClass oc, int64_t M, int64_t N, int esize, int num_cus, c
   Plan p;
   const int E = 16 / esize;
   p.fast = (N % E) == 0 && !force_general;
+  p.forced = ov.G != 0 || ov.V != 0 || ov.block != 0;
   const bool softmax = oc == OC_SOFTMAX_FWD || oc == OC_SOFTMAX_BWD;
   // the general softmax kernels address a 16-bit row through the 16-byte aligned
   // window that holds it, which starts up to E - 1 elements before the row

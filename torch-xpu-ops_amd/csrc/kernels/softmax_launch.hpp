@@ -33,8 +33,77 @@ struct SoftmaxFwdLauncher {
   };
 };
 
+// Short ragged rows through LDS (softmax_fwd_flat_kernel): lanes per row, or 0
+// when the call does not qualify.
+template <class T>
+inline int flat_lanes(const Plan& plan, int64_t M, int N, const void* p0, const void* p1,
+                      const void* p2) {
+  if (plan.fast || plan.forced || M < 1 || N > 64 * flat_max_k<T>()) return 0;
+  if ((((uintptr_t)p0) | ((uintptr_t)p1) | ((uintptr_t)p2)) & 15) return 0;
+  int g = 8;
+  while (g * flat_max_k<T>() < N) g <<= 1;
+  return g;
+}
+
+template <class T>
+bool launch_softmax_fwd_flat(int g, const SoftmaxFwdArgs& a, hipStream_t stream) {
+  const int cr = flat_chunk_rows<T>(a.N, g, kFlatLdsBytes);
+  if (cr < 8) return false;
+  const int64_t grid = (a.M + cr - 1) / cr;
+  if (grid > 0x7fffffff) return false;
+#define ROWNORM_FLAT_FWD(GL)                                                                \
+  case GL:                                                                                  \
+    hipLaunchKernelGGL((softmax_fwd_flat_kernel<T, GL, kFlatBlock, kFlatLdsBytes>),          \
+                       dim3((unsigned)grid), dim3(kFlatBlock), 0, stream, (const T*)a.x,     \
+                       (T*)a.y, a.M, a.N, cr, a.flags);                                     \
+    return true;
+  switch (g) {
+    ROWNORM_FLAT_FWD(8)
+    ROWNORM_FLAT_FWD(16)
+    ROWNORM_FLAT_FWD(32)
+    ROWNORM_FLAT_FWD(64)
+  }
+#undef ROWNORM_FLAT_FWD
+  return false;
+}
+
+template <class T, int LDSB>
+bool launch_softmax_bwd_flat_l(int g, int cr, const SoftmaxBwdArgs& a, hipStream_t stream) {
+  const int64_t grid = (a.M + cr - 1) / cr;
+  if (grid > 0x7fffffff) return false;
+#define ROWNORM_FLAT_BWD(GL)                                                                 \
+  case GL:                                                                                   \
+    hipLaunchKernelGGL((softmax_bwd_flat_kernel<T, GL, kFlatBlock, LDSB>), dim3((unsigned)grid), \
+                       dim3(kFlatBlock), 0, stream, (const T*)a.grad, (const T*)a.y, (T*)a.gi, \
+                       a.M, a.N, cr, a.flags);                                               \
+    return true;
+  switch (g) {
+    ROWNORM_FLAT_BWD(8)
+    ROWNORM_FLAT_BWD(16)
+    ROWNORM_FLAT_BWD(32)
+    ROWNORM_FLAT_BWD(64)
+  }
+#undef ROWNORM_FLAT_BWD
+  return false;
+}
+
+template <class T>
+bool launch_softmax_bwd_flat(int g, const SoftmaxBwdArgs& a, hipStream_t stream) {
+  // half the LDS per tensor where that still holds a full pass of the lane groups' rows
+  const int rpb = kFlatBlock / g < 8 ? 8 : kFlatBlock / g;
+  const int half = flat_chunk_rows<T>(a.N, g, kFlatLdsBytes / 2);
+  if (half >= rpb) return launch_softmax_bwd_flat_l<T, kFlatLdsBytes / 2>(g, half, a, stream);
+  const int cr = flat_chunk_rows<T>(a.N, g, kFlatLdsBytes);
+  if (cr < 8) return false;
+  return launch_softmax_bwd_flat_l<T, kFlatLdsBytes>(g, cr, a, stream);
+}
+
 template <class TI, class TO, bool MASKED>
 int launch_softmax_fwd_m(const Plan& plan, const SoftmaxFwdArgs& a, hipStream_t stream) {
+  if constexpr (!MASKED && std::is_same<TI, TO>::value) {
+    const int g = flat_lanes<TI>(plan, a.M, a.N, a.x, a.y, nullptr);
+    if (g && launch_softmax_fwd_flat<TI>(g, a, stream)) return (int)hipGetLastError();
+  }
   if (plan.resident) {
     SoftmaxFwdCtx<TI, TO> ctx{plan, a, stream};
     const bool launched =
@@ -119,6 +188,10 @@ inline bool launch_log_softmax_bwd_grad_resident(const Plan& plan, const Softmax
 
 template <class TG, class TO, bool MASKED>
 int launch_softmax_bwd_m(const Plan& plan, const SoftmaxBwdArgs& a, hipStream_t stream) {
+  if constexpr (!MASKED && std::is_same<TG, TO>::value) {
+    const int g = flat_lanes<TG>(plan, a.M, a.N, a.grad, a.y, a.gi);
+    if (g && launch_softmax_bwd_flat<TG>(g, a, stream)) return (int)hipGetLastError();
+  }
   if (plan.resident) {
     SoftmaxBwdCtx<TG, TO> ctx{plan, a, stream};
     const bool launched =
