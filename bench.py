@@ -19,8 +19,10 @@ path (the parity target) on all host cores.  `stock_pytorch_rocm` is the same st
 kernels PyTorch-ROCm ships, on the same GPU; `device_copy` is what a plain device-to-device copy
 reaches at the same tensor sizes.  `ops` lists every op of the family at its
 Llama-class configuration, `min_frac_llama_ops` the worst of configurations 2-4 (the target is
-0.70), `reference_microbench` the shapes of the reference's own micro-benchmarks and `config5`
-the irregular shapes of configuration 5 (all informational, measured after the timed region).
+0.70), `reference_microbench` the shapes of the reference's own micro-benchmarks, `model_shapes`
+ragged and oversized shapes of common models (ViT / CLIP attention rows, GroupNorm over 14 x 14
+maps, a 151936-entry vocabulary) and `config5` the irregular shapes of configuration 5 (all
+informational, measured after the timed region).
 """
 import argparse
 import ctypes
@@ -116,6 +118,7 @@ def main():
         rows = per_op_table(torch, cabi, L, dev, stream, P, only=args.only_op,
                             iters=args.steps, warm=args.warmup)
         rows += reference_microbench_table(torch, cabi, L, dev, stream, P, only=args.only_op)
+        rows += model_shapes_table(torch, cabi, L, dev, stream, P, only=args.only_op)
         print(json.dumps({"ops": rows, "steps": args.steps, "warmup": args.warmup}))
         return
 
@@ -214,6 +217,7 @@ def main():
                                      "ops_counted": len(llama)}
         out["norm_width_sweep"] = width_sweep_table(torch, cabi, L, dev, stream, P)
         out["reference_microbench"] = reference_microbench_table(torch, cabi, L, dev, stream, P)
+        out["model_shapes"] = model_shapes_table(torch, cabi, L, dev, stream, P)
         out["config5"] = stress_table(torch, cabi, L, dev, stream, P)
     del sets
     if not args.no_cpu:
@@ -646,6 +650,93 @@ def width_sweep_table(torch, cabi, L, dev, stream, P, only=None):
         worst = min(rows, key=lambda r: r["frac"])
         out["min_frac"] = {"frac": worst["frac"], "op": worst["op"], "target": 0.70}
     return out
+
+
+def model_shapes_table(torch, cabi, L, dev, stream, P, only=None):
+    """Shapes of this op family in common models that are neither whole packs nor in the other
+    tables, bf16, forward and backward: attention scores of ViT-B/16 (rows of 197), ViT-L/14 at
+    336 px (577) and CLIP's text tower (77), which are ragged short rows; GroupNorm over 14 x 14
+    and 7 x 7 feature maps, whose channels are not whole packs; log_softmax over a 151936-entry
+    vocabulary (beyond what one workgroup's registers hold).  Algorithmic GB/s as everywhere;
+    `stock_us` = the kernels PyTorch-ROCm ships."""
+    BF = cabi.BF16
+    bf16 = torch.bfloat16
+    rows = []
+
+    def add(name, nbytes, fns, stock, iters=30):
+        if only is not None and not any(t in name for t in only.split("|")):
+            return
+        us = _time_rotating(torch, fns, iters=iters, warm=max(3, iters // 3))
+        row = {"op": name, "us": round(us, 2), "GB/s": round(nbytes / us / 1e3, 1),
+               "frac": round(nbytes / us / 1e3 / HBM_PEAK_GBS, 4)}
+        if only is None and stock is not None:
+            try:
+                row["stock_us"] = round(_time_rotating(torch, [stock], iters=max(3, iters // 4),
+                                                       warm=2), 2)
+            except Exception as e:
+                row["stock_us"] = None
+                row["stock_error"] = type(e).__name__
+        rows.append(row)
+
+    for name, M, N, lg in (("ViT-B/16 attention _softmax bf16 [64x12x197, 197]", 64 * 12 * 197, 197, 0),
+                           ("ViT-L/14@336 attention _softmax bf16 [16x16x577, 577]", 16 * 16 * 577, 577, 0),
+                           ("CLIP text attention _softmax bf16 [1024x8x77, 77]", 1024 * 8 * 77, 77, 0),
+                           ("_log_softmax bf16 [4096, 151936] (Qwen vocabulary)", 4096, 151936, 1)):
+        if only is not None and not any(t in name + " fwd" or t in name + " bwd" for t in only.split("|")):
+            continue
+        sets = []
+        for _ in range(2 if M * N > (1 << 28) else 3):
+            x = torch.randn(M, N, device=dev, dtype=bf16)
+            sets.append((x, torch.empty_like(x), torch.randn(M, N, device=dev, dtype=bf16),
+                         torch.empty_like(x)))
+        for s_ in sets:
+            L.mi355x_softmax_fwd(P(s_[0]), P(s_[1]), M, N, BF, BF, lg, stream)
+        x0, y0, g0 = sets[0][0], sets[0][1], sets[0][2]
+        aten = torch.ops.aten
+        add(name + " fwd", 2 * M * N * 2,
+            [(lambda s_=s_: L.mi355x_softmax_fwd(P(s_[0]), P(s_[1]), M, N, BF, BF, lg, stream))
+             for s_ in sets],
+            (lambda: aten._log_softmax(x0, -1, False)) if lg else (lambda: aten._softmax(x0, -1, False)))
+        add(name + " bwd", 3 * M * N * 2,
+            [(lambda s_=s_: L.mi355x_softmax_bwd(P(s_[2]), P(s_[1]), P(s_[3]), M, N, BF, BF, lg, stream))
+             for s_ in sets],
+            (lambda: aten._log_softmax_backward_data(g0, y0, -1, bf16)) if lg
+            else (lambda: aten._softmax_backward_data(g0, y0, -1, bf16)))
+        del sets, x0, y0, g0
+        torch.cuda.empty_cache()
+
+    for name, Nb, C, HW, G in (("native_group_norm bf16 [256,1024,14,14] g32", 256, 1024, 196, 32),
+                               ("native_group_norm bf16 [256,2048,7,7] g32", 256, 2048, 49, 32)):
+        if only is not None and not any(t in name + " fwd" or t in name + " bwd" for t in only.split("|")):
+            continue
+        w = (1 + 0.1 * torch.randn(C, device=dev)).to(bf16)
+        b = (0.1 * torch.randn(C, device=dev)).to(bf16)
+        dg, db = torch.empty_like(w), torch.empty_like(w)
+        sets = []
+        for _ in range(3):
+            x = torch.randn(Nb, C, HW, device=dev, dtype=bf16)
+            sets.append((x, torch.randn_like(x), torch.empty_like(x),
+                         torch.empty(Nb * G, device=dev, dtype=bf16),
+                         torch.empty(Nb * G, device=dev, dtype=bf16)))
+        nws = L.mi355x_group_norm_bwd_workspace_bytes(Nb, C, HW, G, BF, BF, 1, 1)
+        ws = torch.empty(max(nws, 1), dtype=torch.uint8, device=dev)
+        fwd = lambda s_: L.mi355x_group_norm_fwd(P(s_[0]), P(w), P(b), P(s_[2]), P(s_[3]), P(s_[4]),
+                                                 Nb, C, HW, G, 1e-5, BF, BF, stream)
+        for s_ in sets:
+            fwd(s_)
+        x0, dy0, m0, r0 = sets[0][0], sets[0][1], sets[0][3], sets[0][4]
+        nb = Nb * C * HW * 2
+        add(name + " fwd", 2 * nb, [(lambda s_=s_: fwd(s_)) for s_ in sets],
+            lambda: torch.ops.aten.native_group_norm(x0, w, b, Nb, C, HW, G, 1e-5))
+        add(name + " bwd", 3 * nb,
+            [(lambda s_=s_: L.mi355x_group_norm_bwd(P(s_[1]), P(s_[0]), P(s_[3]), P(s_[4]), P(w),
+                                                    P(s_[2]), P(dg), P(db), P(ws), nws, Nb, C, HW, G,
+                                                    BF, BF, stream)) for s_ in sets],
+            lambda: torch.ops.aten.native_group_norm_backward(dy0, x0, m0, r0, w, Nb, C, HW, G,
+                                                              [True, True, True]))
+        del sets, ws, x0, dy0, m0, r0
+        torch.cuda.empty_cache()
+    return rows
 
 
 def reference_microbench_table(torch, cabi, L, dev, stream, P, only=None):
