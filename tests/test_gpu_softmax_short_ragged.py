@@ -1,11 +1,11 @@
-"""Short ragged softmax rows (N % pack != 0, N <= 1024 16-bit / 512 float32: attention scores of
+"""Short ragged softmax rows (N % pack != 0, N <= 2048 16-bit / 1024 float32: attention scores of
 ViT / CLIP / Whisper are rows of 197, 577, 77, 1500 elements) through the LDS-staged kernels
 (softmax_fwd_flat_kernel / softmax_bwd_flat_kernel): a workgroup copies a run of whole rows to
 LDS with aligned 128-bit accesses and its lane groups work on the rows there.  The reference
 takes its general (unvectorized) forward for such rows (SoftMaxKernels.cpp:546-684 behind the
 dispatch at :1621-1718).  Checked against the CPU oracle at the family's tolerances (float32
 rtol = atol = 1e-5; 16-bit atol 1e-2, rtol 1.6e-2) and against the general kernels forced on the
-same inputs: every lanes-per-row class, row counts that end inside a workgroup's run of rows and
+same inputs: every lanes-per-row and packs-per-lane class, row counts that end inside a workgroup's run of rows and
 inside a pack, -inf / NaN rows, safe softmax, and tensors off 16-byte alignment (which keep the
 general kernels)."""
 import pytest
@@ -18,7 +18,9 @@ pytestmark = pytest.mark.gpu
 DTYPES = [torch.float32, torch.float16, torch.bfloat16]
 # (rows, N): N picks the lanes per row (8 / 16 / 32 / 64), rows end inside a run and inside a pack
 SHAPES = [(1, 3), (7, 5), (1001, 33), (333, 77), (64, 129), (515, 197), (9, 255), (40, 257),
-          (123, 511), (17, 513), (61, 577), (10, 1001), (24, 1023)]
+          (123, 511), (17, 513), (61, 577), (10, 1001), (24, 1023),
+          # 3 and 4 packs a lane, 4 lanes a row, and rows beyond 1024 elements (32 KB of LDS)
+          (50, 21), (300, 45), (77, 93), (19, 750), (33, 1500), (9, 2047), (5, 1025)]
 
 
 def _general(cabi, op, M, N, dtype, fn):

@@ -569,15 +569,15 @@ softmax_bwd_resident_kernel(const TG* __restrict__ grad, const TG* __restrict__ 
 }
 
 // ---------------------------------------------------------------------------
-// Short ragged rows (N % E != 0, N <= 64 * flat_max_k: ViT / CLIP / Whisper
-// attention scores are rows of 197, 577, 77, 1500 elements) through LDS.  Such
+// Short ragged rows (N % E != 0, N <= 64 lanes * kFlatMaxPacks packs: ViT / CLIP /
+// Whisper attention scores are rows of 197, 577, 77, 1500 elements) through LDS.  Such
 // rows start at every 2-byte (fp32: 4-byte) alignment, and the general kernels
 // pay for it per row: edge packs moved element by element, windows, masks.  But
 // BLOCK / G consecutive rows are one contiguous piece of the tensor that starts
 // and ends on a 16-byte boundary (BLOCK / G is a multiple of 8), so the workgroup
 // copies the piece to LDS with whole aligned 128-bit accesses, each group of G
 // lanes then reads its row from LDS in packs at the row's own alignment (LDS takes
-// unaligned 128-bit accesses; two packs a lane, laid out like the register-
+// unaligned 128-bit accesses; VP packs a lane, laid out like the register-
 // resident kernels'), writes the results back in place, and the piece leaves
 // with whole 128-bit stores.  HBM sees the access
 // pattern of a copy whatever N is.  The reductions stay inside a wavefront
@@ -596,10 +596,10 @@ constexpr int kFlatBlock = ROWNORM_FLAT_BLOCK;
 // -> 25.6 us, backward 36.2 -> 32.9 us ([147712, 577] backward, which needs the
 // 16 KB: 101 -> 94 us); 1024 threads were 50 % slower.
 constexpr int kFlatLdsBytes = 64 * kFlatBlock;
-template <class T>
-constexpr int flat_max_k() {
-  return sizeof(T) == 2 ? 16 : 8;
-}
+// Lanes per row G (4..64) and packs per lane VP (1..kFlatMaxPacks) are chosen so
+// that G * VP leaves as few pack slots idle as possible (flat_layout,
+// softmax_launch.hpp).
+constexpr int kFlatMaxPacks = 4;
 // Rows a workgroup takes at a time: as many as its LDS holds, a multiple of 8
 // so that the piece starts and ends on a 16-byte boundary (and of the rows its
 // lane groups work on at a time, where that many fit).  A
@@ -705,13 +705,12 @@ __device__ __forceinline__ void flat_row_store(T* rowb, int j, int nv, const Pac
   }
 }
 
-template <class T, int G, int BLOCK, int LDSB>
+template <class T, int G, int VP, int BLOCK, int LDSB>
 __global__ void __launch_bounds__(BLOCK)
 softmax_fwd_flat_kernel(const T* __restrict__ x, T* __restrict__ y, int64_t M, int N,
                         int chunk_rows, int flags) {
   constexpr int E = elems_per_pack<T>::value;
   constexpr int RPB = BLOCK / G;
-  constexpr int VP = flat_max_k<T>() / E;  // packs a lane
   constexpr bool PRECISE = sizeof(T) == 4;
   constexpr int U = LDSB / (BLOCK * 16);
   __shared__ __attribute__((aligned(16))) T buf[LDSB / sizeof(T) + E];
@@ -781,13 +780,12 @@ softmax_fwd_flat_kernel(const T* __restrict__ x, T* __restrict__ y, int64_t M, i
 #endif
 }
 
-template <class T, int G, int BLOCK, int LDSB>
+template <class T, int G, int VP, int BLOCK, int LDSB>
 __global__ void __launch_bounds__(BLOCK)
 softmax_bwd_flat_kernel(const T* __restrict__ grad, const T* __restrict__ y, T* __restrict__ gi,
                         int64_t M, int N, int chunk_rows, int flags) {
   constexpr int E = elems_per_pack<T>::value;
   constexpr int RPB = BLOCK / G;
-  constexpr int VP = flat_max_k<T>() / E;
   constexpr bool PRECISE = sizeof(T) == 4;
   constexpr int U = LDSB / (BLOCK * 16);
   __shared__ __attribute__((aligned(16))) T bg[LDSB / sizeof(T) + E];

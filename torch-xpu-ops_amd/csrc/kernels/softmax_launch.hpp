@@ -33,76 +33,118 @@ struct SoftmaxFwdLauncher {
   };
 };
 
-// Short ragged rows through LDS (softmax_fwd_flat_kernel): lanes per row, or 0
-// when the call does not qualify.
+// Short ragged rows through LDS (softmax_fwd_flat_kernel / softmax_bwd_flat_kernel).
+struct FlatLayout {
+  int g = 0;   // lanes per row (0: the call does not qualify)
+  int vp = 0;  // packs per lane
+};
+
+// The (lanes 4..64, packs per lane 1..4) with the fewest idle pack slots; among
+// equals the one nearest two packs a lane, the layout the resident kernels prefer.
+// Measured against "two packs a lane on the fewest lanes that hold the row",
+// interleaved, bf16 forward / backward in us: rows of 13: 19.5 / 18.5 -> 10.6 / 8.6,
+// 21: 30.0 / 25.9 -> 14.1 / 16.1, 45: 20.3 / 22.8 -> 16.5 / 20.6, 577 (73 packs: 32 x 3
+// instead of 64 x 2): 72.1 / 96.5 -> 67.8 / 96.3, 750: 54.0 / 76.2 -> 51.2 / 75.1; 93
+// and 129 lose 5-10 % in the backward (13.1 -> 14.6, 33.1 -> 34.8).
 template <class T>
-inline int flat_lanes(const Plan& plan, int64_t M, int N, const void* p0, const void* p1,
-                      const void* p2) {
-  if (plan.fast || plan.forced || M < 1 || N > 64 * flat_max_k<T>()) return 0;
-  if ((((uintptr_t)p0) | ((uintptr_t)p1) | ((uintptr_t)p2)) & 15) return 0;
-  int g = 8;
-  while (g * flat_max_k<T>() < N) g <<= 1;
-  return g;
+inline FlatLayout flat_layout(const Plan& plan, int64_t M, int N, const void* p0, const void* p1,
+                              const void* p2) {
+  constexpr int E = elems_per_pack<T>::value;
+  FlatLayout f;
+  if (plan.fast || plan.forced || M < 1 || N > 64 * kFlatMaxPacks * E) return f;
+  if ((((uintptr_t)p0) | ((uintptr_t)p1) | ((uintptr_t)p2)) & 15) return f;
+  const int packs = (N + E - 1) / E;
+  int best_slots = 0, best_rank = 0;
+  for (int g = 4; g <= 64; g <<= 1) {
+    const int vp = (packs + g - 1) / g;
+    if (vp > kFlatMaxPacks) continue;
+    const int slots = g * vp;
+    const int rank = vp == 2 ? 0 : (vp == 3 ? 1 : (vp == 1 ? 2 : 3));
+    if (f.g == 0 || slots < best_slots || (slots == best_slots && rank < best_rank)) {
+      f.g = g;
+      f.vp = vp;
+      best_slots = slots;
+      best_rank = rank;
+    }
+  }
+  return f;
 }
 
-template <class T>
-bool launch_softmax_fwd_flat(int g, const SoftmaxFwdArgs& a, hipStream_t stream) {
-  const int cr = flat_chunk_rows<T>(a.N, g, kFlatLdsBytes);
-  if (cr < 8) return false;
+// One case per (lanes, packs per lane) of a launch switch keyed by lanes * 8 + packs.
+#define ROWNORM_FLAT_CASES(CASE, GL) CASE(GL, 1) CASE(GL, 2) CASE(GL, 3) CASE(GL, 4)
+#define ROWNORM_FLAT_ALL(CASE)                                                       \
+  ROWNORM_FLAT_CASES(CASE, 4) ROWNORM_FLAT_CASES(CASE, 8) ROWNORM_FLAT_CASES(CASE, 16) \
+  ROWNORM_FLAT_CASES(CASE, 32) ROWNORM_FLAT_CASES(CASE, 64)
+
+template <class T, int LDSB>
+bool launch_softmax_fwd_flat_l(FlatLayout f, int cr, const SoftmaxFwdArgs& a, hipStream_t stream) {
   const int64_t grid = (a.M + cr - 1) / cr;
   if (grid > 0x7fffffff) return false;
-#define ROWNORM_FLAT_FWD(GL)                                                                \
-  case GL:                                                                                  \
-    hipLaunchKernelGGL((softmax_fwd_flat_kernel<T, GL, kFlatBlock, kFlatLdsBytes>),          \
-                       dim3((unsigned)grid), dim3(kFlatBlock), 0, stream, (const T*)a.x,     \
-                       (T*)a.y, a.M, a.N, cr, a.flags);                                     \
-    return true;
-  switch (g) {
-    ROWNORM_FLAT_FWD(8)
-    ROWNORM_FLAT_FWD(16)
-    ROWNORM_FLAT_FWD(32)
-    ROWNORM_FLAT_FWD(64)
-  }
+#define ROWNORM_FLAT_FWD(GL, VP)                                                                \
+  case GL * 8 + VP:                                                                             \
+    if constexpr (LDSB <= kFlatLdsBytes || (GL == 64 && VP >= 3)) {                             \
+      hipLaunchKernelGGL((softmax_fwd_flat_kernel<T, GL, VP, kFlatBlock, LDSB>),                 \
+                         dim3((unsigned)grid), dim3(kFlatBlock), 0, stream, (const T*)a.x,       \
+                         (T*)a.y, a.M, a.N, cr, a.flags);                                       \
+      return true;                                                                              \
+    }                                                                                           \
+    return false;
+  switch (f.g * 8 + f.vp) { ROWNORM_FLAT_ALL(ROWNORM_FLAT_FWD) }
 #undef ROWNORM_FLAT_FWD
   return false;
 }
 
+template <class T>
+bool launch_softmax_fwd_flat(FlatLayout f, const SoftmaxFwdArgs& a, hipStream_t stream) {
+  // 16 KB of LDS a workgroup; rows beyond 1024 16-bit elements (64 lanes, 3 or 4 packs) need 32 KB
+  int cr = flat_chunk_rows<T>(a.N, f.g, kFlatLdsBytes);
+  if (cr >= 8) return launch_softmax_fwd_flat_l<T, kFlatLdsBytes>(f, cr, a, stream);
+  cr = flat_chunk_rows<T>(a.N, f.g, 2 * kFlatLdsBytes);
+  if (cr >= 8) return launch_softmax_fwd_flat_l<T, 2 * kFlatLdsBytes>(f, cr, a, stream);
+  return false;
+}
+
 template <class T, int LDSB>
-bool launch_softmax_bwd_flat_l(int g, int cr, const SoftmaxBwdArgs& a, hipStream_t stream) {
+bool launch_softmax_bwd_flat_l(FlatLayout f, int cr, const SoftmaxBwdArgs& a, hipStream_t stream) {
   const int64_t grid = (a.M + cr - 1) / cr;
   if (grid > 0x7fffffff) return false;
-#define ROWNORM_FLAT_BWD(GL)                                                                 \
-  case GL:                                                                                   \
-    hipLaunchKernelGGL((softmax_bwd_flat_kernel<T, GL, kFlatBlock, LDSB>), dim3((unsigned)grid), \
-                       dim3(kFlatBlock), 0, stream, (const T*)a.grad, (const T*)a.y, (T*)a.gi, \
-                       a.M, a.N, cr, a.flags);                                               \
-    return true;
-  switch (g) {
-    ROWNORM_FLAT_BWD(8)
-    ROWNORM_FLAT_BWD(16)
-    ROWNORM_FLAT_BWD(32)
-    ROWNORM_FLAT_BWD(64)
-  }
+#define ROWNORM_FLAT_BWD(GL, VP)                                                                \
+  case GL * 8 + VP:                                                                             \
+    if constexpr ((LDSB == kFlatLdsBytes) || (LDSB < kFlatLdsBytes && GL <= 16) ||              \
+                  (LDSB > kFlatLdsBytes && GL == 64 && VP >= 3)) {                              \
+      hipLaunchKernelGGL((softmax_bwd_flat_kernel<T, GL, VP, kFlatBlock, LDSB>),                 \
+                         dim3((unsigned)grid), dim3(kFlatBlock), 0, stream, (const T*)a.grad,    \
+                         (const T*)a.y, (T*)a.gi, a.M, a.N, cr, a.flags);                       \
+      return true;                                                                              \
+    }                                                                                           \
+    return false;
+  switch (f.g * 8 + f.vp) { ROWNORM_FLAT_ALL(ROWNORM_FLAT_BWD) }
 #undef ROWNORM_FLAT_BWD
   return false;
 }
 
 template <class T>
-bool launch_softmax_bwd_flat(int g, const SoftmaxBwdArgs& a, hipStream_t stream) {
-  // half the LDS per tensor where that still holds a full pass of the lane groups' rows
-  const int rpb = kFlatBlock / g < 8 ? 8 : kFlatBlock / g;
-  const int half = flat_chunk_rows<T>(a.N, g, kFlatLdsBytes / 2);
-  if (half >= rpb) return launch_softmax_bwd_flat_l<T, kFlatLdsBytes / 2>(g, half, a, stream);
-  const int cr = flat_chunk_rows<T>(a.N, g, kFlatLdsBytes);
-  if (cr < 8) return false;
-  return launch_softmax_bwd_flat_l<T, kFlatLdsBytes>(g, cr, a, stream);
+bool launch_softmax_bwd_flat(FlatLayout f, const SoftmaxBwdArgs& a, hipStream_t stream) {
+  // per tensor: 8 KB where that still holds a full pass of the lane groups' rows (short
+  // rows: more workgroups a compute unit), else 16 KB, else 32 KB (rows beyond 1024
+  // 16-bit elements)
+  const int rpb = kFlatBlock / f.g < 8 ? 8 : kFlatBlock / f.g;
+  if (f.g <= 16) {
+    const int half = flat_chunk_rows<T>(a.N, f.g, kFlatLdsBytes / 2);
+    if (half >= rpb) return launch_softmax_bwd_flat_l<T, kFlatLdsBytes / 2>(f, half, a, stream);
+  }
+  int cr = flat_chunk_rows<T>(a.N, f.g, kFlatLdsBytes);
+  if (cr >= 8) return launch_softmax_bwd_flat_l<T, kFlatLdsBytes>(f, cr, a, stream);
+  cr = flat_chunk_rows<T>(a.N, f.g, 2 * kFlatLdsBytes);
+  if (cr >= 8) return launch_softmax_bwd_flat_l<T, 2 * kFlatLdsBytes>(f, cr, a, stream);
+  return false;
 }
 
 template <class TI, class TO, bool MASKED>
 int launch_softmax_fwd_m(const Plan& plan, const SoftmaxFwdArgs& a, hipStream_t stream) {
   if constexpr (!MASKED && std::is_same<TI, TO>::value) {
-    const int g = flat_lanes<TI>(plan, a.M, a.N, a.x, a.y, nullptr);
-    if (g && launch_softmax_fwd_flat<TI>(g, a, stream)) return (int)hipGetLastError();
+    const FlatLayout f = flat_layout<TI>(plan, a.M, a.N, a.x, a.y, nullptr);
+    if (f.g && launch_softmax_fwd_flat<TI>(f, a, stream)) return (int)hipGetLastError();
   }
   if (plan.resident) {
     SoftmaxFwdCtx<TI, TO> ctx{plan, a, stream};
@@ -189,8 +231,8 @@ inline bool launch_log_softmax_bwd_grad_resident(const Plan& plan, const Softmax
 template <class TG, class TO, bool MASKED>
 int launch_softmax_bwd_m(const Plan& plan, const SoftmaxBwdArgs& a, hipStream_t stream) {
   if constexpr (!MASKED && std::is_same<TG, TO>::value) {
-    const int g = flat_lanes<TG>(plan, a.M, a.N, a.grad, a.y, a.gi);
-    if (g && launch_softmax_bwd_flat<TG>(g, a, stream)) return (int)hipGetLastError();
+    const FlatLayout f = flat_layout<TG>(plan, a.M, a.N, a.grad, a.y, a.gi);
+    if (f.g && launch_softmax_bwd_flat<TG>(f, a, stream)) return (int)hipGetLastError();
   }
   if (plan.resident) {
     SoftmaxBwdCtx<TG, TO> ctx{plan, a, stream};
