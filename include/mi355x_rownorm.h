@@ -337,7 +337,8 @@ int mi355x_softmax_strided_plan(int backward, int64_t outer, int64_t dim_size, i
  * tensors that start on a 128-byte line; rows of at most 64 packs in tensors
  * that do not take one pack a lane (lanes_per_row = packs rounded up to a
  * power of two).  Unmasked softmax calls on ragged rows (N not a whole number
- * of packs) of at most 1024 16-bit / 512 float32 elements, with 16-byte aligned
+ * of packs) of at most 2048 16-bit / 1024 float32 elements, and on rows of up to
+ * 12 whole packs that fit the reported layout badly, with 16-byte aligned
  * tensors and one dtype, run through LDS-staged kernels instead of the layout
  * reported here (a forced layout keeps the reported kernels). */
 int mi355x_rownorm_plan(rownorm_op op, int64_t M, int64_t N, rownorm_dtype x_dtype,

@@ -20,7 +20,9 @@ DTYPES = [torch.float32, torch.float16, torch.bfloat16]
 SHAPES = [(1, 3), (7, 5), (1001, 33), (333, 77), (64, 129), (515, 197), (9, 255), (40, 257),
           (123, 511), (17, 513), (61, 577), (10, 1001), (24, 1023),
           # 3 and 4 packs a lane, 4 lanes a row, and rows beyond 1024 elements (32 KB of LDS)
-          (50, 21), (300, 45), (77, 93), (19, 750), (33, 1500), (9, 2047), (5, 1025)]
+          (50, 21), (300, 45), (77, 93), (19, 750), (33, 1500), (9, 2047), (5, 1025),
+          # very short rows of whole packs whose pack count fits the resident layouts badly
+          (1000, 24), (333, 72), (129, 80), (77, 88)]
 
 
 def _general(cabi, op, M, N, dtype, fn):

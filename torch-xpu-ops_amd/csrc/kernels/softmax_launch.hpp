@@ -34,6 +34,7 @@ struct SoftmaxFwdLauncher {
 };
 
 // Short ragged rows through LDS (softmax_fwd_flat_kernel / softmax_bwd_flat_kernel).
+constexpr int kFlatWholePackRowsMaxPacks = 12;
 struct FlatLayout {
   int g = 0;   // lanes per row (0: the call does not qualify)
   int vp = 0;  // packs per lane
@@ -51,9 +52,11 @@ inline FlatLayout flat_layout(const Plan& plan, int64_t M, int N, const void* p0
                               const void* p2) {
   constexpr int E = elems_per_pack<T>::value;
   FlatLayout f;
-  if (plan.fast || plan.forced || M < 1 || N > 64 * kFlatMaxPacks * E) return f;
+  if (plan.forced || M < 1 || N > 64 * kFlatMaxPacks * E) return f;
   if ((((uintptr_t)p0) | ((uintptr_t)p1) | ((uintptr_t)p2)) & 15) return f;
   const int packs = (N + E - 1) / E;
+  // rows of whole packs qualify only when they are very short (see below)
+  if (plan.fast && (packs > kFlatWholePackRowsMaxPacks || !plan.resident)) return f;
   int best_slots = 0, best_rank = 0;
   for (int g = 4; g <= 64; g <<= 1) {
     const int vp = (packs + g - 1) / g;
@@ -67,6 +70,12 @@ inline FlatLayout flat_layout(const Plan& plan, int64_t M, int N, const void* p0
       best_rank = rank;
     }
   }
+  // Rows of whole packs: only up to 12 packs and where the resident layout leaves a
+  // quarter of its pack slots idle, e.g. 9 or 10 packs on 8 lanes x 2 (bf16 rows of 72:
+  // 36.6 / 52.5 -> 31.2 / 44.3 us, of 80: 40.9 / 57.6 -> 33.2 / 48.2 us, of 24: 32.1 / 29.4
+  // -> 18.1 / 25.1 us); from 17 packs on it measured the same or slower (520: +2 %, 1032:
+  // the backward +30 %).
+  if (plan.fast && best_slots * 4 > plan.G * plan.V * 3) f = FlatLayout{};
   return f;
 }
 
