@@ -573,18 +573,19 @@ softmax_bwd_resident_kernel(const TG* __restrict__ grad, const TG* __restrict__ 
 // Whisper attention scores are rows of 197, 577, 77, 1500 elements) through LDS.  Such
 // rows start at every 2-byte (fp32: 4-byte) alignment, and the general kernels
 // pay for it per row: edge packs moved element by element, windows, masks.  But
-// BLOCK / G consecutive rows are one contiguous piece of the tensor that starts
-// and ends on a 16-byte boundary (BLOCK / G is a multiple of 8), so the workgroup
-// copies the piece to LDS with whole aligned 128-bit accesses, each group of G
-// lanes then reads its row from LDS in packs at the row's own alignment (LDS takes
-// unaligned 128-bit accesses; VP packs a lane, laid out like the register-
-// resident kernels'), writes the results back in place, and the piece leaves
-// with whole 128-bit stores.  HBM sees the access
-// pattern of a copy whatever N is.  The reductions stay inside a wavefront
-// (G <= 64), so the only barriers are the two around the LDS phase; a lane
-// group walks the rows r, r + BLOCK / G, ... of the workgroup's piece.  Needs
-// 16-byte aligned tensor bases and the same dtype in and out; anything else
-// keeps the general kernels.
+// a run of `chunk_rows` consecutive rows, chunk_rows a multiple of 8, is one
+// contiguous piece of the tensor that starts and ends on a 16-byte boundary, so
+// the workgroup copies the piece to LDS with whole aligned 128-bit accesses, each
+// group of G lanes then reads a row from LDS in packs at the row's own alignment
+// (LDS takes unaligned 128-bit accesses; VP packs a lane, laid out like the
+// register-resident kernels'), writes the results back in place, and the piece
+// leaves with whole 128-bit stores: HBM sees the access pattern of a copy
+// whatever N is.  The reductions stay inside a wavefront (G <= 64), so the only
+// barriers are the two around the LDS phase; a lane group walks the rows r,
+// r + BLOCK / G, ... of the piece.  Needs 16-byte aligned tensor bases and the
+// same dtype in and out; anything else keeps the general kernels.  Very short
+// rows of whole packs whose pack count fits the resident layouts badly take the
+// same path (flat_layout, softmax_launch.hpp).
 #ifndef ROWNORM_FLAT_BLOCK
 #define ROWNORM_FLAT_BLOCK 256
 #endif
@@ -592,9 +593,10 @@ constexpr int kFlatBlock = ROWNORM_FLAT_BLOCK;
 // LDS per tensor a workgroup holds (LDSB; the backward holds two tensors): 16 KB
 // at 256 threads, so that 8 workgroups share a compute unit; the backward takes
 // 8 KB per tensor where that still holds a full pass of rows, for the same
-// reason.  Measured against 512 threads / 32 KB: bf16 [151296, 197] forward 27.0
-// -> 25.6 us, backward 36.2 -> 32.9 us ([147712, 577] backward, which needs the
-// 16 KB: 101 -> 94 us); 1024 threads were 50 % slower.
+// reason; rows beyond 1024 16-bit elements need 32 KB to hold 8 of them.
+// Measured against 512 threads / 32 KB: bf16 [151296, 197] forward 27.0 -> 25.6 us,
+// backward 36.2 -> 32.9 us ([147712, 577] backward, which needs the 16 KB:
+// 101 -> 94 us); 1024 threads were 50 % slower.
 constexpr int kFlatLdsBytes = 64 * kFlatBlock;
 // Lanes per row G (4..64) and packs per lane VP (1..kFlatMaxPacks) are chosen so
 // that G * VP leaves as few pack slots idle as possible (flat_layout,
