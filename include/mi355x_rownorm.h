@@ -294,7 +294,7 @@ int mi355x_group_norm_bwd(const void* dy, const void* x, const void* mean, const
  * slab of (C / groups) * HxW elements; `reserved` is 1 when HxW is a whole
  * number of 16-byte packs (per-pack weight lookup, channel sums fused into the
  * backward), 2 when only the rows are (a pack may straddle two channels: two
- * lookups per pack, sums still fused; needs HxW >= one pack and at most 64
+ * lookups per pack, sums still fused; needs HxW >= one pack and at most 512
  * channels a group), 0 for the general kernels; partial_rows is N for the
  * backward. */
 int mi355x_group_norm_plan(int backward, int64_t N, int64_t C, int64_t HxW, int64_t groups,

@@ -366,15 +366,15 @@ def test_group_norm_validation_and_plans(cabi):
         for (N, C, HxW, G) in ((2, 4, 1, 2), (256, 32, 16, 4), (4, 64, 1024, 32), (2, 320, 4096, 32),
                                (3, 6, 5, 3), (1, 4, 1 << 17, 2), (1, 8, 1 << 20, 2),
                                # 7x7 and 14x14 maps: rows of whole packs, channels not
-                               (4, 64, 49, 8), (2, 1024, 196, 32), (2, 128, 49, 2), (2, 130, 49, 2),
+                               (4, 64, 49, 8), (2, 1024, 196, 32), (2, 128, 49, 2), (2, 130, 49, 2), (1, 1040, 49, 2),
                                (3, 8, 9, 1), (2, 16, 6, 2)):
             for bwd in (0, 1):
                 p = cabi.group_norm_plan(bwd, N, C, HxW, G, dt)
                 Lrow = (C // G) * HxW
                 # 1: every pack in one channel; 2: rows of whole packs whose packs may straddle
-                # two channels (needs a pack per channel at least and at most 64 channels a
+                # two channels (needs a pack per channel at least and at most 512 channels a
                 # group); 0: the general kernels
-                kind = 1 if HxW % E == 0 else (2 if Lrow % E == 0 and HxW >= E and C // G <= 64 else 0)
+                kind = 1 if HxW % E == 0 else (2 if Lrow % E == 0 and HxW >= E and C // G <= 512 else 0)
                 assert p["uniform"] == kind, (N, C, HxW, G, dt, p)
                 assert p["grid_blocks"] >= 1
                 if p["resident"]:

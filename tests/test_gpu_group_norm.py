@@ -33,10 +33,11 @@ SHAPES = [(2, 4, (), 2), (64, 32, (), 4), (256, 32, (), 4), (64, 32, (16,), 4), 
           (4, 12, (8,), 3), (4, 12, (4,), 3), (3, 10, (24,), 5), (2, 6, (5, 8), 2), (2, 9, (1000,), 3),
           (1, 6, (8200,), 2),
           # rows of whole packs whose channels are not (packs straddle two channels): 7x7, 14x14
-          # and 27x27 maps, a channel barely longer than a pack, 64 channels a group (the most
-          # the straddling kernels take) and 65 (general kernels)
+          # and 27x27 maps, a channel barely longer than a pack, 64, 65 and 512 channels a group (the most the
+          # straddling kernels take) and 520 (general kernels)
           (4, 64, (7, 7), 8), (2, 64, (14, 14), 2), (2, 128, (7, 7), 2), (2, 130, (7, 7), 2),
-          (1, 16, (27, 27), 1), (3, 8, (9,), 1), (2, 24, (3, 4), 3), (70, 32, (7, 7), 4)]
+          (1, 16, (27, 27), 1), (3, 8, (9,), 1), (2, 24, (3, 4), 3), (70, 32, (7, 7), 4),
+          (2, 512, (7, 7), 1), (1, 1040, (7, 7), 2)]
 CASES = load_golden("aten_cpu_group_norm.npz")
 
 

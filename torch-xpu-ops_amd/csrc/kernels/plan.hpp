@@ -160,7 +160,7 @@ constexpr bool is_group_class(OpClass oc) { return oc == OC_GROUP_FWD || oc == O
 constexpr int kGnGeneral = 0, kGnUniform = 1, kGnStraddle = 2;
 // Channels per group up to which the straddling kernels are taken (their LDS
 // array for the parts of packs that belong to the next channel).
-constexpr int kGnStraddleMaxD = 64;
+constexpr int kGnStraddleMaxD = 512;
 constexpr int gn_mode(int64_t L, int64_t HxW, int64_t D, int E) {
   if (HxW % E == 0) return kGnUniform;
   if (L % E == 0 && HxW >= E && D <= kGnStraddleMaxD) return kGnStraddle;
