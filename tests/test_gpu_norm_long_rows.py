@@ -1,0 +1,149 @@
+"""LayerNorm / RMSNorm forward rows of 5 to 16 packs a lane on 1024 lanes (16-bit rows of 32776 to
+131072 elements, float32 rows of 16388 to 65536): the register-resident kernel
+(norm_fwd_resident_kernel) with gamma / beta held in registers where they fit and loaded per pack
+of the output where they do not.  The reference serves such rows with its one-work-group-per-row
+forward (RowwiseMomentsFunctor + LayerNormForwardKernelFunctor,
+src/ATen/native/xpu/sycl/LayerNormKernels.cpp:197-260, 590-660 behind the dispatch at :1121-1163).
+Checked through the extern "C" ABI against the CPU oracle at the family's tolerances (float32
+rtol = atol = 1e-5; 16-bit atol 1e-2, rtol 1.6e-2), against the multi-pass kernel forced on the
+same inputs, with and without weights, with float32 weights beside 16-bit rows, with the residual
+add and the output cast fused in, and for run-to-run determinism."""
+import pytest
+import torch
+
+from helpers import assert_close, gen, to_np32
+
+pytestmark = pytest.mark.gpu
+
+DTYPES = [torch.float32, torch.float16, torch.bfloat16]
+NAME = {torch.float32: "f32", torch.float16: "f16", torch.bfloat16: "bf16"}
+# packs a lane -> row length in packs of 1024 lanes (the last two leave lanes without a pack, or
+# with packs outside the row)
+PACKS = [(5, 5 * 1024), (6, 6 * 1024), (6, 5 * 1024 + 1), (8, 7 * 1024), (8, 8 * 1024),
+         (10, 9 * 1024 + 512), (12, 12 * 1024), (16, 12 * 1024 + 4), (16, 16 * 1024)]
+
+
+def _mk(M, N, dtype, wdtype, seed, shift=0.5):
+    g = gen(seed)
+    x = (shift + torch.randn(M, N, generator=g)).to(dtype)
+    gamma = (1 + 0.1 * torch.randn(N, generator=g)).to(wdtype)
+    beta = (0.1 * torch.randn(N, generator=g)).to(wdtype)
+    return x, gamma, beta
+
+
+def _multi_pass(cabi, op, fn):
+    try:
+        cabi.set_override(op, -1, 1)
+        return fn()
+    finally:
+        cabi.clear_overrides()
+
+
+@pytest.mark.parametrize("dtype", DTYPES, ids=str)
+@pytest.mark.parametrize("mixed", [False, True], ids=["w_same", "w_fp32"])
+def test_forward_against_oracle_and_multi_pass_kernel(cabi, oracle, gpu, dtype, mixed):
+    if mixed and dtype == torch.float32:
+        pytest.skip("mixed precision means float32 weights beside 16-bit rows")
+    E = 4 if dtype == torch.float32 else 8
+    wdtype = torch.float32 if mixed else dtype
+    code, wcode = cabi.dtype_code(dtype), cabi.dtype_code(wdtype)
+    for i, (V, packs) in enumerate(PACKS):
+        # (from 10 packs a lane, fewer rows than half the compute units are split over workgroups)
+        M, N = (5 if V < 10 else 128) + i, packs * E
+        print("case long rows", dtype, mixed, (M, N), flush=True)
+        for op in (cabi.OP_LAYER_NORM_FWD, cabi.OP_RMS_NORM_FWD):
+            p = cabi.plan(op, M, N, code, wcode)
+            assert (p["resident"], p["lanes_per_row"], p["packs_per_lane"]) == (1, 1024, V), p
+        x, gamma, beta = _mk(M, N, dtype, wdtype, 1400 + i)
+        xg, gg, bg = x.to(gpu), gamma.to(gpu), beta.to(gpu)
+        what = "[%d, %d] %s" % (M, N, dtype)
+        y, mean, rstd = cabi.layer_norm_fwd(xg, gg, bg, 1e-5)
+        oy, om, orr = oracle.layer_norm_fwd(to_np32(x), (N,), to_np32(gamma), to_np32(beta), 1e-5)
+        assert_close(y, oy, dtype, "layer_norm y " + what)
+        assert_close(mean, om.reshape(-1), torch.float32, "mean " + what)
+        assert_close(rstd, orr.reshape(-1), torch.float32, "rstd " + what)
+        sy, sm, sr = _multi_pass(cabi, cabi.OP_LAYER_NORM_FWD,
+                                 lambda: cabi.layer_norm_fwd(xg, gg, bg, 1e-5))
+        assert_close(y, to_np32(sy), dtype, "layer_norm y against the multi-pass kernel " + what)
+        assert_close(rstd, to_np32(sr), torch.float32, "rstd against the multi-pass kernel " + what)
+        ry, rr = cabi.rms_norm_fwd(xg, gg, 1e-6)
+        roy, ror = oracle.rms_norm_fwd(to_np32(x), (N,), to_np32(gamma), 1e-6)
+        assert_close(ry, roy, dtype, "rms_norm y " + what)
+        assert_close(rr, ror.reshape(-1), torch.float32, "rms rstd " + what)
+        # a second run gives the same bits
+        y2, mean2, rstd2 = cabi.layer_norm_fwd(xg, gg, bg, 1e-5)
+        ry2, rr2 = cabi.rms_norm_fwd(xg, gg, 1e-6)
+        for a, b in ((y, y2), (mean, mean2), (rstd, rstd2), (ry, ry2), (rr, rr2)):
+            assert torch.equal(a.view(torch.uint8), b.view(torch.uint8))
+        if i % 3 == 0:
+            # no weights
+            y0, _, _ = cabi.layer_norm_fwd(xg, None, None, 1e-5)
+            oy0, _, _ = oracle.layer_norm_fwd(to_np32(x), (N,), None, None, 1e-5)
+            assert_close(y0, oy0, dtype, "layer_norm without weights " + what)
+            ry0, _ = cabi.rms_norm_fwd(xg, None, 1e-6)
+            roy0, _ = oracle.rms_norm_fwd(to_np32(x), (N,), None, 1e-6)
+            assert_close(ry0, roy0, dtype, "rms_norm without weights " + what)
+
+
+@pytest.mark.parametrize("dtype", DTYPES, ids=str)
+def test_constant_and_shifted_rows(cabi, oracle, gpu, dtype):
+    """A constant row gives beta bit for bit; rows far from zero keep their statistics."""
+    E = 4 if dtype == torch.float32 else 8
+    N = 6 * 1024 * E
+    x, gamma, beta = _mk(6, N, dtype, dtype, 1450, shift=100.0)
+    x[1] = 3.0
+    x[2, :3] = 0.0  # the head of the row is not representative of it
+    xg, gg, bg = x.to(gpu), gamma.to(gpu), beta.to(gpu)
+    y, mean, rstd = cabi.layer_norm_fwd(xg, gg, bg, 1e-5)
+    assert torch.equal(y[1].cpu(), beta)
+    oy, om, orr = oracle.layer_norm_fwd(to_np32(x), (N,), to_np32(gamma), to_np32(beta), 1e-5)
+    ok = [0, 2, 3, 4, 5]
+    assert_close(y[ok], oy[ok], dtype, "shifted rows y")
+    assert_close(mean[ok], om.reshape(-1)[ok], torch.float32, "shifted rows mean")
+    assert_close(rstd[ok], orr.reshape(-1)[ok], dtype, "shifted rows rstd")
+
+
+@pytest.mark.parametrize("dtype", DTYPES, ids=str)
+def test_fused_add_and_cast(cabi, oracle, gpu, dtype):
+    """Residual add -> norm on rows of 5 to 12 packs a lane (float32 LayerNorm: to 10), and
+    float32 rows written out in bf16; rows beyond that take the multi-pass kernel and agree."""
+    E = 4 if dtype == torch.float32 else 8
+    for i, packs in enumerate((5 * 1024, 8 * 1024, 10 * 1024, 12 * 1024, 16 * 1024)):
+        M, N = (4 if packs < 10 * 1024 else 128) + i, packs * E
+        print("case long rows fused add", dtype, (M, N), flush=True)
+        g = gen(1460 + i)
+        x = torch.randn(M, N, generator=g).to(dtype)
+        res = (2 * torch.randn(M, N, generator=g)).to(dtype)
+        gamma = (1 + 0.1 * torch.randn(N, generator=g)).to(dtype)
+        beta = (0.1 * torch.randn(N, generator=g)).to(dtype)
+        xg, rg, gg, bg = x.to(gpu), res.to(gpu), gamma.to(gpu), beta.to(gpu)
+        h_cpu = x + res
+        y, h, mean, rstd = cabi.add_layer_norm_fwd(xg, rg, gg, bg, 1e-5)
+        assert torch.equal(h.cpu(), h_cpu)
+        oy, om, orr = oracle.layer_norm_fwd(to_np32(h_cpu), (N,), to_np32(gamma), to_np32(beta), 1e-5)
+        assert_close(y, oy, dtype, "add_layer_norm y")
+        assert_close(rstd, orr.reshape(-1), torch.float32, "add_layer_norm rstd")
+        ry, rh, rr = cabi.add_rms_norm_fwd(xg, rg, gg, 1e-6)
+        assert torch.equal(rh.cpu(), h_cpu)
+        roy, ror = oracle.rms_norm_fwd(to_np32(h_cpu), (N,), to_np32(gamma), 1e-6)
+        assert_close(ry, roy, dtype, "add_rms_norm y")
+        assert_close(rr, ror.reshape(-1), torch.float32, "add_rms_norm rstd")
+        if dtype == torch.float32:
+            cy, _, _, crstd = cabi.add_layer_norm_fwd(xg, None, gg, bg, 1e-5, y_dtype=torch.bfloat16)
+            oy0, _, orr0 = oracle.layer_norm_fwd(to_np32(x), (N,), to_np32(gamma), to_np32(beta), 1e-5)
+            assert_close(cy, oy0, torch.bfloat16, "layer_norm with bf16 output")
+            assert_close(crstd, orr0.reshape(-1), torch.float32, "rstd with bf16 output")
+            ay, ah, arr = cabi.add_rms_norm_fwd(xg, rg, gg, 1e-6, y_dtype=torch.bfloat16)
+            assert torch.equal(ah.cpu(), h_cpu)
+            assert_close(ay, roy, torch.bfloat16, "add_rms_norm with bf16 output")
+
+
+def test_host_op_on_a_long_hidden_size(ops, gpu):
+    """aten-signature native_layer_norm on [2, 3, 49152] bf16 (6 packs a lane)."""
+    x = (0.3 + torch.randn(2, 3, 49152, generator=gen(1470))).bfloat16()
+    w = (1 + 0.1 * torch.randn(49152, generator=gen(1471))).bfloat16()
+    b = (0.1 * torch.randn(49152, generator=gen(1472))).bfloat16()
+    y, mean, rstd = ops.native_layer_norm(x.to(gpu), [49152], w.to(gpu), b.to(gpu), 1e-5)
+    ref = torch.nn.functional.layer_norm(x.float(), [49152], w.float(), b.float(), 1e-5)
+    assert_close(y, to_np32(ref), torch.bfloat16, "native_layer_norm long rows")
+    assert mean.shape == (2, 3, 1) and rstd.shape == (2, 3, 1)

@@ -212,7 +212,7 @@ int norm_fwd(const void* x, const void* res, const void* gamma, const void* beta
   if (add) bits |= (uintptr_t)res | (uintptr_t)h;
   const bool off_line = (bits & 127u) != 0;
   if (int e = make_plan(OC_NORM_FWD, M, N, esize_of(xd), current_num_cus(), g_override[op],
-                        false, &plan, false, !RMS, esize_of(wd) > esize_of(xd), off_line))
+                        false, &plan, false, !RMS, esize_of(wd) > esize_of(xd), off_line, add))
     return e;
   NormFwdArgs a{x, gamma, RMS ? nullptr : beta, y, RMS ? nullptr : mean, rstd, M, (int)N, eps};
   if (add) {

@@ -6,7 +6,10 @@
 // workgroup of BLOCK threads handles BLOCK/G rows per iteration and strides
 // over the rows persistently, which lets the per-column quantities (gamma,
 // beta, and in the backward pass the dgamma/dbeta partial sums) stay in
-// registers from the first row to the last.
+// registers from the first row to the last.  Forward rows of more packs a lane
+// than the registers hold beside their weights (norm_fwd_holds_weights() in
+// plan.hpp: 16-bit rows beyond 32768 elements, up to 131072) keep only the row and
+// read gamma / beta, which stay in L2, where the output needs them.
 //
 // What these kernels stand in for in the reference (the arithmetic, not the
 // code shape):
@@ -72,28 +75,36 @@ norm_fwd_resident_kernel(const T* __restrict__ x, const T* res, const WT* __rest
   __shared__ float red[reduce_lds_floats<G, BLOCK, 2 * R>::value];
   int phase = 0;
   const int slot = threadIdx.x / G;
-  const int lane = threadIdx.x % G;
+  const int lane0 = threadIdx.x % G;
   const float fN = (float)N;
   const float inv_n = 1.0f / fN;
 
   // gamma/beta of this lane's columns stay in registers for all rows: widened to
   // fp32 once when they are few, otherwise in storage format and widened per row.
+  // Rows of more packs a lane than norm_fwd_holds_weights() allows leave them in
+  // memory and load each pack of them (from L2) where the output needs it.
   constexpr bool kWideWeights = V * E <= 16;
+  constexpr bool kHold =
+      norm_fwd_holds_weights((int)sizeof(T), (int)sizeof(WT), G, V, FAST, RMS, ADD);
   const bool exact = N == G * V * E;  // every pack of every lane lies inside the row
-  Pack<WT, E> gp[V];
-  Pack<WT, E> bp[RMS ? 1 : V];
+  Pack<WT, E> gp[kHold ? V : 1];
+  Pack<WT, E> bp[RMS || !kHold ? 1 : V];
+  if constexpr (kHold) {
 #pragma unroll
-  for (int c = 0; c < V; ++c) {
-    const int e0 = (c * G + lane) * E;
-    gp[c] = gamma ? load_row_pack<WT, E, false>(gamma, e0, N, true, 1.0f)
-                  : Pack<WT, E>::splat(1.0f);
-    if constexpr (!RMS)
-      bp[c] = beta ? load_row_pack<WT, E, false>(beta, e0, N, true, 0.0f) : Pack<WT, E>::zero();
+    for (int c = 0; c < V; ++c) {
+      const int e0 = (c * G + lane0) * E;
+      gp[c] = gamma ? load_row_pack<WT, E, false>(gamma, e0, N, true, 1.0f)
+                    : Pack<WT, E>::splat(1.0f);
+      if constexpr (!RMS)
+        bp[c] = beta ? load_row_pack<WT, E, false>(beta, e0, N, true, 0.0f) : Pack<WT, E>::zero();
+    }
   }
 
   const int64_t nrb = (M + RPI - 1) / RPI;
   for (int64_t rb = blockIdx.x; rb < nrb; rb += gridDim.x) {
     const int64_t row0 = (rb * RPB + slot) * R;
+    // (many packs a lane: their offsets are formed where they are used, not held)
+    const int lane = lane_again<!kHold>(lane0);
     bool ok[R];
     Pack<T, E> xp[R][V];
 #pragma unroll
@@ -258,6 +269,7 @@ norm_fwd_resident_kernel(const T* __restrict__ x, const T* res, const WT* __rest
     float nm1rs[R];
 #pragma unroll
     for (int r = 0; r < R; ++r) nm1rs[r] = -m1[r] * rs[r];
+    const int ls = lane_after<!kHold>(lane0, nm1rs[0]);
 #pragma unroll
     for (int r = 0; r < R; ++r) {
       TY* yr = y + (row0 + r) * (int64_t)N;
@@ -265,29 +277,39 @@ norm_fwd_resident_kernel(const T* __restrict__ x, const T* res, const WT* __rest
       for (int c = 0; c < V; ++c) {
         keep_packed(xp[r][c]);
         if constexpr (ADD)
-          row_store<T, E, true, FAST>(h + (row0 + r) * (int64_t)N, (c * G + lane) * E, N, ok[r],
+          row_store<T, E, true, FAST>(h + (row0 + r) * (int64_t)N, (c * G + ls) * E, N, ok[r],
                                       xp[r][c]);
-        if constexpr (!kWideWeights) {
+        if constexpr (kHold && !kWideWeights) {
           keep_packed(gp[c]);
           if constexpr (!RMS) keep_packed(bp[c]);
         }
+        Pack<WT, E> gl, bl;
+        if constexpr (!kHold) {
+          const int e0 = (c * G + ls) * E;
+          gl = gamma ? load_row_pack<WT, E, false>(gamma, e0, N, true, 1.0f)
+                     : Pack<WT, E>::splat(1.0f);
+          if constexpr (!RMS)
+            bl = beta ? load_row_pack<WT, E, false>(beta, e0, N, true, 0.0f) : Pack<WT, E>::zero();
+        }
+        const Pack<WT, E>& gc = kHold ? gp[kHold ? c : 0] : gl;
+        const Pack<WT, E>& bc = RMS ? gc : (kHold ? bp[kHold && !RMS ? c : 0] : bl);
         Pack<TY, E> o;
 #pragma unroll
         for (int i = 0; i < E; ++i) {
           float v;
           if constexpr (RMS)
-            v = (xp[r][c].get(i) * rs[r]) * gp[c].get(i);
+            v = (xp[r][c].get(i) * rs[r]) * gc.get(i);
           else if constexpr (sizeof(T) == 2)
             // (x - mean0) * rs - m1 * rs in one FMA: one instruction fewer an element;
             // on a constant row x - mean0 and m1 are exactly zero, so y is still beta
-            v = fmaf(xp[r][c].get(i) - mean0[r], rs[r], nm1rs[r]) * gp[c].get(i) + bp[c].get(i);
+            v = fmaf(xp[r][c].get(i) - mean0[r], rs[r], nm1rs[r]) * gc.get(i) + bc.get(i);
           else
-            v = (((xp[r][c].get(i) - mean0[r]) - m1[r]) * rs[r]) * gp[c].get(i) + bp[c].get(i);
+            v = (((xp[r][c].get(i) - mean0[r]) - m1[r]) * rs[r]) * gc.get(i) + bc.get(i);
           o.set(i, v);
         }
-        row_store<TY, E, true, FAST>(yr, (c * G + lane) * E, N, ok[r], o);
+        row_store<TY, E, true, FAST>(yr, (c * G + ls) * E, N, ok[r], o);
       }
-      if (ok[r] && lane == 0) {
+      if (ok[r] && lane0 == 0) {
         if constexpr (!RMS)
           // (a row with an inf element has NaN variance; its mean is NaN as well, as the
           // Welford recurrence of the CPU kernel gives)

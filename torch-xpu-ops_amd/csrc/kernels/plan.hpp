@@ -75,12 +75,46 @@ constexpr int kSplitMaxChunks = 1024;
 // fewer, fatter lanes on every op of the family.
 constexpr int v_pref(OpClass, int esize) { return esize == 4 ? 4 : 2; }
 
+// The resident norm forward keeps gamma / beta of a lane's columns in registers
+// across its rows while they fit; at 1024 lanes, rows of more packs a lane than
+// the table below leave the weights in memory, load each pack of them (from L2)
+// where the output needs it, and hold only the row.  esize / wsize: bytes of a
+// row / weight element.  Measured, bf16 rows, against the multi-pass kernel that
+// served rows beyond 4 packs a lane before (2048 rows): N = 40960 LayerNorm 84 ->
+// 65 us (fp32 weights 90 -> 72), RMSNorm 66 -> 59; 65536: 109 -> 101 and 104 ->
+// 95; 1024 rows of 131072: 114 -> 105 and 114 -> 98.  Held against looked up, where
+// both fit the registers (8192 rows of 40960 / 4096 of 49152 / 8192 of 65536):
+// LayerNorm bf16 weights 226 / 143 us against 244 / 153; RMSNorm bf16 weights 240 /
+// 147 / 373 against 227 / 144 / 384 (5 and 6 packs held leave one workgroup a
+// compute unit where the lookup keeps two); RMSNorm fp32 weights 222 / 136 / 400
+// against 236 / 145 / 395.  Up to 4 packs the held weights win by 5-20 %.  The fp32
+// LayerNorm with its weights held spilled from 5 packs a lane (N = 20480..32768:
+// 209..229 -> 62..104 us); the fp32 RMSNorm holds 8 packs and is 3 % faster so.
+constexpr int kNormFwdHoldMaxV = 4;
+// With the residual add fused in (a second row in flight a lane) only the lookup
+// fits beyond 4 packs, and rows up to norm_fwd_add_max_v() packs a lane.
+constexpr bool norm_fwd_holds_weights(int esize, int wsize, int G, int V, bool fast, bool rms,
+                                      bool add) {
+  if (!fast || G != 1024 || V <= kNormFwdHoldMaxV) return true;
+  if (add) return false;
+  if (esize == 4) return rms && V <= 8;
+  if (wsize == 2) return rms ? V == 8 : V <= 6;
+  return rms && V <= 6;
+}
+
+constexpr int norm_fwd_add_max_v(int esize, bool rms) { return esize == 4 && !rms ? 10 : 12; }
+
 // Largest packs per lane the register file holds for a G-lane row group.
 // G = 1024 means 16 wavefronts per workgroup, i.e. at most 128 VGPRs a lane.
 constexpr int v_max(OpClass oc, int esize, int G) {
   int v = 1;
   switch (oc) {
-    case OC_NORM_FWD: v = esize == 4 ? 16 : 8; break;
+    // (at 1024 lanes without the weights: 16 packs, a 131072-element 16-bit row or
+    // a 65536-element fp32 row)
+    case OC_NORM_FWD:
+      if (G >= 1024) return 16;
+      v = esize == 4 ? 16 : 8;
+      break;
     case OC_NORM_BWD: v = esize == 4 ? 8 : 4; break;
     // the forward keeps long rows in storage format: 16 packs a lane at any
     // G (a 131072-element 16-bit row, a 65536-element fp32 row)
@@ -195,8 +229,11 @@ constexpr bool variant_built(OpClass oc, int esize, int G, int V, bool fast) {
     // LayerNorm / RMSNorm rows of hidden sizes such as 5120, 6144, 10240, 12288
     // (640, 768, 1280, 1536 16-bit packs): 3 packs a lane; 5 on 512 lanes for the
     // fp32 LayerNorm forward (see norm_layout())
-    if (!is_group_class(oc))
+    if (!is_group_class(oc)) {
+      if (oc == OC_NORM_FWD && G == kMaxG && V > kNormFwdHoldMaxV)
+        return V == 5 || V == 6 || V == 10 || V == 12;
       return G >= 64 && (V == 3 || (V == 5 && oc == OC_NORM_FWD && esize == 4 && G == 512));
+    }
     // (and 6..10 packs on 512 lanes, which make_plan() prefers to 1024 lanes)
     return G == kMaxG || (G >= 64 && (V == 3 || V == 5)) ||
            (G == 512 && V <= group_half_lanes_max_v(oc));
@@ -294,9 +331,11 @@ inline bool norm_layout(OpClass oc, int esize, int64_t packs, bool layer_norm, b
 // layer_norm: the norm op is LayerNorm (statistics of two sums, beta), not RMSNorm.
 // wide_weights: fp32 gamma/beta beside 16-bit rows.
 // off_line: a tensor of the call does not start on a 128-byte cache line.
+// fused_add: the norm forward adds a residual row first (two rows in flight a lane).
 inline int make_plan(OpClass oc, int64_t M, int64_t N, int esize, int num_cus, const Override& ov,
                      bool want_cols, Plan* out, bool force_general = false,
-                     bool layer_norm = false, bool wide_weights = false, bool off_line = false) {
+                     bool layer_norm = false, bool wide_weights = false, bool off_line = false,
+                     bool fused_add = false) {
   Plan p;
   const int E = 16 / esize;
   p.fast = (N % E) == 0 && !force_general;
@@ -386,6 +425,18 @@ inline int make_plan(OpClass oc, int64_t M, int64_t N, int esize, int num_cus, c
       if (softmax && p.fast && G == kMaxG &&
           v_exact <= kMaxV && variant_built(oc, esize, G, (int)v_exact, true))
         V = (int)v_exact;
+      // norm forward rows beyond the packs whose weights a lane holds: the next
+      // pack count that is built (5, 6, 8, 10, 12, 16)
+      if (oc == OC_NORM_FWD && p.fast && G == kMaxG && v_exact > kNormFwdHoldMaxV) {
+        int64_t v = v_exact;
+        while (v < kMaxV && !variant_built(oc, esize, G, (int)v, true)) ++v;
+        V = (int)v;
+        if (fused_add && V > norm_fwd_add_max_v(esize, !layer_norm)) V = kMaxV + 1;  // multi-pass
+        // a handful of the longest rows: one workgroup takes 15 us for a row of 131072
+        // bf16 elements, the split over workgroups 10 us for up to 64 of them (128 rows:
+        // 19 us either way; rows of 65536 and fewer are faster here from 16 rows down)
+        if (V >= 10 && M < num_cus / 2) V = kMaxV + 1;
+      }
       if (!p.fast && V < v_pref(oc, esize)) V = v_pref(oc, esize);
     }
     const bool holds = (int64_t)G * V >= packs;
@@ -463,6 +514,13 @@ inline int make_plan(OpClass oc, int64_t M, int64_t N, int esize, int num_cus, c
       if (nrb <= cap * 32) grid = cap;
     }
   }
+  // Rows whose weights are not held gain nothing from a workgroup that walks
+  // several rows: one workgroup a row (8192 rows of 40960 bf16: LayerNorm 253 ->
+  // 243 us, with fp32 weights 270 -> 254 us, RMSNorm 235 -> 227 us).
+  if (oc == OC_NORM_FWD && p.resident && ov.bpc == 0 &&
+      !norm_fwd_holds_weights(esize, wide_weights ? 4 : esize, p.G, p.V, p.fast, !layer_norm,
+                              fused_add))
+    grid = nrb;
   if (grid > nrb) grid = nrb;
   if (grid > 0x7fffffff) grid = 0x7fffffff;
   if (grid < 1) grid = 1;
