@@ -1,11 +1,12 @@
 """log_softmax backward on vocabulary-sized rows (the cross_entropy case): rows too long for both
 tensors in registers keep grad resident and stream y past it (log_softmax_bwd_grad_resident_kernel;
 the reference walks the row twice in LogSoftmaxBackward, src/ATen/native/xpu/sycl/
-SoftMaxKernels.cpp:991-1150).  Every packs-per-lane count of the kernel (5..16 for 16-bit rows,
-9..16 for float32 rows), with the row end inside and at the end of a lane's last pack, misaligned
+SoftMaxKernels.cpp:991-1150).  Every packs-per-lane count of the kernel (5..20 for 16-bit rows,
+9..20 for float32 rows), with the row end inside and at the end of a lane's last pack, misaligned
 tensors and -inf / NaN entries, against the CPU oracle at the family's tolerances (float32
 rtol = atol = 1e-5; 16-bit atol 1e-2, rtol 1.6e-2) and against the multi-pass kernel forced on
-the same inputs."""
+the same inputs.  The 16-bit forward holds rows of 17..20 packs a lane (the 151936 / 152064-entry
+vocabularies) in registers as well: checked against the oracle and the multi-pass kernel."""
 import pytest
 import torch
 
@@ -44,7 +45,9 @@ def _case(cabi, oracle, gpu, M, N, dtype, off, seed, gi_dtype=None):
 def test_every_pack_count_16bit(cabi, oracle, gpu, dtype):
     # packs a lane = ceil(N / 8192): 5 (one pack into the fifth round), 5 exactly, 6 .. 16
     for i, N in enumerate((32776, 40960, 49144, 50304, 65536, 73728, 81912, 90112, 100000, 106496,
-                           114688, 122880, 128256, 131072)):
+                           114688, 122880, 128256, 131072,
+                           # 17 .. 20: one pack into the round, Qwen's vocabularies, the maximum
+                           131080, 140000, 151936, 152064, 163840)):
         _case(cabi, oracle, gpu, 3, N, dtype, 0, 900 + i)
     _case(cabi, oracle, gpu, 2, 50304, dtype, 3, 950)     # 6 bytes off 16-byte alignment
     _case(cabi, oracle, gpu, 2, 128256, dtype, 1, 951)
@@ -52,7 +55,8 @@ def test_every_pack_count_16bit(cabi, oracle, gpu, dtype):
 
 def test_every_pack_count_float32(cabi, oracle, gpu):
     # float32 rows: 4 elements a pack, the two-tensor kernels end at 32768 elements
-    for i, N in enumerate((32772, 36864, 40000, 45056, 50304, 53248, 57344, 61440, 65536)):
+    for i, N in enumerate((32772, 36864, 40000, 45056, 50304, 53248, 57344, 61440, 65536,
+                           65540, 70000, 75968, 81920)):
         _case(cabi, oracle, gpu, 2, N, torch.float32, 0, 960 + i)
     _case(cabi, oracle, gpu, 2, 50304, torch.float32, 1, 970)
 
@@ -84,3 +88,37 @@ def test_softmax_and_ragged_rows_keep_the_multi_pass_kernel(cabi, oracle, gpu):
         gi = cabi.softmax_bwd(grad.to(gpu), y.to(gpu), is_log)
         assert_close(gi, oracle.softmax_bwd(to_np32(grad), to_np32(y), is_log), torch.bfloat16,
                      "N=%d log=%d" % (N, is_log))
+
+
+@pytest.mark.parametrize("dtype", [torch.bfloat16, torch.float16], ids=str)
+@pytest.mark.parametrize("is_log", [False, True], ids=["softmax", "log_softmax"])
+def test_forward_rows_of_17_to_20_packs_a_lane(cabi, oracle, gpu, dtype, is_log):
+    code = cabi.dtype_code(dtype)
+    for i, (V, N) in enumerate(((17, 131080), (18, 140000), (19, 151936), (19, 152064),
+                                (20, 163840))):
+        M = 3
+        print("case vocabulary forward", dtype, is_log, (M, N), flush=True)
+        p = cabi.plan(cabi.OP_SOFTMAX_FWD, M, N, code, code)
+        assert (p["resident"], p["lanes_per_row"], p["packs_per_lane"]) == (1, 1024, V), p
+        x = (3.0 * torch.randn(M, N, generator=gen(1500 + i))).to(dtype)
+        x[0, N // 2:] = float("-inf")
+        x[1, -1] = 30.0  # the maximum in the last pack of the row
+        xg = x.to(gpu)
+        y = cabi.softmax_fwd(xg, is_log)
+        oy = oracle.softmax_fwd(to_np32(x), is_log)
+        assert_close(y, oy, dtype, "forward [%d, %d] %s" % (M, N, dtype))
+        try:
+            cabi.set_override(cabi.OP_SOFTMAX_FWD, -1, 1)  # the multi-pass kernel
+            ref = cabi.softmax_fwd(xg, is_log)
+        finally:
+            cabi.clear_overrides()
+        assert_close(y, to_np32(ref), dtype, "register-resident vs multi-pass forward %d" % N)
+        assert torch.equal(cabi.softmax_fwd(xg, is_log).view(torch.uint8), y.view(torch.uint8))
+    # float32 output from float16 input (half_to_float, SoftMax.cpp:49-55) on the same kernels
+    if dtype == torch.float16:
+        x = (3.0 * torch.randn(2, 151936, generator=gen(1510))).to(dtype)
+        y32 = cabi.softmax_fwd(x.to(gpu), is_log, out_dtype=torch.float32)
+        assert_close(y32, oracle.softmax_fwd(to_np32(x), is_log), torch.float32,
+                     "half_to_float 151936")
+    # one row more than the registers hold: the multi-pass kernel
+    assert cabi.plan(cabi.OP_SOFTMAX_FWD, 3, 163848, code, code)["resident"] == 0

@@ -148,7 +148,7 @@ int launch_softmax_strided_bwd(const StridedPlan& plan, const SoftmaxStridedBwdA
 template <int... Is>
 struct ilist {};
 using GList = ilist<8, 16, 32, 64, 128, 256, 512, 1024>;
-using VList = ilist<1, 2, 3, 4, 5, 6, 7, 8, 9, 10, 11, 12, 13, 14, 15, 16>;
+using VList = ilist<1, 2, 3, 4, 5, 6, 7, 8, 9, 10, 11, 12, 13, 14, 15, 16, 17, 18, 19, 20>;
 using BList = ilist<256, 512, 1024>;
 
 template <template <int, int, int> class L, class Ctx, int G, int V, int... Bs>

@@ -63,6 +63,14 @@ struct Plan {
 constexpr int kMinG = 8;
 constexpr int kMaxG = 1024;
 constexpr int kMaxV = 16;
+// The 16-bit softmax forward alone goes to 20 packs a lane (163840-element rows:
+// the 151936 / 152064-entry vocabularies).
+constexpr int kSoftmaxFwdMaxV16 = 20;
+// Packs of grad a lane of the grad-resident log_softmax backward holds at most.
+constexpr int kGradResidentMaxV = 20;
+constexpr int max_v_of(OpClass oc, int esize) {
+  return oc == OC_SOFTMAX_FWD && esize == 2 ? kSoftmaxFwdMaxV16 : kMaxV;
+}
 constexpr int kStreamBlock = 1024;
 // Split-row path: a chunk is a whole number of workgroup strides and at least
 // four of them (32768 16-bit elements); a row is cut into at most 1024 chunks.
@@ -118,7 +126,7 @@ constexpr int v_max(OpClass oc, int esize, int G) {
     case OC_NORM_BWD: v = esize == 4 ? 8 : 4; break;
     // the forward keeps long rows in storage format: 16 packs a lane at any
     // G (a 131072-element 16-bit row, a 65536-element fp32 row)
-    case OC_SOFTMAX_FWD: return 16;
+    case OC_SOFTMAX_FWD: return G >= 1024 ? max_v_of(oc, esize) : 16;
     case OC_SOFTMAX_BWD: v = esize == 4 ? 16 : 8; break;
     // GroupNorm lanes hold the row (and dY) only, no weights or column sums, so
     // 16-bit rows keep 8 packs a lane at 1024 lanes (128 VGPRs) and 10 at 512
@@ -211,7 +219,7 @@ constexpr int gn_mode(int64_t L, int64_t HxW, int64_t D, int E) {
 constexpr int group_half_lanes_max_v(OpClass oc) { return oc == OC_GROUP_FWD ? 10 : 7; }
 
 constexpr bool variant_built(OpClass oc, int esize, int G, int V, bool fast) {
-  if (G < kMinG || G > kMaxG || (G & (G - 1)) || V < 1 || V > kMaxV) return false;
+  if (G < kMinG || G > kMaxG || (G & (G - 1)) || V < 1 || V > max_v_of(oc, esize)) return false;
   // GroupNorm rows take the packs they have, not the next power of two (a
   // 40960-element bf16 row is 1024 lanes x 5 packs, not x 8): 3 or 5 packs a
   // lane from one wavefront up, anything up to the budget at 1024 lanes
@@ -423,7 +431,7 @@ inline int make_plan(OpClass oc, int64_t M, int64_t N, int esize, int num_cus, c
       V = pow2_ceil((packs + G - 1) / G);
       const int64_t v_exact = (packs + G - 1) / G;
       if (softmax && p.fast && G == kMaxG &&
-          v_exact <= kMaxV && variant_built(oc, esize, G, (int)v_exact, true))
+          v_exact <= max_v_of(oc, esize) && variant_built(oc, esize, G, (int)v_exact, true))
         V = (int)v_exact;
       // norm forward rows beyond the packs whose weights a lane holds: the next
       // pack count that is built (5, 6, 8, 10, 12, 16)
@@ -570,7 +578,7 @@ inline int make_plan(OpClass oc, int64_t M, int64_t N, int esize, int num_cus, c
     }
   }
   if (oc == OC_SOFTMAX_BWD && !p.resident && p.fast && ov.G == 0 &&
-      packs <= (int64_t)kMaxG * kMaxV)
+      packs <= (int64_t)kMaxG * kGradResidentMaxV)
     p.grad_resident = true;
   *out = p;
   return 0;

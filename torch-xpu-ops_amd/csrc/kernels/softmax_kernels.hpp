@@ -156,7 +156,8 @@ softmax_fwd_resident_kernel(const TI* __restrict__ x, TO* __restrict__ y, MaskRe
     // ragged rows drop from 94 to 54 registers).  From 10 packs a lane one
     // workgroup a compute unit is the better layout for log_softmax, and there
     // recomputing the offsets measured 1-2 % slower, so those keep them.
-    constexpr bool kFreshOffsets = !(FAST && G == 1024 && V > kSoftmaxFreshOffsetsMaxV);
+    constexpr bool kFreshOffsets =
+        !(FAST && G == 1024 && V > kSoftmaxFreshOffsetsMaxV && V <= kMaxV);
     const int lane = lane_again<kFreshOffsets>(lane0);
     const int64_t row = rb * RPB + slot;
     const bool ok = RPB == 1 ? true : row < M;

@@ -204,7 +204,7 @@ struct SoftmaxBwdLauncher {
 };
 
 // log_softmax backward of rows too long for both tensors in registers but not for
-// grad alone: whole packs, at most 1024 lanes x 16 packs.  False: not this case.
+// grad alone: whole packs, at most 1024 lanes x 20 packs.  False: not this case.
 template <class TG, class TO, int V>
 inline void launch_grad_resident_v(const Plan& plan, const SoftmaxBwdArgs& a, hipStream_t stream) {
   hipLaunchKernelGGL((log_softmax_bwd_grad_resident_kernel<TG, TO, V, kStreamBlock>),
@@ -233,6 +233,10 @@ inline bool launch_log_softmax_bwd_grad_resident(const Plan& plan, const Softmax
     case 14: launch_grad_resident_v<TG, TO, 14>(plan, a, stream); return true;
     case 15: launch_grad_resident_v<TG, TO, 15>(plan, a, stream); return true;
     case 16: launch_grad_resident_v<TG, TO, 16>(plan, a, stream); return true;
+    case 17: launch_grad_resident_v<TG, TO, 17>(plan, a, stream); return true;
+    case 18: launch_grad_resident_v<TG, TO, 18>(plan, a, stream); return true;
+    case 19: launch_grad_resident_v<TG, TO, 19>(plan, a, stream); return true;
+    case 20: launch_grad_resident_v<TG, TO, 20>(plan, a, stream); return true;
   }
   return false;
 }
