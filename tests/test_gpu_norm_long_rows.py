@@ -11,7 +11,7 @@ add and the output cast fused in, and for run-to-run determinism."""
 import pytest
 import torch
 
-from helpers import assert_close, gen, to_np32
+from helpers import assert_close, colsum_slack, gen, to_np32
 
 pytestmark = pytest.mark.gpu
 
@@ -147,3 +147,98 @@ def test_host_op_on_a_long_hidden_size(ops, gpu):
     ref = torch.nn.functional.layer_norm(x.float(), [49152], w.float(), b.float(), 1e-5)
     assert_close(y, to_np32(ref), torch.bfloat16, "native_layer_norm long rows")
     assert mean.shape == (2, 3, 1) and rstd.shape == (2, 3, 1)
+
+
+# ---- backward: 16-bit rows of 16392 .. 32768 elements, dgamma sums in LDS ------------------
+
+BWD_N = [(3, 16392), (3, 18432), (3, 20480), (3, 24576), (4, 24584), (4, 28672), (4, 32768)]
+
+
+def _bwd_case(cabi, oracle, gpu, M, N, dtype, wdtype, seed, rms):
+    g = gen(seed)
+    x = (0.3 + torch.randn(M, N, generator=g)).to(dtype)
+    dy = torch.randn(M, N, generator=g).to(dtype)
+    gamma = (1 + 0.1 * torch.randn(N, generator=g)).to(wdtype)
+    xg, dyg, gg = x.to(gpu), dy.to(gpu), gamma.to(gpu)
+    what = "[%d, %d] %s / %s" % (M, N, dtype, wdtype)
+    # float32 column sums: the summation's own rounding is allowed for (helpers.colsum_slack)
+    wide = wdtype == torch.float32
+    if rms:
+        _, rstd = cabi.rms_norm_fwd(xg, gg, 1e-6)
+        sl = colsum_slack(dy.double() * x.double() * rstd.cpu().double().reshape(M, 1)) if wide else None
+        dx, dg = cabi.rms_norm_bwd(dyg, xg, rstd, gg)
+        odx, odg = oracle.rms_norm_bwd(to_np32(dy), to_np32(x), (N,), to_np32(rstd), to_np32(gamma))
+        assert_close(dx, odx, dtype, "rms_norm dx " + what)
+        assert_close(dg, odg, wdtype, "rms_norm dgamma " + what, slack=sl)
+        try:
+            cabi.set_override(cabi.OP_RMS_NORM_BWD, -1, 1)
+            mdx, mdg = cabi.rms_norm_bwd(dyg, xg, rstd, gg)
+        finally:
+            cabi.clear_overrides()
+        assert_close(dx, to_np32(mdx), dtype, "rms_norm dx against the multi-pass kernels " + what)
+        # the same bits on a second run, and with only one of the two results asked for
+        dx2, dg2 = cabi.rms_norm_bwd(dyg, xg, rstd, gg)
+        assert torch.equal(dx2.view(torch.uint8), dx.view(torch.uint8))
+        assert torch.equal(dg2.view(torch.uint8), dg.view(torch.uint8))
+        dx3, none = cabi.rms_norm_bwd(dyg, xg, rstd, gg, want=(True, False))
+        assert none is None and torch.equal(dx3.view(torch.uint8), dx.view(torch.uint8))
+        none, dg3 = cabi.rms_norm_bwd(dyg, xg, rstd, gg, want=(False, True))
+        assert none is None and torch.equal(dg3.view(torch.uint8), dg.view(torch.uint8))
+    else:
+        beta = (0.1 * torch.randn(N, generator=g)).to(wdtype)
+        _, mean, rstd = cabi.layer_norm_fwd(xg, gg, beta.to(gpu), 1e-5)
+        xhat = (x.double() - mean.cpu().double().reshape(M, 1)) * rstd.cpu().double().reshape(M, 1)
+        sl = colsum_slack(dy.double() * xhat) if wide else None
+        dx, dg, db = cabi.layer_norm_bwd(dyg, xg, mean, rstd, gg)
+        odx, odg, odb = oracle.layer_norm_bwd(to_np32(dy), to_np32(x), (N,), to_np32(mean),
+                                              to_np32(rstd), to_np32(gamma))
+        assert_close(dx, odx, dtype, "layer_norm dx " + what)
+        assert_close(dg, odg, wdtype, "layer_norm dgamma " + what, slack=sl)
+        assert_close(db, odb, wdtype, "layer_norm dbeta " + what,
+                     slack=colsum_slack(dy.double()) if wide else None)
+        dx2, dg2, db2 = cabi.layer_norm_bwd(dyg, xg, mean, rstd, gg)
+        for a, b in ((dx, dx2), (dg, dg2), (db, db2)):
+            assert torch.equal(a.view(torch.uint8), b.view(torch.uint8))
+
+
+@pytest.mark.parametrize("dtype", [torch.float16, torch.bfloat16], ids=str)
+@pytest.mark.parametrize("mixed", [False, True], ids=["w_same", "w_fp32"])
+def test_backward_with_dgamma_sums_in_lds(cabi, oracle, gpu, dtype, mixed):
+    wdtype = torch.float32 if mixed else dtype
+    code, wcode = cabi.dtype_code(dtype), cabi.dtype_code(wdtype)
+    for i, (V, N) in enumerate(BWD_N):
+        # one row, fewer rows than workgroups, and more rows than the 256 workgroups of the grid
+        for M in ((1, 37, 300) if i in (1, 6) else (5 + i,)):
+            print("case long rows backward", dtype, mixed, (M, N), flush=True)
+            p = cabi.plan(cabi.OP_RMS_NORM_BWD, M, N, code, wcode)
+            assert (p["resident"], p["lanes_per_row"], p["packs_per_lane"]) == (1, 1024, V), p
+            p = cabi.plan(cabi.OP_LAYER_NORM_BWD, M, N, code, wcode)
+            # the LayerNorm backward with four packs a lane keeps the multi-pass kernels
+            assert p["resident"] == (1 if V == 3 else 0), p
+            _bwd_case(cabi, oracle, gpu, M, N, dtype, wdtype, 1480 + i, True)
+            _bwd_case(cabi, oracle, gpu, M, N, dtype, wdtype, 1490 + i, False)
+
+
+def test_fused_add_backward_on_long_rows(cabi, oracle, gpu):
+    """The residual path's gradient added to dx, bf16 rows of 20480 and 32768 elements."""
+    for i, N in enumerate((20480, 32768)):
+        M = 9 + i
+        g = gen(1495 + i)
+        h = torch.randn(M, N, generator=g).bfloat16()
+        dy = torch.randn(M, N, generator=g).bfloat16()
+        dh_in = torch.randn(M, N, generator=g).bfloat16()
+        gamma = (1 + 0.1 * torch.randn(N, generator=g)).bfloat16()
+        hg, dyg, dhg, gg = h.to(gpu), dy.to(gpu), dh_in.to(gpu), gamma.to(gpu)
+        _, rstd = cabi.rms_norm_fwd(hg, gg, 1e-6)
+        dh, dg = cabi.add_rms_norm_bwd(dyg, dhg, hg, rstd, gg)
+        odh, odg = oracle.add_rms_norm_bwd(to_np32(dy), to_np32(dh_in), to_np32(h), (N,),
+                                           to_np32(rstd), to_np32(gamma))
+        assert_close(dh, odh, torch.bfloat16, "add_rms_norm dh [%d, %d]" % (M, N))
+        assert_close(dg, odg, torch.bfloat16, "add_rms_norm dgamma [%d, %d]" % (M, N))
+        _, mean, rstd = cabi.layer_norm_fwd(hg, gg, gg, 1e-5)
+        dh, dg, db = cabi.add_layer_norm_bwd(dyg, dhg, hg, mean, rstd, gg)
+        odh, odg, odb = oracle.add_layer_norm_bwd(to_np32(dy), to_np32(dh_in), to_np32(h), (N,),
+                                                  to_np32(mean), to_np32(rstd), to_np32(gamma))
+        assert_close(dh, odh, torch.bfloat16, "add_layer_norm dh [%d, %d]" % (M, N))
+        assert_close(dg, odg, torch.bfloat16, "add_layer_norm dgamma [%d, %d]" % (M, N))
+        assert_close(db, odb, torch.bfloat16, "add_layer_norm dbeta [%d, %d]" % (M, N))

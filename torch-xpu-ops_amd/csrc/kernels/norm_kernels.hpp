@@ -9,7 +9,9 @@
 // registers from the first row to the last.  Forward rows of more packs a lane
 // than the registers hold beside their weights (norm_fwd_holds_weights() in
 // plan.hpp: 16-bit rows beyond 32768 elements, up to 131072) keep only the row and
-// read gamma / beta, which stay in L2, where the output needs them.
+// read gamma / beta, which stay in L2, where the output needs them; backward rows
+// of three or four 16-bit packs a lane on 1024 lanes (norm_bwd_sums_in_lds():
+// 16392..32768 elements) keep their dgamma sums in LDS and gamma in L2.
 //
 // What these kernels stand in for in the reference (the arithmetic, not the
 // code shape):
@@ -710,27 +712,52 @@ norm_bwd_resident_kernel(const T* __restrict__ dy, const T* __restrict__ x, cons
   __shared__ float fold[FOLD_FLOATS];
   int phase = 0;
   const int slot = threadIdx.x / G;
-  const int lane = threadIdx.x % G;
+  const int lane0 = threadIdx.x % G;
   const float fN = (float)N;
   const float inv_n = 1.0f / fN;
   const bool want_cols = part_dg != nullptr;  // uniform
   constexpr bool kWideWeights = V * E <= 16;  // few weights: widen to fp32 once, not per row
   constexpr bool PF = R == 1 && norm_bwd_prefetches((int)sizeof(T), G, V, FAST, RMS);
+  // LDSG (norm_bwd_sums_in_lds()): rows of three or four packs a lane on 1024 lanes.
+  // The registers hold the row, dY (twice: the next row is on its way) and the dbeta
+  // sums; the dgamma sums live in LDS, each lane adding to its own 16-byte slots
+  // (no other lane touches them, so no barrier), and gamma stays in memory, each
+  // pack of it loaded (from L2) where it is used.
+  constexpr bool LDSG = norm_bwd_sums_in_lds((int)sizeof(T), G, V, FAST);
+  static_assert(!LDSG || (RPB == 1 && R == 1 && E == 8), "one 16-bit row a workgroup");
+  __shared__ __attribute__((aligned(16))) float ldg[LDSG ? G * V * E : 4];
+  // slot h (0, 1) of pack c of this lane: lanes side by side, 16 bytes each
+  auto ldg_slot = [&](int c, int h) { return ldg + ((c * 2 + h) * G + lane0) * 4; };
 
-  Pack<WT, E> gp[V];
-  float dg[V][E];
+  Pack<WT, E> gp[LDSG ? 1 : V];
+  float dg[LDSG ? 1 : V][LDSG ? 1 : E];
   float db[RMS ? 1 : V][RMS ? 1 : E];
 #pragma unroll
   for (int c = 0; c < V; ++c) {
-    const int e0 = (c * G + lane) * E;
-    gp[c] = gamma ? load_row_pack<WT, E, false>(gamma, e0, N, true, 1.0f)
-                  : Pack<WT, E>::splat(1.0f);
+    const int e0 = (c * G + lane0) * E;
+    if constexpr (!LDSG)
+      gp[c] = gamma ? load_row_pack<WT, E, false>(gamma, e0, N, true, 1.0f)
+                    : Pack<WT, E>::splat(1.0f);
+    if constexpr (LDSG) {
+      *reinterpret_cast<float4*>(ldg_slot(c, 0)) = float4{0.0f, 0.0f, 0.0f, 0.0f};
+      *reinterpret_cast<float4*>(ldg_slot(c, 1)) = float4{0.0f, 0.0f, 0.0f, 0.0f};
+    }
 #pragma unroll
     for (int i = 0; i < E; ++i) {
-      dg[c][i] = 0.0f;
+      if constexpr (!LDSG) dg[c][i] = 0.0f;
       if constexpr (!RMS) db[c][i] = 0.0f;
     }
   }
+  // the weights of pack c, for the lane index `ln` (LDSG: made opaque per use, so the
+  // pack offsets are not carried across the row loop)
+  auto weights = [&](int c, int ln) {
+    if constexpr (LDSG) {
+      return gamma ? load_row_pack<WT, E, false>(gamma, (c * G + ln) * E, N, true, 1.0f)
+                   : Pack<WT, E>::splat(1.0f);
+    } else {
+      return gp[c];
+    }
+  };
 
   const int64_t nrb = (M + RPI - 1) / RPI;
   // A row slot past the end of the tensor gets all-zero x and dy, so it adds
@@ -741,6 +768,7 @@ norm_bwd_resident_kernel(const T* __restrict__ dy, const T* __restrict__ x, cons
   auto fetch = [&](int64_t rb, bool (&fok)[R], float (&fmu)[R], float (&frs)[R],
                    Pack<T, E> (&fx)[R][V], Pack<T, E> (&fd)[R][V]) {
     const int64_t frow0 = (rb * RPB + slot) * R;
+    const int lane = lane_again<LDSG>(lane0);
     // (past the last row block the requests go to row 0 and are never used: a
     // branch around them measured 10-15 % slower over the whole kernel)
 #pragma unroll
@@ -770,6 +798,7 @@ norm_bwd_resident_kernel(const T* __restrict__ dy, const T* __restrict__ x, cons
     else
       fetch(rb, ok, mu, rs, xp, dp);
     float acc[2 * R];
+    const int lane = lane_again<LDSG>(lane0);
 #pragma unroll
     for (int r = 0; r < R; ++r) {
       // 16-bit rows: xhat = x*rs - mu*rs in one FMA (rounding far below a 16-bit
@@ -778,23 +807,43 @@ norm_bwd_resident_kernel(const T* __restrict__ dy, const T* __restrict__ x, cons
       acc[2 * r] = acc[2 * r + 1] = 0.0f;
 #pragma unroll
       for (int c = 0; c < V; ++c) {
-        if constexpr (!kWideWeights) keep_packed(gp[c]);
+        if constexpr (!LDSG && !kWideWeights) keep_packed(gp[c]);
+        const Pack<WT, E> gc = weights(c, lane);
+        float t[LDSG ? E : 1];
+        if constexpr (LDSG) {
+          if (want_cols) {
+            const float4 t0 = *reinterpret_cast<const float4*>(ldg_slot(c, 0));
+            const float4 t1 = *reinterpret_cast<const float4*>(ldg_slot(c, 1));
+            t[0] = t0.x, t[1] = t0.y, t[2] = t0.z, t[3] = t0.w;
+            t[4] = t1.x, t[5] = t1.y, t[6] = t1.z, t[7] = t1.w;
+          }
+        }
 #pragma unroll
         for (int i = 0; i < E; ++i) {
           const float xv = xp[r][c].get(i);
           const float xh = RMS ? xv * rs[r]
                                : (sizeof(T) == 2 ? fmaf(xv, rs[r], nmr) : (xv - mu[r]) * rs[r]);
           const float gy = dp[r][c].get(i);
-          const float g = gy * gp[c].get(i);
+          const float g = gy * gc.get(i);
           if constexpr (!RMS) acc[2 * r] += g;
           acc[2 * r + 1] = fmaf(g, xh, acc[2 * r + 1]);
-          dg[c][i] = fmaf(gy, xh, dg[c][i]);
+          if constexpr (LDSG)
+            t[i] = fmaf(gy, xh, t[i]);
+          else
+            dg[c][i] = fmaf(gy, xh, dg[c][i]);
           if constexpr (!RMS) db[c][i] += gy;
+        }
+        if constexpr (LDSG) {
+          if (want_cols) {
+            *reinterpret_cast<float4*>(ldg_slot(c, 0)) = float4{t[0], t[1], t[2], t[3]};
+            *reinterpret_cast<float4*>(ldg_slot(c, 1)) = float4{t[4], t[5], t[6], t[7]};
+          }
         }
       }
     }
     group_allreduce<G, BLOCK, 2 * R, SumOp>(acc, red, phase);
     if (dx != nullptr) {
+      const int ls = lane_after<LDSG>(lane0, acc[1]);
 #pragma unroll
       for (int r = 0; r < R; ++r) {
         T* dr = dx + (row0 + r) * (int64_t)N;
@@ -813,17 +862,18 @@ norm_bwd_resident_kernel(const T* __restrict__ dy, const T* __restrict__ x, cons
 #pragma unroll
           for (int c = 0; c < V; ++c)
             up[c] = row_load<T, E, true, FAST>(dres + (ok[r] ? row0 + r : 0) * (int64_t)N,
-                                               (c * G + lane) * E, N, ok[r], 0.0f);
+                                               (c * G + ls) * E, N, ok[r], 0.0f);
         }
 #pragma unroll
         for (int c = 0; c < V; ++c) {
           keep_packed(xp[r][c]);
           keep_packed(dp[r][c]);
-          if constexpr (!kWideWeights) keep_packed(gp[c]);
+          if constexpr (!LDSG && !kWideWeights) keep_packed(gp[c]);
+          const Pack<WT, E> gc = weights(c, ls);
           Pack<T, E> o;
 #pragma unroll
           for (int i = 0; i < E; ++i) {
-            const float g = dp[r][c].get(i) * gp[c].get(i);
+            const float g = dp[r][c].get(i) * gc.get(i);
             float f;
             if constexpr (sizeof(T) == 2) {
               f = fmaf(xp[r][c].get(i), -ra, fmaf(g, rs[r], cc));
@@ -838,7 +888,7 @@ norm_bwd_resident_kernel(const T* __restrict__ dy, const T* __restrict__ x, cons
             if constexpr (ADD) f += up[c].get(i);
             o.set(i, f);
           }
-          row_store<T, E, true, FAST>(dr, (c * G + lane) * E, N, ok[r], o);
+          row_store<T, E, true, FAST>(dr, (c * G + ls) * E, N, ok[r], o);
         }
       }
     }
@@ -864,11 +914,17 @@ norm_bwd_resident_kernel(const T* __restrict__ dy, const T* __restrict__ x, cons
   if constexpr (RPB == 1) {
 #pragma unroll
     for (int c = 0; c < V; ++c) {
-      const int e0 = (c * G + lane) * E;
+      const int e0 = (c * G + lane0) * E;
       Pack<float, E> pg, pb;
+      if constexpr (LDSG) {
+        const float4 t0 = *reinterpret_cast<const float4*>(ldg_slot(c, 0));
+        const float4 t1 = *reinterpret_cast<const float4*>(ldg_slot(c, 1));
+        pg.set(0, t0.x), pg.set(1, t0.y), pg.set(2, t0.z), pg.set(3, t0.w);
+        pg.set(4, t1.x), pg.set(5, t1.y), pg.set(6, t1.z), pg.set(7, t1.w);
+      }
 #pragma unroll
       for (int i = 0; i < E; ++i) {
-        pg.set(i, dg[c][i]);
+        if constexpr (!LDSG) pg.set(i, dg[c][i]);
         if constexpr (!RMS) pb.set(i, db[c][i]);
       }
       store_row_pack<float, E, false>(out_g, e0, N, true, pg);
@@ -902,7 +958,7 @@ norm_bwd_resident_kernel(const T* __restrict__ dy, const T* __restrict__ x, cons
         if (unit == u && owner) {
 #pragma unroll
           for (int c = 0; c < V; ++c) {
-            const int e0 = (c * G + lane) * E;
+            const int e0 = (c * G + lane0) * E;
 #pragma unroll
             for (int i = 0; i < E; ++i) {
               const float v = pass == 0 ? dg[c][i] : db[RMS ? 0 : c][RMS ? 0 : i];

@@ -123,7 +123,12 @@ constexpr int v_max(OpClass oc, int esize, int G) {
       if (G >= 1024) return 16;
       v = esize == 4 ? 16 : 8;
       break;
-    case OC_NORM_BWD: v = esize == 4 ? 8 : 4; break;
+    // (16-bit rows at 1024 lanes: 4 packs with the dgamma sums in LDS, see
+    // norm_bwd_sums_in_lds())
+    case OC_NORM_BWD:
+      if (G >= 1024 && esize == 2) return 4;
+      v = esize == 4 ? 8 : 4;
+      break;
     // the forward keeps long rows in storage format: 16 packs a lane at any
     // G (a 131072-element 16-bit row, a 65536-element fp32 row)
     case OC_SOFTMAX_FWD: return G >= 1024 ? max_v_of(oc, esize) : 16;
@@ -164,7 +169,24 @@ constexpr int block_threads(OpClass oc, int G) {
 // unit up to 256 lanes (N = 2048: 44.6 -> 43.3 us, 4096: 78 -> 75 us) and loses a
 // little on 512 (N = 7168: 128 -> 130 us, 8192: 142 -> 144 us).
 constexpr bool norm_bwd_prefetches(int esize, int G, int V, bool fast, bool rms) {
+  if (G >= 1024) return false;  // (3 and 4 packs at 1024 lanes: it spills, 104 -> 172 us)
   return fast && esize == 2 && (V >= 3 || (V == 2 && !rms && G <= 256));
+}
+
+// 16-bit backward rows of 16392..32768 elements (hidden sizes 18432, 20480): three
+// or four packs a lane on 1024 lanes.  The column sums of such a lane would take
+// 48-64 registers beside the row and dY, so the dgamma sums live in LDS (96 / 128
+// KB: every lane adds to its own 16-byte slots), the dbeta sums stay in registers
+// and gamma stays in memory (L2).  Measured at 4096 rows against the multi-pass
+// kernels (two passes over X and dY), bf16: N = 18432 RMSNorm 127 -> 104 us,
+// LayerNorm 133 -> 111 us (fp32 weights 147 -> 126 us); 24576: 162 -> 135, 166 ->
+// 143, 180 -> 151 us; 32768 RMSNorm 231 -> 175 us.  The LayerNorm with four packs
+// spills 29-45 registers and loses (237 -> 302 us): it keeps the multi-pass kernels.
+constexpr bool norm_bwd_sums_in_lds(int esize, int G, int V, bool fast) {
+  return fast && esize == 2 && G == 1024 && V >= 3;
+}
+constexpr bool norm_bwd_lds_layout(int esize, int64_t v_exact, bool layer_norm) {
+  return esize == 2 && (v_exact == 3 || (v_exact == 4 && !layer_norm));
 }
 
 // Workgroup sizes a G-lane variant is compiled for.
@@ -228,7 +250,7 @@ constexpr bool variant_built(OpClass oc, int esize, int G, int V, bool fast) {
     // the aligned window) take three packs on half the lanes as well
     if (!fast)
       return (oc == OC_SOFTMAX_FWD || oc == OC_SOFTMAX_BWD || oc == OC_NORM_FWD || oc == OC_NORM_BWD) && esize == 2 &&
-             G >= 64 && V == 3;
+             G >= 64 && V == 3 && !(oc == OC_NORM_BWD && G == kMaxG);
     if (V > v_max(oc, esize, G)) return false;
     // softmax rows that need all 1024 lanes (vocabulary-sized) likewise
     // (and the 16-bit forward takes three packs a lane where that fits better)
@@ -433,6 +455,9 @@ inline int make_plan(OpClass oc, int64_t M, int64_t N, int esize, int num_cus, c
       if (softmax && p.fast && G == kMaxG &&
           v_exact <= max_v_of(oc, esize) && variant_built(oc, esize, G, (int)v_exact, true))
         V = (int)v_exact;
+      // norm backward beyond two packs a lane on 1024 lanes: norm_bwd_sums_in_lds()
+      if (oc == OC_NORM_BWD && p.fast && G == kMaxG && v_exact > 2 && esize == 2)
+        V = norm_bwd_lds_layout(esize, v_exact, layer_norm) ? (int)v_exact : kMaxV + 1;
       // norm forward rows beyond the packs whose weights a lane holds: the next
       // pack count that is built (5, 6, 8, 10, 12, 16)
       if (oc == OC_NORM_FWD && p.fast && G == kMaxG && v_exact > kNormFwdHoldMaxV) {
