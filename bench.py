@@ -657,7 +657,8 @@ def model_shapes_table(torch, cabi, L, dev, stream, P, only=None):
     tables, bf16, forward and backward: attention scores of ViT-B/16 (rows of 197), ViT-L/14 at
     336 px (577) and CLIP's text tower (77), which are ragged short rows; GroupNorm over 14 x 14
     and 7 x 7 feature maps, whose channels are not whole packs; log_softmax over a 151936-entry
-    vocabulary (beyond what one workgroup's registers hold).  Algorithmic GB/s as everywhere;
+    vocabulary (19 packs a lane); LayerNorm over a hidden size of 18432 (backward with the dgamma
+    sums in LDS).  Algorithmic GB/s as everywhere;
     `stock_us` = the kernels PyTorch-ROCm ships."""
     BF = cabi.BF16
     bf16 = torch.bfloat16
@@ -733,6 +734,37 @@ def model_shapes_table(torch, cabi, L, dev, stream, P, only=None):
                                                     P(s_[2]), P(dg), P(db), P(ws), nws, Nb, C, HW, G,
                                                     BF, BF, stream)) for s_ in sets],
             lambda: torch.ops.aten.native_group_norm_backward(dy0, x0, m0, r0, w, Nb, C, HW, G,
+                                                              [True, True, True]))
+        del sets, ws, x0, dy0, m0, r0
+        torch.cuda.empty_cache()
+
+    # hidden sizes beyond 16384 (Nemotron-4 340B and PaLM 540B: 18432)
+    for name, M, N in (("native_layer_norm bf16 [8192, 18432] (hidden 18432)", 8192, 18432),):
+        if only is not None and not any(t in name + " fwd" or t in name + " bwd" for t in only.split("|")):
+            continue
+        w = (1 + 0.1 * torch.randn(N, device=dev)).to(bf16)
+        b = (0.1 * torch.randn(N, device=dev)).to(bf16)
+        dg, db = torch.empty_like(w), torch.empty_like(w)
+        sets = []
+        for _ in range(3):
+            x = torch.randn(M, N, device=dev, dtype=bf16)
+            sets.append((x, torch.randn_like(x), torch.empty_like(x),
+                         torch.empty(M, device=dev), torch.empty(M, device=dev)))
+        nws = L.mi355x_layer_norm_bwd_workspace_bytes(M, N, BF, BF, 1, 1)
+        ws = torch.empty(max(nws, 1), dtype=torch.uint8, device=dev)
+        fwd = lambda s_: L.mi355x_layer_norm_fwd(P(s_[0]), P(w), P(b), P(s_[2]), P(s_[3]), P(s_[4]),
+                                                 M, N, 1e-5, BF, BF, stream)
+        for s_ in sets:
+            fwd(s_)
+        x0, dy0, m0, r0 = sets[0][0], sets[0][1], sets[0][3].reshape(M, 1), sets[0][4].reshape(M, 1)
+        nb = M * N * 2
+        add(name + " fwd", 2 * nb, [(lambda s_=s_: fwd(s_)) for s_ in sets],
+            lambda: torch.ops.aten.native_layer_norm(x0, [N], w, b, 1e-5))
+        add(name + " bwd", 3 * nb,
+            [(lambda s_=s_: L.mi355x_layer_norm_bwd(P(s_[1]), P(s_[0]), P(s_[3]), P(s_[4]), P(w),
+                                                    P(s_[2]), P(dg), P(db), P(ws), nws, M, N, BF, BF,
+                                                    stream)) for s_ in sets],
+            lambda: torch.ops.aten.native_layer_norm_backward(dy0, x0, [N], m0, r0, w, b,
                                                               [True, True, True]))
         del sets, ws, x0, dy0, m0, r0
         torch.cuda.empty_cache()

@@ -242,3 +242,30 @@ def test_fused_add_backward_on_long_rows(cabi, oracle, gpu):
         assert_close(dh, odh, torch.bfloat16, "add_layer_norm dh [%d, %d]" % (M, N))
         assert_close(dg, odg, torch.bfloat16, "add_layer_norm dgamma [%d, %d]" % (M, N))
         assert_close(db, odb, torch.bfloat16, "add_layer_norm dbeta [%d, %d]" % (M, N))
+
+
+@pytest.mark.parametrize("dtype", [torch.float16, torch.bfloat16], ids=str)
+@pytest.mark.parametrize("mixed", [False, True], ids=["w_same", "w_fp32"])
+def test_forward_rows_of_5_and_6_packs_on_512_lanes(cabi, oracle, gpu, dtype, mixed):
+    """16-bit forward rows of 16392 .. 24576 elements (hidden 18432, 20480, 24576)."""
+    wdtype = torch.float32 if mixed else dtype
+    code, wcode = cabi.dtype_code(dtype), cabi.dtype_code(wdtype)
+    for i, (V, N) in enumerate(((5, 16392), (5, 18432), (5, 20480), (6, 20488), (6, 24576))):
+        M = 7 + i
+        print("case 512-lane long rows", dtype, mixed, (M, N), flush=True)
+        p = cabi.plan(cabi.OP_LAYER_NORM_FWD, M, N, code, wcode)
+        assert (p["resident"], p["lanes_per_row"], p["packs_per_lane"]) == (1, 512, V), p
+        x, gamma, beta = _mk(M, N, dtype, wdtype, 1520 + i)
+        xg, gg, bg = x.to(gpu), gamma.to(gpu), beta.to(gpu)
+        y, mean, rstd = cabi.layer_norm_fwd(xg, gg, bg, 1e-5)
+        oy, om, orr = oracle.layer_norm_fwd(to_np32(x), (N,), to_np32(gamma), to_np32(beta), 1e-5)
+        what = "[%d, %d] %s" % (M, N, dtype)
+        assert_close(y, oy, dtype, "layer_norm y " + what)
+        assert_close(mean, om.reshape(-1), torch.float32, "mean " + what)
+        assert_close(rstd, orr.reshape(-1), torch.float32, "rstd " + what)
+        ry, rr = cabi.rms_norm_fwd(xg, gg, 1e-6)
+        roy, ror = oracle.rms_norm_fwd(to_np32(x), (N,), to_np32(gamma), 1e-6)
+        assert_close(ry, roy, dtype, "rms_norm y " + what)
+        assert_close(rr, ror.reshape(-1), torch.float32, "rms rstd " + what)
+        y2, _, _ = cabi.layer_norm_fwd(xg, gg, bg, 1e-5)
+        assert torch.equal(y2.view(torch.uint8), y.view(torch.uint8))

@@ -260,6 +260,8 @@ constexpr bool variant_built(OpClass oc, int esize, int G, int V, bool fast) {
     // (640, 768, 1280, 1536 16-bit packs): 3 packs a lane; 5 on 512 lanes for the
     // fp32 LayerNorm forward (see norm_layout())
     if (!is_group_class(oc)) {
+      // (16-bit forward rows of 2049..3072 packs: 5 or 6 packs on 512 lanes, see make_plan())
+      if (oc == OC_NORM_FWD && G == 512 && esize == 2 && (V == 5 || V == 6)) return true;
       if (oc == OC_NORM_FWD && G == kMaxG && V > kNormFwdHoldMaxV)
         return V == 5 || V == 6 || V == 10 || V == 12;
       return G >= 64 && (V == 3 || (V == 5 && oc == OC_NORM_FWD && esize == 4 && G == 512));
@@ -390,6 +392,20 @@ inline int make_plan(OpClass oc, int64_t M, int64_t N, int esize, int num_cus, c
     bool group_exact = false;
     if ((oc == OC_NORM_FWD || oc == OC_NORM_BWD) && p.fast && ov.G == 0 && ov.V == 0)
       group_exact = norm_layout(oc, esize, packs, layer_norm, wide_weights, &G, &V);
+    // 16-bit forward rows of 2049..3072 packs (hidden 18432, 20480, 24576) would take
+    // 1024 lanes x 3 or 4 packs, one workgroup a compute unit whose load, reduce and
+    // store phases run one after the other; two 512-lane workgroups with 5 or 6 packs
+    // a lane and their weights held overlap them.  Interleaved A/B at 8192 rows of
+    // bf16, LayerNorm: N = 18432 121 -> 107 us (fp32 weights 122 -> 113), 20480 129 ->
+    // 116 (133 -> 118), 24576 145 -> 138 (148 -> 136); RMSNorm gains 2-4 % with 5 packs
+    // and nothing with 6; 8 packs (32768) lose to 1024 x 4.  The fused residual add
+    // (a second row in flight) keeps 1024 lanes.
+    if (oc == OC_NORM_FWD && p.fast && esize == 2 && !fused_add && ov.G == 0 && ov.V == 0 &&
+        packs > 2048 && (packs <= 2560 || (layer_norm && packs <= 3072))) {
+      G = 512;
+      V = packs <= 2560 ? 5 : 6;
+      group_exact = true;
+    }
     // Norm rows of at most one wavefront of packs: with one pack a lane, a load
     // instruction of a wavefront covers one contiguous span of 64 packs (several
     // whole rows), while with V packs a lane it covers 64/G separate pieces of
