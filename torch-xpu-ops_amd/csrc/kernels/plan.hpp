@@ -397,11 +397,12 @@ inline int make_plan(OpClass oc, int64_t M, int64_t N, int esize, int num_cus, c
     // store phases run one after the other; two 512-lane workgroups with 5 or 6 packs
     // a lane and their weights held overlap them.  Interleaved A/B at 8192 rows of
     // bf16, LayerNorm: N = 18432 121 -> 107 us (fp32 weights 122 -> 113), 20480 129 ->
-    // 116 (133 -> 118), 24576 145 -> 138 (148 -> 136); RMSNorm gains 2-4 % with 5 packs
-    // and nothing with 6; 8 packs (32768) lose to 1024 x 4.  The fused residual add
-    // (a second row in flight) keeps 1024 lanes.
-    if (oc == OC_NORM_FWD && p.fast && esize == 2 && !fused_add && ov.G == 0 && ov.V == 0 &&
-        packs > 2048 && (packs <= 2560 || (layer_norm && packs <= 3072))) {
+    // 116 (133 -> 118), 24576 145 -> 138 (148 -> 136); 8 packs (32768) lose to 1024 x 4.
+    // The RMSNorm and the fused residual add (a second row in flight) keep 1024 lanes,
+    // with exactly the 3 packs such a row has (below): RMSNorm 18432 98.7 us against
+    // 102.8 on 512 x 5 and 105 on 1024 x 4; add + LayerNorm 217 us against 228 on 1024 x 4.
+    if (oc == OC_NORM_FWD && p.fast && esize == 2 && layer_norm && !fused_add && ov.G == 0 &&
+        ov.V == 0 && packs > 2048 && packs <= 3072) {
       G = 512;
       V = packs <= 2560 ? 5 : 6;
       group_exact = true;
@@ -474,6 +475,10 @@ inline int make_plan(OpClass oc, int64_t M, int64_t N, int esize, int num_cus, c
       // norm backward beyond two packs a lane on 1024 lanes: norm_bwd_sums_in_lds()
       if (oc == OC_NORM_BWD && p.fast && G == kMaxG && v_exact > 2 && esize == 2)
         V = norm_bwd_lds_layout(esize, v_exact, layer_norm) ? (int)v_exact : kMaxV + 1;
+      // three packs a lane at 1024 lanes, not four with a quarter of them outside the row
+      if (oc == OC_NORM_FWD && p.fast && G == kMaxG && v_exact == 3 &&
+          variant_built(oc, esize, G, 3, true))
+        V = 3;
       // norm forward rows beyond the packs whose weights a lane holds: the next
       // pack count that is built (5, 6, 8, 10, 12, 16)
       if (oc == OC_NORM_FWD && p.fast && G == kMaxG && v_exact > kNormFwdHoldMaxV) {
