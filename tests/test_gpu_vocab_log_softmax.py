@@ -24,7 +24,9 @@ def _case(cabi, oracle, gpu, M, N, dtype, off, seed, gi_dtype=None):
     put = (lambda t: offset_view(t.to(gpu), off)) if off else (lambda t: t.to(gpu))
     yg, gg = put(y), put(grad)
     p = cabi.plan(cabi.OP_SOFTMAX_BWD, M, N, cabi.dtype_code(dtype), cabi.dtype_code(dtype))
-    assert p["resident"] == 0
+    # 16-bit rows up to 65536 elements hold both tensors in registers (storage format); beyond
+    # that, and for float32 rows beyond 32768, grad alone stays resident
+    assert p["resident"] == (1 if dtype != torch.float32 and N <= 65536 else 0), p
     gi = cabi.softmax_bwd(gg, yg, True, gi_dtype=gi_dtype)
     try:
         cabi.set_override(cabi.OP_SOFTMAX_BWD, -1, 1)     # the multi-pass kernel
@@ -122,3 +124,48 @@ def test_forward_rows_of_17_to_20_packs_a_lane(cabi, oracle, gpu, dtype, is_log)
                      "half_to_float 151936")
     # one row more than the registers hold: the multi-pass kernel
     assert cabi.plan(cabi.OP_SOFTMAX_FWD, 3, 163848, code, code)["resident"] == 0
+
+
+@pytest.mark.parametrize("dtype", [torch.bfloat16, torch.float16], ids=str)
+@pytest.mark.parametrize("is_log", [False, True], ids=["softmax", "log_softmax"])
+def test_backward_rows_of_5_to_8_packs_a_lane_in_storage_format(cabi, oracle, gpu, dtype, is_log):
+    """16-bit rows of 32776 .. 65536 elements: both tensors in registers, kept packed."""
+    code = cabi.dtype_code(dtype)
+    for i, (V, N) in enumerate(((5, 32776), (5, 40960), (6, 49152), (7, 50304), (7, 57344),
+                                (8, 65528), (8, 65536))):
+        M = 3
+        print("case packed softmax backward", dtype, is_log, (M, N), flush=True)
+        p = cabi.plan(cabi.OP_SOFTMAX_BWD, M, N, code, code)
+        assert (p["resident"], p["lanes_per_row"], p["packs_per_lane"]) == (1, 1024, V), p
+        g = gen(1600 + i)
+        x = 2.0 * torch.randn(M, N, generator=g)
+        x[0, N // 3] = float("-inf")
+        y = (torch.log_softmax(x, -1) if is_log else torch.softmax(x, -1)).to(dtype)
+        grad = torch.randn(M, N, generator=g).to(dtype)
+        yg, gg = y.to(gpu), grad.to(gpu)
+        gi = cabi.softmax_bwd(gg, yg, is_log)
+        ogi = oracle.softmax_bwd(to_np32(grad), to_np32(y), is_log)
+        what = "[%d, %d] %s" % (M, N, dtype)
+        assert_close(gi, ogi, dtype, "backward " + what)
+        try:
+            cabi.set_override(cabi.OP_SOFTMAX_BWD, -1, 1)  # the multi-pass kernel
+            ref = cabi.softmax_bwd(gg, yg, is_log)
+        finally:
+            cabi.clear_overrides()
+        assert_close(gi, to_np32(ref), dtype, "register-resident vs multi-pass backward " + what)
+        assert torch.equal(cabi.softmax_bwd(gg, yg, is_log).view(torch.uint8), gi.view(torch.uint8))
+
+
+def test_masked_backward_beyond_4_packs_a_lane_keeps_the_multi_pass_kernel(cabi, oracle, gpu):
+    """The masked backward widens both tensors to float32 registers; rows of 40960 bf16 elements
+    with a mask take the multi-pass kernel and still agree with the oracle."""
+    M, N = 4, 40960
+    g = gen(1650)
+    x = torch.randn(M, N, generator=g)
+    mask = torch.rand(M, N, generator=g) < 0.3
+    mask[:, 0] = False
+    y = torch.softmax(x.masked_fill(mask, float("-inf")), -1).bfloat16()
+    grad = torch.randn(M, N, generator=g).bfloat16()
+    gi = cabi.masked_softmax_bwd(grad.to(gpu), y.to(gpu), mask.to(gpu))
+    ogi = oracle.masked_softmax_bwd(to_np32(grad), to_np32(y), mask.numpy())
+    assert_close(gi, ogi, torch.bfloat16, "masked softmax backward [4, 40960]")

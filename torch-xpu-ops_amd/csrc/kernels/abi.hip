@@ -372,7 +372,7 @@ int softmax_bwd(const void* grad, const void* y, const void* mask, void* gi, int
   const bool off_line = (((uintptr_t)grad | (uintptr_t)y | (uintptr_t)gi) & 127u) != 0;
   if (int e = make_plan(OC_SOFTMAX_BWD, rows, N, esize_of(gd), current_num_cus(),
                         g_override[ROWNORM_OP_SOFTMAX_BWD], false, &plan, false, false, false,
-                        off_line))
+                        off_line, false, mask != nullptr))
     return e;
   SoftmaxBwdArgs a{grad, y, gi, (const uint8_t*)mask, (uint32_t)mr.div, (uint32_t)mr.mod,
                    mr.stride, rows, (int)N, flags};

@@ -132,7 +132,11 @@ constexpr int v_max(OpClass oc, int esize, int G) {
     // the forward keeps long rows in storage format: 16 packs a lane at any
     // G (a 131072-element 16-bit row, a 65536-element fp32 row)
     case OC_SOFTMAX_FWD: return G >= 1024 ? max_v_of(oc, esize) : 16;
-    case OC_SOFTMAX_BWD: v = esize == 4 ? 16 : 8; break;
+    // (16-bit rows at 1024 lanes: 8 packs of each tensor, kept in storage format)
+    case OC_SOFTMAX_BWD:
+      if (G >= 1024 && esize == 2) return 8;
+      v = esize == 4 ? 16 : 8;
+      break;
     // GroupNorm lanes hold the row (and dY) only, no weights or column sums, so
     // 16-bit rows keep 8 packs a lane at 1024 lanes (128 VGPRs) and 10 at 512
     // lanes (two workgroups a compute unit); the fp32 forward holds 11 at 1024
@@ -364,10 +368,11 @@ inline bool norm_layout(OpClass oc, int esize, int64_t packs, bool layer_norm, b
 // wide_weights: fp32 gamma/beta beside 16-bit rows.
 // off_line: a tensor of the call does not start on a 128-byte cache line.
 // fused_add: the norm forward adds a residual row first (two rows in flight a lane).
+// masked: the softmax backward reads a mask (its 16-bit rows then stop at 4 packs a lane).
 inline int make_plan(OpClass oc, int64_t M, int64_t N, int esize, int num_cus, const Override& ov,
                      bool want_cols, Plan* out, bool force_general = false,
                      bool layer_norm = false, bool wide_weights = false, bool off_line = false,
-                     bool fused_add = false) {
+                     bool fused_add = false, bool masked = false) {
   Plan p;
   const int E = 16 / esize;
   p.fast = (N % E) == 0 && !force_general;
@@ -475,6 +480,8 @@ inline int make_plan(OpClass oc, int64_t M, int64_t N, int esize, int num_cus, c
       // norm backward beyond two packs a lane on 1024 lanes: norm_bwd_sums_in_lds()
       if (oc == OC_NORM_BWD && p.fast && G == kMaxG && v_exact > 2 && esize == 2)
         V = norm_bwd_lds_layout(esize, v_exact, layer_norm) ? (int)v_exact : kMaxV + 1;
+      // the masked softmax backward keeps fp32 copies of both tensors: 4 packs at most
+      if (oc == OC_SOFTMAX_BWD && masked && esize == 2 && G == kMaxG && V > 4) V = kMaxV + 1;
       // three packs a lane at 1024 lanes, not four with a quarter of them outside the row
       if (oc == OC_NORM_FWD && p.fast && G == kMaxG && v_exact == 3 &&
           variant_built(oc, esize, G, 3, true))

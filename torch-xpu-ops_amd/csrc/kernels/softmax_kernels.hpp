@@ -486,11 +486,15 @@ softmax_bwd_resident_kernel(const TG* __restrict__ grad, const TG* __restrict__ 
   const bool is_log = (flags & kSoftmaxLog) != 0;
   // y's packs are aligned like grad's when the two base addresses are congruent
   const bool y_whole = WINDOW && same_pack_alignment(grad, y);
+  // 16-bit rows of more than 4 packs a lane on 1024 lanes: both tensors stay in storage
+  // format across the reduction and are widened again for the output (as fp32 copies
+  // they would take 16 registers a pack)
+  constexpr bool kPacked = FAST && !MASKED && G == 1024 && V > 4 && sizeof(TG) == 2;
   const int64_t nrb = (M + RPB - 1) / RPB;
   for (int64_t rb = blockIdx.x; rb < nrb; rb += gridDim.x) {
     // ragged rows: opaque once a row and again before the stores (see the forward;
     // 8192 x 4097 bf16 49.6 -> 41.8 us); whole-pack rows measured 1 % slower with it
-    const int lane = lane_again<!FAST>(lane0);
+    const int lane = lane_again<!FAST || kPacked>(lane0);
     const int64_t row = rb * RPB + slot;
     const bool ok = RPB == 1 ? true : row < M;
     const int64_t rowc = ok ? row : 0;
@@ -512,6 +516,38 @@ softmax_bwd_resident_kernel(const TG* __restrict__ grad, const TG* __restrict__ 
       const int e0 = (c * G + lane) * E;
       row_trim<TG, E, FAST, true>(pg[c], e0, nw, 0.0f, h, WINDOW);
       row_trim<TG, E, FAST, true>(py[c], e0, nw, 0.0f, h, y_whole);
+    }
+    if constexpr (kPacked) {
+      float sum[1] = {0.0f};
+      if (is_log) {
+        ROWNORM_UNIFORM_ARM("log_softmax backward: sum of grad");
+#pragma unroll
+        for (int c = 0; c < V; ++c)
+#pragma unroll
+          for (int i = 0; i < E; ++i) sum[0] += pg[c].get(i);
+      } else {
+        ROWNORM_UNIFORM_ARM("softmax backward: sum of y * grad");
+#pragma unroll
+        for (int c = 0; c < V; ++c)
+#pragma unroll
+          for (int i = 0; i < E; ++i) sum[0] = fmaf(py[c].get(i), pg[c].get(i), sum[0]);
+      }
+      group_allreduce<G, BLOCK, 1, SumOp>(sum, red, phase);
+      float s = sum[0];
+      const int ls = lane_after<true>(lane0, s);
+#pragma unroll
+      for (int c = 0; c < V; ++c) {
+        keep_packed(pg[c]);
+        keep_packed(py[c]);
+        Pack<TO, E> o;
+#pragma unroll
+        for (int i = 0; i < E; ++i) {
+          const float gv = pg[c].get(i), yv = py[c].get(i);
+          o.set(i, is_log ? gv - row_exp<PRECISE>(yv) * s : yv * (gv - s));
+        }
+        row_store<TO, E, true, FAST>(outr, (c * G + ls) * E, nw, ok, o, h);
+      }
+      continue;
     }
     float gf[V][E], yf[V][E];
 #pragma unroll
