@@ -192,11 +192,12 @@ int mi355x_add_rms_norm_bwd(const void* dy, const void* dh_in, const void* h, co
  * hipMalloc.  It has no counterpart in the reference, whose entry point
  * allocates its scratch itself (LayerNormKernels.cpp:1255-1264).  Same
  * arguments and results as mi355x_rms_norm_bwd (bit for bit, given the full
- * workspace) minus the workspace: the fp32 partial rows live in a 16 MiB array
+ * workspace) minus the workspace: the fp32 partial rows live in a 32 MiB array
  * inside the library's device image, one copy per GPU, held until the process
  * ends.  A call that would need more (mi355x_rms_norm_bwd_workspace_bytes()
- * above mi355x_rms_norm_bwd_static_limit_bytes(): on 256 compute units that is
- * N > 8192 with 512-lane layouts) fails with ROWNORM_ERR_SCRATCH_LIMIT and
+ * above mi355x_rms_norm_bwd_static_limit_bytes(): on 256 compute units no launch
+ * plan of the library itself, only a forced larger grid) fails with
+ * ROWNORM_ERR_SCRATCH_LIMIT and
  * launches nothing.  Calls no hipMalloc / hipFree and no allocating library
  * routine.  Every call on one GPU shares that GPU's array: calls that overlap
  * in time on one GPU (two streams, two threads) race; calls on one stream are

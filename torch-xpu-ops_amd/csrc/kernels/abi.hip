@@ -142,7 +142,7 @@ const OverrideTable g_override;
 // the array, at its own address, until the process ends.  The name below is a
 // host-side stand-in only; host code uses the per-device address that
 // hipGetSymbolAddress reports (static_scratch()).
-constexpr size_t kStaticScratchBytes = size_t(16) << 20;
+constexpr size_t kStaticScratchBytes = size_t(32) << 20;
 static __device__ __align__(256) __attribute__((used)) unsigned char scratch[kStaticScratchBytes];
 std::atomic<void*> g_scratch_ptr[kMaxDevices];
 
@@ -442,7 +442,7 @@ const char* mi355x_rownorm_error_string(int code) {
     case ROWNORM_ERR_WORKSPACE: return "mi355x_rownorm: workspace missing or too small";
     case ROWNORM_ERR_OVERRIDE: return "mi355x_rownorm: forced variant cannot run this shape";
     case ROWNORM_ERR_SCRATCH_LIMIT:
-      return "mi355x_rownorm: the call needs more scratch than the library's static 16 MiB";
+      return "mi355x_rownorm: the call needs more scratch than the library's static 32 MiB";
   }
   if (code > 0) return hipGetErrorString((hipError_t)code);
   return "mi355x_rownorm: unknown error code";
