@@ -225,10 +225,12 @@ def test_plan_layouts_for_hidden_sizes_that_are_not_powers_of_two(cabi):
     assert lay(LF, 16384, BF) == (512, 4) and lay(LB, 16384, BF) == (512, 4)
     assert lay(RF, 16384, BF) == (512, 4) and lay(RB, 16384, BF) == (1024, 2)
     assert lay(LF, 32768, BF) == (1024, 4)
-    # ragged 16-bit norm rows just above a power of two: three packs on half the lanes
-    assert lay(LF, 4097, BF) == (256, 3) and lay(LB, 4097, BF) == (256, 3)
+    # ragged 16-bit norm rows just above a power of two: three packs on half the lanes, except
+    # in the LayerNorm backward (its three-pack kernels are over the registers of two workgroups)
+    assert lay(LF, 4097, BF) == (256, 3) and lay(LB, 4097, BF) == (512, 2)
     assert lay(RB, 4097, BF) == (256, 3) and lay(RB, 2049, BF) == (128, 3)
-    assert lay(LB, 8193, BF) == (512, 3) and lay(RB, 8193, BF) == (1024, 2)
+    assert lay(LB, 2049, BF) == (256, 2) and lay(LB, 1025, BF) == (128, 2)
+    assert lay(LB, 8193, BF) == (1024, 2) and lay(RB, 8193, BF) == (512, 3)
     # fp32 rows
     assert lay(LF, 5120, F32) == (512, 3) and lay(LB, 5120, F32) == (512, 3)
     assert lay(LF, 10240, F32) == (512, 5) and lay(RF, 10240, F32) == (1024, 3)
@@ -237,9 +239,9 @@ def test_plan_layouts_for_hidden_sizes_that_are_not_powers_of_two(cabi):
     assert lay(cabi.OP_SOFTMAX_FWD, 4097, cabi.F16) == (256, 3)
     assert lay(cabi.OP_SOFTMAX_BWD, 4097, cabi.F16) == (256, 3)
     assert lay(cabi.OP_SOFTMAX_FWD, 4097, F32) == (512, 4)
-    # ragged 16-bit norm rows: three packs in both directions
+    # ragged 16-bit norm rows: three packs in the forward and the RMSNorm backward
     assert lay(LF, 4097, cabi.F16) == (256, 3) and lay(RF, 4097, BF) == (256, 3)
-    assert lay(LB, 4097, cabi.F16) == (256, 3)
+    assert lay(RB, 4097, cabi.F16) == (256, 3) and lay(LB, 4097, cabi.F16) == (512, 2)
 
 
 def test_group_norm_rows_take_512_lanes_while_two_workgroups_fit(cabi):

@@ -781,7 +781,7 @@ norm_bwd_resident_kernel(const T* __restrict__ dy, const T* __restrict__ x, cons
   auto fetch = [&](int64_t rb, bool (&fok)[R], float (&fmu)[R], float (&frs)[R],
                    Pack<T, E> (&fx)[R][V], Pack<T, E> (&fd)[R][V]) {
     const int64_t frow0 = (rb * RPB + slot) * R;
-    const int lane = lane_again<LDSG>(lane0);
+    const int lane = lane_again<LDSG || !FAST>(lane0);
     // (past the last row block the requests go to row 0 and are never used: a
     // branch around them measured 10-15 % slower over the whole kernel)
 #pragma unroll
@@ -811,7 +811,7 @@ norm_bwd_resident_kernel(const T* __restrict__ dy, const T* __restrict__ x, cons
     else
       fetch(rb, ok, mu, rs, xp, dp);
     float acc[2 * R];
-    const int lane = lane_again<LDSG>(lane0);
+    const int lane = lane_again<LDSG || !FAST>(lane0);
 #pragma unroll
     for (int r = 0; r < R; ++r) {
       // 16-bit rows: xhat = x*rs - mu*rs in one FMA (rounding far below a 16-bit
@@ -856,7 +856,7 @@ norm_bwd_resident_kernel(const T* __restrict__ dy, const T* __restrict__ x, cons
     }
     group_allreduce<G, BLOCK, 2 * R, SumOp>(acc, red, phase);
     if (dx != nullptr) {
-      const int ls = lane_after<LDSG>(lane0, acc[1]);
+      const int ls = lane_after<LDSG || !FAST>(lane0, acc[1]);
 #pragma unroll
       for (int r = 0; r < R; ++r) {
         T* dr = dx + (row0 + r) * (int64_t)N;

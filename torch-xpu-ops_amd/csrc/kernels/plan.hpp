@@ -438,11 +438,12 @@ inline int make_plan(OpClass oc, int64_t M, int64_t N, int esize, int num_cus, c
     // 16-bit softmax rows in both directions and ragged 16-bit norm rows:
     // a row that fills at most three quarters of the two-pack slots takes three
     // packs on half the lanes (softmax N = 5120: 62 -> 56 us, 10240: 120 -> 110 us
-    // at 16384 rows; at 8192 rows LayerNorm N = 4097: forward 60 -> 52 us, backward
-    // 89 -> 77 us, RMSNorm backward 84 -> 69 us; the RMSNorm backward from 1024
-    // lanes is the exception, N = 8193: 116 us against 123 us)
-    const bool ragged_norm = !p.fast && (oc == OC_NORM_FWD ||
-                                         (oc == OC_NORM_BWD && (layer_norm || G < kMaxG)));
+    // at 16384 rows; at 8192 rows LayerNorm forward N = 4097: 60 -> 52 us; RMSNorm
+    // backward 4097: 62 -> 55 us, 8193: 115 -> 97 us).  The ragged LayerNorm backward
+    // is the exception: its three-pack kernels take 155 registers (one workgroup a
+    // compute unit) where two packs on all the lanes keep two (N = 1025: 60 -> 40 us,
+    // 2049: 80 -> 65 us at 16384 rows; 4097: 79 -> 66 us, 5121: 86 -> 76 us at 8192).
+    const bool ragged_norm = !p.fast && (oc == OC_NORM_FWD || (oc == OC_NORM_BWD && !layer_norm));
     if (((softmax && (oc == OC_SOFTMAX_FWD || !p.fast)) || ragged_norm) &&
         esize == 2 && ov.G == 0 && ov.V == 0 &&
         G >= 128 && packs <= (int64_t)G * 2 && packs * 4 <= (int64_t)G * 2 * 3 &&
