@@ -1,8 +1,9 @@
 """log_softmax backward on vocabulary-sized rows (the cross_entropy case): rows too long for both
 tensors in registers keep grad resident and stream y past it (log_softmax_bwd_grad_resident_kernel;
 the reference walks the row twice in LogSoftmaxBackward, src/ATen/native/xpu/sycl/
-SoftMaxKernels.cpp:991-1150).  Every packs-per-lane count of the kernel (5..20 for 16-bit rows,
-9..20 for float32 rows), with the row end inside and at the end of a lane's last pack, misaligned
+SoftMaxKernels.cpp:991-1150).  Every packs-per-lane count of the kernel (9..20; 16-bit rows of
+5..8 packs a lane hold both tensors in registers), with the row end inside and at the end of a
+lane's last pack, misaligned
 tensors and -inf / NaN entries, against the CPU oracle at the family's tolerances (float32
 rtol = atol = 1e-5; 16-bit atol 1e-2, rtol 1.6e-2) and against the multi-pass kernel forced on
 the same inputs.  The 16-bit forward holds rows of 17..20 packs a lane (the 151936 / 152064-entry

@@ -204,7 +204,8 @@ struct SoftmaxBwdLauncher {
 };
 
 // log_softmax backward of rows too long for both tensors in registers but not for
-// grad alone: whole packs, at most 1024 lanes x 20 packs.  False: not this case.
+// grad alone: whole packs, 9 to 20 a lane on 1024 lanes (up to 8 both tensors fit:
+// softmax_bwd_resident_kernel).  False: not this case.
 template <class TG, class TO, int V>
 inline void launch_grad_resident_v(const Plan& plan, const SoftmaxBwdArgs& a, hipStream_t stream) {
   hipLaunchKernelGGL((log_softmax_bwd_grad_resident_kernel<TG, TO, V, kStreamBlock>),
@@ -219,12 +220,6 @@ inline bool launch_log_softmax_bwd_grad_resident(const Plan& plan, const Softmax
   if (!plan.grad_resident || !(a.flags & kSoftmaxLog) || a.N % E != 0) return false;
   const int64_t packs = a.N / E;
   switch ((int)((packs + kStreamBlock - 1) / kStreamBlock)) {
-    case 3: launch_grad_resident_v<TG, TO, 3>(plan, a, stream); return true;
-    case 4: launch_grad_resident_v<TG, TO, 4>(plan, a, stream); return true;
-    case 5: launch_grad_resident_v<TG, TO, 5>(plan, a, stream); return true;
-    case 6: launch_grad_resident_v<TG, TO, 6>(plan, a, stream); return true;
-    case 7: launch_grad_resident_v<TG, TO, 7>(plan, a, stream); return true;
-    case 8: launch_grad_resident_v<TG, TO, 8>(plan, a, stream); return true;
     case 9: launch_grad_resident_v<TG, TO, 9>(plan, a, stream); return true;
     case 10: launch_grad_resident_v<TG, TO, 10>(plan, a, stream); return true;
     case 11: launch_grad_resident_v<TG, TO, 11>(plan, a, stream); return true;
