@@ -341,7 +341,11 @@ int mi355x_softmax_strided_plan(int backward, int64_t outer, int64_t dim_size, i
  * of packs) of at most 2048 16-bit / 1024 float32 elements, and on rows of up to
  * 12 whole packs that fit the reported layout badly, with 16-byte aligned
  * tensors and one dtype, run through LDS-staged kernels instead of the layout
- * reported here (a forced layout keeps the reported kernels). */
+ * reported here (a forced layout keeps the reported kernels).  The query
+ * describes the plain call: the fused residual add keeps 1024 lanes for 16-bit
+ * rows of 16392..24576 elements and takes the multi-pass kernel beyond 12 packs a
+ * lane (float32 LayerNorm: 10), and the masked softmax backward beyond 4 packs a
+ * lane of 16-bit rows. */
 int mi355x_rownorm_plan(rownorm_op op, int64_t M, int64_t N, rownorm_dtype x_dtype,
                         rownorm_dtype w_dtype, rownorm_plan* out);
 
