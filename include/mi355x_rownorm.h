@@ -344,8 +344,9 @@ int mi355x_softmax_strided_plan(int backward, int64_t outer, int64_t dim_size, i
  * reported here (a forced layout keeps the reported kernels).  The query
  * describes the plain call: the fused residual add keeps 1024 lanes for 16-bit
  * rows of 16392..24576 elements and takes the multi-pass kernel beyond 12 packs a
- * lane (float32 LayerNorm: 10), and the masked softmax backward beyond 4 packs a
- * lane of 16-bit rows. */
+ * lane (float32 LayerNorm: 10), and the masked softmax calls beyond 32 elements a
+ * lane on 1024 lanes (rows of more than 32768 elements; a forced layout beyond
+ * that is ROWNORM_ERR_OVERRIDE for a masked call). */
 int mi355x_rownorm_plan(rownorm_op op, int64_t M, int64_t N, rownorm_dtype x_dtype,
                         rownorm_dtype w_dtype, rownorm_plan* out);
 

@@ -348,7 +348,7 @@ int softmax_fwd(const void* x, const void* mask, void* y, int64_t rows, int64_t 
   const bool off_line = (((uintptr_t)x | (uintptr_t)y) & 127u) != 0;
   if (int e = make_plan(OC_SOFTMAX_FWD, rows, N, esize_of(id), current_num_cus(),
                         g_override[ROWNORM_OP_SOFTMAX_FWD], false, &plan, false, false, false,
-                        off_line))
+                        off_line, false, mask != nullptr))
     return e;
   SoftmaxFwdArgs a{x,    y, (const uint8_t*)mask, (uint32_t)mr.div, (uint32_t)mr.mod, mr.stride,
                    rows, (int)N, flags};

@@ -244,6 +244,14 @@ constexpr int gn_mode(int64_t L, int64_t HxW, int64_t D, int E) {
 // backward 66 -> 59 us (96).  Eight packs backward spill and gain nothing.
 constexpr int group_half_lanes_max_v(OpClass oc) { return oc == OC_GROUP_FWD ? 10 : 7; }
 
+// Masked softmax rows are attention scores: the masked kernels exist up to 32
+// elements a lane at 1024 lanes (rows of 32768 elements; the masked 16-bit
+// backward, which keeps fp32 copies of both tensors, would spill beyond that
+// anyway), and longer masked rows take the multi-pass kernels.
+constexpr bool masked_softmax_built(int esize, int G, int V) {
+  return !(G == 1024 && V * (16 / esize) > 32);
+}
+
 constexpr bool variant_built(OpClass oc, int esize, int G, int V, bool fast) {
   if (G < kMinG || G > kMaxG || (G & (G - 1)) || V < 1 || V > max_v_of(oc, esize)) return false;
   // GroupNorm rows take the packs they have, not the next power of two (a
@@ -368,7 +376,7 @@ inline bool norm_layout(OpClass oc, int esize, int64_t packs, bool layer_norm, b
 // wide_weights: fp32 gamma/beta beside 16-bit rows.
 // off_line: a tensor of the call does not start on a 128-byte cache line.
 // fused_add: the norm forward adds a residual row first (two rows in flight a lane).
-// masked: the softmax backward reads a mask (its 16-bit rows then stop at 4 packs a lane).
+// masked: the softmax call reads a mask (see masked_softmax_built()).
 inline int make_plan(OpClass oc, int64_t M, int64_t N, int esize, int num_cus, const Override& ov,
                      bool want_cols, Plan* out, bool force_general = false,
                      bool layer_norm = false, bool wide_weights = false, bool off_line = false,
@@ -481,8 +489,6 @@ inline int make_plan(OpClass oc, int64_t M, int64_t N, int esize, int num_cus, c
       // norm backward beyond two packs a lane on 1024 lanes: norm_bwd_sums_in_lds()
       if (oc == OC_NORM_BWD && p.fast && G == kMaxG && v_exact > 2 && esize == 2)
         V = norm_bwd_lds_layout(esize, v_exact, layer_norm) ? (int)v_exact : kMaxV + 1;
-      // the masked softmax backward keeps fp32 copies of both tensors: 4 packs at most
-      if (oc == OC_SOFTMAX_BWD && masked && esize == 2 && G == kMaxG && V > 4) V = kMaxV + 1;
       // three packs a lane at 1024 lanes, not four with a quarter of them outside the row
       if (oc == OC_NORM_FWD && p.fast && G == kMaxG && v_exact == 3 &&
           variant_built(oc, esize, G, 3, true))
@@ -501,9 +507,12 @@ inline int make_plan(OpClass oc, int64_t M, int64_t N, int esize, int num_cus, c
       }
       if (!p.fast && V < v_pref(oc, esize)) V = v_pref(oc, esize);
     }
+    // masked rows beyond 32 elements a lane at 1024 lanes: the multi-pass kernels
+    if (softmax && masked && ov.V == 0 && !masked_softmax_built(esize, G, V)) V = kMaxV + 1;
     const bool holds = (int64_t)G * V >= packs;
     const int block = ov.block > 0 ? ov.block : block_threads(oc, G);
-    const bool built = variant_built(oc, esize, G, V, p.fast) && block_built(oc, G, block);
+    const bool built = variant_built(oc, esize, G, V, p.fast) && block_built(oc, G, block) &&
+                       !(softmax && masked && !masked_softmax_built(esize, G, V));
     if (ov.G > 0 || ov.V > 0 || ov.block > 0) {
       if (!holds || !built) return -5;
     }

@@ -18,7 +18,8 @@ struct SoftmaxFwdLauncher {
   struct At {
     static bool run(const SoftmaxFwdCtx<TI, TO>& c) {
       if constexpr (variant_built(OC_SOFTMAX_FWD, sizeof(TI), G, V, FAST) &&
-                    block_built(OC_SOFTMAX_FWD, G, BLOCK)) {
+                    block_built(OC_SOFTMAX_FWD, G, BLOCK) &&
+                    (!MASKED || masked_softmax_built(sizeof(TI), G, V))) {
         if (c.plan.G == G && c.plan.V == V && c.plan.block == BLOCK) {
           hipLaunchKernelGGL((softmax_fwd_resident_kernel<TI, TO, G, V, BLOCK, FAST, MASKED>),
                              dim3((unsigned)c.plan.grid), dim3(BLOCK), 0, c.stream,
@@ -188,7 +189,8 @@ struct SoftmaxBwdLauncher {
   struct At {
     static bool run(const SoftmaxBwdCtx<TG, TO>& c) {
       if constexpr (variant_built(OC_SOFTMAX_BWD, sizeof(TG), G, V, FAST) &&
-                    block_built(OC_SOFTMAX_BWD, G, BLOCK)) {
+                    block_built(OC_SOFTMAX_BWD, G, BLOCK) &&
+                    (!MASKED || masked_softmax_built(sizeof(TG), G, V))) {
         if (c.plan.G == G && c.plan.V == V && c.plan.block == BLOCK) {
           hipLaunchKernelGGL((softmax_bwd_resident_kernel<TG, TO, G, V, BLOCK, FAST, MASKED>),
                              dim3((unsigned)c.plan.grid), dim3(BLOCK), 0, c.stream,
