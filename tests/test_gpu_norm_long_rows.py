@@ -211,7 +211,10 @@ def test_backward_with_dgamma_sums_in_lds(cabi, oracle, gpu, dtype, mixed):
         for M in ((1, 37, 300) if i in (1, 6) else (5 + i,)):
             print("case long rows backward", dtype, mixed, (M, N), flush=True)
             p = cabi.plan(cabi.OP_RMS_NORM_BWD, M, N, code, wcode)
-            assert (p["resident"], p["lanes_per_row"], p["packs_per_lane"]) == (1, 1024, V), p
+            # (the RMSNorm with 16-bit weights holds rows of up to 2560 packs in registers alone,
+            # on 512 lanes x 5 packs)
+            want = (1, 512, 5) if (N <= 20480 and not mixed) else (1, 1024, V)
+            assert (p["resident"], p["lanes_per_row"], p["packs_per_lane"]) == want, p
             p = cabi.plan(cabi.OP_LAYER_NORM_BWD, M, N, code, wcode)
             # the LayerNorm backward with four packs a lane keeps the multi-pass kernels
             assert p["resident"] == (1 if V == 3 else 0), p

@@ -280,7 +280,8 @@ int norm_bwd(const void* dy, const void* x, const float* mean, const float* rstd
   Plan plan;
   const int op = RMS ? ROWNORM_OP_RMS_NORM_BWD : ROWNORM_OP_LAYER_NORM_BWD;
   if (int e = make_plan(OC_NORM_BWD, M, N, esize_of(xd), current_num_cus(), g_override[op],
-                        want_cols, &plan, false, !RMS, esize_of(wd) > esize_of(xd)))
+                        want_cols, &plan, false, !RMS, esize_of(wd) > esize_of(xd), false,
+                        dres != nullptr))
     return e;
   float* part_dg = nullptr;
   float* part_db = nullptr;

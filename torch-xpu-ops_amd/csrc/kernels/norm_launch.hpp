@@ -91,7 +91,8 @@ struct NormBwdLauncher {
   struct At {
     static bool run(const NormBwdCtx<T, WT, RMS>& c) {
       if constexpr (variant_built(OC_NORM_BWD, sizeof(T), G, V, FAST) &&
-                    block_built(OC_NORM_BWD, G, BLOCK)) {
+                    block_built(OC_NORM_BWD, G, BLOCK) &&
+                    (!FAST || norm_bwd_instance_ok(sizeof(T), sizeof(WT), G, V, RMS, ADD))) {
         if (c.plan.G == G && c.plan.V == V && c.plan.block == BLOCK) {
           hipLaunchKernelGGL((norm_bwd_resident_kernel<T, WT, G, V, BLOCK, 1, RMS, FAST, ADD>),
                              dim3((unsigned)c.plan.grid), dim3(BLOCK), 0, c.stream,

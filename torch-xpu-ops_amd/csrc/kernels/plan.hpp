@@ -127,6 +127,7 @@ constexpr int v_max(OpClass oc, int esize, int G) {
     // norm_bwd_sums_in_lds())
     case OC_NORM_BWD:
       if (G >= 1024 && esize == 2) return 4;
+      if (G == 512 && esize == 2) return 5;  // (5: norm_bwd_half_lanes_five())
       v = esize == 4 ? 8 : 4;
       break;
     // the forward keeps long rows in storage format: 16 packs a lane at any
@@ -188,6 +189,19 @@ constexpr bool norm_bwd_prefetches(int esize, int G, int V, bool fast, bool rms)
 // spills 29-45 registers and loses (237 -> 302 us): it keeps the multi-pass kernels.
 constexpr bool norm_bwd_sums_in_lds(int esize, int G, int V, bool fast) {
   return fast && esize == 2 && G == 1024 && V >= 3;
+}
+// One case goes through the registers instead: the RMSNorm with 16-bit weights and
+// rows of 2049..2560 packs (hidden 18432, 20480) fits 512 lanes x 5 packs with its
+// next row on the way in 251 registers, one 512-thread workgroup a compute unit
+// (bf16 [16384, 18432] 345 -> 315 us, 72 %; [8192, 20480] 194 -> 176 us).  The
+// LayerNorm, fp32 weights and the fused residual gradient spill there (LayerNorm
+// 199 -> 351 us) and stay with the LDS sums; so do 6 packs (24576).
+constexpr bool norm_bwd_half_lanes_five(int esize, int wsize, int G, int V, bool rms, bool add) {
+  return esize == 2 && wsize == 2 && G == 512 && V == 5 && rms && !add;
+}
+// (a 512 x 5 instance exists for that case only)
+constexpr bool norm_bwd_instance_ok(int esize, int wsize, int G, int V, bool rms, bool add) {
+  return !(esize == 2 && G == 512 && V == 5) || norm_bwd_half_lanes_five(esize, wsize, G, V, rms, add);
 }
 constexpr bool norm_bwd_lds_layout(int esize, int64_t v_exact, bool layer_norm) {
   return esize == 2 && (v_exact == 3 || (v_exact == 4 && !layer_norm));
@@ -272,6 +286,7 @@ constexpr bool variant_built(OpClass oc, int esize, int G, int V, bool fast) {
     // (640, 768, 1280, 1536 16-bit packs): 3 packs a lane; 5 on 512 lanes for the
     // fp32 LayerNorm forward (see norm_layout())
     if (!is_group_class(oc)) {
+      if (oc == OC_NORM_BWD && G == 512 && esize == 2 && V == 5) return true;
       // (16-bit forward rows of 2049..3072 packs: 5 or 6 packs on 512 lanes, see make_plan())
       if (oc == OC_NORM_FWD && G == 512 && esize == 2 && (V == 5 || V == 6)) return true;
       if (oc == OC_NORM_FWD && G == kMaxG && V > kNormFwdHoldMaxV)
@@ -375,7 +390,8 @@ inline bool norm_layout(OpClass oc, int esize, int64_t packs, bool layer_norm, b
 // layer_norm: the norm op is LayerNorm (statistics of two sums, beta), not RMSNorm.
 // wide_weights: fp32 gamma/beta beside 16-bit rows.
 // off_line: a tensor of the call does not start on a 128-byte cache line.
-// fused_add: the norm forward adds a residual row first (two rows in flight a lane).
+// fused_add: the norm forward adds a residual row first (two rows in flight a lane);
+// the norm backward adds the residual path's gradient to dX.
 // masked: the softmax call reads a mask (see masked_softmax_built()).
 inline int make_plan(OpClass oc, int64_t M, int64_t N, int esize, int num_cus, const Override& ov,
                      bool want_cols, Plan* out, bool force_general = false,
@@ -418,6 +434,12 @@ inline int make_plan(OpClass oc, int64_t M, int64_t N, int esize, int num_cus, c
         ov.V == 0 && packs > 2048 && packs <= 3072) {
       G = 512;
       V = packs <= 2560 ? 5 : 6;
+      group_exact = true;
+    }
+    if (oc == OC_NORM_BWD && p.fast && ov.G == 0 && ov.V == 0 && packs > 2048 && packs <= 2560 &&
+        norm_bwd_half_lanes_five(esize, wide_weights ? 4 : esize, 512, 5, !layer_norm, fused_add)) {
+      G = 512;
+      V = 5;
       group_exact = true;
     }
     // Norm rows of at most one wavefront of packs: with one pack a lane, a load
@@ -512,7 +534,10 @@ inline int make_plan(OpClass oc, int64_t M, int64_t N, int esize, int num_cus, c
     const bool holds = (int64_t)G * V >= packs;
     const int block = ov.block > 0 ? ov.block : block_threads(oc, G);
     const bool built = variant_built(oc, esize, G, V, p.fast) && block_built(oc, G, block) &&
-                       !(softmax && masked && !masked_softmax_built(esize, G, V));
+                       !(softmax && masked && !masked_softmax_built(esize, G, V)) &&
+                       !(oc == OC_NORM_BWD && p.fast &&
+                         !norm_bwd_instance_ok(esize, wide_weights ? 4 : esize, G, V, !layer_norm,
+                                               fused_add));
     if (ov.G > 0 || ov.V > 0 || ov.block > 0) {
       if (!holds || !built) return -5;
     }
