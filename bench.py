@@ -12,7 +12,7 @@ Cache so that every step streams from HBM.
     python bench.py [--gpus 1] [--steps K] [--warmup W] [--no-ops] [--no-cpu]
 
 prints ONE JSON line (see the keys below).  `roofline` covers the dominant operation of the step,
-one mi355x_rms_norm_bwd call (norm_bwd_resident_kernel + colsum_finalize_kernel), timed with a
+one mi355x_rms_norm_bwd call (norm_bwd_exact_kernel + colsum_finalize_kernel), timed with a
 one HIP event pair on the launch stream around K back-to-back calls.  `cpu_baseline` is the scalar C oracle
 (oracle/, a port of the same arithmetic) timed on one host core; `cpu_aten` is PyTorch's CPU ATen
 path (the parity target) on all host cores.  `stock_pytorch_rocm` is the same step through the
@@ -151,7 +151,7 @@ def main():
     # the launch stream between ONE HIP event pair, rotating over the same buffer sets (an event
     # record between two launches costs the GPU a few microseconds of idle time, which would be
     # charged to the kernel; back to back, the average equals the kernel durations rocprofv3
-    # reports for norm_bwd_resident_kernel + colsum_finalize_kernel)
+    # reports for norm_bwd_exact_kernel + colsum_finalize_kernel)
     for i in range(min(args.warmup, 10)):
         bwd(sets[i % nsets])
     e0, e1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
@@ -183,7 +183,7 @@ def main():
                    "buffer_sets_rotated": nsets},
         "roofline": {
             "bound": "hbm",
-            "kernel": "mi355x_rms_norm_bwd = norm_bwd_resident_kernel + colsum_finalize_kernel",
+                "kernel": "mi355x_rms_norm_bwd = norm_bwd_exact_kernel + colsum_finalize_kernel",
             "achieved": round(achieved, 1),
             "peak": HBM_PEAK_GBS,
             "unit": "GB/s",
@@ -209,13 +209,16 @@ def main():
         out["stock_pytorch_rocm"] = stock_step(torch, sets, w, M, N, eps, fwd_bytes + bwd_bytes)
         out["device_copy"] = device_copy_table(torch, dev, M, N)
         out["ops"] = per_op_table(torch, cabi, L, dev, stream, P)
+        out["norm_width_sweep"] = width_sweep_table(torch, cabi, L, dev, stream, P)
         # the target of this operator family is one number: every op at its Llama-class bf16
-        # configuration (2, 3 and 4) at or above 70 % of the HBM peak
+        # shapes at or above 70 % of the HBM peak -- the rows of configurations 2, 3 and 4 and
+        # every row of the hidden-size sweep from 4096 to 8192
         llama = [r for r in out["ops"] if r["op"].startswith(("C2 ", "C3 ", "C4 "))]
+        llama += [r for r in out["norm_width_sweep"]["rows"]
+                  if 4096 <= int(r["op"].rsplit(",", 1)[1].rstrip("]")) <= 8192]
         worst = min(llama, key=lambda r: r["frac"])
         out["min_frac_llama_ops"] = {"frac": worst["frac"], "op": worst["op"], "target": 0.70,
                                      "ops_counted": len(llama)}
-        out["norm_width_sweep"] = width_sweep_table(torch, cabi, L, dev, stream, P)
         out["reference_microbench"] = reference_microbench_table(torch, cabi, L, dev, stream, P)
         out["model_shapes"] = model_shapes_table(torch, cabi, L, dev, stream, P)
         out["config5"] = stress_table(torch, cabi, L, dev, stream, P)
@@ -226,12 +229,19 @@ def main():
 
 
 def calibrate_copy(torch, dev):
-    """A plain 256 MiB device copy, 10 times: the kernel of known size that FETCH_SIZE /
-    WRITE_SIZE readings are scaled by."""
+    """A plain 256 MiB device copy, 10 times (torch's copy_, then the library's own
+    stream_probe_kernel): the kernels of known size that FETCH_SIZE / WRITE_SIZE readings are
+    scaled by."""
+    import ctypes
     src = torch.empty(256 << 20, dtype=torch.uint8, device=dev).random_(0, 255)
     dst = torch.empty_like(src)
     for _ in range(10):
         dst.copy_(src)
+    L = load_package().cabi.lib()
+    stream = ctypes.c_void_p(torch.cuda.current_stream().cuda_stream)
+    for _ in range(10):
+        L.mi355x_rownorm_stream_probe(ctypes.c_void_p(src.data_ptr()), None,
+                                      ctypes.c_void_p(dst.data_ptr()), 256 << 20, 0, stream)
     torch.cuda.synchronize()
 
 
@@ -254,7 +264,32 @@ def device_copy_table(torch, dev, M, N):
                      "frac": round(gbs / HBM_PEAK_GBS, 4)})
         del pairs
         torch.cuda.empty_cache()
-    return {"what": "torch copy_ of a tensor of that size: bytes read + written over time", "rows": rows}
+    out = {"what": "torch copy_ of a tensor of that size: bytes read + written over time",
+           "rows": rows}
+    # the library's own plain streaming kernels (mi355x_rownorm_stream_probe) on tensors of the
+    # benchmark's size: the ceiling a kernel of this family's traffic mix can reach on this box
+    import ctypes
+    cabi = load_package().cabi
+    L = cabi.lib()
+    stream = ctypes.c_void_p(torch.cuda.current_stream().cuda_stream)
+    nbytes = M * N * 2
+    bufs = [tuple(torch.empty(nbytes, dtype=torch.uint8, device=dev).random_(0, 255) for _ in range(3))
+            for _ in range(3)]
+    probe = []
+    for mode, what, moved in ((0, "copy (1 read : 1 write, a forward's mix)", 2 * nbytes),
+                              (1, "c = a + b (2 reads : 1 write, a backward's mix)", 3 * nbytes),
+                              (2, "read only (two tensors summed)", 2 * nbytes)):
+        fns = [(lambda t=t: L.mi355x_rownorm_stream_probe(
+            ctypes.c_void_p(t[0].data_ptr()), ctypes.c_void_p(t[1].data_ptr()),
+            ctypes.c_void_p(t[2].data_ptr()), nbytes, mode, stream)) for t in bufs]
+        assert fns[0]() == 0
+        us = _time_rotating(torch, fns, iters=40, warm=10)
+        probe.append({"kernel": what, "tensor_bytes": nbytes, "us": round(us, 2),
+                      "GB/s": round(moved / us / 1e3, 1), "frac": round(moved / us / 1e3 / HBM_PEAK_GBS, 4)})
+    del bufs
+    torch.cuda.empty_cache()
+    out["stream_probe"] = probe
+    return out
 
 
 def stock_step(torch, sets, w, M, N, eps, step_bytes):
@@ -307,18 +342,25 @@ def stock_step(torch, sets, w, M, N, eps, step_bytes):
                 else "F.rms_norm + autograd backward (with autograd's own bookkeeping)")}
 
 
-def _time_rotating(torch, fns, iters=60, warm=30):
+def _time_rotating(torch, fns, iters=60, warm=30, windows=3):
+    """Average microseconds per call: `warm` untimed calls, then `windows` timing windows of
+    `iters` back-to-back calls each between one HIP event pair, rotating over `fns`; the median
+    window is reported (the first window after a pause runs up to a few percent slower while the
+    clocks settle, which a single window charged to whichever op came first)."""
     n = len(fns)
     for i in range(warm):
         fns[i % n]()
     torch.cuda.synchronize()
-    a, b = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
-    a.record()
-    for i in range(iters):
-        fns[i % n]()
-    b.record()
-    torch.cuda.synchronize()
-    return a.elapsed_time(b) * 1e3 / iters
+    times = []
+    for _ in range(windows):
+        a, b = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+        a.record()
+        for i in range(iters):
+            fns[i % n]()
+        b.record()
+        torch.cuda.synchronize()
+        times.append(a.elapsed_time(b) * 1e3 / iters)
+    return sorted(times)[len(times) // 2]
 
 
 def per_op_table(torch, cabi, L, dev, stream, P, only=None, iters=60, warm=30):

@@ -202,7 +202,14 @@ int mi355x_add_rms_norm_bwd(const void* dy, const void* dh_in, const void* h, co
  * routine.  Every call on one GPU shares that GPU's array: calls that overlap
  * in time on one GPU (two streams, two threads) race; calls on one stream are
  * ordered and safe.  Nothing in the array has to start at zero: each launch
- * writes every partial row before its second stage reads it. */
+ * writes every partial row before its second stage reads it.
+ * Two rules for callers.  (1) The current device must be the device of
+ * `stream` (as for any launch): the array's address is looked up for the current
+ * device, each GPU holding its own copy.  (2) Before a call is recorded into a
+ * HIP graph, make one ordinary call of the same shape on that device: the first
+ * call on a device resolves the array's address (hipGetSymbolAddress), and the
+ * first launch of a kernel loads its code object together with the 32 MiB array;
+ * neither belongs inside a capture. */
 size_t mi355x_rms_norm_bwd_static_limit_bytes(void);
 int mi355x_rms_norm_bwd_static(const void* dy, const void* x, const float* rstd,
                                const void* gamma, void* dx, void* dgamma, int64_t M, int64_t N,
@@ -369,6 +376,18 @@ int mi355x_rownorm_plan_at(rownorm_op op, int64_t M, int64_t N, rownorm_dtype x_
  * does a field outside 0..65535. */
 int mi355x_rownorm_set_override(rownorm_op op, int lanes_per_row, int packs_per_lane,
                                 int block_threads, int blocks_per_cu);
+
+/* Measurement aid, no counterpart in the reference: a plain streaming kernel over
+ * `bytes` bytes (a multiple of 16; 16-byte aligned device pointers) of each
+ * tensor, in the read : write mixes of this operator family -- mode 0: c = a
+ * (1 : 1, a forward's traffic), mode 1: c = a + b as 32-bit integers (2 : 1, a
+ * backward's), mode 2: a and b are read and summed, and only
+ * min(bytes / 16384, 2048) * 4096 bytes of c are written.  What such a kernel
+ * reaches is the practical ceiling an operator's fraction of the HBM peak is read
+ * against, and the kernel of known size that rocprofv3's FETCH_SIZE / WRITE_SIZE
+ * readings are scaled by.  Launches on `stream`, allocates nothing. */
+int mi355x_rownorm_stream_probe(const void* a, const void* b, void* c, size_t bytes, int mode,
+                                void* stream);
 
 #ifdef __cplusplus
 }

@@ -127,7 +127,12 @@ static void check_validation() {
   CHECK(p_mi355x_rownorm_plan(ROWNORM_OP_RMS_NORM_BWD, 16384, 4096, ROWNORM_BF16, ROWNORM_BF16,
                               &plan) == 0);
   CHECK(plan.resident == 1 && plan.lanes_per_row * plan.packs_per_lane * 8 >= 4096);
-  CHECK(p_mi355x_rms_norm_bwd_workspace_bytes(16384, 4096, ROWNORM_BF16, ROWNORM_BF16, 1) ==
+  // (the query covers calls with and without dX, which may take different grids)
+  CHECK(p_mi355x_rms_norm_bwd_workspace_bytes(16384, 4096, ROWNORM_BF16, ROWNORM_BF16, 1) >=
+        (size_t)plan.partial_rows * 4096 * sizeof(float));
+  CHECK(p_mi355x_rownorm_plan(ROWNORM_OP_RMS_NORM_BWD, 16384, 4096, ROWNORM_F32, ROWNORM_F32,
+                              &plan) == 0);
+  CHECK(p_mi355x_rms_norm_bwd_workspace_bytes(16384, 4096, ROWNORM_F32, ROWNORM_F32, 1) ==
         (size_t)plan.partial_rows * 4096 * sizeof(float));
 }
 

@@ -2,14 +2,18 @@
 vectors of the main family (tests/golden/aten_cpu_golden.npz: ln_*, lnmix_*, rms_*, sm_*, lsm_* --
 the inputs with +-1e4 outliers, a constant row, a fully masked row, and the CPU ops' own outputs in
 the inputs' dtype, 16-bit outputs included).  Same bounds as tests/test_oracle_golden.py holds the
-oracle to: float32 rtol = atol = 1e-5, 16-bit atol 1e-2 / rtol 1.6e-2, widened by the stated
-factors where the float32 CPU kernel's own float32 sums are the looser side.  The saved statistics
+oracle to: float32 rtol = atol = 1e-5, 16-bit atol 1e-2 / rtol 1.6e-2.  Where a result is a sum
+(the backward, rstd) the stored CPU value is itself a float32 (or rounded 16-bit) evaluation that
+sits some distance from the float64 oracle on these +-1e4 inputs; the comparison against it
+carries exactly that measured distance, |CPU golden - oracle| per element, as slack, so a HIP
+result may be as far from the golden value as the tolerance plus the golden value's own error and
+no farther (no blanket factors).  The saved statistics
 follow the GPU contract (float32, src/ATen/native/xpu/LayerNorm.cpp:72-75 in the reference) and are
 compared with the CPU op's 16-bit ones at the 16-bit tolerance."""
 import pytest
 import torch
 
-from helpers import GOLDEN_DTYPES, assert_close, load_golden, offset_view
+from helpers import GOLDEN_DTYPES, abs_err, assert_close, load_golden, offset_view, to_np32
 
 pytestmark = pytest.mark.gpu
 
@@ -19,11 +23,13 @@ NAMES = sorted(CASES)
 
 @pytest.mark.parametrize("case", NAMES)
 @pytest.mark.parametrize("offset", [0, 1], ids=["aligned", "off1"])
-def test_layer_norm_and_rms_norm_against_golden(cabi, gpu, case, offset):
+def test_layer_norm_and_rms_norm_against_golden(cabi, oracle, gpu, case, offset):
     c = CASES[case]
     dt = GOLDEN_DTYPES[case.split("_")[0]]
+    N = c["x"].shape[1]
     put = (lambda t: offset_view(t.to(gpu), offset)) if offset else (lambda t: t.to(gpu))
     x, dy = put(c["x"]), put(c["dy"])
+    own = lambda golden, exact: abs_err(golden, exact)  # noqa: E731  (the golden value's own error)
     variants = (("ln", c["gamma"], c["beta"]),)
     if dt != torch.float32:
         variants += (("lnmix", c["gamma"].float(), c["beta"].float()),)
@@ -38,21 +44,33 @@ def test_layer_norm_and_rms_norm_against_golden(cabi, gpu, case, offset):
         dx, dg, db = cabi.layer_norm_bwd(dy, x, put(c[pre + "_mean"].float()),
                                          put(c[pre + "_rstd"].float()), put(gamma))
         assert dg.dtype == gamma.dtype and db.dtype == gamma.dtype
+        odx, odg, odb = oracle.layer_norm_bwd(to_np32(c["dy"]), to_np32(c["x"]), (N,),
+                                              to_np32(c[pre + "_mean"]), to_np32(c[pre + "_rstd"]),
+                                              to_np32(gamma))
+        assert_close(dx, odx, dt, case + " " + pre + " dx vs oracle")
         assert_close(dx, c[pre + "_dx"], dt, case + " " + pre + " dx",
-                     scale=4.0 if dt == torch.float32 else 1.0)
-        assert_close(dg, c[pre + "_dgamma"], dt, case + " " + pre + " dgamma", scale=4.0)
-        assert_close(db, c[pre + "_dbeta"], dt, case + " " + pre + " dbeta", scale=4.0)
+                     slack=own(c[pre + "_dx"], odx))
+        assert_close(dg, c[pre + "_dgamma"], dt, case + " " + pre + " dgamma",
+                     slack=own(c[pre + "_dgamma"], odg))
+        assert_close(db, c[pre + "_dbeta"], dt, case + " " + pre + " dbeta",
+                     slack=own(c[pre + "_dbeta"], odb))
     y, rstd = cabi.rms_norm_fwd(x, put(c["gamma"]), 1e-6)
     assert_close(y, c["rms_y"], dt, case + " rms y")
-    assert_close(rstd, c["rms_rstd"], torch.float32, case + " rms rstd", scale=2.0)
+    _, orstd = oracle.rms_norm_fwd(to_np32(c["x"]), (N,), to_np32(c["gamma"]), 1e-6)
+    assert_close(rstd, orstd.reshape(-1), torch.float32, case + " rms rstd vs oracle")
+    assert_close(rstd, c["rms_rstd"], torch.float32, case + " rms rstd",
+                 slack=own(c["rms_rstd"], orstd.reshape(-1)))
     dx, dg = cabi.rms_norm_bwd(dy, x, put(c["rms_rstd"]), put(c["gamma"]))
-    assert_close(dx, c["rms_dx"], dt, case + " rms dx", scale=4.0)
-    assert_close(dg, c["rms_dgamma"], dt, case + " rms dgamma", scale=4.0)
+    odx, odg = oracle.rms_norm_bwd(to_np32(c["dy"]), to_np32(c["x"]), (N,), to_np32(c["rms_rstd"]),
+                                   to_np32(c["gamma"]))
+    assert_close(dx, odx, dt, case + " rms dx vs oracle")
+    assert_close(dx, c["rms_dx"], dt, case + " rms dx", slack=own(c["rms_dx"], odx))
+    assert_close(dg, c["rms_dgamma"], dt, case + " rms dgamma", slack=own(c["rms_dgamma"], odg))
 
 
 @pytest.mark.parametrize("case", NAMES)
 @pytest.mark.parametrize("offset", [0, 1], ids=["aligned", "off1"])
-def test_softmax_against_golden(cabi, gpu, case, offset):
+def test_softmax_against_golden(cabi, oracle, gpu, case, offset):
     c = CASES[case]
     dt = GOLDEN_DTYPES[case.split("_")[0]]
     put = (lambda t: offset_view(t.to(gpu), offset)) if offset else (lambda t: t.to(gpu))
@@ -63,5 +81,6 @@ def test_softmax_against_golden(cabi, gpu, case, offset):
         assert_close(y, c[nm + "_y"], dt, case + " " + nm + " y")
         assert bool(torch.isnan(y[2]).all())  # the fully masked row
         gi = cabi.softmax_bwd(dy, put(c[nm + "_y"]), is_log)
+        ogi = oracle.softmax_bwd(to_np32(c["dy"]), to_np32(c[nm + "_y"]), is_log)
         assert_close(gi, c[nm + "_gi"], dt, case + " " + nm + " grad_input",
-                     scale=8.0 if (is_log and dt == torch.float32) else 1.0)
+                     slack=abs_err(c[nm + "_gi"], ogi))

@@ -106,17 +106,28 @@ def test_limit_is_an_error_before_any_launch(cabi, gpu):
     # does not
     for (m, n) in ((16384, 8192), (16384, 16384), (4096, 18432), (4096, 32768), (4096, 65536)):
         assert L.mi355x_rms_norm_bwd_workspace_bytes(m, n, cabi.BF16, cabi.BF16, 1) <= limit
+    for (m, n) in ((16384, 4096), (4096, 16384), (16384, 8192), (2048, 32768), (64, 1 << 20)):
+        assert L.mi355x_rms_norm_bwd_workspace_bytes(m, n, cabi.F32, cabi.F32, 1) <= limit
+        assert L.mi355x_rms_norm_bwd_workspace_bytes(m, n, cabi.F16, cabi.F32, 1) <= limit
     M, N = 16384, 8192
-    one = ctypes.c_void_p(256)  # never dereferenced
+    # real device memory behind every pointer: should a validation regression ever let one of
+    # these calls launch, it reads and writes memory it owns instead of faulting the GPU
+    bufs = [torch.zeros(M * N, dtype=torch.bfloat16, device=gpu) for _ in range(3)]
+    stat = torch.ones(M, device=gpu)
+    wt = [torch.ones(N, dtype=torch.bfloat16, device=gpu) for _ in range(2)]
+    P = lambda t: ctypes.c_void_p(t.data_ptr())  # noqa: E731
+    stream = ctypes.c_void_p(torch.cuda.current_stream().cuda_stream)
     try:
         cabi.set_override(cabi.OP_RMS_NORM_BWD, 0, 0, 0, 8)
         need = L.mi355x_rms_norm_bwd_workspace_bytes(M, N, cabi.BF16, cabi.BF16, 1)
         assert need > limit
-        assert L.mi355x_rms_norm_bwd_static(one, one, one, one, one, one, M, N, cabi.BF16,
-                                            cabi.BF16, None) == -6
+        assert L.mi355x_rms_norm_bwd_static(P(bufs[0]), P(bufs[1]), P(stat), P(wt[0]), P(bufs[2]),
+                                            P(wt[1]), M, N, cabi.BF16, cabi.BF16, stream) == -6
     finally:
         cabi.clear_overrides()
+    torch.cuda.synchronize()
+    assert float(bufs[2].float().abs().max()) == 0.0 and float(wt[1].float().min()) == 1.0  # untouched
     assert "static" in cabi.error_string(-6)
     # dX alone needs no scratch at that size: accepted (nothing launched here: empty problem)
-    assert L.mi355x_rms_norm_bwd_static(one, one, one, one, one, None, 0, N, cabi.BF16, cabi.BF16,
-                                        None) == 0
+    assert L.mi355x_rms_norm_bwd_static(P(bufs[0]), P(bufs[1]), P(stat), P(wt[0]), P(bufs[2]), None,
+                                        0, N, cabi.BF16, cabi.BF16, stream) == 0

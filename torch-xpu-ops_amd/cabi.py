@@ -29,6 +29,7 @@ EXPORTED_SYMBOLS = (
     "mi355x_softmax_strided_plan", "mi355x_group_norm_fwd",
     "mi355x_group_norm_bwd_workspace_bytes", "mi355x_group_norm_bwd", "mi355x_group_norm_plan",
     "mi355x_rownorm_plan", "mi355x_rownorm_plan_at", "mi355x_rownorm_set_override",
+    "mi355x_rownorm_stream_probe",
 )
 
 
@@ -105,6 +106,8 @@ def lib():
         L.mi355x_rownorm_plan_at.argtypes = [_int, _i64, _i64, _int, _int, _int,
                                              ctypes.POINTER(Plan)]
         L.mi355x_rownorm_set_override.argtypes = [_int, _int, _int, _int, _int]
+        L.mi355x_rownorm_stream_probe.argtypes = [_vp, _vp, _vp, ctypes.c_size_t, _int, _vp]
+        L.mi355x_rownorm_stream_probe.restype = _int
         for name in ("mi355x_layer_norm_fwd", "mi355x_rms_norm_fwd", "mi355x_layer_norm_bwd",
                      "mi355x_rms_norm_bwd", "mi355x_rms_norm_bwd_static",
                      "mi355x_add_layer_norm_fwd", "mi355x_add_rms_norm_fwd",

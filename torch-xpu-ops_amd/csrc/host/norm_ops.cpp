@@ -1,6 +1,7 @@
 // LayerNorm / RMSNorm host operators: shape checks, output allocation, saved
 // statistics layout, then one call into the C ABI.  Contracts follow the
 // reference's src/ATen/native/xpu/LayerNorm.cpp (cited per function).
+#include "dispatch_stub_slot.h"
 #include "norm_ops.h"
 
 #include <ATen/native/layer_norm.h>
@@ -345,16 +346,6 @@ std::tuple<Tensor, Tensor> _fused_rms_norm_backward(const Tensor& dY, const Tens
 
 namespace {
 
-// The GPU slot of one of ATen's DispatchStub objects.  A DispatchStub is a
-// standard-layout class whose only non-static data member is its
-// DispatchStubImpl, so the object's address is that member's address; the
-// class has a setter for the slot but no getter, and uninstalling needs the
-// previous value.
-template <class Stub>
-void*& gpu_slot(Stub& stub) {
-  return reinterpret_cast<at::native::DispatchStubImpl*>(&stub)->cuda_dispatch_ptr;
-}
-
 struct SavedStubs {
   bool installed = false;
   void* forward = nullptr;
@@ -385,17 +376,20 @@ void stub_backward(const Tensor& dY, const Tensor& X, const Tensor& mean, const 
 
 void install_layer_norm_dispatch_stubs() {
   if (g_layer_norm_saved.installed) return;
-  g_layer_norm_saved.forward = gpu_slot(at::native::LayerNormKernel);
-  g_layer_norm_saved.backward = gpu_slot(at::native::LayerNormBackwardKernel);
+  g_layer_norm_saved.forward =
+      install_checked(at::native::LayerNormKernel, &stub_forward, "LayerNormKernel");
+  g_layer_norm_saved.backward = install_checked(at::native::LayerNormBackwardKernel,
+                                                &stub_backward, "LayerNormBackwardKernel");
   g_layer_norm_saved.installed = true;
-  at::native::LayerNormKernel.set_cuda_dispatch_ptr(&stub_forward);
-  at::native::LayerNormBackwardKernel.set_cuda_dispatch_ptr(&stub_backward);
 }
 
 void uninstall_layer_norm_dispatch_stubs() {
   if (!g_layer_norm_saved.installed) return;
-  gpu_slot(at::native::LayerNormKernel) = g_layer_norm_saved.forward;
-  gpu_slot(at::native::LayerNormBackwardKernel) = g_layer_norm_saved.backward;
+  restore<decltype(at::native::LayerNormKernel), std::remove_pointer_t<at::native::forward_fn>>(
+      at::native::LayerNormKernel, g_layer_norm_saved.forward);
+  restore<decltype(at::native::LayerNormBackwardKernel),
+          std::remove_pointer_t<at::native::backward_fn>>(at::native::LayerNormBackwardKernel,
+                                                          g_layer_norm_saved.backward);
   g_layer_norm_saved = SavedStubs{};
 }
 

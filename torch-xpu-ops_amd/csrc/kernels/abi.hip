@@ -254,14 +254,25 @@ size_t split_bytes(const Plan& plan, int64_t M, bool want_cols) {
   return want_cols ? (size_t)M * 2 * sizeof(float) : 0;
 }
 
+// The query does not know whether the call will write dX or add a residual
+// gradient, and the launch layout (hence the partial rows) may depend on both:
+// it returns what the largest of those calls needs.
 size_t norm_bwd_workspace(int op, int64_t M, int64_t N, int xd, int wd, int nparts) {
   if (!norm_dtypes_ok(xd, wd) || shape_check(M, N) || M == 0 || N == 0) return 0;
-  Plan plan;
-  if (make_plan(OC_NORM_BWD, M, N, esize_of(xd), current_num_cus(), g_override[op], nparts > 0,
-                &plan, false, op == ROWNORM_OP_LAYER_NORM_BWD, esize_of(wd) > esize_of(xd)))
-    return 0;
-  return (size_t)plan.partial_rows * (size_t)N * sizeof(float) * (size_t)nparts +
-         split_bytes(plan, M, nparts > 0);
+  size_t most = 0;
+  for (int variant = 0; variant < 4; ++variant) {
+    const bool fused_add = (variant & 1) != 0, want_dx = (variant & 2) != 0;
+    if (fused_add && !want_dx) continue;  // the residual gradient is added to dX
+    Plan plan;
+    if (make_plan(OC_NORM_BWD, M, N, esize_of(xd), current_num_cus(), g_override[op], nparts > 0,
+                  &plan, false, op == ROWNORM_OP_LAYER_NORM_BWD, esize_of(wd) > esize_of(xd),
+                  false, fused_add, false, want_dx))
+      return 0;
+    const size_t need = (size_t)plan.partial_rows * (size_t)N * sizeof(float) * (size_t)nparts +
+                        split_bytes(plan, M, nparts > 0);
+    if (need > most) most = need;
+  }
+  return most;
 }
 
 // dres: the gradient reaching the normalized row by the residual path, added to dx (or null).
@@ -281,7 +292,7 @@ int norm_bwd(const void* dy, const void* x, const float* mean, const float* rstd
   const int op = RMS ? ROWNORM_OP_RMS_NORM_BWD : ROWNORM_OP_LAYER_NORM_BWD;
   if (int e = make_plan(OC_NORM_BWD, M, N, esize_of(xd), current_num_cus(), g_override[op],
                         want_cols, &plan, false, !RMS, esize_of(wd) > esize_of(xd), false,
-                        dres != nullptr))
+                        dres != nullptr && dx != nullptr, false, dx != nullptr))
     return e;
   float* part_dg = nullptr;
   float* part_db = nullptr;

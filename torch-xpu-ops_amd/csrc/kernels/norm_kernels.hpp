@@ -995,6 +995,239 @@ norm_bwd_resident_kernel(const T* __restrict__ dy, const T* __restrict__ x, cons
   }
 }
 
+// ---------------------------------------------------------------------------
+// The same backward for 16-bit rows that fill a two-pack layout exactly: N ==
+// G * V * E with G a whole number of wavefronts (not necessarily a power of two:
+// hidden 5120 is 320 lanes x 2 packs, 7168 is 448 x 2), every row slot of every
+// row block holds a row (M % (BLOCK / G) == 0), and dx is written.
+//
+// No load and no store of the row loop is conditional.  In the kernel above a
+// store sits behind a branch on the execution mask; the compiler cannot know
+// whether it was issued, so its wait for the prefetched row -- older than that
+// store, and the memory counter retires in order -- became a wait for the store as
+// well: every iteration stalled until its predecessor's dX had reached L2.  Here a
+// wait names exactly the operations that may stay in flight, and the rows of the
+// next D - 1 iterations are on their way while the current one is worked on: the
+// lane keeps D register sets and the row loop is unrolled D times, each copy of
+// the body naming its sets statically (a register copy out of a set that is still
+// being loaded would be a wait).  The row index is wavefront-uniform (a row slot
+// is whole wavefronts), so row pointers are scalar arithmetic, mean / rstd are
+// scalar loads and a lane adds a constant 32-bit offset.  One workgroup a compute
+// unit (its lanes may take up to 256 registers): half the partial rows of the
+// two-workgroup grid.  Arithmetic, summation order and partial rows are those of
+// norm_bwd_resident_kernel, bit for bit for the same grid.
+//
+// Measured against norm_bwd_resident_kernel on one MI355X, bf16 rows x 16384
+// (LayerNorm / RMSNorm, us): N = 2048 43.0 / 39.0 -> 40.5 / 37.6; 4096 74.5 / 69.9 ->
+// 71.0 / 68.1; 5120 91.6 / 86.0 -> 89.3 / 85.3; 7168 125.6 / 120.4 -> 118.5 / 117.1;
+// 8192 138.7 / 133.8 -> 134.5 / 130.6; LayerNorm 14336 250.9 -> 245.6 and 16384
+// 285.4 -> 274.8 (with fp32 weights 266 -> 245 and 294 -> 275); 4096 rows of 4096:
+// 28.1 / 25.2 -> 26.4 / 22.8.  Rows of 6144, 10240 and 12288 elements measured the
+// same or slower than their three-pack layouts and keep those.
+template <class T, class WT, int E, int V>
+struct BwdRowSet {
+  float mu, rs;
+  Pack<T, E> x[V], d[V];
+};
+
+template <class T, class WT, int G, int V, int BLOCK, bool RMS, bool ADD, int D>
+__global__ void __launch_bounds__(BLOCK)
+norm_bwd_exact_kernel(const T* __restrict__ dy, const T* __restrict__ x, const T* dres,
+                      const float* __restrict__ mean, const float* __restrict__ rstd,
+                      const WT* __restrict__ gamma, T* dx, float* __restrict__ part_dg,
+                      float* __restrict__ part_db, int64_t M, int N) {
+  constexpr int E = elems_per_pack<T>::value;
+  constexpr int RPB = BLOCK / G;  // row slots of the workgroup
+  static_assert(G >= 64 && D >= 1 && sizeof(T) == 2, "16-bit rows on whole wavefronts");
+  // the column sums of the row slots beyond the first, parked for the first to add
+  constexpr int NSUMS = RMS ? 1 : 2;
+  constexpr int FOLD_FLOATS = (RPB > 1) ? (RPB - 1) * NSUMS * G * V * E : 4;
+  __shared__ float red[reduce_lds_floats<G, BLOCK, 2>::value];
+  __shared__ __attribute__((aligned(16))) float fold[FOLD_FLOATS];
+  int phase = 0;
+  const int slot = threadIdx.x / G;
+  const int lane0 = threadIdx.x % G;
+  const float inv_n = 1.0f / (float)N;
+  const bool want_cols = part_dg != nullptr;  // uniform
+  constexpr bool kWideWeights = V * E <= 16;
+
+  Pack<WT, E> gp[V];
+  float dg[V][E];
+  float db[RMS ? 1 : V][RMS ? 1 : E];
+#pragma unroll
+  for (int c = 0; c < V; ++c) {
+    gp[c] = gamma ? Pack<WT, E>::load(gamma + (c * G + lane0) * E) : Pack<WT, E>::splat(1.0f);
+#pragma unroll
+    for (int i = 0; i < E; ++i) {
+      dg[c][i] = 0.0f;
+      if constexpr (!RMS) db[c][i] = 0.0f;
+    }
+  }
+
+  const int64_t nrb = M / RPB;
+  const int64_t step = gridDim.x;
+  BwdRowSet<T, WT, E, V> ring[D];
+  // (past the last row block the requests go to row block 0 and are never used)
+  // A row slot is a whole number of wavefronts, so the row index is the same in
+  // every lane of a wavefront: it lives in scalar registers, the row pointers are
+  // scalar arithmetic, and a lane adds its constant 32-bit byte offset.
+  const int slot_u = __builtin_amdgcn_readfirstlane(slot);
+  uint32_t voff[V];
+#pragma unroll
+  for (int c = 0; c < V; ++c) voff[c] = (uint32_t)((c * G + lane0) * E * (int)sizeof(T));
+  auto at = [](const T* rowp, uint32_t off) {
+    return reinterpret_cast<const T*>(reinterpret_cast<const char*>(rowp) + off);
+  };
+  auto fetch = [&](int64_t rb, BwdRowSet<T, WT, E, V>& o) {
+    const int64_t row = (rb < nrb ? rb : 0) * RPB + slot_u;
+    o.mu = RMS ? 0.0f : mean[row];
+    o.rs = rstd[row];
+    const T* xr = x + row * (int64_t)N;
+    const T* gr = dy + row * (int64_t)N;
+#pragma unroll
+    for (int c = 0; c < V; ++c) {
+      o.x[c] = Pack<T, E>::load_stream(at(xr, voff[c]));
+      o.d[c] = Pack<T, E>::load_stream(at(gr, voff[c]));
+    }
+  };
+  auto work = [&](int64_t rb, BwdRowSet<T, WT, E, V>& w) {
+    const int64_t row = rb * RPB + slot_u;
+    const float mu = w.mu, rs = w.rs;
+    const float nmr = -mu * rs;
+    float acc[2] = {0.0f, 0.0f};
+#pragma unroll
+    for (int c = 0; c < V; ++c) {
+      if constexpr (!kWideWeights) keep_packed(gp[c]);
+#pragma unroll
+      for (int i = 0; i < E; ++i) {
+        const float xv = w.x[c].get(i);
+        const float xh = RMS ? xv * rs : fmaf(xv, rs, nmr);
+        const float gy = w.d[c].get(i);
+        const float g = gy * gp[c].get(i);
+        if constexpr (!RMS) acc[0] += g;
+        acc[1] = fmaf(g, xh, acc[1]);
+        dg[c][i] = fmaf(gy, xh, dg[c][i]);
+        if constexpr (!RMS) db[c][i] += gy;
+      }
+    }
+    group_allreduce<G, BLOCK, 2, SumOp>(acc, red, phase);
+    T* dr = dx + row * (int64_t)N;
+    const float s1 = acc[0], s2 = acc[1];
+    const float term1 = rs * inv_n;
+    const float a = s2 * term1;
+    const float b = RMS ? 0.0f : s1 * term1;
+    const float ra = rs * a;
+    const float cc = mu * ra - b;
+    Pack<T, E> up[ADD ? V : 1];
+    if constexpr (ADD) {
+#pragma unroll
+      for (int c = 0; c < V; ++c)
+        up[c] = Pack<T, E>::load_stream(at(dres + row * (int64_t)N, voff[c]));
+    }
+#pragma unroll
+    for (int c = 0; c < V; ++c) {
+      keep_packed(w.x[c]);
+      keep_packed(w.d[c]);
+      if constexpr (!kWideWeights) keep_packed(gp[c]);
+      Pack<T, E> o;
+#pragma unroll
+      for (int i = 0; i < E; ++i) {
+        const float g = w.d[c].get(i) * gp[c].get(i);
+        float f = fmaf(w.x[c].get(i), -ra, fmaf(g, rs, cc));
+        if constexpr (ADD) f += up[c].get(i);
+        o.set(i, f);
+      }
+      o.store_stream(const_cast<T*>(at(dr, voff[c])));
+    }
+  };
+
+#pragma unroll
+  for (int k = 0; k < D - 1; ++k) fetch(blockIdx.x + k * step, ring[k]);
+  int64_t rb = blockIdx.x;
+  // whole groups of D row blocks as straight-line code: set k is worked on while the
+  // set worked on before it is refilled with the row block D - 1 steps ahead
+  while (rb + (D - 1) * step < nrb) {
+#pragma unroll
+    for (int k = 0; k < D; ++k) {
+      fetch(rb + (D - 1) * step, ring[(k + D - 1) % D]);
+      work(rb, ring[k]);
+      rb += step;
+    }
+  }
+  // at most D - 1 row blocks are left, and they have been requested
+#pragma unroll
+  for (int k = 0; k < D - 1; ++k) {
+    if (rb < nrb) {  // uniform
+      work(rb, ring[k]);
+      rb += step;
+    }
+  }
+
+  if (!want_cols) return;
+  float* out_g = part_dg + (int64_t)blockIdx.x * N;
+  float* out_b = RMS ? nullptr : part_db + (int64_t)blockIdx.x * N;
+  if constexpr (RPB == 1) {
+#pragma unroll
+    for (int c = 0; c < V; ++c) {
+      const int e0 = (c * G + lane0) * E;
+      Pack<float, E> pg, pb;
+#pragma unroll
+      for (int i = 0; i < E; ++i) {
+        pg.set(i, dg[c][i]);
+        if constexpr (!RMS) pb.set(i, db[c][i]);
+      }
+      pg.store(out_g + e0);
+      if constexpr (!RMS) pb.store(out_b + e0);
+    }
+  } else {
+    // Row slots 1 .. RPB - 1 park their sums in LDS, 16 bytes a lane and half pack
+    // (lanes side by side: no bank conflict), one barrier, and slot 0 adds them to its
+    // own in slot order -- ((s0 + s1) + s2) + ..., the order of the kernel above -- and
+    // writes the partial row with 128-bit stores.
+    auto park = [&](int u, int which, int c, int h) {
+      return reinterpret_cast<float4*>(fold) +
+             ((((u - 1) * NSUMS + which) * V + c) * 2 + h) * G + lane0;
+    };
+    if (slot > 0) {
+#pragma unroll
+      for (int c = 0; c < V; ++c) {
+        *park(slot, 0, c, 0) = float4{dg[c][0], dg[c][1], dg[c][2], dg[c][3]};
+        *park(slot, 0, c, 1) = float4{dg[c][4], dg[c][5], dg[c][6], dg[c][7]};
+        if constexpr (!RMS) {
+          *park(slot, 1, c, 0) = float4{db[c][0], db[c][1], db[c][2], db[c][3]};
+          *park(slot, 1, c, 1) = float4{db[c][4], db[c][5], db[c][6], db[c][7]};
+        }
+      }
+    }
+    __syncthreads();
+    if (slot == 0) {
+#pragma unroll
+      for (int c = 0; c < V; ++c) {
+        const int e0 = (c * G + lane0) * E;
+        Pack<float, E> pg, pb;
+#pragma unroll
+        for (int i = 0; i < E; ++i) {
+          pg.set(i, dg[c][i]);
+          if constexpr (!RMS) pb.set(i, db[c][i]);
+        }
+#pragma unroll 1
+        for (int u = 1; u < RPB; ++u) {
+          const float4 g0 = *park(u, 0, c, 0), g1 = *park(u, 0, c, 1);
+          pg.v[0] += g0.x, pg.v[1] += g0.y, pg.v[2] += g0.z, pg.v[3] += g0.w;
+          pg.v[4] += g1.x, pg.v[5] += g1.y, pg.v[6] += g1.z, pg.v[7] += g1.w;
+          if constexpr (!RMS) {
+            const float4 b0 = *park(u, 1, c, 0), b1 = *park(u, 1, c, 1);
+            pb.v[0] += b0.x, pb.v[1] += b0.y, pb.v[2] += b0.z, pb.v[3] += b0.w;
+            pb.v[4] += b1.x, pb.v[5] += b1.y, pb.v[6] += b1.z, pb.v[7] += b1.w;
+          }
+        }
+        pg.store(out_g + e0);
+        if constexpr (!RMS) pb.store(out_b + e0);
+      }
+    }
+  }
+}
+
 // What a lane of the long-row backward holds of one pack between request and use.
 template <class T, class WT, int E>
 struct LongRowBwdIn {

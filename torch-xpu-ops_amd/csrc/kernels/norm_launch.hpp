@@ -107,11 +107,37 @@ struct NormBwdLauncher {
   };
 };
 
+// The exact two-pack layouts (kNormBwdExact): entry I of the table, if the plan names it.
+template <class T, class WT, bool RMS, bool ADD, int I>
+inline bool launch_norm_bwd_exact_at(const Plan& plan, const NormBwdArgs& a, hipStream_t stream) {
+  constexpr NormBwdExactLayout l = kNormBwdExact[I];
+  if constexpr (sizeof(T) == 2 && (!RMS || l.rms_too)) {
+    if (plan.G == l.G && plan.block == l.block && plan.exact_depth == l.depth) {
+      hipLaunchKernelGGL((norm_bwd_exact_kernel<T, WT, l.G, 2, l.block, RMS, ADD, l.depth>),
+                         dim3((unsigned)plan.grid), dim3(l.block), 0, stream, (const T*)a.dy,
+                         (const T*)a.x, (const T*)a.dres, a.mean, a.rstd, (const WT*)a.gamma,
+                         (T*)a.dx, a.part_dg, a.part_db, a.M, a.N);
+      return true;
+    }
+  }
+  return false;
+}
+template <class T, class WT, bool RMS, bool ADD, int... Is>
+inline bool launch_norm_bwd_exact(const Plan& plan, const NormBwdArgs& a, hipStream_t stream,
+                                  ilist<Is...>) {
+  return (launch_norm_bwd_exact_at<T, WT, RMS, ADD, Is>(plan, a, stream) || ...);
+}
+
 template <class T, class WT, bool RMS, bool ADD>
 int launch_norm_bwd(const Plan& plan, const NormBwdArgs& a, hipStream_t stream) {
   const bool want_cols = a.part_dg != nullptr;
   const T* dres = ADD ? (const T*)a.dres : nullptr;
-  if (plan.resident) {
+  if (plan.resident && plan.exact_depth > 0) {
+    static_assert(kNormBwdExactCount == 7, "one index per table entry below");
+    if (a.dx == nullptr ||
+        !launch_norm_bwd_exact<T, WT, RMS, ADD>(plan, a, stream, ilist<0, 1, 2, 3, 4, 5, 6>{}))
+      return (int)hipErrorInvalidConfiguration;
+  } else if (plan.resident) {
     NormBwdCtx<T, WT, RMS> ctx{plan, a, stream};
     const bool launched =
         plan.fast ? launch_variant<NormBwdLauncher<T, WT, RMS, true, ADD>::template At>(ctx)

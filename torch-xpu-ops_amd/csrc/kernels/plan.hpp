@@ -58,6 +58,9 @@ struct Plan {
   // a layout was asked for by override: kernels chosen by other means than the
   // layout (softmax of short ragged rows through LDS) stand back
   bool forced = false;
+  // norm backward on an exact two-pack layout (norm_bwd_exact_kernel): row blocks a
+  // lane keeps in flight, itself included; 0 = the general resident kernel
+  int exact_depth = 0;
 };
 
 constexpr int kMinG = 8;
@@ -198,6 +201,30 @@ constexpr bool norm_bwd_sums_in_lds(int esize, int G, int V, bool fast) {
 // 199 -> 351 us) and stay with the LDS sums; so do 6 packs (24576).
 constexpr bool norm_bwd_half_lanes_five(int esize, int wsize, int G, int V, bool rms, bool add) {
   return esize == 2 && wsize == 2 && G == 512 && V == 5 && rms && !add;
+}
+// Exact two-pack layouts of the 16-bit norm backward (norm_bwd_exact_kernel): a row
+// of `packs` = 2 * G packs on G lanes, G a whole number of wavefronts.  The table is
+// what measured faster than the general resident kernel on MI355X (see the kernel):
+// lanes, workgroup threads, row blocks in flight (1 = no prefetch), and whether the
+// RMSNorm takes it too (at 896 and 1024 lanes its general kernel already runs this
+// layout at the same speed).
+struct NormBwdExactLayout {
+  int G, block, depth;
+  bool rms_too;
+};
+constexpr NormBwdExactLayout kNormBwdExact[] = {
+    {128, 512, 2, true}, {256, 512, 3, true},  {320, 640, 2, true},   {448, 448, 2, true},
+    {512, 512, 3, true}, {896, 896, 1, false}, {1024, 1024, 1, false}};
+constexpr int kNormBwdExactCount = (int)(sizeof(kNormBwdExact) / sizeof(kNormBwdExact[0]));
+// Index into kNormBwdExact of the layout that serves such a call, or -1.
+constexpr int norm_bwd_exact_index(int esize, int64_t packs, int64_t M, bool layer_norm) {
+  if (esize != 2 || packs % 2 != 0) return -1;
+  for (int i = 0; i < kNormBwdExactCount; ++i) {
+    const NormBwdExactLayout& l = kNormBwdExact[i];
+    if (packs == 2 * (int64_t)l.G && (layer_norm || l.rms_too) && M % (l.block / l.G) == 0)
+      return i;
+  }
+  return -1;
 }
 // (a 512 x 5 instance exists for that case only)
 constexpr bool norm_bwd_instance_ok(int esize, int wsize, int G, int V, bool rms, bool add) {
@@ -393,10 +420,11 @@ inline bool norm_layout(OpClass oc, int esize, int64_t packs, bool layer_norm, b
 // fused_add: the norm forward adds a residual row first (two rows in flight a lane);
 // the norm backward adds the residual path's gradient to dX.
 // masked: the softmax call reads a mask (see masked_softmax_built()).
+// want_dx: the norm backward writes dX (its exact layouts exist for such calls only).
 inline int make_plan(OpClass oc, int64_t M, int64_t N, int esize, int num_cus, const Override& ov,
                      bool want_cols, Plan* out, bool force_general = false,
                      bool layer_norm = false, bool wide_weights = false, bool off_line = false,
-                     bool fused_add = false, bool masked = false) {
+                     bool fused_add = false, bool masked = false, bool want_dx = true) {
   Plan p;
   const int E = 16 / esize;
   p.fast = (N % E) == 0 && !force_general;
@@ -547,6 +575,17 @@ inline int make_plan(OpClass oc, int64_t M, int64_t N, int esize, int num_cus, c
       p.V = V;
       p.block = block;
       p.rpb = p.block / G;
+      // 16-bit backward rows that fill a two-pack layout of whole wavefronts
+      if (oc == OC_NORM_BWD && p.fast && want_dx && !p.forced) {
+        const int xi = norm_bwd_exact_index(esize, packs, M, layer_norm);
+        if (xi >= 0) {
+          p.G = kNormBwdExact[xi].G;
+          p.V = 2;
+          p.block = kNormBwdExact[xi].block;
+          p.rpb = p.block / p.G;
+          p.exact_depth = kNormBwdExact[xi].depth;
+        }
+      }
 
     } else {
       stream = true;
@@ -572,7 +611,7 @@ inline int make_plan(OpClass oc, int64_t M, int64_t N, int esize, int num_cus, c
   // a grid of that size halves the partial rows of the dgamma/dbeta reduction
   // (bf16 [16384, 12288]: LayerNorm 222 -> 208 us, RMSNorm 210 -> 204 us)
   if (ov.bpc == 0 && oc == OC_NORM_BWD && p.resident &&
-      norm_bwd_prefetches(esize, p.G, p.V, p.fast, !layer_norm))
+      (p.exact_depth > 0 || norm_bwd_prefetches(esize, p.G, p.V, p.fast, !layer_norm)))
     bpc = 1;
   int64_t grid = (int64_t)num_cus * bpc;
   // The norm forward beyond a few tens of thousands of rows (measured on bf16 rows
