@@ -242,3 +242,46 @@ def test_host_operators_and_autograd(pkg, ops, gpu, dtype):
         assert a.grad is not None and a.grad.dtype == dtype
         assert_close(a.grad, c.grad, dtype, "chain " + nm, scale=8.0)
     assert torch.equal(leaves[0].grad, leaves[1].grad)  # x and residual share the gradient of h
+
+
+def test_unused_outputs_are_not_materialized_and_direct_ops_refuse_grad(pkg, ops, gpu):
+    """Only y, or only h, feeds the loss: the unused output's gradient reaches backward as None
+    (no tensor of zeros is made for it) and the results equal the unfused composition; the direct
+    operators, which record no autograd graph, refuse tensors that require a gradient."""
+    B, D = 37, 512
+    g = gen(25)
+    dtype = torch.bfloat16
+    x = torch.randn(B, D, generator=g).to(dtype)
+    res = torch.randn(B, D, generator=g).to(dtype)
+    w = (1 + 0.1 * torch.randn(D, generator=g)).to(dtype)
+    b = (0.1 * torch.randn(D, generator=g)).to(dtype)
+    gy = torch.randn(B, D, generator=g).to(dtype)
+    for norm in ("rms", "ln"):
+        for use in ("y", "h"):
+            leaves = [t.to(gpu).requires_grad_() for t in (x, res, w, b)]
+            if norm == "rms":
+                y, h = pkg.fused.add_rms_norm(leaves[0], leaves[1], leaves[2], 1e-6)
+            else:
+                y, h = pkg.fused.add_layer_norm(leaves[0], leaves[1], leaves[2], leaves[3], 1e-5)
+            (y if use == "y" else h).backward(gy.to(gpu))
+            cl = [t.float().requires_grad_() for t in (x, res, w, b)]
+            ch = cl[0] + cl[1]
+            cy = (torch.nn.functional.rms_norm(ch, (D,), cl[2], 1e-6) if norm == "rms"
+                  else torch.nn.functional.layer_norm(ch, (D,), cl[2], cl[3], 1e-5))
+            (cy if use == "y" else ch).backward(gy.float())
+            if use == "h":
+                # the gradient of h passes through to x and residual, the weights get none
+                assert torch.equal(leaves[0].grad.cpu(), gy) and torch.equal(leaves[1].grad.cpu(), gy)
+                assert leaves[2].grad is None and leaves[3].grad is None
+            else:
+                assert_close(leaves[0].grad, cl[0].grad, dtype, norm + " dx, only y used", scale=2.0)
+                assert torch.equal(leaves[0].grad, leaves[1].grad)
+                assert_close(leaves[2].grad, cl[2].grad, dtype, norm + " dweight, only y used",
+                             scale=2.0)
+    xg = x.to(gpu).requires_grad_()
+    with pytest.raises(RuntimeError, match="records no autograd graph"):
+        ops.add_rms_norm(xg, res.to(gpu), [D], w.to(gpu), None)
+    with pytest.raises(RuntimeError, match="records no autograd graph"):
+        ops.add_layer_norm(x.to(gpu), res.to(gpu), [D], w.to(gpu).requires_grad_(), b.to(gpu), 1e-5)
+    with torch.no_grad():
+        ops.add_rms_norm(xg, res.to(gpu), [D], w.to(gpu), None)  # fine: nothing is recorded

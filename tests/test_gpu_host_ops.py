@@ -306,6 +306,48 @@ def test_aten_override_runs_autograd_end_to_end(pkg, gpu):
                 assert_close(a, r, dtype, "%s %s" % (name, nm), scale=4.0)
 
 
+@pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16], ids=str)
+def test_aten_override_routes_the_out_overloads(pkg, cabi, gpu, dtype):
+    """The reference's softmax ops are structured `.out` kernels (src/ATen/native/xpu/SoftMax.cpp:
+    22-100).  After the opt-in, torch.softmax(x, dim, out=o) / torch.log_softmax(..., out=o) and
+    the backward `.out` forms run the MI355X kernels: bit-equal to the C ABI called directly.  The
+    stock kernels' results differ from these in the last bits on this input, which is how the test
+    knows the call was routed."""
+    import warnings
+    x = (3 * torch.randn(64, 3000, generator=gen(30))).to(dtype).to(gpu)
+    g = torch.randn(64, 3000, generator=gen(31)).to(dtype).to(gpu)
+    pkg.restore_aten_ops()
+    stock = torch.empty_like(x)
+    torch.log_softmax(x, -1, out=stock)
+    with warnings.catch_warnings():
+        warnings.simplefilter("ignore")
+        pkg.override_aten_ops()
+    try:
+        for is_log, fn, bwd in ((False, torch.softmax, torch.ops.aten._softmax_backward_data),
+                                (True, torch.log_softmax, torch.ops.aten._log_softmax_backward_data)):
+            want = cabi.softmax_fwd(x, is_log)
+            o = torch.full_like(x, 7.0)
+            r = fn(x, -1, out=o)
+            assert r.data_ptr() == o.data_ptr() and torch.equal(o, want)
+            want_gi = cabi.softmax_bwd(g, want, is_log)
+            gi = torch.full_like(x, 7.0)
+            kw = {"out": gi} if is_log else {"grad_input": gi}
+            bwd.out(g, want, -1, dtype, **kw)
+            assert torch.equal(gi, want_gi)
+            # over a non-innermost dimension too
+            o0 = torch.empty_like(x)
+            fn(x, 0, out=o0)
+            assert torch.equal(o0, getattr(pkg.ops, "_log_softmax" if is_log else "_softmax")(x, 0, False))
+        mine = torch.empty_like(x)
+        torch.log_softmax(x, -1, out=mine)
+        assert_close(mine, stock, dtype, "routed vs stock log_softmax")
+    finally:
+        pkg.restore_aten_ops()
+    again = torch.empty_like(x)
+    torch.log_softmax(x, -1, out=again)
+    assert torch.equal(again, stock)  # the stock kernel is back
+
+
 def test_aten_override_masked_and_safe_softmax_autograd(pkg, gpu):
     """torch._masked_softmax / torch._safe_softmax on GPU tensors after the opt-in, forward and
     through autograd, against the CPU: the sizes, dims and mask types of

@@ -77,6 +77,12 @@ def override_aten_ops():
     lib.impl("_log_softmax", m._log_softmax.default, "CUDA")
     lib.impl("_softmax_backward_data", m._softmax_backward_data.default, "CUDA")
     lib.impl("_log_softmax_backward_data", m._log_softmax_backward_data.default, "CUDA")
+    # the structured `.out` kernels the reference implements (src/ATen/native/xpu/SoftMax.cpp:
+    # 22-100): torch.softmax(x, dim, out=o) and the backward `.out` forms
+    lib.impl("_softmax.out", m._softmax.out, "CUDA")
+    lib.impl("_log_softmax.out", m._log_softmax.out, "CUDA")
+    lib.impl("_softmax_backward_data.out", m._softmax_backward_data.out, "CUDA")
+    lib.impl("_log_softmax_backward_data.out", m._log_softmax_backward_data.out, "CUDA")
     lib.impl("native_group_norm", m.native_group_norm.default, "CUDA")
     lib.impl("native_group_norm_backward", m.native_group_norm_backward.default, "CUDA")
     lib.impl("_safe_softmax", m._safe_softmax.default, "CUDA")

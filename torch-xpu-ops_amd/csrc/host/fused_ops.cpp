@@ -2,6 +2,7 @@
 // (mi355x_add_layer_norm_fwd & co. in include/mi355x_rownorm.h).  Shapes, saved statistics and
 // output masks follow the unfused operators in norm_ops.cpp, i.e. the contracts of the
 // reference's src/ATen/native/xpu/LayerNorm.cpp:35-305.
+#include <ATen/core/grad_mode.h>
 #include "fused_ops.h"
 
 #include <ATen/native/layer_norm.h>
@@ -57,8 +58,22 @@ struct Forward {
 };
 
 // Common part of the two forwards: checks, contiguous operands, h and y.
+// These operators are registered for every dispatch key with no autograd formula
+// of their own: called on a tensor that requires a gradient they would hand back
+// outputs cut off from the graph without a word.  The differentiable forms are
+// torch_xpu_ops_amd.fused.add_rms_norm / add_layer_norm (autograd.Function, whose
+// forward runs with gradient recording off and so passes this check).
+void check_no_grad_wanted(const Tensor& t, const char* op, const char* name) {
+  TORCH_CHECK(!(t.defined() && at::GradMode::is_enabled() && t.requires_grad()), op, ": `", name,
+              "` requires a gradient, but this operator records no autograd graph; call "
+              "fused.add_rms_norm / fused.add_layer_norm (differentiable), or detach the "
+              "tensor / use torch.no_grad()");
+}
+
 Forward prepare_forward(const Tensor& input, const Tensor& residual,
                         std::optional<at::ScalarType> out_dtype, bool inplace, const char* op) {
+  check_no_grad_wanted(input, op, "input");
+  check_no_grad_wanted(residual, op, "residual");
   check_gpu(input, op, "input");
   check_same_device(input, residual, op, "residual");
   TORCH_CHECK(residual.defined() && residual.sizes().equals(input.sizes()) &&
@@ -89,6 +104,8 @@ std::tuple<Tensor, Tensor, Tensor, Tensor> add_layer_norm_impl(
   static const char* op = "mi355x::add_layer_norm";
   const Tensor weight = defined_or_empty(weight_opt);
   const Tensor bias = defined_or_empty(bias_opt);
+  check_no_grad_wanted(weight, op, "weight");
+  check_no_grad_wanted(bias, op, "bias");
   check_same_device(input, weight, op, "weight");
   check_same_device(input, bias, op, "bias");
   const auto [M, N] = at::native::_check_layer_norm_inputs(input, normalized_shape, weight, bias);
@@ -125,6 +142,7 @@ std::tuple<Tensor, Tensor, Tensor> add_rms_norm_impl(const Tensor& input, const 
                                                      bool inplace) {
   static const char* op = "mi355x::add_rms_norm";
   const Tensor weight = defined_or_empty(weight_opt);
+  check_no_grad_wanted(weight, op, "weight");
   check_same_device(input, weight, op, "weight");
   const auto [M, N] =
       at::native::_check_layer_norm_inputs(input, normalized_shape, weight, weight);

@@ -10,6 +10,7 @@
 #include <ATen/ops/native_group_norm_cuda_dispatch.h>
 #include <limits>
 
+#include "dispatch_stub_slot.h"
 #include "host_common.h"
 
 namespace mi355x {
@@ -40,14 +41,6 @@ rownorm_dtype stat_dtype(const Tensor& X, const Tensor& gamma, const Tensor& bet
 
 at::ScalarType to_scalar_type(rownorm_dtype d) {
   return d == ROWNORM_F32 ? at::kFloat : d == ROWNORM_F16 ? at::kHalf : at::kBFloat16;
-}
-
-// The GPU slot of one of ATen's DispatchStub objects (a standard-layout class
-// whose only non-static data member is its DispatchStubImpl; it has a setter
-// for the slot but no getter, and uninstalling needs the previous value).
-template <class Stub>
-void*& gpu_slot(Stub& stub) {
-  return reinterpret_cast<at::native::DispatchStubImpl*>(&stub)->cuda_dispatch_ptr;
 }
 
 struct SavedStubs {
@@ -242,17 +235,22 @@ std::tuple<Tensor, Tensor, Tensor> native_group_norm_backward(
 
 void install_group_norm_dispatch_stubs() {
   if (g_group_norm_saved.installed) return;
-  g_group_norm_saved.forward = gpu_slot(at::native::GroupNormKernel);
-  g_group_norm_saved.backward = gpu_slot(at::native::GroupNormBackwardKernel);
+  g_group_norm_saved.forward =
+      install_checked(at::native::GroupNormKernel, &group_norm_kernel, "GroupNormKernel");
+  g_group_norm_saved.backward = install_checked(at::native::GroupNormBackwardKernel,
+                                                &group_norm_backward_kernel,
+                                                "GroupNormBackwardKernel");
   g_group_norm_saved.installed = true;
-  at::native::GroupNormKernel.set_cuda_dispatch_ptr(&group_norm_kernel);
-  at::native::GroupNormBackwardKernel.set_cuda_dispatch_ptr(&group_norm_backward_kernel);
 }
 
 void uninstall_group_norm_dispatch_stubs() {
   if (!g_group_norm_saved.installed) return;
-  gpu_slot(at::native::GroupNormKernel) = g_group_norm_saved.forward;
-  gpu_slot(at::native::GroupNormBackwardKernel) = g_group_norm_saved.backward;
+  restore<decltype(at::native::GroupNormKernel),
+          std::remove_pointer_t<at::native::forward_fn>>(at::native::GroupNormKernel,
+                                                         g_group_norm_saved.forward);
+  restore<decltype(at::native::GroupNormBackwardKernel),
+          std::remove_pointer_t<at::native::backward_fn>>(at::native::GroupNormBackwardKernel,
+                                                          g_group_norm_saved.backward);
   g_group_norm_saved = SavedStubs{};
 }
 

@@ -26,14 +26,20 @@ class _AddRMSNorm(torch.autograd.Function):
         y, h, rstd = _ops().add_rms_norm(x, residual, normalized_shape, weight, eps, None)
         ctx.save_for_backward(h, rstd, weight)
         ctx.normalized_shape = normalized_shape
+        # an output the loss does not use arrives as None in backward, not as a tensor of
+        # zeros that would be allocated, written and read for nothing
+        ctx.set_materialize_grads(False)
         return y, h
 
     @staticmethod
     def backward(ctx, grad_y, grad_h):
         h, rstd, weight = ctx.saved_tensors
+        if grad_y is None:  # only h feeds the loss: its gradient passes through
+            return grad_h, grad_h, None, None, None
         want_w = weight is not None and ctx.needs_input_grad[2]
-        dh, dw = _ops().add_rms_norm_backward(grad_y.contiguous(), grad_h, h, ctx.normalized_shape,
-                                              rstd, weight, [True, want_w])
+        dh, dw = _ops().add_rms_norm_backward(
+            grad_y.contiguous(), None if grad_h is None else grad_h.contiguous(), h,
+            ctx.normalized_shape, rstd, weight, [True, want_w])
         # h = x + residual: both get the gradient of h
         return dh, dh, dw, None, None
 
@@ -45,16 +51,19 @@ class _AddLayerNorm(torch.autograd.Function):
                                                  None)
         ctx.save_for_backward(h, mean, rstd, weight, bias)
         ctx.normalized_shape = normalized_shape
+        ctx.set_materialize_grads(False)
         return y, h
 
     @staticmethod
     def backward(ctx, grad_y, grad_h):
         h, mean, rstd, weight, bias = ctx.saved_tensors
+        if grad_y is None:
+            return grad_h, grad_h, None, None, None, None
         mask = [True, weight is not None and ctx.needs_input_grad[2],
                 bias is not None and ctx.needs_input_grad[3]]
-        dh, dw, db = _ops().add_layer_norm_backward(grad_y.contiguous(), grad_h, h,
-                                                    ctx.normalized_shape, mean, rstd, weight, bias,
-                                                    mask)
+        dh, dw, db = _ops().add_layer_norm_backward(
+            grad_y.contiguous(), None if grad_h is None else grad_h.contiguous(), h,
+            ctx.normalized_shape, mean, rstd, weight, bias, mask)
         return dh, dh, dw, db, None, None
 
 
