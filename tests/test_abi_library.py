@@ -221,8 +221,19 @@ def test_plan_layouts_for_hidden_sizes_that_are_not_powers_of_two(cabi):
     assert lay(LF, 1024, F32) == (64, 4)
     # rows that fill at most 3/4 of the slots: three packs on fewer lanes (forward)
     for N, want in ((1536, (64, 3)), (3072, (128, 3)), (5120, (256, 3)), (6144, (256, 3))):
-        assert lay(LF, N, BF) == want and lay(RF, N, BF) == want
+        if N != 5120:  # (the norm forward at 5120 takes an exact layout, below)
+            assert lay(LF, N, BF) == want and lay(RF, N, BF) == want
         assert lay(cabi.OP_SOFTMAX_FWD, N, BF) == want
+    # 16-bit forward rows of 4096 and 5120 elements: exact two-pack layouts on 256 / 320 lanes,
+    # two 512-thread / three 320-thread resident workgroups a compute unit; an odd row count on
+    # two row slots a workgroup, and the fused add, keep the general kernel
+    for op in (LF, RF):
+        p = cabi.plan(op, 16384, 4096, BF, BF)
+        assert (p["lanes_per_row"], p["packs_per_lane"], p["block_threads"], p["grid_blocks"]) == (256, 2, 512, 512)
+        p = cabi.plan(op, 16384, 5120, BF, F32)
+        assert (p["lanes_per_row"], p["packs_per_lane"], p["block_threads"], p["grid_blocks"]) == (320, 2, 320, 768)
+        p = cabi.plan(op, 16383, 4096, BF, BF)
+        assert (p["lanes_per_row"], p["block_threads"]) == (256, 256)
     assert lay(LF, 7168, BF) == (512, 2)                       # fills 7/8: the rule stands
     assert lay(LB, 6144, BF) == (256, 3) and lay(RB, 6144, BF) == (256, 3)  # and the 16-bit backward from 513 packs
     # 16-bit backward rows that are two packs on a whole number of wavefronts, where that
@@ -237,7 +248,7 @@ def test_plan_layouts_for_hidden_sizes_that_are_not_powers_of_two(cabi):
     assert (p["block_threads"], p["grid_blocks"], p["partial_rows"]) == (512, 256, 256)
     assert lay(LB, 3072, BF) == (256, 2) and lay(RB, 2560, BF) == (256, 2)  # which keeps its lanes below
     assert lay(LF, 3072, BF, F32) == (256, 2)                  # fp32 weights below 512 lanes
-    assert lay(LF, 5120, BF, F32) == (256, 3)
+    assert lay(LF, 5120, BF, F32) == (320, 2) and lay(LF, 6144, BF, F32) == (256, 3)
     assert lay(cabi.OP_SOFTMAX_BWD, 5120, BF) == (512, 2)
     # 16-bit norm rows beyond 8192 elements: 512 lanes, not 1024
     assert lay(LF, 10240, BF) == (512, 3) and lay(LB, 10240, BF) == (512, 3)
@@ -290,19 +301,24 @@ def test_forward_grid_grows_with_the_row_count(cabi):
     unit while that means at most 32 row blocks a workgroup."""
     BF, F32 = cabi.BF16, cabi.F32
     grid = lambda op, M, N, wd=BF: cabi.plan(op, M, N, BF, wd)["grid_blocks"]
-    assert grid(cabi.OP_RMS_NORM_FWD, 16384, 4096) == 8192       # 256 CUs x 32: the floor
-    assert grid(cabi.OP_LAYER_NORM_FWD, 16384, 4096) == 8192
-    assert grid(cabi.OP_RMS_NORM_FWD, 16384, 4096, F32) == 768     # fp32 weights: three resident workgroups
+    assert grid(cabi.OP_RMS_NORM_FWD, 16384, 2048) == 8192       # 256 CUs x 32: the floor
+    assert grid(cabi.OP_LAYER_NORM_FWD, 16384, 2048) == 8192
+    assert grid(cabi.OP_RMS_NORM_FWD, 16384, 6144, F32) == 768     # fp32 weights: three resident workgroups
     assert grid(cabi.OP_LAYER_NORM_FWD, 16384, 8192) == 512        # LayerNorm on 512 lanes: two
     assert grid(cabi.OP_RMS_NORM_FWD, 16384, 8192) == 8192
     assert grid(cabi.OP_LAYER_NORM_FWD, 16384, 8192, F32) == 512   # 256 CUs x two 512-thread workgroups
-    assert grid(cabi.OP_LAYER_NORM_FWD, 16384, 4096, F32) == 768   # x three 256-thread workgroups
-    assert grid(cabi.OP_LAYER_NORM_FWD, 300, 4096, F32) == 300     # never more workgroups than row blocks
-    assert grid(cabi.OP_LAYER_NORM_FWD, 24576, 4096, F32) == 768   # 32 row blocks a workgroup: the last
-    assert grid(cabi.OP_LAYER_NORM_FWD, 24577, 4096, F32) == 4096
-    assert grid(cabi.OP_RMS_NORM_FWD, 65536, 4096) == 32768
-    assert grid(cabi.OP_LAYER_NORM_FWD, 65536, 4096) == 16384
-    assert grid(cabi.OP_LAYER_NORM_FWD, 65536, 4096, F32) == 8192
+    assert grid(cabi.OP_LAYER_NORM_FWD, 16384, 6144, F32) == 768   # x three 256-thread workgroups
+    assert grid(cabi.OP_LAYER_NORM_FWD, 300, 6144, F32) == 300     # never more workgroups than row blocks
+    assert grid(cabi.OP_LAYER_NORM_FWD, 24576, 6144, F32) == 768   # 32 row blocks a workgroup: the last
+    assert grid(cabi.OP_LAYER_NORM_FWD, 24577, 6144, F32) == 4096
+    assert grid(cabi.OP_RMS_NORM_FWD, 65536, 6144) == 32768
+    assert grid(cabi.OP_LAYER_NORM_FWD, 65536, 6144) == 16384
+    assert grid(cabi.OP_LAYER_NORM_FWD, 65536, 6144, F32) == 8192
+    # the exact layouts of 4096 / 5120 keep one resident grid up to 128 row blocks a workgroup
+    assert grid(cabi.OP_LAYER_NORM_FWD, 300, 4096, F32) == 150
+    assert grid(cabi.OP_RMS_NORM_FWD, 131072, 4096) == 512
+    assert grid(cabi.OP_RMS_NORM_FWD, 262144, 4096) == 131072
+    assert grid(cabi.OP_LAYER_NORM_FWD, 65536, 5120) == 768
     assert grid(cabi.OP_RMS_NORM_FWD, 262144, 2048) == 65536     # two rows a workgroup iteration
     assert grid(cabi.OP_RMS_NORM_BWD, 262144, 4096) == 256       # backward: one partial row each
     assert grid(cabi.OP_RMS_NORM_BWD, 262144, 6144) == 256

@@ -53,6 +53,9 @@ def test_add_norm_forward_and_backward(cabi, oracle, gpu, dtype, shape, mixed):
     xg, rg, dyg, ghg, gg, bg = (t.to(gpu) for t in (x, res, dy, gh, gamma, beta))
     h_cpu = x + res  # an elementwise add in the row dtype: one rounding of the float32 sum
     wtol = gamma.dtype
+    # 16-bit rows of 4096 / 5120 elements: the plain forward takes an exact two-pack layout
+    # (5120: 320 lanes x 2 packs) that the fused add does not have (256 lanes x 3 packs there)
+    same_layout = not (dtype != torch.float32 and N == 5120)
     for rms in (False, True):
         what = "rms_norm" if rms else "layer_norm"
         if rms:
@@ -66,12 +69,19 @@ def test_add_norm_forward_and_backward(cabi, oracle, gpu, dtype, shape, mixed):
             oy, oh, om, orr = oracle.add_layer_norm_fwd(to_np32(x), to_np32(res), (N,),
                                                         to_np32(gamma), to_np32(beta), 1e-5,
                                                         NAME[dtype])
-            assert torch.equal(mean, umean)
+            if same_layout:
+                assert torch.equal(mean, umean)
+            else:
+                assert_close(mean, umean, torch.float32, what + " mean, fused against plain on h")
             assert_close(mean, om.reshape(-1), dtype, what + " mean")
         assert torch.equal(h.cpu(), h_cpu), what + ": h is not the elementwise sum"
         assert torch.equal(torch.from_numpy(oh), h_cpu.float())
-        # the fused kernel and the plain kernel on h share their arithmetic
-        assert torch.equal(rstd, urstd), what
+        # the fused kernel and the plain kernel on h share their arithmetic (and, on the same
+        # lane layout, the order of their sums: bit-equal statistics)
+        if same_layout:
+            assert torch.equal(rstd, urstd), what
+        else:
+            assert_close(rstd, urstd, torch.float32, what + " rstd, fused against plain on h")
         assert_same_arithmetic(y, uy, what + " y, fused against plain on h")
         assert_close(y, oy, dtype, what + " y")
         assert_close(rstd, orr.reshape(-1), dtype, what + " rstd")

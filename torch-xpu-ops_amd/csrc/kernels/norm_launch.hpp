@@ -46,11 +46,34 @@ inline bool norm_fwd_can_split(const Plan& plan, const NormFwdArgs& a) {
          regions_disjoint(a.y, ybytes, a.h, xbytes);
 }
 
+// The exact two-pack forward layouts (kNormFwdExact): entry I of the table, if the plan names it.
+template <class T, class WT, bool RMS, int I>
+inline bool launch_norm_fwd_exact_at(const Plan& plan, const NormFwdArgs& a, hipStream_t stream) {
+  constexpr NormFwdExactLayout l = kNormFwdExact[I];
+  if constexpr (sizeof(T) == 2) {
+    if (plan.G == l.G && plan.block == l.block) {
+      hipLaunchKernelGGL((norm_fwd_exact_kernel<T, WT, l.G, l.block, RMS>),
+                         dim3((unsigned)plan.grid), dim3(l.block), 0, stream, (const T*)a.x,
+                         (const WT*)a.gamma, (const WT*)a.beta, (T*)a.y, a.mean, a.rstd, a.M, a.N,
+                         a.eps);
+      return true;
+    }
+  }
+  return false;
+}
+
 template <class T, class WT, bool RMS, class TY, bool ADD>
 int launch_norm_fwd(const Plan& plan, const NormFwdArgs& a, hipStream_t stream) {
   const T* res = ADD ? (const T*)a.res : nullptr;
   T* h = ADD ? (T*)a.h : nullptr;
-  if (plan.resident) {
+  if (plan.resident && plan.exact_depth > 0) {
+    static_assert(kNormFwdExactCount == 2, "one call per table entry below");
+    bool launched = false;
+    if constexpr (!ADD && std::is_same<T, TY>::value)
+      launched = launch_norm_fwd_exact_at<T, WT, RMS, 0>(plan, a, stream) ||
+                 launch_norm_fwd_exact_at<T, WT, RMS, 1>(plan, a, stream);
+    if (!launched) return (int)hipErrorInvalidConfiguration;
+  } else if (plan.resident) {
     NormFwdCtx<T, WT, RMS> ctx{plan, a, stream};
     const bool launched =
         plan.fast

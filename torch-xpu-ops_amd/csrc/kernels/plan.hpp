@@ -58,8 +58,9 @@ struct Plan {
   // a layout was asked for by override: kernels chosen by other means than the
   // layout (softmax of short ragged rows through LDS) stand back
   bool forced = false;
-  // norm backward on an exact two-pack layout (norm_bwd_exact_kernel): row blocks a
-  // lane keeps in flight, itself included; 0 = the general resident kernel
+  // norm backward / forward on an exact two-pack layout (norm_bwd_exact_kernel,
+  // norm_fwd_exact_kernel): row blocks a lane keeps in flight, itself included (the
+  // forward: 1); 0 = the general resident kernel
   int exact_depth = 0;
 };
 
@@ -222,6 +223,27 @@ constexpr int norm_bwd_exact_index(int esize, int64_t packs, int64_t M, bool lay
   for (int i = 0; i < kNormBwdExactCount; ++i) {
     const NormBwdExactLayout& l = kNormBwdExact[i];
     if (packs == 2 * (int64_t)l.G && (layer_norm || l.rms_too) && M % (l.block / l.G) == 0)
+      return i;
+  }
+  return -1;
+}
+// Exact two-pack layouts of the 16-bit norm forward (norm_fwd_exact_kernel): lanes,
+// workgroup threads, resident workgroups a compute unit.  Hidden 4096 and 5120, where
+// it measured 2-5 % ahead of the general resident kernel; not 8192.
+struct NormFwdExactLayout {
+  int G, block, bpc;
+};
+constexpr NormFwdExactLayout kNormFwdExact[] = {{256, 512, 2}, {320, 320, 3}};
+constexpr int kNormFwdExactCount = (int)(sizeof(kNormFwdExact) / sizeof(kNormFwdExact[0]));
+// (up to 128 row blocks a workgroup: at 262144 rows of 4096 the resident grid runs
+// at 68 % where the general kernel's grid, which grows with the rows, reaches 75 %)
+constexpr int kNormFwdExactMaxIters = 128;
+constexpr int norm_fwd_exact_index(int esize, int64_t packs, int64_t M, int num_cus) {
+  if (esize != 2) return -1;
+  for (int i = 0; i < kNormFwdExactCount; ++i) {
+    const int rpb = kNormFwdExact[i].block / kNormFwdExact[i].G;
+    if (packs == 2 * (int64_t)kNormFwdExact[i].G && M % rpb == 0 &&
+        M / rpb <= (int64_t)num_cus * kNormFwdExact[i].bpc * kNormFwdExactMaxIters)
       return i;
   }
   return -1;
@@ -575,6 +597,17 @@ inline int make_plan(OpClass oc, int64_t M, int64_t N, int esize, int num_cus, c
       p.V = V;
       p.block = block;
       p.rpb = p.block / G;
+      // 16-bit forward rows likewise (plain calls: no residual add, no output cast)
+      if (oc == OC_NORM_FWD && p.fast && !fused_add && !p.forced && ov.bpc == 0) {
+        const int xi = norm_fwd_exact_index(esize, packs, M, num_cus);
+        if (xi >= 0) {
+          p.G = kNormFwdExact[xi].G;
+          p.V = 2;
+          p.block = kNormFwdExact[xi].block;
+          p.rpb = p.block / p.G;
+          p.exact_depth = 1;
+        }
+      }
       // 16-bit backward rows that fill a two-pack layout of whole wavefronts
       if (oc == OC_NORM_BWD && p.fast && want_dx && !p.forced) {
         const int xi = norm_bwd_exact_index(esize, packs, M, layer_norm);
@@ -648,6 +681,10 @@ inline int make_plan(OpClass oc, int64_t M, int64_t N, int esize, int num_cus, c
       const int64_t cap = (int64_t)num_cus * (p.block == 512 ? 2 : 3);
       if (nrb <= cap * 32) grid = cap;
     }
+  }
+  if (oc == OC_NORM_FWD && p.resident && p.exact_depth > 0) {
+    const int xi = norm_fwd_exact_index(esize, packs, M, num_cus);
+    grid = (int64_t)num_cus * kNormFwdExact[xi].bpc;
   }
   // Rows whose weights are not held gain nothing from a workgroup that walks
   // several rows: one workgroup a row (8192 rows of 40960 bf16: LayerNorm 253 ->
