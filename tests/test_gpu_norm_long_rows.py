@@ -214,6 +214,9 @@ def test_backward_with_dgamma_sums_in_lds(cabi, oracle, gpu, dtype, mixed):
             # (the RMSNorm with 16-bit weights holds rows of up to 2560 packs in registers alone,
             # on 512 lanes x 5 packs)
             want = (1, 512, 5) if (N <= 20480 and not mixed) else (1, 1024, V)
+            # with fp32 weights, rows that fill a layout of whole wavefronts exactly take it
+            if mixed:
+                want = {18432: (1, 768, 3), 20480: (1, 640, 4)}.get(N, want)
             assert (p["resident"], p["lanes_per_row"], p["packs_per_lane"]) == want, p
             p = cabi.plan(cabi.OP_LAYER_NORM_BWD, M, N, code, wcode)
             # the LayerNorm backward with four packs a lane keeps the multi-pass kernels

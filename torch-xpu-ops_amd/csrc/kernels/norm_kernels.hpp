@@ -1101,10 +1101,10 @@ norm_bwd_resident_kernel(const T* __restrict__ dy, const T* __restrict__ x, cons
 }
 
 // ---------------------------------------------------------------------------
-// The same backward for 16-bit rows that fill a two-pack layout exactly: N ==
-// G * V * E with G a whole number of wavefronts (not necessarily a power of two:
-// hidden 5120 is 320 lanes x 2 packs, 7168 is 448 x 2), every row slot of every
-// row block holds a row (M % (BLOCK / G) == 0), and dx is written.
+// The same backward for 16-bit rows that fill a layout exactly: N == G * V * E
+// with G a whole number of wavefronts (not necessarily a power of two: hidden 5120
+// is 320 lanes x 2 packs, 7168 is 448 x 2, 18432 is 768 x 3), every row slot of
+// every row block holds a row (M % (BLOCK / G) == 0), and dx is written.
 //
 // No load and no store of the row loop is conditional.  In the kernel above a
 // store sits behind a branch on the execution mask; the compiler cannot know

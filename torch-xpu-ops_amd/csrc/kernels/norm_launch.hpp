@@ -134,9 +134,10 @@ struct NormBwdLauncher {
 template <class T, class WT, bool RMS, bool ADD, int I>
 inline bool launch_norm_bwd_exact_at(const Plan& plan, const NormBwdArgs& a, hipStream_t stream) {
   constexpr NormBwdExactLayout l = kNormBwdExact[I];
-  if constexpr (sizeof(T) == 2 && (!RMS || l.rms_too)) {
-    if (plan.G == l.G && plan.block == l.block && plan.exact_depth == l.depth) {
-      hipLaunchKernelGGL((norm_bwd_exact_kernel<T, WT, l.G, 2, l.block, RMS, ADD, l.depth>),
+  if constexpr (sizeof(T) == 2 &&
+                norm_bwd_exact_serves(l, !RMS, sizeof(WT) > sizeof(T), ADD)) {
+    if (plan.G == l.G && plan.V == l.V && plan.block == l.block && plan.exact_depth == l.depth) {
+      hipLaunchKernelGGL((norm_bwd_exact_kernel<T, WT, l.G, l.V, l.block, RMS, ADD, l.depth>),
                          dim3((unsigned)plan.grid), dim3(l.block), 0, stream, (const T*)a.dy,
                          (const T*)a.x, (const T*)a.dres, a.mean, a.rstd, (const WT*)a.gamma,
                          (T*)a.dx, a.part_dg, a.part_db, a.M, a.N);
@@ -156,9 +157,9 @@ int launch_norm_bwd(const Plan& plan, const NormBwdArgs& a, hipStream_t stream) 
   const bool want_cols = a.part_dg != nullptr;
   const T* dres = ADD ? (const T*)a.dres : nullptr;
   if (plan.resident && plan.exact_depth > 0) {
-    static_assert(kNormBwdExactCount == 7, "one index per table entry below");
-    if (a.dx == nullptr ||
-        !launch_norm_bwd_exact<T, WT, RMS, ADD>(plan, a, stream, ilist<0, 1, 2, 3, 4, 5, 6>{}))
+    static_assert(kNormBwdExactCount == 11, "one index per table entry below");
+    if (a.dx == nullptr || !launch_norm_bwd_exact<T, WT, RMS, ADD>(
+                               plan, a, stream, ilist<0, 1, 2, 3, 4, 5, 6, 7, 8, 9, 10>{}))
       return (int)hipErrorInvalidConfiguration;
   } else if (plan.resident) {
     NormBwdCtx<T, WT, RMS> ctx{plan, a, stream};

@@ -203,26 +203,52 @@ constexpr bool norm_bwd_sums_in_lds(int esize, int G, int V, bool fast) {
 constexpr bool norm_bwd_half_lanes_five(int esize, int wsize, int G, int V, bool rms, bool add) {
   return esize == 2 && wsize == 2 && G == 512 && V == 5 && rms && !add;
 }
-// Exact two-pack layouts of the 16-bit norm backward (norm_bwd_exact_kernel): a row
-// of `packs` = 2 * G packs on G lanes, G a whole number of wavefronts.  The table is
+// Exact layouts of the 16-bit norm backward (norm_bwd_exact_kernel): a row of
+// `packs` = V * G packs on G lanes, G a whole number of wavefronts.  The table is
 // what measured faster than the general resident kernel on MI355X (see the kernel):
-// lanes, workgroup threads, row blocks in flight (1 = no prefetch), and whether the
-// RMSNorm takes it too (at 896 and 1024 lanes its general kernel already runs this
-// layout at the same speed).
+// lanes, packs a lane, workgroup threads, row blocks in flight (1 = no prefetch),
+// and which calls take it -- LayerNorm / RMSNorm, weights in the row dtype / in
+// float32 beside 16-bit rows, with the residual gradient fused in or not.  Two packs
+// a lane serve hidden sizes up to 16384; three and four packs a lane keep rows of
+// 9216, 18432, 20480 and 24576 elements in registers where the general kernel needs
+// its dgamma sums in LDS (bf16 rows x 8192, LayerNorm 18432: 199 -> 165 us, with fp32
+// weights 231 -> 166 us; 24576: 258 -> 222 us; RMSNorm with fp32 weights 18432 185 ->
+// 158 us, 20480 206 -> 181 us, 24576 231 -> 212 us).
+constexpr unsigned kExactLN = 1, kExactLNWide = 2, kExactRMS = 4, kExactRMSWide = 8,
+                   kExactAdd = 16;  // (kExactAdd: also with the fused residual gradient)
+constexpr unsigned kExactAll = kExactLN | kExactLNWide | kExactRMS | kExactRMSWide;
 struct NormBwdExactLayout {
-  int G, block, depth;
-  bool rms_too;
+  int G, V, block, depth;
+  unsigned calls;
 };
 constexpr NormBwdExactLayout kNormBwdExact[] = {
-    {128, 512, 2, true}, {256, 512, 3, true},  {320, 640, 2, true},   {448, 448, 2, true},
-    {512, 512, 3, true}, {896, 896, 1, false}, {1024, 1024, 1, false}};
+    {128, 2, 512, 2, kExactAll | kExactAdd},
+    {256, 2, 512, 3, kExactAll | kExactAdd},
+    {320, 2, 640, 2, kExactAll | kExactAdd},
+    {448, 2, 448, 2, kExactAll | kExactAdd},
+    {512, 2, 512, 3, kExactAll | kExactAdd},
+    // (at 896 and 1024 lanes the RMSNorm's general kernel already runs this layout as fast)
+    {896, 2, 896, 1, kExactLN | kExactLNWide | kExactAdd},
+    {1024, 2, 1024, 1, kExactLN | kExactLNWide | kExactAdd},
+    {384, 3, 384, 2, kExactAll},
+    {768, 3, 768, 1, kExactLN | kExactLNWide | kExactRMSWide},
+    {640, 4, 640, 1, kExactRMSWide},
+    {1024, 3, 1024, 1, kExactAll}};
 constexpr int kNormBwdExactCount = (int)(sizeof(kNormBwdExact) / sizeof(kNormBwdExact[0]));
+constexpr bool norm_bwd_exact_serves(const NormBwdExactLayout& l, bool layer_norm,
+                                     bool wide_weights, bool fused_add) {
+  const unsigned want = layer_norm ? (wide_weights ? kExactLNWide : kExactLN)
+                                   : (wide_weights ? kExactRMSWide : kExactRMS);
+  return (l.calls & want) != 0 && (!fused_add || (l.calls & kExactAdd) != 0);
+}
 // Index into kNormBwdExact of the layout that serves such a call, or -1.
-constexpr int norm_bwd_exact_index(int esize, int64_t packs, int64_t M, bool layer_norm) {
-  if (esize != 2 || packs % 2 != 0) return -1;
+constexpr int norm_bwd_exact_index(int esize, int64_t packs, int64_t M, bool layer_norm,
+                                   bool wide_weights, bool fused_add) {
+  if (esize != 2) return -1;
   for (int i = 0; i < kNormBwdExactCount; ++i) {
     const NormBwdExactLayout& l = kNormBwdExact[i];
-    if (packs == 2 * (int64_t)l.G && (layer_norm || l.rms_too) && M % (l.block / l.G) == 0)
+    if (packs == (int64_t)l.V * l.G && norm_bwd_exact_serves(l, layer_norm, wide_weights, fused_add) &&
+        M % (l.block / l.G) == 0)
       return i;
   }
   return -1;
@@ -610,10 +636,10 @@ inline int make_plan(OpClass oc, int64_t M, int64_t N, int esize, int num_cus, c
       }
       // 16-bit backward rows that fill a two-pack layout of whole wavefronts
       if (oc == OC_NORM_BWD && p.fast && want_dx && !p.forced) {
-        const int xi = norm_bwd_exact_index(esize, packs, M, layer_norm);
+        const int xi = norm_bwd_exact_index(esize, packs, M, layer_norm, wide_weights, fused_add);
         if (xi >= 0) {
           p.G = kNormBwdExact[xi].G;
-          p.V = 2;
+          p.V = kNormBwdExact[xi].V;
           p.block = kNormBwdExact[xi].block;
           p.rpb = p.block / p.G;
           p.exact_depth = kNormBwdExact[xi].depth;
