@@ -287,7 +287,9 @@ def test_group_norm_rows_take_512_lanes_while_two_workgroups_fit(cabi):
     assert lay(0, 192, BF) == (512, 6) and lay(1, 192, BF) == (512, 6)
     assert lay(0, 224, BF) == (512, 7) and lay(1, 224, BF) == (512, 7)
     assert lay(0, 256, BF) == (512, 8) and lay(1, 256, BF) == (1024, 4)
-    assert lay(0, 320, BF) == (512, 10) and lay(1, 320, BF) == (1024, 5)
+    assert lay(0, 320, BF) == (512, 10) and lay(1, 320, F32) is None
+    # (16-bit rows of exactly 512 x 10 packs in whole-wavefront channels: the exact kernels)
+    assert lay(1, 320, BF) == (512, 10) and lay(1, 320, cabi.F16) == (512, 10)
     assert lay(0, 352, BF) == (1024, 6) and lay(1, 352, BF) == (1024, 6)
     assert lay(0, 96, F32) == (512, 6) and lay(1, 96, F32) == (512, 6)
     assert lay(0, 160, F32) == (512, 10) and lay(1, 128, F32) == (1024, 4)

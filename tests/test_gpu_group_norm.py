@@ -37,7 +37,11 @@ SHAPES = [(2, 4, (), 2), (64, 32, (), 4), (256, 32, (), 4), (64, 32, (16,), 4), 
           # straddling kernels take) and 520 (general kernels)
           (4, 64, (7, 7), 8), (2, 64, (14, 14), 2), (2, 128, (7, 7), 2), (2, 130, (7, 7), 2),
           (1, 16, (27, 27), 1), (3, 8, (9,), 1), (2, 24, (3, 4), 3), (70, 32, (7, 7), 4),
-          (2, 512, (7, 7), 1), (1, 1040, (7, 7), 2)]
+          (2, 512, (7, 7), 1), (1, 1040, (7, 7), 2),
+          # 16-bit rows that fill an exact layout, channels of whole runs of 64 packs (32x32 and
+          # 64x64 maps with 10, 20, 30 and 60 channels a group; 10 at 64x64 is above): 256 x 5
+          # (backward), 512 x 5, 768 x 5, 960 x 8
+          (3, 10, (32, 32), 1), (2, 40, (32, 32), 2), (2, 60, (32, 32), 2), (2, 120, (32, 32), 2)]
 CASES = load_golden("aten_cpu_group_norm.npz")
 
 
@@ -173,6 +177,85 @@ def test_edge_cases(cabi, oracle, gpu):
     e = torch.empty(0, 2, device=gpu)
     y, mean, rstd = cabi.group_norm_fwd(e, None, None, 1, 1e-5)
     assert y.shape == (0, 2) and mean.shape == (0, 1)
+
+
+def test_exact_layouts_many_rows_absent_weights_and_special_rows(cabi, oracle, gpu):
+    """The 16-bit kernels for rows that fill a layout of whole wavefronts exactly, channels of whole
+    runs of 64 packs (gn_fwd_exact_kernel / gn_bwd_exact_kernel): more rows than the resident grid
+    has workgroups, weights absent, misaligned weight pointers (a scalar load takes the aligned word
+    around a 16-bit weight), constant and non-finite rows, dX alone and the channel sums alone (the
+    latter is the general kernel's: the two must agree), run-to-run determinism."""
+    bf = torch.bfloat16
+    # [25, 640, 32, 32] / 32: 800 rows of 512 x 5 packs (forward grid 768, backward 512);
+    # [66, 320, 32, 32] / 32: 2112 rows of 256 x 5 packs (backward grid 2048; general forward)
+    for (N, C, sp, G, lay) in ((25, 640, (32, 32), 32, (512, 5)), (66, 320, (32, 32), 32, (256, 5))):
+        HxW = _hxw(sp)
+        for bwd in (0, 1):
+            p = cabi.group_norm_plan(bwd, N, C, HxW, G, cabi.BF16)
+            if bwd or lay != (256, 5):
+                assert (p["lanes_per_row"], p["packs_per_lane"]) == lay and p["grid_blocks"] < N * G, p
+        print("case group_norm exact layouts, many rows", (N, C, sp, G), flush=True)
+        x, dy, gamma, beta = _mk(N, C, sp, bf, 75)
+        x[1, :C // G] = 2.5                      # a constant row
+        x[2, C // G, 3, 3] = float("inf")        # a row with an inf: NaN statistics
+        x[3, 2 * (C // G), 0, 1] = float("nan")
+        xg, dyg, gg, bg = x.to(gpu), dy.to(gpu), gamma.to(gpu), beta.to(gpu)
+        y, mean, rstd = cabi.group_norm_fwd(xg, gg, bg, G, 1e-5)
+        oy, om, orr = oracle.group_norm_fwd(to_np32(x), G, to_np32(gamma), to_np32(beta), 1e-5)
+        oy = torch.as_tensor(oy).float().reshape(x.shape)
+        orr = torch.as_tensor(orr).float().reshape(N, G)
+        fin = torch.isfinite(oy)
+        assert torch.equal(torch.isfinite(y.cpu().float()), fin)
+        assert_close(torch.where(fin, y.cpu().float(), 0), torch.where(fin, oy, 0), bf, "y")
+        assert torch.equal(y[1, :C // G].cpu(), beta[:C // G].view(-1, 1, 1).expand(C // G, *sp))
+        assert bool(torch.isnan(mean[2, 1])) and bool(torch.isnan(rstd[2, 1])) and bool(torch.isnan(mean[3, 2]))
+        okr = torch.isfinite(rstd.cpu().float())
+        assert torch.equal(okr, torch.isfinite(orr))
+        assert_close(torch.where(okr, rstd.cpu().float(), 0), torch.where(okr, orr, 0), bf, "rstd")
+        # backward on finite inputs
+        x[2, C // G, 3, 3] = 1.0
+        x[3, 2 * (C // G), 0, 1] = -1.0
+        xg = x.to(gpu)
+        y, mean, rstd = cabi.group_norm_fwd(xg, gg, bg, G, 1e-5)
+        dx, dg, db = cabi.group_norm_bwd(dyg, xg, mean, rstd, gg, G)
+        odx, odg, odb = oracle.group_norm_bwd(to_np32(dy), to_np32(x), G, to_np32(mean), to_np32(rstd),
+                                              to_np32(gamma))
+        assert_close(dx, odx, bf, "dx")
+        assert_close(dg, odg, bf, "dgamma")
+        assert_close(db, odb, bf, "dbeta")
+        dx1, none1, none2 = cabi.group_norm_bwd(dyg, xg, mean, rstd, gg, G, want=(True, False, False))
+        assert none1 is None and none2 is None and torch.equal(dx1, dx)
+        none0, dg1, db1 = cabi.group_norm_bwd(dyg, xg, mean, rstd, gg, G, want=(False, True, True))
+        assert none0 is None
+        assert_close(dg1, odg, bf, "dgamma alone")
+        assert_close(db1, odb, bf, "dbeta alone")
+        dx2, dg2, db2 = cabi.group_norm_bwd(dyg, xg, mean, rstd, gg, G)
+        assert torch.equal(dx2, dx) and torch.equal(dg2, dg) and torch.equal(db2, db)
+    # absent weights == ones / zeros, and weights that start on an odd 16-bit element
+    for wdt in (bf, torch.float32):
+        N, C, sp, G = 3, 40, (32, 32), 2
+        x, dy, gamma, beta = _mk(N, C, sp, bf, 76, wdt)
+        xg, dyg = x.to(gpu), dy.to(gpu)
+        ones, zeros = torch.ones(C, device=gpu, dtype=wdt), torch.zeros(C, device=gpu, dtype=wdt)
+        y1, m1, r1 = cabi.group_norm_fwd(xg, ones, zeros, G, 1e-5)
+        y2, m2, _ = cabi.group_norm_fwd(xg, ones, None, G, 1e-5)
+        assert torch.equal(y1, y2) and torch.equal(m1, m2)
+        if wdt == bf:
+            y0, m0, r0 = cabi.group_norm_fwd(xg, None, None, G, 1e-5)
+            assert torch.equal(y0, y1) and torch.equal(m0, m1) and torch.equal(r0, r1)
+        dx0, _, _ = cabi.group_norm_bwd(dyg, xg, m1, r1, None, G, want=(True, False, False))
+        dx1, _, _ = cabi.group_norm_bwd(dyg, xg, m1, r1, ones, G)
+        assert torch.equal(dx0, dx1)
+        go, bo = offset_view(gamma.to(gpu), 1), offset_view(beta.to(gpu), 1)
+        ya, ma, ra = cabi.group_norm_fwd(xg, gamma.to(gpu), beta.to(gpu), G, 1e-5)
+        yb, mb, rb = cabi.group_norm_fwd(xg, go, bo, G, 1e-5)
+        assert torch.equal(ya, yb) and torch.equal(ma, mb)
+        # statistics that start on an odd element as well
+        da = cabi.group_norm_bwd(dyg, xg, ma, ra, gamma.to(gpu), G)
+        dbb = cabi.group_norm_bwd(dyg, xg, offset_view(ma.reshape(-1), 1).reshape(ma.shape),
+                                  offset_view(ra.reshape(-1), 1).reshape(ra.shape), go, G)
+        for u, v in zip(da, dbb):
+            assert torch.equal(u, v)
 
 
 @pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16], ids=str)

@@ -418,10 +418,29 @@ int group_dims(int64_t N, int64_t C, int64_t HxW, int64_t groups, GroupDims* out
 
 // The general kernels are taken when neither every pack lies in one channel nor
 // the straddling kernels apply (gn_mode, plan.hpp).
-int group_plan(OpClass oc, int op, const GroupDims& d, int64_t HxW, int esize, Plan* plan) {
+int group_plan(OpClass oc, int op, const GroupDims& d, int64_t HxW, int esize, Plan* plan,
+               bool want_dx = true) {
   const int E = 16 / esize;
-  return make_plan(oc, d.rows, d.L, esize, current_num_cus(), g_override[op], false, plan,
-                   gn_mode(d.L, HxW, d.D, E) == kGnGeneral);
+  const Override& ov = g_override[op];
+  const int num_cus = current_num_cus();
+  if (int e = make_plan(oc, d.rows, d.L, esize, num_cus, ov, false, plan,
+                        gn_mode(d.L, HxW, d.D, E) == kGnGeneral))
+    return e;
+  // 16-bit rows that fill an exact layout and whose channels are whole runs of 64 packs
+  const bool backward = oc == OC_GROUP_BWD;
+  if (plan->resident && plan->fast && !plan->forced && ov.bpc == 0 && (want_dx || !backward)) {
+    const int xi = group_exact_index(backward, esize, d.rows, d.L, HxW, d.D);
+    if (xi >= 0) {
+      const GroupExactLayout& l = kGroupExact[xi];
+      plan->G = plan->block = l.G;
+      plan->V = l.V;
+      plan->rpb = 1;
+      plan->exact_depth = 1;
+      const int64_t cap = (int64_t)num_cus * (backward ? l.bpc_bwd : l.bpc_fwd);
+      plan->grid = d.rows < cap ? d.rows : cap;
+    }
+  }
+  return 0;
 }
 
 int softmax_mode_flags(int mode, bool forward, int* flags) {
@@ -649,7 +668,8 @@ int mi355x_group_norm_bwd(const void* dy, const void* x, const void* mean, const
   if (!dx && !want_cols) return 0;
   if (!dy || !x || !mean || !rstd) return ROWNORM_ERR_NULL;
   Plan plan;
-  if (int e = group_plan(OC_GROUP_BWD, ROWNORM_OP_GROUP_NORM_BWD, d, HxW, esize_of(xd), &plan))
+  if (int e = group_plan(OC_GROUP_BWD, ROWNORM_OP_GROUP_NORM_BWD, d, HxW, esize_of(xd), &plan,
+                         dx != nullptr))
     return e;
   float* part_dg = nullptr;
   float* part_db = nullptr;

@@ -96,6 +96,46 @@ __device__ __forceinline__ void keep_packed(Pack<T, E>& p) {
   }
 }
 
+// Loads from wavefront-uniform addresses of memory that no kernel writes while
+// it runs (inputs, weights, saved statistics).  Through the constant address
+// space the compiler issues them on the scalar unit, where they neither take a
+// vector register nor count among the vector memory operations a row loop waits
+// for; a plain load from a uniform address becomes a vector load as soon as a
+// barrier precedes it, because the barrier's fence may have changed any memory.
+template <class U>
+__device__ __forceinline__ U uniform_load(const void* p) {
+  return *(const __attribute__((address_space(4))) U*)(uintptr_t)p;
+}
+
+// Element i (wavefront-uniform) of an array of 16- or 32-bit values: the aligned
+// 32-bit word that holds it is loaded -- the scalar unit has no 16-bit loads --
+// and value() picks the element out of it.  The word lies within the 4 bytes
+// around the element, so nothing beyond the array's last word is touched.
+template <class WT>
+struct UniformElem {
+  uint32_t word;
+  uint32_t shift;
+  __device__ __forceinline__ static UniformElem load(const WT* w, int64_t i) {
+    const char* p = reinterpret_cast<const char*>(w + i);
+    UniformElem r;
+    r.shift = 0;
+    if constexpr (sizeof(WT) == 2) {
+      const uint32_t odd = (uint32_t)(reinterpret_cast<uintptr_t>(p) & 2);
+      p -= odd;
+      r.shift = odd * 8u;
+    }
+    r.word = uniform_load<uint32_t>(p);
+    return r;
+  }
+  __device__ __forceinline__ float value() const {
+    if constexpr (sizeof(WT) == 4) {
+      return __builtin_bit_cast(float, word);
+    } else {
+      return (float)__builtin_bit_cast(WT, (uint16_t)(word >> shift));
+    }
+  }
+};
+
 // The lane index as a value the compiler cannot trace back to threadIdx, and
 // that exists only once `after` does: the pack offsets derived from it are then
 // computed where they are used (after a reduction, say) instead of ahead of the

@@ -236,6 +236,92 @@ gn_fwd_resident_kernel(const T* __restrict__ x, const WT* __restrict__ gamma,
   }
 }
 
+// ---------------------------------------------------------------------------
+// The same forward for 16-bit rows that fill a layout of whole wavefronts exactly
+// (L == G * V * E, one row a workgroup) and whose channels are whole runs of 64
+// packs (HxW / E a multiple of 64, a diffusion UNet's 64x64 and 32x32 maps): the
+// 64 packs a wavefront moves with one instruction lie in one channel, so a
+// channel's weights are two scalar loads, the row pointer is scalar arithmetic, the
+// head of the row (the centre of the sums) is a scalar load, and no access is
+// conditional.  Arithmetic is that of gn_fwd_resident_kernel for the same layout,
+// bit for bit.  Measured on one MI355X, bf16 [64, 320, 64, 64] with 32 groups (2048
+// rows of 40960 elements on 512 lanes x 10 packs, two workgroups a compute unit):
+// 61.6 -> 58.6 us.  Requesting the next row ahead of the current one (a second and
+// third register set) measured the same or slower at every layout tried.
+template <class T, class WT, int G, int V>
+__global__ void __launch_bounds__(G)
+gn_fwd_exact_kernel(const T* __restrict__ x, const WT* __restrict__ gamma,
+                    const WT* __restrict__ beta, T* __restrict__ y, WT* __restrict__ mean,
+                    WT* __restrict__ rstd, int64_t rows, GroupShape s, float eps) {
+  constexpr int E = elems_per_pack<T>::value;
+  static_assert(sizeof(T) == 2 && G % 64 == 0, "16-bit rows on whole wavefronts");
+  __shared__ float red[reduce_lds_floats<G, G, 2>::value];
+  int phase = 0;
+  const float fL = (float)s.L;
+  const float inv_l = 1.0f / fL;
+  const int wave = __builtin_amdgcn_readfirstlane((int)(threadIdx.x >> 6));
+  const unsigned S = (unsigned)(s.HxW / E);  // packs per channel
+  int chl[V];                                // channel (within the group) of pack c
+#pragma unroll
+  for (int c = 0; c < V; ++c) chl[c] = (int)((unsigned)(c * G + wave * 64) / S);
+  const uint32_t loff = (uint32_t)(threadIdx.x * E * (int)sizeof(T));
+  auto at = [](const T* p, uint32_t off) {
+    return reinterpret_cast<const T*>(reinterpret_cast<const char*>(p) + off);
+  };
+  // absent weights: the loads go to memory that exists and their values are not used
+  const bool has_g = gamma != nullptr, has_b = beta != nullptr;
+  const WT* gsrc = has_g ? gamma : reinterpret_cast<const WT*>(x);
+  const WT* bsrc = has_b ? beta : reinterpret_cast<const WT*>(x);
+  for (int64_t row = blockIdx.x; row < rows; row += gridDim.x) {
+    const int ch0 = (int)((uint32_t)row % (uint32_t)s.groups) * s.D;
+    const T* xr = x + row * (int64_t)s.L;
+    const uint64_t head = uniform_load<uint64_t>(xr);
+    UniformElem<WT> wg[V], wb[V];
+    Pack<T, E> xp[V];
+#pragma unroll
+    for (int c = 0; c < V; ++c) {
+      wg[c] = UniformElem<WT>::load(gsrc, ch0 + chl[c]);
+      wb[c] = UniformElem<WT>::load(bsrc, ch0 + chl[c]);
+      xp[c] = Pack<T, E>::load_stream(at(xr + c * G * E, loff));
+    }
+    const float a = (float)__builtin_bit_cast(T, (uint16_t)head);
+    const float b = (float)__builtin_bit_cast(T, (uint16_t)(head >> 16));
+    const float c3 = (float)__builtin_bit_cast(T, (uint16_t)(head >> 32));
+    const float mean0 = fmaxf(fminf(a, b), fminf(fmaxf(a, b), c3));
+    float acc[2] = {0.0f, 0.0f};
+#pragma unroll
+    for (int c = 0; c < V; ++c) {
+      keep_packed(xp[c]);
+#pragma unroll
+      for (int i = 0; i < E; ++i) {
+        const float d = xp[c].get(i) - mean0;
+        acc[0] += d;
+        acc[1] = fmaf(d, d, acc[1]);
+      }
+    }
+    group_allreduce<G, G, 2, SumOp>(acc, red, phase);
+    const float m1 = row_mean_of<T>(acc[0], fL, inv_l);
+    float var = row_mean_of<T>(acc[1] - acc[0] * m1, fL, inv_l);
+    var = var < 0.0f ? 0.0f : var;  // a select: a NaN row keeps NaN statistics
+    const float rs = row_rstd_of<T>(var + eps);
+    if (threadIdx.x == 0) {
+      if (mean) mean[row] = (WT)(rs == rs ? mean0 + m1 : rs);  // NaN variance: NaN mean
+      if (rstd) rstd[row] = (WT)rs;
+    }
+    T* yr = y + row * (int64_t)s.L;
+#pragma unroll
+    for (int c = 0; c < V; ++c) {
+      keep_packed(xp[c]);
+      const float ga = (has_g ? wg[c].value() : 1.0f) * rs;
+      const float be = has_b ? wb[c].value() : 0.0f;
+      Pack<T, E> o;
+#pragma unroll
+      for (int i = 0; i < E; ++i) o.set(i, ((xp[c].get(i) - mean0) - m1) * ga + be);
+      o.store_stream(const_cast<T*>(at(yr + c * G * E, loff)));
+    }
+  }
+}
+
 // Forward for rows too long for the registers: one workgroup per row, two
 // passes over the row (statistics, normalize).  The statistics are the sums of
 // (x - k) and (x - k)^2 in float64, k = the row's first element: float32 and
@@ -505,6 +591,119 @@ gn_bwd_resident_kernel(const T* __restrict__ dy, const T* __restrict__ x,
         }
         __syncthreads();  // the staging area is reused by the next row
       }
+    }
+  }
+}
+
+// ---------------------------------------------------------------------------
+// The same backward for the rows gn_fwd_exact_kernel serves (L == G * V * E, one
+// row a workgroup, channels of whole runs of 64 packs, dx written): scalar row
+// pointers, statistics and weights, no conditional access.  The 64 packs of a
+// wavefront lie in one channel, so the sums over a pack are reduced over the
+// wavefront in registers and one lane parks them in LDS ahead of the barrier the
+// row's reduction has anyway; after it every wavefront adds the runs of each
+// channel in a fixed order and all of them write the row's D channel sums, the
+// same values to the same addresses: a store by the first wavefront only would be
+// a conditional store, and the compiler then lets the next row's loads wait for
+// it.  dx is that of gn_bwd_resident_kernel for the same layout, bit for bit; the
+// channel sums differ from it in the last bits (another order of the same terms).
+// Measured on one MI355X, bf16 [64, 320, 64, 64] with 32 groups on 512 lanes x 10
+// packs, two workgroups a compute unit: 92.7 -> 87.0 us (before the column pass).
+template <class T, class WT, int G, int V, bool COLS>
+__global__ void __launch_bounds__(G)
+gn_bwd_exact_kernel(const T* __restrict__ dy, const T* __restrict__ x,
+                    const WT* __restrict__ mean, const WT* __restrict__ rstd,
+                    const WT* __restrict__ gamma, T* __restrict__ dx,
+                    float* __restrict__ part_dg, float* __restrict__ part_db, int64_t rows,
+                    GroupShape s) {
+  constexpr int E = elems_per_pack<T>::value;
+  constexpr int NW = G / 64;
+  constexpr int UNITS = V * NW;  // runs of 64 packs in a row
+  static_assert(sizeof(T) == 2 && G % 64 == 0, "16-bit rows on whole wavefronts");
+  __shared__ float red[reduce_lds_floats<G, G, 2>::value];
+  __shared__ float stage[COLS ? 2 * UNITS * 2 : 1];  // [phase][run][dg, db]
+  int phase = 0;
+  const float fL = (float)s.L;
+  const int wave = __builtin_amdgcn_readfirstlane((int)(threadIdx.x >> 6));
+  const int lane = (int)(threadIdx.x & 63);
+  const unsigned S = (unsigned)(s.HxW / E);  // packs per channel
+  const int U = (int)(S / 64u);              // runs per channel
+  int chl[V];
+#pragma unroll
+  for (int c = 0; c < V; ++c) chl[c] = (int)((unsigned)(c * G + wave * 64) / S);
+  // the channel whose sums this lane writes; lanes beyond the row's channels repeat one
+  const int dch = lane % s.D;
+  const uint32_t loff = (uint32_t)(threadIdx.x * E * (int)sizeof(T));
+  auto at = [](const T* p, uint32_t off) {
+    return reinterpret_cast<const T*>(reinterpret_cast<const char*>(p) + off);
+  };
+  const bool has_g = gamma != nullptr;
+  const WT* gsrc = has_g ? gamma : reinterpret_cast<const WT*>(x);
+  for (int64_t row = blockIdx.x; row < rows; row += gridDim.x) {
+    const uint32_t n = (uint32_t)row / (uint32_t)s.groups;
+    const int ch0 = (int)((uint32_t)row - n * (uint32_t)s.groups) * s.D;
+    const UniformElem<WT> wmu = UniformElem<WT>::load(mean, row);
+    const UniformElem<WT> wrs = UniformElem<WT>::load(rstd, row);
+    const T* xr = x + row * (int64_t)s.L;
+    const T* gr = dy + row * (int64_t)s.L;
+    UniformElem<WT> wg[V];
+    Pack<T, E> xp[V], dp[V];
+#pragma unroll
+    for (int c = 0; c < V; ++c) {
+      wg[c] = UniformElem<WT>::load(gsrc, ch0 + chl[c]);
+      xp[c] = Pack<T, E>::load_stream(at(xr + c * G * E, loff));
+      dp[c] = Pack<T, E>::load_stream(at(gr + c * G * E, loff));
+    }
+    const float mu = wmu.value(), rs = wrs.value();
+    float ga[V];
+    float acc[2] = {0.0f, 0.0f};
+    float* st = stage + phase * (2 * UNITS);
+#pragma unroll
+    for (int c = 0; c < V; ++c) {
+      ga[c] = has_g ? wg[c].value() : 1.0f;
+      float pdg = 0.0f, pdb = 0.0f;
+#pragma unroll
+      for (int i = 0; i < E; ++i) {
+        const float gy = dp[c].get(i);
+        pdb += gy;
+        pdg = fmaf(gy, xp[c].get(i) - mu, pdg);
+      }
+      acc[0] = fmaf(pdb, ga[c], acc[0]);
+      acc[1] = fmaf(pdg * rs, ga[c], acc[1]);
+      if constexpr (COLS) {
+        const float wdg = wave_group_allreduce<64, SumOp>(pdg * rs);
+        const float wdb = wave_group_allreduce<64, SumOp>(pdb);
+        if (lane == 0) {
+          st[2 * (c * NW + wave)] = wdg;
+          st[2 * (c * NW + wave) + 1] = wdb;
+        }
+      }
+    }
+    group_allreduce<G, G, 2, SumOp>(acc, red, phase);  // (flips phase)
+    if constexpr (COLS) {
+      float ag = 0.0f, ab = 0.0f;
+      for (int u = 0; u < U; ++u) {
+        ag += st[2 * (dch * U + u)];
+        ab += st[2 * (dch * U + u) + 1];
+      }
+      const int64_t o = (int64_t)n * ((int64_t)s.groups * s.D) + ch0 + dch;
+      part_dg[o] = ag;
+      part_db[o] = ab;
+    }
+    T* dr = dx + row * (int64_t)s.L;
+    const float s1 = acc[0], s2 = acc[1];
+    const float term1 = rs / fL;
+    const float ra = rs * (s2 * term1);
+    const float cc = mu * ra - s1 * term1;
+#pragma unroll
+    for (int c = 0; c < V; ++c) {
+      keep_packed(xp[c]);
+      keep_packed(dp[c]);
+      const float gq = ga[c] * rs;
+      Pack<T, E> o;
+#pragma unroll
+      for (int i = 0; i < E; ++i) o.set(i, fmaf(xp[c].get(i), -ra, fmaf(dp[c].get(i), gq, cc)));
+      o.store_stream(const_cast<T*>(at(dr + c * G * E, loff)));
     }
   }
 }

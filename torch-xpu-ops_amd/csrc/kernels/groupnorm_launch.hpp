@@ -48,9 +48,35 @@ struct GroupNormFwdLauncher {
   };
 };
 
+// The exact layouts (kGroupExact): entry I of the table, if the plan names it.
+template <class T, class WT, int I>
+inline bool launch_group_fwd_exact_at(const Plan& plan, const GroupNormFwdArgs& a,
+                                      hipStream_t stream) {
+  constexpr GroupExactLayout l = kGroupExact[I];
+  if constexpr (sizeof(T) == 2 && l.bpc_fwd > 0) {
+    if (plan.G == l.G && plan.V == l.V) {
+      hipLaunchKernelGGL((gn_fwd_exact_kernel<T, WT, l.G, l.V>), dim3((unsigned)plan.grid),
+                         dim3(l.G), 0, stream, (const T*)a.x, (const WT*)a.gamma,
+                         (const WT*)a.beta, (T*)a.y, (WT*)a.mean, (WT*)a.rstd, a.rows,
+                         group_shape(a.L, a.HxW, a.D, a.groups, elems_per_pack<T>::value), a.eps);
+      return true;
+    }
+  }
+  return false;
+}
+template <class T, class WT, int... Is>
+inline bool launch_group_fwd_exact(const Plan& plan, const GroupNormFwdArgs& a, hipStream_t stream,
+                                   ilist<Is...>) {
+  return (launch_group_fwd_exact_at<T, WT, Is>(plan, a, stream) || ...);
+}
+
 template <class T, class WT>
 int launch_group_norm_fwd(const Plan& plan, const GroupNormFwdArgs& a, hipStream_t stream) {
-  if (plan.resident) {
+  if (plan.resident && plan.exact_depth > 0) {
+    static_assert(kGroupExactCount == 5, "one index per table entry below");
+    if (!launch_group_fwd_exact<T, WT>(plan, a, stream, ilist<0, 1, 2, 3, 4>{}))
+      return (int)hipErrorInvalidConfiguration;
+  } else if (plan.resident) {
     GroupNormFwdCtx<T, WT> ctx{plan, a, stream};
     const int mode = plan.fast ? gn_mode(a.L, a.HxW, a.D, elems_per_pack<T>::value) : kGnGeneral;
     const bool launched =
@@ -108,6 +134,34 @@ inline int gn_tpc_log2(int G, int D, int packs_per_channel) {
   return log2_of_pow2(tpc);
 }
 
+template <class T, class WT, int I>
+inline bool launch_group_bwd_exact_at(const Plan& plan, const GroupNormBwdArgs& a,
+                                      hipStream_t stream) {
+  constexpr GroupExactLayout l = kGroupExact[I];
+  if constexpr (sizeof(T) == 2 && l.bpc_bwd > 0) {
+    if (plan.G == l.G && plan.V == l.V) {
+      const GroupShape shape = group_shape(a.L, a.HxW, a.D, a.groups, elems_per_pack<T>::value);
+      if (a.part_dg != nullptr)
+        hipLaunchKernelGGL((gn_bwd_exact_kernel<T, WT, l.G, l.V, true>), dim3((unsigned)plan.grid),
+                           dim3(l.G), 0, stream, (const T*)a.dy, (const T*)a.x, (const WT*)a.mean,
+                           (const WT*)a.rstd, (const WT*)a.gamma, (T*)a.dx, a.part_dg, a.part_db,
+                           a.rows, shape);
+      else
+        hipLaunchKernelGGL((gn_bwd_exact_kernel<T, WT, l.G, l.V, false>), dim3((unsigned)plan.grid),
+                           dim3(l.G), 0, stream, (const T*)a.dy, (const T*)a.x, (const WT*)a.mean,
+                           (const WT*)a.rstd, (const WT*)a.gamma, (T*)a.dx, a.part_dg, a.part_db,
+                           a.rows, shape);
+      return true;
+    }
+  }
+  return false;
+}
+template <class T, class WT, int... Is>
+inline bool launch_group_bwd_exact(const Plan& plan, const GroupNormBwdArgs& a, hipStream_t stream,
+                                   ilist<Is...>) {
+  return (launch_group_bwd_exact_at<T, WT, Is>(plan, a, stream) || ...);
+}
+
 template <class T, class WT>
 int launch_group_norm_bwd(const Plan& plan, const GroupNormBwdArgs& a, hipStream_t stream) {
   constexpr int E = elems_per_pack<T>::value;
@@ -135,7 +189,12 @@ int launch_group_norm_bwd(const Plan& plan, const GroupNormBwdArgs& a, hipStream
     err = (int)hipGetLastError();
     if (err != 0) return err;
   }
-  if (plan.resident) {
+  if (plan.resident && plan.exact_depth > 0) {
+    GroupNormBwdArgs k = a;
+    if (!want_cols) k.part_dg = k.part_db = nullptr;
+    if (a.dx == nullptr || !launch_group_bwd_exact<T, WT>(plan, k, stream, ilist<0, 1, 2, 3, 4>{}))
+      return (int)hipErrorInvalidConfiguration;
+  } else if (plan.resident) {
     if (a.dx != nullptr || (want_cols && fused_cols)) {
       GroupNormBwdArgs k = a;
       if (!want_cols || !fused_cols) k.part_dg = k.part_db = nullptr;

@@ -58,9 +58,10 @@ struct Plan {
   // a layout was asked for by override: kernels chosen by other means than the
   // layout (softmax of short ragged rows through LDS) stand back
   bool forced = false;
-  // norm backward / forward on an exact two-pack layout (norm_bwd_exact_kernel,
+  // norm backward / forward on an exact layout (norm_bwd_exact_kernel,
   // norm_fwd_exact_kernel): row blocks a lane keeps in flight, itself included (the
-  // forward: 1); 0 = the general resident kernel
+  // forward: 1); GroupNorm on an exact layout (gn_*_exact_kernel): 1; 0 = the
+  // general resident kernel
   int exact_depth = 0;
 };
 
@@ -271,6 +272,37 @@ constexpr int norm_fwd_exact_index(int esize, int64_t packs, int64_t M, int num_
     if (packs == 2 * (int64_t)kNormFwdExact[i].G && M % rpb == 0 &&
         M / rpb <= (int64_t)num_cus * kNormFwdExact[i].bpc * kNormFwdExactMaxIters)
       return i;
+  }
+  return -1;
+}
+// Exact layouts of the 16-bit GroupNorm kernels (gn_fwd_exact_kernel,
+// gn_bwd_exact_kernel): one row a workgroup of G lanes with V packs each, for
+// rows of exactly G * V packs whose channels are whole runs of 64 packs (the
+// 64x64 and 32x32 maps of a diffusion UNet with 32 groups: 10, 20, 30, 40 and 60
+// channels a group at 32x32, 10 at 64x64).  Workgroups a compute unit of the
+// forward and of the backward grid; 0 = the general resident kernel is faster
+// (measured on one MI355X, bf16, 2048 rows; general -> exact, us:
+//   1280 packs  forward 14.2 -> 15.0 (kept general)   backward 26.4 -> 22.2
+//   2560 packs  forward 29.9 -> 29.3                  backward 49.3 -> 43.0
+//   3840 packs  forward 46.6 -> 43.8                  backward 79.4 -> 67.9
+//   5120 packs  forward 61.6 -> 58.6                  backward 96.2 -> 87.0 + 3.5
+//   7680 packs  forward 94.7 -> 90.2                  backward 140.6 -> 128.0).
+struct GroupExactLayout {
+  int G, V, bpc_fwd, bpc_bwd;
+};
+constexpr GroupExactLayout kGroupExact[] = {
+    {256, 5, 0, 8}, {512, 5, 3, 2}, {768, 5, 2, 1}, {512, 10, 2, 2}, {960, 8, 1, 1}};
+constexpr int kGroupExactCount = (int)(sizeof(kGroupExact) / sizeof(kGroupExact[0]));
+constexpr int kGroupExactMaxD = 64;  // channels a group: one lane of a wavefront each
+constexpr int group_exact_index(bool backward, int esize, int64_t rows, int64_t L, int64_t HxW,
+                                int64_t D) {
+  const int E = 8;
+  if (esize != 2 || L % E != 0 || HxW % (64 * E) != 0 || D > kGroupExactMaxD ||
+      rows > ((int64_t)1 << 31))
+    return -1;
+  for (int i = 0; i < kGroupExactCount; ++i) {
+    const GroupExactLayout& l = kGroupExact[i];
+    if (L / E == (int64_t)l.G * l.V && (backward ? l.bpc_bwd : l.bpc_fwd) > 0) return i;
   }
   return -1;
 }
