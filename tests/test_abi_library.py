@@ -235,15 +235,22 @@ def test_plan_layouts_for_hidden_sizes_that_are_not_powers_of_two(cabi):
         p = cabi.plan(op, 16383, 4096, BF, BF)
         assert (p["lanes_per_row"], p["block_threads"]) == (256, 256)
     assert lay(LF, 7168, BF) == (512, 2)                       # fills 7/8: the rule stands
-    assert lay(LB, 6144, BF) == (256, 3) and lay(RB, 6144, BF) == (256, 3)  # and the 16-bit backward from 513 packs
+    # the 16-bit backward from 513 packs: three packs a lane, or an exact layout of six wavefronts
+    assert lay(LB, 6160, BF) == (256, 4) or lay(LB, 6160, BF) == (512, 2)
+    assert lay(LB, 5632, BF) == (256, 3) and lay(RB, 5632, BF) == (256, 3)
+    assert lay(LB, 6144, BF) == (384, 2) and lay(RB, 6144, BF) == (384, 2)
     # 16-bit backward rows that are two packs on a whole number of wavefronts, where that
     # measured faster: the exact layouts (320 lanes for 5120, 448 for 7168, 1024 for the
-    # LayerNorm at 16384); an odd row count on two row slots a workgroup keeps the general kernel
+    # LayerNorm at 16384); an odd row count keeps the general kernel where the layout has two row slots a workgroup
     assert lay(LB, 5120, BF) == (320, 2) and lay(RB, 5120, BF) == (320, 2)
     assert lay(LB, 7168, BF) == (448, 2) and lay(RB, 7168, BF, F32) == (448, 2)
     assert lay(LB, 14336, BF) == (896, 2) and lay(RB, 14336, BF) == (1024, 2)
-    p = cabi.plan(LB, 16383, 5120, BF, BF)
-    assert (p["lanes_per_row"], p["packs_per_lane"]) == (256, 3)
+    p = cabi.plan(LB, 16383, 5120, BF, BF)  # (one row slot a workgroup: any row count)
+    assert (p["lanes_per_row"], p["packs_per_lane"], p["block_threads"]) == (320, 2, 320)
+    p = cabi.plan(RB, 16383, 8192, BF, BF)
+    assert (p["lanes_per_row"], p["packs_per_lane"], p["block_threads"]) == (512, 2, 512)
+    p = cabi.plan(RB, 16383, 2048, BF, BF)  # two row slots and an odd row count: the general kernel
+    assert (p["lanes_per_row"], p["packs_per_lane"], p["block_threads"]) == (128, 2, 512)
     p = cabi.plan(RB, 16384, 4096, BF, BF)
     assert (p["block_threads"], p["grid_blocks"], p["partial_rows"]) == (512, 256, 256)
     assert lay(LB, 3072, BF) == (256, 2) and lay(RB, 2560, BF) == (256, 2)  # which keeps its lanes below

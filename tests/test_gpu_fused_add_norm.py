@@ -95,7 +95,11 @@ def test_add_norm_forward_and_backward(cabi, oracle, gpu, dtype, shape, mixed):
                 y2, h2, _, rstd2 = cabi.add_layer_norm_fwd(xx, rr, gg, bg, 1e-5, h=target)
             assert h2.data_ptr() == target.data_ptr()
             assert torch.equal(h2, h) and torch.equal(y2, y) and torch.equal(rstd2, rstd), (what, over)
-        # backward: dh = norm backward at h + the gradient of the residual path
+        # backward: dh = norm backward at h + the gradient of the residual path.  (16-bit rows of
+        # 5120 and 6144 elements, and LayerNorm rows of 4096, take another lane layout -- another
+        # order of the column sums -- with the residual gradient than without: there the two
+        # are each held to the oracle, below, and not to each other)
+        same_bwd_layout = not (dtype != torch.float32 and (N in (5120, 6144) or (N == 4096 and not rms)))
         if rms:
             dh, dg = cabi.add_rms_norm_bwd(dyg, ghg, h, rstd, gg)
             udx, udg = cabi.rms_norm_bwd(dyg, h, rstd, gg)
@@ -111,11 +115,13 @@ def test_add_norm_forward_and_backward(cabi, oracle, gpu, dtype, shape, mixed):
                                                       to_np32(mean), to_np32(rstd), to_np32(gamma))
             xhat = (h.cpu().double() - mean.cpu().double().reshape(M, 1)) * \
                 rstd.cpu().double().reshape(M, 1)
-            assert_same_arithmetic(db, udb, what + " dbeta, fused against plain")
+            if same_bwd_layout:
+                assert_same_arithmetic(db, udb, what + " dbeta, fused against plain")
             sl = colsum_slack(dy.double()) if wtol == torch.float32 else None
             assert_close(db, odb, wtol, what + " dbeta", slack=sl)
         assert torch.equal(nh, udx), what + ": no residual gradient must be the plain backward"
-        assert_same_arithmetic(dg, udg, what + " dgamma, fused against plain", max_fraction=0.05)
+        if same_bwd_layout:
+            assert_same_arithmetic(dg, udg, what + " dgamma, fused against plain", max_fraction=0.05)
         assert_close(dh, odh, dtype, what + " dh")
         sl = colsum_slack(dy.double() * xhat) if wtol == torch.float32 else None
         assert_close(dg, odg, wtol, what + " dgamma", slack=sl)

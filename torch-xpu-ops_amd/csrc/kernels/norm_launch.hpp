@@ -157,9 +157,9 @@ int launch_norm_bwd(const Plan& plan, const NormBwdArgs& a, hipStream_t stream) 
   const bool want_cols = a.part_dg != nullptr;
   const T* dres = ADD ? (const T*)a.dres : nullptr;
   if (plan.resident && plan.exact_depth > 0) {
-    static_assert(kNormBwdExactCount == 11, "one index per table entry below");
+    static_assert(kNormBwdExactCount == 15, "one index per table entry below");
     if (a.dx == nullptr || !launch_norm_bwd_exact<T, WT, RMS, ADD>(
-                               plan, a, stream, ilist<0, 1, 2, 3, 4, 5, 6, 7, 8, 9, 10>{}))
+                               plan, a, stream, ilist<0, 1, 2, 3, 4, 5, 6, 7, 8, 9, 10, 11, 12, 13, 14>{}))
       return (int)hipErrorInvalidConfiguration;
   } else if (plan.resident) {
     NormBwdCtx<T, WT, RMS> ctx{plan, a, stream};

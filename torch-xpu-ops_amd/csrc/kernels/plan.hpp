@@ -230,8 +230,16 @@ struct NormBwdExactLayout {
 };
 constexpr NormBwdExactLayout kNormBwdExact[] = {
     {128, 2, 512, 2, kExactAll | kExactAdd},
+    // (the first entry that serves a call is taken: one row slot a workgroup where that
+    // measured ahead -- bf16 rows x 16384, LayerNorm 4096 69.4 -> 68.8 us, 5120 88.7 ->
+    // 86.5 us, RMSNorm 5120 86.0 -> 83.2 us, 6144 on 384 x 2 instead of 256 x 3 LayerNorm
+    // 105.9 -> 102.1 us (fp32 weights 107.3 -> 102.6), RMSNorm 101.9 -> 99.7 us)
+    {256, 2, 256, 3, kExactLN | kExactLNWide},
     {256, 2, 512, 3, kExactAll | kExactAdd},
+    {320, 2, 320, 3, kExactLN | kExactLNWide},
+    {320, 2, 320, 2, kExactRMS | kExactRMSWide},
     {320, 2, 640, 2, kExactAll | kExactAdd},
+    {384, 2, 384, 2, kExactAll},
     {448, 2, 448, 2, kExactAll | kExactAdd},
     {512, 2, 512, 3, kExactAll | kExactAdd},
     // (at 896 and 1024 lanes the RMSNorm's general kernel already runs this layout as fast)
@@ -291,13 +299,14 @@ constexpr int norm_fwd_exact_index(int esize, int64_t packs, int64_t M, int num_
 //   1280 packs  forward 14.2 -> 15.0 (kept general)   backward 26.4 -> 22.2
 //   2560 packs  forward 29.9 -> 29.3                  backward 49.3 -> 43.0
 //   3840 packs  forward 46.6 -> 43.8                  backward 79.4 -> 67.9
-//   5120 packs  forward 61.6 -> 58.6                  backward 96.2 -> 87.0 + 3.5
+//   5120 packs  forward 61.6 -> 58.6                  backward 96.2 -> 84.9 + 3.5
+//               (one row a workgroup: 2048 workgroups; a grid of 512 is 2 % behind)
 //   7680 packs  forward 94.7 -> 90.2                  backward 140.6 -> 128.0).
 struct GroupExactLayout {
   int G, V, bpc_fwd, bpc_bwd;
 };
 constexpr GroupExactLayout kGroupExact[] = {
-    {256, 5, 0, 8}, {512, 5, 3, 2}, {768, 5, 2, 1}, {512, 10, 2, 2}, {960, 8, 1, 1}};
+    {256, 5, 0, 8}, {512, 5, 3, 2}, {768, 5, 2, 1}, {512, 10, 8, 8}, {960, 8, 1, 1}};
 constexpr int kGroupExactCount = (int)(sizeof(kGroupExact) / sizeof(kGroupExact[0]));
 constexpr int kGroupExactMaxD = 64;  // channels a group: one lane of a wavefront each
 constexpr int group_exact_index(bool backward, int esize, int64_t rows, int64_t L, int64_t HxW,
