@@ -86,8 +86,9 @@ typedef struct {
   int32_t packs_per_lane;  /* V: 16-byte packs each lane holds per row */
   int32_t block_threads;   /* threads per workgroup */
   int32_t rows_per_block;  /* rows a workgroup handles per iteration: block_threads / lanes_per_row */
-  int32_t reserved;        /* mi355x_rownorm_plan: workgroups a row is split over (norm ops, few very
-                              long rows), else 0; mi355x_group_norm_plan: 1 when every pack lies in one channel */
+  int32_t reserved;        /* mi355x_rownorm_plan: workgroups a row is split over or held by (norm ops,
+                              rows beyond one workgroup's registers), else 0; mi355x_group_norm_plan:
+                              1 when every pack lies in one channel */
   int64_t grid_blocks;     /* workgroups launched (persistent, grid-stride over rows) */
   int64_t partial_rows;    /* rows of the fp32 [partial_rows, N] column-sum workspace (backward only) */
 } rownorm_plan;
@@ -376,6 +377,20 @@ int mi355x_rownorm_plan_at(rownorm_op op, int64_t M, int64_t N, rownorm_dtype x_
  * does a field outside 0..65535. */
 int mi355x_rownorm_set_override(rownorm_op op, int lanes_per_row, int packs_per_lane,
                                 int block_threads, int blocks_per_cu);
+
+/* Test hook for the forward of rows that a team of workgroups holds in registers
+ * (LayerNorm / RMSNorm rows beyond 131072 16-bit or 65536 float32 elements, whole
+ * 16-byte packs, no residual add, no cast): how long a workgroup waits for the
+ * others of its team before the call falls back to the two-pass kernel that is
+ * enqueued behind it, in microseconds; 0xffffffff restores the default, one second.
+ * 0 makes every wait give up at once, which is how the tests exercise the fallback
+ * without making any kernel hang.  Process-global.  Such calls draw an id and one
+ * of 32 bookkeeping slots in library-owned device memory from process-wide
+ * counters; results do not depend on which slot a call gets, and two calls that
+ * share a slot while both run (more than 32 such calls in flight across streams)
+ * each detect it and take the fallback.  On a stream under capture these rows take
+ * the multi-launch kernels instead. */
+int mi355x_rownorm_set_team_wait_us(unsigned int microseconds);
 
 /* Measurement aid, no counterpart in the reference: a plain streaming kernel over
  * `bytes` bytes (a multiple of 16; 16-byte aligned device pointers) of each

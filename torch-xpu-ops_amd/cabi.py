@@ -29,7 +29,7 @@ EXPORTED_SYMBOLS = (
     "mi355x_softmax_strided_plan", "mi355x_group_norm_fwd",
     "mi355x_group_norm_bwd_workspace_bytes", "mi355x_group_norm_bwd", "mi355x_group_norm_plan",
     "mi355x_rownorm_plan", "mi355x_rownorm_plan_at", "mi355x_rownorm_set_override",
-    "mi355x_rownorm_stream_probe",
+    "mi355x_rownorm_stream_probe", "mi355x_rownorm_set_team_wait_us",
 )
 
 
@@ -108,6 +108,8 @@ def lib():
         L.mi355x_rownorm_set_override.argtypes = [_int, _int, _int, _int, _int]
         L.mi355x_rownorm_stream_probe.argtypes = [_vp, _vp, _vp, ctypes.c_size_t, _int, _vp]
         L.mi355x_rownorm_stream_probe.restype = _int
+        L.mi355x_rownorm_set_team_wait_us.argtypes = [ctypes.c_uint]
+        L.mi355x_rownorm_set_team_wait_us.restype = _int
         for name in ("mi355x_layer_norm_fwd", "mi355x_rms_norm_fwd", "mi355x_layer_norm_bwd",
                      "mi355x_rms_norm_bwd", "mi355x_rms_norm_bwd_static",
                      "mi355x_add_layer_norm_fwd", "mi355x_add_rms_norm_fwd",
@@ -172,6 +174,12 @@ def group_norm_plan(backward, N, C, HxW, groups, dtype=F32):
     d = p.as_dict()
     d["uniform"] = p.reserved  # 1: every pack in one channel, 2: packs may straddle two, 0: general kernels
     return d
+
+
+def set_team_wait_us(microseconds=0xffffffff):
+    """Bound of a workgroup's wait in the team forward (rows beyond one workgroup's registers);
+    0: every wait gives up at once and the two-pass kernel behind it does the work."""
+    _check(lib().mi355x_rownorm_set_team_wait_us(ctypes.c_uint(microseconds)), "set_team_wait_us")
 
 
 def clear_overrides():

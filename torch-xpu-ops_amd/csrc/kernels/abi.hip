@@ -165,6 +165,42 @@ int static_scratch(void** out) {
   return 0;
 }
 
+// Bookkeeping memory of norm_fwd_team_kernel (partial sums, arrival counters), one
+// slot a call, slots handed out round-robin; per device, like `scratch`.  Zero at
+// load and never cleared: every word a call reads is tagged with the call's id.
+static __device__ __align__(256) __attribute__((used)) TeamSlot team_slots[kTeamSlots];
+std::atomic<void*> g_team_ptr[kMaxDevices];
+std::atomic<unsigned int> g_team_calls{0};
+// Bound of a workgroup's wait for its team, in ticks of the 100 MHz constant-rate
+// clock: one second unless mi355x_rownorm_set_team_wait_us() says otherwise.
+std::atomic<unsigned long long> g_team_wait_ticks{100000000ull};
+
+// The slot and id of a new call on the current device, or null when the team
+// kernel is not to be used: the address is not known, or the stream is being
+// captured (a replay would run with the id of the capture).
+void* team_slot_for_call(hipStream_t stream, unsigned int* id) {
+  hipStreamCaptureStatus st = hipStreamCaptureStatusNone;
+  if (hipStreamIsCapturing(stream, &st) != hipSuccess) {
+    (void)hipGetLastError();
+    return nullptr;
+  }
+  if (st != hipStreamCaptureStatusNone) return nullptr;
+  int dev = 0;
+  if (hipGetDevice(&dev) != hipSuccess || dev < 0 || dev >= kMaxDevices) return nullptr;
+  void* p = g_team_ptr[dev].load(std::memory_order_acquire);
+  if (p == nullptr) {
+    if (hipGetSymbolAddress(&p, HIP_SYMBOL(team_slots)) != hipSuccess || p == nullptr) {
+      (void)hipGetLastError();
+      return nullptr;
+    }
+    g_team_ptr[dev].store(p, std::memory_order_release);
+  }
+  unsigned int n = g_team_calls.fetch_add(1, std::memory_order_relaxed) + 1;
+  if (n == 0) n = g_team_calls.fetch_add(1, std::memory_order_relaxed) + 1;  // 0 tags nothing
+  *id = n;
+  return (char*)p + (size_t)(n % kTeamSlots) * sizeof(TeamSlot);
+}
+
 int esize_of(int dt) {
   switch (dt) {
     case ROWNORM_F32: return 4;
@@ -220,6 +256,10 @@ int norm_fwd(const void* x, const void* res, const void* gamma, const void* beta
     a.h = h;
   }
   hipStream_t s = (hipStream_t)stream;
+  if (plan.team > 0 && !add && yd == xd) {
+    a.team_slot = team_slot_for_call(s, &a.team_id);
+    a.team_wait_ticks = g_team_wait_ticks.load(std::memory_order_relaxed);
+  }
   if (xd == ROWNORM_F32) {
     if (yd == ROWNORM_BF16)
       return add ? launch_norm_fwd<float, float, RMS, bf16, true>(plan, a, s)
@@ -803,8 +843,9 @@ int mi355x_rownorm_plan_at(rownorm_op op, int64_t M, int64_t N, rownorm_dtype x_
   out->packs_per_lane = plan.V;
   out->block_threads = plan.block;
   out->rows_per_block = plan.rpb;
-  out->reserved = plan.split > 1 ? plan.split : 0;
-  out->grid_blocks = plan.grid;
+  // (a forward row held by a team of workgroups: the team and its grid)
+  out->reserved = plan.team > 0 ? plan.team : (plan.split > 1 ? plan.split : 0);
+  out->grid_blocks = plan.team > 0 ? plan.team_grid : plan.grid;
   out->partial_rows = plan.partial_rows;
   return 0;
 }
@@ -827,6 +868,13 @@ int mi355x_rownorm_set_override(rownorm_op op, int lanes_per_row, int packs_per_
   o.block = block_threads;
   o.bpc = blocks_per_cu;
   g_override_bits[(int)op].store(pack_override(o), std::memory_order_relaxed);
+  return 0;
+}
+
+int mi355x_rownorm_set_team_wait_us(unsigned int microseconds) {
+  g_team_wait_ticks.store(microseconds == 0xffffffffu ? 100000000ull
+                                                      : (unsigned long long)microseconds * 100ull,
+                          std::memory_order_relaxed);
   return 0;
 }
 

@@ -23,6 +23,12 @@ struct NormFwdArgs {
   // (both null: plain norm of x)
   const void* res = nullptr;
   void* h = nullptr;
+  // norm_fwd_team_kernel: its slot of bookkeeping memory (null: that kernel is not
+  // used), the id of this call and the bound of its waits in ticks of the
+  // constant-rate clock
+  void* team_slot = nullptr;
+  unsigned int team_id = 0;
+  unsigned long long team_wait_ticks = 0;
 };
 
 struct NormBwdArgs {

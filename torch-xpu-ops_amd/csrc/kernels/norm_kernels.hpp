@@ -566,6 +566,27 @@ __device__ __forceinline__ void long_row_apply(const T* xr, const T* rr, const W
       });
 }
 
+// Device-scope accesses of the team kernel's bookkeeping memory (see norm_fwd_team_kernel).
+__device__ __forceinline__ unsigned long long team_load(const unsigned long long* p) {
+  return __hip_atomic_load(p, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+}
+__device__ __forceinline__ void team_store(unsigned long long* p, unsigned long long v) {
+  __hip_atomic_store(p, v, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+}
+// Earlier stores of this lane have been acknowledged and its loads have returned.
+__device__ __forceinline__ void team_stores_done() {
+  asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
+}
+
+// Whether every workgroup of a team-kernel grid of `n` stored `id` in its `done` entry;
+// called by the first wavefront of a workgroup, the same answer in all its lanes.
+__device__ __forceinline__ bool team_all_done(const TeamSlot* slot, int n, unsigned int id) {
+  bool ok = true;
+  for (int j = (int)(threadIdx.x & 63); j < n; j += 64)
+    ok = ok && __hip_atomic_load(&slot->done[j], __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT) == id;
+  return __ballot(ok) == __ballot(true);
+}
+
 // ---------------------------------------------------------------------------
 // Forward for rows too wide to hold in registers: one workgroup per row, the
 // row is streamed from memory twice (statistics, normalize); the second pass
@@ -580,7 +601,19 @@ __global__ void __launch_bounds__(BLOCK)
 norm_fwd_stream_kernel(const T* __restrict__ x, const T* res, const WT* __restrict__ gamma,
                        const WT* __restrict__ beta, T* h, TY* __restrict__ y,
                        float* __restrict__ mean, float* __restrict__ rstd, int64_t M, int N,
-                       float eps) {
+                       float eps, const TeamSlot* team_done = nullptr, int team_grid = 0,
+                       unsigned int team_id = 0) {
+  // behind norm_fwd_team_kernel: nothing to do if every workgroup of that launch
+  // completed (see there)
+  if (team_done != nullptr) {
+    __shared__ int skip;
+    if (threadIdx.x < 64) {
+      const bool all = team_all_done(team_done, team_grid, team_id);
+      if (threadIdx.x == 0) skip = all ? 1 : 0;
+    }
+    __syncthreads();
+    if (skip) return;
+  }
   constexpr int E = elems_per_pack<T>::value;
   __shared__ float red[reduce_lds_floats<BLOCK, BLOCK, 2>::value];
   __shared__ double red64[RMS ? 1 : 2 * (BLOCK / 64)];
@@ -647,6 +680,203 @@ norm_fwd_stream_kernel(const T* __restrict__ x, const T* res, const WT* __restri
     // stat[] is rewritten for the next row only after every thread has passed the
     // barrier inside the next block sum, i.e. after it has read this row's values
   }
+}
+
+// ---------------------------------------------------------------------------
+// Forward for rows beyond the registers of one workgroup, in ONE pass over X: a
+// row is held in the registers of a team of workgroups.  The grid is at most one
+// workgroup of 1024 threads a compute unit, all resident at once; workgroup b
+// belongs to team b / team and keeps chunk b % team of the team's current row
+// (up to 16 packs a lane: 256 KiB a workgroup, 64 MiB on 256 compute units).  It
+// sums its chunk (float64 sums about the row's centre, as the split-row kernels
+// below), publishes the two partial sums in its entry of library-owned device
+// memory and waits until every workgroup of its team has; each then adds the
+// team's partial sums in chunk order (the same statistics in every workgroup, run
+// to run), normalizes its chunk out of its registers and writes Y.  X is read once
+// and Y written once, where the split-row kernels read X twice (they remain for the
+// calls this kernel does not serve: a residual add, a cast, ragged rows, a stream
+// under capture).  Role in the reference: the split-row regime of Norm.h:632-812,
+// whose partial results also cross work-groups through global memory, between two
+// launches.
+//
+// What crosses workgroups.  An entry is {tag, s1, s2}; the tag of a finished entry is
+// (call id << 32) | (round + 1), ids being unique per call, so nothing has to be
+// cleared and an entry left by an earlier call or round never counts.  The writer
+// sets the tag to 0 when it starts on a row, later stores s1 and s2, waits for
+// those stores to be acknowledged and stores the tag; a reader accepts s1 and s2
+// only if it read the expected tag before and after them.  Every access is a
+// device-scope atomic store or load, which goes to memory: no read-modify-write (256
+// workgroups counting on one word took hundreds of microseconds), and no release
+// or acquire fence (each writes back or invalidates a whole L2).  Two calls that
+// were handed the same slot while both run -- possible only with more such calls
+// in flight than slots -- overwrite each other's tags and therefore never accept
+// each other's sums.
+//
+// The wait is bounded.  A workgroup stops waiting when its team is complete, when
+// any workgroup of the call has given up (a hint word in the slot), or after
+// `wait_ticks` of the constant-rate clock (the workgroups can only fail to be
+// resident together while other kernels hold compute units for that long).  A
+// workgroup that gives up leaves at once; one that has finished all its rows
+// stores the call id in its `done` entry.  The launch that follows on the stream,
+// norm_fwd_stream_kernel, returns at once when it finds the id in the `done`
+// entries of the whole grid and otherwise computes the whole call in the two-pass
+// way.  Every wave reaches an exit whatever the other workgroups do.
+template <class T, class WT, int V, bool RMS>
+__global__ void __launch_bounds__(kTeamBlock)
+norm_fwd_team_kernel(const T* __restrict__ x, const WT* __restrict__ gamma,
+                     const WT* __restrict__ beta, T* __restrict__ y, float* __restrict__ mean,
+                     float* __restrict__ rstd, int64_t M, int N, float eps, int team,
+                     int64_t chunk_packs, TeamSlot* slot, unsigned int call_id,
+                     unsigned long long wait_ticks) {
+  constexpr int E = elems_per_pack<T>::value;
+  constexpr int BLOCK = kTeamBlock;
+  __shared__ double red[2 * (BLOCK / 64)];
+  __shared__ double tpart[kTeamMaxWorkgroups][2];
+  __shared__ float stat[4];
+  const int tm = (int)blockIdx.x / team;
+  const int c = (int)blockIdx.x - tm * team;
+  const int teams = (int)gridDim.x / team;
+  const int64_t npacks = (int64_t)N / E;
+  const int64_t p0 = (int64_t)c * chunk_packs;
+  const int64_t p1 = p0 + chunk_packs < npacks ? p0 + chunk_packs : npacks;
+  const bool hg = gamma != nullptr, hb = !RMS && beta != nullptr;
+  const double dN = (double)N;
+  // Pack k of the lane lies k * BLOCK + threadIdx.x packs into the chunk: a scalar
+  // pointer per pack and one 32-bit byte offset a lane (no 64-bit address a pack in
+  // vector registers, which 16 packs a lane have no room for).
+  const int nloc = p1 > p0 ? (int)(p1 - p0) : 0;  // packs of this chunk
+  const int64_t pbase = nloc > 0 ? p0 : 0;
+  const uint32_t loff = (uint32_t)(threadIdx.x * 16);
+  auto at = [](auto* p, uint32_t off) {
+    using P = decltype(p);
+    return reinterpret_cast<P>(reinterpret_cast<uintptr_t>(p) + off);
+  };
+  unsigned int round = 0;
+  for (int64_t row = tm; row < M; row += teams, ++round) {
+    TeamEntry* entries = slot->entry[round & 1u];
+    if (threadIdx.x == 0) team_store(&entries[blockIdx.x].tag, 0ull);
+    const T* xr = x + row * (int64_t)N;
+    const T* xb = xr + pbase * E;
+    Pack<T, E> xp[V];
+#pragma unroll
+    for (int k = 0; k < V; ++k) {
+      xp[k] = Pack<T, E>::zero();
+      if (k * BLOCK + (int)threadIdx.x < nloc)
+        xp[k] = Pack<T, E>::load_stream(at(xb + k * BLOCK * E, loff));
+    }
+    const float kf = RMS ? 0.0f : split_row_centre(xr, (const T*)nullptr, N);
+    const double kd = (double)kf;
+    double s1 = 0.0, s2 = 0.0;
+#pragma unroll
+    for (int k = 0; k < V; ++k) {
+      keep_packed(xp[k]);
+      if (k * BLOCK + (int)threadIdx.x < nloc)
+        add_centred_sums<T, E, RMS, true>(xp[k], E, kf, kd, s1, s2);
+    }
+    block_sum2_f64<BLOCK>(s1, s2, red);
+    if (threadIdx.x < 64) {  // the first wavefront publishes, waits and adds up
+      const int lane = (int)threadIdx.x;
+      const unsigned long long expect = ((unsigned long long)call_id << 32) | (round + 1u);
+      if (lane == 0) {
+        TeamEntry* mine = &entries[blockIdx.x];
+        team_stores_done();  // the tag has been 0 in memory before the sums change
+        team_store(&mine->s1, __builtin_bit_cast(unsigned long long, s1));
+        team_store(&mine->s2, __builtin_bit_cast(unsigned long long, s2));
+        team_stores_done();
+        team_store(&mine->tag, expect);
+      }
+      const TeamEntry* mates = entries + tm * team;
+      const unsigned long long t0 = wall_clock64();
+      bool complete = false;
+      for (;;) {
+        bool ok = true;
+        for (int j = lane; j < team; j += 64) ok = ok && team_load(&mates[j].tag) == expect;
+        if (__ballot(ok) == __ballot(true)) {
+          for (int j = lane; j < team; j += 64) {
+            tpart[j][0] = __builtin_bit_cast(double, team_load(&mates[j].s1));
+            tpart[j][1] = __builtin_bit_cast(double, team_load(&mates[j].s2));
+            team_stores_done();  // the sums have returned before the tag is read again
+            ok = ok && team_load(&mates[j].tag) == expect;
+          }
+          if (__ballot(ok) == __ballot(true)) {
+            complete = true;
+            break;
+          }
+        }
+        const unsigned int hint =
+            __hip_atomic_load(&slot->gave_up, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+        if (hint == call_id || wall_clock64() - t0 > wait_ticks) break;
+        __builtin_amdgcn_s_sleep(2);
+      }
+      // (the lanes of a wavefront see one another's LDS stores in program order)
+      if (lane == 0) {
+        if (!complete) {
+          __hip_atomic_store(&slot->gave_up, call_id, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+          stat[3] = 1.0f;
+        } else {
+          double t1 = 0.0, t2 = 0.0;
+          for (int j = 0; j < team; ++j) {
+            t1 += tpart[j][0];
+            t2 += tpart[j][1];
+          }
+          if constexpr (RMS) {
+            stat[0] = 0.0f;
+            stat[1] = 0.0f;
+            stat[2] = (float)(1.0 / sqrt(t2 / dN + (double)eps));
+          } else {
+            const double m1 = t1 / dN;
+            const double mu = kd + m1;
+            double var = (t2 - t1 * m1) / dN;
+            var = var < 0.0 ? 0.0 : var;  // (a select: NaN stays NaN)
+            const float hi = (float)mu;
+            stat[0] = var == var ? hi : (float)var;  // NaN variance: NaN mean
+            stat[1] = (float)(mu - (double)hi);
+            stat[2] = (float)(1.0 / sqrt(var + (double)eps));
+          }
+          stat[3] = 0.0f;
+        }
+      }
+    }
+    __syncthreads();
+    if (stat[3] != 0.0f) return;  // (uniform over the workgroup)
+    const float hi = stat[0], lo = stat[1], rs = stat[2];
+    T* yb = y + row * (int64_t)N + pbase * E;
+    const WT* gb = (hg ? gamma : reinterpret_cast<const WT*>(x)) + pbase * E;
+    const WT* bb = (hb ? beta : reinterpret_cast<const WT*>(x)) + pbase * E;
+    // (opaque: the 2 * V weight addresses, the same for every row, would otherwise be
+    // formed once ahead of the row loop and kept -- spilled -- across it)
+    const uint32_t woff = (uint32_t)(lane_again((int)threadIdx.x) * E * (int)sizeof(WT));
+#pragma unroll
+    for (int k = 0; k < V; ++k) {
+      if (k * BLOCK + (int)threadIdx.x < nloc) {
+        keep_packed(xp[k]);
+        const Pack<WT, E> g =
+            hg ? Pack<WT, E>::load(at(gb + k * BLOCK * E, woff)) : Pack<WT, E>::splat(1.0f);
+        const Pack<WT, E> b =
+            hb ? Pack<WT, E>::load(at(bb + k * BLOCK * E, woff)) : Pack<WT, E>::zero();
+        Pack<T, E> o;
+#pragma unroll
+        for (int i = 0; i < E; ++i) {
+          float v;
+          if constexpr (RMS)
+            v = (xp[k].get(i) * rs) * g.get(i);
+          else
+            v = (((xp[k].get(i) - hi) - lo) * rs) * g.get(i) + b.get(i);
+          o.set(i, v);
+        }
+        o.store_stream(at(yb + k * BLOCK * E, loff));
+      }
+    }
+    if (c == 0 && threadIdx.x == 0) {
+      if constexpr (!RMS)
+        if (mean) mean[row] = hi;
+      if (rstd) rstd[row] = rs;
+    }
+    // (stat[], tpart[] and red[] are rewritten for the next row only behind the barrier
+    // inside the next block sum, which every thread reaches after it has read them)
+  }
+  if (threadIdx.x == 0)
+    __hip_atomic_store(&slot->done[blockIdx.x], call_id, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
 }
 
 // ---------------------------------------------------------------------------

@@ -46,6 +46,16 @@ inline bool norm_fwd_can_split(const Plan& plan, const NormFwdArgs& a) {
          regions_disjoint(a.y, ybytes, a.h, xbytes);
 }
 
+// Whether norm_fwd_team_kernel serves the call: planned, its bookkeeping memory at
+// hand (the caller of this function withholds it on a stream under capture), no
+// residual add, Y in the row dtype.  Y may be the memory of X: a workgroup has read
+// all it needs of its chunk before it writes.
+template <class T, class TY, bool ADD>
+inline bool norm_fwd_team_serves(const Plan& plan, const NormFwdArgs& a) {
+  return plan.team > 0 && a.team_slot != nullptr && !ADD && std::is_same<T, TY>::value &&
+         a.res == nullptr;
+}
+
 // The exact two-pack forward layouts (kNormFwdExact): entry I of the table, if the plan names it.
 template <class T, class WT, bool RMS, int I>
 inline bool launch_norm_fwd_exact_at(const Plan& plan, const NormFwdArgs& a, hipStream_t stream) {
@@ -80,6 +90,29 @@ int launch_norm_fwd(const Plan& plan, const NormFwdArgs& a, hipStream_t stream) 
             ? launch_variant<NormFwdLauncher<T, WT, RMS, true, TY, ADD>::template At>(ctx)
             : launch_variant<NormFwdLauncher<T, WT, RMS, false, TY, ADD>::template At>(ctx);
     if (!launched) return (int)hipErrorInvalidConfiguration;
+  } else if (norm_fwd_team_serves<T, TY, ADD>(plan, a)) {
+    // one pass with the row in the registers of a team of workgroups; should that
+    // launch not complete (see the kernel), the guarded launch behind it does the work
+    TeamSlot* slot = (TeamSlot*)a.team_slot;
+    auto go = [&](auto v) {
+      constexpr int V = decltype(v)::value;
+      hipLaunchKernelGGL((norm_fwd_team_kernel<T, WT, V, RMS>), dim3((unsigned)plan.team_grid),
+                         dim3(kTeamBlock), 0, stream, (const T*)a.x, (const WT*)a.gamma,
+                         (const WT*)a.beta, (T*)a.y, a.mean, a.rstd, a.M, a.N, a.eps, plan.team,
+                         plan.team_chunk_packs, slot, a.team_id, a.team_wait_ticks);
+    };
+    switch (plan.team_v) {
+      case 2: go(std::integral_constant<int, 2>{}); break;
+      case 4: go(std::integral_constant<int, 4>{}); break;
+      case 8: go(std::integral_constant<int, 8>{}); break;
+      case 16: go(std::integral_constant<int, 16>{}); break;
+      default: return (int)hipErrorInvalidConfiguration;
+    }
+    if (int e = (int)hipGetLastError()) return e;
+    hipLaunchKernelGGL((norm_fwd_stream_kernel<T, WT, kStreamBlock, RMS, TY>),
+                       dim3((unsigned)plan.grid), dim3(kStreamBlock), 0, stream, (const T*)a.x,
+                       res, (const WT*)a.gamma, (const WT*)a.beta, h, (TY*)a.y, a.mean, a.rstd,
+                       a.M, a.N, a.eps, (const TeamSlot*)slot, (int)plan.team_grid, a.team_id);
   } else if (norm_fwd_can_split<T, TY, RMS>(plan, a)) {
     const dim3 grid((unsigned)plan.split, (unsigned)a.M);
     hipLaunchKernelGGL((norm_fwd_split_sums_kernel<T, kStreamBlock, RMS, TY>), grid,

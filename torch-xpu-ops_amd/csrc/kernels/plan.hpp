@@ -58,11 +58,35 @@ struct Plan {
   // a layout was asked for by override: kernels chosen by other means than the
   // layout (softmax of short ragged rows through LDS) stand back
   bool forced = false;
+  // norm forward of rows beyond one workgroup's registers held by a team of
+  // workgroups (norm_fwd_team_kernel): workgroups a row, packs a lane the kernel is
+  // compiled for, packs a workgroup, workgroups launched; team == 0: not planned
+  int team = 0, team_v = 0;
+  int64_t team_chunk_packs = 0, team_grid = 0;
   // norm backward / forward on an exact layout (norm_bwd_exact_kernel,
   // norm_fwd_exact_kernel): row blocks a lane keeps in flight, itself included (the
   // forward: 1); GroupNorm on an exact layout (gn_*_exact_kernel): 1; 0 = the
   // general resident kernel
   int exact_depth = 0;
+};
+
+// norm_fwd_team_kernel: threads a workgroup, packs a lane at most, workgroups of
+// the grid at most (one a compute unit), slots of bookkeeping memory.
+constexpr int kTeamBlock = 1024;
+constexpr int kTeamMaxV = 16;
+constexpr int kTeamMaxWorkgroups = 256;
+constexpr int kTeamSlots = 32;
+// One call's bookkeeping memory (see the kernel).
+struct TeamEntry {
+  unsigned long long tag;  // (call id << 32) | (round + 1) once s1, s2 are in place; 0 while they change
+  unsigned long long s1, s2;  // a workgroup's partial sums (float64 bit patterns)
+  unsigned long long pad;
+};
+struct TeamSlot {
+  TeamEntry entry[2][kTeamMaxWorkgroups];  // [round parity][workgroup]
+  unsigned int done[kTeamMaxWorkgroups];   // id of the call the workgroup last completed
+  unsigned int gave_up;                    // id of a call one of whose waits ran out (a hint)
+  unsigned int pad[3];
 };
 
 constexpr int kMinG = 8;
@@ -812,6 +836,31 @@ inline int make_plan(OpClass oc, int64_t M, int64_t N, int esize, int num_cus, c
         p.split = (int)chunks;
         p.chunk_packs = cp;
       }
+    }
+  }
+  // Forward rows beyond one workgroup's registers: a team of workgroups holds the
+  // row (one pass over X).  As few workgroups a row as hold it with 16 packs a lane,
+  // then as many teams as there are rows and compute units, and a row spread over
+  // all the workgroups its team can have (down to one stride of 1024 packs each).
+  if (oc == OC_NORM_FWD && !p.resident && p.fast && !fused_add && ov.G == 0 && ov.V == 0 &&
+      ov.bpc == 0) {
+    const int64_t cus = num_cus < kTeamMaxWorkgroups ? num_cus : kTeamMaxWorkgroups;
+    const int64_t per_wg = (int64_t)kTeamBlock * kTeamMaxV;
+    const int64_t team_min = (packs + per_wg - 1) / per_wg;
+    if (team_min <= cus) {
+      int64_t teams = cus / team_min;
+      if (teams > M) teams = M;
+      int64_t team = cus / teams;
+      const int64_t strides = (packs + kTeamBlock - 1) / kTeamBlock;
+      if (team > strides) team = strides;
+      const int64_t chunk = (packs + team - 1) / team;
+      const int64_t need = (chunk + kTeamBlock - 1) / kTeamBlock;
+      int v = 2;
+      while (v < need) v *= 2;
+      p.team = (int)team;
+      p.team_v = v;
+      p.team_chunk_packs = chunk;
+      p.team_grid = teams * team;
     }
   }
   if (oc == OC_SOFTMAX_BWD && !p.resident && p.fast && ov.G == 0 &&
