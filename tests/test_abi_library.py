@@ -146,13 +146,14 @@ def test_plan_invariants(cabi, op, dt):
                 assert p["block_threads"] % G == 0 and p["block_threads"] <= 1024
                 assert p["rows_per_block"] == p["block_threads"] // G
                 assert p["grid_blocks"] <= (M + p["rows_per_block"] - 1) // p["rows_per_block"]
-            elif op in (cabi.OP_LAYER_NORM_FWD, cabi.OP_RMS_NORM_FWD) and N % E == 0:
-                # rows of whole packs beyond one workgroup's registers: a team of `row_chunks`
-                # workgroups holds a row, at most one workgroup a compute unit, no more teams
-                # than rows, every workgroup with at most 16 packs a lane
+            elif (op in (cabi.OP_LAYER_NORM_FWD, cabi.OP_RMS_NORM_FWD) and N % E == 0 and
+                  p["grid_blocks"] > M):
+                # rows of whole packs beyond one workgroup's registers, 8 teams or more: a team
+                # of `row_chunks` workgroups holds a row, at most one workgroup a compute unit,
+                # no more teams than rows, every workgroup with at most 16 packs a lane
                 team = p["row_chunks"]
                 assert p["rows_per_block"] == 1 and team >= 1 and p["grid_blocks"] % team == 0
-                assert p["grid_blocks"] <= 256 and p["grid_blocks"] // team <= M
+                assert p["grid_blocks"] <= 256 and 8 <= p["grid_blocks"] // team <= M
                 assert team * 1024 * 16 * E >= N
             else:
                 assert p["rows_per_block"] == 1 and p["grid_blocks"] <= M

@@ -15,9 +15,9 @@ from helpers import assert_close, gen, to_np32
 pytestmark = pytest.mark.gpu
 
 DTYPES = [torch.float32, torch.float16, torch.bfloat16]
-# (rows, packs a row): one team of 17 workgroups; four teams of 25; two workgroups a row and
-# three rounds of 128 teams; a row spread over 128 workgroups of two packs a lane
-SHAPES = [(3, 16385), (4, 25000), (300, 17500), (2, 163840)]
+# (rows, packs a row): nine teams of 17 workgroups (one stride of 1024 packs each); twelve teams
+# of 21; two workgroups a row and three rounds of 128 teams; eight teams of 32 with five packs a lane
+SHAPES = [(9, 16385), (12, 25000), (300, 17500), (8, 163840)]
 
 
 def _mk(M, N, dtype, wdtype, seed):
@@ -57,7 +57,10 @@ def test_team_forward_against_oracle_fallback_and_split_kernels(cabi, oracle, gp
         print("case team rows", dtype, mixed, (M, N), flush=True)
         for op in (cabi.OP_LAYER_NORM_FWD, cabi.OP_RMS_NORM_FWD):
             p = cabi.plan(op, M, N, code, wcode)
+            # (the plan of a team launch: workgroups a row, and a grid of whole teams, 8 at least)
             assert p["resident"] == 0 and p["row_chunks"] >= 2 and p["grid_blocks"] <= 256, p
+            assert p["grid_blocks"] % p["row_chunks"] == 0, p
+            assert 8 <= p["grid_blocks"] // p["row_chunks"] <= M, p
         x, gamma, beta = _mk(M, N, dtype, wdtype, 1600 + i)
         x[0, :3] = 0.0  # the head of a row is not representative of it
         if M > 2:
@@ -105,8 +108,21 @@ def test_team_forward_against_oracle_fallback_and_split_kernels(cabi, oracle, gp
             assert torch.equal(yi, y) and torch.equal(mi, mean) and torch.equal(ri, rstd)
 
 
+def test_fewer_than_eight_teams_keep_the_multi_launch_kernels(cabi, oracle, gpu):
+    """Rows that would make fewer than 8 teams (their phases run in step and nothing hides the
+    wait) keep the split-row / two-pass kernels; the result is the same to the tolerance."""
+    for (M, N) in ((3, 16385 * 8), (2, 1310720)):
+        p = cabi.plan(cabi.OP_LAYER_NORM_FWD, M, N, cabi.BF16, cabi.BF16)
+        assert p["resident"] == 0 and p["grid_blocks"] <= M, p
+        x, gamma, beta = _mk(M, N, torch.bfloat16, torch.bfloat16, 1640)
+        y, mean, rstd = cabi.layer_norm_fwd(x.to(gpu), gamma.to(gpu), beta.to(gpu), 1e-5)
+        oy, om, orr = oracle.layer_norm_fwd(to_np32(x), (N,), to_np32(gamma), to_np32(beta), 1e-5)
+        assert_close(y, oy, torch.bfloat16, "y [%d, %d]" % (M, N))
+        assert_close(rstd, orr.reshape(-1), torch.float32, "rstd [%d, %d]" % (M, N))
+
+
 def test_team_forward_non_finite_rows_and_missing_statistics(cabi, oracle, gpu):
-    M, N = 4, 20000 * 8
+    M, N = 9, 20000 * 8
     x, gamma, beta = _mk(M, N, torch.bfloat16, torch.bfloat16, 1650)
     x[1, 70000] = float("inf")
     x[3, N - 1] = float("nan")
@@ -114,9 +130,12 @@ def test_team_forward_non_finite_rows_and_missing_statistics(cabi, oracle, gpu):
     y, mean, rstd = cabi.layer_norm_fwd(xg, gg, bg, 1e-5)
     assert bool(torch.isnan(mean[1])) and bool(torch.isnan(rstd[1])) and bool(torch.isnan(y[1]).all())
     assert bool(torch.isnan(mean[3])) and bool(torch.isnan(y[3]).all())
-    oy, om, orr = oracle.layer_norm_fwd(to_np32(x[[0, 2]]), (N,), to_np32(gamma), to_np32(beta), 1e-5)
-    assert_close(y[[0, 2]], oy, torch.bfloat16, "finite rows beside non-finite ones")
-    assert_close(rstd[[0, 2]], orr.reshape(-1), torch.float32, "rstd of the finite rows")
+    p = cabi.plan(cabi.OP_LAYER_NORM_FWD, M, N, cabi.BF16, cabi.BF16)
+    assert p["grid_blocks"] // max(p["row_chunks"], 1) >= 8, p  # (a team launch)
+    fin = [0, 2, 4, 5, 6, 7, 8]
+    oy, om, orr = oracle.layer_norm_fwd(to_np32(x[fin]), (N,), to_np32(gamma), to_np32(beta), 1e-5)
+    assert_close(y[fin], oy, torch.bfloat16, "finite rows beside non-finite ones")
+    assert_close(rstd[fin], orr.reshape(-1), torch.float32, "rstd of the finite rows")
     ry, rr = cabi.rms_norm_fwd(xg, gg, 1e-6)
     assert float(rr[1]) == 0.0 and bool(torch.isnan(rr[3]))
 

@@ -76,6 +76,7 @@ constexpr int kTeamBlock = 1024;
 constexpr int kTeamMaxV = 16;
 constexpr int kTeamMaxWorkgroups = 256;
 constexpr int kTeamSlots = 32;
+constexpr int kTeamMinTeams = 8;
 // One call's bookkeeping memory (see the kernel).
 struct TeamEntry {
   unsigned long long tag;  // (call id << 32) | (round + 1) once s1, s2 are in place; 0 while they change
@@ -847,9 +848,15 @@ inline int make_plan(OpClass oc, int64_t M, int64_t N, int esize, int num_cus, c
     const int64_t cus = num_cus < kTeamMaxWorkgroups ? num_cus : kTeamMaxWorkgroups;
     const int64_t per_wg = (int64_t)kTeamBlock * kTeamMaxV;
     const int64_t team_min = (packs + per_wg - 1) / per_wg;
-    if (team_min <= cus) {
-      int64_t teams = cus / team_min;
-      if (teams > M) teams = M;
+    int64_t teams = team_min <= cus ? cus / team_min : 0;
+    if (teams > M) teams = M;
+    // Fewer than 8 teams run their load, wait and store phases nearly in step, and
+    // the wait (about 8 us a round) is not hidden by other teams: bf16 [128, 9834496]
+    // (3 teams of 85, 43 rounds) took 1740 us against 1500 us for the two-pass kernel
+    // whose second pass comes out of the memory-side cache, [2, 1310720] 13.2 against
+    // 11.6 us; 8 teams ([8, 4194304], one round) 35.1 against 40.5 us, 64 teams
+    // ([512, 401408], 8 rounds) 177 against 196 us.
+    if (teams >= kTeamMinTeams) {
       int64_t team = cus / teams;
       const int64_t strides = (packs + kTeamBlock - 1) / kTeamBlock;
       if (team > strides) team = strides;
