@@ -371,8 +371,10 @@ int mi355x_rownorm_plan_at(rownorm_op op, int64_t M, int64_t N, rownorm_dtype x_
  * the four fields of an op are stored as one atomic word, so a call that runs
  * while another thread changes the override uses the old or the new variant,
  * never a mix.  Production callers never use it: with no override set (the
- * state a process starts in) every entry point is re-entrant and reads no
- * mutable global state.  A call whose shape the forced variant cannot hold
+ * state a process starts in) every entry point is re-entrant, and the only
+ * mutable global state any of them touches is the call counter and the
+ * bookkeeping slots of the team forward described at
+ * mi355x_rownorm_set_team_wait_us.  A call whose shape the forced variant cannot hold
  * fails with ROWNORM_ERR_OVERRIDE instead of silently choosing another, and so
  * does a field outside 0..65535. */
 int mi355x_rownorm_set_override(rownorm_op op, int lanes_per_row, int packs_per_lane,

@@ -22,13 +22,6 @@ namespace rownorm {
 using f16 = _Float16;
 using bf16 = __bf16;
 
-#ifndef ROWNORM_NT_LOAD
-#define ROWNORM_NT_LOAD 1
-#endif
-#ifndef ROWNORM_NT_STORE
-#define ROWNORM_NT_STORE 1
-#endif
-
 template <class T>
 struct elems_per_pack {
   static constexpr int value = 16 / sizeof(T);
@@ -56,11 +49,7 @@ struct Pack {
   // Streaming (read-once / write-once) accesses carry the non-temporal hint.
   __device__ __forceinline__ static Pack load_stream(const T* p) {
     Pack r;
-#if ROWNORM_NT_LOAD
     r.v = __builtin_nontemporal_load(reinterpret_cast<const uvec_t*>(p));
-#else
-    r.v = *reinterpret_cast<const uvec_t*>(p);
-#endif
     return r;
   }
   __device__ __forceinline__ static Pack load(const T* p) {
@@ -69,11 +58,7 @@ struct Pack {
     return r;
   }
   __device__ __forceinline__ void store_stream(T* p) const {
-#if ROWNORM_NT_STORE
     __builtin_nontemporal_store(v, reinterpret_cast<uvec_t*>(p));
-#else
-    *reinterpret_cast<uvec_t*>(p) = v;
-#endif
   }
   __device__ __forceinline__ void store(T* p) const { *reinterpret_cast<uvec_t*>(p) = v; }
 

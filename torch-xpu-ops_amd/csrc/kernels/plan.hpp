@@ -357,11 +357,7 @@ constexpr bool norm_bwd_lds_layout(int esize, int64_t v_exact, bool layer_norm) 
 // Workgroup sizes a G-lane variant is compiled for.
 constexpr bool block_built(OpClass oc, int G, int block) {
   if (block < G || block < 256 || block > 1024 || (block & (block - 1))) return false;
-#ifdef ROWNORM_TUNE_WIDE
-  return true;
-#else
   return block == block_threads(oc, G);
-#endif
 }
 
 // Workgroups per compute unit of the grid-stride launch.  The norm kernels keep
@@ -449,9 +445,6 @@ constexpr bool variant_built(OpClass oc, int esize, int G, int V, bool fast) {
   // longer ragged rows take the multi-pass kernels (measured faster for softmax
   // at vocabulary sizes such as 50257 than a general kernel with more packs)
   if (!fast) return V == v_pref(oc, esize);
-#ifdef ROWNORM_TUNE_WIDE
-  return true;
-#else
   if (G == kMinG) return V <= v_pref(oc, esize);
   // short rows take one pack a lane on up to one wavefront (see make_plan())
   if ((oc == OC_NORM_FWD || oc == OC_NORM_BWD || oc == OC_SOFTMAX_FWD || oc == OC_SOFTMAX_BWD) &&
@@ -464,7 +457,6 @@ constexpr bool variant_built(OpClass oc, int esize, int G, int V, bool fast) {
   // (a third of the kernels otherwise).
   if ((oc == OC_NORM_FWD || oc == OC_NORM_BWD) && esize == 2 && G == 512 && V == 4) return true;
   return V == v_pref(oc, esize);
-#endif
 }
 
 inline int pow2_ceil(int64_t v) {
@@ -488,9 +480,6 @@ inline int pow2_ceil(int64_t v) {
 //  * fp32 LayerNorm forward rows of 2049..2560 packs: 512 lanes x 5 (N = 10240:
 //    261 -> 222 us).
 // Returns false where the general rule stands.
-#ifndef ROWNORM_BWD_SPARSE_MIN_G2
-#define ROWNORM_BWD_SPARSE_MIN_G2 512
-#endif
 inline bool norm_layout(OpClass oc, int esize, int64_t packs, bool layer_norm, bool wide_weights,
                         int* G_out, int* V_out) {
   const int vp = v_pref(oc, esize);
@@ -513,7 +502,7 @@ inline bool norm_layout(OpClass oc, int esize, int64_t packs, bool layer_norm, b
       // (fp32 gamma and beta beside 16-bit rows: three packs of each are 48
       // registers, and below 512 lanes the two-pack layout stays ahead)
       G = G2 / 2, V = 3;
-    } else if (!fwd && sparse && G2 >= ROWNORM_BWD_SPARSE_MIN_G2) {
+    } else if (!fwd && sparse && G2 >= 512) {
       // the backward with three packs a lane requests its next rows ahead:
       // N = 5120: LayerNorm 95 -> 93 us, RMSNorm 92 -> 87 us; 6144: 112 -> 107 us
       // and 108 -> 102 us

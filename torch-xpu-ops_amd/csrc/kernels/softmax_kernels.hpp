@@ -74,10 +74,6 @@ __device__ __forceinline__ Pack<T, E> stream_load(const T* row, int e0, int n, b
 // the exponential in log_softmax's output pass and in softmax's backward too).
 #define ROWNORM_UNIFORM_ARM(tag) asm volatile("; " tag)
 
-#ifndef ROWNORM_SOFTMAX_ONLINE_WIDE
-#define ROWNORM_SOFTMAX_ONLINE_WIDE 1
-#endif
-
 // Packs a thread of the multi-pass kernels requests before using the first.
 constexpr int kStreamUnroll = 2;
 
@@ -123,13 +119,10 @@ __device__ __forceinline__ Pack<uint8_t, E> load_mask_pack(const uint8_t* mrow, 
 // second argument of __launch_bounds__ in HIP): eight, i.e. two 1024-thread
 // workgroups a compute unit and 64 registers, for 1024-lane rows of 5..9 packs a
 // lane; otherwise what the workgroup size implies.
-#ifndef ROWNORM_SOFTMAX_TWO_BLOCKS_MAX_V
-#define ROWNORM_SOFTMAX_TWO_BLOCKS_MAX_V 9
-#endif
-constexpr int kSoftmaxFreshOffsetsMaxV = ROWNORM_SOFTMAX_TWO_BLOCKS_MAX_V;
+constexpr int kSoftmaxFreshOffsetsMaxV = 9;
 template <class TI, int G, int V, bool FAST, bool MASKED>
 constexpr int softmax_fwd_min_blocks() {
-  return (G == 1024 && FAST && !MASKED && V >= 5 && V <= ROWNORM_SOFTMAX_TWO_BLOCKS_MAX_V) ? 8 : 1;
+  return (G == 1024 && FAST && !MASKED && V >= 5 && V <= kSoftmaxFreshOffsetsMaxV) ? 8 : 1;
 }
 
 template <class TI, class TO, int G, int V, int BLOCK, bool FAST, bool MASKED>
@@ -192,7 +185,7 @@ softmax_fwd_resident_kernel(const TI* __restrict__ x, TO* __restrict__ y, MaskRe
       float mx[1] = {-INFINITY};
       float sum[1] = {0.0f};
       float m;
-      if constexpr (ROWNORM_SOFTMAX_ONLINE_WIDE && !MASKED && FAST && V >= 8) {
+      if constexpr (!MASKED && FAST && V >= 8) {
         // the lane's packs in two halves, each with its own maximum and sum of
         // exp(x - maximum): the first half is worked on while the second is still
         // arriving, and the exponentials no longer wait for the block maximum
@@ -623,10 +616,7 @@ softmax_bwd_resident_kernel(const TG* __restrict__ grad, const TG* __restrict__ 
 // same dtype in and out; anything else keeps the general kernels.  Very short
 // rows of whole packs whose pack count fits the resident layouts badly take the
 // same path (flat_layout, softmax_launch.hpp).
-#ifndef ROWNORM_FLAT_BLOCK
-#define ROWNORM_FLAT_BLOCK 256
-#endif
-constexpr int kFlatBlock = ROWNORM_FLAT_BLOCK;
+constexpr int kFlatBlock = 256;
 // LDS per tensor a workgroup holds (LDSB; the backward holds two tensors): 16 KB
 // at 256 threads, so that 8 workgroups share a compute unit; the backward takes
 // 8 KB per tensor where that still holds a full pass of rows, for the same
@@ -806,17 +796,11 @@ softmax_fwd_flat_kernel(const T* __restrict__ x, T* __restrict__ y, int64_t M, i
 #pragma unroll
       for (int i = 0; i < E; ++i)
         o.set(i, is_log ? v[c][i] - kf : (zero_row ? 0.0f : v[c][i] * kf));
-#ifdef ROWNORM_FLAT_DIRECT_OUT
-      if (j < N) store_row_pack<T, E, true>(y + (row0 + r) * (int64_t)N, j, N, true, o);
-#else
       if (j < N) flat_row_store<T, E>(rowb, j, N - j, o);
-#endif
     }
   }
-#ifndef ROWNORM_FLAT_DIRECT_OUT
   __syncthreads();
   flat_stage_out<T, BLOCK, U>(y + row0 * (int64_t)N, buf, nelem);
-#endif
 }
 
 template <class T, int G, int VP, int BLOCK, int LDSB>
@@ -864,17 +848,11 @@ softmax_bwd_flat_kernel(const T* __restrict__ grad, const T* __restrict__ y, T* 
 #pragma unroll
       for (int i = 0; i < E; ++i)
         o.set(i, is_log ? gf[c][i] - row_exp<PRECISE>(yf[c][i]) * sum : yf[c][i] * (gf[c][i] - sum));
-#ifdef ROWNORM_FLAT_DIRECT_OUT
-      if (j < N) store_row_pack<T, E, true>(gi + (row0 + r) * (int64_t)N, j, N, true, o);
-#else
       if (j < N) flat_row_store<T, E>(rg, j, N - j, o);
-#endif
     }
   }
-#ifndef ROWNORM_FLAT_DIRECT_OUT
   __syncthreads();
   flat_stage_out<T, BLOCK, U>(gi + row0 * (int64_t)N, bg, nelem);
-#endif
 }
 
 // log_softmax backward for rows beyond what the registers hold of TWO tensors
