@@ -89,18 +89,27 @@ norm_fwd_resident_kernel(const T* __restrict__ x, const T* res, const WT* __rest
   constexpr bool kHold =
       norm_fwd_holds_weights((int)sizeof(T), (int)sizeof(WT), G, V, FAST, RMS, ADD);
   const bool exact = N == G * V * E;  // every pack of every lane lies inside the row
+  // WINDOW (norm_row_window()): ragged 16-bit rows are addressed through the 16-byte
+  // aligned window that holds the row, `hd` elements ahead of it; the held weights
+  // are those of the window's columns and are loaded again should a row of this lane
+  // group sit at another head (the planner's grids keep it constant).
+  constexpr bool WINDOW = norm_row_window((int)sizeof(T), G, FAST);
+  static_assert(!WINDOW || (R == 1 && kHold), "windowed rows: one row a lane group, weights held");
   Pack<WT, E> gp[kHold ? V : 1];
   Pack<WT, E> bp[RMS || !kHold ? 1 : V];
-  if constexpr (kHold) {
+  auto load_weights = [&](int head) {
 #pragma unroll
     for (int c = 0; c < V; ++c) {
-      const int e0 = (c * G + lane0) * E;
-      gp[c] = gamma ? load_row_pack<WT, E, false>(gamma, e0, N, true, 1.0f)
-                    : Pack<WT, E>::splat(1.0f);
+      const int e0 = (c * G + lane0) * E - head;
+      gp[kHold ? c : 0] = gamma ? load_row_pack<WT, E, false>(gamma, e0, N, true, 1.0f)
+                                : Pack<WT, E>::splat(1.0f);
       if constexpr (!RMS)
-        bp[c] = beta ? load_row_pack<WT, E, false>(beta, e0, N, true, 0.0f) : Pack<WT, E>::zero();
+        bp[kHold ? c : 0] =
+            beta ? load_row_pack<WT, E, false>(beta, e0, N, true, 0.0f) : Pack<WT, E>::zero();
     }
-  }
+  };
+  int held_head = -1;
+  if constexpr (kHold && !WINDOW) load_weights(0);
 
   const int64_t nrb = (M + RPI - 1) / RPI;
   for (int64_t rb = blockIdx.x; rb < nrb; rb += gridDim.x) {
@@ -109,23 +118,39 @@ norm_fwd_resident_kernel(const T* __restrict__ x, const T* res, const WT* __rest
     const int lane = lane_again<!kHold>(lane0);
     bool ok[R];
     Pack<T, E> xp[R][V];
+    int hd = 0;  // the window's head; N + hd: the row's end in window elements
+    if constexpr (WINDOW) {
+      hd = window_head<T, E>(x + ((RPI == 1 || row0 < M) ? row0 : 0) * (int64_t)N);
+      if (hd != held_head) {
+        load_weights(hd);
+        held_head = hd;
+      }
+    }
+    const int nw = N + hd;
 #pragma unroll
     for (int r = 0; r < R; ++r) {
       ok[r] = (RPI == 1) ? true : row0 + r < M;
-      const T* xr = x + (ok[r] ? row0 + r : 0) * (int64_t)N;
+      const T* xr = x + (ok[r] ? row0 + r : 0) * (int64_t)N - hd;
 #pragma unroll
       for (int c = 0; c < V; ++c)
-        xp[r][c] = row_load<T, E, true, FAST>(xr, (c * G + lane) * E, N, ok[r], 0.0f);
+        xp[r][c] = row_load<T, E, true, FAST>(xr, (c * G + lane) * E, nw, ok[r], 0.0f, hd, WINDOW);
       if constexpr (ADD) {
-        const T* rr = res + (ok[r] ? row0 + r : 0) * (int64_t)N;
+        const T* rr = res + (ok[r] ? row0 + r : 0) * (int64_t)N - hd;
         Pack<T, E> rp[V];
 #pragma unroll
         for (int c = 0; c < V; ++c)
-          rp[c] = row_load<T, E, true, FAST>(rr, (c * G + lane) * E, N, ok[r], 0.0f);
+          rp[c] = row_load<T, E, true, FAST>(rr, (c * G + lane) * E, nw, ok[r], 0.0f, hd, WINDOW);
 #pragma unroll
         for (int c = 0; c < V; ++c)
 #pragma unroll
           for (int i = 0; i < E; ++i) xp[r][c].set(i, xp[r][c].get(i) + rp[c].get(i));
+      }
+      // (the RMSNorm sums squares: the window's elements outside the row become zero;
+      // the LayerNorm replaces them by its centre below)
+      if constexpr (WINDOW && RMS) {
+#pragma unroll
+        for (int c = 0; c < V; ++c)
+          row_trim<T, E, FAST>(xp[r][c], (c * G + lane) * E, nw, 0.0f, hd, WINDOW);
       }
     }
 
@@ -192,11 +217,12 @@ norm_fwd_resident_kernel(const T* __restrict__ x, const T* res, const WT* __rest
           // rows of 2047: 41 -> 38.5 us at 16384 rows, of 257: 35 -> 32.4 us at 65536)
 #pragma unroll
           for (int c = 0; c < V; ++c) {
-            const int nvalid = ok[r] ? N - (c * G + lane) * E : 0;
-            if (nvalid < E) {
+            const int nvalid = ok[r] ? nw - (c * G + lane) * E : 0;
+            const int nahead = WINDOW ? hd - (c * G + lane) * E : 0;  // (the window's first pack)
+            if (nvalid < E || nahead > 0) {
 #pragma unroll
               for (int i = 0; i < E; ++i)
-                if (i >= nvalid) xp[r][c].set(i, k);
+                if (i >= nvalid || i < nahead) xp[r][c].set(i, k);
             }
           }
         }
@@ -287,13 +313,13 @@ norm_fwd_resident_kernel(const T* __restrict__ x, const T* res, const WT* __rest
     const int ls = lane_after<!kHold>(lane0, nm1rs[0]);
 #pragma unroll
     for (int r = 0; r < R; ++r) {
-      TY* yr = y + (row0 + r) * (int64_t)N;
+      TY* yr = y + (row0 + r) * (int64_t)N - hd;
 #pragma unroll
       for (int c = 0; c < V; ++c) {
         keep_packed(xp[r][c]);
         if constexpr (ADD)
-          row_store<T, E, true, FAST>(h + (row0 + r) * (int64_t)N, (c * G + ls) * E, N, ok[r],
-                                      xp[r][c]);
+          row_store<T, E, true, FAST>(h + (row0 + r) * (int64_t)N - hd, (c * G + ls) * E, nw, ok[r],
+                                      xp[r][c], hd);
         if constexpr (kHold && !kWideWeights) {
           keep_packed(gp[c]);
           if constexpr (!RMS) keep_packed(bp[c]);
@@ -322,7 +348,7 @@ norm_fwd_resident_kernel(const T* __restrict__ x, const T* res, const WT* __rest
             v = (((xp[r][c].get(i) - mean0[r]) - m1[r]) * rs[r]) * gc.get(i) + bc.get(i);
           o.set(i, v);
         }
-        row_store<TY, E, true, FAST>(yr, (c * G + ls) * E, N, ok[r], o);
+        row_store<TY, E, true, FAST>(yr, (c * G + ls) * E, nw, ok[r], o, hd);
       }
       if (ok[r] && lane0 == 0) {
         if constexpr (!RMS)

@@ -68,6 +68,10 @@ struct Plan {
   // forward: 1); GroupNorm on an exact layout (gn_*_exact_kernel): 1; 0 = the
   // general resident kernel
   int exact_depth = 0;
+  // ragged 16-bit norm rows addressed through the 16-byte aligned window that holds
+  // each row (norm_row_window()): G * V holds the packs of that window, and a
+  // workgroup that walks several row blocks strides by a multiple of 8 rows
+  bool window = false;
 };
 
 // norm_fwd_team_kernel: threads a workgroup, packs a lane at most, workgroups of
@@ -112,6 +116,25 @@ constexpr int kSplitMaxChunks = 1024;
 // keeps the register count low enough for 8 wavefronts per SIMD, which beats
 // fewer, fatter lanes on every op of the family.
 constexpr int v_pref(OpClass, int esize) { return esize == 4 ? 4 : 2; }
+
+// Ragged 16-bit rows of the norm forward (every row at another 2-byte alignment,
+// where a 128-bit access costs about twice an aligned one) on 256 lanes or more are
+// addressed through the 16-byte aligned window that holds the row: it starts up to
+// 7 elements before the row and can hold one pack more than the row.  Every whole
+// pack of the window is an aligned access, the two end packs are trimmed (loads)
+// or written element by element (stores), and gamma / beta are held shifted by the
+// window's head: loaded once per workgroup when all its rows have the same head,
+// i.e. when it strides by a multiple of 8 rows, which make_plan() sees to (and
+// again per row otherwise).  fp16, 8192 rows that start 2 elements into their
+// buffers: N = 4097 LayerNorm 43.6 -> 34.6 us, RMSNorm 31.2 -> 29.9 us; 8193: 68.8 ->
+// 61.0 and 58.9 -> 51.1 us.  Shorter rows lose (the two end packs weigh more: N =
+// 2049 LayerNorm 20.0 -> 20.9 us, RMSNorm 15.3 -> 17.3 us) and keep the row-start
+// addressing; so does the backward, which measured no gain (N = 4097 LayerNorm 68.6
+// -> 68.1 us) or a loss (RMSNorm 53.8 -> 71.6 us: 132 registers against 127, one
+// workgroup a compute unit instead of two).
+constexpr bool norm_row_window(int esize, int G, bool fast) {
+  return !fast && esize == 2 && G >= 256;
+}
 
 // The resident norm forward keeps gamma / beta of a lane's columns in registers
 // across its rows while they fit; at 1024 lanes, rows of more packs a lane than
@@ -521,6 +544,21 @@ inline bool norm_layout(OpClass oc, int esize, int64_t packs, bool layer_norm, b
   return true;
 }
 
+// Lanes a ragged 16-bit row of `packs` packs takes in the norm forward (the rule of
+// make_plan() below for such rows: two packs a lane, or three on half the lanes when
+// the row fills at most three quarters of the two-pack slots), computed ahead of the
+// plan because the lanes decide whether `packs` counts the row's window or the row.
+inline int ragged_norm_fwd_lanes(int64_t packs, const Override& ov) {
+  if (ov.G > 0) return ov.G;
+  int G = pow2_ceil((packs + 1) / 2);
+  if (G < kMinG) G = kMinG;
+  if (G > kMaxG) G = kMaxG;
+  if (ov.V == 0 && G >= 128 && packs <= (int64_t)G * 2 && packs * 4 <= (int64_t)G * 2 * 3 &&
+      variant_built(OC_NORM_FWD, 2, G / 2, 3, false))
+    G /= 2;
+  return G;
+}
+
 // Returns 0, or -5 (ROWNORM_ERR_OVERRIDE) when a forced variant cannot hold the row.
 // force_general: take the general (ragged-row) kernels even when N % E == 0.
 // layer_norm: the norm op is LayerNorm (statistics of two sums, beta), not RMSNorm.
@@ -541,7 +579,17 @@ inline int make_plan(OpClass oc, int64_t M, int64_t N, int esize, int num_cus, c
   const bool softmax = oc == OC_SOFTMAX_FWD || oc == OC_SOFTMAX_BWD;
   // the general softmax kernels address a 16-bit row through the 16-byte aligned
   // window that holds it, which starts up to E - 1 elements before the row
-  const int64_t packs = ((softmax && !p.fast && esize == 2 ? N + E - 1 : N) + E - 1) / E;
+  int64_t packs = ((softmax && !p.fast && esize == 2 ? N + E - 1 : N) + E - 1) / E;
+  // and so does the general norm forward on 256 lanes or more (norm_row_window()): the
+  // lanes a row takes follow from its window's packs (halved below when three packs
+  // a lane fit better, hence 512 here)
+  if (oc == OC_NORM_FWD && !p.fast && esize == 2 && ov.G >= 0) {
+    const int64_t wpacks = (N + E - 1 + E - 1) / E;
+    if (norm_row_window(esize, ragged_norm_fwd_lanes(wpacks, ov), false)) {
+      p.window = true;
+      packs = wpacks;
+    }
+  }
   if (num_cus <= 0) num_cus = 256;
   bool stream = ov.G < 0;
   if (!stream) {
@@ -780,9 +828,20 @@ inline int make_plan(OpClass oc, int64_t M, int64_t N, int esize, int num_cus, c
       !norm_fwd_holds_weights(esize, wide_weights ? 4 : esize, p.G, p.V, p.fast, !layer_norm,
                               fused_add))
     grid = nrb;
+  if (!p.resident) p.window = false;
+  // windowed rows: 1024 threads a compute unit, all resident at once, so that a
+  // workgroup loads its shifted weights once for all its rows (fp16 [8192, 4097]
+  // LayerNorm: 4 workgroups of 256 a compute unit 34.6 us, 2: 45.9, 8: 40.0, one row a
+  // workgroup 52.3; [8192, 8193] on 512 threads: 2 a compute unit 61.0 us, 1: 83.9, 4: 69.5)
+  if (p.window && ov.bpc == 0) grid = (int64_t)num_cus * (1024 / p.block);
   if (grid > nrb) grid = nrb;
   if (grid > 0x7fffffff) grid = 0x7fffffff;
   if (grid < 1) grid = 1;
+  // (the kernel takes the window from its lanes: the two must agree)
+  if (p.resident && oc == OC_NORM_FWD && p.window != norm_row_window(esize, p.G, p.fast)) return -5;
+  // windowed rows: a workgroup that walks several row blocks strides by a multiple of
+  // 8 rows, so that every row of a lane group has the same window head
+  if (p.window && grid < nrb && grid % 8 != 0) grid = grid > 8 ? grid - grid % 8 : (nrb < 8 ? nrb : 8);
   p.grid = grid;
   p.partial_rows = 0;
   if (oc == OC_NORM_BWD && want_cols) {
