@@ -153,8 +153,8 @@ def test_plan_invariants(cabi, op, dt):
                 # no more teams than rows, every workgroup with at most 16 packs a lane
                 team = p["row_chunks"]
                 assert p["rows_per_block"] == 1 and team >= 1 and p["grid_blocks"] % team == 0
-                assert p["grid_blocks"] <= 256 and 8 <= p["grid_blocks"] // team <= M
-                assert team * 1024 * 16 * E >= N
+                assert p["grid_blocks"] <= 512 and 8 <= p["grid_blocks"] // team <= M
+                assert team * 512 * 16 * E >= N
             else:
                 assert p["rows_per_block"] == 1 and p["grid_blocks"] <= M
             if op in (cabi.OP_LAYER_NORM_BWD, cabi.OP_RMS_NORM_BWD):

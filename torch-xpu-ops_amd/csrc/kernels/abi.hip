@@ -165,9 +165,9 @@ int static_scratch(void** out) {
   return 0;
 }
 
-// Bookkeeping memory of norm_fwd_team_kernel (partial sums, arrival counters), one
-// slot a call, slots handed out round-robin; per device, like `scratch`.  Zero at
-// load and never cleared: every word a call reads is tagged with the call's id.
+// Bookkeeping memory of norm_fwd_team_kernel (the workgroups' partial sums), one slot
+// a call, slots handed out round-robin; per device, like `scratch`.  Zero at load and
+// never cleared: every word a call reads is tagged with the call's id.
 static __device__ __align__(256) __attribute__((used)) TeamSlot team_slots[kTeamSlots];
 std::atomic<void*> g_team_ptr[kMaxDevices];
 std::atomic<unsigned int> g_team_calls{0};
@@ -256,7 +256,12 @@ int norm_fwd(const void* x, const void* res, const void* gamma, const void* beta
     a.h = h;
   }
   hipStream_t s = (hipStream_t)stream;
-  if (plan.team > 0 && !add && yd == xd) {
+  // (not in place: a workgroup of the team kernel whose team does not come together
+  // reads the whole row of X, which must then still be X)
+  const uintptr_t xb = (uintptr_t)x, yb = (uintptr_t)y;
+  const uintptr_t nbytes = (uintptr_t)M * (uintptr_t)N * (uintptr_t)esize_of(xd);
+  const bool y_on_x = xb < yb + nbytes && yb < xb + nbytes;
+  if (plan.team > 0 && !add && yd == xd && !y_on_x) {
     a.team_slot = team_slot_for_call(s, &a.team_id);
     a.team_wait_ticks = g_team_wait_ticks.load(std::memory_order_relaxed);
   }

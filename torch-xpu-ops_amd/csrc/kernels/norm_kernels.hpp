@@ -604,15 +604,6 @@ __device__ __forceinline__ void team_stores_done() {
   asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
 }
 
-// Whether every workgroup of a team-kernel grid of `n` stored `id` in its `done` entry;
-// called by the first wavefront of a workgroup, the same answer in all its lanes.
-__device__ __forceinline__ bool team_all_done(const TeamSlot* slot, int n, unsigned int id) {
-  bool ok = true;
-  for (int j = (int)(threadIdx.x & 63); j < n; j += 64)
-    ok = ok && __hip_atomic_load(&slot->done[j], __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT) == id;
-  return __ballot(ok) == __ballot(true);
-}
-
 // ---------------------------------------------------------------------------
 // Forward for rows too wide to hold in registers: one workgroup per row, the
 // row is streamed from memory twice (statistics, normalize); the second pass
@@ -627,19 +618,7 @@ __global__ void __launch_bounds__(BLOCK)
 norm_fwd_stream_kernel(const T* __restrict__ x, const T* res, const WT* __restrict__ gamma,
                        const WT* __restrict__ beta, T* h, TY* __restrict__ y,
                        float* __restrict__ mean, float* __restrict__ rstd, int64_t M, int N,
-                       float eps, const TeamSlot* team_done = nullptr, int team_grid = 0,
-                       unsigned int team_id = 0) {
-  // behind norm_fwd_team_kernel: nothing to do if every workgroup of that launch
-  // completed (see there)
-  if (team_done != nullptr) {
-    __shared__ int skip;
-    if (threadIdx.x < 64) {
-      const bool all = team_all_done(team_done, team_grid, team_id);
-      if (threadIdx.x == 0) skip = all ? 1 : 0;
-    }
-    __syncthreads();
-    if (skip) return;
-  }
+                       float eps) {
   constexpr int E = elems_per_pack<T>::value;
   __shared__ float red[reduce_lds_floats<BLOCK, BLOCK, 2>::value];
   __shared__ double red64[RMS ? 1 : 2 * (BLOCK / 64)];
@@ -710,45 +689,51 @@ norm_fwd_stream_kernel(const T* __restrict__ x, const T* res, const WT* __restri
 
 // ---------------------------------------------------------------------------
 // Forward for rows beyond the registers of one workgroup, in ONE pass over X: a
-// row is held in the registers of a team of workgroups.  The grid is at most one
-// workgroup of 1024 threads a compute unit, all resident at once; workgroup b
-// belongs to team b / team and keeps chunk b % team of the team's current row
-// (up to 16 packs a lane: 256 KiB a workgroup, 64 MiB on 256 compute units).  It
-// sums its chunk (float64 sums about the row's centre, as the split-row kernels
-// below), publishes the two partial sums in its entry of library-owned device
-// memory and waits until every workgroup of its team has; each then adds the
-// team's partial sums in chunk order (the same statistics in every workgroup, run
-// to run), normalizes its chunk out of its registers and writes Y.  X is read once
-// and Y written once, where the split-row kernels read X twice (they remain for the
-// calls this kernel does not serve: a residual add, a cast, ragged rows, a stream
-// under capture).  Role in the reference: the split-row regime of Norm.h:632-812,
-// whose partial results also cross work-groups through global memory, between two
+// row is held in the registers of a team of workgroups.  The grid is at most two
+// workgroups of 512 threads a compute unit, all resident at once; workgroup b
+// belongs to team b / team and keeps chunk b % team of the team's current row: V
+// packs a lane, V * 512 packs a workgroup (up to 16: 128 KiB a workgroup, 64 MiB on
+// 256 compute units; the last chunk of a row may hold fewer).  It sums its chunk
+// (float64 sums about the row's centre, as the split-row kernels below), publishes
+// the two partial sums in its entry of library-owned device memory and waits until
+// every workgroup of its team has; each then adds the team's partial sums in chunk
+// order (the same statistics in every workgroup, run to run), normalizes its chunk
+// out of its registers and writes Y.  X is read once and Y written once, where the
+// split-row kernels read X twice (they remain for the calls this kernel does not
+// serve: a residual add, a cast, ragged rows, Y on top of X, a stream under
+// capture).  Role in the reference: the split-row regime of Norm.h:632-812, whose
+// partial results also cross work-groups through global memory, between two
 // launches.
 //
-// What crosses workgroups.  An entry is {tag, s1, s2}; the tag of a finished entry is
-// (call id << 32) | (round + 1), ids being unique per call, so nothing has to be
-// cleared and an entry left by an earlier call or round never counts.  The writer
-// sets the tag to 0 when it starts on a row, later stores s1 and s2, waits for
-// those stores to be acknowledged and stores the tag; a reader accepts s1 and s2
-// only if it read the expected tag before and after them.  Every access is a
-// device-scope atomic store or load, which goes to memory: no read-modify-write (256
-// workgroups counting on one word took hundreds of microseconds), and no release
-// or acquire fence (each writes back or invalidates a whole L2).  Two calls that
-// were handed the same slot while both run -- possible only with more such calls
-// in flight than slots -- overwrite each other's tags and therefore never accept
-// each other's sums.
+// A full chunk runs straight-line code: V unconditional loads in flight a lane,
+// and on the way out the weights of the next kTeamGroup packs are requested before
+// the current ones are normalized and stored, so no pack waits for the store of the
+// pack before it (bf16 [512, 401408]: 177 -> 170 us).
 //
-// The wait is bounded.  A workgroup stops waiting when its team is complete, when
-// any workgroup of the call has given up (a hint word in the slot), or after
-// `wait_ticks` of the constant-rate clock (the workgroups can only fail to be
-// resident together while other kernels hold compute units for that long).  A
-// workgroup that gives up leaves at once; one that has finished all its rows
-// stores the call id in its `done` entry.  The launch that follows on the stream,
-// norm_fwd_stream_kernel, returns at once when it finds the id in the `done`
-// entries of the whole grid and otherwise computes the whole call in the two-pass
-// way.  Every wave reaches an exit whatever the other workgroups do.
+// What crosses workgroups.  An entry is {tag, s1, s2}, 128 bytes apart; the tag of a
+// finished entry is (call id << 32) | (round + 1), ids being unique per call, so
+// nothing has to be cleared and an entry left by an earlier call or round never
+// counts.  The writer sets the tag to 0 when it starts on a row, later stores s1
+// and s2, waits for those stores to be acknowledged and stores the tag; a reader
+// accepts s1 and s2 only if it read the expected tag before and after them.  Every
+// access is a device-scope atomic store or load, which goes to memory: no
+// read-modify-write (256 workgroups counting on one word took hundreds of
+// microseconds), and no release or acquire fence (each writes back or invalidates a
+// whole L2).  Two calls that were handed the same slot while both run -- possible
+// only with more such calls in flight than slots -- overwrite each other's tags and
+// therefore never accept each other's sums.
+//
+// The wait is bounded, and no workgroup depends on another to finish.  A workgroup
+// stops waiting when its team is complete, when any workgroup of the call has given
+// up before (a hint word in the slot), or after `wait_ticks` of the constant-rate
+// clock (the workgroups can only fail to be resident together while other kernels
+// hold compute units for that long).  A workgroup that stops without its team sums
+// the whole row itself -- a second pass over X, whose statistics agree with the
+// team's to rounding -- loads its chunk again and goes on; it keeps publishing its
+// partial sums for the workgroups that do wait.  Every wave reaches the end of the
+// kernel whatever the other workgroups do, and every row is written.
 template <class T, class WT, int V, bool RMS>
-__global__ void __launch_bounds__(kTeamBlock)
+__global__ void __launch_bounds__(kTeamBlock, kTeamPerCu * kTeamBlock / 256)
 norm_fwd_team_kernel(const T* __restrict__ x, const WT* __restrict__ gamma,
                      const WT* __restrict__ beta, T* __restrict__ y, float* __restrict__ mean,
                      float* __restrict__ rstd, int64_t M, int N, float eps, int team,
@@ -771,11 +756,32 @@ norm_fwd_team_kernel(const T* __restrict__ x, const WT* __restrict__ gamma,
   // pointer per pack and one 32-bit byte offset a lane (no 64-bit address a pack in
   // vector registers, which 16 packs a lane have no room for).
   const int nloc = p1 > p0 ? (int)(p1 - p0) : 0;  // packs of this chunk
+  const bool full = nloc == V * BLOCK;  // (uniform) every lane holds V packs: all chunks but a row's last
   const int64_t pbase = nloc > 0 ? p0 : 0;
   const uint32_t loff = (uint32_t)(threadIdx.x * 16);
+  // (the sum is formed as a pointer into global memory: a pointer made from an integer
+  // is otherwise a generic one, and generic accesses wait for everything outstanding)
   auto at = [](auto* p, uint32_t off) {
-    using P = decltype(p);
-    return reinterpret_cast<P>(reinterpret_cast<uintptr_t>(p) + off);
+    using Elem = std::remove_pointer_t<decltype(p)>;
+    typedef __attribute__((address_space(1))) Elem* GlobalPtr;
+    return (Elem*)reinterpret_cast<GlobalPtr>(reinterpret_cast<uintptr_t>(p) + off);
+  };
+  // mean = hi + lo and rstd of a row from its centred sums (see the split-row kernels)
+  auto set_stats = [&](double t1, double t2, double kd) {
+    if constexpr (RMS) {
+      stat[0] = 0.0f;
+      stat[1] = 0.0f;
+      stat[2] = (float)(1.0 / sqrt(t2 / dN + (double)eps));
+    } else {
+      const double m1 = t1 / dN;
+      const double mu = kd + m1;
+      double var = (t2 - t1 * m1) / dN;
+      var = var < 0.0 ? 0.0 : var;  // (a select: NaN stays NaN)
+      const float hi = (float)mu;
+      stat[0] = var == var ? hi : (float)var;  // NaN variance: NaN mean
+      stat[1] = (float)(mu - (double)hi);
+      stat[2] = (float)(1.0 / sqrt(var + (double)eps));
+    }
   };
   unsigned int round = 0;
   for (int64_t row = tm; row < M; row += teams, ++round) {
@@ -784,11 +790,17 @@ norm_fwd_team_kernel(const T* __restrict__ x, const WT* __restrict__ gamma,
     const T* xr = x + row * (int64_t)N;
     const T* xb = xr + pbase * E;
     Pack<T, E> xp[V];
+    if (full) {
+      // (straight-line code: V requests in flight a lane, nothing conditional)
 #pragma unroll
-    for (int k = 0; k < V; ++k) {
-      xp[k] = Pack<T, E>::zero();
-      if (k * BLOCK + (int)threadIdx.x < nloc)
-        xp[k] = Pack<T, E>::load_stream(at(xb + k * BLOCK * E, loff));
+      for (int k = 0; k < V; ++k) xp[k] = Pack<T, E>::load_stream(at(xb + k * BLOCK * E, loff));
+    } else {
+#pragma unroll
+      for (int k = 0; k < V; ++k) {
+        xp[k] = Pack<T, E>::zero();
+        if (k * BLOCK + (int)threadIdx.x < nloc)
+          xp[k] = Pack<T, E>::load_stream(at(xb + k * BLOCK * E, loff));
+      }
     }
     const float kf = RMS ? 0.0f : split_row_centre(xr, (const T*)nullptr, N);
     const double kd = (double)kf;
@@ -796,7 +808,7 @@ norm_fwd_team_kernel(const T* __restrict__ x, const WT* __restrict__ gamma,
 #pragma unroll
     for (int k = 0; k < V; ++k) {
       keep_packed(xp[k]);
-      if (k * BLOCK + (int)threadIdx.x < nloc)
+      if (full || k * BLOCK + (int)threadIdx.x < nloc)
         add_centred_sums<T, E, RMS, true>(xp[k], E, kf, kd, s1, s2);
     }
     block_sum2_f64<BLOCK>(s1, s2, red);
@@ -814,6 +826,7 @@ norm_fwd_team_kernel(const T* __restrict__ x, const WT* __restrict__ gamma,
       const TeamEntry* mates = entries + tm * team;
       const unsigned long long t0 = wall_clock64();
       bool complete = false;
+      unsigned int polls = 0;
       for (;;) {
         bool ok = true;
         for (int j = lane; j < team; j += 64) ok = ok && team_load(&mates[j].tag) == expect;
@@ -829,10 +842,14 @@ norm_fwd_team_kernel(const T* __restrict__ x, const WT* __restrict__ gamma,
             break;
           }
         }
-        const unsigned int hint =
-            __hip_atomic_load(&slot->gave_up, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
-        if (hint == call_id || wall_clock64() - t0 > wait_ticks) break;
-        __builtin_amdgcn_s_sleep(2);
+        // (the hint word is one address for the whole grid: looked at every 16th time)
+        if ((polls++ & 15u) == 0) {
+          const unsigned int hint =
+              __hip_atomic_load(&slot->gave_up, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+          if (hint == call_id) break;
+        }
+        if (wall_clock64() - t0 > wait_ticks) break;
+        __builtin_amdgcn_s_sleep(8);
       }
       // (the lanes of a wavefront see one another's LDS stores in program order)
       if (lane == 0) {
@@ -845,26 +862,28 @@ norm_fwd_team_kernel(const T* __restrict__ x, const WT* __restrict__ gamma,
             t1 += tpart[j][0];
             t2 += tpart[j][1];
           }
-          if constexpr (RMS) {
-            stat[0] = 0.0f;
-            stat[1] = 0.0f;
-            stat[2] = (float)(1.0 / sqrt(t2 / dN + (double)eps));
-          } else {
-            const double m1 = t1 / dN;
-            const double mu = kd + m1;
-            double var = (t2 - t1 * m1) / dN;
-            var = var < 0.0 ? 0.0 : var;  // (a select: NaN stays NaN)
-            const float hi = (float)mu;
-            stat[0] = var == var ? hi : (float)var;  // NaN variance: NaN mean
-            stat[1] = (float)(mu - (double)hi);
-            stat[2] = (float)(1.0 / sqrt(var + (double)eps));
-          }
+          set_stats(t1, t2, kd);
           stat[3] = 0.0f;
         }
       }
     }
     __syncthreads();
-    if (stat[3] != 0.0f) return;  // (uniform over the workgroup)
+    if (stat[3] != 0.0f) {  // (uniform over the workgroup)
+      // The team did not come together: this workgroup sums the whole row itself (the
+      // row is X, which no workgroup writes), then takes its chunk again, whose
+      // registers the pass over the row has used.
+      double w1 = 0.0, w2 = 0.0;
+      long_row_sums<T, E, BLOCK, RMS, false>(xr, (const T*)nullptr, N, 0, npacks, kf, w1, w2);
+      block_sum2_f64<BLOCK>(w1, w2, red);
+      if (threadIdx.x == 0) set_stats(w1, w2, kd);
+      __syncthreads();
+#pragma unroll
+      for (int k = 0; k < V; ++k) {
+        xp[k] = Pack<T, E>::zero();
+        if (k * BLOCK + (int)threadIdx.x < nloc)
+          xp[k] = Pack<T, E>::load_stream(at(xb + k * BLOCK * E, loff));
+      }
+    }
     const float hi = stat[0], lo = stat[1], rs = stat[2];
     T* yb = y + row * (int64_t)N + pbase * E;
     const WT* gb = (hg ? gamma : reinterpret_cast<const WT*>(x)) + pbase * E;
@@ -872,6 +891,65 @@ norm_fwd_team_kernel(const T* __restrict__ x, const WT* __restrict__ gamma,
     // (opaque: the 2 * V weight addresses, the same for every row, would otherwise be
     // formed once ahead of the row loop and kept -- spilled -- across it)
     const uint32_t woff = (uint32_t)(lane_again((int)threadIdx.x) * E * (int)sizeof(WT));
+    auto normalized = [&](const Pack<T, E>& xk, const Pack<WT, E>& g, const Pack<WT, E>& b) {
+      Pack<T, E> o;
+#pragma unroll
+      for (int i = 0; i < E; ++i) {
+        float v;
+        if constexpr (RMS)
+          v = (xk.get(i) * rs) * g.get(i);
+        else
+          v = (((xk.get(i) - hi) - lo) * rs) * g.get(i) + b.get(i);
+        o.set(i, v);
+      }
+      return o;
+    };
+    if (full && hg && (RMS || hb)) {
+      // A full chunk with its weights: straight-line code in groups of kTeamGroup packs.
+      // The weights of the next group are requested before the current group is worked
+      // on and stored, so the wait for a group's weights never includes the stores of
+      // the group before it (requests complete in order: behind a conditional store,
+      // or a weight load issued after it, every pack would wait for the one before to
+      // be written).
+      // (as many packs' weights ahead as the registers beside the row allow: two, one,
+      // or -- 16 packs a lane with float32 weights beside 16-bit rows -- none)
+      constexpr int WP = (RMS ? 1 : 2) * (int)sizeof(WT) * E / 4;  // registers of a pack's weights
+      constexpr int ROOM = 92 - 4 * V;
+      constexpr int GS = ROOM >= 4 * WP ? kTeamGroup : 1, NG = (V + GS - 1) / GS;
+      constexpr int NB = ROOM >= 2 * WP ? 2 : 1;
+      Pack<WT, E> wg[NB][GS], wb[RMS ? 1 : NB][RMS ? 1 : GS];
+      auto request = [&](int g, int buf) {
+#pragma unroll
+        for (int u = 0; u < GS; ++u) {
+          const int k = g * GS + u;
+          if (k < V) {
+            wg[buf][u] = Pack<WT, E>::load(at(gb + k * BLOCK * E, woff));
+            if constexpr (!RMS) wb[buf][u] = Pack<WT, E>::load(at(bb + k * BLOCK * E, woff));
+          }
+        }
+      };
+      if constexpr (NB == 2) request(0, 0);
+#pragma unroll
+      for (int g = 0; g < NG; ++g) {
+        if constexpr (NB == 2) {
+          if (g + 1 < NG) request(g + 1, (g + 1) & 1);
+        } else {
+          request(g, 0);
+        }
+        __builtin_amdgcn_sched_barrier(0);
+#pragma unroll
+        for (int u = 0; u < GS; ++u) {
+          const int k = g * GS + u;
+          if (k < V) {
+            keep_packed(xp[k]);
+            const int buf = NB == 2 ? (g & 1) : 0;
+            const Pack<T, E> o = normalized(xp[k], wg[buf][u], wb[RMS ? 0 : buf][RMS ? 0 : u]);
+            o.store_stream(at(yb + k * BLOCK * E, loff));
+          }
+        }
+        __builtin_amdgcn_sched_barrier(0);
+      }
+    } else {
 #pragma unroll
     for (int k = 0; k < V; ++k) {
       if (k * BLOCK + (int)threadIdx.x < nloc) {
@@ -880,18 +958,9 @@ norm_fwd_team_kernel(const T* __restrict__ x, const WT* __restrict__ gamma,
             hg ? Pack<WT, E>::load(at(gb + k * BLOCK * E, woff)) : Pack<WT, E>::splat(1.0f);
         const Pack<WT, E> b =
             hb ? Pack<WT, E>::load(at(bb + k * BLOCK * E, woff)) : Pack<WT, E>::zero();
-        Pack<T, E> o;
-#pragma unroll
-        for (int i = 0; i < E; ++i) {
-          float v;
-          if constexpr (RMS)
-            v = (xp[k].get(i) * rs) * g.get(i);
-          else
-            v = (((xp[k].get(i) - hi) - lo) * rs) * g.get(i) + b.get(i);
-          o.set(i, v);
-        }
-        o.store_stream(at(yb + k * BLOCK * E, loff));
+        normalized(xp[k], g, b).store_stream(at(yb + k * BLOCK * E, loff));
       }
+    }
     }
     if (c == 0 && threadIdx.x == 0) {
       if constexpr (!RMS)
@@ -901,8 +970,6 @@ norm_fwd_team_kernel(const T* __restrict__ x, const WT* __restrict__ gamma,
     // (stat[], tpart[] and red[] are rewritten for the next row only behind the barrier
     // inside the next block sum, which every thread reaches after it has read them)
   }
-  if (threadIdx.x == 0)
-    __hip_atomic_store(&slot->done[blockIdx.x], call_id, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
 }
 
 // ---------------------------------------------------------------------------

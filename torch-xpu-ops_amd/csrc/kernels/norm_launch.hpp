@@ -48,8 +48,8 @@ inline bool norm_fwd_can_split(const Plan& plan, const NormFwdArgs& a) {
 
 // Whether norm_fwd_team_kernel serves the call: planned, its bookkeeping memory at
 // hand (the caller of this function withholds it on a stream under capture), no
-// residual add, Y in the row dtype.  Y may be the memory of X: a workgroup has read
-// all it needs of its chunk before it writes.
+// residual add, Y in the row dtype.  (The caller also withholds the memory when Y
+// overlaps X: a workgroup whose team does not come together reads the whole row.)
 template <class T, class TY, bool ADD>
 inline bool norm_fwd_team_serves(const Plan& plan, const NormFwdArgs& a) {
   return plan.team > 0 && a.team_slot != nullptr && !ADD && std::is_same<T, TY>::value &&
@@ -91,8 +91,7 @@ int launch_norm_fwd(const Plan& plan, const NormFwdArgs& a, hipStream_t stream) 
             : launch_variant<NormFwdLauncher<T, WT, RMS, false, TY, ADD>::template At>(ctx);
     if (!launched) return (int)hipErrorInvalidConfiguration;
   } else if (norm_fwd_team_serves<T, TY, ADD>(plan, a)) {
-    // one pass with the row in the registers of a team of workgroups; should that
-    // launch not complete (see the kernel), the guarded launch behind it does the work
+    // one pass with the row in the registers of a team of workgroups
     TeamSlot* slot = (TeamSlot*)a.team_slot;
     auto go = [&](auto v) {
       constexpr int V = decltype(v)::value;
@@ -101,18 +100,16 @@ int launch_norm_fwd(const Plan& plan, const NormFwdArgs& a, hipStream_t stream) 
                          (const WT*)a.beta, (T*)a.y, a.mean, a.rstd, a.M, a.N, a.eps, plan.team,
                          plan.team_chunk_packs, slot, a.team_id, a.team_wait_ticks);
     };
+    static_assert(kTeamMaxV == 16, "one case per pack count below");
     switch (plan.team_v) {
-      case 2: go(std::integral_constant<int, 2>{}); break;
-      case 4: go(std::integral_constant<int, 4>{}); break;
-      case 8: go(std::integral_constant<int, 8>{}); break;
-      case 16: go(std::integral_constant<int, 16>{}); break;
+#define ROWNORM_TEAM_CASE(v) case v: go(std::integral_constant<int, v>{}); break;
+      ROWNORM_TEAM_CASE(1) ROWNORM_TEAM_CASE(2) ROWNORM_TEAM_CASE(3) ROWNORM_TEAM_CASE(4)
+      ROWNORM_TEAM_CASE(5) ROWNORM_TEAM_CASE(6) ROWNORM_TEAM_CASE(7) ROWNORM_TEAM_CASE(8)
+      ROWNORM_TEAM_CASE(9) ROWNORM_TEAM_CASE(10) ROWNORM_TEAM_CASE(11) ROWNORM_TEAM_CASE(12)
+      ROWNORM_TEAM_CASE(13) ROWNORM_TEAM_CASE(14) ROWNORM_TEAM_CASE(15) ROWNORM_TEAM_CASE(16)
+#undef ROWNORM_TEAM_CASE
       default: return (int)hipErrorInvalidConfiguration;
     }
-    if (int e = (int)hipGetLastError()) return e;
-    hipLaunchKernelGGL((norm_fwd_stream_kernel<T, WT, kStreamBlock, RMS, TY>),
-                       dim3((unsigned)plan.grid), dim3(kStreamBlock), 0, stream, (const T*)a.x,
-                       res, (const WT*)a.gamma, (const WT*)a.beta, h, (TY*)a.y, a.mean, a.rstd,
-                       a.M, a.N, a.eps, (const TeamSlot*)slot, (int)plan.team_grid, a.team_id);
   } else if (norm_fwd_can_split<T, TY, RMS>(plan, a)) {
     const dim3 grid((unsigned)plan.split, (unsigned)a.M);
     hipLaunchKernelGGL((norm_fwd_split_sums_kernel<T, kStreamBlock, RMS, TY>), grid,

@@ -76,20 +76,21 @@ struct Plan {
 
 // norm_fwd_team_kernel: threads a workgroup, packs a lane at most, workgroups of
 // the grid at most (one a compute unit), slots of bookkeeping memory.
-constexpr int kTeamBlock = 1024;
+constexpr int kTeamBlock = 512;
+constexpr int kTeamPerCu = 2;  // workgroups of a team launch a compute unit holds
 constexpr int kTeamMaxV = 16;
-constexpr int kTeamMaxWorkgroups = 256;
-constexpr int kTeamSlots = 32;
+constexpr int kTeamGroup = 2;  // packs whose weights are requested together
+constexpr int kTeamMaxWorkgroups = 512;
+constexpr int kTeamSlots = 16;
 constexpr int kTeamMinTeams = 8;
 // One call's bookkeeping memory (see the kernel).
 struct TeamEntry {
   unsigned long long tag;  // (call id << 32) | (round + 1) once s1, s2 are in place; 0 while they change
   unsigned long long s1, s2;  // a workgroup's partial sums (float64 bit patterns)
-  unsigned long long pad;
+  unsigned long long pad[13];  // 128 bytes an entry: neighbours' polls go to other memory channels
 };
 struct TeamSlot {
   TeamEntry entry[2][kTeamMaxWorkgroups];  // [round parity][workgroup]
-  unsigned int done[kTeamMaxWorkgroups];   // id of the call the workgroup last completed
   unsigned int gave_up;                    // id of a call one of whose waits ran out (a hint)
   unsigned int pad[3];
 };
@@ -893,7 +894,7 @@ inline int make_plan(OpClass oc, int64_t M, int64_t N, int esize, int num_cus, c
   // all the workgroups its team can have (down to one stride of 1024 packs each).
   if (oc == OC_NORM_FWD && !p.resident && p.fast && !fused_add && ov.G == 0 && ov.V == 0 &&
       ov.bpc == 0) {
-    const int64_t cus = num_cus < kTeamMaxWorkgroups ? num_cus : kTeamMaxWorkgroups;
+    const int64_t cus = num_cus * kTeamPerCu < kTeamMaxWorkgroups ? num_cus * kTeamPerCu : kTeamMaxWorkgroups;
     const int64_t per_wg = (int64_t)kTeamBlock * kTeamMaxV;
     const int64_t team_min = (packs + per_wg - 1) / per_wg;
     int64_t teams = team_min <= cus ? cus / team_min : 0;
@@ -905,16 +906,16 @@ inline int make_plan(OpClass oc, int64_t M, int64_t N, int esize, int num_cus, c
     // 11.6 us; 8 teams ([8, 4194304], one round) 35.1 against 40.5 us, 64 teams
     // ([512, 401408], 8 rounds) 177 against 196 us.
     if (teams >= kTeamMinTeams) {
-      int64_t team = cus / teams;
+      // a chunk is a whole number of workgroup strides, exactly the packs a lane the
+      // kernel is compiled for: every workgroup but a row's last runs straight-line code
+      int64_t team_max = cus / teams;
       const int64_t strides = (packs + kTeamBlock - 1) / kTeamBlock;
-      if (team > strides) team = strides;
-      const int64_t chunk = (packs + team - 1) / team;
-      const int64_t need = (chunk + kTeamBlock - 1) / kTeamBlock;
-      int v = 2;
-      while (v < need) v *= 2;
+      if (team_max > strides) team_max = strides;
+      const int64_t v = (strides + team_max - 1) / team_max;
+      const int64_t team = (strides + v - 1) / v;
       p.team = (int)team;
-      p.team_v = v;
-      p.team_chunk_packs = chunk;
+      p.team_v = (int)v;
+      p.team_chunk_packs = v * kTeamBlock;
       p.team_grid = teams * team;
     }
   }
