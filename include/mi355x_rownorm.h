@@ -382,16 +382,17 @@ int mi355x_rownorm_set_override(rownorm_op op, int lanes_per_row, int packs_per_
 
 /* Test hook for the forward of rows that a team of workgroups holds in registers
  * (LayerNorm / RMSNorm rows beyond 131072 16-bit or 65536 float32 elements, whole
- * 16-byte packs, no residual add, no cast): how long a workgroup waits for the
- * others of its team before the call falls back to the two-pass kernel that is
- * enqueued behind it, in microseconds; 0xffffffff restores the default, one second.
- * 0 makes every wait give up at once, which is how the tests exercise the fallback
- * without making any kernel hang.  Process-global.  Such calls draw an id and one
- * of 32 bookkeeping slots in library-owned device memory from process-wide
- * counters; results do not depend on which slot a call gets, and two calls that
- * share a slot while both run (more than 32 such calls in flight across streams)
- * each detect it and take the fallback.  On a stream under capture these rows take
- * the multi-launch kernels instead. */
+ * 16-byte packs, no residual add, no cast, y not overlapping x): how long a
+ * workgroup waits for the others of its team before it sums the whole row itself
+ * (a second pass over x, the same result to rounding), in microseconds; 0xffffffff
+ * restores the default, one second.  0 makes every wait give up at once, which is
+ * how the tests exercise that path without making any kernel hang.  Process-global.
+ * Such calls draw an id and one of 16 bookkeeping slots in library-owned device
+ * memory from process-wide counters; results do not depend on which slot a call
+ * gets, and two calls that share a slot while both run (more than 16 such calls in
+ * flight across streams) each detect it, their workgroups summing their rows
+ * themselves.  On a stream under capture these rows take the multi-launch kernels
+ * instead. */
 int mi355x_rownorm_set_team_wait_us(unsigned int microseconds);
 
 /* Measurement aid, no counterpart in the reference: a plain streaming kernel over

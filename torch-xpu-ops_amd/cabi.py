@@ -178,7 +178,7 @@ def group_norm_plan(backward, N, C, HxW, groups, dtype=F32):
 
 def set_team_wait_us(microseconds=0xffffffff):
     """Bound of a workgroup's wait in the team forward (rows beyond one workgroup's registers);
-    0: every wait gives up at once and the two-pass kernel behind it does the work."""
+    0: every wait gives up at once and each workgroup sums its rows itself."""
     _check(lib().mi355x_rownorm_set_team_wait_us(ctypes.c_uint(microseconds)), "set_team_wait_us")
 
 
