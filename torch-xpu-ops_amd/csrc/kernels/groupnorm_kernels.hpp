@@ -115,6 +115,17 @@ template <class WT>
 __device__ __forceinline__ float gn_weight(const WT* w, int ch, float dflt) {
   return w ? (float)w[(unsigned)ch] : dflt;  // ch >= 0: a 32-bit offset from a scalar base
 }
+// The same when the caller knows whether the weight exists (HAVE): with it, a plain
+// load.  The test of the pointer above is a branch around the load, and the join of
+// a branch waits for every request outstanding, so lookups that go through it
+// complete one after the other, each behind whatever was stored before it.
+template <bool HAVE, class WT>
+__device__ __forceinline__ float gn_weight_known(const WT* w, int ch, float dflt) {
+  if constexpr (HAVE)
+    return (float)w[(unsigned)ch];
+  else
+    return gn_weight(w, ch, dflt);
+}
 
 // ---------------------------------------------------------------------------
 // Forward, row resident in registers.  Statistics as in the LayerNorm kernel:
@@ -197,37 +208,72 @@ gn_fwd_resident_kernel(const T* __restrict__ x, const WT* __restrict__ gamma,
     var = var < 0.0f ? 0.0f : var;  // a select, not v_max_f32: a NaN row keeps NaN statistics
     const float rs = row_rstd_of<T>(var + eps);
     T* yr = y + row * (int64_t)s.L;
+    if constexpr (UNIFORM) {
+      // The weights of pack c + 1 are requested before pack c is normalized and stored:
+      // requests complete in order, stores included, so a pack that looked its weights
+      // up on its own turn waited for the store of the pack before it.
+      struct PackWeights {
+        float ga0, ga1, be0, be1;
+        int bnd;
+      };
+      auto normalize = [&](auto have) {
+        constexpr bool HAVE = decltype(have)::value;  // gamma and beta both given
+        auto lookup = [&](int c) {
+          PackWeights w;
+          if constexpr (STRADDLE) {
+            const GnStraddle sw = gn_straddle(s, (c * G + lane) * E, E);
+            const int c0 = g * s.D + sw.ch;
+            const int c1 = sw.ch + 1 < s.D ? c0 + 1 : c0;
+            w.ga0 = gn_weight_known<HAVE>(gamma, c0, 1.0f);
+            w.ga1 = gn_weight_known<HAVE>(gamma, c1, 1.0f);
+            w.be0 = gn_weight_known<HAVE>(beta, c0, 0.0f);
+            w.be1 = gn_weight_known<HAVE>(beta, c1, 0.0f);
+            w.bnd = sw.bnd;
+          } else {
+            const int ch = gn_pack_channel(s, g, c * G + lane);
+            w.ga0 = w.ga1 = gn_weight_known<HAVE>(gamma, ch, 1.0f);
+            w.be0 = w.be1 = gn_weight_known<HAVE>(beta, ch, 0.0f);
+            w.bnd = E;
+          }
+          return w;
+        };
+        PackWeights wn = lookup(0);
 #pragma unroll
-    for (int c = 0; c < V; ++c) {
-      keep_packed(xp[c]);
-      const int e0 = (c * G + lane) * E;
-      Pack<T, E> o;
-      if constexpr (STRADDLE) {
-        const GnStraddle w = gn_straddle(s, e0, E);
-        const int c0 = g * s.D + w.ch;
-        const int c1 = w.ch + 1 < s.D ? c0 + 1 : c0;
-        const float ga0 = gn_weight(gamma, c0, 1.0f) * rs, ga1 = gn_weight(gamma, c1, 1.0f) * rs;
-        const float be0 = gn_weight(beta, c0, 0.0f), be1 = gn_weight(beta, c1, 0.0f);
+        for (int c = 0; c < V; ++c) {
+          const PackWeights w = wn;
+          if (c + 1 < V) wn = lookup(c + 1);
+          __builtin_amdgcn_sched_barrier(0);
+          keep_packed(xp[c]);
+          const float ga0 = w.ga0 * rs, ga1 = w.ga1 * rs;
+          Pack<T, E> o;
 #pragma unroll
-        for (int i = 0; i < E; ++i) {
-          const bool first = i < w.bnd;
-          o.set(i, ((xp[c].get(i) - mean0) - m1) * (first ? ga0 : ga1) + (first ? be0 : be1));
+          for (int i = 0; i < E; ++i) {
+            const bool first = !STRADDLE || i < w.bnd;
+            o.set(i,
+                  ((xp[c].get(i) - mean0) - m1) * (first ? ga0 : ga1) + (first ? w.be0 : w.be1));
+          }
+          row_store<T, E, true, UNIFORM>(yr, (c * G + lane) * E, s.L, ok, o);
+          __builtin_amdgcn_sched_barrier(0);
         }
-      } else if constexpr (UNIFORM) {
-        const int ch = gn_pack_channel(s, g, c * G + lane);
-        const float ga = gn_weight(gamma, ch, 1.0f) * rs;
-        const float be = gn_weight(beta, ch, 0.0f);
+      };
+      if (gamma != nullptr && beta != nullptr)
+        normalize(std::true_type{});
+      else
+        normalize(std::false_type{});
+    } else {
 #pragma unroll
-        for (int i = 0; i < E; ++i) o.set(i, ((xp[c].get(i) - mean0) - m1) * ga + be);
-      } else {
+      for (int c = 0; c < V; ++c) {
+        keep_packed(xp[c]);
+        const int e0 = (c * G + lane) * E;
+        Pack<T, E> o;
 #pragma unroll
         for (int i = 0; i < E; ++i) {
           const int ch = gn_channel(s, g, e0 + i);
           const float ga = gn_weight(gamma, ch, 1.0f) * rs;
           o.set(i, ((xp[c].get(i) - mean0) - m1) * ga + gn_weight(beta, ch, 0.0f));
         }
+        row_store<T, E, true, UNIFORM>(yr, e0, s.L, ok, o);
       }
-      row_store<T, E, true, UNIFORM>(yr, e0, s.L, ok, o);
     }
     if (ok && lane == 0) {
       if (mean) mean[row] = (WT)(rs == rs ? mean0 + m1 : rs);  // NaN variance: NaN mean

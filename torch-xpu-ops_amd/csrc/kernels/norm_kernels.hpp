@@ -314,6 +314,24 @@ norm_fwd_resident_kernel(const T* __restrict__ x, const T* res, const WT* __rest
 #pragma unroll
     for (int r = 0; r < R; ++r) {
       TY* yr = y + (row0 + r) * (int64_t)N - hd;
+      // Weights that are not held (rows of whole packs only) are looked up with plain
+      // loads, pack c + 1 before pack c is stored.  A test of the pointer would be a
+      // branch around the load, whose join waits for every request outstanding, and
+      // requests complete in order: a lookup issued behind a store waits for that store.
+      // An absent weight is read from the head of X (such a row is long enough) and
+      // replaced.
+      auto lookup = [&](const WT* w, int c, float dflt) {
+        const bool have = w != nullptr;
+        Pack<WT, E> p = row_load<WT, E, false, true>(
+            have ? w : reinterpret_cast<const WT*>(x), have ? (c * G + ls) * E : 0, N, true, dflt);
+        if (!have) p = Pack<WT, E>::splat(dflt);
+        return p;
+      };
+      Pack<WT, E> gahead, bahead;
+      if constexpr (!kHold) {
+        gahead = lookup(gamma, 0, 1.0f);
+        if constexpr (!RMS) bahead = lookup(beta, 0, 0.0f);
+      }
 #pragma unroll
       for (int c = 0; c < V; ++c) {
         keep_packed(xp[r][c]);
@@ -326,11 +344,13 @@ norm_fwd_resident_kernel(const T* __restrict__ x, const T* res, const WT* __rest
         }
         Pack<WT, E> gl, bl;
         if constexpr (!kHold) {
-          const int e0 = (c * G + ls) * E;
-          gl = gamma ? load_row_pack<WT, E, false>(gamma, e0, N, true, 1.0f)
-                     : Pack<WT, E>::splat(1.0f);
-          if constexpr (!RMS)
-            bl = beta ? load_row_pack<WT, E, false>(beta, e0, N, true, 0.0f) : Pack<WT, E>::zero();
+          gl = gahead;
+          if constexpr (!RMS) bl = bahead;
+          if (c + 1 < V) {
+            gahead = lookup(gamma, c + 1, 1.0f);
+            if constexpr (!RMS) bahead = lookup(beta, c + 1, 0.0f);
+          }
+          __builtin_amdgcn_sched_barrier(0);
         }
         const Pack<WT, E>& gc = kHold ? gp[kHold ? c : 0] : gl;
         const Pack<WT, E>& bc = RMS ? gc : (kHold ? bp[kHold && !RMS ? c : 0] : bl);
@@ -349,6 +369,7 @@ norm_fwd_resident_kernel(const T* __restrict__ x, const T* res, const WT* __rest
           o.set(i, v);
         }
         row_store<TY, E, true, FAST>(yr, (c * G + ls) * E, nw, ok[r], o, hd);
+        if constexpr (!kHold) __builtin_amdgcn_sched_barrier(0);
       }
       if (ok[r] && lane0 == 0) {
         if constexpr (!RMS)
@@ -1191,10 +1212,18 @@ norm_bwd_resident_kernel(const T* __restrict__ dy, const T* __restrict__ x, cons
   }
   // the weights of pack c, for the lane index `ln` (LDSG: made opaque per use, so the
   // pack offsets are not carried across the row loop)
+  // (LDSG: a plain load, nothing conditional -- a test of the pointer is a branch around
+  // the load, and the join of a branch waits for every request outstanding, the stores
+  // of the packs before included.  Without gamma the load goes to the head of dY, which
+  // such a row makes long enough, and its result is replaced.)
+  const bool have_g = gamma != nullptr;
+  const WT* wsrc = have_g ? gamma : reinterpret_cast<const WT*>(dy);
   auto weights = [&](int c, int ln) {
     if constexpr (LDSG) {
-      return gamma ? load_row_pack<WT, E, false>(gamma, (c * G + ln) * E, N, true, 1.0f)
-                   : Pack<WT, E>::splat(1.0f);
+      Pack<WT, E> w =
+          row_load<WT, E, false, true>(wsrc, have_g ? (c * G + ln) * E : 0, N, true, 1.0f);
+      if (!have_g) w = Pack<WT, E>::splat(1.0f);
+      return w;
     } else {
       return gp[c];
     }
@@ -1312,12 +1341,25 @@ norm_bwd_resident_kernel(const T* __restrict__ dy, const T* __restrict__ x, cons
             up[c] = row_load<T, E, true, FAST>(dres + (ok[r] ? row0 + r : 0) * (int64_t)N,
                                                (c * G + ls) * E, N, ok[r], 0.0f);
         }
+        // (LDSG, gamma looked up again: the weights of pack c + 1 are requested before
+        // pack c is stored -- requests complete in order, so a lookup issued behind a
+        // store would wait for that store)
+        constexpr bool kAhead = LDSG && !kKeepG;
+        Pack<WT, E> gahead;
+        if constexpr (kAhead) gahead = weights(0, ls);
 #pragma unroll
         for (int c = 0; c < V; ++c) {
           keep_packed(xp[r][c]);
           keep_packed(dp[r][c]);
           if constexpr (!LDSG && !kWideWeights) keep_packed(gp[c]);
-          const Pack<WT, E> gc = kKeepG ? gk[kKeepG ? c : 0] : weights(c, ls);
+          Pack<WT, E> gc;
+          if constexpr (kAhead) {
+            gc = gahead;
+            if (c + 1 < V) gahead = weights(c + 1, ls);
+            __builtin_amdgcn_sched_barrier(0);
+          } else {
+            gc = kKeepG ? gk[kKeepG ? c : 0] : weights(c, ls);
+          }
           Pack<T, E> o;
 #pragma unroll
           for (int i = 0; i < E; ++i) {
@@ -1337,6 +1379,7 @@ norm_bwd_resident_kernel(const T* __restrict__ dy, const T* __restrict__ x, cons
             o.set(i, f);
           }
           row_store<T, E, true, FAST>(dr, (c * G + ls) * E, N, ok[r], o);
+          if constexpr (kAhead) __builtin_amdgcn_sched_barrier(0);
         }
       }
     }
