@@ -699,23 +699,34 @@ softmax_strided_split_bwd_partial_kernel(const TG* __restrict__ grad, const TG* 
     float sum[E], unused[E];
 #pragma unroll
     for (int i = 0; i < E; ++i) sum[i] = unused[i] = 0.0f;
-    for (int d = d0 + ty; d < d1; d += TY * U) {
-      Pack<TG, E> pg[U], py[U];
+    // (one loop per variant: a test of the variant around the load of y inside the loop
+    // is a branch whose join waits for every request outstanding, which made the 2 * U
+    // loads of an iteration complete one after the other)
+    auto add_rows = [&](auto log_variant) {
+      constexpr bool LOG = decltype(log_variant)::value;
+      for (int d = d0 + ty; d < d1; d += TY * U) {
+        Pack<TG, E> pg[U], py[LOG ? 1 : U];
 #pragma unroll
-      for (int u = 0; u < U; ++u) {
-        const int dd = d + u * TY;
-        const bool ok = tile.valid && dd < d1;
-        const int64_t off = (int64_t)(ok ? dd : d0) * inner;
-        pg[u] = load_row_pack<TG, E, false>(gs + off, tile.e0, inner, ok, 0.0f);
-        py[u] = Pack<TG, E>::zero();
-        if (!is_log) py[u] = load_row_pack<TG, E, false>(ys + off, tile.e0, inner, ok, 0.0f);
+        for (int u = 0; u < U; ++u) {
+          const int dd = d + u * TY;
+          const bool ok = tile.valid && dd < d1;
+          const int64_t off = (int64_t)(ok ? dd : d0) * inner;
+          pg[u] = load_row_pack<TG, E, false>(gs + off, tile.e0, inner, ok, 0.0f);
+          if constexpr (!LOG)
+            py[u] = load_row_pack<TG, E, false>(ys + off, tile.e0, inner, ok, 0.0f);
+        }
+#pragma unroll
+        for (int u = 0; u < U; ++u)
+#pragma unroll
+          for (int i = 0; i < E; ++i)
+            sum[i] = LOG ? sum[i] + pg[u].get(i)
+                         : fmaf(py[LOG ? 0 : u].get(i), pg[u].get(i), sum[i]);
       }
-#pragma unroll
-      for (int u = 0; u < U; ++u)
-#pragma unroll
-        for (int i = 0; i < E; ++i)
-          sum[i] = is_log ? sum[i] + pg[u].get(i) : fmaf(py[u].get(i), pg[u].get(i), sum[i]);
-    }
+    };
+    if (is_log)
+      add_rows(std::true_type{});
+    else
+      add_rows(std::false_type{});
     column_allreduce<BLOCK, E, SumOp>(sum, lay, red, phase);
     if (ty == 0)
       split_slot_store<TO, E, 1>(gi + tile.slab + (int64_t)d0 * inner, inner, tile.e0, tile.valid,
