@@ -445,3 +445,30 @@ def test_group_norm_validation_and_plans(cabi):
     # the diffusion-UNet shape keeps its 40960-element rows in registers
     assert cabi.group_norm_plan(0, 2, 320, 4096, 32, cabi.BF16)["resident"] == 1
     assert cabi.group_norm_plan(1, 2, 320, 4096, 32, cabi.BF16)["resident"] == 1
+
+
+def test_plan_queries_of_empty_and_extreme_shapes(cabi):
+    """The plan and workspace queries take any shape the entry points accept, empty ones included
+    (the entry points return before they plan an empty call, the queries do not): no division by a
+    zero row or tile count, and a shape beyond the limits is an error code, not a crash."""
+    ops = (cabi.OP_LAYER_NORM_FWD, cabi.OP_LAYER_NORM_BWD, cabi.OP_RMS_NORM_FWD, cabi.OP_RMS_NORM_BWD,
+           cabi.OP_SOFTMAX_FWD, cabi.OP_SOFTMAX_BWD)
+    L = cabi.lib()
+    for op in ops:
+        for M, N in ((0, 0), (0, 4096), (0, 4194304), (5, 0), (0, 1), (1, 4194304), (3, 2 ** 30)):
+            for dt in (cabi.F32, cabi.BF16):
+                p = cabi.plan(op, M, N, dt, dt)
+                assert p["grid_blocks"] >= 0 and p["block_threads"] > 0, (op, M, N, p)
+        p = cabi.Plan()
+        assert L.mi355x_rownorm_plan(op, 1, 2 ** 30 + 1, cabi.F32, cabi.F32, p) < 0
+        assert L.mi355x_rownorm_plan(op, -1, 8, cabi.F32, cabi.F32, p) < 0
+    for M, N in ((0, 0), (0, 4194304), (7, 0)):
+        assert L.mi355x_layer_norm_bwd_workspace_bytes(M, N, cabi.BF16, cabi.BF16, 1, 1) == 0
+        assert L.mi355x_rms_norm_bwd_workspace_bytes(M, N, cabi.BF16, cabi.BF16, 1) == 0
+    for backward in (0, 1):
+        for outer, D, inner in ((0, 8, 8), (4, 0, 8), (4, 8, 0), (0, 0, 0), (1, 8192, 8192)):
+            p = cabi.strided_plan(backward, outer, D, inner, cabi.BF16)
+            assert p["grid_blocks"] >= 0, (outer, D, inner, p)
+        for N_, C, HxW in ((0, 32, 16), (4, 32, 0), (4, 0, 16)):
+            p = cabi.group_norm_plan(backward, N_, C, HxW, 32 if C else 1, cabi.BF16)
+            assert p["grid_blocks"] >= 0, (N_, C, HxW, p)

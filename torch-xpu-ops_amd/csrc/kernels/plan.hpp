@@ -870,7 +870,7 @@ inline int make_plan(OpClass oc, int64_t M, int64_t N, int esize, int num_cus, c
     int64_t want = 1;
     if (ov.G < 0 && ov.V > 0)
       want = ov.V;
-    else if (M < 2 * (int64_t)num_cus)
+    else if (M > 0 && M < 2 * (int64_t)num_cus)
       want = (4 * (int64_t)num_cus + M - 1) / M;
     if (want > kSplitMaxChunks) want = kSplitMaxChunks;
     if (want > 1) {
@@ -967,6 +967,12 @@ inline int make_strided_plan(bool backward, int64_t outer, int64_t D, int64_t in
   const int64_t packs = (inner + E - 1) / E;
   p.fast = (inner % E) == 0;
   p.block = kStridedBlock;
+  // an empty tensor launches nothing (the entry points return before they plan; the
+  // plan query gets a plan with no workgroups)
+  if (outer < 1 || D < 1 || inner < 1) {
+    *out = p;
+    return 0;
+  }
   if (num_cus <= 0) num_cus = 256;
   const int px = packs >= 64 ? 64 : pow2_ceil(packs);  // lanes a row of `inner` can use
   // packs a lane may hold: 8, or 4 for the 16-bit backward (two packed rows per
