@@ -501,64 +501,72 @@ gn_bwd_resident_kernel(const T* __restrict__ dy, const T* __restrict__ x,
     int bnd[STRADDLE ? V : 1];   //              and the elements that belong to the first
     float* st = stage + slot * (UNIFORM ? 2 * G * V : 0);
     float* sn = stage_next + slot * gn_stage_floats<G, V, BLOCK, MODE>::next_per_slot;
+    // (one copy of the loop per case of gamma: see gn_weight_known)
+    auto row_sums = [&](auto have) {
+      constexpr bool HAVE = decltype(have)::value;
 #pragma unroll
-    for (int c = 0; c < V; ++c) {
-      const int e0 = (c * G + lane) * E;
-      if constexpr (STRADDLE) {
-        const GnStraddle w = gn_straddle(s, e0, E);
-        const bool has_next = w.bnd < E && w.ch + 1 < s.D;
-        const float ga = gu[c] = gn_weight(gamma, g * s.D + w.ch, 1.0f);
-        const float gb = gv[c] = gn_weight(gamma, g * s.D + (has_next ? w.ch + 1 : w.ch), 1.0f);
-        bnd[c] = w.bnd;
-        float pdg = 0.0f, pdb = 0.0f, fdg = 0.0f, fdb = 0.0f;  // whole pack / first channel
+      for (int c = 0; c < V; ++c) {
+        const int e0 = (c * G + lane) * E;
+        if constexpr (STRADDLE) {
+          const GnStraddle w = gn_straddle(s, e0, E);
+          const bool has_next = w.bnd < E && w.ch + 1 < s.D;
+          const float ga = gu[c] = gn_weight_known<HAVE>(gamma, g * s.D + w.ch, 1.0f);
+          const float gb = gv[c] = gn_weight_known<HAVE>(gamma, g * s.D + (has_next ? w.ch + 1 : w.ch), 1.0f);
+          bnd[c] = w.bnd;
+          float pdg = 0.0f, pdb = 0.0f, fdg = 0.0f, fdb = 0.0f;  // whole pack / first channel
 #pragma unroll
-        for (int i = 0; i < E; ++i) {
-          const float gy = dp[c].get(i);
-          const float t = gy * (xp[c].get(i) - mu);
-          pdb += gy;
-          pdg += t;
-          fdb += i < w.bnd ? gy : 0.0f;
-          fdg += i < w.bnd ? t : 0.0f;
-        }
-        // (a pack that lies in one channel adds the same terms to both pairs: the
-        // second channel's share is then exactly zero)
-        const float ndg = pdg - fdg, ndb = pdb - fdb;
-        acc[0] = fmaf(fdb, ga, fmaf(ndb, gb, acc[0]));
-        acc[1] = fmaf(fdg * rs, ga, fmaf(ndg * rs, gb, acc[1]));
-        if (want_cols) {
-          st[2 * (c * G + lane)] = fdg * rs;
-          st[2 * (c * G + lane) + 1] = fdb;
-          if (has_next && e0 < s.L) {
-            sn[2 * (w.ch + 1)] = ndg * rs;
-            sn[2 * (w.ch + 1) + 1] = ndb;
+          for (int i = 0; i < E; ++i) {
+            const float gy = dp[c].get(i);
+            const float t = gy * (xp[c].get(i) - mu);
+            pdb += gy;
+            pdg += t;
+            fdb += i < w.bnd ? gy : 0.0f;
+            fdg += i < w.bnd ? t : 0.0f;
+          }
+          // (a pack that lies in one channel adds the same terms to both pairs: the
+          // second channel's share is then exactly zero)
+          const float ndg = pdg - fdg, ndb = pdb - fdb;
+          acc[0] = fmaf(fdb, ga, fmaf(ndb, gb, acc[0]));
+          acc[1] = fmaf(fdg * rs, ga, fmaf(ndg * rs, gb, acc[1]));
+          if (want_cols) {
+            st[2 * (c * G + lane)] = fdg * rs;
+            st[2 * (c * G + lane) + 1] = fdb;
+            if (has_next && e0 < s.L) {
+              sn[2 * (w.ch + 1)] = ndg * rs;
+              sn[2 * (w.ch + 1) + 1] = ndb;
+            }
+          }
+        } else if constexpr (UNIFORM) {
+          const float ga = gu[c] = gn_weight_known<HAVE>(gamma, gn_pack_channel(s, g, c * G + lane), 1.0f);
+          float pdg = 0.0f, pdb = 0.0f;
+#pragma unroll
+          for (int i = 0; i < E; ++i) {
+            const float gy = dp[c].get(i);
+            pdb += gy;
+            pdg = fmaf(gy, xp[c].get(i) - mu, pdg);
+          }
+          // zero-filled packs (row slot or pack out of range) add nothing
+          acc[0] = fmaf(pdb, ga, acc[0]);
+          acc[1] = fmaf(pdg * rs, ga, acc[1]);
+          if (want_cols) {
+            st[2 * (c * G + lane)] = pdg * rs;
+            st[2 * (c * G + lane) + 1] = pdb;
+          }
+        } else {
+#pragma unroll
+          for (int i = 0; i < E; ++i) {
+            const float ga = gn_weight_known<HAVE>(gamma, gn_channel(s, g, e0 + i), 1.0f);
+            const float gv = dp[c].get(i) * ga;
+            acc[0] += gv;
+            acc[1] = fmaf(gv, (xp[c].get(i) - mu) * rs, acc[1]);
           }
         }
-      } else if constexpr (UNIFORM) {
-        const float ga = gu[c] = gn_weight(gamma, gn_pack_channel(s, g, c * G + lane), 1.0f);
-        float pdg = 0.0f, pdb = 0.0f;
-#pragma unroll
-        for (int i = 0; i < E; ++i) {
-          const float gy = dp[c].get(i);
-          pdb += gy;
-          pdg = fmaf(gy, xp[c].get(i) - mu, pdg);
-        }
-        // zero-filled packs (row slot or pack out of range) add nothing
-        acc[0] = fmaf(pdb, ga, acc[0]);
-        acc[1] = fmaf(pdg * rs, ga, acc[1]);
-        if (want_cols) {
-          st[2 * (c * G + lane)] = pdg * rs;
-          st[2 * (c * G + lane) + 1] = pdb;
-        }
-      } else {
-#pragma unroll
-        for (int i = 0; i < E; ++i) {
-          const float ga = gn_weight(gamma, gn_channel(s, g, e0 + i), 1.0f);
-          const float gv = dp[c].get(i) * ga;
-          acc[0] += gv;
-          acc[1] = fmaf(gv, (xp[c].get(i) - mu) * rs, acc[1]);
-        }
       }
-    }
+    };
+    if (gamma != nullptr)
+      row_sums(std::true_type{});
+    else
+      row_sums(std::false_type{});
     group_allreduce<G, BLOCK, 2, SumOp>(acc, red, phase);
     if (dx != nullptr) {
       T* dr = dx + row * (int64_t)s.L;

@@ -1008,8 +1008,9 @@ inline int make_strided_plan(bool backward, int64_t outer, int64_t D, int64_t in
     return -5;
   }
   if (stream) {
-    // one group per workgroup, rows of up to 8 lanes (128 bytes)
-    TX = px < 8 ? px : 8;
+    // one group per workgroup, rows of up to 16 lanes (256 bytes; [8192, 8192] over dim 0,
+    // forward / backward: 8 lanes 81.6 / 120.9 us, 16 lanes 80.1 / 113.9, 32 lanes 84.2 / 115.2)
+    TX = px < 16 ? px : 16;
     TY = kStridedBlock / TX;
     V = 0;
     // Too few tiles to fill the machine (softmax over dim 0 of [8192, 8192] is 128
