@@ -305,7 +305,10 @@ int mi355x_group_norm_bwd(const void* dy, const void* x, const void* mean, const
  * backward), 2 when only the rows are (a pack may straddle two channels: two
  * lookups per pack, sums still fused; needs HxW >= one pack and at most 512
  * channels a group), 0 for the general kernels; partial_rows is N for the
- * backward. */
+ * backward.  resident == 0: slabs beyond one workgroup's registers; the forward
+ * of such slabs whose channels are whole packs is held by teams of workgroups
+ * (one pass; the rules of mi355x_rownorm_set_team_wait_us apply), and
+ * grid_blocks is then that launch's grid. */
 int mi355x_group_norm_plan(int backward, int64_t N, int64_t C, int64_t HxW, int64_t groups,
                            rownorm_dtype x_dtype, rownorm_plan* out);
 

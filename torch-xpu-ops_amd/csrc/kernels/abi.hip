@@ -675,6 +675,14 @@ int mi355x_group_norm_fwd(const void* x, const void* gamma, const void* beta, vo
   GroupNormFwdArgs a{x,      gamma,      beta,     y,          mean,        rstd,
                      d.rows, (int)d.L, (int)HxW, (int)d.D, (int)groups, eps};
   hipStream_t s = (hipStream_t)stream;
+  // slabs beyond the registers: the team forward, under the rules of the norm forward
+  // (not on top of X, not on a stream under capture)
+  const uintptr_t xb = (uintptr_t)x, yb = (uintptr_t)y;
+  const uintptr_t nbytes = (uintptr_t)d.rows * (uintptr_t)d.L * (uintptr_t)esize_of(xd);
+  if (plan.team > 0 && !(xb < yb + nbytes && yb < xb + nbytes)) {
+    a.team_slot = team_slot_for_call(s, &a.team_id);
+    a.team_wait_ticks = g_team_wait_ticks.load(std::memory_order_relaxed);
+  }
   if (xd == ROWNORM_F32) return launch_group_norm_fwd<float, float>(plan, a, s);
   if (xd == ROWNORM_F16)
     return wd == ROWNORM_F32 ? launch_group_norm_fwd<f16, float>(plan, a, s)
@@ -753,6 +761,9 @@ int mi355x_group_norm_plan(int backward, int64_t N, int64_t C, int64_t HxW, int6
   out->rows_per_block = plan.rpb;
   out->reserved = plan.fast ? gn_mode(d.L, HxW, d.D, 16 / esize_of((int)x_dtype)) : kGnGeneral;
   out->grid_blocks = plan.grid;
+  // (forward slabs beyond the registers whose channels are whole packs: the team launch)
+  if (!backward && plan.team > 0 && HxW % (16 / esize_of((int)x_dtype)) == 0)
+    out->grid_blocks = plan.team_grid;
   out->partial_rows = backward ? N : 0;
   return 0;
 }

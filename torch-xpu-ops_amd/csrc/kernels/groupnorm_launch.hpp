@@ -84,6 +84,33 @@ int launch_group_norm_fwd(const Plan& plan, const GroupNormFwdArgs& a, hipStream
         : mode == kGnStraddle ? launch_variant<GroupNormFwdLauncher<T, WT, kGnStraddle>::template At>(ctx)
                               : launch_variant<GroupNormFwdLauncher<T, WT, kGnGeneral>::template At>(ctx);
     if (!launched) return (int)hipErrorInvalidConfiguration;
+  } else if (plan.team > 0 && a.team_slot != nullptr &&
+             a.HxW % elems_per_pack<T>::value == 0) {
+    // slabs beyond one workgroup's registers whose channels are whole packs: one pass,
+    // a slab in the registers of a team of workgroups (norm_fwd_team_kernel, GROUP)
+    TeamGroupShape gs;
+    gs.groups = a.groups;
+    gs.channels = a.D;
+    gs.packs_per_channel = a.HxW / elems_per_pack<T>::value;
+    auto go = [&](auto v) {
+      constexpr int V = decltype(v)::value;
+      hipLaunchKernelGGL((norm_fwd_team_kernel<T, WT, V, false, true, WT>),
+                         dim3((unsigned)plan.team_grid), dim3(kTeamBlock), 0, stream,
+                         (const T*)a.x, (const WT*)a.gamma, (const WT*)a.beta, (T*)a.y,
+                         (WT*)a.mean, (WT*)a.rstd, a.rows, a.L, a.eps, plan.team,
+                         plan.team_chunk_packs, (TeamSlot*)a.team_slot, a.team_id,
+                         a.team_wait_ticks, gs);
+    };
+    static_assert(kTeamMaxV == 16, "one case per pack count below");
+    switch (plan.team_v) {
+#define ROWNORM_TEAM_CASE(v) case v: go(std::integral_constant<int, v>{}); break;
+      ROWNORM_TEAM_CASE(1) ROWNORM_TEAM_CASE(2) ROWNORM_TEAM_CASE(3) ROWNORM_TEAM_CASE(4)
+      ROWNORM_TEAM_CASE(5) ROWNORM_TEAM_CASE(6) ROWNORM_TEAM_CASE(7) ROWNORM_TEAM_CASE(8)
+      ROWNORM_TEAM_CASE(9) ROWNORM_TEAM_CASE(10) ROWNORM_TEAM_CASE(11) ROWNORM_TEAM_CASE(12)
+      ROWNORM_TEAM_CASE(13) ROWNORM_TEAM_CASE(14) ROWNORM_TEAM_CASE(15) ROWNORM_TEAM_CASE(16)
+#undef ROWNORM_TEAM_CASE
+      default: return (int)hipErrorInvalidConfiguration;
+    }
   } else {
     hipLaunchKernelGGL((gn_fwd_stream_kernel<T, WT, kStreamBlock>), dim3((unsigned)plan.grid),
                        dim3(kStreamBlock), 0, stream, (const T*)a.x, (const WT*)a.gamma,

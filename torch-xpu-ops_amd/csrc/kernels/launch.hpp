@@ -102,6 +102,10 @@ struct GroupNormFwdArgs {
   int64_t rows;
   int L, HxW, D, groups;
   float eps;
+  // bookkeeping memory, call id and wait bound of the team forward (see NormFwdArgs)
+  void* team_slot = nullptr;
+  unsigned int team_id = 0;
+  unsigned long long team_wait_ticks = 0;
 };
 
 struct GroupNormBwdArgs {

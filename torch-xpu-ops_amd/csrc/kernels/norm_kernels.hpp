@@ -753,13 +753,25 @@ norm_fwd_stream_kernel(const T* __restrict__ x, const T* res, const WT* __restri
 // team's to rounding -- loads its chunk again and goes on; it keeps publishing its
 // partial sums for the workgroups that do wait.  Every wave reaches the end of the
 // kernel whatever the other workgroups do, and every row is written.
-template <class T, class WT, int V, bool RMS>
+//
+// GROUP: the rows are the (sample, group) slabs of a GroupNorm whose channels are whole
+// packs (`group.packs_per_channel` packs each): gamma and beta hold one value a channel,
+// looked up by the pack's position in the row, and mean / rstd leave in the weight
+// dtype ST, as native_group_norm returns them.  Everything else is the LayerNorm's.
+struct TeamGroupShape {
+  int groups = 1;             // groups a sample: row r belongs to group r % groups
+  int channels = 1;           // channels a group
+  int packs_per_channel = 1;  // HxW / E
+};
+
+template <class T, class WT, int V, bool RMS, bool GROUP = false, class ST = float>
 __global__ void __launch_bounds__(kTeamBlock, kTeamPerCu * kTeamBlock / 256)
 norm_fwd_team_kernel(const T* __restrict__ x, const WT* __restrict__ gamma,
-                     const WT* __restrict__ beta, T* __restrict__ y, float* __restrict__ mean,
-                     float* __restrict__ rstd, int64_t M, int N, float eps, int team,
+                     const WT* __restrict__ beta, T* __restrict__ y, ST* __restrict__ mean,
+                     ST* __restrict__ rstd, int64_t M, int N, float eps, int team,
                      int64_t chunk_packs, TeamSlot* slot, unsigned int call_id,
-                     unsigned long long wait_ticks) {
+                     unsigned long long wait_ticks, TeamGroupShape group = TeamGroupShape{}) {
+  static_assert(!(GROUP && RMS), "GroupNorm is a LayerNorm over a slab");
   constexpr int E = elems_per_pack<T>::value;
   constexpr int BLOCK = kTeamBlock;
   __shared__ double red[2 * (BLOCK / 64)];
@@ -912,6 +924,71 @@ norm_fwd_team_kernel(const T* __restrict__ x, const WT* __restrict__ gamma,
     // (opaque: the 2 * V weight addresses, the same for every row, would otherwise be
     // formed once ahead of the row loop and kept -- spilled -- across it)
     const uint32_t woff = (uint32_t)(lane_again((int)threadIdx.x) * E * (int)sizeof(WT));
+    if constexpr (GROUP) {
+      // one gamma and one beta a pack: those of the channel the pack lies in
+      const int ch0 = (int)(row % group.groups) * group.channels;
+      const uint32_t pk0 = (uint32_t)pbase + (uint32_t)lane_again((int)threadIdx.x);
+      auto channel = [&](int k) {
+        return ch0 + (int)((pk0 + (uint32_t)(k * BLOCK)) / (uint32_t)group.packs_per_channel);
+      };
+      auto normalized1 = [&](const Pack<T, E>& xk, float ga, float be) {
+        Pack<T, E> o;
+        const float gr = ga * rs;
+#pragma unroll
+        for (int i = 0; i < E; ++i) o.set(i, ((xk.get(i) - hi) - lo) * gr + be);
+        return o;
+      };
+      if (full && hg && hb) {
+        // (as below: the weights of the next packs are requested before these are stored)
+        constexpr int GS = kTeamGroup, NG = (V + GS - 1) / GS;
+        // (kept as loaded: widening a value waits for it, and that belongs to the turn
+        // that uses it)
+        WT wg[2][GS], wb[2][GS];
+        auto request = [&](int g, int buf) {
+#pragma unroll
+          for (int u = 0; u < GS; ++u) {
+            const int k = g * GS + u;
+            if (k < V) {
+              const int ch = channel(k);
+              wg[buf][u] = gamma[ch];
+              wb[buf][u] = beta[ch];
+            }
+          }
+        };
+        request(0, 0);
+#pragma unroll
+        for (int g = 0; g < NG; ++g) {
+          if (g + 1 < NG) request(g + 1, (g + 1) & 1);
+          __builtin_amdgcn_sched_barrier(0);
+#pragma unroll
+          for (int u = 0; u < GS; ++u) {
+            const int k = g * GS + u;
+            if (k < V) {
+              keep_packed(xp[k]);
+              normalized1(xp[k], (float)wg[g & 1][u], (float)wb[g & 1][u])
+                  .store_stream(at(yb + k * BLOCK * E, loff));
+            }
+          }
+          __builtin_amdgcn_sched_barrier(0);
+        }
+      } else {
+#pragma unroll
+        for (int k = 0; k < V; ++k) {
+          if (k * BLOCK + (int)threadIdx.x < nloc) {
+            keep_packed(xp[k]);
+            const int ch = channel(k);
+            const float ga = hg ? (float)gamma[ch] : 1.0f;
+            const float be = hb ? (float)beta[ch] : 0.0f;
+            normalized1(xp[k], ga, be).store_stream(at(yb + k * BLOCK * E, loff));
+          }
+        }
+      }
+      if (c == 0 && threadIdx.x == 0) {
+        if (mean) mean[row] = (ST)hi;
+        if (rstd) rstd[row] = (ST)rs;
+      }
+      continue;
+    }
     auto normalized = [&](const Pack<T, E>& xk, const Pack<WT, E>& g, const Pack<WT, E>& b) {
       Pack<T, E> o;
 #pragma unroll
@@ -985,8 +1062,8 @@ norm_fwd_team_kernel(const T* __restrict__ x, const WT* __restrict__ gamma,
     }
     if (c == 0 && threadIdx.x == 0) {
       if constexpr (!RMS)
-        if (mean) mean[row] = hi;
-      if (rstd) rstd[row] = rs;
+        if (mean) mean[row] = (ST)hi;
+      if (rstd) rstd[row] = (ST)rs;
     }
     // (stat[], tpart[] and red[] are rewritten for the next row only behind the barrier
     // inside the next block sum, which every thread reaches after it has read them)

@@ -892,8 +892,10 @@ inline int make_plan(OpClass oc, int64_t M, int64_t N, int esize, int num_cus, c
   // row (one pass over X).  As few workgroups a row as hold it with 16 packs a lane,
   // then as many teams as there are rows and compute units, and a row spread over
   // all the workgroups its team can have (down to one stride of 1024 packs each).
-  if (oc == OC_NORM_FWD && !p.resident && p.fast && !fused_add && ov.G == 0 && ov.V == 0 &&
-      ov.bpc == 0) {
+  // (GroupNorm forward slabs likewise; the caller takes the team only where the channels
+  // are whole packs)
+  if ((oc == OC_NORM_FWD || oc == OC_GROUP_FWD) && !p.resident && p.fast && !fused_add &&
+      ov.G == 0 && ov.V == 0 && ov.bpc == 0) {
     const int64_t cus = num_cus * kTeamPerCu < kTeamMaxWorkgroups ? num_cus * kTeamPerCu : kTeamMaxWorkgroups;
     const int64_t per_wg = (int64_t)kTeamBlock * kTeamMaxV;
     const int64_t team_min = (packs + per_wg - 1) / per_wg;
