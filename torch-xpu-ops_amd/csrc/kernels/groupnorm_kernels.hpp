@@ -802,6 +802,39 @@ gn_bwd_dx_from_sums_kernel(const T* __restrict__ dy, const T* __restrict__ x,
     const T* xr = x + row * (int64_t)s.L;
     const T* gr = dy + row * (int64_t)s.L;
     T* dr = dx + row * (int64_t)s.L;
+    // A chunk that lies wholly inside a row whose channels are whole packs: straight-line
+    // code, all 2 * kGnChunkPacks loads of a lane requested before the first is used and
+    // one weight a pack (the general loop below tests every pack against the row end and
+    // the weight pointer, and each such branch waits for what is outstanding).
+    const int64_t pk_first = (int64_t)chunk * kGnChunkPacks * BLOCK;
+    if (uniform && gamma != nullptr && (pk_first + (int64_t)kGnChunkPacks * BLOCK) * E <= s.L) {
+      const uint32_t pk0 = (uint32_t)pk_first + threadIdx.x;
+      const uint32_t S = (uint32_t)(s.HxW / E);  // packs a channel
+      Pack<T, E> px[kGnChunkPacks], pd[kGnChunkPacks];
+      WT gw[kGnChunkPacks];
+#pragma unroll
+      for (int k = 0; k < kGnChunkPacks; ++k) {
+        const uint32_t pk = pk0 + (uint32_t)(k * BLOCK);
+        px[k] = Pack<T, E>::load_stream(xr + (int64_t)pk * E);
+        pd[k] = Pack<T, E>::load_stream(gr + (int64_t)pk * E);
+        gw[k] = gamma[g * s.D + (int)(pk / S)];
+      }
+#pragma unroll
+      for (int k = 0; k < kGnChunkPacks; ++k) {
+        const uint32_t pk = pk0 + (uint32_t)(k * BLOCK);
+        const float ga = (float)gw[k];
+        Pack<T, E> o;
+#pragma unroll
+        for (int i = 0; i < E; ++i) {
+          float f = fL * (pd[k].get(i) * ga);
+          f -= ((px[k].get(i) - mu) * rs) * s2;
+          f -= s1;
+          o.set(i, f * term1);
+        }
+        o.store_stream(dr + (int64_t)pk * E);
+      }
+      continue;
+    }
 #pragma unroll
     for (int k = 0; k < kGnChunkPacks; ++k) {
       const int64_t pk = ((int64_t)chunk * kGnChunkPacks + k) * BLOCK + threadIdx.x;
@@ -855,7 +888,29 @@ gn_channel_sums_kernel(const T* __restrict__ dy, const T* __restrict__ x,
     const T* xr = x + rc * (int64_t)s.HxW;
     const T* gr = dy + rc * (int64_t)s.HxW;
     float acc[2] = {0.0f, 0.0f};
-    for (int pk = sub; pk < npacks; pk += LANES) {
+    int pk = sub;
+    if ((s.HxW % E) == 0) {
+      // channels of whole packs: four pack pairs a lane in flight, nothing conditional
+      // (a row slot past the last row reads row 0 and stores nothing)
+      constexpr int U = 4;
+      for (; pk + (U - 1) * LANES < npacks; pk += U * LANES) {
+        Pack<T, E> px[U], pd[U];
+#pragma unroll
+        for (int u = 0; u < U; ++u) {
+          px[u] = Pack<T, E>::load_stream(xr + (int64_t)(pk + u * LANES) * E);
+          pd[u] = Pack<T, E>::load_stream(gr + (int64_t)(pk + u * LANES) * E);
+        }
+#pragma unroll
+        for (int u = 0; u < U; ++u)
+#pragma unroll
+          for (int i = 0; i < E; ++i) {
+            const float gy = pd[u].get(i);
+            acc[1] += gy;
+            acc[0] = fmaf(gy, px[u].get(i) - mu, acc[0]);
+          }
+      }
+    }
+    for (; pk < npacks; pk += LANES) {
       const Pack<T, E> px = load_row_pack<T, E, true>(xr, pk * E, s.HxW, ok, 0.0f);
       const Pack<T, E> pd = load_row_pack<T, E, true>(gr, pk * E, s.HxW, ok, 0.0f);
       const int nvalid = s.HxW - pk * E;

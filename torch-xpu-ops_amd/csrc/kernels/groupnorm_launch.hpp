@@ -201,18 +201,26 @@ int launch_group_norm_bwd(const Plan& plan, const GroupNormBwdArgs& a, hipStream
   const int C = a.groups * a.D;
   int err = 0;
   if (need_sums && !fused_cols) {
-    constexpr int CB = 256;
     const int packs = (a.HxW + E - 1) / E;
-    // long channel rows take a whole workgroup each
-    const int lanes = packs >= 8 * CB ? CB : (packs >= 64 ? 64 : pow2_ceil(packs));
     const int64_t nc_rows = N * C;
-    const int rpb = CB / lanes;
-    int64_t grid = (nc_rows + rpb - 1) / rpb;
-    if (grid > (1 << 22)) grid = 1 << 22;
-    hipLaunchKernelGGL((gn_channel_sums_kernel<T, WT, CB>), dim3((unsigned)grid), dim3(CB), 0,
-                       stream, (const T*)a.dy, (const T*)a.x, (const WT*)a.mean,
-                       (const WT*)a.rstd, a.part_dg, a.part_db, nc_rows, shape,
-                       log2_of_pow2(lanes));
+    auto sums = [&](auto cb) {
+      constexpr int CB = decltype(cb)::value;
+      // long channel rows take a whole workgroup each
+      const int lanes = packs >= 8 * CB ? CB : (packs >= 64 ? 64 : pow2_ceil(packs));
+      const int rpb = CB / lanes;
+      int64_t grid = (nc_rows + rpb - 1) / rpb;
+      if (grid > (1 << 22)) grid = 1 << 22;
+      hipLaunchKernelGGL((gn_channel_sums_kernel<T, WT, CB>), dim3((unsigned)grid), dim3(CB), 0,
+                         stream, (const T*)a.dy, (const T*)a.x, (const WT*)a.mean,
+                         (const WT*)a.rstd, a.part_dg, a.part_db, nc_rows, shape,
+                         log2_of_pow2(lanes));
+    };
+    // (channel rows of 8192 packs and more -- 256 x 256 maps in 16 bits -- on 1024 threads:
+    // there are few of them, and each lane keeps four pack pairs in flight)
+    if (packs >= 8 * 1024)
+      sums(std::integral_constant<int, 1024>{});
+    else
+      sums(std::integral_constant<int, 256>{});
     err = (int)hipGetLastError();
     if (err != 0) return err;
   }
