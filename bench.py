@@ -698,7 +698,8 @@ def model_shapes_table(torch, cabi, L, dev, stream, P, only=None):
     """Shapes of this op family in common models that are neither whole packs nor in the other
     tables, bf16, forward and backward: attention scores of ViT-B/16 (rows of 197), ViT-L/14 at
     336 px (577) and CLIP's text tower (77), which are ragged short rows; GroupNorm over 14 x 14
-    and 7 x 7 feature maps, whose channels are not whole packs; log_softmax over a 151936-entry
+    and 7 x 7 feature maps, whose channels are not whole packs, and over the 256 x 256 and 512 x 512
+    maps of a VAE decoder, whose slabs are beyond one workgroup's registers; log_softmax over a 151936-entry
     vocabulary (19 packs a lane); LayerNorm over a hidden size of 18432 (backward with the dgamma
     sums in LDS).  Algorithmic GB/s as everywhere;
     `stock_us` = the kernels PyTorch-ROCm ships."""
@@ -749,7 +750,11 @@ def model_shapes_table(torch, cabi, L, dev, stream, P, only=None):
         torch.cuda.empty_cache()
 
     for name, Nb, C, HW, G in (("native_group_norm bf16 [256,1024,14,14] g32", 256, 1024, 196, 32),
-                               ("native_group_norm bf16 [256,2048,7,7] g32", 256, 2048, 49, 32)):
+                               ("native_group_norm bf16 [256,2048,7,7] g32", 256, 2048, 49, 32),
+                               ("native_group_norm bf16 [2,256,256,256] g32 (VAE decoder map)",
+                                2, 256, 65536, 32),
+                               ("native_group_norm bf16 [1,128,512,512] g32 (VAE decoder map)",
+                                1, 128, 262144, 32)):
         if only is not None and not any(t in name + " fwd" or t in name + " bwd" for t in only.split("|")):
             continue
         w = (1 + 0.1 * torch.randn(C, device=dev)).to(bf16)

@@ -393,7 +393,42 @@ gn_fwd_stream_kernel(const T* __restrict__ x, const WT* __restrict__ gamma,
     T* yr = y + row * (int64_t)s.L;
     const double k = (double)(float)xr[0];
     double s1 = 0.0, s2 = 0.0;
-    for (int pk = threadIdx.x; pk < npacks; pk += BLOCK) {
+    // rows of whole packs: four packs a lane in flight, nothing conditional; the pack
+    // sums in float32 about k, their totals in float64 (as add_centred_sums)
+    constexpr int U = 4;
+    const bool whole = (s.L % E) == 0;  // uniform
+    const bool one_weight = (s.HxW % E) == 0 && gamma != nullptr && beta != nullptr;  // uniform
+    int pk = threadIdx.x;
+    if (whole) {
+      const float kf = (float)k;
+      for (; pk + (U - 1) * BLOCK < npacks; pk += U * BLOCK) {
+        Pack<T, E> p[U];
+#pragma unroll
+        for (int u = 0; u < U; ++u) p[u] = Pack<T, E>::load(xr + (int64_t)(pk + u * BLOCK) * E);
+#pragma unroll
+        for (int u = 0; u < U; ++u) {
+          if constexpr (sizeof(T) == 2) {
+            float t1 = 0.0f, t2 = 0.0f;
+#pragma unroll
+            for (int i = 0; i < E; ++i) {
+              const float d = p[u].get(i) - kf;
+              t1 += d;
+              t2 = fmaf(d, d, t2);
+            }
+            s1 += (double)t1;
+            s2 += (double)t2;
+          } else {
+#pragma unroll
+            for (int i = 0; i < E; ++i) {
+              const double d = (double)p[u].get(i) - k;
+              s1 += d;
+              s2 = fma(d, d, s2);
+            }
+          }
+        }
+      }
+    }
+    for (; pk < npacks; pk += BLOCK) {
       const Pack<T, E> p = load_row_pack<T, E, false>(xr, pk * E, s.L, true, 0.0f);
       const int nvalid = s.L - pk * E;
 #pragma unroll
@@ -416,7 +451,32 @@ gn_fwd_stream_kernel(const T* __restrict__ x, const WT* __restrict__ gamma,
     }
     __syncthreads();
     const float hi = stat[0], lo = stat[1], rs = stat[2];
-    for (int pk = threadIdx.x; pk < npacks; pk += BLOCK) {
+    pk = threadIdx.x;
+    if (whole && one_weight) {
+      // channels of whole packs as well: one gamma and one beta a pack
+      const uint32_t S = (uint32_t)(s.HxW / E);
+      for (; pk + (U - 1) * BLOCK < npacks; pk += U * BLOCK) {
+        Pack<T, E> p[U];
+        WT gw[U], bw[U];
+#pragma unroll
+        for (int u = 0; u < U; ++u) {
+          const uint32_t q = (uint32_t)(pk + u * BLOCK);
+          p[u] = Pack<T, E>::load_stream(xr + (int64_t)q * E);
+          const int ch = g * s.D + (int)(q / S);
+          gw[u] = gamma[ch];
+          bw[u] = beta[ch];
+        }
+#pragma unroll
+        for (int u = 0; u < U; ++u) {
+          const float ga = (float)gw[u] * rs, be = (float)bw[u];
+          Pack<T, E> o;
+#pragma unroll
+          for (int i = 0; i < E; ++i) o.set(i, ((p[u].get(i) - hi) - lo) * ga + be);
+          o.store_stream(yr + (int64_t)(pk + u * BLOCK) * E);
+        }
+      }
+    }
+    for (; pk < npacks; pk += BLOCK) {
       const int e0 = pk * E;
       const Pack<T, E> p = load_row_pack<T, E, true>(xr, e0, s.L, true, 0.0f);
       Pack<T, E> o;
