@@ -72,10 +72,48 @@ inline bool launch_norm_fwd_exact_at(const Plan& plan, const NormFwdArgs& a, hip
   return false;
 }
 
+// Short ragged rows through LDS (norm_fwd_flat_kernel): 16 KB a workgroup, 32 KB for rows
+// beyond 1024 16-bit elements.
+template <class T, class WT, bool RMS, int LDSB>
+bool launch_norm_fwd_flat_l(FlatLayout f, int cr, const NormFwdArgs& a, hipStream_t stream) {
+  const int64_t grid = (a.M + cr - 1) / cr;
+  if (grid > 0x7fffffff) return false;
+#define ROWNORM_FLAT_NORM_FWD(GL, VP)                                                           \
+  case GL * 8 + VP:                                                                             \
+    if constexpr (LDSB <= kFlatLdsBytes || (GL == 64 && VP >= 3)) {                             \
+      hipLaunchKernelGGL((norm_fwd_flat_kernel<T, WT, GL, VP, kFlatBlock, LDSB, RMS>),           \
+                         dim3((unsigned)grid), dim3(kFlatBlock), 0, stream, (const T*)a.x,       \
+                         (const WT*)a.gamma, (const WT*)a.beta, (T*)a.y, a.mean, a.rstd, a.M,    \
+                         a.N, cr, a.eps);                                                       \
+      return true;                                                                              \
+    }                                                                                           \
+    return false;
+  switch (f.g * 8 + f.vp) { ROWNORM_FLAT_ALL(ROWNORM_FLAT_NORM_FWD) }
+#undef ROWNORM_FLAT_NORM_FWD
+  return false;
+}
+
+template <class T, class WT, bool RMS>
+bool launch_norm_fwd_flat(FlatLayout f, const NormFwdArgs& a, hipStream_t stream) {
+  int cr = flat_chunk_rows<T>(a.N, f.g, kFlatLdsBytes);
+  if (cr >= 8) return launch_norm_fwd_flat_l<T, WT, RMS, kFlatLdsBytes>(f, cr, a, stream);
+  cr = flat_chunk_rows<T>(a.N, f.g, 2 * kFlatLdsBytes);
+  if (cr >= 8) return launch_norm_fwd_flat_l<T, WT, RMS, 2 * kFlatLdsBytes>(f, cr, a, stream);
+  return false;
+}
+
 template <class T, class WT, bool RMS, class TY, bool ADD>
 int launch_norm_fwd(const Plan& plan, const NormFwdArgs& a, hipStream_t stream) {
   const T* res = ADD ? (const T*)a.res : nullptr;
   T* h = ADD ? (T*)a.h : nullptr;
+  // short ragged rows (no residual add, no cast, 16-byte aligned X and Y): staged through LDS
+  if constexpr (!ADD && std::is_same<T, TY>::value) {
+    if (plan.resident && !plan.fast && plan.exact_depth == 0 && !plan.window) {
+      const FlatLayout f = flat_layout<T>(plan, a.M, a.N, a.x, a.y, nullptr);
+      if (f.g != 0 && launch_norm_fwd_flat<T, WT, RMS>(f, a, stream))
+        return (int)hipGetLastError();
+    }
+  }
   if (plan.resident && plan.exact_depth > 0) {
     static_assert(kNormFwdExactCount == 2, "one call per table entry below");
     bool launched = false;

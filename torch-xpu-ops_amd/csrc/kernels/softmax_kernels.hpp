@@ -27,6 +27,7 @@
 // zeros instead of NaN.
 #pragma once
 #include "device/pack.hpp"
+#include "device/flat_rows.hpp"
 #include "device/reduce.hpp"
 #include "launch.hpp"
 #include <type_traits>
@@ -599,141 +600,7 @@ softmax_bwd_resident_kernel(const TG* __restrict__ grad, const TG* __restrict__ 
 }
 
 // ---------------------------------------------------------------------------
-// Short ragged rows (N % E != 0, N <= 64 lanes * kFlatMaxPacks packs: ViT / CLIP /
-// Whisper attention scores are rows of 197, 577, 77, 1500 elements) through LDS.  Such
-// rows start at every 2-byte (fp32: 4-byte) alignment, and the general kernels
-// pay for it per row: edge packs moved element by element, windows, masks.  But
-// a run of `chunk_rows` consecutive rows, chunk_rows a multiple of 8, is one
-// contiguous piece of the tensor that starts and ends on a 16-byte boundary, so
-// the workgroup copies the piece to LDS with whole aligned 128-bit accesses, each
-// group of G lanes then reads a row from LDS in packs at the row's own alignment
-// (LDS takes unaligned 128-bit accesses; VP packs a lane, laid out like the
-// register-resident kernels'), writes the results back in place, and the piece
-// leaves with whole 128-bit stores: HBM sees the access pattern of a copy
-// whatever N is.  The reductions stay inside a wavefront (G <= 64), so the only
-// barriers are the two around the LDS phase; a lane group walks the rows r,
-// r + BLOCK / G, ... of the piece.  Needs 16-byte aligned tensor bases and the
-// same dtype in and out; anything else keeps the general kernels.  Very short
-// rows of whole packs whose pack count fits the resident layouts badly take the
-// same path (flat_layout, softmax_launch.hpp).
-constexpr int kFlatBlock = 256;
-// LDS per tensor a workgroup holds (LDSB; the backward holds two tensors): 16 KB
-// at 256 threads, so that 8 workgroups share a compute unit; the backward takes
-// 8 KB per tensor where that still holds a full pass of rows, for the same
-// reason; rows beyond 1024 16-bit elements need 32 KB to hold 8 of them.
-// Measured against 512 threads / 32 KB: bf16 [151296, 197] forward 27.0 -> 25.6 us,
-// backward 36.2 -> 32.9 us ([147712, 577] backward, which needs the 16 KB:
-// 101 -> 94 us); 1024 threads were 50 % slower.
-constexpr int kFlatLdsBytes = 64 * kFlatBlock;
-// Lanes per row G (4..64) and packs per lane VP (1..kFlatMaxPacks) are chosen so
-// that G * VP leaves as few pack slots idle as possible (flat_layout,
-// softmax_launch.hpp).
-constexpr int kFlatMaxPacks = 4;
-// Rows a workgroup takes at a time: as many as its LDS holds, a multiple of 8
-// so that the piece starts and ends on a 16-byte boundary (and of the rows its
-// lane groups work on at a time, where that many fit).  A
-// workgroup must have tens of KB on their way to keep HBM busy: with one row per
-// lane group (BLOCK / G rows, 9 KB at N = 577) the kernel ran slower than the
-// general one.
-template <class T>
-constexpr int flat_chunk_rows(int N, int lanes, int ldsb) {
-  const int rpb = kFlatBlock / lanes < 8 ? 8 : kFlatBlock / lanes;  // rows per pass, and 8 | rows
-  const int cap = ldsb / (int)sizeof(T) / N;
-  return cap >= rpb ? cap / rpb * rpb : cap / 8 * 8;
-}
-
-// Copies the `nelem` elements at `src` (16-byte aligned) into LDS and back out:
-// whole packs, all of a thread's loads requested before the first is written
-// to LDS (a loop of load-then-write would wait for memory once per round), and
-// the tail of the tensor's last piece element by element.
-template <class T, int BLOCK, int U>  // U packs a thread: BLOCK * U packs = the LDS of one tensor
-__device__ __forceinline__ void flat_stage_in(const T* __restrict__ src, T* buf, int nelem) {
-  constexpr int E = elems_per_pack<T>::value;
-  typedef typename Pack<T, E>::vec_t vec_t;
-  const int nfull = nelem / E;
-  Pack<T, E> p[U];
-#pragma unroll
-  for (int u = 0; u < U; ++u) {
-    const int pk = (int)threadIdx.x + u * BLOCK;
-    if (u * BLOCK < nfull)  // uniform
-      p[u] = Pack<T, E>::load_stream(src + (pk < nfull ? pk : 0) * E);
-  }
-#pragma unroll
-  for (int u = 0; u < U; ++u) {
-    const int pk = (int)threadIdx.x + u * BLOCK;
-    if (u * BLOCK < nfull && pk < nfull) *reinterpret_cast<vec_t*>(buf + pk * E) = p[u].v;
-  }
-  const int t = nfull * E + (int)threadIdx.x;
-  if (t < nelem) buf[t] = src[t];
-}
-// The same for two tensors (the backward's grad and y): all loads of both before
-// the first LDS write.
-template <class T, int BLOCK, int U>
-__device__ __forceinline__ void flat_stage_in2(const T* __restrict__ src0, T* buf0,
-                                               const T* __restrict__ src1, T* buf1, int nelem) {
-  constexpr int E = elems_per_pack<T>::value;
-  typedef typename Pack<T, E>::vec_t vec_t;
-  const int nfull = nelem / E;
-  Pack<T, E> p[U], q[U];
-#pragma unroll
-  for (int u = 0; u < U; ++u) {
-    const int pk = (int)threadIdx.x + u * BLOCK;
-    if (u * BLOCK < nfull) {  // uniform
-      p[u] = Pack<T, E>::load_stream(src0 + (pk < nfull ? pk : 0) * E);
-      q[u] = Pack<T, E>::load_stream(src1 + (pk < nfull ? pk : 0) * E);
-    }
-  }
-#pragma unroll
-  for (int u = 0; u < U; ++u) {
-    const int pk = (int)threadIdx.x + u * BLOCK;
-    if (u * BLOCK < nfull && pk < nfull) {
-      *reinterpret_cast<vec_t*>(buf0 + pk * E) = p[u].v;
-      *reinterpret_cast<vec_t*>(buf1 + pk * E) = q[u].v;
-    }
-  }
-  const int t = nfull * E + (int)threadIdx.x;
-  if (t < nelem) {
-    buf0[t] = src0[t];
-    buf1[t] = src1[t];
-  }
-}
-template <class T, int BLOCK, int U>
-__device__ __forceinline__ void flat_stage_out(T* __restrict__ dst, const T* buf, int nelem) {
-  constexpr int E = elems_per_pack<T>::value;
-  typedef typename Pack<T, E>::vec_t vec_t;
-  const int nfull = nelem / E;
-#pragma unroll
-  for (int u = 0; u < U; ++u) {
-    const int pk = (int)threadIdx.x + u * BLOCK;
-    if (u * BLOCK < nfull && pk < nfull) {
-      Pack<T, E> p;
-      p.v = *reinterpret_cast<const vec_t*>(buf + pk * E);
-      p.store_stream(dst + pk * E);
-    }
-  }
-  const int t = nfull * E + (int)threadIdx.x;
-  if (t < nelem) dst[t] = buf[t];
-}
-
-// A lane's pack c of a row held in LDS: elements (c * G + lane) * E ... + E of the
-// row, read with one LDS access at the row's own (element) alignment.  Reads may
-// run past the row end into the next row or the padding of the buffer; `nv` is
-// the number of elements that belong to the row.
-template <class T, int E>
-__device__ __forceinline__ Pack<T, E> flat_row_pack(const T* rowb, int j) {
-  return Pack<T, E>::load(rowb + j);
-}
-template <class T, int E>
-__device__ __forceinline__ void flat_row_store(T* rowb, int j, int nv, const Pack<T, E>& p) {
-  if (nv >= E) {
-    p.store(rowb + j);
-  } else {
-#pragma unroll
-    for (int i = 0; i < E; ++i)
-      if (i < nv) rowb[j + i] = p.v[i];
-  }
-}
-
+// Short ragged rows through LDS: see device/flat_rows.hpp.
 template <class T, int G, int VP, int BLOCK, int LDSB>
 __global__ void __launch_bounds__(BLOCK)
 softmax_fwd_flat_kernel(const T* __restrict__ x, T* __restrict__ y, int64_t M, int N,

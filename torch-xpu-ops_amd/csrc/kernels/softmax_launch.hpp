@@ -34,58 +34,6 @@ struct SoftmaxFwdLauncher {
   };
 };
 
-// Short ragged rows through LDS (softmax_fwd_flat_kernel / softmax_bwd_flat_kernel).
-constexpr int kFlatWholePackRowsMaxPacks = 12;
-struct FlatLayout {
-  int g = 0;   // lanes per row (0: the call does not qualify)
-  int vp = 0;  // packs per lane
-};
-
-// The (lanes 4..64, packs per lane 1..4) with the fewest idle pack slots; among
-// equals the one nearest two packs a lane, the layout the resident kernels prefer.
-// Measured against "two packs a lane on the fewest lanes that hold the row",
-// interleaved, bf16 forward / backward in us: rows of 13: 19.5 / 18.5 -> 10.6 / 8.6,
-// 21: 30.0 / 25.9 -> 14.1 / 16.1, 45: 20.3 / 22.8 -> 16.5 / 20.6, 577 (73 packs: 32 x 3
-// instead of 64 x 2): 72.1 / 96.5 -> 67.8 / 96.3, 750: 54.0 / 76.2 -> 51.2 / 75.1; 93
-// and 129 lose 5-10 % in the backward (13.1 -> 14.6, 33.1 -> 34.8).
-template <class T>
-inline FlatLayout flat_layout(const Plan& plan, int64_t M, int N, const void* p0, const void* p1,
-                              const void* p2) {
-  constexpr int E = elems_per_pack<T>::value;
-  FlatLayout f;
-  if (plan.forced || M < 1 || N > 64 * kFlatMaxPacks * E) return f;
-  if ((((uintptr_t)p0) | ((uintptr_t)p1) | ((uintptr_t)p2)) & 15) return f;
-  const int packs = (N + E - 1) / E;
-  // rows of whole packs qualify only when they are very short (see below)
-  if (plan.fast && (packs > kFlatWholePackRowsMaxPacks || !plan.resident)) return f;
-  int best_slots = 0, best_rank = 0;
-  for (int g = 4; g <= 64; g <<= 1) {
-    const int vp = (packs + g - 1) / g;
-    if (vp > kFlatMaxPacks) continue;
-    const int slots = g * vp;
-    const int rank = vp == 2 ? 0 : (vp == 3 ? 1 : (vp == 1 ? 2 : 3));
-    if (f.g == 0 || slots < best_slots || (slots == best_slots && rank < best_rank)) {
-      f.g = g;
-      f.vp = vp;
-      best_slots = slots;
-      best_rank = rank;
-    }
-  }
-  // Rows of whole packs: only up to 12 packs and where the resident layout leaves a
-  // quarter of its pack slots idle, e.g. 9 or 10 packs on 8 lanes x 2 (bf16 rows of 72:
-  // 36.6 / 52.5 -> 31.2 / 44.3 us, of 80: 40.9 / 57.6 -> 33.2 / 48.2 us, of 24: 32.1 / 29.4
-  // -> 18.1 / 25.1 us); from 17 packs on it measured the same or slower (520: +2 %, 1032:
-  // the backward +30 %).
-  if (plan.fast && best_slots * 4 > plan.G * plan.V * 3) f = FlatLayout{};
-  return f;
-}
-
-// One case per (lanes, packs per lane) of a launch switch keyed by lanes * 8 + packs.
-#define ROWNORM_FLAT_CASES(CASE, GL) CASE(GL, 1) CASE(GL, 2) CASE(GL, 3) CASE(GL, 4)
-#define ROWNORM_FLAT_ALL(CASE)                                                       \
-  ROWNORM_FLAT_CASES(CASE, 4) ROWNORM_FLAT_CASES(CASE, 8) ROWNORM_FLAT_CASES(CASE, 16) \
-  ROWNORM_FLAT_CASES(CASE, 32) ROWNORM_FLAT_CASES(CASE, 64)
-
 template <class T, int LDSB>
 bool launch_softmax_fwd_flat_l(FlatLayout f, int cr, const SoftmaxFwdArgs& a, hipStream_t stream) {
   const int64_t grid = (a.M + cr - 1) / cr;
