@@ -29,6 +29,13 @@ SHAPES = [(7, 64), (5, 127), (33, 1024), (9, 4097), (12, 4096), (4, 5120), (6, 8
           (520, 40000), (2, 300000)]
 
 
+def _staged(dtype, N):
+    """Short ragged rows: the plain kernels (no add, no cast) stage them through LDS and sum a row
+    in another order than the kernels with the add or the cast, which take the general layout."""
+    E = 4 if dtype == torch.float32 else 8
+    return N % E != 0 and N <= 256 * E
+
+
 def _mk(M, N, dtype, seed, wdtype=None):
     g = gen(seed)
     x = torch.randn(M, N, generator=g).to(dtype)
@@ -55,7 +62,7 @@ def test_add_norm_forward_and_backward(cabi, oracle, gpu, dtype, shape, mixed):
     wtol = gamma.dtype
     # 16-bit rows of 4096 / 5120 elements: the plain forward takes an exact two-pack layout
     # (5120: 320 lanes x 2 packs) that the fused add does not have (256 lanes x 3 packs there)
-    same_layout = not (dtype != torch.float32 and N == 5120)
+    same_layout = not (dtype != torch.float32 and N == 5120) and not _staged(dtype, N)
     for rms in (False, True):
         what = "rms_norm" if rms else "layer_norm"
         if rms:
@@ -82,7 +89,9 @@ def test_add_norm_forward_and_backward(cabi, oracle, gpu, dtype, shape, mixed):
             assert torch.equal(rstd, urstd), what
         else:
             assert_close(rstd, urstd, torch.float32, what + " rstd, fused against plain on h")
-        assert_same_arithmetic(y, uy, what + " y, fused against plain on h")
+        if not _staged(dtype, N):
+            assert_same_arithmetic(y, uy, what + " y, fused against plain on h")
+        assert_close(uy, oy, dtype, what + " y, plain on h")
         assert_close(y, oy, dtype, what + " y")
         assert_close(rstd, orr.reshape(-1), dtype, what + " rstd")
         # in place on the residual stream (h written over res) and over x
@@ -100,6 +109,7 @@ def test_add_norm_forward_and_backward(cabi, oracle, gpu, dtype, shape, mixed):
         # order of the column sums -- with the residual gradient than without: there the two
         # are each held to the oracle, below, and not to each other)
         same_bwd_layout = not (dtype != torch.float32 and (N in (5120, 6144) or (N == 4096 and not rms)))
+        same_bwd_layout = same_bwd_layout and not _staged(dtype, N)
         if rms:
             dh, dg = cabi.add_rms_norm_bwd(dyg, ghg, h, rstd, gg)
             udx, udg = cabi.rms_norm_bwd(dyg, h, rstd, gg)
@@ -119,6 +129,13 @@ def test_add_norm_forward_and_backward(cabi, oracle, gpu, dtype, shape, mixed):
                 assert_same_arithmetic(db, udb, what + " dbeta, fused against plain")
             sl = colsum_slack(dy.double()) if wtol == torch.float32 else None
             assert_close(db, odb, wtol, what + " dbeta", slack=sl)
+        if _staged(dtype, N):
+            pdx = (oracle.rms_norm_bwd(to_np32(dy), to_np32(h), (N,), to_np32(rstd), to_np32(gamma))
+                   if rms else oracle.layer_norm_bwd(to_np32(dy), to_np32(h), (N,), to_np32(mean),
+                                                     to_np32(rstd), to_np32(gamma)))[0]
+            assert_close(udx, pdx, dtype, what + " plain dx")
+            assert_close(udg, odg, wtol, what + " plain dgamma",
+                         slack=colsum_slack(dy.double() * xhat) if wtol == torch.float32 else None)
         assert torch.equal(nh, udx), what + ": no residual gradient must be the plain backward"
         if same_bwd_layout:
             assert_same_arithmetic(dg, udg, what + " dgamma, fused against plain", max_fraction=0.05)
@@ -152,10 +169,18 @@ def test_output_cast_of_float32_rows(cabi, oracle, gpu, ydtype):
                 else:
                     y, h, mean, rstd = cabi.add_layer_norm_fwd(xg, r, gg, bg, 1e-5, y_dtype=ydtype)
                     y32, h32, mean32, rstd32 = cabi.add_layer_norm_fwd(xg, r, gg, bg, 1e-5)
-                    assert torch.equal(mean, mean32)
+                    if _staged(torch.float32, N) and not add:
+                        assert_close(mean, to_np32(mean32), torch.float32, "mean, cast against plain")
+                    else:
+                        assert torch.equal(mean, mean32)
                 assert y.dtype == ydtype
-                assert_same_arithmetic(y, y32.to(ydtype), "cast y against the float32 y converted")
-                assert torch.equal(rstd, rstd32)
+                if _staged(torch.float32, N) and not add:
+                    # (the float32 y comes from the LDS-staged kernel, the cast one does not)
+                    assert_close(y, to_np32(y32), ydtype, "cast y against the float32 y")
+                    assert_close(rstd, to_np32(rstd32), torch.float32, "rstd, cast against plain")
+                else:
+                    assert_same_arithmetic(y, y32.to(ydtype), "cast y against the float32 y converted")
+                    assert torch.equal(rstd, rstd32)
                 if add:
                     assert torch.equal(h, h32) and torch.equal(h.cpu(), x + res)
                 else:

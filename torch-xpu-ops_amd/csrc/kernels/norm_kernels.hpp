@@ -743,6 +743,132 @@ norm_fwd_flat_kernel(const T* __restrict__ x, const WT* __restrict__ gamma,
 }
 
 // ---------------------------------------------------------------------------
+// Backward for the rows norm_fwd_flat_kernel serves (short ragged rows, 16-byte aligned
+// dY, X and dX): pieces of `chunk_rows` consecutive rows of dY and X enter LDS with
+// whole aligned accesses, a group of G lanes works a row there (s1, s2 reduced inside
+// the wavefront, dX written over the row of dY in LDS), and the piece of dX leaves with
+// whole 128-bit stores.  A lane owns the same columns in every row, so it keeps their
+// dgamma / dbeta sums in registers over all the pieces its workgroup walks (a grid-stride
+// loop over pieces, so the partial rows are as many as the general kernel's).  At the
+// end the lane groups of the workgroup are folded through LDS in a fixed order and one
+// fp32 row goes to the [gridDim.x, N] partial buffers; colsum_finalize_kernel adds those.
+// Arithmetic of a row: that of norm_bwd_resident_kernel.
+template <class T, class WT, int G, int VP, int BLOCK, int LDSB, bool RMS>
+__global__ void __launch_bounds__(BLOCK)
+norm_bwd_flat_kernel(const T* __restrict__ dy, const T* __restrict__ x,
+                     const float* __restrict__ mean, const float* __restrict__ rstd,
+                     const WT* __restrict__ gamma, T* __restrict__ dx,
+                     float* __restrict__ part_dg, float* __restrict__ part_db, int64_t M, int N,
+                     int chunk_rows) {
+  constexpr int E = elems_per_pack<T>::value;
+  constexpr int RPB = BLOCK / G;
+  constexpr int U = LDSB / (BLOCK * 16);
+  // two tensors of a piece; afterwards the fold of the column sums (RPB * G * VP * E floats)
+  constexpr int kBufElems = LDSB / (int)sizeof(T) + E;
+  constexpr int kFoldBytes = BLOCK * VP * E * (int)sizeof(float);
+  constexpr int kBytes = 2 * kBufElems * (int)sizeof(T) > kFoldBytes
+                             ? 2 * kBufElems * (int)sizeof(T) : kFoldBytes;
+  __shared__ __attribute__((aligned(16))) unsigned char lds[kBytes];
+  T* bd = reinterpret_cast<T*>(lds);
+  T* bx = bd + kBufElems;
+  const int lane = threadIdx.x % G;
+  const int slot = threadIdx.x / G;
+  const bool want_cols = part_dg != nullptr;  // uniform
+  const float fN = (float)N, inv_n = 1.0f / fN;
+  Pack<WT, E> gp[VP];
+  float dg[VP][E], db[RMS ? 1 : VP][RMS ? 1 : E];
+#pragma unroll
+  for (int c = 0; c < VP; ++c) {
+    const int j = (c * G + lane) * E;
+    gp[c] = gamma ? load_row_pack<WT, E, false>(gamma, j, N, true, 1.0f) : Pack<WT, E>::splat(1.0f);
+#pragma unroll
+    for (int i = 0; i < E; ++i) {
+      dg[c][i] = 0.0f;
+      if constexpr (!RMS) db[c][i] = 0.0f;
+    }
+  }
+  const int64_t npieces = (M + chunk_rows - 1) / chunk_rows;
+  for (int64_t piece = blockIdx.x; piece < npieces; piece += gridDim.x) {
+    const int64_t row0 = piece * chunk_rows;
+    const int rows_here = M - row0 < chunk_rows ? (int)(M - row0) : chunk_rows;
+    const int nelem = rows_here * N;
+    flat_stage_in2<T, BLOCK, U>(dy + row0 * (int64_t)N, bd, x + row0 * (int64_t)N, bx, nelem);
+    __syncthreads();
+    for (int r = slot; r < rows_here; r += RPB) {
+      T* rd = bd + r * N;
+      const T* rx = bx + r * N;
+      const float mu = RMS ? 0.0f : mean[row0 + r];
+      const float rs = rstd[row0 + r];
+      float gy[VP][E], xh[VP][E];
+      float s1 = 0.0f, s2 = 0.0f;
+#pragma unroll
+      for (int c = 0; c < VP; ++c) {
+        const int j = (c * G + lane) * E;
+        Pack<T, E> pd = Pack<T, E>::zero(), px = Pack<T, E>::zero();
+        if (j < N) {
+          pd = flat_row_pack<T, E>(rd, j);
+          px = flat_row_pack<T, E>(rx, j);
+        }
+#pragma unroll
+        for (int i = 0; i < E; ++i) {
+          const bool in = j + i < N;
+          gy[c][i] = in ? pd.get(i) : 0.0f;
+          xh[c][i] = in ? (px.get(i) - mu) * rs : 0.0f;
+          const float g = gy[c][i] * gp[c].get(i);
+          if constexpr (!RMS) s1 += g;
+          s2 = fmaf(g, xh[c][i], s2);
+          dg[c][i] = fmaf(gy[c][i], xh[c][i], dg[c][i]);
+          if constexpr (!RMS) db[c][i] += gy[c][i];
+        }
+      }
+      if constexpr (!RMS) s1 = wave_group_allreduce<G, SumOp>(s1);
+      s2 = wave_group_allreduce<G, SumOp>(s2);
+      const float term1 = row_mean_of<T>(rs, fN, inv_n);
+#pragma unroll
+      for (int c = 0; c < VP; ++c) {
+        const int j = (c * G + lane) * E;
+        Pack<T, E> o;
+#pragma unroll
+        for (int i = 0; i < E; ++i) {
+          // dx = (rs / N) * (N * g - xhat * s2 - s1), g = dy * gamma
+          float f = fN * (gy[c][i] * gp[c].get(i));
+          f -= xh[c][i] * s2;
+          if constexpr (!RMS) f -= s1;
+          o.set(i, f * term1);
+        }
+        if (j < N) flat_row_store<T, E>(rd, j, N - j, o);
+      }
+    }
+    __syncthreads();
+    if (dx != nullptr) flat_stage_out<T, BLOCK, U>(dx + row0 * (int64_t)N, bd, nelem);
+    __syncthreads();  // the buffers are filled again, or folded over, next
+  }
+  if (!want_cols) return;
+  // fold the lane groups that own the same columns, in slot order, one sum kind at a time
+  float* fold = reinterpret_cast<float*>(lds);
+  float* out_g = part_dg + (int64_t)blockIdx.x * N;
+  float* out_b = RMS ? nullptr : part_db + (int64_t)blockIdx.x * N;
+  constexpr int NPASS = RMS ? 1 : 2;
+  constexpr int COLS = G * VP * E;  // columns a lane group covers
+#pragma unroll
+  for (int pass = 0; pass < NPASS; ++pass) {
+#pragma unroll
+    for (int c = 0; c < VP; ++c)
+#pragma unroll
+      for (int i = 0; i < E; ++i)
+        fold[slot * COLS + (c * G + lane) * E + i] =
+            pass == 0 ? dg[c][i] : db[RMS ? 0 : c][RMS ? 0 : i];
+    __syncthreads();
+    for (int j = threadIdx.x; j < N; j += BLOCK) {
+      float t = 0.0f;
+      for (int sl = 0; sl < RPB; ++sl) t += fold[sl * COLS + j];
+      (pass == 0 ? out_g : out_b)[j] = t;
+    }
+    __syncthreads();
+  }
+}
+
+// ---------------------------------------------------------------------------
 // Forward for rows too wide to hold in registers: one workgroup per row, the
 // row is streamed from memory twice (statistics, normalize); the second pass
 // hits L2 / Infinity Cache for any realistic row.  LayerNorm sums (x - k) and

@@ -220,11 +220,73 @@ inline bool launch_norm_bwd_exact(const Plan& plan, const NormBwdArgs& a, hipStr
   return (launch_norm_bwd_exact_at<T, WT, RMS, ADD, Is>(plan, a, stream) || ...);
 }
 
+// Backward of short ragged rows through LDS (norm_bwd_flat_kernel): two tensors of a piece
+// in 16 KB each, 32 KB each for rows beyond 1024 16-bit elements.  The grid walks the pieces
+// with a stride, as many workgroups as the plan has partial rows (the size of the caller's
+// workspace); `*rows_out` receives how many partial rows the launch fills.
+// 16-bit rows take it on up to 8 lanes a row (24 packs, 192 elements), fp32 rows at every
+// length it covers: with 8 elements a pack the lane's gy / xhat / dgamma / dbeta registers are
+// twice the fp32 kernel's and the general kernel wins from 16 lanes on.  131072 rows, LayerNorm /
+// RMSNorm in us, general kernel -> this one: bf16 N = 17 31.7 / 24.7 -> 13.8 / 13.5, 100 42.6 /
+// 36.9 -> 28.6 / 27.3, 127 54.1 / 48.8 -> 35.6 / 34.6, 150 54.3 / 48.7 -> 49.1 / 45.9, 257 (16
+// lanes) 74.0 / 67.0 -> 85.1 / 76.8, 1001 169 / 163 -> 203 / 202; fp32 N = 17 30.6 / 23.0 -> 16.3 /
+// 15.2, 63 47.2 / 41.4 -> 27.7 / 27.1, 127 78.9 / 74.1 -> 45.3 / 44.0, 257 96.2 / 90.9 -> 94.9 /
+// 92.4, 1001 329 / 323 -> 312 / 306.  More workgroups than the plan's partial rows (3, 4 or 8 a
+// compute unit instead of 2) measured slower at most lengths.
+constexpr bool norm_bwd_flat_serves(size_t esize, int lanes) { return esize == 4 || lanes <= 8; }
+template <class T, class WT, bool RMS, int LDSB>
+bool launch_norm_bwd_flat_l(const Plan& plan, FlatLayout f, int cr, const NormBwdArgs& a,
+                            hipStream_t stream, int* rows_out) {
+  const int64_t pieces = (a.M + cr - 1) / cr;
+  const int64_t cap = a.part_dg != nullptr ? (int64_t)plan.partial_rows : (int64_t)0x7fffffff;
+  const int64_t grid = pieces < cap ? pieces : cap;
+  if (grid < 1) return false;
+#define ROWNORM_FLAT_NORM_BWD(GL, VP)                                                           \
+  case GL * 8 + VP:                                                                             \
+    if constexpr ((LDSB <= kFlatLdsBytes || (GL == 64 && VP >= 3)) &&                           \
+                  norm_bwd_flat_serves(sizeof(T), GL)) {                                        \
+      hipLaunchKernelGGL((norm_bwd_flat_kernel<T, WT, GL, VP, kFlatBlock, LDSB, RMS>),           \
+                         dim3((unsigned)grid), dim3(kFlatBlock), 0, stream, (const T*)a.dy,      \
+                         (const T*)a.x, a.mean, a.rstd, (const WT*)a.gamma, (T*)a.dx, a.part_dg, \
+                         a.part_db, a.M, a.N, cr);                                              \
+      *rows_out = (int)grid;                                                                    \
+      return true;                                                                              \
+    }                                                                                           \
+    return false;
+  switch (f.g * 8 + f.vp) { ROWNORM_FLAT_ALL(ROWNORM_FLAT_NORM_BWD) }
+#undef ROWNORM_FLAT_NORM_BWD
+  return false;
+}
+
+template <class T, class WT, bool RMS>
+bool launch_norm_bwd_flat(const Plan& plan, FlatLayout f, const NormBwdArgs& a, hipStream_t stream,
+                          int* rows_out) {
+  int cr = flat_chunk_rows<T>(a.N, f.g, kFlatLdsBytes);
+  if (cr >= 8)
+    return launch_norm_bwd_flat_l<T, WT, RMS, kFlatLdsBytes>(plan, f, cr, a, stream, rows_out);
+  cr = flat_chunk_rows<T>(a.N, f.g, 2 * kFlatLdsBytes);
+  if (cr >= 8)
+    return launch_norm_bwd_flat_l<T, WT, RMS, 2 * kFlatLdsBytes>(plan, f, cr, a, stream, rows_out);
+  return false;
+}
+
 template <class T, class WT, bool RMS, bool ADD>
 int launch_norm_bwd(const Plan& plan, const NormBwdArgs& a, hipStream_t stream) {
   const bool want_cols = a.part_dg != nullptr;
   const T* dres = ADD ? (const T*)a.dres : nullptr;
-  if (plan.resident && plan.exact_depth > 0) {
+  int partial_rows = (int)plan.partial_rows;
+  bool flat = false;
+  // short ragged rows (no residual gradient, 16-byte aligned dY, X and dX): staged through LDS
+  if constexpr (!ADD) {
+    if (plan.resident && !plan.fast && plan.exact_depth == 0 && !plan.window) {
+      const FlatLayout f = flat_layout<T>(plan, a.M, a.N, a.dy, a.x, a.dx);
+      flat = f.g != 0 && norm_bwd_flat_serves(sizeof(T), f.g) &&
+             launch_norm_bwd_flat<T, WT, RMS>(plan, f, a, stream, &partial_rows);
+    }
+  }
+  if (flat) {
+    // (launched above)
+  } else if (plan.resident && plan.exact_depth > 0) {
     static_assert(kNormBwdExactCount == 15, "one index per table entry below");
     if (a.dx == nullptr || !launch_norm_bwd_exact<T, WT, RMS, ADD>(
                                plan, a, stream, ilist<0, 1, 2, 3, 4, 5, 6, 7, 8, 9, 10, 11, 12, 13, 14>{}))
@@ -296,7 +358,7 @@ int launch_norm_bwd(const Plan& plan, const NormBwdArgs& a, hipStream_t stream) 
   const unsigned gx = (unsigned)((a.N + kFinalizeCols - 1) / kFinalizeCols);
   hipLaunchKernelGGL((colsum_finalize_kernel<WT>), dim3(gx, RMS ? 1 : 2), dim3(1024), 0, stream,
                      (const float*)a.part_dg, (const float*)a.part_db, (WT*)a.dgamma,
-                     (WT*)a.dbeta, (int)plan.partial_rows, a.N);
+                     (WT*)a.dbeta, partial_rows, a.N);
   return (int)hipGetLastError();
 }
 
