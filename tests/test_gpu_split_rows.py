@@ -156,3 +156,40 @@ def test_fallbacks_keep_a_row_on_one_workgroup(cabi, oracle, gpu):
     assert L.mi355x_layer_norm_bwd(P(dyg), P(xg), P(mean_g), P(rstd_g), P(gg), P(dx2), None, None,
                                    None, 0, M, N, F32, F32, stream) == 0
     assert_close(dx2, odx, torch.float32, "dx, no workspace")
+
+
+@pytest.mark.parametrize("wdtype", [torch.bfloat16, torch.float32], ids=str)
+def test_one_partial_row_writes_the_column_sums_itself(cabi, oracle, gpu, wdtype):
+    """Rows so long that the columns alone fill the machine (bf16 from 1048576 elements) take one
+    partial row, and the column-sum kernels then write dgamma / dbeta themselves, rounded once
+    from the fp32 sums, without a second stage (the reference's second stage is the at::sum over
+    its block buffers, LayerNormKernels.cpp:1312-1314): each wanted alone, both with dX (the fused
+    dX + column-sum kernel), a ragged row end, and RMSNorm."""
+    for (M, N) in ((3, 1048576 + 24), (5, 1048576 + 3)):
+        p = cabi.plan(cabi.OP_LAYER_NORM_BWD, M, N, cabi.BF16, cabi.dtype_code(wdtype))
+        assert p["resident"] == 0 and p["partial_rows"] == 1, p
+        g = gen(1700 + M)
+        x = (0.5 + torch.randn(M, N, generator=g)).bfloat16()
+        dy = torch.randn(M, N, generator=g).bfloat16()
+        gamma = (1 + 0.1 * torch.randn(N, generator=g)).to(wdtype)
+        xg, dyg, gg = x.to(gpu), dy.to(gpu), gamma.to(gpu)
+        what = "[%d, %d] weights %s" % (M, N, wdtype)
+        _, mean, rstd = cabi.layer_norm_fwd(xg, gg, None, 1e-5)
+        odx, odg, odb = oracle.layer_norm_bwd(to_np32(dy), to_np32(x), (N,), to_np32(mean),
+                                              to_np32(rstd), to_np32(gamma))
+        dx, dg, db = cabi.layer_norm_bwd(dyg, xg, mean, rstd, gg)
+        assert_close(dx, odx, torch.bfloat16, "dx " + what)
+        assert_close(dg, odg, wdtype, "dgamma " + what)
+        assert_close(db, odb, wdtype, "dbeta " + what)
+        _, dg1, n1 = cabi.layer_norm_bwd(dyg, xg, mean, rstd, gg, want=(False, True, False))
+        _, n2, db1 = cabi.layer_norm_bwd(dyg, xg, mean, rstd, gg, want=(False, False, True))
+        assert n1 is None and n2 is None
+        assert_close(dg1, odg, wdtype, "dgamma alone " + what)
+        assert_close(db1, odb, wdtype, "dbeta alone " + what)
+        dx2, dg2, n3 = cabi.layer_norm_bwd(dyg, xg, mean, rstd, gg, want=(True, True, False))
+        assert n3 is None and torch.equal(dx2, dx) and torch.equal(dg2, dg)
+        _, rr = cabi.rms_norm_fwd(xg, gg, 1e-6)
+        rdx, rdg = cabi.rms_norm_bwd(dyg, xg, rr, gg)
+        rodx, rodg = oracle.rms_norm_bwd(to_np32(dy), to_np32(x), (N,), to_np32(rr), to_np32(gamma))
+        assert_close(rdx, rodx, torch.bfloat16, "rms dx " + what)
+        assert_close(rdg, rodg, wdtype, "rms dgamma " + what)

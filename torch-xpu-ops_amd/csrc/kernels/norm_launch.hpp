@@ -275,6 +275,8 @@ int launch_norm_bwd(const Plan& plan, const NormBwdArgs& a, hipStream_t stream) 
   const bool want_cols = a.part_dg != nullptr;
   const T* dres = ADD ? (const T*)a.dres : nullptr;
   int partial_rows = (int)plan.partial_rows;
+  // one partial row (few, very long rows): the column-sum kernels write dgamma / dbeta themselves
+  const bool direct = want_cols && !plan.resident && plan.partial_rows == 1;
   bool flat = false;
   // short ragged rows (no residual gradient, 16-byte aligned dY, X and dX): staged through LDS
   if constexpr (!ADD) {
@@ -323,7 +325,7 @@ int launch_norm_bwd(const Plan& plan, const NormBwdArgs& a, hipStream_t stream) 
                            dim3(gx, (unsigned)plan.partial_rows), dim3(CB), 0, stream,
                            (const T*)a.dy, (const T*)a.x, dres, a.mean, a.rstd,
                            (const WT*)a.gamma, (const float*)totals, (T*)a.dx, a.part_dg,
-                           a.part_db, a.M, a.N);
+                           a.part_db, (WT*)a.dgamma, (WT*)a.dbeta, (int)direct, a.M, a.N);
         cols_done = true;
       } else {
         hipLaunchKernelGGL((norm_bwd_split_dx_kernel<T, WT, kStreamBlock, RMS>), grid,
@@ -340,14 +342,14 @@ int launch_norm_bwd(const Plan& plan, const NormBwdArgs& a, hipStream_t stream) 
     if (want_cols && !cols_done) {
       constexpr int CB = 256;
       const unsigned gx = (unsigned)((a.N + CB * E - 1) / (CB * E));
-      hipLaunchKernelGGL((norm_bwd_stream_colsum_kernel<T, CB, RMS>),
+      hipLaunchKernelGGL((norm_bwd_stream_colsum_kernel<T, WT, CB, RMS>),
                          dim3(gx, (unsigned)plan.partial_rows), dim3(CB), 0, stream,
                          (const T*)a.dy, (const T*)a.x, a.mean, a.rstd, a.part_dg, a.part_db,
-                         a.M, a.N);
+                         (WT*)a.dgamma, (WT*)a.dbeta, (int)direct, a.M, a.N);
     }
   }
   int err = (int)hipGetLastError();
-  if (err != 0 || !want_cols) return err;
+  if (err != 0 || !want_cols || direct) return err;
   if (!plan.resident && plan.partial_rows <= kFinalizeFlatRows) {
     const unsigned gx = (unsigned)((a.N + kFinalizeFlatCols - 1) / kFinalizeFlatCols);
     hipLaunchKernelGGL((colsum_finalize_flat_kernel<WT>), dim3(gx, RMS ? 1 : 2), dim3(256), 0,
