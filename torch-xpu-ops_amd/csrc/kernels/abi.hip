@@ -410,6 +410,19 @@ int softmax_fwd(const void* x, const void* mask, void* y, int64_t rows, int64_t 
   SoftmaxFwdArgs a{x,    y, (const uint8_t*)mask, (uint32_t)mr.div, (uint32_t)mr.mod, mr.stride,
                    rows, (int)N, flags};
   hipStream_t s = (hipStream_t)stream;
+  // few very long rows: the team forward (whole packs on 16-byte aligned tensors, no mask,
+  // Y apart from X -- a workgroup whose team does not come together reads the whole row
+  // again -- and no stream capture)
+  if (plan.team > 0 && !mask && ((((uintptr_t)x) | ((uintptr_t)y)) & 15u) == 0) {
+    const char* xb = (const char*)x;
+    const char* yb = (const char*)y;
+    const size_t xbytes = (size_t)rows * (size_t)N * (size_t)esize_of(id);
+    const size_t ybytes = (size_t)rows * (size_t)N * (size_t)esize_of(od);
+    if (!(xb < yb + ybytes && yb < xb + xbytes)) {
+      a.team_slot = team_slot_for_call(s, &a.team_id);
+      a.team_wait_ticks = g_team_wait_ticks.load(std::memory_order_relaxed);
+    }
+  }
   if (id == ROWNORM_F32) return launch_softmax_fwd<float, float>(plan, a, s);
   if (id == ROWNORM_BF16) return launch_softmax_fwd<bf16, bf16>(plan, a, s);
   return od == ROWNORM_F32 ? launch_softmax_fwd<f16, float>(plan, a, s)
@@ -434,6 +447,22 @@ int softmax_bwd(const void* grad, const void* y, const void* mask, void* gi, int
   SoftmaxBwdArgs a{grad, y, gi, (const uint8_t*)mask, (uint32_t)mr.div, (uint32_t)mr.mod,
                    mr.stride, rows, (int)N, flags};
   hipStream_t s = (hipStream_t)stream;
+  // few very long rows: the team backward, under the rules of the forward (gi apart from
+  // grad and y)
+  if (plan.team > 0 && !mask &&
+      ((((uintptr_t)grad) | ((uintptr_t)y) | ((uintptr_t)gi)) & 15u) == 0) {
+    const char* ob = (const char*)gi;
+    const size_t ibytes = (size_t)rows * (size_t)N * (size_t)esize_of(gd);
+    const size_t obytes = (size_t)rows * (size_t)N * (size_t)esize_of(od);
+    auto apart = [&](const void* in) {
+      const char* ib = (const char*)in;
+      return !(ib < ob + obytes && ob < ib + ibytes);
+    };
+    if (apart(grad) && apart(y)) {
+      a.team_slot = team_slot_for_call(s, &a.team_id);
+      a.team_wait_ticks = g_team_wait_ticks.load(std::memory_order_relaxed);
+    }
+  }
   if (gd == ROWNORM_BF16) return launch_softmax_bwd<bf16, bf16>(plan, a, s);
   if (gd == ROWNORM_F16) return launch_softmax_bwd<f16, f16>(plan, a, s);
   return od == ROWNORM_F16 ? launch_softmax_bwd<float, f16>(plan, a, s)

@@ -1,0 +1,98 @@
+// Device side of the exchange between the workgroups of a team (norm_fwd_team_kernel,
+// softmax_fwd_team_kernel): a row too long for one workgroup is held in the registers of
+// several, which pass two numbers each through library-owned device memory.
+//
+// What crosses workgroups.  An entry is {tag, s1, s2}, 128 bytes apart; the tag of a
+// finished entry is (call id << 32) | (round + 1), ids being unique per call, so
+// nothing has to be cleared and an entry left by an earlier call or round never
+// counts.  The writer sets the tag to 0 when it starts on a row, later stores s1
+// and s2, waits for those stores to be acknowledged and stores the tag; a reader
+// accepts s1 and s2 only if it read the expected tag before and after them.  Every
+// access is a device-scope atomic store or load, which goes to memory: no
+// read-modify-write (256 workgroups counting on one word took hundreds of
+// microseconds), and no release or acquire fence (each writes back or invalidates a
+// whole L2).  Two calls that were handed the same slot while both run -- possible
+// only with more such calls in flight than slots -- overwrite each other's tags and
+// therefore never accept each other's numbers.
+//
+// The wait is bounded, and no workgroup depends on another to finish.  A workgroup
+// stops waiting when its team is complete, when any workgroup of the call has given
+// up before (a hint word in the slot), or after `wait_ticks` of the constant-rate
+// clock (the workgroups can only fail to be resident together while other kernels
+// hold compute units for that long).  What a workgroup does without its team is the
+// kernel's business; it keeps publishing its own numbers for the workgroups that do
+// wait.
+#pragma once
+
+#include <stdint.h>
+
+#include "../plan.hpp"
+
+namespace rownorm {
+
+__device__ __forceinline__ unsigned long long team_load(const unsigned long long* p) {
+  return __hip_atomic_load(p, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+}
+__device__ __forceinline__ void team_store(unsigned long long* p, unsigned long long v) {
+  __hip_atomic_store(p, v, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+}
+// Earlier stores of this lane have been acknowledged and its loads have returned.
+__device__ __forceinline__ void team_stores_done() {
+  asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
+}
+
+// For the first wavefront of a workgroup (all 64 lanes, threadIdx.x < 64), whose entry
+// `entries[blockIdx.x]` has had the tag 0 since the workgroup started on the row:
+// publishes (a, b), waits for the `team` entries from `entries[tm * team]` on and leaves
+// them in part[j][0..1] (LDS).  True when the team came together (the same in every lane);
+// false after the wait ran out or another workgroup of the call gave up, which this one
+// then records in the slot's hint word.
+__device__ __forceinline__ bool team_publish_and_gather(TeamSlot* slot, TeamEntry* entries, int tm,
+                                                        int team, unsigned int call_id,
+                                                        unsigned int round,
+                                                        unsigned long long wait_ticks, double a,
+                                                        double b, double (*part)[2]) {
+  const int lane = (int)threadIdx.x;
+  const unsigned long long expect = ((unsigned long long)call_id << 32) | (round + 1u);
+  if (lane == 0) {
+    TeamEntry* mine = &entries[blockIdx.x];
+    team_stores_done();  // the tag has been 0 in memory before the numbers change
+    team_store(&mine->s1, __builtin_bit_cast(unsigned long long, a));
+    team_store(&mine->s2, __builtin_bit_cast(unsigned long long, b));
+    team_stores_done();
+    team_store(&mine->tag, expect);
+  }
+  const TeamEntry* mates = entries + tm * team;
+  const unsigned long long t0 = wall_clock64();
+  bool complete = false;
+  unsigned int polls = 0;
+  for (;;) {
+    bool ok = true;
+    for (int j = lane; j < team; j += 64) ok = ok && team_load(&mates[j].tag) == expect;
+    if (__ballot(ok) == __ballot(true)) {
+      for (int j = lane; j < team; j += 64) {
+        part[j][0] = __builtin_bit_cast(double, team_load(&mates[j].s1));
+        part[j][1] = __builtin_bit_cast(double, team_load(&mates[j].s2));
+        team_stores_done();  // the numbers have returned before the tag is read again
+        ok = ok && team_load(&mates[j].tag) == expect;
+      }
+      if (__ballot(ok) == __ballot(true)) {
+        complete = true;
+        break;
+      }
+    }
+    // (the hint word is one address for the whole grid: looked at every 16th time)
+    if ((polls++ & 15u) == 0) {
+      const unsigned int hint =
+          __hip_atomic_load(&slot->gave_up, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+      if (hint == call_id) break;
+    }
+    if (wall_clock64() - t0 > wait_ticks) break;
+    __builtin_amdgcn_s_sleep(8);
+  }
+  if (lane == 0 && !complete)
+    __hip_atomic_store(&slot->gave_up, call_id, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+  return complete;
+}
+
+}  // namespace rownorm

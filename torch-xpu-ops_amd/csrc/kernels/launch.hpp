@@ -60,6 +60,11 @@ struct SoftmaxFwdArgs {
   int64_t M;
   int N;
   int flags;  // kSoftmaxLog | kSoftmaxSafe
+  // few very long rows held by teams of workgroups (softmax_fwd_team_kernel): the call's
+  // slot of bookkeeping memory, its id and the bound of a wait; null = not for this call
+  void* team_slot = nullptr;
+  unsigned int team_id = 0;
+  unsigned long long team_wait_ticks = 0;
 };
 
 struct SoftmaxBwdArgs {
@@ -72,6 +77,10 @@ struct SoftmaxBwdArgs {
   int64_t M;
   int N;
   int flags;
+  // few very long rows held by teams of workgroups (softmax_bwd_team_kernel), as in the forward
+  void* team_slot = nullptr;
+  unsigned int team_id = 0;
+  unsigned long long team_wait_ticks = 0;
 };
 
 struct SoftmaxStridedFwdArgs {

@@ -36,6 +36,7 @@
 #include "device/pack.hpp"
 #include "plan.hpp"
 #include "device/reduce.hpp"
+#include "device/team.hpp"
 
 namespace rownorm {
 
@@ -614,18 +615,6 @@ __device__ __forceinline__ void long_row_apply(const T* xr, const T* rr, const W
       });
 }
 
-// Device-scope accesses of the team kernel's bookkeeping memory (see norm_fwd_team_kernel).
-__device__ __forceinline__ unsigned long long team_load(const unsigned long long* p) {
-  return __hip_atomic_load(p, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
-}
-__device__ __forceinline__ void team_store(unsigned long long* p, unsigned long long v) {
-  __hip_atomic_store(p, v, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
-}
-// Earlier stores of this lane have been acknowledged and its loads have returned.
-__device__ __forceinline__ void team_stores_done() {
-  asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
-}
-
 // ---------------------------------------------------------------------------
 // Forward for short ragged rows (N % E != 0, up to 64 lanes x kFlatMaxPacks packs) through
 // LDS, as the softmax kernels for such rows (device/flat_rows.hpp): a run of
@@ -974,28 +963,11 @@ norm_fwd_stream_kernel(const T* __restrict__ x, const T* res, const WT* __restri
 // the current ones are normalized and stored, so no pack waits for the store of the
 // pack before it (bf16 [512, 401408]: 177 -> 170 us).
 //
-// What crosses workgroups.  An entry is {tag, s1, s2}, 128 bytes apart; the tag of a
-// finished entry is (call id << 32) | (round + 1), ids being unique per call, so
-// nothing has to be cleared and an entry left by an earlier call or round never
-// counts.  The writer sets the tag to 0 when it starts on a row, later stores s1
-// and s2, waits for those stores to be acknowledged and stores the tag; a reader
-// accepts s1 and s2 only if it read the expected tag before and after them.  Every
-// access is a device-scope atomic store or load, which goes to memory: no
-// read-modify-write (256 workgroups counting on one word took hundreds of
-// microseconds), and no release or acquire fence (each writes back or invalidates a
-// whole L2).  Two calls that were handed the same slot while both run -- possible
-// only with more such calls in flight than slots -- overwrite each other's tags and
-// therefore never accept each other's sums.
-//
-// The wait is bounded, and no workgroup depends on another to finish.  A workgroup
-// stops waiting when its team is complete, when any workgroup of the call has given
-// up before (a hint word in the slot), or after `wait_ticks` of the constant-rate
-// clock (the workgroups can only fail to be resident together while other kernels
-// hold compute units for that long).  A workgroup that stops without its team sums
-// the whole row itself -- a second pass over X, whose statistics agree with the
-// team's to rounding -- loads its chunk again and goes on; it keeps publishing its
-// partial sums for the workgroups that do wait.  Every wave reaches the end of the
-// kernel whatever the other workgroups do, and every row is written.
+// What crosses workgroups and how the wait is bounded: device/team.hpp.  A workgroup
+// that stops waiting without its team sums the whole row itself -- a second pass over X,
+// whose statistics agree with the team's to rounding -- loads its chunk again and goes
+// on.  Every wave reaches the end of the kernel whatever the other workgroups do, and
+// every row is written.
 //
 // GROUP: the rows are the (sample, group) slabs of a GroupNorm whose channels are whole
 // packs (`group.packs_per_channel` packs each): gamma and beta hold one value a channel,
@@ -1090,47 +1062,11 @@ norm_fwd_team_kernel(const T* __restrict__ x, const WT* __restrict__ gamma,
     block_sum2_f64<BLOCK>(s1, s2, red);
     if (threadIdx.x < 64) {  // the first wavefront publishes, waits and adds up
       const int lane = (int)threadIdx.x;
-      const unsigned long long expect = ((unsigned long long)call_id << 32) | (round + 1u);
-      if (lane == 0) {
-        TeamEntry* mine = &entries[blockIdx.x];
-        team_stores_done();  // the tag has been 0 in memory before the sums change
-        team_store(&mine->s1, __builtin_bit_cast(unsigned long long, s1));
-        team_store(&mine->s2, __builtin_bit_cast(unsigned long long, s2));
-        team_stores_done();
-        team_store(&mine->tag, expect);
-      }
-      const TeamEntry* mates = entries + tm * team;
-      const unsigned long long t0 = wall_clock64();
-      bool complete = false;
-      unsigned int polls = 0;
-      for (;;) {
-        bool ok = true;
-        for (int j = lane; j < team; j += 64) ok = ok && team_load(&mates[j].tag) == expect;
-        if (__ballot(ok) == __ballot(true)) {
-          for (int j = lane; j < team; j += 64) {
-            tpart[j][0] = __builtin_bit_cast(double, team_load(&mates[j].s1));
-            tpart[j][1] = __builtin_bit_cast(double, team_load(&mates[j].s2));
-            team_stores_done();  // the sums have returned before the tag is read again
-            ok = ok && team_load(&mates[j].tag) == expect;
-          }
-          if (__ballot(ok) == __ballot(true)) {
-            complete = true;
-            break;
-          }
-        }
-        // (the hint word is one address for the whole grid: looked at every 16th time)
-        if ((polls++ & 15u) == 0) {
-          const unsigned int hint =
-              __hip_atomic_load(&slot->gave_up, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
-          if (hint == call_id) break;
-        }
-        if (wall_clock64() - t0 > wait_ticks) break;
-        __builtin_amdgcn_s_sleep(8);
-      }
+      const bool complete = team_publish_and_gather(slot, entries, tm, team, call_id, round,
+                                                    wait_ticks, s1, s2, tpart);
       // (the lanes of a wavefront see one another's LDS stores in program order)
       if (lane == 0) {
         if (!complete) {
-          __hip_atomic_store(&slot->gave_up, call_id, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
           stat[3] = 1.0f;
         } else {
           double t1 = 0.0, t2 = 0.0;

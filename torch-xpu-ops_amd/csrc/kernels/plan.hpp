@@ -95,6 +95,11 @@ struct TeamSlot {
   unsigned int pad[3];
 };
 
+// softmax_fwd_team_kernel / softmax_bwd_team_kernel: rows of at least this many packs (64 KiB),
+// and the packs a lane the backward holds of each of its two tensors at most.
+constexpr int64_t kSoftmaxTeamMinPacks = 4096;
+constexpr int kSoftmaxBwdTeamMaxV = 8;
+
 constexpr int kMinG = 8;
 constexpr int kMaxG = 1024;
 constexpr int kMaxV = 16;
@@ -924,6 +929,35 @@ inline int make_plan(OpClass oc, int64_t M, int64_t N, int esize, int num_cus, c
       p.team_v = (int)v;
       p.team_chunk_packs = v * kTeamBlock;
       p.team_grid = teams * team;
+    }
+  }
+  // Softmax forward / backward of few, very long rows of whole packs: one workgroup a row
+  // would leave most compute units idle, so each row is held by a team of workgroups
+  // (softmax_fwd_team_kernel / softmax_bwd_team_kernel): as few workgroups a row as hold it
+  // with 16 (backward: 8 of each tensor) packs a lane, then as many teams as there are rows
+  // and room, and a row spread over all the workgroups its team can have.  More rows than
+  // teams run in rounds; even then, and with few teams whose waits nothing hides, one
+  // workgroup a row is several times slower (fp32 [2, 16777216]: 4800 us).
+  if (softmax && p.fast && !masked && ov.G == 0 && ov.V == 0 && ov.bpc == 0 && ov.block == 0 &&
+      2 * M <= num_cus && packs >= kSoftmaxTeamMinPacks) {
+    const int64_t cus = num_cus * kTeamPerCu < kTeamMaxWorkgroups ? num_cus * kTeamPerCu : kTeamMaxWorkgroups;
+    const int max_v = oc == OC_SOFTMAX_FWD ? kTeamMaxV : kSoftmaxBwdTeamMaxV;
+    const int64_t per_wg = (int64_t)kTeamBlock * max_v;
+    const int64_t team_min = (packs + per_wg - 1) / per_wg;
+    int64_t teams = team_min <= cus ? cus / team_min : 0;
+    if (teams > M) teams = M;
+    if (teams >= 1) {
+      int64_t team_max = cus / teams;
+      const int64_t strides = (packs + kTeamBlock - 1) / kTeamBlock;
+      if (team_max > strides) team_max = strides;
+      const int64_t v = (strides + team_max - 1) / team_max;
+      const int64_t team = (strides + v - 1) / v;
+      if (team >= 2) {
+        p.team = (int)team;
+        p.team_v = (int)v;
+        p.team_chunk_packs = v * kTeamBlock;
+        p.team_grid = teams * team;
+      }
     }
   }
   if (oc == OC_SOFTMAX_BWD && !p.resident && p.fast && ov.G == 0 &&

@@ -29,6 +29,7 @@
 #include "device/pack.hpp"
 #include "device/flat_rows.hpp"
 #include "device/reduce.hpp"
+#include "device/team.hpp"
 #include "launch.hpp"
 #include <type_traits>
 
@@ -463,6 +464,192 @@ softmax_fwd_stream_kernel(const TI* __restrict__ x, TO* __restrict__ y, MaskRef 
   }
 }
 
+// ---------------------------------------------------------------------------
+// Forward for few, very long rows of whole packs (fewer rows than half the compute units;
+// 16-byte aligned X and Y, no mask): a row is held in the registers of a team of
+// workgroups, as in the norm forward for rows beyond the registers (norm_fwd_team_kernel).
+// The grid is at most two workgroups of 512 threads a compute unit, all resident at once;
+// workgroup b belongs to team b / team and keeps chunk b % team of the team's current
+// row, V packs a lane.  It finds its chunk's maximum m_c and s_c = sum exp(x - m_c),
+// publishes the pair and waits (bounded) for its team's pairs (device/team.hpp); each
+// workgroup then merges them in chunk order -- M = max m_c, S = sum s_c * exp(m_c - M),
+// the same values in every workgroup, run to run -- and writes its chunk of the output
+// out of its registers.  X is read once, and the whole machine works on a handful of
+// rows, where one workgroup a row (the reference's layout for such rows,
+// SoftMaxKernels.cpp:546-684, and softmax_fwd_stream_kernel here) leaves most compute
+// units idle.  A workgroup whose wait runs out takes the whole row's maximum and sum
+// itself (a second pass over X, which no workgroup writes: Y must not overlap X), loads
+// its chunk again and goes on; every wave reaches the end of the kernel whatever the
+// other workgroups do.
+template <class TI, class TO, int V>
+__global__ void __launch_bounds__(kTeamBlock, kTeamPerCu * kTeamBlock / 256)
+softmax_fwd_team_kernel(const TI* __restrict__ x, TO* __restrict__ y, int64_t M, int N, int flags,
+                        int team, int64_t chunk_packs, TeamSlot* slot, unsigned int call_id,
+                        unsigned long long wait_ticks) {
+  constexpr int E = elems_per_pack<TI>::value;
+  constexpr int BLOCK = kTeamBlock;
+  constexpr bool PRECISE = sizeof(TO) == 4;
+  __shared__ float red[reduce_lds_floats<BLOCK, BLOCK, 1>::value];
+  __shared__ double tpart[kTeamMaxWorkgroups][2];
+  __shared__ float stat[4];  // the row's maximum, 1 / sum or log(sum), -, whether the team failed
+  int phase = 0;
+  const bool is_log = (flags & kSoftmaxLog) != 0;
+  const bool is_safe = (flags & kSoftmaxSafe) != 0;
+  const int tm = (int)blockIdx.x / team;
+  const int c = (int)blockIdx.x - tm * team;
+  const int teams = (int)gridDim.x / team;
+  const int npacks = N / E;
+  const int64_t p0 = (int64_t)c * chunk_packs;
+  const int64_t p1 = p0 + chunk_packs < npacks ? p0 + chunk_packs : npacks;
+  const int nloc = p1 > p0 ? (int)(p1 - p0) : 0;  // packs of this chunk
+  const bool full = nloc == V * BLOCK;  // (uniform) all chunks but a row's last
+  const int64_t pbase = nloc > 0 ? p0 : 0;
+  const uint32_t loff = (uint32_t)(threadIdx.x * 16);
+  const uint32_t ooff = (uint32_t)(threadIdx.x * E * sizeof(TO));
+  // (the sum is formed as a pointer into global memory: a pointer made from an integer
+  // is otherwise a generic one, and generic accesses wait for everything outstanding)
+  auto at = [](auto* p, uint32_t off) {
+    using Elem = std::remove_pointer_t<decltype(p)>;
+    typedef __attribute__((address_space(1))) Elem* GlobalPtr;
+    return (Elem*)reinterpret_cast<GlobalPtr>(reinterpret_cast<uintptr_t>(p) + off);
+  };
+  unsigned int round = 0;
+  for (int64_t row = tm; row < M; row += teams, ++round) {
+    TeamEntry* entries = slot->entry[round & 1u];
+    if (threadIdx.x == 0) team_store(&entries[blockIdx.x].tag, 0ull);
+    const TI* xr = x + row * (int64_t)N;
+    const TI* xb = xr + pbase * E;
+    Pack<TI, E> xp[V];
+    auto load_chunk = [&]() {
+      if (full) {
+        // (straight-line code: V requests in flight a lane, nothing conditional)
+#pragma unroll
+        for (int k = 0; k < V; ++k) xp[k] = Pack<TI, E>::load_stream(at(xb + k * BLOCK * E, loff));
+      } else {
+#pragma unroll
+        for (int k = 0; k < V; ++k) {
+          xp[k] = Pack<TI, E>::splat(-INFINITY);
+          if (k * BLOCK + (int)threadIdx.x < nloc)
+            xp[k] = Pack<TI, E>::load_stream(at(xb + k * BLOCK * E, loff));
+        }
+      }
+    };
+    load_chunk();
+    float pm = -INFINITY;
+#pragma unroll
+    for (int k = 0; k < V; ++k)
+#pragma unroll
+      for (int i = 0; i < E; ++i) pm = fmaxf(pm, xp[k].get(i));
+    // (the chunk stays in storage format across the reductions and the wait)
+#pragma unroll
+    for (int k = 0; k < V; ++k) keep_packed(xp[k]);
+    float mx[1] = {pm};
+    group_allreduce<BLOCK, BLOCK, 1, MaxOp>(mx, red, phase);
+    const float m_c = mx[0];
+    // (nothing finite in the chunk: against 0, -inf elements add 0 and NaN still poisons)
+    const float ref = m_c == -INFINITY ? 0.0f : m_c;
+    float acc = 0.0f;
+#pragma unroll
+    for (int k = 0; k < V; ++k)
+#pragma unroll
+      for (int i = 0; i < E; ++i) acc += row_exp<PRECISE>(xp[k].get(i) - ref);
+#pragma unroll
+    for (int k = 0; k < V; ++k) keep_packed(xp[k]);
+    float sm[1] = {acc};
+    group_allreduce<BLOCK, BLOCK, 1, SumOp>(sm, red, phase);
+    if (threadIdx.x < 64) {  // the first wavefront publishes, waits and merges
+      const int lane = (int)threadIdx.x;
+      const bool complete = team_publish_and_gather(slot, entries, tm, team, call_id, round,
+                                                    wait_ticks, (double)m_c, (double)sm[0], tpart);
+      // (the lanes of a wavefront see one another's LDS stores in program order)
+      if (complete) {
+        float mm = -INFINITY;
+        for (int j = lane; j < team; j += 64) mm = fmaxf(mm, (float)tpart[j][0]);
+        mm = wave_group_allreduce<64, MaxOp>(mm);
+        // a chunk with nothing finite adds 0; a row with nothing finite gives NaN, as
+        // exp(-inf - -inf) does in the three-pass form
+        float ss = 0.0f;
+        for (int j = lane; j < team; j += 64) {
+          const float mj = (float)tpart[j][0], sj = (float)tpart[j][1];
+          ss += sj == 0.0f ? (mm == -INFINITY ? NAN : 0.0f) : sj * row_exp<PRECISE>(mj - mm);
+        }
+        ss = wave_group_allreduce<64, SumOp>(ss);
+        if (lane == 0) {
+          stat[0] = mm;
+          stat[1] = is_log ? logf(ss) : 1.0f / ss;
+          stat[3] = 0.0f;
+        }
+      } else if (lane == 0) {
+        stat[3] = 1.0f;
+      }
+    }
+    __syncthreads();
+    if (stat[3] != 0.0f) {  // (uniform over the workgroup)
+      // The team did not come together: the running maximum and sum of the whole row, as
+      // softmax_fwd_stream_kernel takes them, then the chunk again, whose registers the pass
+      // over the row has used.
+      float m_t = -INFINITY, s_t = 0.0f;
+      for (int pk0 = threadIdx.x; pk0 < npacks; pk0 += kStreamUnroll * BLOCK) {
+        Pack<TI, E> pv[kStreamUnroll];
+#pragma unroll
+        for (int u = 0; u < kStreamUnroll; ++u) {
+          const int pk = pk0 + u * BLOCK;
+          pv[u] = Pack<TI, E>::splat(-INFINITY);
+          if (pk < npacks) pv[u] = Pack<TI, E>::load(xr + (int64_t)pk * E);
+        }
+#pragma unroll
+        for (int u = 0; u < kStreamUnroll; ++u) {
+          float q = -INFINITY;
+#pragma unroll
+          for (int i = 0; i < E; ++i) q = fmaxf(q, pv[u].get(i));
+          const float nm = fmaxf(m_t, q);
+          const float rf = nm == -INFINITY ? 0.0f : nm;
+          float a2 = s_t * row_exp<PRECISE>(m_t - rf);
+#pragma unroll
+          for (int i = 0; i < E; ++i) a2 += row_exp<PRECISE>(pv[u].get(i) - rf);
+          s_t = a2;
+          m_t = nm;
+        }
+      }
+      float wm[1] = {m_t};
+      group_allreduce<BLOCK, BLOCK, 1, MaxOp>(wm, red, phase);
+      float ws[1] = {s_t == 0.0f ? (wm[0] == -INFINITY ? NAN : 0.0f)
+                                 : s_t * row_exp<PRECISE>(m_t - wm[0])};
+      group_allreduce<BLOCK, BLOCK, 1, SumOp>(ws, red, phase);
+      if (threadIdx.x == 0) {
+        stat[0] = wm[0];
+        stat[1] = is_log ? logf(ws[0]) : 1.0f / ws[0];
+      }
+      __syncthreads();
+      load_chunk();
+    }
+    const float m = stat[0], kk = stat[1];
+    const bool zero_row = is_safe && m == -INFINITY;
+    TO* yb = y + row * (int64_t)N + pbase * E;
+#pragma unroll
+    for (int k = 0; k < V; ++k) {
+      if (full || k * BLOCK + (int)threadIdx.x < nloc) {
+        Pack<TO, E> o;
+        if (is_log) {
+          ROWNORM_UNIFORM_ARM("log_softmax");
+#pragma unroll
+          for (int i = 0; i < E; ++i) o.set(i, (xp[k].get(i) - m) - kk);
+        } else {
+          ROWNORM_UNIFORM_ARM("softmax");
+#pragma unroll
+          for (int i = 0; i < E; ++i) {
+            const float v = row_exp<PRECISE>(xp[k].get(i) - m) * kk;
+            o.set(i, zero_row ? 0.0f : v);
+          }
+        }
+        o.store_stream(at(yb + k * BLOCK * E, ooff));
+      }
+    }
+    // stat[] is rewritten for the next row only after every thread has passed the
+    // barriers of the next block reductions, i.e. after it has read this row's values
+  }
+}
+
 // Backward.  TG: dtype of grad and of y (the saved forward output); TO: dtype
 // of the input gradient.
 template <class TG, class TO, int G, int V, int BLOCK, bool FAST, bool MASKED>
@@ -879,6 +1066,167 @@ softmax_bwd_stream_kernel(const TG* __restrict__ grad, const TG* __restrict__ y,
         store_row_pack<TO, E, true>(outr, pk * E, nw, pk < npacks, o, h);
       }
     }
+  }
+}
+
+// ---------------------------------------------------------------------------
+// Backward for the rows softmax_fwd_team_kernel serves: a team of workgroups holds a row
+// of grad and y in registers (V packs a lane of each, up to 8), each workgroup publishes
+// its chunk's sum -- of y * grad, or of grad for log_softmax --, the team's sums are added
+// in chunk order, and each workgroup writes its chunk of the gradient out of its
+// registers.  grad and y are read once.  A workgroup whose wait runs out sums the whole
+// row itself (gi must not overlap grad or y) and loads its chunk again.
+template <class TG, class TO, int V>
+__global__ void __launch_bounds__(kTeamBlock, kTeamPerCu * kTeamBlock / 256)
+softmax_bwd_team_kernel(const TG* __restrict__ grad, const TG* __restrict__ y, TO* __restrict__ gi,
+                        int64_t M, int N, int flags, int team, int64_t chunk_packs, TeamSlot* slot,
+                        unsigned int call_id, unsigned long long wait_ticks) {
+  constexpr int E = elems_per_pack<TG>::value;
+  constexpr int BLOCK = kTeamBlock;
+  constexpr bool PRECISE = sizeof(TO) == 4 && sizeof(TG) == 4;
+  __shared__ float red[reduce_lds_floats<BLOCK, BLOCK, 1>::value];
+  __shared__ double tpart[kTeamMaxWorkgroups][2];
+  __shared__ float stat[4];  // the row's sum, -, -, whether the team failed
+  int phase = 0;
+  const bool is_log = (flags & kSoftmaxLog) != 0;
+  const int tm = (int)blockIdx.x / team;
+  const int c = (int)blockIdx.x - tm * team;
+  const int teams = (int)gridDim.x / team;
+  const int npacks = N / E;
+  const int64_t p0 = (int64_t)c * chunk_packs;
+  const int64_t p1 = p0 + chunk_packs < npacks ? p0 + chunk_packs : npacks;
+  const int nloc = p1 > p0 ? (int)(p1 - p0) : 0;  // packs of this chunk
+  const bool full = nloc == V * BLOCK;  // (uniform) all chunks but a row's last
+  const int64_t pbase = nloc > 0 ? p0 : 0;
+  const uint32_t loff = (uint32_t)(threadIdx.x * 16);
+  const uint32_t ooff = (uint32_t)(threadIdx.x * E * sizeof(TO));
+  // (a pointer into global memory, as in the forward)
+  auto at = [](auto* p, uint32_t off) {
+    using Elem = std::remove_pointer_t<decltype(p)>;
+    typedef __attribute__((address_space(1))) Elem* GlobalPtr;
+    return (Elem*)reinterpret_cast<GlobalPtr>(reinterpret_cast<uintptr_t>(p) + off);
+  };
+  unsigned int round = 0;
+  for (int64_t row = tm; row < M; row += teams, ++round) {
+    TeamEntry* entries = slot->entry[round & 1u];
+    if (threadIdx.x == 0) team_store(&entries[blockIdx.x].tag, 0ull);
+    const TG* gr = grad + row * (int64_t)N;
+    const TG* yr = y + row * (int64_t)N;
+    const TG* gb = gr + pbase * E;
+    const TG* yb = yr + pbase * E;
+    Pack<TG, E> gp[V], yp[V];
+    auto load_chunk = [&]() {
+      if (full) {
+        // (straight-line code: 2 V requests in flight a lane, nothing conditional)
+#pragma unroll
+        for (int k = 0; k < V; ++k) {
+          gp[k] = Pack<TG, E>::load_stream(at(gb + k * BLOCK * E, loff));
+          yp[k] = Pack<TG, E>::load_stream(at(yb + k * BLOCK * E, loff));
+        }
+      } else {
+#pragma unroll
+        for (int k = 0; k < V; ++k) {
+          gp[k] = Pack<TG, E>::zero();
+          yp[k] = Pack<TG, E>::zero();
+          if (k * BLOCK + (int)threadIdx.x < nloc) {
+            gp[k] = Pack<TG, E>::load_stream(at(gb + k * BLOCK * E, loff));
+            yp[k] = Pack<TG, E>::load_stream(at(yb + k * BLOCK * E, loff));
+          }
+        }
+      }
+    };
+    load_chunk();
+    float sum[1] = {0.0f};
+    if (is_log) {
+      ROWNORM_UNIFORM_ARM("log_softmax backward: sum of grad");
+#pragma unroll
+      for (int k = 0; k < V; ++k) {
+#pragma unroll
+        for (int i = 0; i < E; ++i) sum[0] += gp[k].get(i);
+        __builtin_amdgcn_sched_barrier(0);  // (one pack widened at a time: registers)
+      }
+    } else {
+      ROWNORM_UNIFORM_ARM("softmax backward: sum of y * grad");
+#pragma unroll
+      for (int k = 0; k < V; ++k) {
+#pragma unroll
+        for (int i = 0; i < E; ++i) sum[0] = fmaf(yp[k].get(i), gp[k].get(i), sum[0]);
+        __builtin_amdgcn_sched_barrier(0);
+      }
+    }
+    // (the chunk stays in storage format across the reduction and the wait)
+#pragma unroll
+    for (int k = 0; k < V; ++k) {
+      keep_packed(gp[k]);
+      keep_packed(yp[k]);
+    }
+    group_allreduce<BLOCK, BLOCK, 1, SumOp>(sum, red, phase);
+    if (threadIdx.x < 64) {  // the first wavefront publishes, waits and adds up
+      const int lane = (int)threadIdx.x;
+      const bool complete = team_publish_and_gather(slot, entries, tm, team, call_id, round,
+                                                    wait_ticks, (double)sum[0], 0.0, tpart);
+      // (the lanes of a wavefront see one another's LDS stores in program order)
+      if (complete) {
+        float ss = 0.0f;
+        for (int j = lane; j < team; j += 64) ss += (float)tpart[j][0];
+        ss = wave_group_allreduce<64, SumOp>(ss);
+        if (lane == 0) {
+          stat[0] = ss;
+          stat[3] = 0.0f;
+        }
+      } else if (lane == 0) {
+        stat[3] = 1.0f;
+      }
+    }
+    __syncthreads();
+    if (stat[3] != 0.0f) {  // (uniform over the workgroup)
+      // The team did not come together: the sum over the whole row, then the chunk again.
+      float ws[1] = {0.0f};
+      for (int pk0 = threadIdx.x; pk0 < npacks; pk0 += kStreamUnroll * BLOCK) {
+        Pack<TG, E> pg[kStreamUnroll], py[kStreamUnroll];
+#pragma unroll
+        for (int u = 0; u < kStreamUnroll; ++u) {
+          const int pk = pk0 + u * BLOCK;
+          pg[u] = Pack<TG, E>::zero();
+          py[u] = Pack<TG, E>::zero();
+          if (pk < npacks) {
+            pg[u] = Pack<TG, E>::load(gr + (int64_t)pk * E);
+            if (!is_log) py[u] = Pack<TG, E>::load(yr + (int64_t)pk * E);
+          }
+        }
+#pragma unroll
+        for (int u = 0; u < kStreamUnroll; ++u)
+#pragma unroll
+          for (int i = 0; i < E; ++i)
+            ws[0] = is_log ? ws[0] + pg[u].get(i) : fmaf(py[u].get(i), pg[u].get(i), ws[0]);
+      }
+      group_allreduce<BLOCK, BLOCK, 1, SumOp>(ws, red, phase);
+      if (threadIdx.x == 0) stat[0] = ws[0];
+      __syncthreads();
+      load_chunk();
+    }
+    const float s = stat[0];
+    TO* ob = gi + row * (int64_t)N + pbase * E;
+#pragma unroll
+    for (int k = 0; k < V; ++k) {
+      if (full || k * BLOCK + (int)threadIdx.x < nloc) {
+        Pack<TO, E> o;
+        if (is_log) {
+          ROWNORM_UNIFORM_ARM("log_softmax backward");
+#pragma unroll
+          for (int i = 0; i < E; ++i) o.set(i, gp[k].get(i) - row_exp<PRECISE>(yp[k].get(i)) * s);
+        } else {
+          ROWNORM_UNIFORM_ARM("softmax backward");
+#pragma unroll
+          for (int i = 0; i < E; ++i) o.set(i, yp[k].get(i) * (gp[k].get(i) - s));
+        }
+        o.store_stream(at(ob + k * BLOCK * E, ooff));
+      }
+      // (pack k + 1 is widened after pack k has been stored, not before: registers)
+      __builtin_amdgcn_sched_barrier(0);
+    }
+    // stat[] is rewritten for the next row only after every thread has passed the
+    // barrier of the next block reduction, i.e. after it has read this row's value
   }
 }
 

@@ -104,6 +104,29 @@ int launch_softmax_fwd_m(const Plan& plan, const SoftmaxFwdArgs& a, hipStream_t 
     const FlatLayout f = flat_layout<TI>(plan, a.M, a.N, a.x, a.y, nullptr);
     if (f.g && launch_softmax_fwd_flat<TI>(f, a, stream)) return (int)hipGetLastError();
   }
+  if constexpr (!MASKED) {
+    if (plan.team > 0 && a.team_slot != nullptr) {
+      // few very long rows: each in the registers of a team of workgroups
+      TeamSlot* slot = (TeamSlot*)a.team_slot;
+      auto go = [&](auto v) {
+        constexpr int V = decltype(v)::value;
+        hipLaunchKernelGGL((softmax_fwd_team_kernel<TI, TO, V>), dim3((unsigned)plan.team_grid),
+                           dim3(kTeamBlock), 0, stream, (const TI*)a.x, (TO*)a.y, a.M, a.N, a.flags,
+                           plan.team, plan.team_chunk_packs, slot, a.team_id, a.team_wait_ticks);
+      };
+      static_assert(kTeamMaxV == 16, "one case per pack count below");
+      switch (plan.team_v) {
+#define ROWNORM_TEAM_CASE(v) case v: go(std::integral_constant<int, v>{}); break;
+        ROWNORM_TEAM_CASE(1) ROWNORM_TEAM_CASE(2) ROWNORM_TEAM_CASE(3) ROWNORM_TEAM_CASE(4)
+        ROWNORM_TEAM_CASE(5) ROWNORM_TEAM_CASE(6) ROWNORM_TEAM_CASE(7) ROWNORM_TEAM_CASE(8)
+        ROWNORM_TEAM_CASE(9) ROWNORM_TEAM_CASE(10) ROWNORM_TEAM_CASE(11) ROWNORM_TEAM_CASE(12)
+        ROWNORM_TEAM_CASE(13) ROWNORM_TEAM_CASE(14) ROWNORM_TEAM_CASE(15) ROWNORM_TEAM_CASE(16)
+#undef ROWNORM_TEAM_CASE
+        default: return (int)hipErrorInvalidConfiguration;
+      }
+      return (int)hipGetLastError();
+    }
+  }
   if (plan.resident) {
     SoftmaxFwdCtx<TI, TO> ctx{plan, a, stream};
     const bool launched =
@@ -191,6 +214,28 @@ int launch_softmax_bwd_m(const Plan& plan, const SoftmaxBwdArgs& a, hipStream_t 
   if constexpr (!MASKED && std::is_same<TG, TO>::value) {
     const FlatLayout f = flat_layout<TG>(plan, a.M, a.N, a.grad, a.y, a.gi);
     if (f.g && launch_softmax_bwd_flat<TG>(f, a, stream)) return (int)hipGetLastError();
+  }
+  if constexpr (!MASKED) {
+    if (plan.team > 0 && a.team_slot != nullptr) {
+      // few very long rows: each in the registers of a team of workgroups
+      TeamSlot* slot = (TeamSlot*)a.team_slot;
+      auto go = [&](auto v) {
+        constexpr int V = decltype(v)::value;
+        hipLaunchKernelGGL((softmax_bwd_team_kernel<TG, TO, V>), dim3((unsigned)plan.team_grid),
+                           dim3(kTeamBlock), 0, stream, (const TG*)a.grad, (const TG*)a.y,
+                           (TO*)a.gi, a.M, a.N, a.flags, plan.team, plan.team_chunk_packs, slot,
+                           a.team_id, a.team_wait_ticks);
+      };
+      static_assert(kSoftmaxBwdTeamMaxV == 8, "one case per pack count below");
+      switch (plan.team_v) {
+#define ROWNORM_TEAM_CASE(v) case v: go(std::integral_constant<int, v>{}); break;
+        ROWNORM_TEAM_CASE(1) ROWNORM_TEAM_CASE(2) ROWNORM_TEAM_CASE(3) ROWNORM_TEAM_CASE(4)
+        ROWNORM_TEAM_CASE(5) ROWNORM_TEAM_CASE(6) ROWNORM_TEAM_CASE(7) ROWNORM_TEAM_CASE(8)
+#undef ROWNORM_TEAM_CASE
+        default: return (int)hipErrorInvalidConfiguration;
+      }
+      return (int)hipGetLastError();
+    }
   }
   if (plan.resident) {
     SoftmaxBwdCtx<TG, TO> ctx{plan, a, stream};
