@@ -725,7 +725,9 @@ def model_shapes_table(torch, cabi, L, dev, stream, P, only=None):
     for name, M, N, lg in (("ViT-B/16 attention _softmax bf16 [64x12x197, 197]", 64 * 12 * 197, 197, 0),
                            ("ViT-L/14@336 attention _softmax bf16 [16x16x577, 577]", 16 * 16 * 577, 577, 0),
                            ("CLIP text attention _softmax bf16 [1024x8x77, 77]", 1024 * 8 * 77, 77, 0),
-                           ("_log_softmax bf16 [4096, 151936] (Qwen vocabulary)", 4096, 151936, 1)):
+                           ("_log_softmax bf16 [4096, 151936] (Qwen vocabulary)", 4096, 151936, 1),
+                           ("_softmax bf16 [64, 151936] (a decode batch over the vocabulary)", 64, 151936, 0),
+                           ("_softmax bf16 [32, 1048576] (few very long rows)", 32, 1048576, 0)):
         if only is not None and not any(t in name + " fwd" or t in name + " bwd" for t in only.split("|")):
             continue
         sets = []

@@ -15,8 +15,10 @@ pytestmark = pytest.mark.gpu
 
 # (N, C, HxW, groups): 64 slabs of 131072 elements (2 workgroups a slab); 32 slabs of 262144 with a
 # ragged last chunk; 9 slabs of 81920 + 8 (a slab that is one pack longer than 20 strides);
-# 16 slabs of 1 M elements (16 workgroups a slab)
-SHAPES = [(2, 256, 16384, 32), (4, 64, 32776, 8), (3, 6, 40964 * 8 // 2, 3), (1, 128, 131072, 16)]
+# 16 slabs of 1 M elements (16 workgroups a slab); 2 slabs of 4 M elements (fewer slabs than the
+# 8 teams a launch otherwise asks for: all at once, 256 workgroups a slab)
+SHAPES = [(2, 256, 16384, 32), (4, 64, 32776, 8), (3, 6, 40964 * 8 // 2, 3), (1, 128, 131072, 16),
+          (2, 8, 524288, 1)]
 
 
 def _with_wait(cabi, us, fn):

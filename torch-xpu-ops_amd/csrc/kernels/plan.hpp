@@ -917,7 +917,9 @@ inline int make_plan(OpClass oc, int64_t M, int64_t N, int esize, int num_cus, c
     // whose second pass comes out of the memory-side cache, [2, 1310720] 13.2 against
     // 11.6 us; 8 teams ([8, 4194304], one round) 35.1 against 40.5 us, 64 teams
     // ([512, 401408], 8 rounds) 177 against 196 us.
-    if (teams >= kTeamMinTeams) {
+    // (GroupNorm slabs have no split-row kernels to fall back on: with fewer slabs than 8
+    // teams, all at once, the alternative is one workgroup a slab)
+    if (teams >= kTeamMinTeams || (oc == OC_GROUP_FWD && teams >= 1 && teams == M)) {
       // a chunk is a whole number of workgroup strides, exactly the packs a lane the
       // kernel is compiled for: every workgroup but a row's last runs straight-line code
       int64_t team_max = cus / teams;
