@@ -220,7 +220,11 @@ int mi355x_rms_norm_bwd_static(const void* dy, const void* x, const float* rstd,
  * tensor.  Replaces _softmax_kernel / _log_softmax_kernel (SoftMaxKernels.h:19-29)
  * for the inner_size == 1 case (SoftMaxKernels.cpp:1663-1720).  out_dtype is
  * in_dtype, or ROWNORM_F32 with a ROWNORM_F16 input (half_to_float,
- * SoftMaxKernels.cpp:2131-2135). */
+ * SoftMaxKernels.cpp:2131-2135).  Few, very long rows (fewer rows than half the
+ * compute units, 4096 16-byte packs a row or more, 16-byte aligned x and y that do
+ * not overlap) are each held by a team of workgroups, under the rules described at
+ * mi355x_rownorm_set_team_wait_us; mi355x_softmax_bwd likewise (gi apart from grad
+ * and y). */
 int mi355x_softmax_fwd(const void* x, void* y, int64_t rows, int64_t N, rownorm_dtype in_dtype,
                        rownorm_dtype out_dtype, int is_log, void* stream);
 
@@ -383,11 +387,13 @@ int mi355x_rownorm_plan_at(rownorm_op op, int64_t M, int64_t N, rownorm_dtype x_
 int mi355x_rownorm_set_override(rownorm_op op, int lanes_per_row, int packs_per_lane,
                                 int block_threads, int blocks_per_cu);
 
-/* Test hook for the forward of rows that a team of workgroups holds in registers
- * (LayerNorm / RMSNorm rows beyond 131072 16-bit or 65536 float32 elements, whole
- * 16-byte packs, no residual add, no cast, y not overlapping x): how long a
- * workgroup waits for the others of its team before it sums the whole row itself
- * (a second pass over x, the same result to rounding), in microseconds; 0xffffffff
+/* Test hook for the rows that a team of workgroups holds in registers (LayerNorm /
+ * RMSNorm forward rows beyond 131072 16-bit or 65536 float32 elements, whole
+ * 16-byte packs, no residual add, no cast, y not overlapping x; GroupNorm forward
+ * slabs of that size; softmax / log_softmax forward and backward of few, very long
+ * rows): how long a workgroup waits for the others of its team before it sums the
+ * whole row itself (a second pass over the inputs, the same result to rounding), in
+ * microseconds; 0xffffffff
  * restores the default, one second.  0 makes every wait give up at once, which is
  * how the tests exercise that path without making any kernel hang.  Process-global.
  * Such calls draw an id and one of 16 bookkeeping slots in library-owned device

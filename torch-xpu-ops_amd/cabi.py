@@ -177,8 +177,9 @@ def group_norm_plan(backward, N, C, HxW, groups, dtype=F32):
 
 
 def set_team_wait_us(microseconds=0xffffffff):
-    """Bound of a workgroup's wait in the team forward (rows beyond one workgroup's registers);
-    0: every wait gives up at once and each workgroup sums its rows itself."""
+    """Bound of a workgroup's wait in the team kernels (norm forward rows beyond one workgroup's
+    registers, softmax forward / backward of few very long rows); 0: every wait gives up at once
+    and each workgroup sums its rows itself."""
     _check(lib().mi355x_rownorm_set_team_wait_us(ctypes.c_uint(microseconds)), "set_team_wait_us")
 
 
