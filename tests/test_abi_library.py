@@ -137,7 +137,16 @@ def test_plan_invariants(cabi, op, dt):
         for M in (1, 3, 1000, 1 << 20):
             p = cabi.plan(op, M, N, dt, dt)
             assert p["grid_blocks"] >= 1
-            if p["resident"]:
+            if op in (cabi.OP_SOFTMAX_FWD, cabi.OP_SOFTMAX_BWD) and p["row_chunks"] > 0:
+                # few, very long softmax rows of whole packs: a team of `row_chunks` workgroups
+                # of 512 threads holds a row (16 packs a lane at most, the backward 8 of each
+                # tensor), no more teams than rows
+                team = p["row_chunks"]
+                assert N % E == 0 and N // E >= 4096 and 2 * M <= 256, (M, N, p)
+                assert team >= 2 and p["grid_blocks"] % team == 0 and p["grid_blocks"] <= 512
+                assert 1 <= p["grid_blocks"] // team <= M
+                assert team * 512 * (16 if op == cabi.OP_SOFTMAX_FWD else 8) * E >= N
+            elif p["resident"]:
                 G, V = p["lanes_per_row"], p["packs_per_lane"]
                 # a power of two, or (exact two-pack layouts of the 16-bit norm backward) a
                 # whole number of wavefronts
