@@ -167,3 +167,39 @@ def test_microbench_shape_of_the_reference(cabi, oracle, gpu):
         assert_close(y, to_np32(fy), torch.bfloat16, "y, team against fallback")
         del fy
         torch.cuda.empty_cache()
+
+
+@pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16], ids=str)
+def test_few_rows_that_one_workgroup_would_hold(cabi, oracle, gpu, dtype):
+    """Rows of exactly 16384 packs (16 a lane on 1024 lanes: the longest one workgroup holds), too
+    few of them for the compute units: the teams take them as well; with one row more than half
+    the compute units the register-resident kernel keeps them."""
+    E = 4 if dtype == torch.float32 else 8
+    N = 16384 * E
+    code = cabi.dtype_code(dtype)
+    for M in (100, 128):
+        p = cabi.plan(cabi.OP_LAYER_NORM_FWD, M, N, code, code)
+        assert p["row_chunks"] >= 2 and p["grid_blocks"] % p["row_chunks"] == 0, p
+        assert p["grid_blocks"] // p["row_chunks"] == M and p["grid_blocks"] <= 512, p
+    p = cabi.plan(cabi.OP_LAYER_NORM_FWD, 129, N, code, code)
+    assert p["resident"] == 1 and p["grid_blocks"] <= 129, p
+    M = 100
+    x, gamma, beta = _mk(M, N, dtype, dtype, 1680)
+    x[7] = 1.25
+    xg, gg, bg = x.to(gpu), gamma.to(gpu), beta.to(gpu)
+    y, mean, rstd = cabi.layer_norm_fwd(xg, gg, bg, 1e-5)
+    oy, om, orr = oracle.layer_norm_fwd(to_np32(x), (N,), to_np32(gamma), to_np32(beta), 1e-5)
+    assert_close(y, oy, dtype, "layer_norm y")
+    assert_close(mean, om.reshape(-1), torch.float32, "mean")
+    assert_close(rstd, orr.reshape(-1), torch.float32, "rstd")
+    assert torch.equal(y[7].cpu(), beta), "a constant row gives beta bit for bit"
+    fy, fm, fr = _with_wait(cabi, 0, lambda: cabi.layer_norm_fwd(xg, gg, bg, 1e-5))
+    assert_close(fy, oy, dtype, "fallback y")
+    assert_close(rstd, to_np32(fr), torch.float32, "rstd, team against fallback")
+    ry, rr = cabi.rms_norm_fwd(xg, gg, 1e-6)
+    roy, ror = oracle.rms_norm_fwd(to_np32(x), (N,), to_np32(gamma), 1e-6)
+    assert_close(ry, roy, dtype, "rms_norm y")
+    assert_close(rr, ror.reshape(-1), torch.float32, "rms rstd")
+    xc = xg.clone()
+    yi, _, ri = cabi.layer_norm_fwd(xc, gg, bg, 1e-5, y=xc)  # in place: the resident kernel
+    assert_close(yi, oy, dtype, "in place y")

@@ -114,21 +114,7 @@ int launch_norm_fwd(const Plan& plan, const NormFwdArgs& a, hipStream_t stream) 
         return (int)hipGetLastError();
     }
   }
-  if (plan.resident && plan.exact_depth > 0) {
-    static_assert(kNormFwdExactCount == 2, "one call per table entry below");
-    bool launched = false;
-    if constexpr (!ADD && std::is_same<T, TY>::value)
-      launched = launch_norm_fwd_exact_at<T, WT, RMS, 0>(plan, a, stream) ||
-                 launch_norm_fwd_exact_at<T, WT, RMS, 1>(plan, a, stream);
-    if (!launched) return (int)hipErrorInvalidConfiguration;
-  } else if (plan.resident) {
-    NormFwdCtx<T, WT, RMS> ctx{plan, a, stream};
-    const bool launched =
-        plan.fast
-            ? launch_variant<NormFwdLauncher<T, WT, RMS, true, TY, ADD>::template At>(ctx)
-            : launch_variant<NormFwdLauncher<T, WT, RMS, false, TY, ADD>::template At>(ctx);
-    if (!launched) return (int)hipErrorInvalidConfiguration;
-  } else if (norm_fwd_team_serves<T, TY, ADD>(plan, a)) {
+  if (norm_fwd_team_serves<T, TY, ADD>(plan, a)) {
     // one pass with the row in the registers of a team of workgroups
     TeamSlot* slot = (TeamSlot*)a.team_slot;
     auto go = [&](auto v) {
@@ -148,6 +134,20 @@ int launch_norm_fwd(const Plan& plan, const NormFwdArgs& a, hipStream_t stream) 
 #undef ROWNORM_TEAM_CASE
       default: return (int)hipErrorInvalidConfiguration;
     }
+  } else if (plan.resident && plan.exact_depth > 0) {
+    static_assert(kNormFwdExactCount == 2, "one call per table entry below");
+    bool launched = false;
+    if constexpr (!ADD && std::is_same<T, TY>::value)
+      launched = launch_norm_fwd_exact_at<T, WT, RMS, 0>(plan, a, stream) ||
+                 launch_norm_fwd_exact_at<T, WT, RMS, 1>(plan, a, stream);
+    if (!launched) return (int)hipErrorInvalidConfiguration;
+  } else if (plan.resident) {
+    NormFwdCtx<T, WT, RMS> ctx{plan, a, stream};
+    const bool launched =
+        plan.fast
+            ? launch_variant<NormFwdLauncher<T, WT, RMS, true, TY, ADD>::template At>(ctx)
+            : launch_variant<NormFwdLauncher<T, WT, RMS, false, TY, ADD>::template At>(ctx);
+    if (!launched) return (int)hipErrorInvalidConfiguration;
   } else if (norm_fwd_can_split<T, TY, RMS>(plan, a)) {
     const dim3 grid((unsigned)plan.split, (unsigned)a.M);
     hipLaunchKernelGGL((norm_fwd_split_sums_kernel<T, kStreamBlock, RMS, TY>), grid,

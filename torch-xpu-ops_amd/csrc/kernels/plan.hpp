@@ -904,8 +904,14 @@ inline int make_plan(OpClass oc, int64_t M, int64_t N, int esize, int num_cus, c
   // all the workgroups its team can have (down to one stride of 1024 packs each).
   // (GroupNorm forward slabs likewise; the caller takes the team only where the channels
   // are whole packs)
-  if ((oc == OC_NORM_FWD || oc == OC_GROUP_FWD) && !p.resident && p.fast && !fused_add &&
-      ov.G == 0 && ov.V == 0 && ov.bpc == 0) {
+  // (also rows that one workgroup still holds, 16 packs a lane on 1024 lanes, when there are
+  // too few of them for the compute units: bf16 [128, 131072] LayerNorm 17.4 -> 13.8 us, fp32
+  // [128, 65536] 19.2 -> 13.3 us; from 8192 packs down the resident kernel is as fast or faster,
+  // its 4-6 us against the team's 6-8)
+  const bool few_rows = oc == OC_NORM_FWD && p.resident && 2 * M <= num_cus &&
+                        packs >= (int64_t)kMaxG * kMaxV;
+  if ((oc == OC_NORM_FWD || oc == OC_GROUP_FWD) && (!p.resident || few_rows) && p.fast && !fused_add &&
+      ov.G == 0 && ov.V == 0 && ov.bpc == 0 && ov.block == 0) {
     const int64_t cus = num_cus * kTeamPerCu < kTeamMaxWorkgroups ? num_cus * kTeamPerCu : kTeamMaxWorkgroups;
     const int64_t per_wg = (int64_t)kTeamBlock * kTeamMaxV;
     const int64_t team_min = (packs + per_wg - 1) / per_wg;
@@ -919,7 +925,7 @@ inline int make_plan(OpClass oc, int64_t M, int64_t N, int esize, int num_cus, c
     // ([512, 401408], 8 rounds) 177 against 196 us.
     // (GroupNorm slabs have no split-row kernels to fall back on: with fewer slabs than 8
     // teams, all at once, the alternative is one workgroup a slab)
-    if (teams >= kTeamMinTeams || (oc == OC_GROUP_FWD && teams >= 1 && teams == M)) {
+    if (teams >= kTeamMinTeams || ((oc == OC_GROUP_FWD || few_rows) && teams >= 1 && teams == M)) {
       // a chunk is a whole number of workgroup strides, exactly the packs a lane the
       // kernel is compiled for: every workgroup but a row's last runs straight-line code
       int64_t team_max = cus / teams;
