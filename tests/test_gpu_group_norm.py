@@ -41,7 +41,10 @@ SHAPES = [(2, 4, (), 2), (64, 32, (), 4), (256, 32, (), 4), (64, 32, (16,), 4), 
           # 16-bit rows that fill an exact layout, channels of whole runs of 64 packs (32x32 and
           # 64x64 maps with 10, 20, 30 and 60 channels a group; 10 at 64x64 is above): 256 x 5
           # (backward), 512 x 5, 768 x 5, 960 x 8
-          (3, 10, (32, 32), 1), (2, 40, (32, 32), 2), (2, 60, (32, 32), 2), (2, 120, (32, 32), 2)]
+          (3, 10, (32, 32), 1), (2, 40, (32, 32), 2), (2, 60, (32, 32), 2), (2, 120, (32, 32), 2),
+          # from 8192 samples under few channels the backward's second stage first folds its
+          # partial rows (one a sample) in place, 512 at a time: 16 folds and a ragged 17th
+          (8269, 24, (), 4), (8200, 16, (3,), 2)]
 CASES = load_golden("aten_cpu_group_norm.npz")
 
 

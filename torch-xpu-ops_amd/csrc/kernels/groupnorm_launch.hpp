@@ -189,6 +189,10 @@ inline bool launch_group_bwd_exact(const Plan& plan, const GroupNormBwdArgs& a, 
   return (launch_group_bwd_exact_at<T, WT, Is>(plan, a, stream) || ...);
 }
 
+// Partial rows (one a sample) the second stage of the backward folds in place at a time, where
+// there are very many samples.
+constexpr int kGnFoldRows = 512;
+
 template <class T, class WT>
 int launch_group_norm_bwd(const Plan& plan, const GroupNormBwdArgs& a, hipStream_t stream) {
   constexpr int E = elems_per_pack<T>::value;
@@ -256,6 +260,19 @@ int launch_group_norm_bwd(const Plan& plan, const GroupNormBwdArgs& a, hipStream
   err = (int)hipGetLastError();
   if (err != 0 || !want_cols) return err;
   const unsigned gx = (unsigned)((C + kFinalizeCols - 1) / kFinalizeCols);
+  // one partial row a sample: with very many samples under few channels the rows are first
+  // folded in place, kGnFoldRows at a time, by as many workgroups as that gives (bf16
+  // [1048576, 32] in 8 groups: the second stage alone took 4 ms on its one workgroup)
+  if (N >= 16 * kGnFoldRows && N <= 65535 * (int64_t)kGnFoldRows && gx <= 32) {
+    const unsigned folds = (unsigned)((N + kGnFoldRows - 1) / kGnFoldRows);
+    hipLaunchKernelGGL((colsum_finalize_kernel<float, true>), dim3(gx, 2, folds), dim3(1024), 0,
+                       stream, (const float*)a.part_dg, (const float*)a.part_db, (float*)nullptr,
+                       (float*)nullptr, (int)N, C, (int64_t)C, kGnFoldRows);
+    hipLaunchKernelGGL((colsum_finalize_kernel<WT>), dim3(gx, 2), dim3(1024), 0, stream,
+                       (const float*)a.part_dg, (const float*)a.part_db, (WT*)a.dgamma,
+                       (WT*)a.dbeta, (int)folds, C, (int64_t)kGnFoldRows * C, 0);
+    return (int)hipGetLastError();
+  }
   hipLaunchKernelGGL((colsum_finalize_kernel<WT>), dim3(gx, 2), dim3(1024), 0, stream,
                      (const float*)a.part_dg, (const float*)a.part_db, (WT*)a.dgamma,
                      (WT*)a.dbeta, (int)N, C);

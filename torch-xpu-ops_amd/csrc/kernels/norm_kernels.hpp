@@ -2276,14 +2276,29 @@ norm_bwd_stream_colsum_kernel(const T* __restrict__ dy, const T* __restrict__ x,
 // buffers in the reference (LayerNormKernels.cpp:1312-1314).
 constexpr int kFinalizeCols = 64;
 
-template <class WT>
+//
+// Very many partial rows under few columns (a GroupNorm over [N, C] with N in the hundreds of
+// thousands: one partial row a sample, C / 64 workgroups) first FOLD: blockIdx.z takes the
+// partial rows [z * fold_rows, (z + 1) * fold_rows) and leaves their fp32 sum in the first
+// of them, in place (a workgroup reads and writes only its own columns of its own rows);
+// the second launch then adds every fold_rows-th row (`row_stride` = fold_rows * N).
+template <class WT, bool FOLD = false>
 __global__ void __launch_bounds__(1024)
-colsum_finalize_kernel(const float* __restrict__ part0, const float* __restrict__ part1,
-                       WT* __restrict__ out0, WT* __restrict__ out1, int P, int N) {
+colsum_finalize_kernel(const float* part0, const float* part1, WT* __restrict__ out0,
+                       WT* __restrict__ out1, int P, int N, int64_t row_stride = 0,
+                       int fold_rows = 0) {
   constexpr int CQ = kFinalizeCols / 4, RL = 1024 / CQ;
   __shared__ float tile[RL][kFinalizeCols + 1];
   const float* part = blockIdx.y == 0 ? part0 : part1;
   WT* out = blockIdx.y == 0 ? out0 : out1;
+  if (row_stride == 0) row_stride = N;
+  if constexpr (FOLD) {
+    if (part == nullptr) return;
+    const int first = (int)blockIdx.z * fold_rows;
+    part += (int64_t)first * row_stride;
+    out = const_cast<WT*>(reinterpret_cast<const WT*>(part));  // (WT is float here)
+    P = P - first < fold_rows ? P - first : fold_rows;
+  }
   if (part == nullptr || out == nullptr) return;  // uniform per workgroup
   const int cq = threadIdx.x % CQ, rl = threadIdx.x / CQ;
   const int col0 = blockIdx.x * kFinalizeCols + cq * 4;
@@ -2296,8 +2311,8 @@ colsum_finalize_kernel(const float* __restrict__ part0, const float* __restrict_
 #pragma unroll
     for (int u = 0; u < U; ++u) {
       const int p = p0 + u * RL;
-      v[u] = load_row_pack<float, 4, false>(part + (int64_t)(p < P ? p : 0) * N, col0, N, p < P,
-                                            0.0f);
+      v[u] = load_row_pack<float, 4, false>(part + (int64_t)(p < P ? p : 0) * row_stride, col0, N,
+                                            p < P, 0.0f);
     }
 #pragma unroll
     for (int u = 0; u < U; ++u)
