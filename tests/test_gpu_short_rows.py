@@ -97,3 +97,53 @@ def test_short_softmax_rows_match_the_oracle(cabi, oracle, gpu, dtype, offset):
                 y32 = cabi.softmax_fwd(xg, is_log, y=place(torch.empty(M, N)))
                 assert_close(y32, oracle.softmax_fwd(to_np32(x), is_log), torch.float32,
                              "softmax float16 -> float32 N=%d log=%d" % (N, is_log))
+
+
+@pytest.mark.parametrize("dtype", DTYPES, ids=str)
+def test_rows_of_one_to_four_packs_over_many_rows(cabi, oracle, gpu, dtype):
+    """Rows of 16 to 64 bytes (one, two or four whole packs) in tensors on a 16-byte boundary are
+    staged through LDS on one, two or four lanes a row: more rows than one launch of workgroups
+    holds at a time (each walks several pieces), a ragged last piece, the forward in place, dX
+    alone and the column sums alone, twice the same bits."""
+    E = 16 // torch.empty(0, dtype=dtype).element_size()
+    for packs in (1, 2, 3, 4):
+        N = packs * E
+        for M in (5, 300007):
+            print("case rows of few packs", dtype, (M, N), flush=True)
+            g = gen(990 + packs)
+            x = (0.5 + torch.randn(M, N, generator=g)).to(dtype)
+            x[M // 2] = -2.5  # a constant row
+            dy = torch.randn(M, N, generator=g).to(dtype)
+            gamma = (1 + 0.1 * torch.randn(N, generator=g)).to(dtype)
+            beta = (0.1 * torch.randn(N, generator=g)).to(dtype)
+            xg, dyg, gg, bg = x.to(gpu), dy.to(gpu), gamma.to(gpu), beta.to(gpu)
+            what = "[%d, %d] %s" % (M, N, dtype)
+            y, mean, rstd = cabi.layer_norm_fwd(xg, gg, bg, 1e-5)
+            oy, om, orr = oracle.layer_norm_fwd(to_np32(x), (N,), to_np32(gamma), to_np32(beta), 1e-5)
+            assert_close(y, oy, dtype, "layer_norm y " + what)
+            assert_close(mean, om.reshape(-1), torch.float32, "mean " + what)
+            assert_close(rstd, orr.reshape(-1), torch.float32, "rstd " + what)
+            assert torch.equal(y[M // 2].cpu(), beta), "a constant row gives beta " + what
+            xc = xg.clone()
+            yi, mi, ri = cabi.layer_norm_fwd(xc, gg, bg, 1e-5, y=xc)
+            assert torch.equal(yi, y) and torch.equal(mi, mean) and torch.equal(ri, rstd)
+            ry, rr = cabi.rms_norm_fwd(xg, gg, 1e-6)
+            roy, ror = oracle.rms_norm_fwd(to_np32(x), (N,), to_np32(gamma), 1e-6)
+            assert_close(ry, roy, dtype, "rms_norm y " + what)
+            assert_close(rr, ror.reshape(-1), torch.float32, "rms rstd " + what)
+            dx, dg, db = cabi.layer_norm_bwd(dyg, xg, mean, rstd, gg)
+            odx, odg, odb = oracle.layer_norm_bwd(to_np32(dy), to_np32(x), (N,), to_np32(mean),
+                                                  to_np32(rstd), to_np32(gamma))
+            xhat = (x.float() - mean.cpu().reshape(M, 1)) * rstd.cpu().reshape(M, 1)
+            assert_close(dx, odx, dtype, "layer_norm dx " + what)
+            assert_close(dg, odg, dtype, "dgamma " + what, slack=colsum_slack(dy.float() * xhat))
+            assert_close(db, odb, dtype, "dbeta " + what, slack=colsum_slack(dy.float()))
+            dx1, n1, n2 = cabi.layer_norm_bwd(dyg, xg, mean, rstd, gg, want=(True, False, False))
+            assert n1 is None and n2 is None and torch.equal(dx1, dx), "dX alone " + what
+            n0, dg1, db1 = cabi.layer_norm_bwd(dyg, xg, mean, rstd, gg, want=(False, True, True))
+            assert n0 is None and torch.equal(dg1, dg) and torch.equal(db1, db), "sums alone " + what
+            rdx, rdg = cabi.rms_norm_bwd(dyg, xg, rr, gg)
+            rodx, rodg = oracle.rms_norm_bwd(to_np32(dy), to_np32(x), (N,), to_np32(rr), to_np32(gamma))
+            assert_close(rdx, rodx, dtype, "rms_norm dx " + what)
+            assert_close(rdg, rodg, dtype, "rms dgamma " + what,
+                         slack=colsum_slack(dy.float() * x.float() * rr.cpu().reshape(M, 1)))

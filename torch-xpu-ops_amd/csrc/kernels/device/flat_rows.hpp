@@ -35,7 +35,7 @@ constexpr int kFlatBlock = 256;
 // backward 36.2 -> 32.9 us ([147712, 577] backward, which needs the 16 KB:
 // 101 -> 94 us); 1024 threads were 50 % slower.
 constexpr int kFlatLdsBytes = 64 * kFlatBlock;
-// Lanes per row G (4..64) and packs per lane VP (1..kFlatMaxPacks) are chosen so
+// Lanes per row G (1..64) and packs per lane VP (1..kFlatMaxPacks) are chosen so
 // that G * VP leaves as few pack slots idle as possible (flat_layout below).
 constexpr int kFlatMaxPacks = 4;
 // Rows a workgroup takes at a time: as many as its LDS holds, a multiple of 8
@@ -150,7 +150,7 @@ struct FlatLayout {
   int vp = 0;  // packs per lane
 };
 
-// The (lanes 4..64, packs per lane 1..4) with the fewest idle pack slots; among
+// The (lanes 1..64, packs per lane 1..4) with the fewest idle pack slots; among
 // equals the one nearest two packs a lane, the layout the resident kernels prefer.
 // Measured against "two packs a lane on the fewest lanes that hold the row",
 // interleaved, bf16 forward / backward in us: rows of 13: 19.5 / 18.5 -> 10.6 / 8.6,
@@ -168,9 +168,12 @@ inline FlatLayout flat_layout(const Plan& plan, int64_t M, int N, const void* p0
   // rows of whole packs qualify only when they are very short (see below)
   if (plan.fast && (packs > kFlatWholePackRowsMaxPacks || !plan.resident)) return f;
   int best_slots = 0, best_rank = 0;
-  for (int g = 4; g <= 64; g <<= 1) {
+  for (int g = 1; g <= 64; g <<= 1) {
     const int vp = (packs + g - 1) / g;
     if (vp > kFlatMaxPacks) continue;
+    // (one or two lanes a row: rows of 1, 2 and 4 packs, which fill them exactly; 3 packs on
+    // 2 x 2 measured 5-10 % behind 4 x 1 in the forward)
+    if (g < 4 && (vp > 2 || g * vp != packs)) continue;
     const int slots = g * vp;
     const int rank = vp == 2 ? 0 : (vp == 3 ? 1 : (vp == 1 ? 2 : 3));
     if (f.g == 0 || slots < best_slots || (slots == best_slots && rank < best_rank)) {
@@ -191,8 +194,10 @@ inline FlatLayout flat_layout(const Plan& plan, int64_t M, int N, const void* p0
 
 // One case per (lanes, packs per lane) of a launch switch keyed by lanes * 8 + packs.
 #define ROWNORM_FLAT_CASES(CASE, GL) CASE(GL, 1) CASE(GL, 2) CASE(GL, 3) CASE(GL, 4)
+#define ROWNORM_FLAT_CASES_NARROW(CASE, GL) CASE(GL, 1) CASE(GL, 2)
 #define ROWNORM_FLAT_ALL(CASE)                                                       \
-  ROWNORM_FLAT_CASES(CASE, 4) ROWNORM_FLAT_CASES(CASE, 8) ROWNORM_FLAT_CASES(CASE, 16) \
-  ROWNORM_FLAT_CASES(CASE, 32) ROWNORM_FLAT_CASES(CASE, 64)
+  ROWNORM_FLAT_CASES_NARROW(CASE, 1) ROWNORM_FLAT_CASES_NARROW(CASE, 2) ROWNORM_FLAT_CASES(CASE, 4) \
+  ROWNORM_FLAT_CASES(CASE, 8) ROWNORM_FLAT_CASES(CASE, 16) ROWNORM_FLAT_CASES(CASE, 32) \
+  ROWNORM_FLAT_CASES(CASE, 64)
 
 }  // namespace rownorm

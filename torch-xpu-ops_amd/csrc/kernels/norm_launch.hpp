@@ -108,7 +108,7 @@ int launch_norm_fwd(const Plan& plan, const NormFwdArgs& a, hipStream_t stream) 
   T* h = ADD ? (T*)a.h : nullptr;
   // short ragged rows (no residual add, no cast, 16-byte aligned X and Y): staged through LDS
   if constexpr (!ADD && std::is_same<T, TY>::value) {
-    if (plan.resident && !plan.fast && plan.exact_depth == 0 && !plan.window) {
+    if (plan.resident && plan.exact_depth == 0 && !plan.window) {
       const FlatLayout f = flat_layout<T>(plan, a.M, a.N, a.x, a.y, nullptr);
       if (f.g != 0 && launch_norm_fwd_flat<T, WT, RMS>(f, a, stream))
         return (int)hipGetLastError();
@@ -233,7 +233,13 @@ inline bool launch_norm_bwd_exact(const Plan& plan, const NormBwdArgs& a, hipStr
 // 15.2, 63 47.2 / 41.4 -> 27.7 / 27.1, 127 78.9 / 74.1 -> 45.3 / 44.0, 257 96.2 / 90.9 -> 94.9 /
 // 92.4, 1001 329 / 323 -> 312 / 306.  More workgroups than the plan's partial rows (3, 4 or 8 a
 // compute unit instead of 2) measured slower at most lengths.
+// Rows of whole packs (which the resident kernel addresses without conditions) only up to 64
+// bytes, 32 in fp32: bf16 N = 8 80 -> 32 us, 16 45 -> 30, 32 31 -> 29 but 72 30 -> 40, 96 28 -> 34;
+// fp32 N = 4 116 -> 53, 8 66 -> 54 but 16 44 -> 54 (2097152 / 1048576 / ... rows, LayerNorm).
 constexpr bool norm_bwd_flat_serves(size_t esize, int lanes) { return esize == 4 || lanes <= 8; }
+constexpr bool norm_bwd_flat_serves_whole_packs(size_t esize, int N) {
+  return (size_t)N * esize <= (esize == 4 ? 32u : 64u);
+}
 template <class T, class WT, bool RMS, int LDSB>
 bool launch_norm_bwd_flat_l(const Plan& plan, FlatLayout f, int cr, const NormBwdArgs& a,
                             hipStream_t stream, int* rows_out) {
@@ -280,9 +286,10 @@ int launch_norm_bwd(const Plan& plan, const NormBwdArgs& a, hipStream_t stream) 
   bool flat = false;
   // short ragged rows (no residual gradient, 16-byte aligned dY, X and dX): staged through LDS
   if constexpr (!ADD) {
-    if (plan.resident && !plan.fast && plan.exact_depth == 0 && !plan.window) {
+    if (plan.resident && plan.exact_depth == 0 && !plan.window) {
       const FlatLayout f = flat_layout<T>(plan, a.M, a.N, a.dy, a.x, a.dx);
       flat = f.g != 0 && norm_bwd_flat_serves(sizeof(T), f.g) &&
+             (!plan.fast || norm_bwd_flat_serves_whole_packs(sizeof(T), a.N)) &&
              launch_norm_bwd_flat<T, WT, RMS>(plan, f, a, stream, &partial_rows);
     }
   }
