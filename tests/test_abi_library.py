@@ -164,6 +164,20 @@ def test_plan_invariants(cabi, op, dt):
                 assert p["rows_per_block"] == 1 and team >= 1 and p["grid_blocks"] % team == 0
                 assert p["grid_blocks"] <= 512 and 8 <= p["grid_blocks"] // team <= M
                 assert team * 512 * 16 * E >= N
+            elif (op in (cabi.OP_LAYER_NORM_BWD, cabi.OP_RMS_NORM_BWD) and N % E == 0 and
+                  p["row_chunks"] >= 2 and p["block_threads"] == 512 and p["packs_per_lane"] == 2):
+                # backward rows of whole packs beyond one workgroup's registers: a team of
+                # `row_chunks` workgroups holds four rows at a time, two strides of 512 packs a
+                # workgroup, one workgroup a compute unit, no more teams than groups of four
+                # rows, one partial row a team
+                team = p["row_chunks"]
+                assert team == (N // E + 1023) // 1024 and p["grid_blocks"] <= 256
+                assert p["grid_blocks"] % team == 0 and 1 <= p["grid_blocks"] // team <= (M + 3) // 4
+                assert p["partial_rows"] >= p["grid_blocks"] // team
+                # from 8 (RMSNorm: 5) rounds on, and no row whose last workgroup is mostly idle
+                rounds = ((M + 3) // 4) // (p["grid_blocks"] // team)
+                assert rounds >= (8 if op == cabi.OP_LAYER_NORM_BWD else 5)
+                assert 5 * (N // E) >= 4 * team * 1024
             else:
                 assert p["rows_per_block"] == 1 and p["grid_blocks"] <= M
             if op in (cabi.OP_LAYER_NORM_BWD, cabi.OP_RMS_NORM_BWD):

@@ -293,6 +293,13 @@ int norm_fwd(const void* x, const void* res, const void* gamma, const void* beta
 // [M, 2] row totals behind them; rows that stay on one workgroup but not in its
 // registers keep their [M, 2] row sums there when the column sums are wanted as
 // well (dX and the column sums then share one pass over X and dY).  0: neither.
+// Partial rows of column sums a backward call may leave: those of the launch the plan names
+// and, where teams of workgroups may hold the rows instead, one a team.
+size_t bwd_partial_rows(const Plan& plan) {
+  return (size_t)(plan.partial_rows > plan.team_partial_rows ? plan.partial_rows
+                                                             : plan.team_partial_rows);
+}
+
 size_t split_bytes(const Plan& plan, int64_t M, bool want_cols) {
   if (plan.resident) return 0;
   if (plan.split > 1) return (size_t)M * ((size_t)plan.split + 1) * 2 * sizeof(float);
@@ -313,7 +320,7 @@ size_t norm_bwd_workspace(int op, int64_t M, int64_t N, int xd, int wd, int npar
                   &plan, false, op == ROWNORM_OP_LAYER_NORM_BWD, esize_of(wd) > esize_of(xd),
                   false, fused_add, false, want_dx))
       return 0;
-    const size_t need = (size_t)plan.partial_rows * (size_t)N * sizeof(float) * (size_t)nparts +
+    const size_t need = bwd_partial_rows(plan) * (size_t)N * sizeof(float) * (size_t)nparts +
                         split_bytes(plan, M, nparts > 0);
     if (need > most) most = need;
   }
@@ -343,7 +350,7 @@ int norm_bwd(const void* dy, const void* x, const float* mean, const float* rstd
   float* part_db = nullptr;
   size_t need = 0;
   if (want_cols) {
-    const size_t one = (size_t)plan.partial_rows * (size_t)N * sizeof(float);
+    const size_t one = bwd_partial_rows(plan) * (size_t)N * sizeof(float);
     need = one * (RMS ? 1 : 2);
     if (!workspace || workspace_bytes < need) return ROWNORM_ERR_WORKSPACE;
     part_dg = (float*)workspace;
@@ -356,6 +363,19 @@ int norm_bwd(const void* dy, const void* x, const float* mean, const float* rstd
       workspace_bytes >= need + split_bytes(plan, M, want_cols))
     a.split_ws = (float*)((char*)workspace + need);
   hipStream_t s = (hipStream_t)stream;
+  // rows beyond the registers: the team backward (whole packs on 16-byte aligned tensors, dX
+  // apart from dY and X -- a workgroup whose team does not come together reads whole rows of
+  // both while others write theirs)
+  if (plan.team > 0 && dx && !dres &&
+      ((((uintptr_t)dy) | ((uintptr_t)x) | ((uintptr_t)dx) | ((uintptr_t)gamma) |
+        ((uintptr_t)workspace)) & 15u) == 0) {
+    const size_t nbytes = (size_t)M * (size_t)N * (size_t)esize_of(xd);
+    const char *db = (const char*)dx, *gb = (const char*)dy, *xb = (const char*)x;
+    if (!(db < gb + nbytes && gb < db + nbytes) && !(db < xb + nbytes && xb < db + nbytes)) {
+      a.team_slot = team_slot_for_call(s, &a.team_id);
+      a.team_wait_ticks = g_team_wait_ticks.load(std::memory_order_relaxed);
+    }
+  }
   if (dres != nullptr && dx != nullptr) {
     a.dres = dres;
     if (xd == ROWNORM_F32) return launch_norm_bwd<float, float, RMS, true>(plan, a, s);
@@ -891,7 +911,13 @@ int mi355x_rownorm_plan_at(rownorm_op op, int64_t M, int64_t N, rownorm_dtype x_
   // (a forward row held by a team of workgroups: the team and its grid)
   out->reserved = plan.team > 0 ? plan.team : (plan.split > 1 ? plan.split : 0);
   out->grid_blocks = plan.team > 0 ? plan.team_grid : plan.grid;
-  out->partial_rows = plan.partial_rows;
+  out->partial_rows = (int64_t)bwd_partial_rows(plan);
+  // (backward rows held by teams: the workgroup, and the packs of a row a lane holds)
+  if (plan.team > 0 && (op == ROWNORM_OP_LAYER_NORM_BWD || op == ROWNORM_OP_RMS_NORM_BWD)) {
+    out->lanes_per_row = kTeamBlock;
+    out->block_threads = kTeamBlock;
+    out->packs_per_lane = plan.team_v;
+  }
   return 0;
 }
 

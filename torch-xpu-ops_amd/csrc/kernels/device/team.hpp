@@ -27,6 +27,7 @@
 #include <stdint.h>
 
 #include "../plan.hpp"
+#include "reduce.hpp"
 
 namespace rownorm {
 
@@ -77,6 +78,83 @@ __device__ __forceinline__ bool team_publish_and_gather(TeamSlot* slot, TeamEntr
         ok = ok && team_load(&mates[j].tag) == expect;
       }
       if (__ballot(ok) == __ballot(true)) {
+        complete = true;
+        break;
+      }
+    }
+    // (the hint word is one address for the whole grid: looked at every 16th time)
+    if ((polls++ & 15u) == 0) {
+      const unsigned int hint =
+          __hip_atomic_load(&slot->gave_up, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+      if (hint == call_id) break;
+    }
+    if (wall_clock64() - t0 > wait_ticks) break;
+    __builtin_amdgcn_s_sleep(8);
+  }
+  if (lane == 0 && !complete)
+    __hip_atomic_store(&slot->gave_up, call_id, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+  return complete;
+}
+
+// The two halves of such an exchange with K 64-bit words a workgroup (K <= 15: an entry's s1,
+// s2 and the words behind them), for kernels that put other work between them.  Word k holds
+// the float32 values v[2k] and v[2k + 1].
+//
+// team_publish_words: for lane 0 of a wavefront whose entry `mine` has had the tag 0 since
+// the workgroup started on the round.
+template <int K>
+__device__ __forceinline__ void team_publish_words(TeamEntry* mine, unsigned int call_id,
+                                                   unsigned int round, const float (&v)[2 * K]) {
+  static_assert(K >= 1 && K <= 15, "an entry holds a tag and 15 words");
+  unsigned long long* words = &mine->s1;
+  team_stores_done();  // the tag has been 0 in memory before the numbers change
+#pragma unroll
+  for (int k = 0; k < K; ++k) {
+    const unsigned long long lo = __builtin_bit_cast(unsigned int, v[2 * k]);
+    const unsigned long long hi = __builtin_bit_cast(unsigned int, v[2 * k + 1]);
+    team_store(&words[k], lo | (hi << 32));
+  }
+  team_stores_done();
+  team_store(&mine->tag, ((unsigned long long)call_id << 32) | (round + 1u));
+}
+
+// team_gather_sums: for the first wavefront of a workgroup (all 64 lanes); waits for the
+// `team` entries from `mates` on to carry the round's tag and leaves in v[] the sums of their
+// values over the team, added in a fixed order (entries lane, lane + 64, ... per lane, then
+// across the lanes): the same bits in every lane and in every workgroup of the team.  False
+// as in team_publish_and_gather (v[] is then not meaningful).
+template <int K>
+__device__ __forceinline__ bool team_gather_sums(TeamSlot* slot, const TeamEntry* mates, int team,
+                                                 unsigned int call_id, unsigned int round,
+                                                 unsigned long long wait_ticks,
+                                                 float (&v)[2 * K]) {
+  const int lane = (int)threadIdx.x;
+  const unsigned long long expect = ((unsigned long long)call_id << 32) | (round + 1u);
+  const unsigned long long t0 = wall_clock64();
+  bool complete = false;
+  unsigned int polls = 0;
+  for (;;) {
+    bool ok = true;
+    for (int j = lane; j < team; j += 64) ok = ok && team_load(&mates[j].tag) == expect;
+    if (__ballot(ok) == __ballot(true)) {
+#pragma unroll
+      for (int k = 0; k < 2 * K; ++k) v[k] = 0.0f;
+      for (int j = lane; j < team; j += 64) {
+        const unsigned long long* words = &mates[j].s1;
+        unsigned long long w[K];
+#pragma unroll
+        for (int k = 0; k < K; ++k) w[k] = team_load(&words[k]);
+        team_stores_done();  // the numbers have returned before the tag is read again
+        ok = ok && team_load(&mates[j].tag) == expect;
+#pragma unroll
+        for (int k = 0; k < K; ++k) {
+          v[2 * k] += __builtin_bit_cast(float, (unsigned int)(w[k] & 0xffffffffull));
+          v[2 * k + 1] += __builtin_bit_cast(float, (unsigned int)(w[k] >> 32));
+        }
+      }
+      if (__ballot(ok) == __ballot(true)) {
+#pragma unroll
+        for (int k = 0; k < 2 * K; ++k) v[k] = wave_group_allreduce<64, SumOp>(v[k]);
         complete = true;
         break;
       }

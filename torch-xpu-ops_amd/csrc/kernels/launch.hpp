@@ -46,6 +46,12 @@ struct NormBwdArgs {
   int N;
   float* split_ws = nullptr;  // [M, plan.split + 1, 2] fp32 for the split-row path, or null: not split
   const void* dres = nullptr;  // gradient reaching the normalized row by the residual path, added to dx
+  // norm_bwd_team_kernel (rows beyond the registers held by teams of workgroups): the call's
+  // slot of bookkeeping memory, its id and the bound of a wait, as in NormFwdArgs; null = not
+  // for this call.  part_dg / part_db then hold plan.team_partial_rows rows.
+  void* team_slot = nullptr;
+  unsigned int team_id = 0;
+  unsigned long long team_wait_ticks = 0;
 };
 
 constexpr int kSoftmaxLog = 1;   // log_softmax instead of softmax

@@ -2363,4 +2363,250 @@ colsum_finalize_flat_kernel(const float* __restrict__ part0, const float* __rest
     if (col0 + i < N) out[col0 + i] = (WT)a[i];
 }
 
+// ---------------------------------------------------------------------------
+// Backward of rows beyond one workgroup's registers, dY and X read once: a team of workgroups
+// holds R rows at a time, workgroup c of the team the packs [c * V * BLOCK, (c + 1) * V * BLOCK)
+// of each -- V packs of dY and of X a lane and row, so a lane meets the same V * E columns in
+// every row and its column sums (dgamma, dbeta) are 2 * V * E numbers however long the row is
+// (kept in LDS).  The R rows' partial s1 = sum dy*gamma, s2 = sum dy*gamma*xhat cross the team
+// in one exchange (team_publish_and_sum), every workgroup writes dX for what it holds, and the
+// next R rows the team takes have been requested before the exchange began: two sets of R
+// rows a lane, one being exchanged and written while the other arrives.  Team tm takes the
+// row groups tm, tm + teams, ...; at the end each workgroup leaves its column sums in row
+// tm of the [teams, N] partial buffers (the second stage adds them).  A workgroup whose wait
+// runs out sums its R rows itself (dX must not overlap dY or X) and loads its packs again.
+// One workgroup a compute unit: the two sets of rows take about 200 registers a lane.
+template <class T, class WT, bool RMS, int R, int V>
+__global__ void __launch_bounds__(kTeamBlock, kTeamBlock / 256)
+norm_bwd_team_kernel(const T* __restrict__ dy, const T* __restrict__ x,
+                     const float* __restrict__ mean, const float* __restrict__ rstd,
+                     const WT* __restrict__ gamma, T* __restrict__ dx,
+                     float* __restrict__ part_dg, float* __restrict__ part_db, int64_t M, int N,
+                     int team, TeamSlot* slot, unsigned int call_id,
+                     unsigned long long wait_ticks) {
+  constexpr int E = elems_per_pack<T>::value;
+  constexpr int BLOCK = kTeamBlock;
+  constexpr int Q = E / 4;  // pieces of four floats in a pack's column sums
+  __shared__ float red[reduce_lds_floats<BLOCK, BLOCK, 2 * R>::value];
+  __shared__ float stat[2 * R + 1];  // the rows' s1, s2; whether the team failed
+  // a lane's column sums, four floats a piece: piece q of pack k at colsum[(k * Q + q)][lane]
+  // for dgamma, behind them the same for dbeta
+  __shared__ Pack<float, 4> colsum[(RMS ? 1 : 2) * V * Q][BLOCK];
+  int phase = 0;
+  const int tm = (int)blockIdx.x / team;
+  const int c = (int)blockIdx.x - tm * team;
+  const int teams = (int)gridDim.x / team;
+  const int npacks = N / E;
+  // pack k of the lane: pk0 + k * BLOCK of the row, held only if it lies in the row
+  const int pk0 = c * (V * BLOCK) + (int)threadIdx.x;
+  const int64_t ngroups = (M + R - 1) / R;
+  const float fN = (float)N;
+  Pack<WT, E> pg[V];
+#pragma unroll
+  for (int k = 0; k < V; ++k) {
+    pg[k] = Pack<WT, E>::splat(1.0f);
+    if (gamma != nullptr && pk0 + k * BLOCK < npacks)
+      pg[k] = Pack<WT, E>::load(gamma + (int64_t)(pk0 + k * BLOCK) * E);
+  }
+#pragma unroll
+  for (int q = 0; q < (RMS ? 1 : 2) * V * Q; ++q) colsum[q][threadIdx.x] = Pack<float, 4>::zero();
+
+  // (a scalar pointer a row and one 32-bit byte offset a lane, formed as a pointer into
+  // global memory: see norm_fwd_team_kernel)
+  const uint32_t loff = (uint32_t)(pk0 < npacks ? pk0 : 0) * 16u;
+  auto at = [](auto* p, uint32_t off) {
+    using Elem = std::remove_pointer_t<decltype(p)>;
+    typedef __attribute__((address_space(1))) Elem* GlobalPtr;
+    return (Elem*)reinterpret_cast<GlobalPtr>(reinterpret_cast<uintptr_t>(p) + off);
+  };
+  // the lane's packs of the rows of group g (zeros beyond the tensor and beyond the row)
+  auto load_group = [&](int64_t g, Pack<T, E> (&pd)[R * V], Pack<T, E> (&px)[R * V]) {
+#pragma unroll
+    for (int r = 0; r < R; ++r) {
+      const int64_t row = g * R + r;
+#pragma unroll
+      for (int k = 0; k < V; ++k) {
+        pd[r * V + k] = Pack<T, E>::zero();
+        px[r * V + k] = Pack<T, E>::zero();
+        if (pk0 + k * BLOCK < npacks && row < M) {
+          pd[r * V + k] = Pack<T, E>::load_stream(at(dy + row * (int64_t)N + k * BLOCK * E, loff));
+          px[r * V + k] = Pack<T, E>::load_stream(at(x + row * (int64_t)N + k * BLOCK * E, loff));
+        }
+      }
+    }
+  };
+  // The partial sums of the rows of group g (held in pd / px), published as round `round`.
+  auto sums_and_publish = [&](int64_t g, unsigned int round, Pack<T, E> (&pd)[R * V],
+                              Pack<T, E> (&px)[R * V]) {
+    TeamEntry* mine = &slot->entry[round & 3u][blockIdx.x];
+    if (threadIdx.x == 0) team_store(&mine->tag, 0ull);
+    float acc[2 * R];
+#pragma unroll
+    for (int r = 0; r < R; ++r) acc[2 * r] = acc[2 * r + 1] = 0.0f;
+#pragma unroll
+    for (int k = 0; k < V; ++k) {
+#pragma unroll
+      for (int r = 0; r < R; ++r) {
+        const int64_t row = g * R + r < M ? g * R + r : M - 1;
+        const float mu = RMS ? 0.0f : uniform_load<float>(mean + row);
+        const float rs = uniform_load<float>(rstd + row);
+#pragma unroll
+        for (int i = 0; i < E; ++i) {
+          const float gd = pd[r * V + k].get(i) * pg[k].get(i);
+          acc[2 * r] += gd;
+          acc[2 * r + 1] = fmaf(gd, (px[r * V + k].get(i) - mu) * rs, acc[2 * r + 1]);
+        }
+        keep_packed(pd[r * V + k]);
+        keep_packed(px[r * V + k]);
+        __builtin_amdgcn_sched_barrier(0);  // (one pack widened at a time: registers)
+      }
+    }
+    group_allreduce<BLOCK, BLOCK, 2 * R, SumOp>(acc, red, phase);
+    if (threadIdx.x == 0) team_publish_words<R>(mine, call_id, round, acc);
+  };
+  // The sums of group g (published as round `round`) across the team, its dX, its share of
+  // the column sums; each pack's registers are given to the same pack of group gn (< 0:
+  // none) as soon as its dX has been stored.  (go, po*: the group held in the other register
+  // set, loaded again after the rare pass over whole rows so that nothing stays live
+  // across that pass)
+  auto finish = [&](int64_t g, unsigned int round, Pack<T, E> (&pd)[R * V], Pack<T, E> (&px)[R * V],
+                    int64_t gn, int64_t go, Pack<T, E> (&pod)[R * V], Pack<T, E> (&pox)[R * V]) {
+    // (every thread has read the stat[] of the round before: a team's last rounds have no
+    // block reduction between two of these)
+    __syncthreads();
+    if (threadIdx.x < 64) {  // the first wavefront waits and adds up
+      float tot[2 * R];
+      const bool complete =
+          team_gather_sums<R>(slot, slot->entry[round & 3u] + tm * team, team, call_id, round,
+                              wait_ticks, tot);
+      if (threadIdx.x == 0) {
+#pragma unroll
+        for (int k = 0; k < 2 * R; ++k) stat[k] = tot[k];
+        stat[2 * R] = complete ? 0.0f : 1.0f;
+      }
+    }
+    __syncthreads();
+    if (stat[2 * R] != 0.0f) {  // (uniform over the workgroup)
+      // The team did not come together: the sums over the whole rows, then the packs again.
+      // (one pack of each tensor a lane in flight: laid out for few registers, not for speed)
+      for (int r = 0; r < R; ++r) {
+        const int64_t row = g * R + r < M ? g * R + r : M - 1;
+        const T* xr = x + row * (int64_t)N;
+        const T* gr = dy + row * (int64_t)N;
+        const float wmu = RMS ? 0.0f : mean[row], wrs = rstd[row];
+        float ws[2] = {0.0f, 0.0f};
+        for (int q = (int)threadIdx.x; q < npacks; q += BLOCK) {
+          const Pack<T, E> qx = Pack<T, E>::load(xr + (int64_t)q * E);
+          const Pack<T, E> qd = Pack<T, E>::load(gr + (int64_t)q * E);
+          const Pack<WT, E> qg =
+              gamma != nullptr ? Pack<WT, E>::load(gamma + (int64_t)q * E) : Pack<WT, E>::splat(1.0f);
+#pragma unroll
+          for (int i = 0; i < E; ++i) {
+            const float gd = qd.get(i) * qg.get(i);
+            ws[0] += gd;
+            ws[1] = fmaf(gd, (qx.get(i) - wmu) * wrs, ws[1]);
+          }
+        }
+        group_allreduce<BLOCK, BLOCK, 2, SumOp>(ws, red, phase);
+        __syncthreads();  // (every thread has read stat[] before thread 0 rewrites it)
+        if (threadIdx.x == 0) {
+          stat[2 * r] = ws[0];
+          stat[2 * r + 1] = ws[1];
+        }
+      }
+      __syncthreads();
+      load_group(g, pd, px);
+      load_group(go >= 0 ? go : M, pod, pox);  // (a group beyond the tensor: zeros)
+    }
+#pragma unroll
+    for (int k = 0; k < V; ++k) {
+      const bool held = pk0 + k * BLOCK < npacks;
+      // (the pack's column sums stay in registers over its R rows)
+      Pack<float, 4> cg[Q], cb[Q];
+#pragma unroll
+      for (int q = 0; q < Q; ++q) {
+        cg[q] = colsum[k * Q + q][threadIdx.x];
+        if constexpr (!RMS) cb[q] = colsum[V * Q + k * Q + q][threadIdx.x];
+      }
+#pragma unroll
+      for (int r = 0; r < R; ++r) {
+        const int64_t row = g * R + r;
+        const int64_t rowc = row < M ? row : M - 1;
+        const float mu = RMS ? 0.0f : uniform_load<float>(mean + rowc);
+        const float rs = uniform_load<float>(rstd + rowc);
+        const float s1 = stat[2 * r], s2 = stat[2 * r + 1];
+        const float term1 = rs / fN;
+        Pack<T, E> o;
+#pragma unroll
+        for (int i = 0; i < E; ++i) {
+          const float d = pd[r * V + k].get(i);
+          const float xh = (px[r * V + k].get(i) - mu) * rs;
+          float f = fN * (d * pg[k].get(i));
+          f -= xh * s2;
+          if constexpr (!RMS) f -= s1;
+          o.set(i, f * term1);
+          cg[i / 4].v[i % 4] = fmaf(d, xh, cg[i / 4].v[i % 4]);
+          if constexpr (!RMS) cb[i / 4].v[i % 4] += d;
+        }
+        if (held && row < M)
+          o.store_stream(at(dx + row * (int64_t)N + k * BLOCK * E, loff));
+        // the registers go to the same pack of group gn
+        if (gn >= 0) {
+          const int64_t rown = gn * R + r;
+          pd[r * V + k] = Pack<T, E>::zero();
+          px[r * V + k] = Pack<T, E>::zero();
+          if (held && rown < M) {
+            pd[r * V + k] = Pack<T, E>::load_stream(at(dy + rown * (int64_t)N + k * BLOCK * E, loff));
+            px[r * V + k] = Pack<T, E>::load_stream(at(x + rown * (int64_t)N + k * BLOCK * E, loff));
+          }
+        }
+        // (the next pack is widened after this one has been stored, not before: registers)
+        __builtin_amdgcn_sched_barrier(0);
+      }
+#pragma unroll
+      for (int q = 0; q < Q; ++q) {
+        colsum[k * Q + q][threadIdx.x] = cg[q];
+        if constexpr (!RMS) colsum[V * Q + k * Q + q][threadIdx.x] = cb[q];
+      }
+    }
+  };
+
+  // Group j of the team (tm + j * teams) lives in register set j % 2: requested while group
+  // j - 2 is written, summed and published one round before it is gathered and written, so
+  // that neither the loads nor the exchange are waited for with nothing else to do.
+  Pack<T, E> ad[R * V], ax[R * V], bd[R * V], bx[R * V];
+  int64_t g = tm;
+  unsigned int round = 0;
+  if (g < ngroups) {
+    load_group(g, ad, ax);
+    if (g + teams < ngroups) load_group(g + teams, bd, bx);
+    sums_and_publish(g, 0, ad, ax);
+  }
+  while (g < ngroups) {
+    const int64_t g1 = g + teams, g2 = g + 2 * (int64_t)teams, g3 = g + 3 * (int64_t)teams;
+    if (g1 < ngroups) sums_and_publish(g1, round + 1, bd, bx);
+    finish(g, round, ad, ax, g2 < ngroups ? g2 : -1, g1 < ngroups ? g1 : -1, bd, bx);
+    if (g1 >= ngroups) break;
+    if (g2 < ngroups) sums_and_publish(g2, round + 2, ad, ax);
+    finish(g1, round + 1, bd, bx, g3 < ngroups ? g3 : -1, g2 < ngroups ? g2 : -1, ad, ax);
+    g = g2;
+    round += 2;
+  }
+  if (part_dg != nullptr) {
+#pragma unroll
+    for (int k = 0; k < V; ++k) {
+      if (pk0 + k * BLOCK >= npacks) continue;
+      const int64_t e0 = (int64_t)(pk0 + k * BLOCK) * E;
+      float* pgr = part_dg + (int64_t)tm * N + e0;
+#pragma unroll
+      for (int q = 0; q < Q; ++q) colsum[k * Q + q][threadIdx.x].store(pgr + 4 * q);
+      if constexpr (!RMS) {
+        float* pbr = part_db + (int64_t)tm * N + e0;
+#pragma unroll
+        for (int q = 0; q < Q; ++q) colsum[V * Q + k * Q + q][threadIdx.x].store(pbr + 4 * q);
+      }
+    }
+  }
+}
+
 }  // namespace rownorm

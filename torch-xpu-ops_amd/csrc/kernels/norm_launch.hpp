@@ -282,7 +282,8 @@ int launch_norm_bwd(const Plan& plan, const NormBwdArgs& a, hipStream_t stream) 
   const T* dres = ADD ? (const T*)a.dres : nullptr;
   int partial_rows = (int)plan.partial_rows;
   // one partial row (few, very long rows): the column-sum kernels write dgamma / dbeta themselves
-  const bool direct = want_cols && !plan.resident && plan.partial_rows == 1;
+  const bool team_call = !ADD && !plan.resident && plan.team > 0 && a.team_slot != nullptr && a.dx != nullptr;
+  const bool direct = want_cols && !plan.resident && plan.partial_rows == 1 && !team_call;
   bool flat = false;
   // short ragged rows (no residual gradient, 16-byte aligned dY, X and dX): staged through LDS
   if constexpr (!ADD) {
@@ -306,6 +307,13 @@ int launch_norm_bwd(const Plan& plan, const NormBwdArgs& a, hipStream_t stream) 
         plan.fast ? launch_variant<NormBwdLauncher<T, WT, RMS, true, ADD>::template At>(ctx)
                   : launch_variant<NormBwdLauncher<T, WT, RMS, false, ADD>::template At>(ctx);
     if (!launched) return (int)hipErrorInvalidConfiguration;
+  } else if (team_call) {
+    // rows beyond the registers, dY and X read once: teams of workgroups, one partial row each
+    hipLaunchKernelGGL((norm_bwd_team_kernel<T, WT, RMS, kTeamBwdRows, kTeamBwdPacks>), dim3((unsigned)plan.team_grid),
+                       dim3(kTeamBlock), 0, stream, (const T*)a.dy, (const T*)a.x, a.mean, a.rstd,
+                       (const WT*)a.gamma, (T*)a.dx, a.part_dg, a.part_db, a.M, a.N, plan.team,
+                       (TeamSlot*)a.team_slot, a.team_id, a.team_wait_ticks);
+    partial_rows = (int)(plan.team_grid / plan.team);
   } else {
     constexpr int E = elems_per_pack<T>::value;
     bool cols_done = false;
@@ -357,11 +365,11 @@ int launch_norm_bwd(const Plan& plan, const NormBwdArgs& a, hipStream_t stream) 
   }
   int err = (int)hipGetLastError();
   if (err != 0 || !want_cols || direct) return err;
-  if (!plan.resident && plan.partial_rows <= kFinalizeFlatRows) {
+  if (!plan.resident && partial_rows <= kFinalizeFlatRows) {
     const unsigned gx = (unsigned)((a.N + kFinalizeFlatCols - 1) / kFinalizeFlatCols);
     hipLaunchKernelGGL((colsum_finalize_flat_kernel<WT>), dim3(gx, RMS ? 1 : 2), dim3(256), 0,
                        stream, (const float*)a.part_dg, (const float*)a.part_db, (WT*)a.dgamma,
-                       (WT*)a.dbeta, (int)plan.partial_rows, a.N);
+                       (WT*)a.dbeta, partial_rows, a.N);
     return (int)hipGetLastError();
   }
   const unsigned gx = (unsigned)((a.N + kFinalizeCols - 1) / kFinalizeCols);

@@ -37,7 +37,9 @@ enum OpClass {
 
 struct Override {
   // 0 = automatic; G = -1 = force the streaming kernel, and then V = 1 keeps every
-  // row on one workgroup, V > 1 splits every row over V workgroups (norm ops)
+  // row on one workgroup, V > 1 splits every row over V workgroups (norm ops), V = 0 with
+  // block = 1 sends a norm backward of whole packs to teams of workgroups however few
+  // rounds they make
   int G = 0, V = 0, block = 0, bpc = 0;
 };
 
@@ -63,6 +65,11 @@ struct Plan {
   // compiled for, packs a workgroup, workgroups launched; team == 0: not planned
   int team = 0, team_v = 0;
   int64_t team_chunk_packs = 0, team_grid = 0;
+  // norm backward of such rows held R = team_v rows at a time by teams of workgroups
+  // (norm_bwd_team_kernel): the same fields, one stride of packs a workgroup, and the
+  // partial rows of column sums that launch leaves (one a team; partial_rows is what
+  // the kernels behind it would use)
+  int64_t team_partial_rows = 0;
   // norm backward / forward on an exact layout (norm_bwd_exact_kernel,
   // norm_fwd_exact_kernel): row blocks a lane keeps in flight, itself included (the
   // forward: 1); GroupNorm on an exact layout (gn_*_exact_kernel): 1; 0 = the
@@ -83,6 +90,11 @@ constexpr int kTeamGroup = 2;  // packs whose weights are requested together
 constexpr int kTeamMaxWorkgroups = 512;
 constexpr int kTeamSlots = 16;
 constexpr int kTeamMinTeams = 8;
+// norm_bwd_team_kernel: rows a team holds at a time, packs of a row a lane holds of each
+// tensor, workgroups a compute unit
+constexpr int kTeamBwdRows = 4;
+constexpr int kTeamBwdPacks = 2;
+constexpr int kTeamBwdPerCu = 1;
 // One call's bookkeeping memory (see the kernel).
 struct TeamEntry {
   unsigned long long tag;  // (call id << 32) | (round + 1) once s1, s2 are in place; 0 while they change
@@ -90,7 +102,9 @@ struct TeamEntry {
   unsigned long long pad[13];  // 128 bytes an entry: neighbours' polls go to other memory channels
 };
 struct TeamSlot {
-  TeamEntry entry[2][kTeamMaxWorkgroups];  // [round parity][workgroup]
+  // [round parity][workgroup]; norm_bwd_team_kernel, which publishes a round before it
+  // gathers the one before, goes round all four
+  TeamEntry entry[4][kTeamMaxWorkgroups];
   unsigned int gave_up;                    // id of a call one of whose waits ran out (a hint)
   unsigned int pad[3];
 };
@@ -937,6 +951,39 @@ inline int make_plan(OpClass oc, int64_t M, int64_t N, int esize, int num_cus, c
       p.team_v = (int)v;
       p.team_chunk_packs = v * kTeamBlock;
       p.team_grid = teams * team;
+    }
+  }
+  // Backward rows beyond one workgroup's registers (whole packs, dX wanted, no residual
+  // gradient): teams of workgroups hold kTeamBwdRows rows at a time, kTeamBwdPacks strides of
+  // packs a workgroup, dY and X read once (norm_bwd_team_kernel).
+  // (override G = -1 with block = 1: the team launch whatever the rounds, for tests)
+  const bool team_bwd_forced = ov.G == -1 && ov.V == 0 && ov.block == 1 && ov.bpc == 0;
+  if (oc == OC_NORM_BWD && !p.resident && p.fast && !fused_add && want_dx &&
+      ((ov.G == 0 && ov.V == 0 && ov.bpc == 0 && ov.block == 0) || team_bwd_forced)) {
+    const int64_t cus = num_cus * kTeamBwdPerCu < kTeamMaxWorkgroups ? num_cus * kTeamBwdPerCu : kTeamMaxWorkgroups;
+    const int64_t chunk = (int64_t)kTeamBwdPacks * kTeamBlock;
+    const int64_t team = (packs + chunk - 1) / chunk;
+    const int64_t ngroups = (M + kTeamBwdRows - 1) / kTeamBwdRows;
+    if (team >= 2 && team <= cus) {
+      int64_t teams = cus / team;
+      if (teams > ngroups) teams = ngroups;
+      // Worth it from a handful of rounds on (a call costs about 28 us beside 9.5 (RMSNorm) to
+      // 11.6 us (LayerNorm) a round, where the two passes of the other kernels cost about
+      // 14.6 us for a round's rows), and where the last workgroup of a row is not mostly idle
+      // (bf16 [8192, 24584], four workgroups a row one of which holds a single pack: 380 us
+      // either way).  Measured, bf16, team / two passes in us: [512, 401408] (26 rounds)
+      // LayerNorm 302 / 360, RMSNorm 257 / 350; [4096, 65536] (64) 381 / 477, 329 / 468;
+      // [256, 1048576] (32) 387 / 518, 331 / 511; [64, 1048576] (8) 115 / 117, 98 / 114;
+      // [1024, 40960] (5) 90 / 81, 76 / 76; [16, 1048576] (2) 41.6 / 35.6, 34.2 / 34.9.
+      const bool rounds_ok = teams >= 1 && ngroups >= (layer_norm ? 8 : 5) * teams;
+      const bool full_ok = 5 * packs >= 4 * team * chunk;
+      if (teams >= 1 && ((rounds_ok && full_ok) || team_bwd_forced)) {
+        p.team = (int)team;
+        p.team_v = kTeamBwdPacks;
+        p.team_chunk_packs = chunk;
+        p.team_grid = teams * team;
+        p.team_partial_rows = want_cols ? teams : 0;
+      }
     }
   }
   // Softmax forward / backward of few, very long rows of whole packs: one workgroup a row
