@@ -115,7 +115,12 @@ int mi355x_layer_norm_fwd(const void* x, const void* gamma, const void* beta, vo
  * ROWNORM_ERR_WORKSPACE), and, for a few rows far too long for the registers,
  * the partial sums of the split-row dX (the regime of Norm.h:632-812), which
  * follow the column sums.  A workspace that holds the first part only is
- * accepted: every row's dX then stays on one workgroup. */
+ * accepted: every row's dX then stays on one workgroup.  Rows beyond one
+ * workgroup's registers in calls of many rows may be held four at a time by teams
+ * of workgroups (dY and X read once; whole packs, 16-byte aligned tensors and
+ * workspace, dx apart from dy and x, the bookkeeping and the bounded wait of
+ * mi355x_rownorm_set_team_wait_us): the first part then holds one row a team,
+ * which this query counts. */
 size_t mi355x_layer_norm_bwd_workspace_bytes(int64_t M, int64_t N, rownorm_dtype x_dtype,
                                              rownorm_dtype w_dtype, int want_dgamma,
                                              int want_dbeta);
@@ -374,7 +379,9 @@ int mi355x_rownorm_plan_at(rownorm_op op, int64_t M, int64_t N, rownorm_dtype x_
 
 /* Test and tuning hook: force lanes_per_row / packs_per_lane / threads per
  * workgroup / workgroups per compute unit for one op (0 keeps the automatic
- * choice for that field; lanes_per_row == -1 forces the multi-pass kernel).  Process-global;
+ * choice for that field; lanes_per_row == -1 forces the multi-pass kernel, and with
+ * block_threads == 1 beside it a norm backward goes to teams of workgroups however few
+ * rounds of rows they make).  Process-global;
  * the four fields of an op are stored as one atomic word, so a call that runs
  * while another thread changes the override uses the old or the new variant,
  * never a mix.  Production callers never use it: with no override set (the
@@ -391,7 +398,8 @@ int mi355x_rownorm_set_override(rownorm_op op, int lanes_per_row, int packs_per_
  * RMSNorm forward rows beyond 131072 16-bit or 65536 float32 elements, whole
  * 16-byte packs, no residual add, no cast, y not overlapping x; GroupNorm forward
  * slabs of that size; softmax / log_softmax forward and backward of few, very long
- * rows): how long a workgroup waits for the others of its team before it sums the
+ * rows; LayerNorm / RMSNorm backward rows beyond one workgroup's registers in calls of
+ * many rows): how long a workgroup waits for the others of its team before it sums the
  * whole row itself (a second pass over the inputs, the same result to rounding), in
  * microseconds; 0xffffffff
  * restores the default, one second.  0 makes every wait give up at once, which is
