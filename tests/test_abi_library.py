@@ -156,6 +156,18 @@ def test_plan_invariants(cabi, op, dt):
                 assert p["rows_per_block"] == p["block_threads"] // G
                 assert p["grid_blocks"] <= (M + p["rows_per_block"] - 1) // p["rows_per_block"]
             elif (op in (cabi.OP_LAYER_NORM_FWD, cabi.OP_RMS_NORM_FWD) and N % E == 0 and
+                  p["row_chunks"] >= 2 and p["block_threads"] == 512 and
+                  p["packs_per_lane"] == 10):
+                # many forward rows of whole packs too long for eight teams at a time: a team of
+                # `row_chunks` workgroups a row, ten packs a lane, one workgroup a compute unit,
+                # three rows in flight; from 16 rounds on
+                team = p["row_chunks"]
+                assert p["rows_per_block"] == 1
+                assert team == (N // E + 5119) // 5120 and p["grid_blocks"] <= 256
+                teams = p["grid_blocks"] // team
+                assert p["grid_blocks"] % team == 0 and 1 <= teams <= M
+                assert M >= 16 * teams and 5 * (N // E) >= 4 * team * 5120
+            elif (op in (cabi.OP_LAYER_NORM_FWD, cabi.OP_RMS_NORM_FWD) and N % E == 0 and
                   p["grid_blocks"] > M):
                 # rows of whole packs beyond one workgroup's registers, 8 teams or more: a team
                 # of `row_chunks` workgroups holds a row, at most one workgroup a compute unit,

@@ -912,11 +912,18 @@ int mi355x_rownorm_plan_at(rownorm_op op, int64_t M, int64_t N, rownorm_dtype x_
   out->reserved = plan.team > 0 ? plan.team : (plan.split > 1 ? plan.split : 0);
   out->grid_blocks = plan.team > 0 ? plan.team_grid : plan.grid;
   out->partial_rows = (int64_t)bwd_partial_rows(plan);
-  // (backward rows held by teams: the workgroup, and the packs of a row a lane holds)
+  // (groups of rows held by teams: the workgroup, the packs of a row a lane holds, the rows)
   if (plan.team > 0 && (op == ROWNORM_OP_LAYER_NORM_BWD || op == ROWNORM_OP_RMS_NORM_BWD)) {
     out->lanes_per_row = kTeamBlock;
     out->block_threads = kTeamBlock;
     out->packs_per_lane = plan.team_v;
+    out->rows_per_block = kTeamBwdRows;
+  }
+  if (plan.team > 0 && plan.team_r > 0) {
+    out->lanes_per_row = kTeamBlock;
+    out->block_threads = kTeamBlock;
+    out->packs_per_lane = plan.team_v;
+    out->rows_per_block = plan.team_r;
   }
   return 0;
 }

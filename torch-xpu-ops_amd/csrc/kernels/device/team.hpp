@@ -123,11 +123,16 @@ __device__ __forceinline__ void team_publish_words(TeamEntry* mine, unsigned int
 // values over the team, added in a fixed order (entries lane, lane + 64, ... per lane, then
 // across the lanes): the same bits in every lane and in every workgroup of the team.  False
 // as in team_publish_and_gather (v[] is then not meaningful).
+// (A lane's entries are read four at a time -- tags, then all their words, then the tags
+// again: three round trips to memory for a team of up to 256, however many entries a lane has.)
+constexpr int kTeamGatherBatch = 4;
+
 template <int K>
 __device__ __forceinline__ bool team_gather_sums(TeamSlot* slot, const TeamEntry* mates, int team,
                                                  unsigned int call_id, unsigned int round,
                                                  unsigned long long wait_ticks,
                                                  float (&v)[2 * K]) {
+  constexpr int B = kTeamGatherBatch;
   const int lane = (int)threadIdx.x;
   const unsigned long long expect = ((unsigned long long)call_id << 32) | (round + 1u);
   const unsigned long long t0 = wall_clock64();
@@ -135,29 +140,139 @@ __device__ __forceinline__ bool team_gather_sums(TeamSlot* slot, const TeamEntry
   unsigned int polls = 0;
   for (;;) {
     bool ok = true;
-    for (int j = lane; j < team; j += 64) ok = ok && team_load(&mates[j].tag) == expect;
-    if (__ballot(ok) == __ballot(true)) {
 #pragma unroll
-      for (int k = 0; k < 2 * K; ++k) v[k] = 0.0f;
-      for (int j = lane; j < team; j += 64) {
-        const unsigned long long* words = &mates[j].s1;
-        unsigned long long w[K];
+    for (int k = 0; k < 2 * K; ++k) v[k] = 0.0f;
+    for (int j0 = lane; j0 < team && ok; j0 += 64 * B) {
+      unsigned long long tag0[B], tag1[B], w[B][K];
 #pragma unroll
-        for (int k = 0; k < K; ++k) w[k] = team_load(&words[k]);
-        team_stores_done();  // the numbers have returned before the tag is read again
-        ok = ok && team_load(&mates[j].tag) == expect;
-#pragma unroll
-        for (int k = 0; k < K; ++k) {
-          v[2 * k] += __builtin_bit_cast(float, (unsigned int)(w[k] & 0xffffffffull));
-          v[2 * k + 1] += __builtin_bit_cast(float, (unsigned int)(w[k] >> 32));
-        }
+      for (int b = 0; b < B; ++b) {
+        const int j = j0 + 64 * b;
+        tag0[b] = j < team ? team_load(&mates[j].tag) : expect;
       }
-      if (__ballot(ok) == __ballot(true)) {
 #pragma unroll
-        for (int k = 0; k < 2 * K; ++k) v[k] = wave_group_allreduce<64, SumOp>(v[k]);
-        complete = true;
+      for (int b = 0; b < B; ++b) ok = ok && tag0[b] == expect;
+      if (__ballot(ok) != __ballot(true)) {
+        ok = false;
         break;
       }
+#pragma unroll
+      for (int b = 0; b < B; ++b) {
+        const int j = j0 + 64 * b;
+        const unsigned long long* words = &mates[j < team ? j : 0].s1;
+#pragma unroll
+        for (int k = 0; k < K; ++k) w[b][k] = team_load(&words[k]);
+      }
+      team_stores_done();  // the numbers have returned before the tags are read again
+#pragma unroll
+      for (int b = 0; b < B; ++b) {
+        const int j = j0 + 64 * b;
+        tag1[b] = j < team ? team_load(&mates[j].tag) : expect;
+      }
+#pragma unroll
+      for (int b = 0; b < B; ++b) {
+        ok = ok && tag1[b] == expect;
+        if (j0 + 64 * b < team) {
+#pragma unroll
+          for (int k = 0; k < K; ++k) {
+            v[2 * k] += __builtin_bit_cast(float, (unsigned int)(w[b][k] & 0xffffffffull));
+            v[2 * k + 1] += __builtin_bit_cast(float, (unsigned int)(w[b][k] >> 32));
+          }
+        }
+      }
+    }
+    if (__ballot(ok) == __ballot(true)) {
+#pragma unroll
+      for (int k = 0; k < 2 * K; ++k) v[k] = wave_group_allreduce<64, SumOp>(v[k]);
+      complete = true;
+      break;
+    }
+    // (the hint word is one address for the whole grid: looked at every 16th time)
+    if ((polls++ & 15u) == 0) {
+      const unsigned int hint =
+          __hip_atomic_load(&slot->gave_up, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+      if (hint == call_id) break;
+    }
+    if (wall_clock64() - t0 > wait_ticks) break;
+    __builtin_amdgcn_s_sleep(8);
+  }
+  if (lane == 0 && !complete)
+    __hip_atomic_store(&slot->gave_up, call_id, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+  return complete;
+}
+
+// The same two halves with K float64 values a workgroup (K <= 15), summed over the team in
+// the same fixed order.
+template <int K>
+__device__ __forceinline__ void team_publish_f64(TeamEntry* mine, unsigned int call_id,
+                                                 unsigned int round, const double (&v)[K]) {
+  static_assert(K >= 1 && K <= 15, "an entry holds a tag and 15 words");
+  unsigned long long* words = &mine->s1;
+  team_stores_done();  // the tag has been 0 in memory before the numbers change
+#pragma unroll
+  for (int k = 0; k < K; ++k) team_store(&words[k], __builtin_bit_cast(unsigned long long, v[k]));
+  team_stores_done();
+  team_store(&mine->tag, ((unsigned long long)call_id << 32) | (round + 1u));
+}
+
+template <int K>
+__device__ __forceinline__ bool team_gather_sums_f64(TeamSlot* slot, const TeamEntry* mates,
+                                                     int team, unsigned int call_id,
+                                                     unsigned int round,
+                                                     unsigned long long wait_ticks,
+                                                     double (&v)[K]) {
+  constexpr int B = kTeamGatherBatch;
+  const int lane = (int)threadIdx.x;
+  const unsigned long long expect = ((unsigned long long)call_id << 32) | (round + 1u);
+  const unsigned long long t0 = wall_clock64();
+  bool complete = false;
+  unsigned int polls = 0;
+  for (;;) {
+    bool ok = true;
+#pragma unroll
+    for (int k = 0; k < K; ++k) v[k] = 0.0;
+    for (int j0 = lane; j0 < team && ok; j0 += 64 * B) {
+      unsigned long long tag0[B], tag1[B], w[B][K];
+#pragma unroll
+      for (int b = 0; b < B; ++b) {
+        const int j = j0 + 64 * b;
+        tag0[b] = j < team ? team_load(&mates[j].tag) : expect;
+      }
+#pragma unroll
+      for (int b = 0; b < B; ++b) ok = ok && tag0[b] == expect;
+      if (__ballot(ok) != __ballot(true)) {
+        ok = false;
+        break;
+      }
+#pragma unroll
+      for (int b = 0; b < B; ++b) {
+        const int j = j0 + 64 * b;
+        const unsigned long long* words = &mates[j < team ? j : 0].s1;
+#pragma unroll
+        for (int k = 0; k < K; ++k) w[b][k] = team_load(&words[k]);
+      }
+      team_stores_done();  // the numbers have returned before the tags are read again
+#pragma unroll
+      for (int b = 0; b < B; ++b) {
+        const int j = j0 + 64 * b;
+        tag1[b] = j < team ? team_load(&mates[j].tag) : expect;
+      }
+#pragma unroll
+      for (int b = 0; b < B; ++b) {
+        ok = ok && tag1[b] == expect;
+        if (j0 + 64 * b < team) {
+#pragma unroll
+          for (int k = 0; k < K; ++k) v[k] += __builtin_bit_cast(double, w[b][k]);
+        }
+      }
+    }
+    if (__ballot(ok) == __ballot(true)) {
+#pragma unroll
+      for (int k = 0; k < K; ++k) {
+#pragma unroll
+        for (int off = 32; off > 0; off >>= 1) v[k] += __shfl_xor(v[k], off, 64);
+      }
+      complete = true;
+      break;
     }
     // (the hint word is one address for the whole grid: looked at every 16th time)
     if ((polls++ & 15u) == 0) {

@@ -1250,6 +1250,256 @@ norm_fwd_team_kernel(const T* __restrict__ x, const WT* __restrict__ gamma,
 }
 
 // ---------------------------------------------------------------------------
+// The forward of such rows when a team has many of them to do: the team holds R rows at a
+// time, workgroup c the packs [c * V * BLOCK, (c + 1) * V * BLOCK) of each (V packs a lane and
+// row), so a lane meets the same columns in every row and keeps their gamma / beta in
+// registers for the whole call (norm_fwd_team_kernel looks them up again for every row: at
+// ten million elements a row that is as much traffic as X).  Three register sets: group j of
+// a team lives in set j % 3; in round j a workgroup requests group j + 2, sums group j + 1
+// (requested a round ago) and publishes its 2 R float64 sums, gathers group j (published a
+// round earlier) and writes its Y: neither the loads nor the exchange are waited for with
+// nothing else to do.  One workgroup a compute unit.  The statistics are those of norm_fwd_team_kernel (float64 sums about the median of
+// the row's first three elements; mean = hi + lo).  A workgroup whose wait runs out sums its
+// R rows itself (Y must not overlap X) and loads its packs again.
+template <class T, class WT, bool RMS, int R, int V>
+__global__ void __launch_bounds__(kTeamBlock, kTeamBlock / 256)
+norm_fwd_rows_team_kernel(const T* __restrict__ x, const WT* __restrict__ gamma,
+                          const WT* __restrict__ beta, T* __restrict__ y,
+                          float* __restrict__ mean, float* __restrict__ rstd, int64_t M, int N,
+                          float eps, int team, TeamSlot* slot, unsigned int call_id,
+                          unsigned long long wait_ticks) {
+  constexpr int E = elems_per_pack<T>::value;
+  constexpr int BLOCK = kTeamBlock;
+  constexpr int K = 2 * R;
+  __shared__ double red[(BLOCK / 64) * K];
+  __shared__ float stat[R][3];  // a row's mean (hi, lo) and rstd
+  __shared__ int failed;
+  // from five packs a lane on gamma lives in LDS (a pack a lane and k), not in registers
+  constexpr bool GL = V > 4;
+  __shared__ Pack<WT, E> gl[GL ? V : 1][GL ? BLOCK : 1];
+  const int tm = (int)blockIdx.x / team;
+  const int c = (int)blockIdx.x - tm * team;
+  const int teams = (int)gridDim.x / team;
+  const int npacks = N / E;
+  const int pk0 = c * (V * BLOCK) + (int)threadIdx.x;
+  const int64_t ngroups = (M + R - 1) / R;
+  const double dN = (double)N;
+  const bool hb = !RMS && beta != nullptr;
+  Pack<WT, E> pg[GL ? 1 : V], pb[RMS ? 1 : V];
+#pragma unroll
+  for (int k = 0; k < V; ++k) {
+    const bool held = pk0 + k * BLOCK < npacks;
+    Pack<WT, E> gk = Pack<WT, E>::splat(1.0f);
+    if (gamma != nullptr && held) gk = Pack<WT, E>::load(gamma + (int64_t)(pk0 + k * BLOCK) * E);
+    if constexpr (GL)
+      gl[k][threadIdx.x] = gk;  // (read back by the same lane only)
+    else
+      pg[k] = gk;
+    if constexpr (!RMS) {
+      pb[k] = Pack<WT, E>::zero();
+      if (hb && held) pb[k] = Pack<WT, E>::load(beta + (int64_t)(pk0 + k * BLOCK) * E);
+    }
+  }
+  const uint32_t loff = (uint32_t)(pk0 < npacks ? pk0 : 0) * 16u;
+  auto at = [](auto* p, uint32_t off) {
+    using Elem = std::remove_pointer_t<decltype(p)>;
+    typedef __attribute__((address_space(1))) Elem* GlobalPtr;
+    return (Elem*)reinterpret_cast<GlobalPtr>(reinterpret_cast<uintptr_t>(p) + off);
+  };
+  auto row_of = [&](int64_t g, int r) { return g * R + r < M ? g * R + r : M - 1; };
+  // the lane's packs of the rows of group g (zeros beyond the tensor and beyond the row)
+  auto load_group = [&](int64_t g, Pack<T, E> (&px)[R * V]) {
+#pragma unroll
+    for (int r = 0; r < R; ++r) {
+      const int64_t row = g * R + r;
+#pragma unroll
+      for (int k = 0; k < V; ++k) {
+        px[r * V + k] = Pack<T, E>::zero();
+        if (pk0 + k * BLOCK < npacks && row < M)
+          px[r * V + k] = Pack<T, E>::load_stream(at(x + row * (int64_t)N + k * BLOCK * E, loff));
+      }
+    }
+  };
+  // mean = hi + lo and rstd of a row from its centred sums (see the split-row kernels)
+  auto set_stats = [&](int r, double t1, double t2, double kd) {
+    if constexpr (RMS) {
+      stat[r][0] = 0.0f;
+      stat[r][1] = 0.0f;
+      stat[r][2] = (float)(1.0 / sqrt(t2 / dN + (double)eps));
+    } else {
+      const double m1 = t1 / dN;
+      const double mu = kd + m1;
+      double var = (t2 - t1 * m1) / dN;
+      var = var < 0.0 ? 0.0 : var;  // (a select: NaN stays NaN)
+      const float hi = (float)mu;
+      stat[r][0] = var == var ? hi : (float)var;  // NaN variance: NaN mean
+      stat[r][1] = (float)(mu - (double)hi);
+      stat[r][2] = (float)(1.0 / sqrt(var + (double)eps));
+    }
+  };
+  // The centred float64 sums of the rows of group g (held in px), published as round `round`.
+  auto sums_and_publish = [&](int64_t g, unsigned int round, Pack<T, E> (&px)[R * V]) {
+    TeamEntry* mine = &slot->entry[round & 3u][blockIdx.x];
+    if (threadIdx.x == 0) team_store(&mine->tag, 0ull);
+    double acc[K];
+#pragma unroll
+    for (int r = 0; r < R; ++r) {
+      const float kf = RMS ? 0.0f : split_row_centre(x + row_of(g, r) * (int64_t)N, (const T*)nullptr, N);
+      const double kd = (double)kf;
+      double s1 = 0.0, s2 = 0.0;
+#pragma unroll
+      for (int k = 0; k < V; ++k) {
+        keep_packed(px[r * V + k]);
+        // (a pack beyond the row or the tensor holds zeros, which are not x - k = 0)
+        if (pk0 + k * BLOCK < npacks && g * R + r < M)
+          add_centred_sums<T, E, RMS, true>(px[r * V + k], E, kf, kd, s1, s2);
+      }
+      acc[2 * r] = s1;
+      acc[2 * r + 1] = s2;
+    }
+    // over the workgroup, in a fixed order; thread 0 holds the result
+#pragma unroll
+    for (int k = 0; k < K; ++k) {
+#pragma unroll
+      for (int off = 32; off > 0; off >>= 1) acc[k] += __shfl_down(acc[k], off, 64);
+    }
+    const int wave = threadIdx.x >> 6;
+    if ((threadIdx.x & 63) == 0) {
+#pragma unroll
+      for (int k = 0; k < K; ++k) red[wave * K + k] = acc[k];
+    }
+    __syncthreads();
+    if (threadIdx.x == 0) {
+#pragma unroll
+      for (int k = 0; k < K; ++k) {
+        double t = red[k];
+#pragma unroll
+        for (int w = 1; w < BLOCK / 64; ++w) t += red[w * K + k];
+        acc[k] = t;
+      }
+      team_publish_f64<K>(mine, call_id, round, acc);
+    }
+  };
+  // The sums of group g across the team, its statistics, its Y.  (g1 / p1, g2 / p2: the groups
+  // held in the other two register sets, loaded again after the rare pass over whole rows so
+  // that nothing stays live across that pass; the first wavefront requests g2 only here,
+  // behind its gather: the exchange waits for everything the wavefront has outstanding, and
+  // a request made before it would put the machine's whole burst of loads in its way.)
+  auto finish = [&](int64_t g, unsigned int round, Pack<T, E> (&px)[R * V], int64_t g1,
+                    Pack<T, E> (&p1)[R * V], int64_t g2, Pack<T, E> (&p2)[R * V]) {
+    // (every thread has read the stat[] of the round before and thread 0 its red[])
+    __syncthreads();
+    if (threadIdx.x < 64) {  // the first wavefront waits and adds up
+      double tot[K];
+      const bool complete =
+          team_gather_sums_f64<K>(slot, slot->entry[round & 3u] + tm * team, team, call_id, round,
+                                  wait_ticks, tot);
+      if (threadIdx.x == 0) {
+        failed = complete ? 0 : 1;
+        if (complete) {
+#pragma unroll
+          for (int r = 0; r < R; ++r) {
+            const float kf =
+                RMS ? 0.0f : split_row_centre(x + row_of(g, r) * (int64_t)N, (const T*)nullptr, N);
+            set_stats(r, tot[2 * r], tot[2 * r + 1], (double)kf);
+          }
+        }
+      }
+      if (complete && g2 >= 0) load_group(g2, p2);
+    }
+    __syncthreads();
+    if (failed != 0) {  // (uniform over the workgroup)
+      // The team did not come together: the sums over the whole rows (X, which no
+      // workgroup writes), then the packs again.
+      for (int r = 0; r < R; ++r) {
+        const T* xr = x + row_of(g, r) * (int64_t)N;
+        const float kf = RMS ? 0.0f : split_row_centre(xr, (const T*)nullptr, N);
+        double w1 = 0.0, w2 = 0.0;
+        long_row_sums<T, E, BLOCK, RMS, false>(xr, (const T*)nullptr, N, 0, npacks, kf, w1, w2);
+        __syncthreads();  // (red[] of the sum before has been read)
+        block_sum2_f64<BLOCK>(w1, w2, red);
+        if (threadIdx.x == 0) set_stats(r, w1, w2, (double)kf);
+      }
+      __syncthreads();
+      load_group(g, px);
+      load_group(g1 >= 0 ? g1 : M, p1);  // (a group beyond the tensor: zeros)
+      load_group(g2 >= 0 ? g2 : M, p2);
+    }
+#pragma unroll
+    for (int r = 0; r < R; ++r) {
+      const int64_t row = g * R + r;
+      const float hi = stat[r][0], lo = stat[r][1], rs = stat[r][2];
+#pragma unroll
+      for (int k = 0; k < V; ++k) {
+        const bool held = pk0 + k * BLOCK < npacks;
+        Pack<WT, E> gk;
+        if constexpr (GL) {
+          gk = gl[k][threadIdx.x];
+        } else {
+          keep_packed(pg[k]);  // (widened here, for this pack: not once ahead of the row loop)
+          gk = pg[k];
+        }
+        if constexpr (!RMS) keep_packed(pb[k]);
+        Pack<T, E> o;
+#pragma unroll
+        for (int i = 0; i < E; ++i) {
+          float v;
+          if constexpr (RMS)
+            v = (px[r * V + k].get(i) * rs) * gk.get(i);
+          else
+            v = (((px[r * V + k].get(i) - hi) - lo) * rs) * gk.get(i) + pb[k].get(i);
+          o.set(i, v);
+        }
+        if (held && row < M) o.store_stream(at(y + row * (int64_t)N + k * BLOCK * E, loff));
+        // (the next pack is widened after this one has been stored, not before: registers)
+        __builtin_amdgcn_sched_barrier(0);
+      }
+      if (c == 0 && threadIdx.x == 0 && row < M) {
+        if constexpr (!RMS)
+          if (mean) mean[row] = hi;
+        if (rstd) rstd[row] = rs;
+      }
+    }
+  };
+
+  // Group j of the team (tm + j * teams) lives in register set j % 3: requested at the start
+  // of round j - 2, summed and published in round j - 1, gathered and written in round j.
+  Pack<T, E> ax[R * V], bx[R * V], cx[R * V];
+  const bool later = threadIdx.x < 64;  // the exchanging wavefront requests inside finish()
+  const int64_t st = teams;
+  int64_t g = tm;
+  unsigned int round = 0;
+  if (g < ngroups) {
+    load_group(g, ax);
+    if (g + st < ngroups) load_group(g + st, bx);
+    sums_and_publish(g, 0, ax);
+  }
+  auto valid = [&](int64_t q) { return q < ngroups ? q : (int64_t)-1; };
+  while (g < ngroups) {
+    // (a, b, c) = (ax, bx, cx)
+    if (g + 2 * st < ngroups && !later) load_group(g + 2 * st, cx);
+    if (g + st < ngroups) sums_and_publish(g + st, round + 1, bx);
+    finish(g, round, ax, valid(g + st), bx, valid(g + 2 * st), cx);
+    g += st;
+    ++round;
+    if (g >= ngroups) break;
+    // (a, b, c) = (bx, cx, ax)
+    if (g + 2 * st < ngroups && !later) load_group(g + 2 * st, ax);
+    if (g + st < ngroups) sums_and_publish(g + st, round + 1, cx);
+    finish(g, round, bx, valid(g + st), cx, valid(g + 2 * st), ax);
+    g += st;
+    ++round;
+    if (g >= ngroups) break;
+    // (a, b, c) = (cx, ax, bx)
+    if (g + 2 * st < ngroups && !later) load_group(g + 2 * st, bx);
+    if (g + st < ngroups) sums_and_publish(g + st, round + 1, ax);
+    finish(g, round, cx, valid(g + st), ax, valid(g + 2 * st), bx);
+    g += st;
+    ++round;
+  }
+}
+
+// ---------------------------------------------------------------------------
 // Split-row forward: few rows, each far beyond the registers (the regime of the
 // reference's split-row kernels, Norm.h:632-812).  A row is cut into `chunks`
 // chunks of `chunk_packs` packs (the last one takes the remainder as well, at

@@ -114,7 +114,25 @@ int launch_norm_fwd(const Plan& plan, const NormFwdArgs& a, hipStream_t stream) 
         return (int)hipGetLastError();
     }
   }
-  if (norm_fwd_team_serves<T, TY, ADD>(plan, a)) {
+  if (norm_fwd_team_serves<T, TY, ADD>(plan, a) && plan.team_r > 0) {
+    // one pass with three rows in flight in the registers of a team of workgroups, weights held
+    if constexpr (!ADD && std::is_same<T, TY>::value) {
+      TeamSlot* slot = (TeamSlot*)a.team_slot;
+      auto go = [&](auto r, auto v) {
+        constexpr int R = decltype(r)::value, V = decltype(v)::value;
+        hipLaunchKernelGGL((norm_fwd_rows_team_kernel<T, WT, RMS, R, V>),
+                           dim3((unsigned)plan.team_grid), dim3(kTeamBlock), 0, stream,
+                           (const T*)a.x, (const WT*)a.gamma, (const WT*)a.beta, (T*)a.y, a.mean,
+                           a.rstd, a.M, a.N, a.eps, plan.team, slot, a.team_id, a.team_wait_ticks);
+      };
+      if (sizeof(WT) == sizeof(T) && plan.team_r == 1 && plan.team_v == kTeamFwdLongPacks) {
+        if constexpr (sizeof(WT) == sizeof(T))
+          go(std::integral_constant<int, 1>{}, std::integral_constant<int, kTeamFwdLongPacks>{});
+      } else {
+        return (int)hipErrorInvalidConfiguration;
+      }
+    }
+  } else if (norm_fwd_team_serves<T, TY, ADD>(plan, a)) {
     // one pass with the row in the registers of a team of workgroups
     TeamSlot* slot = (TeamSlot*)a.team_slot;
     auto go = [&](auto v) {

@@ -70,6 +70,9 @@ struct Plan {
   // partial rows of column sums that launch leaves (one a team; partial_rows is what
   // the kernels behind it would use)
   int64_t team_partial_rows = 0;
+  // norm forward of such rows with three rows in flight a workgroup, team_v packs of a row
+  // a lane and the weights held (norm_fwd_rows_team_kernel): 1; 0: norm_fwd_team_kernel
+  int team_r = 0;
   // norm backward / forward on an exact layout (norm_bwd_exact_kernel,
   // norm_fwd_exact_kernel): row blocks a lane keeps in flight, itself included (the
   // forward: 1); GroupNorm on an exact layout (gn_*_exact_kernel): 1; 0 = the
@@ -95,6 +98,9 @@ constexpr int kTeamMinTeams = 8;
 constexpr int kTeamBwdRows = 4;
 constexpr int kTeamBwdPacks = 2;
 constexpr int kTeamBwdPerCu = 1;
+// norm_fwd_rows_team_kernel: packs of a row a lane, and the rounds from which it is taken
+constexpr int kTeamFwdLongPacks = 10;
+constexpr int kTeamFwdMinRounds = 16;
 // One call's bookkeeping memory (see the kernel).
 struct TeamEntry {
   unsigned long long tag;  // (call id << 32) | (round + 1) once s1, s2 are in place; 0 while they change
@@ -951,6 +957,31 @@ inline int make_plan(OpClass oc, int64_t M, int64_t N, int esize, int num_cus, c
       p.team_v = (int)v;
       p.team_chunk_packs = v * kTeamBlock;
       p.team_grid = teams * team;
+    }
+  }
+  // Forward rows too long for at least eight such teams (beyond 256 / 8 * 16 * 512 packs),
+  // many of them, weights no wider than the rows: one team over the machine, one workgroup a
+  // compute unit, kTeamFwdLongPacks packs a lane, three rows in flight a workgroup and gamma /
+  // beta held for the whole call (norm_fwd_rows_team_kernel).
+  // (override G = -1 with block = 1: whatever the rounds and the other teams, for tests)
+  const bool team_rows_forced = ov.G == -1 && ov.V == 0 && ov.block == 1 && ov.bpc == 0;
+  if (oc == OC_NORM_FWD && !p.resident && p.fast && !fused_add && !wide_weights &&
+      ((ov.G == 0 && ov.V == 0 && ov.bpc == 0 && ov.block == 0 && p.team == 0) || team_rows_forced)) {
+    const int64_t cus = num_cus < kTeamMaxWorkgroups ? num_cus : kTeamMaxWorkgroups;
+    const int64_t chunk = (int64_t)kTeamFwdLongPacks * kTeamBlock;
+    const int64_t team = (packs + chunk - 1) / chunk;
+    if (team >= 2 && team <= cus) {
+      int64_t teams = cus / team;
+      if (teams > M) teams = M;
+      const bool rounds_ok = M >= kTeamFwdMinRounds * teams;
+      const bool full_ok = 5 * packs >= 4 * team * chunk;
+      if (teams >= 1 && ((rounds_ok && full_ok) || team_rows_forced)) {
+        p.team = (int)team;
+        p.team_v = kTeamFwdLongPacks;
+        p.team_r = 1;
+        p.team_chunk_packs = chunk;
+        p.team_grid = teams * team;
+      }
     }
   }
   // Backward rows beyond one workgroup's registers (whole packs, dX wanted, no residual
