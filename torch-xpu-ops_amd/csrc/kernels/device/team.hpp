@@ -1,6 +1,9 @@
 // Device side of the exchange between the workgroups of a team (norm_fwd_team_kernel,
 // softmax_fwd_team_kernel): a row too long for one workgroup is held in the registers of
-// several, which pass two numbers each through library-owned device memory.
+// several, which pass two numbers each through library-owned device memory.  Below it: the
+// same exchange in two halves for K float64 values (norm_fwd_rows_team_kernel, which puts
+// a round of other work between publishing and gathering) and a lighter one of
+// self-validating words for float32 values (norm_bwd_team_kernel).
 //
 // What crosses workgroups.  An entry is {tag, s1, s2}, 128 bytes apart; the tag of a
 // finished entry is (call id << 32) | (round + 1), ids being unique per call, so
@@ -96,112 +99,104 @@ __device__ __forceinline__ bool team_publish_and_gather(TeamSlot* slot, TeamEntr
   return complete;
 }
 
-// The two halves of such an exchange with K 64-bit words a workgroup (K <= 15: an entry's s1,
-// s2 and the words behind them), for kernels that put other work between them.  Word k holds
-// the float32 values v[2k] and v[2k + 1].
-//
-// team_publish_words: for lane 0 of a wavefront whose entry `mine` has had the tag 0 since
-// the workgroup started on the round.
-template <int K>
-__device__ __forceinline__ void team_publish_words(TeamEntry* mine, unsigned int call_id,
-                                                   unsigned int round, const float (&v)[2 * K]) {
-  static_assert(K >= 1 && K <= 15, "an entry holds a tag and 15 words");
-  unsigned long long* words = &mine->s1;
-  team_stores_done();  // the tag has been 0 in memory before the numbers change
-#pragma unroll
-  for (int k = 0; k < K; ++k) {
-    const unsigned long long lo = __builtin_bit_cast(unsigned int, v[2 * k]);
-    const unsigned long long hi = __builtin_bit_cast(unsigned int, v[2 * k + 1]);
-    team_store(&words[k], lo | (hi << 32));
-  }
-  team_stores_done();
-  team_store(&mine->tag, ((unsigned long long)call_id << 32) | (round + 1u));
-}
-
-// team_gather_sums: for the first wavefront of a workgroup (all 64 lanes); waits for the
-// `team` entries from `mates` on to carry the round's tag and leaves in v[] the sums of their
-// values over the team, added in a fixed order (entries lane, lane + 64, ... per lane, then
-// across the lanes): the same bits in every lane and in every workgroup of the team.  False
-// as in team_publish_and_gather (v[] is then not meaningful).
-// (A lane's entries are read four at a time -- tags, then all their words, then the tags
-// again: three round trips to memory for a team of up to 256, however many entries a lane has.)
+// (A lane's entries are read four at a time: a round trip to memory for a team of up to 256,
+// however many entries a lane has.)
 constexpr int kTeamGatherBatch = 4;
 
+// A lighter exchange for float32 values: every 64-bit word carries its own tag, so a word is
+// valid or not by itself and neither side orders anything.  Word k of an entry holds
+// {v[k], tag}, tag = ((call id mod 2^26 - 1) + 1) << 6 | (round mod 64): never 0 (the memory
+// starts as zeros), different for the rounds that share a buffer (a buffer is reused every
+// fourth round, and workgroups of a team whose gathers succeed are never more than three
+// rounds apart), different from call to call.  The words live in an entry's pad[], which no
+// other exchange writes: whatever a word holds was put there by this one.  Publishing is K
+// plain stores with nothing to
+// wait for.  Gathering reads every word of a lane's entries in one round trip, accepts them
+// if every tag is the round's, and then -- a second round trip, after the words have
+// returned -- makes sure no workgroup of the call has given up: a workgroup that no longer
+// waits for its team can be any number of rounds ahead, tags repeat after 64 rounds, and
+// it records that it gave up (and waits for that store) before it goes on, so words it
+// writes later are never accepted by a gather that still saw the record unset.
+__device__ __forceinline__ unsigned int team_word_tag(unsigned int call_id, unsigned int round) {
+  return ((call_id % 0x3ffffffu) + 1u) << 6 | (round & 63u);
+}
+
 template <int K>
-__device__ __forceinline__ bool team_gather_sums(TeamSlot* slot, const TeamEntry* mates, int team,
-                                                 unsigned int call_id, unsigned int round,
-                                                 unsigned long long wait_ticks,
-                                                 float (&v)[2 * K]) {
+__device__ __forceinline__ void team_publish_tagged(TeamEntry* mine, unsigned int call_id,
+                                                    unsigned int round, const float (&v)[K]) {
+  static_assert(K >= 1 && K <= 13, "an entry's pad[] holds 13 words");
+  unsigned long long* words = &mine->pad[0];
+  const unsigned long long tag = (unsigned long long)team_word_tag(call_id, round) << 32;
+#pragma unroll
+  for (int k = 0; k < K; ++k)
+    team_store(&words[k], tag | (unsigned long long)__builtin_bit_cast(unsigned int, v[k]));
+}
+
+// For the first wavefront of a workgroup (all 64 lanes).  On success v[] holds the sums over
+// the team, added in a fixed order (entries lane, lane + 64, ... per lane, then across the
+// lanes): the same bits in every lane and in every workgroup of the team.  False when the
+// wait ran out or a workgroup of the call has given up (recorded in the slot, and the store
+// waited for, before this returns).
+template <int K>
+__device__ __forceinline__ bool team_gather_tagged(TeamSlot* slot, const TeamEntry* mates, int team,
+                                                   unsigned int call_id, unsigned int round,
+                                                   unsigned long long wait_ticks, float (&v)[K]) {
   constexpr int B = kTeamGatherBatch;
   const int lane = (int)threadIdx.x;
-  const unsigned long long expect = ((unsigned long long)call_id << 32) | (round + 1u);
+  const unsigned int expect = team_word_tag(call_id, round);
   const unsigned long long t0 = wall_clock64();
   bool complete = false;
-  unsigned int polls = 0;
   for (;;) {
     bool ok = true;
 #pragma unroll
-    for (int k = 0; k < 2 * K; ++k) v[k] = 0.0f;
-    for (int j0 = lane; j0 < team && ok; j0 += 64 * B) {
-      unsigned long long tag0[B], tag1[B], w[B][K];
+    for (int k = 0; k < K; ++k) v[k] = 0.0f;
+    for (int j0 = lane; j0 < team; j0 += 64 * B) {
+      unsigned long long w[B][K];
 #pragma unroll
       for (int b = 0; b < B; ++b) {
         const int j = j0 + 64 * b;
-        tag0[b] = j < team ? team_load(&mates[j].tag) : expect;
-      }
-#pragma unroll
-      for (int b = 0; b < B; ++b) ok = ok && tag0[b] == expect;
-      if (__ballot(ok) != __ballot(true)) {
-        ok = false;
-        break;
-      }
-#pragma unroll
-      for (int b = 0; b < B; ++b) {
-        const int j = j0 + 64 * b;
-        const unsigned long long* words = &mates[j < team ? j : 0].s1;
+        const unsigned long long* words = &mates[j < team ? j : 0].pad[0];
 #pragma unroll
         for (int k = 0; k < K; ++k) w[b][k] = team_load(&words[k]);
       }
-      team_stores_done();  // the numbers have returned before the tags are read again
 #pragma unroll
       for (int b = 0; b < B; ++b) {
-        const int j = j0 + 64 * b;
-        tag1[b] = j < team ? team_load(&mates[j].tag) : expect;
-      }
-#pragma unroll
-      for (int b = 0; b < B; ++b) {
-        ok = ok && tag1[b] == expect;
         if (j0 + 64 * b < team) {
 #pragma unroll
           for (int k = 0; k < K; ++k) {
-            v[2 * k] += __builtin_bit_cast(float, (unsigned int)(w[b][k] & 0xffffffffull));
-            v[2 * k + 1] += __builtin_bit_cast(float, (unsigned int)(w[b][k] >> 32));
+            ok = ok && (unsigned int)(w[b][k] >> 32) == expect;
+            v[k] += __builtin_bit_cast(float, (unsigned int)(w[b][k] & 0xffffffffull));
           }
         }
       }
     }
+    const unsigned int hint =
+        __hip_atomic_load(&slot->gave_up, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+    if (hint == call_id) break;
     if (__ballot(ok) == __ballot(true)) {
+      // (the record is read again only now that the words have returned)
+      team_stores_done();
+      const unsigned int after =
+          __hip_atomic_load(&slot->gave_up, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+      if (after == call_id) break;
 #pragma unroll
-      for (int k = 0; k < 2 * K; ++k) v[k] = wave_group_allreduce<64, SumOp>(v[k]);
+      for (int k = 0; k < K; ++k) v[k] = wave_group_allreduce<64, SumOp>(v[k]);
       complete = true;
       break;
-    }
-    // (the hint word is one address for the whole grid: looked at every 16th time)
-    if ((polls++ & 15u) == 0) {
-      const unsigned int hint =
-          __hip_atomic_load(&slot->gave_up, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
-      if (hint == call_id) break;
     }
     if (wall_clock64() - t0 > wait_ticks) break;
     __builtin_amdgcn_s_sleep(8);
   }
-  if (lane == 0 && !complete)
-    __hip_atomic_store(&slot->gave_up, call_id, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+  if (!complete) {
+    if (lane == 0)
+      __hip_atomic_store(&slot->gave_up, call_id, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+    team_stores_done();
+  }
   return complete;
 }
 
 // The same two halves with K float64 values a workgroup (K <= 15), summed over the team in
-// the same fixed order.
+// the same fixed order as team_gather_tagged.
 template <int K>
 __device__ __forceinline__ void team_publish_f64(TeamEntry* mine, unsigned int call_id,
                                                  unsigned int round, const double (&v)[K]) {

@@ -1271,9 +1271,11 @@ norm_fwd_rows_team_kernel(const T* __restrict__ x, const WT* __restrict__ gamma,
   constexpr int E = elems_per_pack<T>::value;
   constexpr int BLOCK = kTeamBlock;
   constexpr int K = 2 * R;
-  __shared__ double red[(BLOCK / 64) * K];
-  __shared__ float stat[R][3];  // a row's mean (hi, lo) and rstd
-  __shared__ int failed;
+  // (red, stat and failed by round parity: a round's values are read while the next round's
+  // are already being written)
+  __shared__ double red[2][(BLOCK / 64) * K];
+  __shared__ float stat[2][R][3];  // a row's mean (hi, lo) and rstd
+  __shared__ int failed[2];
   // from five packs a lane on gamma lives in LDS (a pack a lane and k), not in registers
   constexpr bool GL = V > 4;
   __shared__ Pack<WT, E> gl[GL ? V : 1][GL ? BLOCK : 1];
@@ -1307,57 +1309,101 @@ norm_fwd_rows_team_kernel(const T* __restrict__ x, const WT* __restrict__ gamma,
     return (Elem*)reinterpret_cast<GlobalPtr>(reinterpret_cast<uintptr_t>(p) + off);
   };
   auto row_of = [&](int64_t g, int r) { return g * R + r < M ? g * R + r : M - 1; };
-  // the lane's packs of the rows of group g (zeros beyond the tensor and beyond the row)
-  auto load_group = [&](int64_t g, Pack<T, E> (&px)[R * V]) {
+  // A register set: the lane's packs of the R rows of a group and the rows' first three
+  // elements (the centre of a row's sums is their median: requested with the packs, so
+  // that nothing waits for them later).
+  struct Set {
+    Pack<T, E> px[R * V];
+    T head[R][3];
+  };
+  auto load_group = [&](int64_t g, Set& s) {
+    const int i1 = N > 1 ? 1 : 0, i2 = N > 2 ? 2 : 0;
 #pragma unroll
     for (int r = 0; r < R; ++r) {
       const int64_t row = g * R + r;
+      if constexpr (!RMS) {
+        const T* xr = x + row_of(g, r) * (int64_t)N;
+        s.head[r][0] = xr[0];
+        s.head[r][1] = xr[i1];
+        s.head[r][2] = xr[i2];
+      }
 #pragma unroll
       for (int k = 0; k < V; ++k) {
-        px[r * V + k] = Pack<T, E>::zero();
+        s.px[r * V + k] = Pack<T, E>::zero();
         if (pk0 + k * BLOCK < npacks && row < M)
-          px[r * V + k] = Pack<T, E>::load_stream(at(x + row * (int64_t)N + k * BLOCK * E, loff));
+          s.px[r * V + k] = Pack<T, E>::load_stream(at(x + row * (int64_t)N + k * BLOCK * E, loff));
       }
     }
   };
+  // (split_row_centre of the row, from the elements the set holds)
+  auto centre = [&](const Set& s, int r) {
+    if constexpr (RMS) return 0.0f;
+    const float a = (float)s.head[r][0], b = (float)s.head[r][1], cc = (float)s.head[r][2];
+    return fmaxf(fminf(a, b), fminf(fmaxf(a, b), cc));
+  };
   // mean = hi + lo and rstd of a row from its centred sums (see the split-row kernels)
-  auto set_stats = [&](int r, double t1, double t2, double kd) {
+  auto set_stats = [&](int par, int r, double t1, double t2, double kd) {
     if constexpr (RMS) {
-      stat[r][0] = 0.0f;
-      stat[r][1] = 0.0f;
-      stat[r][2] = (float)(1.0 / sqrt(t2 / dN + (double)eps));
+      stat[par][r][0] = 0.0f;
+      stat[par][r][1] = 0.0f;
+      stat[par][r][2] = (float)(1.0 / sqrt(t2 / dN + (double)eps));
     } else {
       const double m1 = t1 / dN;
       const double mu = kd + m1;
       double var = (t2 - t1 * m1) / dN;
       var = var < 0.0 ? 0.0 : var;  // (a select: NaN stays NaN)
       const float hi = (float)mu;
-      stat[r][0] = var == var ? hi : (float)var;  // NaN variance: NaN mean
-      stat[r][1] = (float)(mu - (double)hi);
-      stat[r][2] = (float)(1.0 / sqrt(var + (double)eps));
+      stat[par][r][0] = var == var ? hi : (float)var;  // NaN variance: NaN mean
+      stat[par][r][1] = (float)(mu - (double)hi);
+      stat[par][r][2] = (float)(1.0 / sqrt(var + (double)eps));
     }
   };
-  // The centred float64 sums of the rows of group g (held in px), published as round `round`.
-  auto sums_and_publish = [&](int64_t g, unsigned int round, Pack<T, E> (&px)[R * V]) {
+  // First wavefront, at the start of a round: the sums of group g (in set s, published a
+  // round ago) across the team and its statistics, for the threads behind the round's
+  // barrier; then the wavefront's request of group g2 into s2 -- only now: the exchange
+  // waits for everything the wavefront has outstanding, and a request made before it would
+  // put the machine's whole burst of loads in its way.
+  auto gather = [&](int64_t g, unsigned int round, const Set& s, int64_t g2, Set& s2) {
+    const int par = (int)(round & 1u);
+    double tot[K];
+    const bool complete =
+        team_gather_sums_f64<K>(slot, slot->entry[round & 3u] + tm * team, team, call_id, round,
+                                wait_ticks, tot);
+    if (threadIdx.x == 0) {
+      failed[par] = complete ? 0 : 1;
+      if (complete) {
+#pragma unroll
+        for (int r = 0; r < R; ++r) set_stats(par, r, tot[2 * r], tot[2 * r + 1], (double)centre(s, r));
+      }
+    }
+    if (g2 >= 0) load_group(g2, s2);
+  };
+  // The centred float64 sums of the rows of group g (held in s), published as round `round`
+  // by the first thread of the second wavefront while the others go on (the first
+  // wavefront gathers: the two halves of the exchange do not queue behind each other).
+  // Every thread passes one barrier.
+  constexpr int kPublisher = 64;
+  auto sums_and_publish = [&](int64_t g, unsigned int round, Set& s) {
     TeamEntry* mine = &slot->entry[round & 3u][blockIdx.x];
-    if (threadIdx.x == 0) team_store(&mine->tag, 0ull);
+    double* rd = red[round & 1u];
+    if (threadIdx.x == kPublisher) team_store(&mine->tag, 0ull);
     double acc[K];
 #pragma unroll
     for (int r = 0; r < R; ++r) {
-      const float kf = RMS ? 0.0f : split_row_centre(x + row_of(g, r) * (int64_t)N, (const T*)nullptr, N);
+      const float kf = centre(s, r);
       const double kd = (double)kf;
       double s1 = 0.0, s2 = 0.0;
 #pragma unroll
       for (int k = 0; k < V; ++k) {
-        keep_packed(px[r * V + k]);
+        keep_packed(s.px[r * V + k]);
         // (a pack beyond the row or the tensor holds zeros, which are not x - k = 0)
         if (pk0 + k * BLOCK < npacks && g * R + r < M)
-          add_centred_sums<T, E, RMS, true>(px[r * V + k], E, kf, kd, s1, s2);
+          add_centred_sums<T, E, RMS, true>(s.px[r * V + k], E, kf, kd, s1, s2);
       }
       acc[2 * r] = s1;
       acc[2 * r + 1] = s2;
     }
-    // over the workgroup, in a fixed order; thread 0 holds the result
+    // over the workgroup, in a fixed order; the publisher holds the result
 #pragma unroll
     for (int k = 0; k < K; ++k) {
 #pragma unroll
@@ -1366,49 +1412,26 @@ norm_fwd_rows_team_kernel(const T* __restrict__ x, const WT* __restrict__ gamma,
     const int wave = threadIdx.x >> 6;
     if ((threadIdx.x & 63) == 0) {
 #pragma unroll
-      for (int k = 0; k < K; ++k) red[wave * K + k] = acc[k];
+      for (int k = 0; k < K; ++k) rd[wave * K + k] = acc[k];
     }
     __syncthreads();
-    if (threadIdx.x == 0) {
+    if (threadIdx.x == kPublisher) {
 #pragma unroll
       for (int k = 0; k < K; ++k) {
-        double t = red[k];
+        double t = rd[k];
 #pragma unroll
-        for (int w = 1; w < BLOCK / 64; ++w) t += red[w * K + k];
+        for (int w = 1; w < BLOCK / 64; ++w) t += rd[w * K + k];
         acc[k] = t;
       }
       team_publish_f64<K>(mine, call_id, round, acc);
     }
   };
-  // The sums of group g across the team, its statistics, its Y.  (g1 / p1, g2 / p2: the groups
-  // held in the other two register sets, loaded again after the rare pass over whole rows so
-  // that nothing stays live across that pass; the first wavefront requests g2 only here,
-  // behind its gather: the exchange waits for everything the wavefront has outstanding, and
-  // a request made before it would put the machine's whole burst of loads in its way.)
-  auto finish = [&](int64_t g, unsigned int round, Pack<T, E> (&px)[R * V], int64_t g1,
-                    Pack<T, E> (&p1)[R * V], int64_t g2, Pack<T, E> (&p2)[R * V]) {
-    // (every thread has read the stat[] of the round before and thread 0 its red[])
-    __syncthreads();
-    if (threadIdx.x < 64) {  // the first wavefront waits and adds up
-      double tot[K];
-      const bool complete =
-          team_gather_sums_f64<K>(slot, slot->entry[round & 3u] + tm * team, team, call_id, round,
-                                  wait_ticks, tot);
-      if (threadIdx.x == 0) {
-        failed = complete ? 0 : 1;
-        if (complete) {
-#pragma unroll
-          for (int r = 0; r < R; ++r) {
-            const float kf =
-                RMS ? 0.0f : split_row_centre(x + row_of(g, r) * (int64_t)N, (const T*)nullptr, N);
-            set_stats(r, tot[2 * r], tot[2 * r + 1], (double)kf);
-          }
-        }
-      }
-      if (complete && g2 >= 0) load_group(g2, p2);
-    }
-    __syncthreads();
-    if (failed != 0) {  // (uniform over the workgroup)
+  // Y of group g (set s) from the statistics its round's gather left.  (g1 / s1, g2 / s2:
+  // the groups of the other two sets, loaded again after the rare pass over whole rows so
+  // that nothing stays live across that pass.)
+  auto write = [&](int64_t g, unsigned int round, Set& s, int64_t g1, Set& s1, int64_t g2, Set& s2) {
+    const int par = (int)(round & 1u);
+    if (failed[par] != 0) {  // (uniform over the workgroup)
       // The team did not come together: the sums over the whole rows (X, which no
       // workgroup writes), then the packs again.
       for (int r = 0; r < R; ++r) {
@@ -1417,18 +1440,18 @@ norm_fwd_rows_team_kernel(const T* __restrict__ x, const WT* __restrict__ gamma,
         double w1 = 0.0, w2 = 0.0;
         long_row_sums<T, E, BLOCK, RMS, false>(xr, (const T*)nullptr, N, 0, npacks, kf, w1, w2);
         __syncthreads();  // (red[] of the sum before has been read)
-        block_sum2_f64<BLOCK>(w1, w2, red);
-        if (threadIdx.x == 0) set_stats(r, w1, w2, (double)kf);
+        block_sum2_f64<BLOCK>(w1, w2, red[0]);
+        if (threadIdx.x == 0) set_stats(par, r, w1, w2, (double)kf);
       }
       __syncthreads();
-      load_group(g, px);
-      load_group(g1 >= 0 ? g1 : M, p1);  // (a group beyond the tensor: zeros)
-      load_group(g2 >= 0 ? g2 : M, p2);
+      load_group(g, s);
+      load_group(g1 >= 0 ? g1 : M, s1);  // (a group beyond the tensor: zeros)
+      load_group(g2 >= 0 ? g2 : M, s2);
     }
 #pragma unroll
     for (int r = 0; r < R; ++r) {
       const int64_t row = g * R + r;
-      const float hi = stat[r][0], lo = stat[r][1], rs = stat[r][2];
+      const float hi = stat[par][r][0], lo = stat[par][r][1], rs = stat[par][r][2];
 #pragma unroll
       for (int k = 0; k < V; ++k) {
         const bool held = pk0 + k * BLOCK < npacks;
@@ -1445,9 +1468,9 @@ norm_fwd_rows_team_kernel(const T* __restrict__ x, const WT* __restrict__ gamma,
         for (int i = 0; i < E; ++i) {
           float v;
           if constexpr (RMS)
-            v = (px[r * V + k].get(i) * rs) * gk.get(i);
+            v = (s.px[r * V + k].get(i) * rs) * gk.get(i);
           else
-            v = (((px[r * V + k].get(i) - hi) - lo) * rs) * gk.get(i) + pb[k].get(i);
+            v = (((s.px[r * V + k].get(i) - hi) - lo) * rs) * gk.get(i) + pb[k].get(i);
           o.set(i, v);
         }
         if (held && row < M) o.store_stream(at(y + row * (int64_t)N + k * BLOCK * E, loff));
@@ -1461,39 +1484,45 @@ norm_fwd_rows_team_kernel(const T* __restrict__ x, const WT* __restrict__ gamma,
       }
     }
   };
-
-  // Group j of the team (tm + j * teams) lives in register set j % 3: requested at the start
-  // of round j - 2, summed and published in round j - 1, gathered and written in round j.
-  Pack<T, E> ax[R * V], bx[R * V], cx[R * V];
-  const bool later = threadIdx.x < 64;  // the exchanging wavefront requests inside finish()
+  // One round: group g in set a (published a round ago) is gathered by the first wavefront
+  // while the others request group g + 2 teams into set c and sum group g + teams in set
+  // b; behind the barrier of that sum one thread publishes it and everyone writes Y of g.
+  const bool first = threadIdx.x < 64;
   const int64_t st = teams;
+  auto valid = [&](int64_t q) { return q < ngroups ? q : (int64_t)-1; };
+  auto one_round = [&](int64_t g, unsigned int round, Set& a, Set& b, Set& cs) {
+    const int64_t g1 = valid(g + st), g2 = valid(g + 2 * st);
+    if (first)
+      gather(g, round, a, g2, cs);
+    else if (g2 >= 0)
+      load_group(g2, cs);
+    if (g1 >= 0)
+      sums_and_publish(g1, round + 1, b);
+    else
+      __syncthreads();  // (the statistics of this round, for every thread)
+    write(g, round, a, g1, b, g2, cs);
+  };
+
+  // Group j of the team (tm + j * teams) lives in register set j % 3: requested in round
+  // j - 2, summed and published in round j - 1, gathered and written in round j.
+  Set sa, sb, sc;
   int64_t g = tm;
   unsigned int round = 0;
   if (g < ngroups) {
-    load_group(g, ax);
-    if (g + st < ngroups) load_group(g + st, bx);
-    sums_and_publish(g, 0, ax);
+    load_group(g, sa);
+    if (g + st < ngroups) load_group(g + st, sb);
+    sums_and_publish(g, 0, sa);
   }
-  auto valid = [&](int64_t q) { return q < ngroups ? q : (int64_t)-1; };
   while (g < ngroups) {
-    // (a, b, c) = (ax, bx, cx)
-    if (g + 2 * st < ngroups && !later) load_group(g + 2 * st, cx);
-    if (g + st < ngroups) sums_and_publish(g + st, round + 1, bx);
-    finish(g, round, ax, valid(g + st), bx, valid(g + 2 * st), cx);
+    one_round(g, round, sa, sb, sc);
     g += st;
     ++round;
     if (g >= ngroups) break;
-    // (a, b, c) = (bx, cx, ax)
-    if (g + 2 * st < ngroups && !later) load_group(g + 2 * st, ax);
-    if (g + st < ngroups) sums_and_publish(g + st, round + 1, cx);
-    finish(g, round, bx, valid(g + st), cx, valid(g + 2 * st), ax);
+    one_round(g, round, sb, sc, sa);
     g += st;
     ++round;
     if (g >= ngroups) break;
-    // (a, b, c) = (cx, ax, bx)
-    if (g + 2 * st < ngroups && !later) load_group(g + 2 * st, bx);
-    if (g + st < ngroups) sums_and_publish(g + st, round + 1, ax);
-    finish(g, round, cx, valid(g + st), ax, valid(g + 2 * st), bx);
+    one_round(g, round, sc, sa, sb);
     g += st;
     ++round;
   }
@@ -2689,7 +2718,6 @@ norm_bwd_team_kernel(const T* __restrict__ dy, const T* __restrict__ x,
   auto sums_and_publish = [&](int64_t g, unsigned int round, Pack<T, E> (&pd)[R * V],
                               Pack<T, E> (&px)[R * V]) {
     TeamEntry* mine = &slot->entry[round & 3u][blockIdx.x];
-    if (threadIdx.x == 0) team_store(&mine->tag, 0ull);
     float acc[2 * R];
 #pragma unroll
     for (int r = 0; r < R; ++r) acc[2 * r] = acc[2 * r + 1] = 0.0f;
@@ -2712,7 +2740,7 @@ norm_bwd_team_kernel(const T* __restrict__ dy, const T* __restrict__ x,
       }
     }
     group_allreduce<BLOCK, BLOCK, 2 * R, SumOp>(acc, red, phase);
-    if (threadIdx.x == 0) team_publish_words<R>(mine, call_id, round, acc);
+    if (threadIdx.x == 0) team_publish_tagged<2 * R>(mine, call_id, round, acc);
   };
   // The sums of group g (published as round `round`) across the team, its dX, its share of
   // the column sums; each pack's registers are given to the same pack of group gn (< 0:
@@ -2727,8 +2755,8 @@ norm_bwd_team_kernel(const T* __restrict__ dy, const T* __restrict__ x,
     if (threadIdx.x < 64) {  // the first wavefront waits and adds up
       float tot[2 * R];
       const bool complete =
-          team_gather_sums<R>(slot, slot->entry[round & 3u] + tm * team, team, call_id, round,
-                              wait_ticks, tot);
+          team_gather_tagged<2 * R>(slot, slot->entry[round & 3u] + tm * team, team, call_id,
+                                    round, wait_ticks, tot);
       if (threadIdx.x == 0) {
 #pragma unroll
         for (int k = 0; k < 2 * R; ++k) stat[k] = tot[k];
