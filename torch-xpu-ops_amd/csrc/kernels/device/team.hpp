@@ -5,18 +5,21 @@
 // a round of other work between publishing and gathering) and a lighter one of
 // self-validating words for float32 values (norm_bwd_team_kernel).
 //
-// What crosses workgroups.  An entry is {tag, s1, s2}, 128 bytes apart; the tag of a
-// finished entry is (call id << 32) | (round + 1), ids being unique per call, so
-// nothing has to be cleared and an entry left by an earlier call or round never
-// counts.  The writer sets the tag to 0 when it starts on a row, later stores s1
-// and s2, waits for those stores to be acknowledged and stores the tag; a reader
-// accepts s1 and s2 only if it read the expected tag before and after them.  Every
-// access is a device-scope atomic store or load, which goes to memory: no
-// read-modify-write (256 workgroups counting on one word took hundreds of
-// microseconds), and no release or acquire fence (each writes back or invalidates a
-// whole L2).  Two calls that were handed the same slot while both run -- possible
-// only with more such calls in flight than slots -- overwrite each other's tags and
-// therefore never accept each other's numbers.
+// What crosses workgroups.  An entry is 128 bytes (neighbours' polls go to other memory
+// channels).  The two-number exchange (team_publish_and_gather) uses {tag, s1, s2}: the tag
+// of a finished entry is (call id << 32) | (round + 1), ids being unique per call, so nothing
+// has to be cleared and an entry left by an earlier call or round never counts.  The writer
+// sets the tag to 0 when it starts on a row, later stores s1 and s2, waits for those stores
+// to be acknowledged and stores the tag; a reader accepts s1 and s2 only if it read the
+// expected tag before and after them.  The exchanges in two halves further down write
+// self-validating 64-bit words {32 bits of payload, tag} into the entry's pad[] instead: a
+// word is valid or not by itself, so the writer orders nothing and waits for nothing and a
+// reader needs one round trip (see team_publish_tagged).  Every access is a device-scope
+// atomic store or load, which goes to memory: no read-modify-write (256 workgroups
+// counting on one word took hundreds of microseconds), and no release or acquire fence
+// (each writes back or invalidates a whole L2).  Two calls that were handed the same slot
+// while both run -- possible only with more such calls in flight than slots -- overwrite
+// each other's tags and therefore never accept each other's numbers.
 //
 // The wait is bounded, and no workgroup depends on another to finish.  A workgroup
 // stops waiting when its team is complete, when any workgroup of the call has given
@@ -44,6 +47,32 @@ __device__ __forceinline__ void team_store(unsigned long long* p, unsigned long 
 __device__ __forceinline__ void team_stores_done() {
   asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
 }
+
+// team_word_tag: the tag every word of the exchanges below carries -- ((call id mod 2^25 - 1)
+// + 1) << 6 | (round mod 64): never 0 (the memory starts as zeros), different for the rounds
+// that share a buffer, different from call to call; bit 31 is clear.
+//
+// A workgroup that has stopped waiting for its team (`lost`) never publishes a valid word
+// again: its words carry team_lost_tag -- the call's tag with bit 31 set, whatever the round
+// -- and a gather that meets one gives up at once.  So the rest of its team follows it
+// promptly, and -- tags repeat after 64 rounds -- nothing a workgroup writes while it runs
+// ahead of its team on its own can be taken for the numbers of an earlier round.  The
+// slot's hint word spreads the news to the other teams of the call, which look at it now
+// and then.
+__device__ __forceinline__ unsigned int team_word_tag(unsigned int call_id, unsigned int round) {
+  return ((call_id % 0x1ffffffu) + 1u) << 6 | (round & 63u);
+}
+__device__ __forceinline__ unsigned int team_lost_tag(unsigned int call_id) {
+  return 0x80000000u | team_word_tag(call_id, 0);
+}
+// (whether a word's tag is the call's lost tag)
+__device__ __forceinline__ bool team_tag_is_lost(unsigned int tag, unsigned int call_id) {
+  return (tag | 63u) == (team_lost_tag(call_id) | 63u);
+}
+
+// (A lane's entries are read four at a time: a round trip to memory for a team of up to 256,
+// however many entries a lane has.)
+constexpr int kTeamGatherBatch = 4;
 
 // For the first wavefront of a workgroup (all 64 lanes, threadIdx.x < 64), whose entry
 // `entries[blockIdx.x]` has had the tag 0 since the workgroup started on the row:
@@ -99,34 +128,23 @@ __device__ __forceinline__ bool team_publish_and_gather(TeamSlot* slot, TeamEntr
   return complete;
 }
 
-// (A lane's entries are read four at a time: a round trip to memory for a team of up to 256,
-// however many entries a lane has.)
-constexpr int kTeamGatherBatch = 4;
-
-// A lighter exchange for float32 values: every 64-bit word carries its own tag, so a word is
-// valid or not by itself and neither side orders anything.  Word k of an entry holds
-// {v[k], tag}, tag = ((call id mod 2^26 - 1) + 1) << 6 | (round mod 64): never 0 (the memory
-// starts as zeros), different for the rounds that share a buffer (a buffer is reused every
-// fourth round, and workgroups of a team whose gathers succeed are never more than three
-// rounds apart), different from call to call.  The words live in an entry's pad[], which no
-// other exchange writes: whatever a word holds was put there by this one.  Publishing is K
-// plain stores with nothing to
-// wait for.  Gathering reads every word of a lane's entries in one round trip, accepts them
-// if every tag is the round's, and then -- a second round trip, after the words have
-// returned -- makes sure no workgroup of the call has given up: a workgroup that no longer
-// waits for its team can be any number of rounds ahead, tags repeat after 64 rounds, and
-// it records that it gave up (and waits for that store) before it goes on, so words it
-// writes later are never accepted by a gather that still saw the record unset.
-__device__ __forceinline__ unsigned int team_word_tag(unsigned int call_id, unsigned int round) {
-  return ((call_id % 0x3ffffffu) + 1u) << 6 | (round & 63u);
-}
-
+// The exchange in two halves, for kernels that put other work between them; float32 values.
+// Every 64-bit word carries its own tag, so a word is valid or not by itself and neither
+// side orders anything.  Word k of an entry holds {v[k], tag}, tag = team_word_tag():
+// different for the rounds that share a buffer (a buffer is reused every second or fourth
+// round, and workgroups of a team whose gathers succeed are never more than three rounds
+// apart), different from call to call.  The words live in an entry's pad[], which nothing
+// else writes: whatever a word holds was put there by one of these exchanges.  Publishing
+// is K plain stores with nothing to wait for; gathering reads every word of a lane's entries
+// in one round trip and accepts them if every tag is the round's.  `lost`: see team_word_tag.
 template <int K>
 __device__ __forceinline__ void team_publish_tagged(TeamEntry* mine, unsigned int call_id,
-                                                    unsigned int round, const float (&v)[K]) {
+                                                    unsigned int round, const float (&v)[K],
+                                                    bool lost) {
   static_assert(K >= 1 && K <= 13, "an entry's pad[] holds 13 words");
   unsigned long long* words = &mine->pad[0];
-  const unsigned long long tag = (unsigned long long)team_word_tag(call_id, round) << 32;
+  const unsigned long long tag =
+      (unsigned long long)(lost ? team_lost_tag(call_id) : team_word_tag(call_id, round)) << 32;
 #pragma unroll
   for (int k = 0; k < K; ++k)
     team_store(&words[k], tag | (unsigned long long)__builtin_bit_cast(unsigned int, v[k]));
@@ -134,20 +152,21 @@ __device__ __forceinline__ void team_publish_tagged(TeamEntry* mine, unsigned in
 
 // For the first wavefront of a workgroup (all 64 lanes).  On success v[] holds the sums over
 // the team, added in a fixed order (entries lane, lane + 64, ... per lane, then across the
-// lanes): the same bits in every lane and in every workgroup of the team.  False when the
-// wait ran out or a workgroup of the call has given up (recorded in the slot, and the store
-// waited for, before this returns).
+// lanes): the same bits in every lane and in every workgroup of the team.  False as in
+// team_publish_and_gather; the workgroup publishes as `lost` from then on.
 template <int K>
-__device__ __forceinline__ bool team_gather_tagged(TeamSlot* slot, const TeamEntry* mates, int team,
-                                                   unsigned int call_id, unsigned int round,
+__device__ __forceinline__ bool team_gather_tagged(TeamSlot* slot, const TeamEntry* mates,
+                                                   int team, unsigned int call_id,
+                                                   unsigned int round,
                                                    unsigned long long wait_ticks, float (&v)[K]) {
   constexpr int B = kTeamGatherBatch;
   const int lane = (int)threadIdx.x;
   const unsigned int expect = team_word_tag(call_id, round);
   const unsigned long long t0 = wall_clock64();
   bool complete = false;
+  unsigned int polls = 0;
   for (;;) {
-    bool ok = true;
+    bool ok = true, lost_seen = false;
 #pragma unroll
     for (int k = 0; k < K; ++k) v[k] = 0.0f;
     for (int j0 = lane; j0 < team; j0 += 64 * B) {
@@ -155,9 +174,13 @@ __device__ __forceinline__ bool team_gather_tagged(TeamSlot* slot, const TeamEnt
 #pragma unroll
       for (int b = 0; b < B; ++b) {
         const int j = j0 + 64 * b;
-        const unsigned long long* words = &mates[j < team ? j : 0].pad[0];
 #pragma unroll
-        for (int k = 0; k < K; ++k) w[b][k] = team_load(&words[k]);
+        for (int k = 0; k < K; ++k) w[b][k] = 0;
+        if (j < team) {
+          const unsigned long long* words = &mates[j].pad[0];
+#pragma unroll
+          for (int k = 0; k < K; ++k) w[b][k] = team_load(&words[k]);
+        }
       }
 #pragma unroll
       for (int b = 0; b < B; ++b) {
@@ -165,48 +188,50 @@ __device__ __forceinline__ bool team_gather_tagged(TeamSlot* slot, const TeamEnt
 #pragma unroll
           for (int k = 0; k < K; ++k) {
             ok = ok && (unsigned int)(w[b][k] >> 32) == expect;
+            lost_seen = lost_seen || team_tag_is_lost((unsigned int)(w[b][k] >> 32), call_id);
             v[k] += __builtin_bit_cast(float, (unsigned int)(w[b][k] & 0xffffffffull));
           }
         }
       }
     }
-    const unsigned int hint =
-        __hip_atomic_load(&slot->gave_up, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
-    if (hint == call_id) break;
+    if (__ballot(lost_seen) != 0) break;
     if (__ballot(ok) == __ballot(true)) {
-      // (the record is read again only now that the words have returned)
-      team_stores_done();
-      const unsigned int after =
-          __hip_atomic_load(&slot->gave_up, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
-      if (after == call_id) break;
 #pragma unroll
       for (int k = 0; k < K; ++k) v[k] = wave_group_allreduce<64, SumOp>(v[k]);
       complete = true;
       break;
     }
+    // (the hint word is one address for the whole grid: looked at every 16th time)
+    if ((polls++ & 15u) == 0) {
+      const unsigned int hint =
+          __hip_atomic_load(&slot->gave_up, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+      if (hint == call_id) break;
+    }
     if (wall_clock64() - t0 > wait_ticks) break;
     __builtin_amdgcn_s_sleep(8);
   }
-  if (!complete) {
-    if (lane == 0)
-      __hip_atomic_store(&slot->gave_up, call_id, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
-    team_stores_done();
-  }
+  if (!complete && lane == 0)
+    __hip_atomic_store(&slot->gave_up, call_id, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
   return complete;
 }
 
-// The same two halves with K float64 values a workgroup (K <= 15), summed over the team in
-// the same fixed order as team_gather_tagged.
+// The same two halves for K float64 values a workgroup (K <= 6), each cut into two words
+// {32 bits, tag} of pad[] as in team_publish_and_gather, summed over the team in the fixed
+// order of team_gather_tagged.
 template <int K>
 __device__ __forceinline__ void team_publish_f64(TeamEntry* mine, unsigned int call_id,
-                                                 unsigned int round, const double (&v)[K]) {
-  static_assert(K >= 1 && K <= 15, "an entry holds a tag and 15 words");
-  unsigned long long* words = &mine->s1;
-  team_stores_done();  // the tag has been 0 in memory before the numbers change
+                                                 unsigned int round, const double (&v)[K],
+                                                 bool lost) {
+  static_assert(K >= 1 && 2 * K <= 13, "an entry's pad[] holds 13 words");
+  unsigned long long* words = &mine->pad[0];
+  const unsigned long long tag =
+      (unsigned long long)(lost ? team_lost_tag(call_id) : team_word_tag(call_id, round)) << 32;
 #pragma unroll
-  for (int k = 0; k < K; ++k) team_store(&words[k], __builtin_bit_cast(unsigned long long, v[k]));
-  team_stores_done();
-  team_store(&mine->tag, ((unsigned long long)call_id << 32) | (round + 1u));
+  for (int k = 0; k < K; ++k) {
+    const unsigned long long bits = __builtin_bit_cast(unsigned long long, v[k]);
+    team_store(&words[2 * k], tag | (bits & 0xffffffffull));
+    team_store(&words[2 * k + 1], tag | (bits >> 32));
+  }
 }
 
 template <int K>
@@ -217,49 +242,42 @@ __device__ __forceinline__ bool team_gather_sums_f64(TeamSlot* slot, const TeamE
                                                      double (&v)[K]) {
   constexpr int B = kTeamGatherBatch;
   const int lane = (int)threadIdx.x;
-  const unsigned long long expect = ((unsigned long long)call_id << 32) | (round + 1u);
+  const unsigned int expect = team_word_tag(call_id, round);
   const unsigned long long t0 = wall_clock64();
   bool complete = false;
   unsigned int polls = 0;
   for (;;) {
-    bool ok = true;
+    bool ok = true, lost_seen = false;
 #pragma unroll
     for (int k = 0; k < K; ++k) v[k] = 0.0;
-    for (int j0 = lane; j0 < team && ok; j0 += 64 * B) {
-      unsigned long long tag0[B], tag1[B], w[B][K];
+    for (int j0 = lane; j0 < team; j0 += 64 * B) {
+      unsigned long long w[B][2 * K];
 #pragma unroll
       for (int b = 0; b < B; ++b) {
         const int j = j0 + 64 * b;
-        tag0[b] = j < team ? team_load(&mates[j].tag) : expect;
-      }
 #pragma unroll
-      for (int b = 0; b < B; ++b) ok = ok && tag0[b] == expect;
-      if (__ballot(ok) != __ballot(true)) {
-        ok = false;
-        break;
-      }
+        for (int k = 0; k < 2 * K; ++k) w[b][k] = 0;
+        if (j < team) {
+          const unsigned long long* words = &mates[j].pad[0];
 #pragma unroll
-      for (int b = 0; b < B; ++b) {
-        const int j = j0 + 64 * b;
-        const unsigned long long* words = &mates[j < team ? j : 0].s1;
-#pragma unroll
-        for (int k = 0; k < K; ++k) w[b][k] = team_load(&words[k]);
-      }
-      team_stores_done();  // the numbers have returned before the tags are read again
-#pragma unroll
-      for (int b = 0; b < B; ++b) {
-        const int j = j0 + 64 * b;
-        tag1[b] = j < team ? team_load(&mates[j].tag) : expect;
+          for (int k = 0; k < 2 * K; ++k) w[b][k] = team_load(&words[k]);
+        }
       }
 #pragma unroll
       for (int b = 0; b < B; ++b) {
-        ok = ok && tag1[b] == expect;
         if (j0 + 64 * b < team) {
 #pragma unroll
-          for (int k = 0; k < K; ++k) v[k] += __builtin_bit_cast(double, w[b][k]);
+          for (int k = 0; k < K; ++k) {
+            ok = ok && (unsigned int)(w[b][2 * k] >> 32) == expect &&
+                 (unsigned int)(w[b][2 * k + 1] >> 32) == expect;
+            lost_seen = lost_seen || team_tag_is_lost((unsigned int)(w[b][2 * k] >> 32), call_id);
+            v[k] += __builtin_bit_cast(double,
+                                       (w[b][2 * k] & 0xffffffffull) | (w[b][2 * k + 1] << 32));
+          }
         }
       }
     }
+    if (__ballot(lost_seen) != 0) break;
     if (__ballot(ok) == __ballot(true)) {
 #pragma unroll
       for (int k = 0; k < K; ++k) {
@@ -278,7 +296,7 @@ __device__ __forceinline__ bool team_gather_sums_f64(TeamSlot* slot, const TeamE
     if (wall_clock64() - t0 > wait_ticks) break;
     __builtin_amdgcn_s_sleep(8);
   }
-  if (lane == 0 && !complete)
+  if (!complete && lane == 0)
     __hip_atomic_store(&slot->gave_up, call_id, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
   return complete;
 }

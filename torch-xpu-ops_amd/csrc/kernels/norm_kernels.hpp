@@ -1276,6 +1276,8 @@ norm_fwd_rows_team_kernel(const T* __restrict__ x, const WT* __restrict__ gamma,
   __shared__ double red[2][(BLOCK / 64) * K];
   __shared__ float stat[2][R][3];  // a row's mean (hi, lo) and rstd
   __shared__ int failed[2];
+  __shared__ int lost;  // the workgroup has stopped waiting for its team (see team_word_tag)
+  if (threadIdx.x == 0) lost = 0;  // (read behind the barrier of the first sum at the earliest)
   // from five packs a lane on gamma lives in LDS (a pack a lane and k), not in registers
   constexpr bool GL = V > 4;
   __shared__ Pack<WT, E> gl[GL ? V : 1][GL ? BLOCK : 1];
@@ -1371,6 +1373,7 @@ norm_fwd_rows_team_kernel(const T* __restrict__ x, const WT* __restrict__ gamma,
                                 wait_ticks, tot);
     if (threadIdx.x == 0) {
       failed[par] = complete ? 0 : 1;
+      if (!complete) lost = 1;
       if (complete) {
 #pragma unroll
         for (int r = 0; r < R; ++r) set_stats(par, r, tot[2 * r], tot[2 * r + 1], (double)centre(s, r));
@@ -1386,7 +1389,6 @@ norm_fwd_rows_team_kernel(const T* __restrict__ x, const WT* __restrict__ gamma,
   auto sums_and_publish = [&](int64_t g, unsigned int round, Set& s) {
     TeamEntry* mine = &slot->entry[round & 3u][blockIdx.x];
     double* rd = red[round & 1u];
-    if (threadIdx.x == kPublisher) team_store(&mine->tag, 0ull);
     double acc[K];
 #pragma unroll
     for (int r = 0; r < R; ++r) {
@@ -1423,7 +1425,7 @@ norm_fwd_rows_team_kernel(const T* __restrict__ x, const WT* __restrict__ gamma,
         for (int w = 1; w < BLOCK / 64; ++w) t += rd[w * K + k];
         acc[k] = t;
       }
-      team_publish_f64<K>(mine, call_id, round, acc);
+      team_publish_f64<K>(mine, call_id, round, acc, lost != 0);
     }
   };
   // Y of group g (set s) from the statistics its round's gather left.  (g1 / s1, g2 / s2:
@@ -2672,6 +2674,7 @@ norm_bwd_team_kernel(const T* __restrict__ dy, const T* __restrict__ x,
   // for dgamma, behind them the same for dbeta
   __shared__ Pack<float, 4> colsum[(RMS ? 1 : 2) * V * Q][BLOCK];
   int phase = 0;
+  bool lost = false;  // (first wavefront) the workgroup has stopped waiting for its team
   const int tm = (int)blockIdx.x / team;
   const int c = (int)blockIdx.x - tm * team;
   const int teams = (int)gridDim.x / team;
@@ -2740,7 +2743,7 @@ norm_bwd_team_kernel(const T* __restrict__ dy, const T* __restrict__ x,
       }
     }
     group_allreduce<BLOCK, BLOCK, 2 * R, SumOp>(acc, red, phase);
-    if (threadIdx.x == 0) team_publish_tagged<2 * R>(mine, call_id, round, acc);
+    if (threadIdx.x == 0) team_publish_tagged<2 * R>(mine, call_id, round, acc, lost);
   };
   // The sums of group g (published as round `round`) across the team, its dX, its share of
   // the column sums; each pack's registers are given to the same pack of group gn (< 0:
@@ -2757,6 +2760,7 @@ norm_bwd_team_kernel(const T* __restrict__ dy, const T* __restrict__ x,
       const bool complete =
           team_gather_tagged<2 * R>(slot, slot->entry[round & 3u] + tm * team, team, call_id,
                                     round, wait_ticks, tot);
+      lost = lost || !complete;
       if (threadIdx.x == 0) {
 #pragma unroll
         for (int k = 0; k < 2 * R; ++k) stat[k] = tot[k];

@@ -103,9 +103,13 @@ constexpr int kTeamFwdLongPacks = 10;
 constexpr int kTeamFwdMinRounds = 16;
 // One call's bookkeeping memory (see the kernel).
 struct TeamEntry {
-  unsigned long long tag;  // (call id << 32) | (round + 1) once s1, s2 are in place; 0 while they change
-  unsigned long long s1, s2;  // a workgroup's partial sums (float64 bit patterns)
-  unsigned long long pad[13];  // 128 bytes an entry: neighbours' polls go to other memory channels
+  // the two-number exchange: (call id << 32) | (round + 1) once s1, s2 are in place, 0 while
+  // they change; a workgroup's partial sums (float64 bit patterns)
+  unsigned long long tag;
+  unsigned long long s1, s2;
+  // the exchanges of self-validating words {32 bits of payload, tag}: see device/team.hpp
+  // (128 bytes an entry: neighbours' polls go to other memory channels)
+  unsigned long long pad[13];
 };
 struct TeamSlot {
   // [round parity][workgroup]; norm_bwd_team_kernel, which publishes a round before it
