@@ -11,8 +11,8 @@ LayerNormKernels.cpp:1218-1406 over Norm.h:632-812) and the long-row shapes of i
 float32 partial sums), against the path a workgroup takes when its wait gives up (forced from the
 host by a wait of zero: no kernel hangs), against the multi-launch kernels (in place, which they
 serve; forced by override), and for run-to-run determinism.  The plan sends a call to teams from
-8 (LayerNorm) or 5 (RMSNorm) rounds of four rows a team on; the small shapes here reach the kernel
-through the override that asks for it whatever the rounds, the last test through the plan itself."""
+the second round of four rows a team on; the shapes here also ask for it by override, whatever the
+rounds, the last test goes through the plan alone."""
 import pytest
 import torch
 
@@ -155,17 +155,17 @@ def _team_backward_cases(cabi, oracle, gpu, dtype, mixed):
 
 def test_team_backward_plans_and_workspace(cabi):
     """The plan of a team backward: whole teams of row_chunks workgroups, at most 256 workgroups,
-    and a workspace that holds one partial row a team of each column sum wanted; fewer than 8
-    (RMSNorm: 5) rounds, or a last workgroup of a row that is mostly idle, keep the multi-launch
-    kernels."""
-    for (M, N, team) in ((512, 401408, True), (4096, 65536, True), (100, 401408, False),
-                         (8192, 24584, False), (1024, 40960, False)):
+    and a workspace that holds one partial row a team of each column sum wanted; a single round
+    (and, for a LayerNorm on teams of more than 64 workgroups, fewer than four) keeps the
+    multi-launch kernels."""
+    for (M, N, ln_team, rms_team) in ((512, 401408, True, True), (4096, 65536, True, True),
+                                      (100, 401408, True, True), (8192, 24584, True, None),
+                                      (16, 1048576, False, True), (16, 401408, False, False)):
         for op, nparts in ((cabi.OP_LAYER_NORM_BWD, 2), (cabi.OP_RMS_NORM_BWD, 1)):
             p = cabi.plan(op, M, N, cabi.BF16, cabi.BF16)
-            if p["resident"]:
+            team = ln_team if op == cabi.OP_LAYER_NORM_BWD else rms_team
+            if p["resident"] or team is None:
                 continue
-            if op == cabi.OP_RMS_NORM_BWD and (M, N) in ((100, 401408), (1024, 40960)):
-                team = True  # (five rounds)
             assert _team_planned(cabi, op, M, N, cabi.BF16, cabi.BF16) == team, (M, N, op, p)
             if not team:
                 continue

@@ -1002,17 +1002,18 @@ inline int make_plan(OpClass oc, int64_t M, int64_t N, int esize, int num_cus, c
     if (team >= 2 && team <= cus) {
       int64_t teams = cus / team;
       if (teams > ngroups) teams = ngroups;
-      // Worth it from a handful of rounds on (a call costs about 28 us beside 9.5 (RMSNorm) to
-      // 11.6 us (LayerNorm) a round, where the two passes of the other kernels cost about
-      // 14.6 us for a round's rows), and where the last workgroup of a row is not mostly idle
-      // (bf16 [8192, 24584], four workgroups a row one of which holds a single pack: 380 us
-      // either way).  Measured, bf16, team / two passes in us: [512, 401408] (26 rounds)
-      // LayerNorm 302 / 360, RMSNorm 257 / 350; [4096, 65536] (64) 381 / 477, 329 / 468;
-      // [256, 1048576] (32) 387 / 518, 331 / 511; [64, 1048576] (8) 115 / 117, 98 / 114;
-      // [1024, 40960] (5) 90 / 81, 76 / 76; [16, 1048576] (2) 41.6 / 35.6, 34.2 / 34.9.
-      const bool rounds_ok = teams >= 1 && ngroups >= (layer_norm ? 8 : 5) * teams;
-      const bool full_ok = 5 * packs >= 4 * team * chunk;
-      if (teams >= 1 && ((rounds_ok && full_ok) || team_bwd_forced)) {
+      // Worth it from the second round on (a call costs about 25 us beside 9.5-10 us a round,
+      // where the two passes of the other kernels cost about 14.6 us for a round's rows); a
+      // LayerNorm on large teams (more than 64 workgroups a row) from the fourth.  Measured,
+      // bf16, LayerNorm / RMSNorm, team against two passes in us: [512, 401408] (26 rounds)
+      // 258 / 243 against 359 / 350; [4096, 65536] (64) 330 / 308 against 478 / 468; [100,
+      // 401408] (5) 66 / 59 against 80 / 75; [1024, 40960] (5) 82 / 72 against 81 / 75; [512,
+      // 65536] (4) 62 / 52 against 68 / 63; [32, 401408] (2) 34 / 29 against 41 / 37; [64,
+      // 262144] (2) 41 / 32 against 41 / 38; [16, 1048576] (2, 128 workgroups a row) 41 / 31
+      // against 35 / 34; [8192, 24584] (a row's last workgroup holds a single pack) 327
+      // against 380.
+      const bool rounds_ok = layer_norm && team > 64 ? ngroups >= 4 * teams : ngroups > teams;
+      if (teams >= 1 && (rounds_ok || team_bwd_forced)) {
         p.team = (int)team;
         p.team_v = kTeamBwdPacks;
         p.team_chunk_packs = chunk;
