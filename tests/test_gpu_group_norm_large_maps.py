@@ -117,3 +117,76 @@ def test_special_slabs_and_channels_that_are_not_whole_packs(cabi, oracle, gpu):
     y, mean, rstd = cabi.group_norm_fwd(x.to(gpu), gg, bg, groups, 1e-5)
     oy, om, orr = oracle.group_norm_fwd(to_np32(x), groups, to_np32(gamma), to_np32(beta), 1e-5)
     assert_close(y, oy, torch.bfloat16, "channels of 2048.5 packs")
+
+
+# (N, C, HxW, groups) for the backward: 64 slabs of 8 channels of 2048 packs (bf16: four packs a
+# lane, a workgroup a channel); slabs of 8 channels of 4097 packs (two workgroups a channel, the
+# second nearly empty: the multi-launch kernels keep them) and of 6000 packs (two workgroups a
+# channel, the second ragged); 16 slabs of 8 channels of 16384 packs (four workgroups a channel,
+# 32 a slab); one group of 3 channels of 300 packs in fp32 terms (one pack a lane, idle lanes)
+BWD_SHAPES = [(2, 256, 16384, 32), (2, 16, 4097 * 8, 2), (3, 16, 6000 * 8, 2), (1, 128, 131072, 16),
+              (5, 3, 2400, 1)]
+
+
+@pytest.mark.parametrize("dtype", [torch.float32, torch.float16, torch.bfloat16], ids=str)
+@pytest.mark.parametrize("mixed", [False, True], ids=["w_same", "w_fp32"])
+def test_team_backward_against_oracle_and_the_give_up_path(cabi, oracle, gpu, dtype, mixed):
+    """native_group_norm_backward on slabs beyond one workgroup's registers whose channels are
+    whole packs: gn_bwd_team_kernel holds a slab in the registers of a team of workgroups, one or
+    several a channel, the channel sums cross the team once, dY and X are read once (the
+    reference: two kernels over the slab, GroupNormKernels.cpp:1088-1165 and 1353-1589).
+    Against the oracle, with every wait given up (a workgroup then sums the slab itself), in
+    place and with dX over X (the multi-launch kernels), without gamma, dX alone, twice the
+    same bits."""
+    if mixed and dtype == torch.float32:
+        pytest.skip("mixed precision means float32 weights beside 16-bit rows")
+    wdtype = torch.float32 if mixed else dtype
+    E = 4 if dtype == torch.float32 else 8
+    for i, (N, C, HxW, groups) in enumerate(BWD_SHAPES):
+        if HxW % E:
+            continue
+        print("case group norm large maps backward", dtype, mixed, (N, C, HxW, groups), flush=True)
+        g = gen(1860 + i)
+        x = (0.5 + torch.randn(N, C, HxW, generator=g)).to(dtype)
+        dy = torch.randn(N, C, HxW, generator=g).to(dtype)
+        x[N - 1, C - 1] = 1.25  # a constant channel
+        gamma = (1 + 0.1 * torch.randn(C, generator=g)).to(wdtype)
+        xg, dyg, gg = x.to(gpu), dy.to(gpu), gamma.to(gpu)
+        what = "[%d, %d, %d] in %d groups %s" % (N, C, HxW, groups, dtype)
+        _, mean, rstd = cabi.group_norm_fwd(xg, gg, None, groups, 1e-5)
+        dx, dg, db = cabi.group_norm_bwd(dyg, xg, mean, rstd, gg, groups)
+        odx, odg, odb = oracle.group_norm_bwd(to_np32(dy), to_np32(x), groups, to_np32(mean.float()),
+                                              to_np32(rstd.float()), to_np32(gamma))
+        D = C // groups
+        mu = mean.float().cpu().reshape(N, groups, 1, 1)
+        rs = rstd.float().cpu().reshape(N, groups, 1, 1)
+        xhat = ((x.float().reshape(N, groups, D, HxW) - mu) * rs).reshape(N, C, HxW)
+        # (float32 partial sums: a few ulps of the sum of the magnitudes, per channel)
+        sl_g = (dy.float() * xhat).abs().sum(dim=(0, 2)) * 2.0 ** -22
+        sl_b = dy.float().abs().sum(dim=(0, 2)) * 2.0 ** -22
+        assert_close(dx, odx, dtype, "group_norm dx " + what)
+        assert_close(dg.float(), odg, wdtype, "dgamma " + what, slack=sl_g)
+        assert_close(db.float(), odb, wdtype, "dbeta " + what, slack=sl_b)
+        dx2, dg2, db2 = cabi.group_norm_bwd(dyg, xg, mean, rstd, gg, groups)
+        for a, b in ((dx, dx2), (dg, dg2), (db, db2)):
+            assert torch.equal(a.view(torch.uint8), b.view(torch.uint8)), "twice the same bits " + what
+        fdx, fdg, fdb = _with_wait(cabi, 0, lambda: cabi.group_norm_bwd(dyg, xg, mean, rstd, gg, groups))
+        assert_close(fdx, odx, dtype, "dx, every wait given up " + what)
+        assert_close(fdg.float(), odg, wdtype, "dgamma, every wait given up " + what, slack=sl_g)
+        assert_close(fdb.float(), odb, wdtype, "dbeta, every wait given up " + what, slack=sl_b)
+        # in place over dY and over X: the multi-launch kernels
+        for over in ("dy", "x"):
+            dyc, xc = dyg.clone(), xg.clone()
+            target = dyc if over == "dy" else xc
+            idx, idg, idb = cabi.group_norm_bwd(dyc, xc, mean, rstd, gg, groups, dx=target)
+            assert idx.data_ptr() == target.data_ptr()
+            assert_close(idx, odx, dtype, "dx over %s %s" % (over, what))
+            assert_close(idg.float(), odg, wdtype, "dgamma, dx over %s %s" % (over, what), slack=sl_g)
+        if i % 2 == 0:
+            dx1, n1, n2 = cabi.group_norm_bwd(dyg, xg, mean, rstd, gg, groups, want=(True, False, False))
+            assert n1 is None and n2 is None and torch.equal(dx1, dx), "dX alone " + what
+            dx0, dg0, db0 = cabi.group_norm_bwd(dyg, xg, mean, rstd, None, groups)
+            odx0, odg0, odb0 = oracle.group_norm_bwd(to_np32(dy), to_np32(x), groups,
+                                                     to_np32(mean.float()), to_np32(rstd.float()), None)
+            assert_close(dx0, odx0, dtype, "dx without gamma " + what)
+            assert_close(dg0.float(), odg0, wdtype, "dgamma without gamma " + what, slack=sl_g)

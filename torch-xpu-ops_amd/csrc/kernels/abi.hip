@@ -784,6 +784,41 @@ int mi355x_group_norm_bwd(const void* dy, const void* x, const void* mean, const
   GroupNormBwdArgs a{dy,      x,       mean,   rstd,     gamma,    dx,       dgamma,     dbeta,
                      part_dg, part_db, d.rows, (int)d.L, (int)HxW, (int)d.D, (int)groups};
   hipStream_t s = (hipStream_t)stream;
+  // slabs beyond the registers whose channels are whole packs, 16-byte aligned tensors, dX
+  // apart from dY and X (a workgroup whose team does not come together reads the whole slab
+  // of both while others write theirs): teams of workgroups, dY and X read once.  As few
+  // packs a lane (1, 2, 4, 8 of each tensor) as hold a channel on one workgroup, else 8 and
+  // several workgroups a channel, the last of them at least half full.
+  const int64_t E = 16 / esize_of(xd);
+  if (!plan.resident && dx && HxW % E == 0 &&
+      ((((uintptr_t)dy) | ((uintptr_t)x) | ((uintptr_t)dx)) & 15u) == 0) {
+    const size_t nbytes = (size_t)d.rows * (size_t)d.L * (size_t)esize_of(xd);
+    const char *ob = (const char*)dx, *gb = (const char*)dy, *xb = (const char*)x;
+    const int64_t cp = HxW / E;
+    int v = 8;
+    for (int t = 1; t < 8; t *= 2)
+      if ((int64_t)t * kTeamBlock >= cp) {
+        v = t;
+        break;
+      }
+    const int64_t chunk = (int64_t)v * kTeamBlock;
+    const int64_t wpc = (cp + chunk - 1) / chunk;
+    const int64_t team = d.D * wpc;
+    const int64_t cus = current_num_cus() * kTeamPerCu < kTeamMaxWorkgroups
+                            ? current_num_cus() * kTeamPerCu
+                            : kTeamMaxWorkgroups;
+    const bool apart = !(ob < gb + nbytes && gb < ob + nbytes) && !(ob < xb + nbytes && xb < ob + nbytes);
+    if (apart && team >= 2 && team <= cus && 2 * cp >= wpc * chunk) {
+      int64_t teams = cus / team;
+      if (teams > d.rows) teams = d.rows;
+      a.team = (int)team;
+      a.team_wpc = (int)wpc;
+      a.team_v = v;
+      a.team_grid = teams * team;
+      a.team_slot = team_slot_for_call(s, &a.team_id);
+      a.team_wait_ticks = g_team_wait_ticks.load(std::memory_order_relaxed);
+    }
+  }
   if (xd == ROWNORM_F32) return launch_group_norm_bwd<float, float>(plan, a, s);
   if (xd == ROWNORM_F16)
     return wd == ROWNORM_F32 ? launch_group_norm_bwd<f16, float>(plan, a, s)

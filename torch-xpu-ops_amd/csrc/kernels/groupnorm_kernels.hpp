@@ -52,6 +52,7 @@
 
 #include "device/pack.hpp"
 #include "device/reduce.hpp"
+#include "device/team.hpp"
 #include "plan.hpp"
 
 namespace rownorm {
@@ -993,6 +994,183 @@ gn_channel_sums_kernel(const T* __restrict__ dy, const T* __restrict__ x,
       part_dg[r] = acc[0] * rs;
       if (part_db) part_db[r] = acc[1];
     }
+  }
+}
+
+// ---------------------------------------------------------------------------
+// Backward of slabs beyond one workgroup's registers whose channels are whole packs, dY and
+// X read once: a team of workgroups holds a (sample, group) slab, `wpc` workgroups a channel,
+// V packs of dY and of X a lane.  A workgroup publishes its piece's sums of dy * (x - mean)
+// * rstd and of dy (team_publish_and_gather); every workgroup adds the team's numbers channel
+// by channel in a fixed order, forms s1 = sum_c gamma_c * db_c and s2 = sum_c gamma_c * dg_c
+// (the reference's ComputeBackwardFusedParamsFunctor, GroupNormKernels.cpp:1088-1165) and
+// writes dX for what it holds; the first workgroup of a channel leaves the channel's sums in
+// the [N, C] partial buffers (the second stage adds them over the samples).  A workgroup
+// whose wait runs out takes the slab's sums itself in a pass over the whole slab (dX must
+// not overlap dY or X) and loads its packs again.
+template <class T, class WT, int V>
+__global__ void __launch_bounds__(kTeamBlock, kTeamPerCu * kTeamBlock / 256)
+gn_bwd_team_kernel(const T* __restrict__ dy, const T* __restrict__ x,
+                   const WT* __restrict__ mean, const WT* __restrict__ rstd,
+                   const WT* __restrict__ gamma, T* __restrict__ dx,
+                   float* __restrict__ part_dg, float* __restrict__ part_db, int64_t rows,
+                   GroupShape s, int team, int wpc, TeamSlot* slot, unsigned int call_id,
+                   unsigned long long wait_ticks) {
+  constexpr int E = elems_per_pack<T>::value;
+  constexpr int BLOCK = kTeamBlock;
+  __shared__ float red[reduce_lds_floats<BLOCK, BLOCK, 4>::value];
+  __shared__ double tpart[kTeamMaxWorkgroups][2];
+  __shared__ float stat[4];  // s1, s2, -, whether the team failed
+  int phase = 0;
+  const int tm = (int)blockIdx.x / team;
+  const int c = (int)blockIdx.x - tm * team;
+  const int teams = (int)gridDim.x / team;
+  const int ch = c / wpc;             // the channel of the group this workgroup works on
+  const int piece = c - ch * wpc;     // and its piece of the channel
+  const int cp = s.HxW / E;           // packs a channel
+  const int pk0 = piece * (V * BLOCK) + (int)threadIdx.x;
+  const float fL = (float)s.L;
+  const uint32_t loff = (uint32_t)(pk0 < cp ? pk0 : 0) * 16u;
+  // (a pointer into global memory, as in the other team kernels)
+  auto at = [](auto* p, uint32_t off) {
+    using Elem = std::remove_pointer_t<decltype(p)>;
+    typedef __attribute__((address_space(1))) Elem* GlobalPtr;
+    return (Elem*)reinterpret_cast<GlobalPtr>(reinterpret_cast<uintptr_t>(p) + off);
+  };
+  unsigned int round = 0;
+  for (int64_t row = tm; row < rows; row += teams, ++round) {
+    TeamEntry* entries = slot->entry[round & 1u];
+    if (threadIdx.x == 0) team_store(&entries[blockIdx.x].tag, 0ull);
+    const int g = (int)((uint32_t)row % (uint32_t)s.groups);
+    const int64_t n = row / s.groups;
+    const float mu = (float)mean[row], rs = (float)rstd[row];
+    const int64_t base = row * (int64_t)s.L + (int64_t)ch * s.HxW;
+    const T* gb = dy + base;
+    const T* xb = x + base;
+    Pack<T, E> dp[V], xp[V];
+    auto load_chunk = [&]() {
+#pragma unroll
+      for (int k = 0; k < V; ++k) {
+        dp[k] = Pack<T, E>::zero();
+        xp[k] = Pack<T, E>::zero();
+        if (pk0 + k * BLOCK < cp) {
+          dp[k] = Pack<T, E>::load_stream(at(gb + k * BLOCK * E, loff));
+          xp[k] = Pack<T, E>::load_stream(at(xb + k * BLOCK * E, loff));
+        }
+      }
+    };
+    load_chunk();
+    float acc[2] = {0.0f, 0.0f};
+#pragma unroll
+    for (int k = 0; k < V; ++k) {
+      if (pk0 + k * BLOCK < cp) {
+#pragma unroll
+        for (int i = 0; i < E; ++i) {
+          const float gy = dp[k].get(i);
+          acc[1] += gy;
+          acc[0] = fmaf(gy, xp[k].get(i) - mu, acc[0]);
+        }
+      }
+      keep_packed(dp[k]);
+      keep_packed(xp[k]);
+      __builtin_amdgcn_sched_barrier(0);  // (one pack widened at a time: registers)
+    }
+    group_allreduce<BLOCK, BLOCK, 2, SumOp>(acc, red, phase);
+    if (threadIdx.x < 64) {  // the first wavefront publishes, waits and adds up
+      const int lane = (int)threadIdx.x;
+      const bool complete =
+          team_publish_and_gather(slot, entries, tm, team, call_id, round, wait_ticks,
+                                  (double)(acc[0] * rs), (double)acc[1], tpart);
+      // (the lanes of a wavefront see one another's LDS stores in program order)
+      if (complete) {
+        float s1 = 0.0f, s2 = 0.0f;
+        for (int d = lane; d < s.D; d += 64) {
+          float dg = 0.0f, db = 0.0f;
+          for (int q = 0; q < wpc; ++q) {
+            dg += (float)tpart[d * wpc + q][0];
+            db += (float)tpart[d * wpc + q][1];
+          }
+          const float ga = gn_weight(gamma, g * s.D + d, 1.0f);
+          s1 = fmaf(db, ga, s1);
+          s2 = fmaf(dg, ga, s2);
+          if (d == ch && piece == 0 && part_dg != nullptr) {
+            const int64_t o = n * ((int64_t)s.groups * s.D) + (int64_t)g * s.D + d;
+            part_dg[o] = dg;
+            if (part_db != nullptr) part_db[o] = db;
+          }
+        }
+        s1 = wave_group_allreduce<64, SumOp>(s1);
+        s2 = wave_group_allreduce<64, SumOp>(s2);
+        if (lane == 0) {
+          stat[0] = s1;
+          stat[1] = s2;
+          stat[3] = 0.0f;
+        }
+      } else if (lane == 0) {
+        stat[3] = 1.0f;
+      }
+    }
+    __syncthreads();
+    if (stat[3] != 0.0f) {  // (uniform over the workgroup)
+      // The team did not come together: the slab's sums in a pass over the whole slab --
+      // s1, s2 and, for the partial buffers, this workgroup's own channel --, then the
+      // packs again.
+      const T* gr = dy + row * (int64_t)s.L;
+      const T* xr = x + row * (int64_t)s.L;
+      float w[4] = {0.0f, 0.0f, 0.0f, 0.0f};  // s1, s2 / rstd, own channel's dg / rstd and db
+      for (int pk = (int)threadIdx.x; pk < s.D * cp; pk += BLOCK) {
+        const int d = pk / cp;
+        const Pack<T, E> pd = Pack<T, E>::load(gr + (int64_t)pk * E);
+        const Pack<T, E> px = Pack<T, E>::load(xr + (int64_t)pk * E);
+        const float ga = gn_weight(gamma, g * s.D + d, 1.0f);
+        float a = 0.0f, b = 0.0f;
+#pragma unroll
+        for (int i = 0; i < E; ++i) {
+          const float gy = pd.get(i);
+          b += gy;
+          a = fmaf(gy, px.get(i) - mu, a);
+        }
+        w[0] = fmaf(b, ga, w[0]);
+        w[1] = fmaf(a, ga, w[1]);
+        if (d == ch) {
+          w[2] += a;
+          w[3] += b;
+        }
+      }
+      group_allreduce<BLOCK, BLOCK, 4, SumOp>(w, red, phase);
+      if (threadIdx.x == 0) {
+        stat[0] = w[0];
+        stat[1] = w[1] * rs;
+        if (piece == 0 && part_dg != nullptr) {
+          const int64_t o = n * ((int64_t)s.groups * s.D) + (int64_t)g * s.D + ch;
+          part_dg[o] = w[2] * rs;
+          if (part_db != nullptr) part_db[o] = w[3];
+        }
+      }
+      __syncthreads();
+      load_chunk();
+    }
+    const float s1 = stat[0], s2 = stat[1], term1 = rs / fL;
+    const float ga = gn_weight(gamma, g * s.D + ch, 1.0f);
+    T* ob = dx + base;
+#pragma unroll
+    for (int k = 0; k < V; ++k) {
+      if (pk0 + k * BLOCK < cp) {
+        Pack<T, E> o;
+#pragma unroll
+        for (int i = 0; i < E; ++i) {
+          float f = fL * (dp[k].get(i) * ga);
+          f -= ((xp[k].get(i) - mu) * rs) * s2;
+          f -= s1;
+          o.set(i, f * term1);
+        }
+        o.store_stream(at(ob + k * BLOCK * E, loff));
+      }
+      // (pack k + 1 is widened after pack k has been stored, not before: registers)
+      __builtin_amdgcn_sched_barrier(0);
+    }
+    // stat[] is rewritten for the next slab only after every thread has passed the
+    // barrier of the next block reduction, i.e. after it has read this slab's values
   }
 }
 

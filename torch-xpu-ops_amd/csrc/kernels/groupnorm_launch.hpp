@@ -204,7 +204,27 @@ int launch_group_norm_bwd(const Plan& plan, const GroupNormBwdArgs& a, hipStream
   const int64_t N = a.rows / a.groups;
   const int C = a.groups * a.D;
   int err = 0;
-  if (need_sums && !fused_cols) {
+  const bool teams = !plan.resident && a.team > 0 && a.team_slot != nullptr && a.dx != nullptr;
+  if (teams) {
+    // slabs beyond the registers, dY and X read once: teams of workgroups
+    GroupNormBwdArgs k = a;
+    if (!want_cols) k.part_dg = k.part_db = nullptr;
+    auto go = [&](auto v) {
+      constexpr int V = decltype(v)::value;
+      hipLaunchKernelGGL((gn_bwd_team_kernel<T, WT, V>), dim3((unsigned)a.team_grid),
+                         dim3(kTeamBlock), 0, stream, (const T*)a.dy, (const T*)a.x,
+                         (const WT*)a.mean, (const WT*)a.rstd, (const WT*)a.gamma, (T*)a.dx,
+                         k.part_dg, k.part_db, a.rows, shape, a.team, a.team_wpc,
+                         (TeamSlot*)a.team_slot, a.team_id, a.team_wait_ticks);
+    };
+    switch (a.team_v) {
+      case 1: go(std::integral_constant<int, 1>{}); break;
+      case 2: go(std::integral_constant<int, 2>{}); break;
+      case 4: go(std::integral_constant<int, 4>{}); break;
+      case 8: go(std::integral_constant<int, 8>{}); break;
+      default: return (int)hipErrorInvalidConfiguration;
+    }
+  } else if (need_sums && !fused_cols) {
     const int packs = (a.HxW + E - 1) / E;
     const int64_t nc_rows = N * C;
     auto sums = [&](auto cb) {
@@ -228,7 +248,9 @@ int launch_group_norm_bwd(const Plan& plan, const GroupNormBwdArgs& a, hipStream
     err = (int)hipGetLastError();
     if (err != 0) return err;
   }
-  if (plan.resident && plan.exact_depth > 0) {
+  if (teams) {
+    // (launched above)
+  } else if (plan.resident && plan.exact_depth > 0) {
     GroupNormBwdArgs k = a;
     if (!want_cols) k.part_dg = k.part_db = nullptr;
     if (a.dx == nullptr || !launch_group_bwd_exact<T, WT>(plan, k, stream, ilist<0, 1, 2, 3, 4>{}))

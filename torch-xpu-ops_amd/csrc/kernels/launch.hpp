@@ -136,6 +136,15 @@ struct GroupNormBwdArgs {
   float* part_db;
   int64_t rows;
   int L, HxW, D, groups;
+  // gn_bwd_team_kernel (slabs beyond the registers held by teams of workgroups): workgroups a
+  // slab and a channel, packs a lane of each tensor, workgroups launched; the call's slot of
+  // bookkeeping memory, its id and the bound of a wait, as in GroupNormFwdArgs; team == 0 or
+  // a null slot: not for this call
+  int team = 0, team_wpc = 0, team_v = 0;
+  int64_t team_grid = 0;
+  void* team_slot = nullptr;
+  unsigned int team_id = 0;
+  unsigned long long team_wait_ticks = 0;
 };
 
 inline bool regions_disjoint(const void* a, int64_t abytes, const void* b, int64_t bbytes) {
