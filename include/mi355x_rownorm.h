@@ -399,7 +399,7 @@ int mi355x_rownorm_set_override(rownorm_op op, int lanes_per_row, int packs_per_
  * 16-byte packs, no residual add, no cast, y not overlapping x; GroupNorm forward
  * slabs of that size; softmax / log_softmax forward and backward of few, very long
  * rows; LayerNorm / RMSNorm backward rows beyond one workgroup's registers in calls of
- * many rows): how long a workgroup waits for the others of its team before it sums the
+ * many rows; GroupNorm backward slabs of long whole-pack channels): how long a workgroup waits for the others of its team before it sums the
  * whole row itself (a second pass over the inputs, the same result to rounding), in
  * microseconds; 0xffffffff
  * restores the default, one second.  0 makes every wait give up at once, which is

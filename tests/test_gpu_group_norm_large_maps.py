@@ -123,7 +123,8 @@ def test_special_slabs_and_channels_that_are_not_whole_packs(cabi, oracle, gpu):
 # lane, a workgroup a channel); slabs of 8 channels of 4097 packs (two workgroups a channel, the
 # second nearly empty: the multi-launch kernels keep them) and of 6000 packs (two workgroups a
 # channel, the second ragged); 16 slabs of 8 channels of 16384 packs (four workgroups a channel,
-# 32 a slab); one group of 3 channels of 300 packs in fp32 terms (one pack a lane, idle lanes)
+# 32 a slab); one group of 3 channels of 300 to 600 packs (short channels keep the multi-launch
+# kernels)
 BWD_SHAPES = [(2, 256, 16384, 32), (2, 16, 4097 * 8, 2), (3, 16, 6000 * 8, 2), (1, 128, 131072, 16),
               (5, 3, 2400, 1)]
 

@@ -787,7 +787,7 @@ int mi355x_group_norm_bwd(const void* dy, const void* x, const void* mean, const
   // slabs beyond the registers whose channels are whole packs, 16-byte aligned tensors, dX
   // apart from dY and X (a workgroup whose team does not come together reads the whole slab
   // of both while others write theirs): teams of workgroups, dY and X read once.  As few
-  // packs a lane (1, 2, 4, 8 of each tensor) as hold a channel on one workgroup, else 8 and
+  // packs a lane (4 or 8 of each tensor) as hold a channel on one workgroup, else 8 and
   // several workgroups a channel, the last of them at least half full.
   const int64_t E = 16 / esize_of(xd);
   if (!plan.resident && dx && HxW % E == 0 &&
@@ -808,7 +808,10 @@ int mi355x_group_norm_bwd(const void* dy, const void* x, const void* mean, const
                             ? current_num_cus() * kTeamPerCu
                             : kTeamMaxWorkgroups;
     const bool apart = !(ob < gb + nbytes && gb < ob + nbytes) && !(ob < xb + nbytes && xb < ob + nbytes);
-    if (apart && team >= 2 && team <= cus && 2 * cp >= wpc * chunk) {
+    // (channels of at most 1024 packs -- one or two packs a lane -- move too little between
+    // two exchanges: bf16 [2, 2048, 64, 64] in 32 groups, 8 rounds of 8 KB a workgroup and
+    // tensor, 56.6 us against 35.0 us for the two launches)
+    if (apart && v >= 4 && team >= 2 && team <= cus && 2 * cp >= wpc * chunk) {
       int64_t teams = cus / team;
       if (teams > d.rows) teams = d.rows;
       a.team = (int)team;

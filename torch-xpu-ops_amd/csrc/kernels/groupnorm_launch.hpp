@@ -218,8 +218,6 @@ int launch_group_norm_bwd(const Plan& plan, const GroupNormBwdArgs& a, hipStream
                          (TeamSlot*)a.team_slot, a.team_id, a.team_wait_ticks);
     };
     switch (a.team_v) {
-      case 1: go(std::integral_constant<int, 1>{}); break;
-      case 2: go(std::integral_constant<int, 2>{}); break;
       case 4: go(std::integral_constant<int, 4>{}); break;
       case 8: go(std::integral_constant<int, 8>{}); break;
       default: return (int)hipErrorInvalidConfiguration;
