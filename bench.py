@@ -787,8 +787,10 @@ def model_shapes_table(torch, cabi, L, dev, stream, P, only=None):
         del sets, ws, x0, dy0, m0, r0
         torch.cuda.empty_cache()
 
-    # hidden sizes beyond 16384 (Nemotron-4 340B and PaLM 540B: 18432)
-    for name, M, N in (("native_layer_norm bf16 [8192, 18432] (hidden 18432)", 8192, 18432),):
+    # hidden sizes beyond 16384 (Nemotron-4 340B and PaLM 540B: 18432), and rows beyond one
+    # workgroup's registers in a call of many rows (the backward: teams of workgroups)
+    for name, M, N in (("native_layer_norm bf16 [8192, 18432] (hidden 18432)", 8192, 18432),
+                       ("native_layer_norm bf16 [4096, 65536] (rows of 64 K elements)", 4096, 65536)):
         if only is not None and not any(t in name + " fwd" or t in name + " bwd" for t in only.split("|")):
             continue
         w = (1 + 0.1 * torch.randn(N, device=dev)).to(bf16)
