@@ -132,3 +132,48 @@ def test_softmax_fwd_bwd_beyond_2_31_elements(cabi, oracle, gpu):
                 del g32
             del y32
         del y, gi
+
+
+def test_long_rows_held_by_teams_beyond_2_31_elements(cabi, oracle, gpu):
+    """bf16 [32771, 65544] (2 147 942 424 elements, 4.3 GB a tensor): rows beyond one workgroup's
+    registers, whose backward teams of workgroups hold four rows at a time (norm_bwd_team_kernel)
+    and whose last groups of rows lie beyond the 32-bit offsets.  RMSNorm forward and backward:
+    the first, middle and last rows against the oracle; every row against sum_j dx_j x_j = 0;
+    dweight against the closed form in float64 on the GPU."""
+    M, N = 32771, 65544
+    assert M * N > (1 << 31)
+    p = cabi.plan(cabi.OP_RMS_NORM_BWD, M, N, cabi.BF16, cabi.BF16)
+    assert p["resident"] == 0 and p["block_threads"] == 512 and p["packs_per_lane"] == 2, p
+    print("case large long rows", (M, N), flush=True)
+    rows = 2048  # rows per step of the all-rows checks
+    g = torch.Generator(device=gpu).manual_seed(21)
+    x = torch.empty(M, N, dtype=BF, device=gpu)
+    dy = torch.empty(M, N, dtype=BF, device=gpu)
+    for r0 in range(0, M, rows):
+        r = slice(r0, min(M, r0 + rows))
+        x[r] = torch.randn(r.stop - r.start, N, generator=g, device=gpu).to(BF)
+        dy[r] = torch.randn(r.stop - r.start, N, generator=g, device=gpu).to(BF)
+    w = (1 + 0.1 * torch.randn(N, device=gpu)).to(BF)
+    y, rstd = cabi.rms_norm_fwd(x, w, 1e-6)
+    del y
+    dx, dw = cabi.rms_norm_bwd(dy, x, rstd, w)
+    for r in (slice(0, 8), slice(M // 2, M // 2 + 8), slice(M - 8, M)):
+        odx, _ = oracle.rms_norm_bwd(to_np32(dy[r]), to_np32(x[r]), (N,), to_np32(rstd[r]),
+                                     to_np32(w), mask=(True, False))
+        assert_close(dx[r], odx, BF, "dx rows %d.." % r.start)
+    ref_dw = torch.zeros(N, dtype=torch.float64, device=gpu)
+    mag_dw = torch.zeros(N, dtype=torch.float64, device=gpu)
+    for r0 in range(0, M, rows):
+        r = slice(r0, min(M, r0 + rows))
+        dxr, xr = dx[r].double(), x[r].double()
+        dot = (dxr * xr).sum(1)
+        mag = (dxr * xr).abs().sum(1)
+        # (dx is rounded to bf16: each term carries up to 2^-9 of relative error)
+        assert bool((dot.abs() <= mag * 2.0 ** -7 + 1e-6).all()), "sum_j dx_j x_j, rows %d.." % r0
+        t = dy[r].double() * xr * rstd[r].double().reshape(-1, 1)
+        ref_dw += t.sum(0)
+        mag_dw += t.abs().sum(0)
+        del dxr, xr, t
+    err = (dw.double() - ref_dw).abs()
+    # bf16 rounding of dweight plus the float32 partial sums of the kernel
+    assert bool((err <= 1e-2 + 1.6e-2 * ref_dw.abs() + mag_dw * 2.0 ** -20).all()), float(err.max())
